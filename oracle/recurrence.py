@@ -1,0 +1,69 @@
+"""TEST INFRASTRUCTURE ONLY -- the per-timestep PyTorch recurrences.
+
+These are the differentiable, one-step-at-a-time statements of the two fast
+weight programmers that the reference's authors use to check their CUDA
+kernels (SRWM: supervised_learning/self_ref_v0/__init__.py:298-361; delta rule:
+supervised_learning/fast_weight/__init__.py:167-195): batched ``torch.bmm``
+readouts over a ``(B*H, ...)`` view, softmax / sigmoid, and a rank-1 ``bmm``
+write per step.  Autograd provides the gradients, so this file is an
+independent check of the hand-derived reverse-time backward in
+``fastweight_oracle.c`` -- and it is the "reference PyTorch recurrence" whose
+host-CPU throughput the bench reports beside the GPU number.
+
+Differences from the authors' script, on purpose: wrapped in functions, device
+and dtype follow the inputs, and the write is also applied at the last step
+(the kernels do so, self_ref_v0.cu:335-350, and the carried state depends on
+it; outputs and gradients of a plain call are unaffected).
+"""
+import torch
+import torch.nn.functional as F
+
+
+def srwm_recurrence(x, W_y, W_q, W_k, w_b):
+    """x [N,H,L,E]; W_* [N,H,E,E]; w_b [N,H,E,4] -> (out [N,H,L,E], final 4-state)."""
+    N, H, L, E = x.shape
+    xs = x.permute(2, 0, 1, 3).reshape(L, N * H, E)
+    Wy = W_y.reshape(N * H, E, E)
+    Wq = W_q.reshape(N * H, E, E)
+    Wk = W_k.reshape(N * H, E, E)
+    wb = w_b.reshape(N * H, E, 4)
+    outs = []
+    for t in range(L):
+        xt = xs[t].unsqueeze(1)                                   # (B*H, 1, E)
+        outs.append(torch.bmm(xt, Wy).squeeze(1))
+        q = F.softmax(torch.bmm(xt, Wq).squeeze(1), dim=-1)
+        k = F.softmax(torch.bmm(xt, Wk).squeeze(1), dim=-1)
+        beta = torch.sigmoid(torch.bmm(xt, wb).squeeze(1))
+        b_y, b_q, b_k, b_b = torch.split(beta, [1, 1, 1, 1], dim=-1)
+        ku, qu = k.unsqueeze(1), q.unsqueeze(1)
+        y_ins = b_y * (torch.bmm(qu, Wy) - torch.bmm(ku, Wy)).squeeze(1)
+        q_ins = b_q * (torch.bmm(qu, Wq) - torch.bmm(ku, Wq)).squeeze(1)
+        k_ins = b_k * (torch.bmm(qu, Wk) - torch.bmm(ku, Wk)).squeeze(1)
+        b_ins = b_b * (torch.bmm(qu, wb) - torch.bmm(ku, wb)).squeeze(1)
+        kc = k.unsqueeze(2)
+        Wy = Wy + torch.bmm(kc, y_ins.unsqueeze(1))
+        Wq = Wq + torch.bmm(kc, q_ins.unsqueeze(1))
+        Wk = Wk + torch.bmm(kc, k_ins.unsqueeze(1))
+        wb = wb + torch.bmm(kc, b_ins.unsqueeze(1))
+    out = torch.stack(outs).view(L, N, H, E).permute(1, 2, 0, 3)
+    final = (Wy.view(N, H, E, E), Wq.view(N, H, E, E), Wk.view(N, H, E, E), wb.view(N, H, E, 4))
+    return out, final
+
+
+def delta_recurrence(Q, K, V, beta, W0):
+    """Q,K [N,H,L,E]; V [N,H,L,M]; beta [N,H,L,1]; W0 [N,H,E,M] -> (out [N,H,L,M], W_L)."""
+    N, H, L, E = Q.shape
+    M = V.shape[-1]
+    qs = Q.permute(2, 0, 1, 3).reshape(L, N * H, E)
+    ks = K.permute(2, 0, 1, 3).reshape(L, N * H, E)
+    vs = V.permute(2, 0, 1, 3).reshape(L, N * H, M)
+    bs = beta.permute(2, 0, 1, 3).reshape(L, N * H, 1)
+    W = W0.reshape(N * H, E, M).transpose(1, 2)                     # kept as (B*H, M, E)
+    outs = []
+    for t in range(L):
+        v_old = torch.bmm(W, ks[t].unsqueeze(2)).squeeze(2)
+        v_ins = bs[t] * (vs[t] - v_old)
+        W = W + torch.bmm(v_ins.unsqueeze(2), ks[t].unsqueeze(1))
+        outs.append(torch.bmm(W, qs[t].unsqueeze(2)).squeeze(2))
+    out = torch.stack(outs).view(L, N, H, M).permute(1, 2, 0, 3)
+    return out, W.transpose(1, 2).reshape(N, H, E, M)

@@ -1,0 +1,116 @@
+"""Pins the delta-rule CPU oracle without the GPU: closed forms (beta = 0, exact
+retrieval with orthonormal keys, one-hot keys == causal linear attention),
+fp64 autograd of the per-timestep torch recurrence, finite differences."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle.recurrence import delta_recurrence
+from helpers import delta_inputs, rel_err
+
+
+def _np(ts):
+    return [t.numpy() for t in ts]
+
+
+def test_beta_zero_reads_the_initial_state():
+    q, k, v, beta, W0, go = delta_inputs(2, 2, 9, 6, 5, seed=1, w0_std=1.0)
+    beta = torch.zeros_like(beta)
+    f = oracle.delta_forward(*_np((q, k, v, beta, W0)))
+    assert rel_err(f["out"], torch.matmul(q, W0).numpy()) < 1e-14
+    assert rel_err(f["W"], W0.numpy()) == 0.0
+
+
+def test_first_step_from_empty_memory():
+    q, k, v, beta, W0, _ = delta_inputs(1, 3, 1, 4, 7, seed=2)
+    f = oracle.delta_forward(*_np((q, k, v, beta, W0)))
+    ref = beta * (k * q).sum(-1, keepdim=True) * v          # beta_0 (k_0.q_0) v_0
+    assert rel_err(f["out"], ref.numpy()) < 1e-14
+
+
+def test_orthonormal_keys_with_beta_one_retrieve_exactly():
+    E, M, L = 6, 4, 6
+    g = torch.Generator().manual_seed(3)
+    Qm, _ = torch.linalg.qr(torch.randn(E, E, generator=g, dtype=torch.float64))
+    k = Qm[:L].reshape(1, 1, L, E)
+    v = torch.randn(1, 1, L, M, generator=g, dtype=torch.float64)
+    beta = torch.ones(1, 1, L, 1, dtype=torch.float64)
+    f = oracle.delta_forward(*_np((k, k, v, beta, torch.zeros(1, 1, E, M, dtype=torch.float64))))
+    # querying with the key just written returns its value; all earlier ones stay retrievable
+    assert rel_err(f["out"], v.numpy()) < 1e-13
+    assert rel_err(np.einsum("em,le->lm", f["W"][0, 0], k[0, 0].numpy()), v[0, 0].numpy()) < 1e-13
+
+
+def test_one_hot_keys_reduce_to_causal_linear_attention():
+    """Distinct one-hot keys, beta = 1, W_0 = 0 => v_old = 0 => out = tril(Q K^T) V,
+    and the gradients are those of that masked product."""
+    N, H, L, E, M = 2, 2, 5, 7, 3
+    q, _, v, _, W0, go = delta_inputs(N, H, L, E, M, seed=4)
+    perm = torch.stack([torch.randperm(E, generator=torch.Generator().manual_seed(i))[:L]
+                        for i in range(N * H)]).view(N, H, L)
+    k = torch.nn.functional.one_hot(perm, E).to(torch.float64)
+    beta = torch.ones(N, H, L, 1, dtype=torch.float64)
+    f = oracle.delta_forward(*_np((q, k, v, beta, W0)))
+    qt, kt, vt = (t.clone().requires_grad_(True) for t in (q, k, v))
+    ref = torch.matmul(torch.tril(torch.matmul(qt, kt.transpose(-1, -2))), vt)
+    assert rel_err(f["out"], ref.detach().numpy()) < 1e-14
+    assert np.abs(f["v_old"]).max() == 0.0
+    (ref * go).sum().backward()
+    b = oracle.delta_backward(*_np((q, k, v, beta)), f, go.numpy())
+    assert rel_err(b["grad_Q"], qt.grad.numpy()) < 1e-13
+    assert rel_err(b["grad_V"], vt.grad.numpy()) < 1e-13
+
+
+@pytest.mark.parametrize("shape,qk,w0", [
+    ((3, 5, 11, 64, 64), "sumnorm", 0.0),   # the reference self-test's shape and input style
+    ((2, 2, 33, 16, 16), "softmax", 0.0),
+    ((2, 3, 17, 8, 12), "l2", 0.5),          # E != M and a non-zero initial memory
+])
+def test_c_oracle_matches_autograd_of_the_torch_recurrence(shape, qk, w0):
+    q, k, v, beta, W0, go = delta_inputs(*shape, seed=5, qk=qk, w0_std=w0)
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, beta, W0)]
+    out, WL = delta_recurrence(*leaves)
+    (out * go).sum().backward()
+    f = oracle.delta_forward(*_np((q, k, v, beta, W0)))
+    assert rel_err(f["out"], out.detach().numpy()) < 1e-12
+    assert rel_err(f["W"], WL.detach().numpy()) < 1e-12
+    b = oracle.delta_backward(*_np((q, k, v, beta)), f, go.numpy(), want_grad_W=True)
+    for name, leaf in zip(("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W"), leaves):
+        assert rel_err(b[name], leaf.grad.numpy()) < 1e-10, name
+    # the backward sweep leaves the memory reverted to its initial value
+    assert np.abs(b["W0"] - W0.numpy()).max() < 1e-12
+
+
+def test_torch_recurrence_passes_finite_difference_gradcheck():
+    ts = delta_inputs(1, 2, 4, 3, 2, seed=6, w0_std=0.5)[:5]
+    ts = [t.requires_grad_(True) for t in ts]
+    assert torch.autograd.gradcheck(lambda *a: delta_recurrence(*a)[0], ts, eps=1e-6, atol=1e-7)
+
+
+def test_c_oracle_backward_against_central_differences():
+    q, k, v, beta, W0, go = delta_inputs(1, 2, 6, 4, 5, seed=7, w0_std=0.5)
+    rng = np.random.default_rng(1)
+    base = _np((q, k, v, beta, W0))
+    dirs = [rng.standard_normal(a.shape) for a in base]
+    loss = lambda args: float((oracle.delta_forward(*args)["out"] * go.numpy()).sum())
+    h = 1e-6
+    fd = (loss([a + h * d for a, d in zip(base, dirs)]) -
+          loss([a - h * d for a, d in zip(base, dirs)])) / (2 * h)
+    f = oracle.delta_forward(*base)
+    b = oracle.delta_backward(*base[:4], f, go.numpy(), want_grad_W=True)
+    an = sum((b[n] * d).sum() for n, d in
+             zip(("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W"), dirs))
+    assert abs(fd - an) < 1e-7 * max(1.0, abs(an))
+
+
+def test_f32_oracle_tracks_f64():
+    q, k, v, beta, W0, go = delta_inputs(2, 2, 64, 16, 16, seed=8)
+    base = _np((q, k, v, beta, W0))
+    f64 = oracle.delta_forward(*base)
+    f32 = oracle.delta_forward(*base, dtype=np.float32)
+    assert rel_err(f32["out"], f64["out"]) < 1e-5
+    b64 = oracle.delta_backward(*base[:4], f64, go.numpy())
+    b32 = oracle.delta_backward(*base[:4], f32, go.numpy(), dtype=np.float32)
+    for n in ("grad_Q", "grad_K", "grad_V", "grad_beta"):
+        assert rel_err(b32[n], b64[n]) < 1e-4, n

@@ -1,0 +1,212 @@
+"""Pins the SRWM CPU oracle (oracle/fastweight_oracle.c) WITHOUT the GPU.
+
+No reference fixture exists for this path (the reference's only check is a
+GPU-only script), so the oracle is pinned by what the mathematics fixes:
+closed forms, brute force with Python floats, invariants, an independent
+autograd statement of the recurrence and finite differences.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle.recurrence import srwm_recurrence
+from helpers import rel_err, srwm_inputs
+
+
+def _np(ts):
+    return [t.numpy() for t in ts]
+
+
+# ---------------------------------------------------------------- closed forms
+
+def test_beta_zero_is_a_plain_matmul():
+    """w_b very negative and x >= 0 => beta ~ 0 => W never changes => y = x @ W_y."""
+    x, W, go = srwm_inputs(2, 3, 9, 8, seed=1, w_std=0.5, x_softmax=True)
+    W[3] = torch.full_like(W[3], -60.0)
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    ref = torch.matmul(x, W[0]).numpy()
+    assert rel_err(f["out"], ref) < 1e-14
+    for got, w0 in zip((f["W_y"], f["W_q"], f["W_k"]), W[:3]):
+        assert rel_err(got, w0.numpy()) < 1e-14
+    assert f["beta"].max() < 1e-20
+    b = oracle.srwm_backward(x.numpy(), f, go.numpy())
+    # y_t = W_y^T x_t only: dL/dW_y = sum_t x_t (x) go_t, dL/dx_t = W_y go_t
+    assert rel_err(b["grad_W_y"], torch.matmul(x.transpose(-1, -2), go).numpy()) < 1e-13
+    assert rel_err(b["grad_x"], torch.matmul(go, W[0].transpose(-1, -2)).numpy()) < 1e-13
+    assert np.abs(b["grad_W_q"]).max() < 1e-15 and np.abs(b["grad_W_k"]).max() < 1e-15
+
+
+def test_equal_query_and_key_maps_freeze_the_state():
+    """W_q == W_k => q_t == k_t => diff = 0 at any beta => y = x @ W_y."""
+    x, W, _ = srwm_inputs(2, 2, 7, 6, seed=2, w_std=0.7)
+    W[2] = W[1].clone()
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    assert rel_err(f["out"], torch.matmul(x, W[0]).numpy()) < 1e-14
+    assert np.abs(f["y_diff"]).max() < 1e-14 and np.abs(f["beta_diff"]).max() < 1e-14
+    assert rel_err(f["W_k"], W[2].numpy()) < 1e-14
+    assert f["beta"].mean() > 0.2 and f["beta"].max() > 0.8  # beta is NOT degenerate here
+
+
+# ------------------------------------------------- brute force on a tiny case
+
+def _brute_force_step(x, Wy, Wq, Wk, wb):
+    """One SRWM step with Python floats and explicit index loops (lists of lists)."""
+    E = len(x)
+    col = lambda W, v, m: sum(W[e][m] * v[e] for e in range(E))
+    y = [col(Wy, x, m) for m in range(E)]
+    qp = [col(Wq, x, m) for m in range(E)]
+    kp = [col(Wk, x, m) for m in range(E)]
+    bp = [col(wb, x, j) for j in range(4)]
+    sm = lambda v: [math.exp(a - max(v)) / sum(math.exp(b - max(v)) for b in v) for a in v]
+    q, k = sm(qp), sm(kp)
+    beta = [1.0 / (1.0 + math.exp(-a)) for a in bp]
+    new = []
+    for W, b, n in ((Wy, beta[0], E), (Wq, beta[1], E), (Wk, beta[2], E), (wb, beta[3], 4)):
+        ins = [b * (col(W, q, m) - col(W, k, m)) for m in range(n)]
+        new.append([[W[e][m] + k[e] * ins[m] for m in range(n)] for e in range(E)])
+    return y, q, k, beta, new
+
+
+@pytest.mark.parametrize("E", [2, 3, 4])
+def test_brute_force_two_steps(E):
+    x, W, _ = srwm_inputs(1, 1, 2, E, seed=10 + E, w_std=1.0)
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    st = [w[0, 0].tolist() for w in W]
+    for t in range(2):
+        y, q, k, beta, st = _brute_force_step(x[0, 0, t].tolist(), *st)
+        assert np.allclose(f["out"][0, 0, t], y, rtol=1e-13, atol=1e-15)
+        assert np.allclose(f["q"][0, 0, t], q, rtol=1e-13)
+        assert np.allclose(f["k"][0, 0, t], k, rtol=1e-13)
+        assert np.allclose(f["beta"][0, 0, t], beta, rtol=1e-13)
+    for name, s in zip(("W_y", "W_q", "W_k", "w_b"), st):
+        assert np.allclose(f[name][0, 0], np.array(s), rtol=1e-12, atol=1e-15)
+
+
+# ------------------------------------------------------------------ invariants
+
+def test_emitted_vectors_are_consistent_with_the_state_trajectory():
+    N, H, L, E = 1, 2, 6, 5
+    x, W, _ = srwm_inputs(N, H, L, E, seed=3, w_std=0.8)
+    full = oracle.srwm_forward(x.numpy(), *_np(W))
+    assert np.allclose(full["q"].sum(-1), 1.0) and np.allclose(full["k"].sum(-1), 1.0)
+    assert (full["beta"] > 0).all() and (full["beta"] < 1).all()
+    pack = lambda d: np.concatenate([d["W_y"], d["W_q"], d["W_k"], d["w_b"]], axis=-1)
+    for t in range(L):
+        if t == 0:
+            Wprev = np.concatenate(_np(W), axis=-1)
+        else:
+            Wprev = pack(oracle.srwm_forward(x[:, :, :t].numpy(), *_np(W)))
+        Wnext = pack(oracle.srwm_forward(x[:, :, :t + 1].numpy(), *_np(W)))
+        q, k, beta = full["q"][:, :, t], full["k"][:, :, t], full["beta"][:, :, t]
+        diff = np.concatenate([full[n][:, :, t] for n in ("y_diff", "q_diff", "k_diff", "beta_diff")], -1)
+        # (vi) emitted diff is W_{t-1}^T (q_t - k_t)
+        assert np.allclose(np.einsum("nhem,nhe->nhm", Wprev, q - k), diff, rtol=1e-12, atol=1e-14)
+        # (iv) reading with k after the write: W_t^T k = W_{t-1}^T k + (k.k) ins
+        bb = np.concatenate([np.repeat(beta[..., j:j + 1], E if j < 3 else 4, -1) for j in range(4)], -1)
+        ins = bb * diff
+        lhs = np.einsum("nhem,nhe->nhm", Wnext, k)
+        rhs = np.einsum("nhem,nhe->nhm", Wprev, k) + (k * k).sum(-1, keepdims=True) * ins
+        assert np.allclose(lhs, rhs, rtol=1e-12, atol=1e-14)
+        # the write is exactly rank one along k
+        assert np.allclose(Wnext - Wprev, np.einsum("nhe,nhm->nhem", k, ins), rtol=1e-11, atol=1e-14)
+
+
+def test_backward_reverts_the_state_to_W0():
+    x, W, go = srwm_inputs(2, 2, 40, 8, seed=4, w_std=0.5)
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    b = oracle.srwm_backward(x.numpy(), f, go.numpy())
+    for name, w0 in zip(("W0_y", "W0_q", "W0_k", "w0_b"), W):
+        assert rel_err(b[name], w0.numpy()) < 1e-12
+
+
+# ----------------------------------- independent statement: autograd in fp64
+
+@pytest.mark.parametrize("shape,w_std,xsm", [
+    ((3, 5, 11, 8), 0.6, True),     # the reference self-test's shape and input style
+    ((2, 4, 64, 16), 0.02, False),  # BASELINE config 1 (CPU parity anchor)
+    ((2, 2, 20, 32), 1 / math.sqrt(32), True),
+    ((1, 3, 5, 7), 1.0, False),     # odd head dim
+])
+def test_c_oracle_matches_autograd_of_the_torch_recurrence(shape, w_std, xsm):
+    x, W, go = srwm_inputs(*shape, seed=5, w_std=w_std, x_softmax=xsm, per_batch_state=True)
+    xt = x.clone().requires_grad_(True)
+    Wt = [w.clone().requires_grad_(True) for w in W]
+    out, final = srwm_recurrence(xt, *Wt)
+    (out * go).sum().backward()
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    assert rel_err(f["out"], out.detach().numpy()) < 1e-12
+    for name, fw in zip(("W_y", "W_q", "W_k", "w_b"), final):
+        assert rel_err(f[name], fw.detach().numpy()) < 1e-12
+    b = oracle.srwm_backward(x.numpy(), f, go.numpy())
+    assert rel_err(b["grad_x"], xt.grad.numpy()) < 1e-10
+    for name, w in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), Wt):
+        assert rel_err(b[name], w.grad.numpy()) < 1e-10, name
+
+
+def test_gradient_through_the_returned_state_matches_autograd():
+    """Stateful use: the loss also depends on the final state W_L."""
+    x, W, go = srwm_inputs(2, 2, 6, 5, seed=6, w_std=0.7, per_batch_state=True)
+    g = torch.Generator().manual_seed(60)
+    gs = [torch.randn(w.shape, generator=g, dtype=torch.float64) for w in W]
+    xt = x.clone().requires_grad_(True)
+    Wt = [w.clone().requires_grad_(True) for w in W]
+    out, final = srwm_recurrence(xt, *Wt)
+    loss = (out * go).sum() + sum((f * s).sum() for f, s in zip(final, gs))
+    loss.backward()
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    b = oracle.srwm_backward(x.numpy(), f, go.numpy(), grad_state=_np(gs))
+    assert rel_err(b["grad_x"], xt.grad.numpy()) < 1e-10
+    for name, w in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), Wt):
+        assert rel_err(b[name], w.grad.numpy()) < 1e-10, name
+
+
+def test_torch_recurrence_passes_finite_difference_gradcheck():
+    x, W, _ = srwm_inputs(1, 2, 3, 3, seed=7, w_std=0.9, per_batch_state=True)
+    inputs = [x.requires_grad_(True)] + [w.requires_grad_(True) for w in W]
+    assert torch.autograd.gradcheck(lambda *a: srwm_recurrence(*a)[0], inputs, eps=1e-6, atol=1e-7)
+
+
+def test_c_oracle_backward_against_central_differences():
+    """Directional derivative of sum(out*go) computed by the C oracle alone."""
+    x, W, go = srwm_inputs(1, 2, 5, 4, seed=8, w_std=0.9, per_batch_state=True)
+    rng = np.random.default_rng(0)
+    dirs = [rng.standard_normal(t.shape) for t in [x] + W]
+    loss = lambda xs, Ws: float((oracle.srwm_forward(xs, *Ws)["out"] * go.numpy()).sum())
+    h = 1e-6
+    xp = x.numpy() + h * dirs[0]
+    xm = x.numpy() - h * dirs[0]
+    Wp = [w.numpy() + h * d for w, d in zip(W, dirs[1:])]
+    Wm = [w.numpy() - h * d for w, d in zip(W, dirs[1:])]
+    fd = (loss(xp, Wp) - loss(xm, Wm)) / (2 * h)
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    b = oracle.srwm_backward(x.numpy(), f, go.numpy())
+    an = sum((b[n] * d).sum() for n, d in
+             zip(("grad_x", "grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), dirs))
+    assert abs(fd - an) < 1e-7 * max(1.0, abs(an))
+
+
+def test_backward_is_linear_in_grad_out():
+    x, W, go = srwm_inputs(1, 2, 8, 6, seed=9, w_std=0.5)
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    go2 = torch.randn(go.shape, generator=torch.Generator().manual_seed(1), dtype=torch.float64)
+    a = oracle.srwm_backward(x.numpy(), f, go.numpy())
+    b = oracle.srwm_backward(x.numpy(), f, go2.numpy())
+    c = oracle.srwm_backward(x.numpy(), f, (2 * go - 3 * go2).numpy())
+    for n in ("grad_x", "grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"):
+        assert rel_err(c[n], 2 * a[n] - 3 * b[n]) < 1e-11
+
+
+# ---------------------------------------------------------- float32 flavour
+
+def test_f32_oracle_tracks_f64():
+    x, W, go = srwm_inputs(2, 4, 64, 16, seed=0, w_std=0.02)
+    f64 = oracle.srwm_forward(x.numpy(), *_np(W))
+    f32 = oracle.srwm_forward(x.numpy(), *_np(W), dtype=np.float32)
+    assert rel_err(f32["out"], f64["out"]) < 1e-5
+    b64 = oracle.srwm_backward(x.numpy(), f64, go.numpy())
+    b32 = oracle.srwm_backward(x.numpy(), f32, go.numpy(), dtype=np.float32)
+    for n in ("grad_x", "grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"):
+        assert rel_err(b32[n], b64[n]) < 1e-4, n
