@@ -1,0 +1,136 @@
+/*
+ * srwm_hip.h -- C ABI of libsrwm_hip.so: recurrent fast-weight kernels for
+ * AMD MI355X (gfx950), SRWM (self-referential weight matrix) and delta rule.
+ *
+ * Conventions shared by every entry point
+ *   - All pointers are DEVICE pointers on the calling thread's current HIP
+ *     device.  Nothing is allocated, freed or synchronised by the library.
+ *   - `stream` is a hipStream_t (NULL = the default stream).  Kernels are only
+ *     enqueued; the call returns immediately.
+ *   - N = batch, H = heads, L = time steps, E = key/query width (d_head),
+ *     M = value width.  One "sequence" is one (n, h) pair.
+ *   - "dense" tensors are row-major with no padding.  "strided" tensors come
+ *     with `int64_t s[3]` = element strides of the n, h and l axes; the last
+ *     axis must have stride 1 (the callers pass permute(1,2,0,3) views of
+ *     (L, N, H, d) storage, whose last axis is contiguous).
+ *   - Return value: 0 on success; negative SRWM_E* for an argument the library
+ *     rejects (nothing was launched); positive = the hipError_t of a failed
+ *     launch.  The library never throws and never calls exit/abort.
+ *   - Re-entrant: no mutable global state; safe from several host threads on
+ *     different streams/devices.
+ *   - `flags`: bitwise OR of SRWM_FLAG_*.
+ */
+#ifndef SRWM_HIP_H
+#define SRWM_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SRWM_API __attribute__((visibility("default")))
+
+#define SRWM_OK 0
+#define SRWM_EINVAL (-1)   /* null pointer, non-positive size, bad flag combination */
+#define SRWM_ESIZE (-2)    /* E / M not supported by any kernel (state does not fit in LDS) */
+#define SRWM_ESTRIDE (-3)  /* stride makes an access misaligned or overflows 32-bit indexing */
+
+/* backward: what the grad-state buffers hold on entry / exit */
+#define SRWM_GRAD_STATE_ZERO 0u   /* entry contents ignored (dL/dW_L = 0); exit: dL/dW_0 */
+#define SRWM_GRAD_STATE_IN 1u     /* entry: dL/dW_L; exit: dL/dW_0 (autograd-correct stateful op) */
+#define SRWM_GRAD_STATE_ACCUM 2u  /* entry: dL/dW_L = A; exit: A + dL/dW_0.  What the reference kernel
+                                     does (it initialises its gradient accumulator from the buffer,
+                                     self_ref_v0.cu:676-683, and atomically adds the result back into
+                                     it, :1213-1229); equal to ZERO when the buffers arrive zeroed. */
+#define SRWM_GRAD_STATE_MASK 3u
+#define SRWM_FLAG_GENERIC 16u     /* force the any-size LDS-resident kernel (testing / comparison) */
+
+/*
+ * SRWM forward.  Replaces self_ref_forward(), supervised_learning/self_ref_v0/
+ * self_ref_v0.cu:436-530 (kernel :24-432).  For t = 0..L-1, per sequence, with the
+ * state W = [W_y | W_q | W_k | w_b]  (E x (3E+4)):
+ *     [y | q~ | k~ | b~] = W^T x_t;  q = softmax(q~), k = softmax(k~), beta = sigmoid(b~)
+ *     diff = W^T (q - k);  W += k (x) (beta_blk * diff)
+ * and emits y_t plus the per-step vectors the backward needs.
+ *   x                strided [N,H,L,E]
+ *   Wy,Wq,Wk         dense [N,H,E,E], in: W_0, out: W_L (overwritten in place, as the
+ *   wb               dense [N,H,E,4]  reference does, :420-431)
+ *   q,k,ydiff,qdiff,kdiff,out   dense [N,H,L,E]  (overwritten; need not be zeroed)
+ *   beta,bdiff                  dense [N,H,L,4]
+ */
+SRWM_API int srwm_forward_f32(const float *x, const int64_t x_strides[3],
+                     float *Wy, float *Wq, float *Wk, float *wb,
+                     float *q, float *k, float *beta,
+                     float *ydiff, float *qdiff, float *kdiff, float *bdiff,
+                     float *out,
+                     int N, int H, int L, int E, unsigned flags, void *stream);
+
+/*
+ * SRWM backward.  Replaces self_ref_backward(), self_ref_v0.cu:1238-1341 (kernel
+ * :534-1234).  Walks t = L-1..0 starting from the final state, reverting each
+ * write (W_{t-1} = W_t - k_t (x) ins_t) while carrying dL/dW.
+ *   x, grad_out                       strided [N,H,L,E]
+ *   q,k,ydiff,qdiff,kdiff             dense   [N,H,L,E]  (as emitted by the forward)
+ *   beta,bdiff                        dense   [N,H,L,4]
+ *   Wy,Wq,Wk,wb                       dense, the FINAL state W_L; read only
+ *   grad_x                            dense [N,H,L,E], overwritten
+ *   gWy,gWq,gWk,gwb                   dense, same shapes as the state; see SRWM_GRAD_STATE_*
+ */
+SRWM_API int srwm_backward_f32(const float *x, const int64_t x_strides[3],
+                      const float *q, const float *k, const float *beta,
+                      const float *ydiff, const float *qdiff, const float *kdiff,
+                      const float *bdiff,
+                      const float *grad_out, const int64_t grad_out_strides[3],
+                      const float *Wy, const float *Wq, const float *Wk, const float *wb,
+                      float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb,
+                      int N, int H, int L, int E, unsigned flags, void *stream);
+
+/*
+ * Delta-rule forward.  Replaces fast_weight_forward(), supervised_learning/
+ * fast_weight/fast_weight_cuda.cu:182-240 (kernel :17-178).  Per sequence, W is E x M:
+ *     v_old = W^T k_t;  ins = beta_t (v_t - v_old);  W += k_t (x) ins;  out_t = W^T q_t
+ *   Q,K      strided [N,H,L,E];  V strided [N,H,L,M];  beta strided [N,H,L,1]
+ *   v_old, v_insert, out   dense [N,H,L,M] (overwritten)
+ *   W        dense [N,H,E,M], in: W_0, out: W_L (in place, as the reference, :171-177)
+ */
+SRWM_API int delta_forward_f32(const float *Q, const int64_t q_strides[3],
+                      const float *K, const int64_t k_strides[3],
+                      const float *V, const int64_t v_strides[3],
+                      const float *beta, const int64_t beta_strides[3],
+                      float *v_old, float *v_insert, float *W, float *out,
+                      int N, int H, int L, int E, int M, unsigned flags, void *stream);
+
+/*
+ * Delta-rule backward.  Replaces fast_weight_backward(), fast_weight_cuda.cu:564-664
+ * (kernels :244-393 and :397-560) with ONE reverse sweep and no global temporaries.
+ *   W        dense [N,H,E,M], in: W_L, out: W_0 (the reference's query/key sweep also
+ *            leaves the reverted state in the caller's tensor, :391)
+ *   gQ,gK    dense [N,H,L,E];  gV dense [N,H,L,M];  gbeta dense [N,H,L,1]  (overwritten)
+ *   gW       dense [N,H,E,M] or NULL.  With NULL the state gradient is dropped (the
+ *            reference returns None for it).  Otherwise see SRWM_GRAD_STATE_*.
+ */
+SRWM_API int delta_backward_f32(const float *Q, const int64_t q_strides[3],
+                       const float *K, const int64_t k_strides[3],
+                       const float *V, const int64_t v_strides[3],
+                       const float *beta, const int64_t beta_strides[3],
+                       const float *v_old, const float *v_insert,
+                       const float *grad_out, const int64_t grad_out_strides[3],
+                       float *W,
+                       float *gQ, float *gK, float *gV, float *gbeta, float *gW,
+                       int N, int H, int L, int E, int M, unsigned flags, void *stream);
+
+/* Largest E the SRWM entry points accept (forward / backward), and the largest
+ * E == M the delta entry points accept, on the current device. */
+SRWM_API int srwm_hip_limits(int *srwm_fwd_max_E, int *srwm_bwd_max_E, int *delta_max_EM);
+
+/* Human-readable text for a return code of the functions above. */
+SRWM_API const char *srwm_hip_strerror(int code);
+
+/* ABI version of this header (bumped on any signature change). */
+SRWM_API int srwm_hip_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SRWM_HIP_H */

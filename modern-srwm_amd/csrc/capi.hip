@@ -1,0 +1,165 @@
+// extern "C" boundary of libsrwm_hip.so (declared in include/srwm_hip.h): argument
+// checks, kernel selection, launch.  No allocation, no synchronisation, no global state.
+#include "../../include/srwm_hip.h"
+
+#include "common.h"
+
+namespace {
+
+using namespace fw;
+
+bool stride_ok(const int64_t s[3], int N, int H, int L, int width) {
+    if (!s) return false;
+    // float4 / float2 accesses start at multiples of the row, so rows must stay 16-byte
+    // aligned relative to the base whenever the row itself is (width % 4 == 0).
+    const int64_t ext = (int64_t)(N - 1) * (s[0] < 0 ? -s[0] : s[0]) +
+                        (int64_t)(H - 1) * (s[1] < 0 ? -s[1] : s[1]) +
+                        (int64_t)(L - 1) * (s[2] < 0 ? -s[2] : s[2]) + width;
+    return ext > 0 && ext < ((int64_t)1 << 40);
+}
+
+bool dims_ok(int N, int H, int L, int E) {
+    if (N <= 0 || H <= 0 || L <= 0 || E <= 0) return false;
+    return (int64_t)N * H < ((int64_t)1 << 31) && (int64_t)N * H * L * (int64_t)E < ((int64_t)1 << 40);
+}
+
+size_t lds_limit() {
+    int dev = 0, v = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 64 * 1024;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess || v <= 0)
+        return 64 * 1024;
+    return (size_t)v < kMaxLdsBytes ? (size_t)v : kMaxLdsBytes;
+}
+
+int max_E_for(size_t (*bytes)(int), size_t limit) {
+    int e = 0;
+    while (e < 4096 && bytes(e + 1) <= limit) ++e;
+    return e;
+}
+
+size_t delta_fwd_sq(int e) { return delta_fwd_generic_lds_bytes(e, e); }
+size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
+
+}  // namespace
+
+extern "C" {
+
+int srwm_hip_abi_version(void) { return 1; }
+
+const char *srwm_hip_strerror(int code) {
+    switch (code) {
+        case SRWM_OK: return "success";
+        case SRWM_EINVAL: return "invalid argument (null pointer, non-positive size or bad flags)";
+        case SRWM_ESIZE: return "head size not supported: the state does not fit in the CU's LDS";
+        case SRWM_ESTRIDE: return "unsupported stride";
+        default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown srwm_hip error";
+    }
+}
+
+int srwm_hip_limits(int *srwm_fwd_max_E, int *srwm_bwd_max_E, int *delta_max_EM) {
+    const size_t lim = lds_limit();
+    if (srwm_fwd_max_E) *srwm_fwd_max_E = max_E_for(srwm_fwd_generic_lds_bytes, lim);
+    if (srwm_bwd_max_E) *srwm_bwd_max_E = max_E_for(srwm_bwd_generic_lds_bytes, lim);
+    if (delta_max_EM) {
+        const int f = max_E_for(delta_fwd_sq, lim), b = max_E_for(delta_bwd_sq, lim);
+        *delta_max_EM = f < b ? f : b;
+    }
+    return SRWM_OK;
+}
+
+int srwm_forward_f32(const float *x, const int64_t xs[3], float *Wy, float *Wq, float *Wk, float *wb,
+                     float *q, float *k, float *beta, float *ydiff, float *qdiff, float *kdiff,
+                     float *bdiff, float *out, int N, int H, int L, int E, unsigned flags,
+                     void *stream) {
+    if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
+        !out || !xs)
+        return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || (flags & ~(SRWM_FLAG_GENERIC))) return SRWM_EINVAL;
+    if (!stride_ok(xs, N, H, L, E)) return SRWM_ESTRIDE;
+    SrwmFwdParams p{x, xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff,
+                    out, N, H, L, E};
+    hipStream_t s = (hipStream_t)stream;
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_srwm_fwd_tiled(p, s);
+        if (r >= 0) return r;
+    }
+    if (srwm_fwd_generic_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
+    return launch_srwm_fwd_generic(p, s);
+}
+
+int srwm_backward_f32(const float *x, const int64_t xs[3], const float *q, const float *k,
+                      const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
+                      const float *bdiff, const float *grad_out, const int64_t gs[3], const float *Wy,
+                      const float *Wq, const float *Wk, const float *wb, float *grad_x, float *gWy,
+                      float *gWq, float *gWk, float *gwb, int N, int H, int L, int E, unsigned flags,
+                      void *stream) {
+    if (!x || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff || !grad_out || !Wy || !Wq ||
+        !Wk || !wb || !grad_x || !gWy || !gWq || !gWk || !gwb || !xs || !gs)
+        return SRWM_EINVAL;
+    const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
+    if (!dims_ok(N, H, L, E) || mode == 3u || (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)))
+        return SRWM_EINVAL;
+    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, E)) return SRWM_ESTRIDE;
+    SrwmBwdParams p{x, xs[0], xs[1], xs[2], q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out,
+                    gs[0], gs[1], gs[2], Wy, Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, N, H, L, E, mode};
+    hipStream_t s = (hipStream_t)stream;
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_srwm_bwd_tiled(p, s);
+        if (r >= 0) return r;
+    }
+    if (srwm_bwd_generic_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
+    return launch_srwm_bwd_generic(p, s);
+}
+
+int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],
+                      const float *V, const int64_t vs[3], const float *beta, const int64_t bs[3],
+                      float *v_old, float *v_insert, float *W, float *out, int N, int H, int L, int E,
+                      int M, unsigned flags, void *stream) {
+    if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
+        return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~(SRWM_FLAG_GENERIC)))
+        return SRWM_EINVAL;
+    if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
+        !stride_ok(bs, N, H, L, 1))
+        return SRWM_ESTRIDE;
+    DeltaFwdParams p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
+                     {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
+                     N, H, L, E, M};
+    hipStream_t s = (hipStream_t)stream;
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_delta_fwd_tiled(p, s);
+        if (r >= 0) return r;
+    }
+    if (delta_fwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
+    return launch_delta_fwd_generic(p, s);
+}
+
+int delta_backward_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],
+                       const float *V, const int64_t vs[3], const float *beta, const int64_t bs[3],
+                       const float *v_old, const float *v_insert, const float *grad_out,
+                       const int64_t gs[3], float *W, float *gQ, float *gK, float *gV, float *gbeta,
+                       float *gW, int N, int H, int L, int E, int M, unsigned flags, void *stream) {
+    if (!Q || !K || !V || !beta || !v_old || !v_insert || !grad_out || !W || !gQ || !gK || !gV ||
+        !gbeta || !qs || !ks || !vs || !bs || !gs)
+        return SRWM_EINVAL;
+    const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u ||
+        (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)))
+        return SRWM_EINVAL;
+    if (!gW && mode != SRWM_GRAD_STATE_ZERO) return SRWM_EINVAL;
+    if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
+        !stride_ok(bs, N, H, L, 1) || !stride_ok(gs, N, H, L, M))
+        return SRWM_ESTRIDE;
+    DeltaBwdParams p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
+                     {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, grad_out,
+                     {gs[0], gs[1], gs[2]}, W, gQ, gK, gV, gbeta, gW, N, H, L, E, M, mode};
+    hipStream_t s = (hipStream_t)stream;
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_delta_bwd_tiled(p, s);
+        if (r >= 0) return r;
+    }
+    if (delta_bwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
+    return launch_delta_bwd_generic(p, s);
+}
+
+}  // extern "C"

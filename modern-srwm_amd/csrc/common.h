@@ -1,0 +1,85 @@
+// Shared declarations for the fast-weight kernels: parameter blocks passed by value to
+// the kernels, wave64 reduction helpers, and the launcher prototypes the C ABI dispatches to.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fw {
+
+constexpr int kWave = 64;
+
+struct SrwmFwdParams {
+    const float *x;
+    int64_t xs_n, xs_h, xs_l;
+    float *Wy, *Wq, *Wk, *wb;
+    float *q, *k, *beta, *ydiff, *qdiff, *kdiff, *bdiff, *out;
+    int N, H, L, E;
+};
+
+struct SrwmBwdParams {
+    const float *x;
+    int64_t xs_n, xs_h, xs_l;
+    const float *q, *k, *beta, *ydiff, *qdiff, *kdiff, *bdiff;
+    const float *go;
+    int64_t gs_n, gs_h, gs_l;
+    const float *Wy, *Wq, *Wk, *wb;
+    float *gx, *gWy, *gWq, *gWk, *gwb;
+    int N, H, L, E;
+    unsigned grad_state_mode;  // SRWM_GRAD_STATE_*
+};
+
+struct Strided3 {
+    int64_t n, h, l;
+};
+
+struct DeltaFwdParams {
+    const float *Q, *K, *V, *beta;
+    Strided3 qs, ks, vs, bs;
+    float *vold, *vins, *W, *out;
+    int N, H, L, E, M;
+};
+
+struct DeltaBwdParams {
+    const float *Q, *K, *V, *beta;
+    Strided3 qs, ks, vs, bs;
+    const float *vold, *vins, *go;
+    Strided3 gs;
+    float *W, *gQ, *gK, *gV, *gbeta, *gW;
+    int N, H, L, E, M;
+    unsigned grad_state_mode;
+};
+
+// ---- wave64 all-reduce helpers (every lane receives the result) -----------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// ---- launchers (each returns a hipError_t as int, 0 = launched) -----------------
+// LDS-resident kernels that accept any E (M) whose state fits in the CU's LDS.
+size_t srwm_fwd_generic_lds_bytes(int E);
+size_t srwm_bwd_generic_lds_bytes(int E);
+size_t delta_fwd_generic_lds_bytes(int E, int M);
+size_t delta_bwd_generic_lds_bytes(int E, int M);
+int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s);
+int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s);
+int launch_delta_fwd_generic(const DeltaFwdParams &p, hipStream_t s);
+int launch_delta_bwd_generic(const DeltaBwdParams &p, hipStream_t s);
+
+// Register-resident kernels for the head sizes that are compiled in; return -1
+// when E (E, M) has no specialisation so the caller can fall back to the generic kernel.
+int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s);
+int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s);
+int launch_delta_fwd_tiled(const DeltaFwdParams &p, hipStream_t s);
+int launch_delta_bwd_tiled(const DeltaBwdParams &p, hipStream_t s);
+
+constexpr size_t kMaxLdsBytes = 160 * 1024;  // gfx950: 160 KB of LDS per CU / workgroup
+
+}  // namespace fw

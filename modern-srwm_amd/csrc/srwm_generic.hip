@@ -1,0 +1,267 @@
+// SRWM forward / backward for ANY head size: one workgroup per (batch, head) sequence,
+// the packed state W = [W_y | W_q | W_k | w_b] (E x (3E+4), plus the gradient G in the
+// backward) resident in LDS for the whole sequence, one launch for all L steps.
+//
+// This is the fallback behind the register-resident kernels of srwm_tiled.hip: column
+// passes give one thread one column (bank-conflict free: consecutive lanes read
+// consecutive words), row passes give one wave one row and finish with a wave64
+// shuffle reduction.  No atomics anywhere; every output element is written once.
+//
+// Replaces self_ref_forward_kernel / self_ref_backward_kernel of the reference
+// (supervised_learning/self_ref_v0/self_ref_v0.cu:24-432, :534-1234).
+#include "common.h"
+
+namespace fw {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWave;
+
+__device__ __forceinline__ int padded_cols(int C) { return C | 1; }
+
+__device__ __forceinline__ void load_state(float *W, int Cp, const float *Wy, const float *Wq,
+                                           const float *Wk, const float *wb, int E, int tid) {
+    for (int i = tid; i < E * E; i += kThreads) {
+        const int e = i / E, m = i - e * E;
+        W[e * Cp + m] = Wy[i];
+        W[e * Cp + E + m] = Wq[i];
+        W[e * Cp + 2 * E + m] = Wk[i];
+    }
+    for (int i = tid; i < E * 4; i += kThreads) W[(i >> 2) * Cp + 3 * E + (i & 3)] = wb[i];
+}
+
+__global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParams p) {
+    extern __shared__ float smem[];
+    const int E = p.E, C = 3 * E + 4, Cp = padded_cols(C);
+    float *W = smem;         // [E][Cp]
+    float *xs = W + E * Cp;  // [E]
+    float *pre = xs + E;     // [C]: y | q | k | beta (activated in place)
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const int64_t sEE = seq * E * E, sE4 = seq * E * 4;
+
+    load_state(W, Cp, p.Wy + sEE, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, E, tid);
+    __syncthreads();
+
+    for (int t = 0; t < p.L; ++t) {
+        const float *xt = p.x + n * p.xs_n + h * p.xs_h + t * p.xs_l;
+        const int64_t o = (seq * p.L + t) * E, ob = (seq * p.L + t) * 4;
+        for (int e = tid; e < E; e += kThreads) xs[e] = xt[e];
+        __syncthreads();
+        // main readout: pre = W^T x
+        for (int m = tid; m < C; m += kThreads) {
+            float a = 0.f;
+            for (int e = 0; e < E; ++e) a = fmaf(W[e * Cp + m], xs[e], a);
+            pre[m] = a;
+            if (m < E) p.out[o + m] = a;
+        }
+        __syncthreads();
+        // activations: wave 0 -> softmax(q~), wave 1 -> softmax(k~), wave 2 -> sigmoid(b~)
+        if (wave < 2) {
+            float *v = pre + E + wave * E;
+            float mx = -INFINITY;
+            for (int i = lane; i < E; i += kWave) mx = fmaxf(mx, v[i]);
+            mx = wave_max(mx);
+            float s = 0.f;
+            for (int i = lane; i < E; i += kWave) {
+                const float ex = expf(v[i] - mx);
+                v[i] = ex;
+                s += ex;
+            }
+            s = wave_sum(s);
+            float *dst = (wave == 0 ? p.q : p.k) + o;
+            for (int i = lane; i < E; i += kWave) {
+                const float r = v[i] / s;
+                v[i] = r;
+                dst[i] = r;
+            }
+        } else if (wave == 2 && lane < 4) {
+            const float b = 1.f / (1.f + expf(-pre[3 * E + lane]));
+            pre[3 * E + lane] = b;
+            p.beta[ob + lane] = b;
+        }
+        __syncthreads();
+        // diff = W^T (q - k), then the rank-1 write of the thread's own column
+        for (int m = tid; m < C; m += kThreads) {
+            float a = 0.f;
+            for (int e = 0; e < E; ++e) a = fmaf(W[e * Cp + m], pre[E + e] - pre[2 * E + e], a);
+            const int blk = m < 3 * E ? m / E : 3;
+            if (blk == 0) p.ydiff[o + m] = a;
+            else if (blk == 1) p.qdiff[o + m - E] = a;
+            else if (blk == 2) p.kdiff[o + m - 2 * E] = a;
+            else p.bdiff[ob + m - 3 * E] = a;
+            const float ins = pre[3 * E + blk] * a;
+            for (int e = 0; e < E; ++e) W[e * Cp + m] = fmaf(pre[2 * E + e], ins, W[e * Cp + m]);
+        }
+        __syncthreads();
+    }
+
+    for (int i = tid; i < E * E; i += kThreads) {
+        const int e = i / E, m = i - e * E;
+        p.Wy[sEE + i] = W[e * Cp + m];
+        p.Wq[sEE + i] = W[e * Cp + E + m];
+        p.Wk[sEE + i] = W[e * Cp + 2 * E + m];
+    }
+    for (int i = tid; i < E * 4; i += kThreads) p.wb[sE4 + i] = W[(i >> 2) * Cp + 3 * E + (i & 3)];
+}
+
+__global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParams p) {
+    extern __shared__ float smem[];
+    const int E = p.E, C = 3 * E + 4, Cp = padded_cols(C);
+    float *W = smem;             // [E][Cp]  state, reverted step by step
+    float *G = W + E * Cp;       // [E][Cp]  dL/dW
+    float *xs = G + E * Cp;      // [E]
+    float *qs = xs + E;          // [E]
+    float *ks = qs + E;          // [E]
+    float *gq = ks + E;          // [E]
+    float *gk = gq + E;          // [E]
+    float *diff = gk + E;        // [C]
+    float *ins = diff + C;       // [C]
+    float *gdiff = ins + C;      // [C]
+    float *gpre = gdiff + C;     // [C]
+    float *prod = gpre + C;      // [C]  gins * diff, summed per block for the beta gradient
+    float *bt = prod + C;        // [4]
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const int64_t sEE = seq * E * E, sE4 = seq * E * 4;
+
+    load_state(W, Cp, p.Wy + sEE, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, E, tid);
+    if (p.grad_state_mode == 0u) {
+        for (int i = tid; i < E * Cp; i += kThreads) G[i] = 0.f;
+    } else {
+        load_state(G, Cp, p.gWy + sEE, p.gWq + sEE, p.gWk + sEE, p.gwb + sE4, E, tid);
+    }
+    __syncthreads();
+
+    for (int t = p.L - 1; t >= 0; --t) {
+        const float *xt = p.x + n * p.xs_n + h * p.xs_h + t * p.xs_l;
+        const float *got = p.go + n * p.gs_n + h * p.gs_h + t * p.gs_l;
+        const int64_t o = (seq * p.L + t) * E, ob = (seq * p.L + t) * 4;
+        for (int e = tid; e < E; e += kThreads) {
+            xs[e] = xt[e];
+            qs[e] = p.q[o + e];
+            ks[e] = p.k[o + e];
+            diff[e] = p.ydiff[o + e];
+            diff[E + e] = p.qdiff[o + e];
+            diff[2 * E + e] = p.kdiff[o + e];
+            gpre[e] = got[e];
+        }
+        if (tid < 4) {
+            bt[tid] = p.beta[ob + tid];
+            diff[3 * E + tid] = p.bdiff[ob + tid];
+        }
+        __syncthreads();
+        // column pass: revert W, g_ins = G^T k
+        for (int m = tid; m < C; m += kThreads) {
+            const float b = bt[m < 3 * E ? m / E : 3];
+            const float im = b * diff[m];
+            float gi = 0.f;
+            for (int e = 0; e < E; ++e) {
+                const float ke = ks[e];
+                W[e * Cp + m] = fmaf(-ke, im, W[e * Cp + m]);
+                gi = fmaf(G[e * Cp + m], ke, gi);
+            }
+            ins[m] = im;
+            gdiff[m] = b * gi;
+            prod[m] = gi * diff[m];
+        }
+        __syncthreads();
+        // row pass: gk = G ins - W_{t-1} g_diff ; gq = W_{t-1} g_diff
+        for (int e = wave; e < E; e += kWaves) {
+            float a = 0.f, u = 0.f;
+            for (int m = lane; m < C; m += kWave) {
+                a = fmaf(G[e * Cp + m], ins[m], a);
+                u = fmaf(W[e * Cp + m], gdiff[m], u);
+            }
+            a = wave_sum(a);
+            u = wave_sum(u);
+            if (lane == 0) {
+                gq[e] = u;
+                gk[e] = a - u;
+            }
+        }
+        __syncthreads();
+        // softmax / sigmoid backward -> gradient of the main readout
+        if (wave < 2) {
+            const float *g = wave == 0 ? gq : gk;
+            const float *s = wave == 0 ? qs : ks;
+            float d = 0.f;
+            for (int i = lane; i < E; i += kWave) d = fmaf(g[i], s[i], d);
+            d = wave_sum(d);
+            for (int i = lane; i < E; i += kWave) gpre[(1 + wave) * E + i] = s[i] * (g[i] - d);
+        } else if (wave == 2) {
+            for (int j = 0; j < 4; ++j) {
+                const int lo = j * E, hi = j < 3 ? lo + E : lo + 4;
+                float a = 0.f;
+                for (int m = lo + lane; m < hi; m += kWave) a += prod[m];
+                a = wave_sum(a);
+                if (lane == 0) gpre[3 * E + j] = a * bt[j] * (1.f - bt[j]);
+            }
+        }
+        __syncthreads();
+        // row pass: grad_x = W_{t-1} g_pre
+        for (int e = wave; e < E; e += kWaves) {
+            float a = 0.f;
+            for (int m = lane; m < C; m += kWave) a = fmaf(W[e * Cp + m], gpre[m], a);
+            a = wave_sum(a);
+            if (lane == 0) p.gx[o + e] = a;
+        }
+        // column pass: G += (q - k) (x) g_diff + x (x) g_pre
+        for (int m = tid; m < C; m += kThreads) {
+            const float gd = gdiff[m], gp = gpre[m];
+            for (int e = 0; e < E; ++e)
+                G[e * Cp + m] += fmaf(qs[e] - ks[e], gd, xs[e] * gp);
+        }
+        __syncthreads();
+    }
+
+    const bool accum = p.grad_state_mode == 2u;
+    for (int i = tid; i < E * E; i += kThreads) {
+        const int e = i / E, m = i - e * E;
+        const float gy = G[e * Cp + m], gqv = G[e * Cp + E + m], gkv = G[e * Cp + 2 * E + m];
+        p.gWy[sEE + i] = accum ? p.gWy[sEE + i] + gy : gy;
+        p.gWq[sEE + i] = accum ? p.gWq[sEE + i] + gqv : gqv;
+        p.gWk[sEE + i] = accum ? p.gWk[sEE + i] + gkv : gkv;
+    }
+    for (int i = tid; i < E * 4; i += kThreads) {
+        const float g = G[(i >> 2) * Cp + 3 * E + (i & 3)];
+        p.gwb[sE4 + i] = accum ? p.gwb[sE4 + i] + g : g;
+    }
+}
+
+}  // namespace
+
+size_t srwm_fwd_generic_lds_bytes(int E) {
+    const size_t C = 3 * (size_t)E + 4, Cp = C | 1;
+    return sizeof(float) * (E * Cp + E + C);
+}
+
+size_t srwm_bwd_generic_lds_bytes(int E) {
+    const size_t C = 3 * (size_t)E + 4, Cp = C | 1;
+    return sizeof(float) * (2 * E * Cp + 5 * E + 5 * C + 4);
+}
+
+int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s) {
+    const size_t lds = srwm_fwd_generic_lds_bytes(p.E);
+    hipError_t err = hipFuncSetAttribute((const void *)srwm_fwd_generic_kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (err != hipSuccess) return (int)err;
+    hipLaunchKernelGGL(srwm_fwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
+    return (int)hipGetLastError();
+}
+
+int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s) {
+    const size_t lds = srwm_bwd_generic_lds_bytes(p.E);
+    hipError_t err = hipFuncSetAttribute((const void *)srwm_bwd_generic_kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (err != hipSuccess) return (int)err;
+    hipLaunchKernelGGL(srwm_bwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
+    return (int)hipGetLastError();
+}
+
+}  // namespace fw

@@ -1,0 +1,53 @@
+"""Delta-rule fast weight operator, drop-in for the reference's `fast_weight` package
+(supervised_learning/fast_weight/__init__.py:26-100): same autograd Function, same call
+signature, same in-place semantics -- backed by libsrwm_hip.so.
+
+    out = fast_weight_delta(Q, K, V, beta, W)
+
+Q, K: (N, H, L, E); V: (N, H, L, M); beta: (N, H, L, 1) (already sigmoid-ed); W: (N, H, E, M);
+float32 on the GPU.  W is OVERWRITTEN with the memory after the last step; the backward
+starts from it and leaves it reverted to its initial value, like the reference's kernels.
+No gradient is returned for W (the reference returns None).
+"""
+import torch
+
+import srwm_hip
+
+causal_dot_product_cuda = srwm_hip.fast_weight_forward
+causal_dot_backward_cuda = srwm_hip.fast_weight_backward
+
+
+class DeltaFastWeight(torch.autograd.Function):
+    """Fast weight using the delta update rule."""
+    dot = {"cuda": causal_dot_product_cuda}
+    dot_backward = {"cuda": causal_dot_backward_cuda}
+
+    @staticmethod
+    def forward(ctx, Q, K, V, beta, W):
+        for t in (Q, K, V, beta, W):
+            assert t.device.type != "cpu"
+        device = Q.device
+        N, H, L, E = Q.shape
+        _, _, _, M = V.shape
+        out = torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
+        V_old = torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
+        V_insert = torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
+        DeltaFastWeight.dot[device.type](Q.data, K.data, V.data, beta.data, V_old, V_insert, W, out)
+        ctx.save_for_backward(Q, K, V, beta, V_old, V_insert, W)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        Q, K, V, beta, V_old, V_insert, W = ctx.saved_tensors
+        grad_Q = torch.empty(Q.shape, device=Q.device, dtype=Q.dtype)
+        grad_K = torch.empty(K.shape, device=Q.device, dtype=Q.dtype)
+        grad_V = torch.empty(V.shape, device=Q.device, dtype=Q.dtype)
+        grad_beta = torch.empty(beta.shape, device=Q.device, dtype=Q.dtype)
+        DeltaFastWeight.dot_backward[Q.device.type](
+            Q.data, K.data, V.data, beta.data, V_old.data, V_insert.data, grad_out, W.data,
+            grad_Q, grad_K, grad_V, grad_beta)
+        return grad_Q, grad_K, grad_V, grad_beta, None
+
+
+# Alias the autograd functions to python style snake case naming
+fast_weight_delta = DeltaFastWeight.apply

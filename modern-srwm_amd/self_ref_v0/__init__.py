@@ -1,0 +1,101 @@
+"""SRWM operator, drop-in for the reference's `self_ref_v0` package
+(supervised_learning/self_ref_v0/__init__.py:34-217): same autograd Function classes,
+same call signatures, same in-place final-state semantics -- backed by libsrwm_hip.so.
+
+    out = self_ref_v0(x, W_y, W_q, W_k, w_b)
+    out, W_y, W_q, W_k, w_b = stateful_self_ref_v0(x, W_y, W_q, W_k, w_b)
+
+x: (N, H, L, E); W_y, W_q, W_k: (N, H, E, E); w_b: (N, H, E, 4); float32 on the GPU.
+The weight tensors are OVERWRITTEN with the state after the last step (the layers read
+them back as the carried state); the backward starts from that mutated tensor.
+"""
+import torch
+
+import srwm_hip
+
+self_ref_fwd_cuda = srwm_hip.self_ref_forward
+self_ref_bwd_cuda = srwm_hip.self_ref_backward
+
+# The reference's stateful backward returns (incoming grad) + (propagated grad) for the
+# weight tensors because its kernel both starts from and accumulates into the same buffer
+# (self_ref_v0/__init__.py:182-212, self_ref_v0.cu:676-683, :1213-1229).  The default here
+# is the gradient autograd of the recurrence gives; set this to True to reproduce the
+# reference's values exactly.
+REFERENCE_STATEFUL_GRAD = False
+
+
+def _check_shapes(x, W_y, W_q, W_k, w_b):
+    N, H, L, E = x.shape
+    assert W_y.shape == (N, H, E, E), "Reshape/unsqueeze if needed."
+    assert W_q.shape == (N, H, E, E), "Reshape/unsqueeze if needed."
+    assert W_k.shape == (N, H, E, E), "Reshape/unsqueeze if needed."
+    assert w_b.shape == (N, H, E, 4), "Reshape/unsqueeze if needed."
+    return N, H, L, E
+
+
+def _forward(dot, ctx, x, W_y, W_q, W_k, w_b):
+    device = x.device
+    N, H, L, E = _check_shapes(x, W_y, W_q, W_k, w_b)
+    fn = dot[device.type]
+    # every element is written by the kernel, so no zero-fill is needed
+    big = lambda: torch.empty((N, H, L, E), device=device, dtype=x.dtype)
+    small = lambda: torch.empty((N, H, L, 4), device=device, dtype=x.dtype)
+    out = big()
+    q_main, k_main, beta_main = big(), big(), small()
+    y_diff, q_diff, k_diff, beta_diff = big(), big(), big(), small()
+    fn(x, W_y, W_q, W_k, w_b, q_main, k_main, beta_main, y_diff, q_diff, k_diff, beta_diff, out)
+    ctx.save_for_backward(x, q_main, k_main, beta_main, y_diff, q_diff, k_diff, beta_diff,
+                          W_y, W_q, W_k, w_b)
+    return out
+
+
+class SelfRefv0(torch.autograd.Function):
+
+    dot = {"cuda": self_ref_fwd_cuda}
+    dot_backward = {"cuda": self_ref_bwd_cuda}
+
+    @staticmethod
+    def forward(ctx, x, W_y, W_q, W_k, w_b):
+        return _forward(SelfRefv0.dot, ctx, x, W_y, W_q, W_k, w_b)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, W_y, W_q, W_k, w_b) = ctx.saved_tensors
+        grad_x = torch.empty(x.shape, device=x.device, dtype=x.dtype)
+        grad_W_y = torch.empty_like(W_y, memory_format=torch.contiguous_format)
+        grad_W_q = torch.empty_like(W_q, memory_format=torch.contiguous_format)
+        grad_W_k = torch.empty_like(W_k, memory_format=torch.contiguous_format)
+        grad_w_b = torch.empty_like(w_b, memory_format=torch.contiguous_format)
+        SelfRefv0.dot_backward[x.device.type](
+            x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out, W_y, W_q, W_k, w_b,
+            grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b, flags=srwm_hip.GRAD_STATE_ZERO)
+        return grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b
+
+
+class StatefulSelfRefv0(torch.autograd.Function):
+
+    dot = {"cuda": self_ref_fwd_cuda}
+    dot_backward = {"cuda": self_ref_bwd_cuda}
+
+    @staticmethod
+    def forward(ctx, x, W_y, W_q, W_k, w_b):
+        out = _forward(StatefulSelfRefv0.dot, ctx, x, W_y, W_q, W_k, w_b)
+        return out, W_y, W_q, W_k, w_b
+
+    @staticmethod
+    def backward(ctx, grad_out, grad_W_y, grad_W_q, grad_W_k, grad_w_b):
+        (x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, W_y, W_q, W_k, w_b) = ctx.saved_tensors
+        grad_x = torch.empty(x.shape, device=x.device, dtype=x.dtype)
+        # work on private contiguous copies: autograd may hand the same buffers elsewhere
+        gs = [g.clone(memory_format=torch.contiguous_format) for g in
+              (grad_W_y, grad_W_q, grad_W_k, grad_w_b)]
+        mode = srwm_hip.GRAD_STATE_ACCUM if REFERENCE_STATEFUL_GRAD else srwm_hip.GRAD_STATE_IN
+        StatefulSelfRefv0.dot_backward[x.device.type](
+            x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out, W_y, W_q, W_k, w_b,
+            grad_x, *gs, flags=mode)
+        return (grad_x, *gs)
+
+
+# Alias the autograd functions to python style snake case naming
+self_ref_v0 = SelfRefv0.apply
+stateful_self_ref_v0 = StatefulSelfRefv0.apply

@@ -1,0 +1,254 @@
+"""Host side of libsrwm_hip.so: loads the C-ABI library with ctypes and exposes the four
+extension-level functions with the positional tensor lists of the reference's pybind
+modules (supervised_learning/self_ref_v0/self_ref_v0.cu:1344-1356,
+supervised_learning/fast_weight/fast_weight_cuda.cu:667-679):
+
+    self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out)
+    self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out,
+                      W_y, W_q, W_k, w_b, grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b)
+    fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out)
+    fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv,
+                         grad_q, grad_k, grad_v, grad_beta)
+
+PyTorch is used for device memory and streams only.  There is no CPU path: a missing
+library, a CPU tensor or a non-float32 tensor raises.
+"""
+import ctypes
+import os
+import subprocess
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_PKG = os.path.dirname(_HERE)
+LIB_PATH = os.path.join(_PKG, "lib", "libsrwm_hip.so")
+CSRC = os.path.join(_PKG, "csrc")
+
+# flags of include/srwm_hip.h
+GRAD_STATE_ZERO = 0
+GRAD_STATE_IN = 1
+GRAD_STATE_ACCUM = 2
+FLAG_GENERIC = 16
+
+ABI_VERSION = 1
+
+_lib = None
+
+_F = ctypes.c_void_p      # device float*
+_S = ctypes.POINTER(ctypes.c_int64)
+_I = ctypes.c_int
+_U = ctypes.c_uint
+
+_SIGNATURES = {
+    "srwm_forward_f32": [_F, _S] + [_F] * 12 + [_I] * 4 + [_U, ctypes.c_void_p],
+    "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
+    "delta_forward_f32": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_backward_f32": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
+}
+
+
+def build(verbose=False):
+    """Compile libsrwm_hip.so for gfx950 with hipcc (always recompiles)."""
+    out = None if verbose else subprocess.DEVNULL
+    subprocess.check_call(["make", "-C", CSRC, "-B", "-j8"], stdout=out, stderr=out)
+    return LIB_PATH
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built -- there is no fallback."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C {CSRC}` "
+                "(or __graft_entry__.build()); the HIP kernels have no CPU/PyTorch fallback")
+        L = ctypes.CDLL(LIB_PATH)
+        L.srwm_hip_abi_version.restype = _I
+        if L.srwm_hip_abi_version() != ABI_VERSION:
+            raise RuntimeError("libsrwm_hip.so ABI version mismatch; rebuild the library")
+        for name, args in _SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.argtypes = args
+            fn.restype = _I
+        L.srwm_hip_strerror.restype = ctypes.c_char_p
+        L.srwm_hip_strerror.argtypes = [_I]
+        L.srwm_hip_limits.argtypes = [ctypes.POINTER(_I)] * 3
+        L.srwm_hip_limits.restype = _I
+        _lib = L
+    return _lib
+
+
+def limits(device=None):
+    """(max E of SRWM forward, max E of SRWM backward, max E == M of the delta rule)."""
+    a, b, c = _I(), _I(), _I()
+    with torch.cuda.device(device):
+        lib().srwm_hip_limits(ctypes.byref(a), ctypes.byref(b), ctypes.byref(c))
+    return a.value, b.value, c.value
+
+
+def _check(code, what):
+    if code != 0:
+        msg = lib().srwm_hip_strerror(code).decode()
+        raise RuntimeError(f"{what} failed with code {code}: {msg}")
+
+
+def _require(t, name, shape=None):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError(f"{name} must be a torch.Tensor")
+    if t.device.type != "cuda":
+        raise RuntimeError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
+    if t.dtype != torch.float32:
+        raise TypeError(f"{name} must be float32 (got {t.dtype})")
+    if shape is not None and tuple(t.shape) != tuple(shape):
+        raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _strided(t):
+    """A tensor the kernels can read through (n, h, l) strides: last axis contiguous, rows
+    16-byte aligned.  Anything else is copied."""
+    ok = t.stride(-1) == 1 or t.shape[-1] == 1
+    if ok and t.shape[-1] % 4 == 0:
+        ok = t.data_ptr() % 16 == 0 and all(s % 4 == 0 for s in t.stride()[:3])
+    if not ok:
+        t = t.contiguous()
+    return t, (ctypes.c_int64 * 3)(*t.stride()[:3])
+
+
+class _Dense:
+    """Context for tensors the kernels address densely: contiguous ones pass through; others
+    are staged through a contiguous copy that is written back on exit when `writeback`."""
+
+    def __init__(self, tensors, writeback):
+        self.orig = list(tensors)
+        self.writeback = writeback
+        self.work = [t if t.is_contiguous() else t.contiguous() for t in self.orig]
+
+    def __enter__(self):
+        return self.work
+
+    def __exit__(self, *exc):
+        if self.writeback and exc[0] is None:
+            for o, w in zip(self.orig, self.work):
+                if o is not w:
+                    o.copy_(w)
+        return False
+
+
+def _stream(device):
+    return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out,
+                     flags=0):
+    """SRWM forward over the whole sequence.  W_y, W_q, W_k, w_b are overwritten with the
+    final state; q ... out are overwritten with the per-step vectors."""
+    _require(x, "x")
+    N, H, L, E = x.shape
+    for t, nm in ((W_y, "W_y"), (W_q, "W_q"), (W_k, "W_k")):
+        _require(t, nm, (N, H, E, E))
+    _require(w_b, "w_b", (N, H, E, 4))
+    for t, nm in ((q, "q"), (k, "k"), (y_diff, "y_diff"), (q_diff, "q_diff"), (k_diff, "k_diff"),
+                  (out, "out")):
+        _require(t, nm, (N, H, L, E))
+    _require(beta, "beta", (N, H, L, 4))
+    _require(beta_diff, "beta_diff", (N, H, L, 4))
+    if x.numel() == 0:
+        return
+    xs, xstr = _strided(x)
+    with torch.cuda.device(x.device), \
+            _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out], True) as d:
+        code = lib().srwm_forward_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
+                                      _stream(x.device))
+    _check(code, "srwm_forward_f32")
+
+
+def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out,
+                      W_y, W_q, W_k, w_b, grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b,
+                      flags=GRAD_STATE_ACCUM):
+    """SRWM backward.  W_* must hold the final state the forward left behind.  By default
+    behaves like the reference extension function: the grad_W buffers are read as the
+    gradient w.r.t. the final state and the result is added to them (identical to a plain
+    overwrite when they arrive zero-filled, which is how SelfRefv0.backward calls it)."""
+    _require(x, "x")
+    N, H, L, E = x.shape
+    for t, nm in ((q, "q"), (k, "k"), (y_diff, "y_diff"), (q_diff, "q_diff"), (k_diff, "k_diff"),
+                  (grad_out, "grad_out"), (grad_x, "grad_x")):
+        _require(t, nm, (N, H, L, E))
+    _require(beta, "beta", (N, H, L, 4))
+    _require(beta_diff, "beta_diff", (N, H, L, 4))
+    for t, nm in ((W_y, "W_y"), (W_q, "W_q"), (W_k, "W_k"), (grad_W_y, "grad_W_y"),
+                  (grad_W_q, "grad_W_q"), (grad_W_k, "grad_W_k")):
+        _require(t, nm, (N, H, E, E))
+    _require(w_b, "w_b", (N, H, E, 4))
+    _require(grad_w_b, "grad_w_b", (N, H, E, 4))
+    if x.numel() == 0:
+        return
+    xs, xstr = _strided(x)
+    gos, gstr = _strided(grad_out)
+    with torch.cuda.device(x.device), \
+            _Dense([q, k, beta, y_diff, q_diff, k_diff, beta_diff], False) as sv, \
+            _Dense([W_y, W_q, W_k, w_b], False) as st, \
+            _Dense([grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b], True) as gr:
+        code = lib().srwm_backward_f32(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
+                                       *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
+                                       N, H, L, E, flags, _stream(x.device))
+    _check(code, "srwm_backward_f32")
+
+
+def fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=0):
+    """Delta-rule forward.  kv ([N,H,E,M]) is overwritten with the final memory."""
+    _require(q, "q")
+    N, H, L, E = q.shape
+    _require(k, "k", (N, H, L, E))
+    _require(v, "v")
+    M = v.shape[-1]
+    _require(v, "v", (N, H, L, M))
+    _require(beta, "beta", (N, H, L, 1))
+    for t, nm in ((v_old, "v_old"), (v_insert, "v_insert"), (out, "out")):
+        _require(t, nm, (N, H, L, M))
+    _require(kv, "kv", (N, H, E, M))
+    if q.numel() == 0 or v.numel() == 0:
+        return
+    (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr) = (_strided(t) for t in (q, k, v, beta))
+    with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv, out], True) as d:
+        code = lib().delta_forward_f32(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
+                                       *[_ptr(t) for t in d], N, H, L, E, M, flags,
+                                       _stream(q.device))
+    _check(code, "delta_forward_f32")
+
+
+def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v,
+                         grad_beta, grad_kv=None, flags=GRAD_STATE_ZERO):
+    """Delta-rule backward.  kv must hold the final memory and is reverted to the initial
+    one.  grad_kv (optional, beyond the reference's list): gradient of the memory, see
+    the SRWM_GRAD_STATE_* flags."""
+    _require(q, "q")
+    N, H, L, E = q.shape
+    _require(k, "k", (N, H, L, E))
+    _require(v, "v")
+    M = v.shape[-1]
+    _require(beta, "beta", (N, H, L, 1))
+    for t, nm in ((v_old, "v_old"), (v_insert, "v_insert"), (grad_out, "grad_out"), (grad_v, "grad_v")):
+        _require(t, nm, (N, H, L, M))
+    _require(kv, "kv", (N, H, E, M))
+    _require(grad_q, "grad_q", (N, H, L, E))
+    _require(grad_k, "grad_k", (N, H, L, E))
+    _require(grad_beta, "grad_beta", (N, H, L, 1))
+    if grad_kv is not None:
+        _require(grad_kv, "grad_kv", (N, H, E, M))
+    if q.numel() == 0 or v.numel() == 0:
+        return
+    (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr), (gos, gstr) = (
+        _strided(t) for t in (q, k, v, beta, grad_out))
+    outs = [kv, grad_q, grad_k, grad_v, grad_beta] + ([grad_kv] if grad_kv is not None else [])
+    with torch.cuda.device(q.device), _Dense([v_old, v_insert], False) as sv, _Dense(outs, True) as d:
+        gkv = _ptr(d[5]) if grad_kv is not None else ctypes.c_void_p(None)
+        code = lib().delta_backward_f32(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
+                                        _ptr(sv[0]), _ptr(sv[1]), _ptr(gos), gstr,
+                                        *[_ptr(t) for t in d[:5]], gkv, N, H, L, E, M, flags,
+                                        _stream(q.device))
+    _check(code, "delta_backward_f32")

@@ -1,0 +1,81 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol that
+include/srwm_hip.h declares, and the host layer refuses what it must refuse.  No kernel is
+launched here."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "srwm_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    return re.findall(r"^SRWM_API\s+(?:const\s+)?\w+\s*\*?\s*(\w+)\s*\(", text, flags=re.M)
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_symbols()
+    for must in ("srwm_forward_f32", "srwm_backward_f32", "delta_forward_f32", "delta_backward_f32",
+                 "srwm_hip_limits", "srwm_hip_strerror", "srwm_hip_abi_version"):
+        assert must in names
+
+
+def test_library_exports_every_declared_symbol():
+    import srwm_hip
+    assert os.path.exists(srwm_hip.LIB_PATH), "build the library first (make -C modern-srwm_amd/csrc)"
+    L = ctypes.CDLL(srwm_hip.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(L, name), name
+    assert srwm_hip.lib().srwm_hip_abi_version() == srwm_hip.ABI_VERSION
+
+
+def test_error_strings():
+    import srwm_hip
+    L = srwm_hip.lib()
+    assert b"success" in L.srwm_hip_strerror(0)
+    assert b"invalid" in L.srwm_hip_strerror(-1)
+    assert b"not supported" in L.srwm_hip_strerror(-2)
+    assert b"stride" in L.srwm_hip_strerror(-3)
+
+
+def test_cpu_tensors_are_refused_loudly():
+    """There is no CPU or PyTorch fallback behind the operators."""
+    import srwm_hip
+    from self_ref_v0 import self_ref_v0
+    from fast_weight import fast_weight_delta
+    x = torch.zeros(1, 1, 2, 8)
+    W = [torch.zeros(1, 1, 8, 8) for _ in range(3)] + [torch.zeros(1, 1, 8, 4)]
+    with pytest.raises(KeyError):          # same failure as the reference: no "cpu" entry in .dot
+        self_ref_v0(x, *W)
+    outs = [torch.zeros(1, 1, 2, 8)] * 2 + [torch.zeros(1, 1, 2, 4)] + [torch.zeros(1, 1, 2, 8)] * 3 + \
+           [torch.zeros(1, 1, 2, 4), torch.zeros(1, 1, 2, 8)]
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        srwm_hip.self_ref_forward(x, *W, *outs)
+    q = torch.zeros(1, 1, 2, 8)
+    with pytest.raises((RuntimeError, AssertionError)):
+        fast_weight_delta(q, q, q, torch.zeros(1, 1, 2, 1), torch.zeros(1, 1, 8, 8))
+
+
+def test_shape_asserts_match_the_reference_wording():
+    from self_ref_v0 import SelfRefv0, StatefulSelfRefv0, self_ref_v0, stateful_self_ref_v0
+    x = torch.zeros(2, 3, 4, 8)
+    good = torch.zeros(2, 3, 8, 8)
+    with pytest.raises(AssertionError, match="Reshape/unsqueeze if needed."):
+        self_ref_v0(x, good, good, good, torch.zeros(2, 3, 8, 3))
+    with pytest.raises(AssertionError, match="Reshape/unsqueeze if needed."):
+        stateful_self_ref_v0(x, good[:1], good, good, torch.zeros(2, 3, 8, 4))
+    assert set(SelfRefv0.dot) == {"cuda"} and set(StatefulSelfRefv0.dot_backward) == {"cuda"}
+
+
+def test_host_layer_uses_no_oracle_and_no_torch_math():
+    """The product path must not import the oracle (it is test infrastructure)."""
+    pkg = os.path.join(ROOT, "modern-srwm_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text, f

@@ -1,0 +1,143 @@
+"""GPU parity of the delta-rule kernels (through the C ABI) against the fp64 CPU oracle.
+
+Tolerance: 1e-5 relative (max|a-b| / max|b| per tensor), fp32 kernels vs the fp64 oracle.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import delta_inputs, rel_err
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+KERNELS = [pytest.param(0, id="default"), pytest.param(16, id="generic")]
+
+
+def _dev():
+    return torch.device("cuda:0")
+
+
+def run_hip(q, k, v, beta, W0, go, flags=0, grad_state=None, want_grad_W=False):
+    import srwm_hip
+    dev = _dev()
+    N, H, L, E = q.shape
+    M = v.shape[-1]
+    qd, kd, vd, bd, god = (t.to(dev, torch.float32) for t in (q, k, v, beta, go))
+    W = W0.to(dev, torch.float32).contiguous()
+    nan = lambda *s: torch.full(s, float("nan"), device=dev)
+    vold, vins, out = nan(N, H, L, M), nan(N, H, L, M), nan(N, H, L, M)
+    srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out, flags=flags)
+    f = dict(out=out, v_old=vold, v_insert=vins, W=W.clone())
+    gq, gk, gv, gb = nan(N, H, L, E), nan(N, H, L, E), nan(N, H, L, M), nan(N, H, L, 1)
+    gW, mode = None, srwm_hip.GRAD_STATE_ZERO
+    if grad_state is not None:
+        gW, mode = grad_state.to(dev, torch.float32).contiguous(), srwm_hip.GRAD_STATE_IN
+    elif want_grad_W:
+        gW = nan(N, H, E, M)
+    srwm_hip.fast_weight_backward(qd, kd, vd, bd, vold, vins, god, W, gq, gk, gv, gb, grad_kv=gW,
+                                  flags=flags | mode)
+    torch.cuda.synchronize()
+    b = dict(grad_Q=gq, grad_K=gk, grad_V=gv, grad_beta=gb, W0=W)
+    if gW is not None:
+        b["grad_W"] = gW
+    return f, b
+
+
+@pytest.mark.parametrize("flags", KERNELS)
+@pytest.mark.parametrize("shape,qk,w0", [
+    ((3, 5, 11, 64, 64), "sumnorm", 0.0),   # the reference self-test's shape / input style
+    ((4, 8, 256, 64, 64), "softmax", 0.0),  # BASELINE config 2, batch slice
+    ((2, 3, 50, 16, 16), "softmax", 0.3),
+    ((2, 2, 40, 32, 32), "l2", 0.0),
+    ((1, 4, 300, 128, 128), "l2", 0.0),     # BASELINE config 5's state size, fp32 I/O, short
+    ((2, 3, 17, 8, 12), "l2", 0.5),          # E != M -> generic kernel
+    ((2, 2, 1, 16, 16), "softmax", 0.2),     # L = 1
+])
+def test_matches_fp64_oracle(shape, qk, w0, flags):
+    print(f"case shape={shape} qk={qk} flags={flags}", flush=True)
+    q, k, v, beta, W0, go = delta_inputs(*shape, seed=0, qk=qk, w0_std=w0)
+    f, b = run_hip(q, k, v, beta, W0, go, flags, want_grad_W=True)
+    base = [t.numpy() for t in (q, k, v, beta, W0)]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, go.numpy(), want_grad_W=True)
+    errs = {n: rel_err(f[n].cpu().numpy(), of[n]) for n in ("out", "v_old", "v_insert", "W")}
+    errs.update({n: rel_err(b[n].cpu().numpy(), ob[n])
+                 for n in ("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W")})
+    # after the backward the caller's memory tensor is back at its initial value
+    errs["W0"] = float(np.abs(b["W0"].cpu().numpy() - W0.numpy()).max() /
+                       max(1e-30, np.abs(of["W"]).max()))
+    bad = {n: e for n, e in errs.items() if not (e < TOL)}
+    assert not bad, f"over tolerance {TOL}: {bad}  (all: {errs})"
+
+
+@pytest.mark.parametrize("flags", KERNELS)
+def test_incoming_state_gradient(flags):
+    print(f"case incoming grad flags={flags}", flush=True)
+    q, k, v, beta, W0, go = delta_inputs(2, 2, 12, 16, 16, seed=4, w0_std=0.4)
+    gs = torch.randn(W0.shape, generator=torch.Generator().manual_seed(5), dtype=torch.float64)
+    base = [t.numpy() for t in (q, k, v, beta, W0)]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, go.numpy(), grad_state=gs.numpy())
+    _, b = run_hip(q, k, v, beta, W0, go, flags, grad_state=gs)
+    for n in ("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W"):
+        assert rel_err(b[n].cpu().numpy(), ob[n]) < TOL, n
+
+
+def test_autograd_function_drop_in_with_layer_style_views():
+    """Call pattern of FastFFlayer: q, k, v, beta are permuted views of one (L, N, H, 3E+1)
+    projection; W starts at zero; loss on the output."""
+    print("case autograd drop-in", flush=True)
+    from fast_weight import fast_weight_delta
+    L, N, H, E = 13, 3, 4, 16
+    dev = _dev()
+    g = torch.Generator().manual_seed(21)
+    qkvb = torch.randn(L, N, H, 3 * E + 1, generator=g, dtype=torch.float64)
+    leaf = qkvb.to(dev, torch.float32).requires_grad_(True)
+
+    def heads(t):
+        hq, hk, hv, hb = torch.split(t, (E,) * 3 + (1,), -1)
+        hb = torch.sigmoid(hb)
+        hq, hk, hv, hb = (a.permute(1, 2, 0, 3) for a in (hq, hk, hv, hb))
+        hq = torch.nn.functional.elu(hq, 1., False) + 1.
+        hk = torch.nn.functional.elu(hk, 1., False) + 1.
+        return hq / hq.sum(-1, keepdim=True), hk / hk.sum(-1, keepdim=True), hv, hb
+
+    hq, hk, hv, hb = heads(leaf)
+    W = torch.zeros(N, H, E, E, device=dev)
+    out = fast_weight_delta(hq, hk, hv, hb, W)
+    go = torch.randn(N, H, L, E, generator=g, dtype=torch.float64)
+    (out * go.to(dev, torch.float32)).sum().backward()
+
+    ref_leaf = qkvb.clone().requires_grad_(True)
+    from oracle.recurrence import delta_recurrence
+    rq, rk, rv, rb = heads(ref_leaf)
+    ref_out, WL = delta_recurrence(rq, rk, rv, rb, torch.zeros(N, H, E, E, dtype=torch.float64))
+    (ref_out * go).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), ref_out.detach().numpy()) < TOL
+    assert rel_err(leaf.grad.cpu().numpy(), ref_leaf.grad.numpy()) < TOL
+    # W was mutated to W_L by the forward and reverted to W_0 = 0 by the backward
+    assert W.abs().max().item() < 1e-5 * WL.abs().max().item()
+
+
+def test_full_config2_properties():
+    """BASELINE config 2 at full size: finite outputs, revert-to-W0 round trip, linearity in
+    grad_out, oracle on a sample of sequences."""
+    print("case full C2 properties", flush=True)
+    q, k, v, beta, W0, go = delta_inputs(32, 8, 256, 64, 64, seed=0)
+    f, b = run_hip(q, k, v, beta, W0, go, 0)
+    assert all(torch.isfinite(t).all() for t in list(f.values()) + list(b.values()))
+    assert b["W0"].abs().max().item() < 1e-5 * f["W"].abs().max().item()   # forward -> backward round trip
+    go2 = torch.randn(go.shape, generator=torch.Generator().manual_seed(2), dtype=torch.float64)
+    _, b2 = run_hip(q, k, v, beta, W0, go2, 0)
+    _, b3 = run_hip(q, k, v, beta, W0, go - 2 * go2, 0)
+    for n in ("grad_Q", "grad_K", "grad_V", "grad_beta"):
+        assert rel_err(b3[n].cpu().numpy(), (b[n] - 2 * b2[n]).cpu().numpy()) < 5e-5, n
+    rows = [0, 17, 31]
+    base = [t[rows].numpy() for t in (q, k, v, beta, W0)]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, go[rows].numpy())
+    assert rel_err(f["out"][rows].cpu().numpy(), of["out"]) < TOL
+    for n in ("grad_Q", "grad_K", "grad_V", "grad_beta"):
+        assert rel_err(b[n][rows].cpu().numpy(), ob[n]) < TOL, n

@@ -1,0 +1,224 @@
+"""GPU parity of the SRWM kernels (through the C ABI) against the fp64 CPU oracle.
+
+Tolerance: 1e-5 relative (max|a-b| / max|b| per tensor), fp32 kernels vs the fp64 oracle,
+on the same seeded inputs.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import rel_err, srwm_inputs
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-5
+FWD_NAMES = ("q", "k", "beta", "y_diff", "q_diff", "k_diff", "beta_diff", "out")
+
+
+def _dev():
+    return torch.device("cuda:0")
+
+
+def run_hip(x, W, go, flags=0, grad_state=None, mode=None):
+    """Runs forward + backward through srwm_hip (the ctypes layer over the C ABI)."""
+    import srwm_hip
+    dev = _dev()
+    N, H, L, E = x.shape
+    xd = x.to(dev, torch.float32)
+    Wd = [w.to(dev, torch.float32).contiguous() for w in W]
+    big = lambda: torch.full((N, H, L, E), float("nan"), device=dev)
+    small = lambda: torch.full((N, H, L, 4), float("nan"), device=dev)
+    f = dict(q=big(), k=big(), beta=small(), y_diff=big(), q_diff=big(), k_diff=big(),
+             beta_diff=small(), out=big())
+    srwm_hip.self_ref_forward(xd, *Wd, *[f[n] for n in FWD_NAMES], flags=flags)
+    f.update(W_y=Wd[0], W_q=Wd[1], W_k=Wd[2], w_b=Wd[3])
+    if go is None:
+        return f, None
+    god = go.to(dev, torch.float32)
+    gx = torch.full((N, H, L, E), float("nan"), device=dev)
+    if grad_state is None:
+        g = [torch.full_like(w, float("nan")) for w in Wd]
+        mode = srwm_hip.GRAD_STATE_ZERO
+    else:
+        g = [s.to(dev, torch.float32).contiguous() for s in grad_state]
+    srwm_hip.self_ref_backward(xd, *[f[n] for n in FWD_NAMES[:-1]], god, *Wd, gx, *g,
+                               flags=flags | mode)
+    torch.cuda.synchronize()
+    b = dict(grad_x=gx, grad_W_y=g[0], grad_W_q=g[1], grad_W_k=g[2], grad_w_b=g[3])
+    return f, b
+
+
+def check_against_oracle(x, W, go, flags, tol=TOL):
+    f, b = run_hip(x, W, go, flags)
+    of = oracle.srwm_forward(x.numpy(), *[w.numpy() for w in W])
+    ob = oracle.srwm_backward(x.numpy(), of, go.numpy())
+    errs = {}
+    for n in FWD_NAMES + ("W_y", "W_q", "W_k", "w_b"):
+        errs[n] = rel_err(f[n].cpu().numpy(), of[n])
+    for n in ("grad_x", "grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"):
+        errs[n] = rel_err(b[n].cpu().numpy(), ob[n])
+    bad = {n: e for n, e in errs.items() if not (e < tol)}
+    assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
+    return errs
+
+
+KERNELS = [pytest.param(0, id="default"), pytest.param(16, id="generic")]
+
+
+@pytest.mark.parametrize("flags", KERNELS)
+@pytest.mark.parametrize("shape,w_std,xsm,per_batch", [
+    ((3, 5, 11, 8), 0.6, True, True),                  # the reference self-test's shape / input style
+    ((2, 4, 64, 16), 0.02, False, False),              # BASELINE config 1
+    ((4, 8, 100, 32), 1 / math.sqrt(32), True, False),  # BASELINE config 3, batch slice
+    ((2, 16, 512, 64), 0.02, False, False),            # BASELINE config 4 (headline), batch slice
+    ((1, 3, 7, 5), 0.8, False, True),                  # odd head size -> generic kernel
+    ((2, 2, 1, 16), 0.3, True, True),                  # L = 1 (how the RL actors call it)
+    ((1, 2, 33, 64), 0.1, True, True),                 # E = 64 with a stronger state
+    ((1, 1, 40, 12), 0.4, False, True),                # E not a power of two
+])
+def test_matches_fp64_oracle(shape, w_std, xsm, per_batch, flags):
+    print(f"case shape={shape} w_std={w_std} flags={flags}", flush=True)
+    x, W, go = srwm_inputs(*shape, seed=0, w_std=w_std, x_softmax=xsm, per_batch_state=per_batch)
+    check_against_oracle(x, W, go, flags)
+
+
+@pytest.mark.parametrize("flags", KERNELS)
+def test_grad_state_modes(flags):
+    import srwm_hip
+    print(f"case grad_state_modes flags={flags}", flush=True)
+    x, W, go = srwm_inputs(2, 3, 9, 16, seed=3, w_std=0.5, per_batch_state=True)
+    g = torch.Generator().manual_seed(7)
+    gs = [torch.randn(w.shape, generator=g, dtype=torch.float64) for w in W]
+    of = oracle.srwm_forward(x.numpy(), *[w.numpy() for w in W])
+    ob = oracle.srwm_backward(x.numpy(), of, go.numpy(), grad_state=[s.numpy() for s in gs])
+    _, b_in = run_hip(x, W, go, flags, grad_state=gs, mode=srwm_hip.GRAD_STATE_IN)
+    _, b_acc = run_hip(x, W, go, flags, grad_state=gs, mode=srwm_hip.GRAD_STATE_ACCUM)
+    assert rel_err(b_in["grad_x"].cpu().numpy(), ob["grad_x"]) < TOL
+    for n, s in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), gs):
+        assert rel_err(b_in[n].cpu().numpy(), ob[n]) < TOL, n
+        # reference-compatible mode: incoming gradient added on top of the propagated one
+        assert rel_err(b_acc[n].cpu().numpy(), ob[n] + s.numpy()) < TOL, n
+
+
+@pytest.mark.parametrize("flags", KERNELS)
+def test_strided_views_as_the_layers_pass_them(flags):
+    """x and grad_out arrive as permuted views of (L, N, H, E) storage."""
+    print(f"case strided flags={flags}", flush=True)
+    import srwm_hip
+    N, H, L, E = 3, 4, 10, 16
+    x, W, go = srwm_inputs(N, H, L, E, seed=5, w_std=0.3)
+    dev = _dev()
+    x_lnhe = x.permute(2, 0, 1, 3).contiguous().to(dev, torch.float32)
+    go_lnhe = go.permute(2, 0, 1, 3).contiguous().to(dev, torch.float32)
+    xv, gov = x_lnhe.permute(1, 2, 0, 3), go_lnhe.permute(1, 2, 0, 3)
+    assert not xv.is_contiguous()
+    Wd = [w.to(dev, torch.float32).contiguous() for w in W]
+    big = lambda: torch.empty((N, H, L, E), device=dev)
+    small = lambda: torch.empty((N, H, L, 4), device=dev)
+    f = [big(), big(), small(), big(), big(), big(), small(), big()]
+    srwm_hip.self_ref_forward(xv, *Wd, *f, flags=flags)
+    gx = big()
+    g = [torch.empty_like(w) for w in Wd]
+    srwm_hip.self_ref_backward(xv, *f[:-1], gov, *Wd, gx, *g, flags=flags)
+    of = oracle.srwm_forward(x.numpy(), *[w.numpy() for w in W])
+    ob = oracle.srwm_backward(x.numpy(), of, go.numpy())
+    assert rel_err(f[-1].cpu().numpy(), of["out"]) < TOL
+    assert rel_err(gx.cpu().numpy(), ob["grad_x"]) < TOL
+    assert rel_err(g[0].cpu().numpy(), ob["grad_W_y"]) < TOL
+
+
+def test_autograd_function_drop_in():
+    """The reference's call pattern: repeat()-ed weights, loss on the output, .backward()."""
+    print("case autograd drop-in", flush=True)
+    from self_ref_v0 import self_ref_v0, stateful_self_ref_v0
+    N, H, L, E = 3, 5, 11, 8
+    x, W, go = srwm_inputs(N, H, L, E, seed=9, w_std=0.6, x_softmax=True)
+    dev = _dev()
+    params = [w[:1].to(dev, torch.float32).clone().requires_grad_(True) for w in W]
+    xd = x.to(dev, torch.float32).requires_grad_(True)
+    bc = [p.repeat(N, 1, 1, 1) for p in params]
+    out = self_ref_v0(xd, *bc)
+    (out * go.to(dev, torch.float32)).sum().backward()
+    of = oracle.srwm_forward(x.numpy(), *[w.numpy() for w in W])
+    ob = oracle.srwm_backward(x.numpy(), of, go.numpy())
+    assert rel_err(out.detach().cpu().numpy(), of["out"]) < TOL
+    assert rel_err(xd.grad.cpu().numpy(), ob["grad_x"]) < TOL
+    for p, n in zip(params, ("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b")):
+        assert rel_err(p.grad.cpu().numpy(), ob[n].sum(0, keepdims=True)) < TOL, n
+    # the broadcast copies now hold the final state (read back by the RL layers)
+    for t, n in zip(bc, ("W_y", "W_q", "W_k", "w_b")):
+        assert rel_err(t.detach().cpu().numpy(), of[n]) < TOL, n
+
+    # stateful variant: loss on the returned state as well
+    params2 = [w[:1].to(dev, torch.float32).clone().requires_grad_(True) for w in W]
+    xd2 = x.to(dev, torch.float32).requires_grad_(True)
+    bc2 = [p.repeat(N, 1, 1, 1) for p in params2]
+    g = torch.Generator().manual_seed(11)
+    gs = [torch.randn(w.shape, generator=g, dtype=torch.float64) for w in W]
+    out2, *state = stateful_self_ref_v0(xd2, *bc2)
+    loss = (out2 * go.to(dev, torch.float32)).sum()
+    loss = loss + sum((s * t.to(dev, torch.float32)).sum() for s, t in zip(state, gs))
+    loss.backward()
+    ob2 = oracle.srwm_backward(x.numpy(), of, go.numpy(), grad_state=[s.numpy() for s in gs])
+    assert rel_err(xd2.grad.cpu().numpy(), ob2["grad_x"]) < TOL
+    for p, n in zip(params2, ("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b")):
+        assert rel_err(p.grad.cpu().numpy(), ob2[n].sum(0, keepdims=True)) < TOL, n
+
+
+def test_full_headline_shape_properties():
+    """BASELINE config 4 at full size (N=32, H=16, L=512, E=64): size-independent properties
+    plus the oracle on a sample of the 512 sequences."""
+    print("case full C4 properties", flush=True)
+    N, H, L, E = 32, 16, 512, 64
+    x, W, go = srwm_inputs(N, H, L, E, seed=0, w_std=0.02)
+    f, b = run_hip(x, W, go, 0)
+    q, k, beta = f["q"], f["k"], f["beta"]
+    assert torch.allclose(q.sum(-1), torch.ones_like(q[..., 0]), atol=1e-5)
+    assert torch.allclose(k.sum(-1), torch.ones_like(k[..., 0]), atol=1e-5)
+    assert (beta > 0).all() and (beta < 1).all()
+    assert all(torch.isfinite(v).all() for v in list(f.values()) + list(b.values()))
+    # linearity of the backward in grad_out
+    go2 = torch.randn(go.shape, generator=torch.Generator().manual_seed(1), dtype=torch.float64)
+    _, b2 = run_hip(x, W, go2, 0)
+    _, b3 = run_hip(x, W, 2 * go - 3 * go2, 0)
+    for n in b:
+        lin = 2 * b[n] - 3 * b2[n]
+        assert rel_err(b3[n].cpu().numpy(), lin.cpu().numpy()) < 5e-5, n
+    # oracle on a sample of sequences (batch rows 0, 13, 31)
+    rows = [0, 13, 31]
+    xs, gos = x[rows], go[rows]
+    Ws = [w[rows] for w in W]
+    of = oracle.srwm_forward(xs.numpy(), *[w.numpy() for w in Ws])
+    ob = oracle.srwm_backward(xs.numpy(), of, gos.numpy())
+    for n in FWD_NAMES + ("W_y", "W_q", "W_k", "w_b"):
+        assert rel_err(f[n][rows].cpu().numpy(), of[n]) < TOL, n
+    for n in ob:
+        if n in b:
+            assert rel_err(b[n][rows].cpu().numpy(), ob[n]) < TOL, n
+
+
+def test_errors_are_reported_not_swallowed():
+    import srwm_hip
+    dev = _dev()
+    x = torch.zeros(1, 1, 2, 8, device=dev)
+    W = [torch.zeros(1, 1, 8, 8, device=dev) for _ in range(3)] + [torch.zeros(1, 1, 8, 4, device=dev)]
+    outs = [torch.zeros(1, 1, 2, 8, device=dev) for _ in range(2)] + [torch.zeros(1, 1, 2, 4, device=dev)] + \
+           [torch.zeros(1, 1, 2, 8, device=dev) for _ in range(3)] + [torch.zeros(1, 1, 2, 4, device=dev)] + \
+           [torch.zeros(1, 1, 2, 8, device=dev)]
+    with pytest.raises(ValueError):
+        srwm_hip.self_ref_forward(x, W[0], W[1], W[2], W[0], *outs)          # w_b has the wrong shape
+    with pytest.raises(TypeError):
+        srwm_hip.self_ref_forward(x.double(), *W, *outs)                     # float64 is not accepted
+    with pytest.raises(RuntimeError):
+        srwm_hip.self_ref_forward(x.cpu(), *W, *outs)                        # no CPU path
+    big = 512                                                                # state cannot fit in LDS
+    xb = torch.zeros(1, 1, 1, big, device=dev)
+    Wb = [torch.zeros(1, 1, big, big, device=dev) for _ in range(3)] + [torch.zeros(1, 1, big, 4, device=dev)]
+    ob = [torch.zeros(1, 1, 1, big, device=dev) for _ in range(2)] + [torch.zeros(1, 1, 1, 4, device=dev)] + \
+         [torch.zeros(1, 1, 1, big, device=dev) for _ in range(3)] + [torch.zeros(1, 1, 1, 4, device=dev)] + \
+         [torch.zeros(1, 1, 1, big, device=dev)]
+    with pytest.raises(RuntimeError, match="not supported"):
+        srwm_hip.self_ref_forward(xb, *Wb, *ob)
