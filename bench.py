@@ -1,0 +1,228 @@
+#!/usr/bin/env python3
+"""Headline benchmark: SRWM forward+backward tokens/s on one MI355X.
+
+A "step" is one forward + one backward pass of the SRWM operator over one batch of
+synthetic input (N=32, H=16, L=512, d_head=64, fp32 -- BASELINE.json configs[3], the
+configuration the metric is quoted on), including the re-initialisation of the per-batch
+state copies that the layer's `.repeat()` performs every call.  All tensors are resident
+in HBM before the timed region; kernels are launched through the C ABI on torch's current
+stream, so torch.cuda.Event brackets exactly the stream the kernels run on.
+
+Prints ONE JSON line (see the keys below).  `roofline` prices the dominant kernel (the
+backward) against the LDS-bandwidth yardstick of 6 passes over the 64x196 fp32 state per
+(sequence, step); `roofline_fwd_bwd` does the same for the forward+backward pair
+(9 passes), which is the figure the target (>= 50 %) is stated on; `roofline_hbm` gives the
+achieved HBM rate of the operator's I/O contract.  `cpu_baseline` is the per-timestep
+PyTorch recurrence (oracle/recurrence.py) timed on the host cores on a batch slice.
+
+Other workloads (parity-test configurations, not the headline): --workload
+{srwm_c3, delta_c2, delta_c5f32}.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "modern-srwm_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+LDS_PEAK_GBS = 256 * 128 * 2.4          # 256 CUs x 128 B/clk x 2.4 GHz = 78 643 GB/s
+HBM_PEAK_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (op, N, H, L, E)
+    "srwm_c4": ("srwm", 32, 16, 512, 64),
+    "srwm_c3": ("srwm", 32, 8, 100, 32),
+    "delta_c2": ("delta", 32, 8, 256, 64),
+    "delta_c5f32": ("delta", 8, 16, 4096, 128),
+}
+
+
+def srwm_setup(N, H, L, E, dev):
+    import torch
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(N, H, L, E, generator=g)
+    W0 = [torch.randn(1, H, E, E, generator=g) * 0.02 for _ in range(3)]
+    W0.append(torch.randn(1, H, E, 4, generator=g) * 0.02)
+    go = torch.randn(N, H, L, E, generator=g)
+    t = dict(x=x.to(dev), go=go.to(dev), W0=[w.repeat(N, 1, 1, 1).to(dev) for w in W0])
+    t["W"] = [torch.empty_like(w) for w in t["W0"]]
+    big = lambda: torch.empty(N, H, L, E, device=dev)
+    small = lambda: torch.empty(N, H, L, 4, device=dev)
+    t["saved"] = [big(), big(), small(), big(), big(), big(), small()]
+    t["out"] = big()
+    t["gx"] = big()
+    t["gW"] = [torch.empty_like(w) for w in t["W0"]]
+    return t
+
+
+def srwm_step(t, ev=None):
+    import srwm_hip
+    for w, w0 in zip(t["W"], t["W0"]):
+        w.copy_(w0)                     # what `.repeat(bsz,1,1,1)` does in the layer
+    if ev:
+        ev[0].record()
+    srwm_hip.self_ref_forward(t["x"], *t["W"], *t["saved"], t["out"])
+    if ev:
+        ev[1].record()
+    srwm_hip.self_ref_backward(t["x"], *t["saved"], t["go"], *t["W"], t["gx"], *t["gW"],
+                               flags=srwm_hip.GRAD_STATE_ZERO)
+    if ev:
+        ev[2].record()
+
+
+def delta_setup(N, H, L, E, dev):
+    import torch
+    g = torch.Generator().manual_seed(0)
+    M = E
+    if E >= 128:
+        q = torch.randn(N, H, L, E, generator=g)
+        k = torch.randn(N, H, L, E, generator=g)
+        q, k = q / q.norm(dim=-1, keepdim=True), k / k.norm(dim=-1, keepdim=True)
+    else:
+        q = torch.softmax(torch.randn(N, H, L, E, generator=g), -1)
+        k = torch.softmax(torch.randn(N, H, L, E, generator=g), -1)
+    v = torch.randn(N, H, L, M, generator=g)
+    beta = torch.sigmoid(torch.randn(N, H, L, 1, generator=g))
+    go = torch.randn(N, H, L, M, generator=g)
+    t = dict(q=q.to(dev), k=k.to(dev), v=v.to(dev), beta=beta.to(dev), go=go.to(dev))
+    t["W"] = torch.empty(N, H, E, M, device=dev)
+    bigm = lambda: torch.empty(N, H, L, M, device=dev)
+    bige = lambda: torch.empty(N, H, L, E, device=dev)
+    t["vold"], t["vins"], t["out"] = bigm(), bigm(), bigm()
+    t["gq"], t["gk"], t["gv"] = bige(), bige(), bigm()
+    t["gb"] = torch.empty(N, H, L, 1, device=dev)
+    return t
+
+
+def delta_step(t, ev=None):
+    import srwm_hip
+    t["W"].zero_()
+    if ev:
+        ev[0].record()
+    srwm_hip.fast_weight_forward(t["q"], t["k"], t["v"], t["beta"], t["vold"], t["vins"], t["W"], t["out"])
+    if ev:
+        ev[1].record()
+    srwm_hip.fast_weight_backward(t["q"], t["k"], t["v"], t["beta"], t["vold"], t["vins"], t["go"],
+                                  t["W"], t["gq"], t["gk"], t["gv"], t["gb"])
+    if ev:
+        ev[2].record()
+
+
+def algorithmic_bytes(op, N, H, L, E):
+    """(lds_fwd, lds_bwd, hbm_total) bytes per launch pair."""
+    hs = N * H * L
+    if op == "srwm":
+        S = E * (3 * E + 4)
+        return 3 * S * 4 * hs, 6 * S * 4 * hs, (15 * E + 16) * 4 * hs + 4 * S * 4 * N * H
+    S = E * E
+    return 2 * S * 4 * hs, 4 * S * 4 * hs, (6 * E + 9 * E + 3) * 4 * hs + 3 * S * 4 * N * H
+
+
+def cpu_baseline(op, N, H, L, E, budget_s=20.0):
+    """Per-timestep PyTorch recurrence (forward + autograd backward) on the host cores, on a
+    batch slice sized to about `budget_s` seconds; tokens/s = slice_N * L / time."""
+    import torch
+    from oracle.recurrence import delta_recurrence, srwm_recurrence
+    cores = torch.get_num_threads()
+    g = torch.Generator().manual_seed(0)
+
+    def run(n):
+        if op == "srwm":
+            x = torch.randn(n, H, L, E, generator=g).requires_grad_(True)
+            W = [(torch.randn(n, H, E, E, generator=g) * 0.02).requires_grad_(True) for _ in range(3)]
+            W.append((torch.randn(n, H, E, 4, generator=g) * 0.02).requires_grad_(True))
+            go = torch.randn(n, H, L, E, generator=g)
+            t0 = time.perf_counter()
+            out, _ = srwm_recurrence(x, *W)
+        else:
+            q = torch.softmax(torch.randn(n, H, L, E, generator=g), -1).requires_grad_(True)
+            k = torch.softmax(torch.randn(n, H, L, E, generator=g), -1).requires_grad_(True)
+            v = torch.randn(n, H, L, E, generator=g).requires_grad_(True)
+            b = torch.sigmoid(torch.randn(n, H, L, 1, generator=g)).requires_grad_(True)
+            go = torch.randn(n, H, L, E, generator=g)
+            t0 = time.perf_counter()
+            out, _ = delta_recurrence(q, k, v, b, torch.zeros(n, H, E, E))
+        (out * go).sum().backward()
+        return time.perf_counter() - t0
+
+    run(1)                                  # warm-up (thread pool, allocator)
+    t1 = run(1)
+    n = max(1, min(N, int(budget_s / max(t1, 1e-3))))
+    tn = run(n) if n > 1 else t1
+    return {"value": n * L / tn, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"oracle/recurrence.py ({op}) fwd+autograd bwd, fp32, batch slice N={n} of {N} "
+                      f"(H={H}, L={L}, E={E}) in {tn:.2f}s, torch {cores} threads; "
+                      "sequences are independent so tokens/s does not depend on the slice"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="srwm_c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-budget", type=float, default=20.0)
+    a = ap.parse_args()
+    if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this operator runs on ONE GPU (sequences shard over GPUs without any "
+              "collective; no multi-GPU figure is produced). Use --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import srwm_hip
+    srwm_hip.lib()                          # fail loudly if the HIP library is not built
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    op, N, H, L, E = WORKLOADS[a.workload]
+    setup, step = (srwm_setup, srwm_step) if op == "srwm" else (delta_setup, delta_step)
+    t = setup(N, H, L, E, dev)
+
+    for _ in range(a.warmup):
+        step(t)
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(a.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(a.steps):
+        step(t, evs[i])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / a.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / a.steps
+    ms_per_step = elapsed * 1e3 / a.steps
+    tokens_per_s = N * L * a.steps / elapsed
+    lds_f, lds_b, hbm = algorithmic_bytes(op, N, H, L, E)
+
+    def roof(bound, bytes_, ms, peak):
+        ach = bytes_ / (ms * 1e-3) / 1e9
+        return {"bound": bound, "achieved": round(ach, 1), "peak": round(peak, 1), "unit": "GB/s",
+                "frac": round(ach / peak, 4), "traffic": None}
+
+    res = {
+        "metric": "fwd+bwd tokens/sec SRWM B=32 H=16 T=512 d=64; % LDS/HBM roofline"
+                  if a.workload == "srwm_c4" else f"fwd+bwd tokens/sec {a.workload}",
+        "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
+        "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{a.workload}: {op} fwd+bwd N={N} H={H} L={L} E={E} fp32, "
+                               "state re-initialised per step, x~N(0,1), W0~N(0,0.02), grad~N(0,1)"},
+        "kernel_ms": {"forward": round(fwd_ms, 4), "backward": round(bwd_ms, 4)},
+        "roofline": dict(roof("lds", lds_b, bwd_ms, LDS_PEAK_GBS), kernel="backward"),
+        "roofline_fwd_bwd": roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS),
+        "roofline_hbm": roof("hbm", hbm, fwd_ms + bwd_ms, HBM_PEAK_GBS),
+    }
+    if not a.no_cpu_baseline:
+        res["cpu_baseline"] = cpu_baseline(op, N, H, L, E, a.cpu_budget)
+    print(json.dumps(res))
+
+
+if __name__ == "__main__":
+    main()
