@@ -1,5 +1,528 @@
+// Register-resident SRWM kernels for the compiled-in head sizes (E = 8, 16, 32, 64).
+//
+// One workgroup of NW wave64s owns one (batch, head) sequence for all L steps.  The packed
+// state W = [W_y | W_q | W_k | w_b] never leaves the register file:
+//   * the three E x E blocks are cut into tiles of R rows x CB columns per block; lane
+//     (rg, cg) holds rows [R*rg, R*rg+R) of columns [CB*cg, CB*cg+CB) of EACH block, so a
+//     lane's 3*CB columns are y_c, q_c, k_c for the same c.  The RG = E/R lanes that share
+//     a column group are consecutive lanes, so a column sum (readout W^T v) finishes with
+//     log2(RG) DPP adds inside a 16-lane row and leaves the result in every one of them --
+//     exactly where the rank-1 write needs it;
+//   * the E x 4 block w_b has one element per thread: thread tid holds w_b[tid % E][tid / E].
+// Per step the only workgroup barrier is the hand-over of the raw q~/k~/b~ readout; every
+// wave then runs both softmaxes redundantly with lane <-> element (one exp per lane), which
+// puts q, k and q-k for row `lane % E` in the lane that owns that row of w_b, and passes
+// the R-row operand slices to the tile lanes through a wave-private LDS strip.
+// x is streamed through LDS in tiles of TT steps, fetched one tile ahead.
+//
+// Replaces self_ref_forward_kernel / self_ref_backward_kernel of the reference
+// (supervised_learning/self_ref_v0/self_ref_v0.cu:24-432, :534-1234).
 #include "common.h"
+#include "xlane.h"
+
 namespace fw {
-int launch_srwm_fwd_tiled(const SrwmFwdParams &, hipStream_t) { return -1; }
-int launch_srwm_bwd_tiled(const SrwmBwdParams &, hipStream_t) { return -1; }
+
+namespace {
+
+template <int E, int NW, int R>
+struct Tiling {
+    static constexpr int NT = NW * kWave;   // threads per workgroup
+    static constexpr int RG = E / R;        // lanes that share a column group (row groups)
+    static constexpr int CGW = kWave / RG;  // column groups per wave
+    static constexpr int NCG = NW * CGW;    // column groups per workgroup
+    static constexpr int CB = E / NCG;      // columns per block per lane
+    static constexpr int NC = 3 * CB;       // columns per lane
+    static constexpr int TT = 4 * NT / E;   // steps per input tile: one float4 per thread per vector
+    static_assert(RG * R == E && CGW * RG == kWave && CB * NCG == E && CB >= 1, "tiling");
+    static_assert(RG <= 16, "column sums must stay inside a DPP row");
+    static_assert(E <= kWave && kWave % E == 0, "softmax is done with lane <-> element");
+    static_assert(TT * E == 4 * NT, "tile loader");
+};
+
+template <int N>
+__device__ __forceinline__ void lds_read_vec(float (&dst)[N], const float *src) {
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 4; ++i) {
+            const float4 v = reinterpret_cast<const float4 *>(src)[i];
+            dst[4 * i] = v.x; dst[4 * i + 1] = v.y; dst[4 * i + 2] = v.z; dst[4 * i + 3] = v.w;
+        }
+    } else if constexpr (N == 2) {
+        const float2 v = *reinterpret_cast<const float2 *>(src);
+        dst[0] = v.x; dst[1] = v.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) dst[i] = src[i];
+    }
+}
+
+template <int N>
+__device__ __forceinline__ void store_vec(float *dst, const float *src) {
+    if constexpr (N == 4) {
+        *reinterpret_cast<float4 *>(dst) = make_float4(src[0], src[1], src[2], src[3]);
+    } else if constexpr (N == 2) {
+        *reinterpret_cast<float2 *>(dst) = make_float2(src[0], src[1]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) dst[i] = src[i];
+    }
+}
+
+template <int E, int NW, int R>
+__global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams p) {
+    using T = Tiling<E, NW, R>;
+    constexpr int RG = T::RG, CGW = T::CGW, CB = T::CB, NC = T::NC, TT = T::TT;
+
+    __shared__ __attribute__((aligned(16))) float xt[2][TT][E];   // input tiles, double buffered
+    __shared__ __attribute__((aligned(16))) float raw[2][2][E];   // q~ | k~ of the step, by parity
+    __shared__ float rawb[2][4];                                  // b~
+    __shared__ __attribute__((aligned(16))) float exch[NW][2][E]; // per wave: q-k | k
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int rg = lane % RG, cg = wave * CGW + lane / RG;
+    const int r0 = rg * R, c0 = cg * CB;
+    const int el = lane % E;                 // softmax element == row of this thread's w_b entry
+    const int jb = tid / E;                  // column of this thread's w_b entry
+    const bool has_b = jb < 4;
+
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const int64_t sEE = seq * E * E, sE4 = seq * E * 4;
+    const float *xbase = p.x + n * p.xs_n + h * p.xs_h;
+
+    float w[R][NC];
+    {
+        const float *src[3] = {p.Wy + sEE, p.Wq + sEE, p.Wk + sEE};
+#pragma unroll
+        for (int b = 0; b < 3; ++b)
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < CB; ++c) w[i][b * CB + c] = src[b][(r0 + i) * E + c0 + c];
+    }
+    float wbe = has_b ? p.wb[sE4 + el * 4 + jb] : 0.f;
+
+    // tile loader: thread -> (step tid / (E/4), 4 consecutive elements)
+    const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
+    auto load_tile = [&](int tile) -> float4 {
+        const int t = tile * TT + ld_row;
+        if (t < p.L) return *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col);
+        return make_float4(0.f, 0.f, 0.f, 0.f);
+    };
+    const int ntiles = (p.L + TT - 1) / TT;
+    *reinterpret_cast<float4 *>(&xt[0][ld_row][ld_col]) = load_tile(0);
+    __syncthreads();
+
+    for (int tile = 0; tile < ntiles; ++tile) {
+        const int buf = tile & 1;
+        const int tlen = min(TT, p.L - tile * TT);
+        float4 xnext = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (tile + 1 < ntiles) xnext = load_tile(tile + 1);
+
+        for (int tt = 0; tt < tlen; ++tt) {
+            const int t = tile * TT + tt, par = t & 1;
+            const int64_t o = (seq * p.L + t) * E, ob = (seq * p.L + t) * 4;
+
+            // ---- main readout: [y | q~ | k~ | b~] = W^T x_t
+            float xr[R];
+            lds_read_vec<R>(xr, &xt[buf][tt][r0]);
+            const float xb = xt[buf][tt][el];
+            float acc[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) acc[c] = 0.f;
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < NC; ++c) acc[c] = fmaf(w[i][c], xr[i], acc[c]);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) acc[c] = group_sum<RG>(acc[c]);
+            const float pb = group_sum<E>(wbe * xb);
+            if (rg == 0) {
+                store_vec<CB>(p.out + o + c0, &acc[0]);
+                store_vec<CB>(&raw[par][0][c0], &acc[CB]);
+                store_vec<CB>(&raw[par][1][c0], &acc[2 * CB]);
+            }
+            if (has_b && el == 0) rawb[par][jb] = pb;
+            if (tt == tlen - 1 && tile + 1 < ntiles)
+                *reinterpret_cast<float4 *>(&xt[buf ^ 1][ld_row][ld_col]) = xnext;
+            __syncthreads();
+
+            // ---- activations, redundantly in every wave, lane <-> element el
+            const float qraw = raw[par][0][el], kraw = raw[par][1][el], braw = rawb[par][lane & 3];
+            const float mq = group_max<E>(qraw), mk = group_max<E>(kraw);
+            const float eq = expf(qraw - mq), ek = expf(kraw - mk);
+            const float sq = group_sum<E>(eq), sk = group_sum<E>(ek);
+            const float qn = eq * fast_rcp(sq), kn = ek * fast_rcp(sk);
+            const float sg = fast_rcp(1.f + expf(-braw));
+            const float bt[4] = {quad_broadcast<0>(sg), quad_broadcast<1>(sg), quad_broadcast<2>(sg),
+                                 quad_broadcast<3>(sg)};
+            const float dv = qn - kn;
+            if (wave == 0 && lane < E) {
+                p.q[o + lane] = qn;
+                p.k[o + lane] = kn;
+            }
+            if (wave == NW - 1 && lane < 4) p.beta[ob + lane] = sg;
+            if (lane < E) {
+                exch[wave][0][lane] = dv;
+                exch[wave][1][lane] = kn;
+            }
+            wave_lds_fence();
+            float dvr[R], kr[R];
+            lds_read_vec<R>(dvr, &exch[wave][0][r0]);
+            lds_read_vec<R>(kr, &exch[wave][1][r0]);
+
+            // ---- diff = W^T (q - k)
+            float dif[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) dif[c] = 0.f;
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < NC; ++c) dif[c] = fmaf(w[i][c], dvr[i], dif[c]);
+#pragma unroll
+            for (int c = 0; c < NC; ++c) dif[c] = group_sum<RG>(dif[c]);
+            const float pbd = group_sum<E>(wbe * dv);
+            if (rg == 0) {
+                store_vec<CB>(p.ydiff + o + c0, &dif[0]);
+                store_vec<CB>(p.qdiff + o + c0, &dif[CB]);
+                store_vec<CB>(p.kdiff + o + c0, &dif[2 * CB]);
+            }
+            if (has_b && el == 0) p.bdiff[ob + jb] = pbd;
+
+            // ---- rank-1 write W += k (x) (beta_blk * diff)
+            float ins[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) ins[c] = bt[c / CB] * dif[c];
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < NC; ++c) w[i][c] = fmaf(kr[i], ins[c], w[i][c]);
+            wbe = fmaf(kn, bt[3] * pbd, wbe);
+        }
+    }
+
+    {
+        float *dst[3] = {p.Wy + sEE, p.Wq + sEE, p.Wk + sEE};
+#pragma unroll
+        for (int b = 0; b < 3; ++b)
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < CB; ++c) dst[b][(r0 + i) * E + c0 + c] = w[i][b * CB + c];
+    }
+    if (has_b) p.wb[sE4 + el * 4 + jb] = wbe;
+}
+
+// ---------------------------------------------------------------------------------------
+// Backward: reverse-time sweep with W (reverted step by step) and G = dL/dW in registers,
+// same tiling as the forward.  Per step:
+//   column sum   g_ins = G^T k                        (DPP all-reduce inside the column group)
+//   row sums     G ins, W_{t-1} g_diff, W_{t-1} g_pre (per lane R partial rows -> reduce-scatter
+//                over the wave's 8 column groups with v_permlane{32,16}_swap + one DPP step,
+//                then summed over the waves through LDS)
+// and two workgroup barriers (after the first pair of row sums, after the grad_x row sum).
+// The seven per-step vectors and beta are streamed through a single LDS tile of TT steps;
+// the next tile is fetched into registers one tile ahead.
+template <int E, int NW, int R>
+__global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams p) {
+    using T = Tiling<E, NW, R>;
+    constexpr int RG = T::RG, CGW = T::CGW, NCG = T::NCG, CB = T::CB, NC = T::NC, TT = T::TT;
+    static_assert(RG == 8, "row-sum reduction assumes column groups 8 lanes apart");
+    enum { VX, VQ, VK, VYD, VQD, VKD, VGO, NVEC };
+
+    __shared__ __attribute__((aligned(16))) float tl[NVEC][TT][E];  // per-step vectors of the tile
+    __shared__ __attribute__((aligned(16))) float tb[2][TT][4];     // beta | beta_diff
+    __shared__ __attribute__((aligned(16))) float rowm[3][NW][E];   // row sums per wave: G ins | W gdiff | W gpre
+    __shared__ __attribute__((aligned(16))) float rowb[3][4][E];    // same, contribution of the w_b block
+    __shared__ __attribute__((aligned(16))) float gbp[NCG][4];      // per column group: sum gins*diff per block
+    __shared__ __attribute__((aligned(16))) float gbp3[4];          // same for the four w_b columns
+    __shared__ __attribute__((aligned(16))) float exch[NW][2][E];   // per wave: g_pre of the q | k block
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int rg = lane % RG, cgl = lane / RG, cg = wave * CGW + cgl;
+    const int r0 = rg * R, c0 = cg * CB;
+    const int el = lane % E;
+    const int jb = tid / E;
+    const bool has_b = jb < 4;
+
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const int64_t sEE = seq * E * E, sE4 = seq * E * 4;
+    const float *xbase = p.x + n * p.xs_n + h * p.xs_h;
+    const float *gobase = p.go + n * p.gs_n + h * p.gs_h;
+
+    float w[R][NC], g[R][NC];
+    {
+        const float *src[3] = {p.Wy + sEE, p.Wq + sEE, p.Wk + sEE};
+        const float *gsrc[3] = {p.gWy + sEE, p.gWq + sEE, p.gWk + sEE};
+#pragma unroll
+        for (int b = 0; b < 3; ++b)
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < CB; ++c) {
+                    w[i][b * CB + c] = src[b][(r0 + i) * E + c0 + c];
+                    g[i][b * CB + c] = p.grad_state_mode ? gsrc[b][(r0 + i) * E + c0 + c] : 0.f;
+                }
+    }
+    float wbe = has_b ? p.wb[sE4 + el * 4 + jb] : 0.f;
+    float gbe = (has_b && p.grad_state_mode) ? p.gwb[sE4 + el * 4 + jb] : 0.f;
+
+    const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
+    struct TileRegs {
+        float4 v[NVEC];
+        float4 b, bd;
+    };
+    auto load_tile = [&](int tile) -> TileRegs {
+        TileRegs r;
+        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+        const int t = tile * TT + ld_row;
+        const bool ok = t < p.L;
+        const int64_t o = (seq * p.L + t) * E + ld_col;
+        r.v[VX] = ok ? *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col) : z;
+        r.v[VGO] = ok ? *reinterpret_cast<const float4 *>(gobase + t * p.gs_l + ld_col) : z;
+        r.v[VQ] = ok ? *reinterpret_cast<const float4 *>(p.q + o) : z;
+        r.v[VK] = ok ? *reinterpret_cast<const float4 *>(p.k + o) : z;
+        r.v[VYD] = ok ? *reinterpret_cast<const float4 *>(p.ydiff + o) : z;
+        r.v[VQD] = ok ? *reinterpret_cast<const float4 *>(p.qdiff + o) : z;
+        r.v[VKD] = ok ? *reinterpret_cast<const float4 *>(p.kdiff + o) : z;
+        r.b = z;
+        r.bd = z;
+        const int tb_t = tile * TT + tid;
+        if (tid < TT && tb_t < p.L) {
+            r.b = *reinterpret_cast<const float4 *>(p.beta + (seq * p.L + tb_t) * 4);
+            r.bd = *reinterpret_cast<const float4 *>(p.bdiff + (seq * p.L + tb_t) * 4);
+        }
+        return r;
+    };
+    auto store_tile = [&](const TileRegs &r) {
+#pragma unroll
+        for (int v = 0; v < NVEC; ++v) *reinterpret_cast<float4 *>(&tl[v][ld_row][ld_col]) = r.v[v];
+        if (tid < TT) {
+            *reinterpret_cast<float4 *>(&tb[0][tid][0]) = r.b;
+            *reinterpret_cast<float4 *>(&tb[1][tid][0]) = r.bd;
+        }
+    };
+
+    const int ntiles = (p.L + TT - 1) / TT;
+    store_tile(load_tile(ntiles - 1));
+    __syncthreads();
+
+    for (int tile = ntiles - 1; tile >= 0; --tile) {
+        const int tlen = min(TT, p.L - tile * TT);
+        TileRegs nxt;
+        if (tile > 0) nxt = load_tile(tile - 1);
+
+        for (int tt = tlen - 1; tt >= 0; --tt) {
+            const int t = tile * TT + tt;
+            const int64_t o = (seq * p.L + t) * E;
+
+            // ---- operands of the step
+            float kr[R], dvr[R], xr[R];
+            lds_read_vec<R>(kr, &tl[VK][tt][r0]);
+            lds_read_vec<R>(dvr, &tl[VQ][tt][r0]);
+            lds_read_vec<R>(xr, &tl[VX][tt][r0]);
+#pragma unroll
+            for (int i = 0; i < R; ++i) dvr[i] -= kr[i];
+            float dif[NC], gpre[NC];
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[0]), &tl[VYD][tt][c0]);
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[CB]), &tl[VQD][tt][c0]);
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[2 * CB]), &tl[VKD][tt][c0]);
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[0]), &tl[VGO][tt][c0]);
+            float bt[4];
+            lds_read_vec<4>(bt, &tb[0][tt][0]);
+            const float bd = tb[1][tt][jb & 3];
+            const float kb = tl[VK][tt][el], qb = tl[VQ][tt][el], xb = tl[VX][tt][el];
+            const float dvb = qb - kb;
+
+            // ---- revert the write: W_{t-1} = W_t - k (x) ins
+            float ins[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) ins[c] = bt[c / CB] * dif[c];
+            const float insb = bt[3] * bd;
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < NC; ++c) w[i][c] = fmaf(-kr[i], ins[c], w[i][c]);
+            wbe = fmaf(-kb, insb, wbe);
+
+            // ---- g_ins = G^T k (column sums), g_diff = beta_blk * g_ins
+            float gdif[NC];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) gdif[c] = 0.f;
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < NC; ++c) gdif[c] = fmaf(g[i][c], kr[i], gdif[c]);
+            float pg[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const float gi = group_sum<RG>(gdif[c]);
+                pg[c / CB] = fmaf(gi, dif[c], pg[c / CB]);
+                gdif[c] = bt[c / CB] * gi;
+            }
+            const float ginsb = group_sum<E>(gbe * kb);
+            const float gdifb = bt[3] * ginsb;
+
+            // ---- row sums  a = G ins,  u = W_{t-1} g_diff
+            float a[R], u[R];
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                a[i] = 0.f;
+                u[i] = 0.f;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    a[i] = fmaf(g[i][c], ins[c], a[i]);
+                    u[i] = fmaf(w[i][c], gdif[c], u[i]);
+                }
+            }
+            stride8_reduce_store<R>(a, &rowm[0][wave][r0], lane);
+            stride8_reduce_store<R>(u, &rowm[1][wave][r0], lane);
+            if (has_b) {
+                rowb[0][jb][el] = gbe * insb;
+                rowb[1][jb][el] = wbe * gdifb;
+                if (el == 0) gbp3[jb] = ginsb * bd;
+            }
+            if (rg == 0) *reinterpret_cast<float4 *>(&gbp[cg][0]) = make_float4(pg[0], pg[1], pg[2], 0.f);
+            __syncthreads();
+
+            // ---- every wave, lane <-> element el: gradients of q, k, beta before activation
+            float gq = 0.f, gk = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < NW; ++wv) {
+                gk += rowm[0][wv][el];
+                gq += rowm[1][wv][el];
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                gk += rowb[0][j][el];
+                gq += rowb[1][j][el];
+            }
+            gk -= gq;
+            const float dq = group_sum<E>(gq * qb), dk = group_sum<E>(gk * kb);
+            const float gpq = qb * (gq - dq), gpk = kb * (gk - dk);
+            float gb[4];
+            {
+                float part[4];
+                lds_read_vec<4>(part, &gbp[lane % NCG][0]);
+#pragma unroll
+                for (int j = 0; j < 3; ++j) gb[j] = group_sum<NCG>(part[j]);
+                float p3[4];
+                lds_read_vec<4>(p3, &gbp3[0]);
+                gb[3] = (p3[0] + p3[1]) + (p3[2] + p3[3]);
+            }
+            float gpb[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) gpb[j] = gb[j] * bt[j] * (1.f - bt[j]);
+            const float gpreb = jb == 0 ? gpb[0] : jb == 1 ? gpb[1] : jb == 2 ? gpb[2] : gpb[3];
+            if (lane < E) {
+                exch[wave][0][lane] = gpq;
+                exch[wave][1][lane] = gpk;
+            }
+            wave_lds_fence();
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[CB]), &exch[wave][0][c0]);
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[2 * CB]), &exch[wave][1][c0]);
+
+            // ---- grad_x = W_{t-1} g_pre (row sums)
+            float sx[R];
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                sx[i] = 0.f;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) sx[i] = fmaf(w[i][c], gpre[c], sx[i]);
+            }
+            stride8_reduce_store<R>(sx, &rowm[2][wave][r0], lane);
+            if (has_b) rowb[2][jb][el] = wbe * gpreb;
+            __syncthreads();
+            if (tid < E) {
+                float s = 0.f;
+#pragma unroll
+                for (int wv = 0; wv < NW; ++wv) s += rowm[2][wv][tid];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) s += rowb[2][j][tid];
+                p.gx[o + tid] = s;
+            }
+
+            // ---- G_{t-1} = G_t + (q - k) (x) g_diff + x (x) g_pre
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < NC; ++c)
+                    g[i][c] = fmaf(dvr[i], gdif[c], fmaf(xr[i], gpre[c], g[i][c]));
+            gbe = fmaf(dvb, gdifb, fmaf(xb, gpreb, gbe));
+
+            if (tt == 0 && tile > 0) {
+                // every wave is past its last read of this tile (all reads precede the
+                // first barrier of the step)
+                store_tile(nxt);
+                __syncthreads();
+            }
+        }
+    }
+
+    {
+        float *dst[3] = {p.gWy + sEE, p.gWq + sEE, p.gWk + sEE};
+        const bool accum = p.grad_state_mode == 2u;
+#pragma unroll
+        for (int b = 0; b < 3; ++b)
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < CB; ++c) {
+                    float *d = &dst[b][(r0 + i) * E + c0 + c];
+                    *d = accum ? *d + g[i][b * CB + c] : g[i][b * CB + c];
+                }
+        if (has_b) {
+            float *d = &p.gwb[sE4 + el * 4 + jb];
+            *d = accum ? *d + gbe : gbe;
+        }
+    }
+}
+
+template <int E, int NW, int R>
+int launch_bwd(const SrwmBwdParams &p, hipStream_t s) {
+    hipLaunchKernelGGL((srwm_bwd_tiled_kernel<E, NW, R>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    return (int)hipGetLastError();
+}
+
+template <int E, int NW, int R>
+int launch_fwd(const SrwmFwdParams &p, hipStream_t s) {
+    hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    return (int)hipGetLastError();
+}
+
+bool aligned16(const void *ptr, int64_t a, int64_t b, int64_t c) {
+    return ((uintptr_t)ptr % 16 == 0) && a % 4 == 0 && b % 4 == 0 && c % 4 == 0;
+}
+
+}  // namespace
+
+int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
+    if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l)) return -1;
+    const void *dense[] = {p.q, p.k, p.beta, p.ydiff, p.qdiff, p.kdiff, p.bdiff, p.out};
+    for (const void *d : dense)
+        if ((uintptr_t)d % 16) return -1;
+    switch (p.E) {
+        case 64: return launch_fwd<64, 4, 8>(p, s);
+        case 32: return launch_fwd<32, 4, 4>(p, s);
+        case 16: return launch_fwd<16, 1, 2>(p, s);
+        case 8: return launch_fwd<8, 1, 1>(p, s);
+        default: return -1;
+    }
+}
+
+int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s) {
+    if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l) || !aligned16(p.go, p.gs_n, p.gs_h, p.gs_l)) return -1;
+    const void *dense[] = {p.q, p.k, p.beta, p.ydiff, p.qdiff, p.kdiff, p.bdiff, p.gx};
+    for (const void *d : dense)
+        if ((uintptr_t)d % 16) return -1;
+    switch (p.E) {
+        case 64: return launch_bwd<64, 4, 8>(p, s);
+        case 32: return launch_bwd<32, 4, 4>(p, s);
+        case 16: return launch_bwd<16, 1, 2>(p, s);
+        case 8: return launch_bwd<8, 1, 1>(p, s);
+        default: return -1;
+    }
+}
+
 }  // namespace fw
