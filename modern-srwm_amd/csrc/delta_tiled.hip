@@ -1,5 +1,392 @@
+// Register-resident delta-rule kernels for square memories (E == M = D in {8,16,32,64,128}).
+//
+// One workgroup of NW wave64s owns one (batch, head) sequence for all L steps; the D x D
+// memory W (and its gradient G in the backward) lives in registers, cut into tiles of
+// R rows x CC columns: lane (rg, cg) holds rows [R*rg, R*rg+R) of columns [CC*cg, CC*cg+CC).
+// The 8 lanes of a column group are consecutive, so every column sum (W^T k, W^T q, G^T k)
+// -- the only reductions the recurrence itself depends on -- finishes with three DPP adds
+// inside the wave.  Columns of the delta rule evolve independently, so the waves never
+// have to meet inside a step:
+//   forward   no workgroup barrier per step at all (one per input tile);
+//   backward  the row sums (grad_q, grad_k) and grad_beta are outputs only: each wave
+//             reduces its part with v_permlane{32,16}_swap, parks it in LDS, and the
+//             workgroup adds the per-wave parts once per tile and stores them coalesced.
+// The backward is ONE reverse sweep (the reference needs two plus a [N,H,L,M] temporary).
+//
+// Replaces fast_weight_forward_kernel, fast_weight_backward_value_beta_kernel and
+// fast_weight_backward_query_key_kernel of the reference
+// (supervised_learning/fast_weight/fast_weight_cuda.cu:17-178, :397-560, :244-393).
 #include "common.h"
+#include "xlane.h"
+
 namespace fw {
-int launch_delta_fwd_tiled(const DeltaFwdParams &, hipStream_t) { return -1; }
-int launch_delta_bwd_tiled(const DeltaBwdParams &, hipStream_t) { return -1; }
+
+namespace {
+
+template <int D, int NW, int R, int TT_>
+struct DTiling {
+    static constexpr int NT = NW * kWave;
+    static constexpr int RG = D / R;          // lanes per column group
+    static constexpr int CGW = kWave / RG;    // column groups per wave
+    static constexpr int NCG = NW * CGW;      // column groups per workgroup
+    static constexpr int CC = D / NCG;        // columns per lane
+    static constexpr int TT = TT_;            // steps per tile
+    static constexpr int NV4 = TT * D / 4;    // float4s per tile vector
+    static constexpr int LD = (NV4 + NT - 1) / NT;  // float4 loads per thread per vector
+    static_assert(RG == 8 && RG * R == D && CC * NCG == D && CC >= 1, "tiling");
+    static_assert(TT <= NT, "beta loader");
+};
+
+template <int N>
+__device__ __forceinline__ void rd(float (&dst)[N], const float *src) {
+    if constexpr (N % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < N / 4; ++i) {
+            const float4 v = reinterpret_cast<const float4 *>(src)[i];
+            dst[4 * i] = v.x; dst[4 * i + 1] = v.y; dst[4 * i + 2] = v.z; dst[4 * i + 3] = v.w;
+        }
+    } else if constexpr (N == 2) {
+        const float2 v = *reinterpret_cast<const float2 *>(src);
+        dst[0] = v.x; dst[1] = v.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) dst[i] = src[i];
+    }
+}
+
+template <int N>
+__device__ __forceinline__ void wr(float *dst, const float (&src)[N]) {
+    if constexpr (N == 4) {
+        *reinterpret_cast<float4 *>(dst) = make_float4(src[0], src[1], src[2], src[3]);
+    } else if constexpr (N == 2) {
+        *reinterpret_cast<float2 *>(dst) = make_float2(src[0], src[1]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) dst[i] = src[i];
+    }
+}
+
+// One tile vector (TT steps x D floats) moved global -> registers -> LDS as float4s.
+template <class T>
+struct TileVec {
+    float4 r[T::LD];
+    __device__ __forceinline__ void load(const float *base, int64_t step_stride, int t0, int L, int tid) {
+#pragma unroll
+        for (int j = 0; j < T::LD; ++j) {
+            const int f = tid + j * T::NT;
+            const int row = f / (T::NV4 / T::TT), col = (f % (T::NV4 / T::TT)) * 4;
+            const bool ok = f < T::NV4 && t0 + row < L;
+            r[j] = ok ? *reinterpret_cast<const float4 *>(base + (int64_t)(t0 + row) * step_stride + col)
+                      : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    __device__ __forceinline__ void store(float *lds, int tid) const {
+#pragma unroll
+        for (int j = 0; j < T::LD; ++j) {
+            const int f = tid + j * T::NT;
+            if (f < T::NV4) reinterpret_cast<float4 *>(lds)[f] = r[j];
+        }
+    }
+};
+
+template <int D, int NW, int R, int TT>
+__global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(DeltaFwdParams p) {
+    using T = DTiling<D, NW, R, TT>;
+    constexpr int RG = T::RG, CGW = T::CGW, CC = T::CC;
+    enum { VQ, VK, VV, NVEC };
+    __shared__ __attribute__((aligned(16))) float tl[2][NVEC][TT][D];
+    __shared__ float tbeta[2][TT];
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int rg = lane % RG, cg = wave * CGW + lane / RG;
+    const int r0 = rg * R, c0 = cg * CC;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const float *qb = p.Q + n * p.qs.n + h * p.qs.h;
+    const float *kb = p.K + n * p.ks.n + h * p.ks.h;
+    const float *vb = p.V + n * p.vs.n + h * p.vs.h;
+    const float *bb = p.beta + n * p.bs.n + h * p.bs.h;
+    float *Wg = p.W + seq * D * D;
+
+    float w[R][CC];
+#pragma unroll
+    for (int i = 0; i < R; ++i) rd<CC>(w[i], Wg + (r0 + i) * D + c0);
+
+    TileVec<T> nq, nk, nv;
+    float nb = 0.f;
+    auto load_tile = [&](int tile) {
+        const int t0 = tile * TT;
+        nq.load(qb, p.qs.l, t0, p.L, tid);
+        nk.load(kb, p.ks.l, t0, p.L, tid);
+        nv.load(vb, p.vs.l, t0, p.L, tid);
+        nb = (tid < TT && t0 + tid < p.L) ? bb[(int64_t)(t0 + tid) * p.bs.l] : 0.f;
+    };
+    auto store_tile = [&](int buf) {
+        nq.store(&tl[buf][VQ][0][0], tid);
+        nk.store(&tl[buf][VK][0][0], tid);
+        nv.store(&tl[buf][VV][0][0], tid);
+        if (tid < TT) tbeta[buf][tid] = nb;
+    };
+
+    const int ntiles = (p.L + TT - 1) / TT;
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    for (int tile = 0; tile < ntiles; ++tile) {
+        const int buf = tile & 1;
+        const int tlen = min(TT, p.L - tile * TT);
+        if (tile + 1 < ntiles) load_tile(tile + 1);
+
+        for (int tt = 0; tt < tlen; ++tt) {
+            const int64_t om = (seq * p.L + tile * TT + tt) * D + c0;
+            float kr[R], qr[R], vc[CC];
+            rd<R>(kr, &tl[buf][VK][tt][r0]);
+            rd<R>(qr, &tl[buf][VQ][tt][r0]);
+            rd<CC>(vc, &tl[buf][VV][tt][c0]);
+            const float b = tbeta[buf][tt];
+            // v_old = W^T k and W^T q in one pass over the tile, plus k.q
+            float vo[CC], oq[CC], kq = 0.f;
+#pragma unroll
+            for (int c = 0; c < CC; ++c) vo[c] = oq[c] = 0.f;
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                kq = fmaf(kr[i], qr[i], kq);
+#pragma unroll
+                for (int c = 0; c < CC; ++c) {
+                    vo[c] = fmaf(w[i][c], kr[i], vo[c]);
+                    oq[c] = fmaf(w[i][c], qr[i], oq[c]);
+                }
+            }
+            kq = group_sum<RG>(kq);
+            float ins[CC], out[CC];
+#pragma unroll
+            for (int c = 0; c < CC; ++c) {
+                vo[c] = group_sum<RG>(vo[c]);
+                oq[c] = group_sum<RG>(oq[c]);
+                ins[c] = b * (vc[c] - vo[c]);
+                out[c] = fmaf(kq, ins[c], oq[c]);  // (W + k (x) ins)^T q
+            }
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < CC; ++c) w[i][c] = fmaf(kr[i], ins[c], w[i][c]);
+            if (rg == 0) {
+                wr<CC>(p.vold + om, vo);
+                wr<CC>(p.vins + om, ins);
+                wr<CC>(p.out + om, out);
+            }
+        }
+        if (tile + 1 < ntiles) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+#pragma unroll
+    for (int i = 0; i < R; ++i) wr<CC>(Wg + (r0 + i) * D + c0, w[i]);
+}
+
+template <int D, int NW, int R, int TT>
+__global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(DeltaBwdParams p) {
+    using T = DTiling<D, NW, R, TT>;
+    constexpr int RG = T::RG, CGW = T::CGW, NCG = T::NCG, CC = T::CC, NT = T::NT;
+    enum { VQ, VK, VV, VVO, VVI, VGO, NVEC };
+    __shared__ __attribute__((aligned(16))) float tl[2][NVEC][TT][D];
+    __shared__ float tbeta[2][TT];
+    __shared__ __attribute__((aligned(16))) float rowq[TT][NW][D];  // per-wave parts of grad_q
+    __shared__ __attribute__((aligned(16))) float rowk[TT][NW][D];  // per-wave parts of grad_k
+    __shared__ float gbp[TT][NCG];                                  // per column group parts of grad_beta
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int rg = lane % RG, cg = wave * CGW + lane / RG;
+    const int r0 = rg * R, c0 = cg * CC;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const float *qb = p.Q + n * p.qs.n + h * p.qs.h;
+    const float *kb = p.K + n * p.ks.n + h * p.ks.h;
+    const float *vb = p.V + n * p.vs.n + h * p.vs.h;
+    const float *gob = p.go + n * p.gs.n + h * p.gs.h;
+    const float *bb = p.beta + n * p.bs.n + h * p.bs.h;
+    const float *vob = p.vold + seq * p.L * D;
+    const float *vib = p.vins + seq * p.L * D;
+    float *Wg = p.W + seq * D * D;
+    float *gWg = p.gW ? p.gW + seq * D * D : nullptr;
+    const bool g_in = gWg && p.grad_state_mode != 0u;
+
+    float w[R][CC], g[R][CC];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        rd<CC>(w[i], Wg + (r0 + i) * D + c0);
+        if (g_in) {
+            rd<CC>(g[i], gWg + (r0 + i) * D + c0);
+        } else {
+#pragma unroll
+            for (int c = 0; c < CC; ++c) g[i][c] = 0.f;
+        }
+    }
+
+    TileVec<T> nv[NVEC];
+    float nb = 0.f;
+    auto load_tile = [&](int tile) {
+        const int t0 = tile * TT;
+        nv[VQ].load(qb, p.qs.l, t0, p.L, tid);
+        nv[VK].load(kb, p.ks.l, t0, p.L, tid);
+        nv[VV].load(vb, p.vs.l, t0, p.L, tid);
+        nv[VVO].load(vob, D, t0, p.L, tid);
+        nv[VVI].load(vib, D, t0, p.L, tid);
+        nv[VGO].load(gob, p.gs.l, t0, p.L, tid);
+        nb = (tid < TT && t0 + tid < p.L) ? bb[(int64_t)(t0 + tid) * p.bs.l] : 0.f;
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int v = 0; v < NVEC; ++v) nv[v].store(&tl[buf][v][0][0], tid);
+        if (tid < TT) tbeta[buf][tid] = nb;
+    };
+
+    const int ntiles = (p.L + TT - 1) / TT;
+    load_tile(ntiles - 1);
+    store_tile((ntiles - 1) & 1);
+    __syncthreads();
+
+    for (int tile = ntiles - 1; tile >= 0; --tile) {
+        const int buf = tile & 1;
+        const int tlen = min(TT, p.L - tile * TT);
+        if (tile > 0) load_tile(tile - 1);
+
+        for (int tt = tlen - 1; tt >= 0; --tt) {
+            const int64_t om = (seq * p.L + tile * TT + tt) * D + c0;
+            float kr[R], qr[R], go[CC], vi[CC], dvv[CC], vo[CC];
+            rd<R>(kr, &tl[buf][VK][tt][r0]);
+            rd<R>(qr, &tl[buf][VQ][tt][r0]);
+            rd<CC>(go, &tl[buf][VGO][tt][c0]);
+            rd<CC>(vi, &tl[buf][VVI][tt][c0]);
+            rd<CC>(dvv, &tl[buf][VV][tt][c0]);
+            rd<CC>(vo, &tl[buf][VVO][tt][c0]);
+            const float b = tbeta[buf][tt];
+
+            // out_t = W_t^T q_t :  G += q (x) go ;  grad_q = W_t go
+            float aq[R], ak[R], r[CC];
+#pragma unroll
+            for (int c = 0; c < CC; ++c) r[c] = 0.f;
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                aq[i] = 0.f;
+                ak[i] = 0.f;
+#pragma unroll
+                for (int c = 0; c < CC; ++c) {
+                    g[i][c] = fmaf(qr[i], go[c], g[i][c]);
+                    aq[i] = fmaf(w[i][c], go[c], aq[i]);
+                    r[c] = fmaf(g[i][c], kr[i], r[c]);      // dL/d ins = G^T k
+                    ak[i] = fmaf(g[i][c], vi[c], ak[i]);    // grad_k, part through the write
+                }
+            }
+            float gvo[CC], gv[CC], pb = 0.f;
+#pragma unroll
+            for (int c = 0; c < CC; ++c) {
+                r[c] = group_sum<RG>(r[c]);
+                gv[c] = b * r[c];
+                gvo[c] = -gv[c];                            // dL/dv_old
+                pb = fmaf(r[c], dvv[c] - vo[c], pb);
+            }
+            // revert the write, then the part of grad_k through v_old = W_{t-1}^T k
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < CC; ++c) {
+                    w[i][c] = fmaf(-kr[i], vi[c], w[i][c]);
+                    ak[i] = fmaf(w[i][c], gvo[c], ak[i]);
+                    g[i][c] = fmaf(kr[i], gvo[c], g[i][c]);
+                }
+            stride8_reduce_store<R>(aq, &rowq[tt][wave][r0], lane);
+            stride8_reduce_store<R>(ak, &rowk[tt][wave][r0], lane);
+            if (rg == 0) {
+                wr<CC>(p.gV + om, gv);
+                gbp[tt][cg] = pb;
+            }
+        }
+        __syncthreads();
+        // add the per-wave parts of this tile and store grad_q, grad_k, grad_beta coalesced
+        for (int idx = tid; idx < tlen * D; idx += NT) {
+            const int tt = idx / D, e = idx - tt * D;
+            float sq = 0.f, sk = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < NW; ++wv) {
+                sq += rowq[tt][wv][e];
+                sk += rowk[tt][wv][e];
+            }
+            const int64_t oe = (seq * p.L + tile * TT + tt) * D + e;
+            p.gQ[oe] = sq;
+            p.gK[oe] = sk;
+        }
+        if (tid < tlen) {
+            float s = 0.f;
+#pragma unroll
+            for (int c = 0; c < NCG; ++c) s += gbp[tid][c];
+            p.gbeta[seq * p.L + tile * TT + tid] = s;
+        }
+        if (tile > 0) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    const bool accum = gWg && p.grad_state_mode == 2u;
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        wr<CC>(Wg + (r0 + i) * D + c0, w[i]);
+        if (gWg) {
+            float *d = gWg + (r0 + i) * D + c0;
+#pragma unroll
+            for (int c = 0; c < CC; ++c) d[c] = accum ? d[c] + g[i][c] : g[i][c];
+        }
+    }
+}
+
+template <int D, int NW, int R, int TT>
+int launch_f(const DeltaFwdParams &p, hipStream_t s) {
+    hipLaunchKernelGGL((delta_fwd_tiled_kernel<D, NW, R, TT>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    return (int)hipGetLastError();
+}
+
+template <int D, int NW, int R, int TT>
+int launch_b(const DeltaBwdParams &p, hipStream_t s) {
+    hipLaunchKernelGGL((delta_bwd_tiled_kernel<D, NW, R, TT>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    return (int)hipGetLastError();
+}
+
+bool ok16(const void *ptr, const Strided3 &s) {
+    return ((uintptr_t)ptr % 16 == 0) && s.n % 4 == 0 && s.h % 4 == 0 && s.l % 4 == 0;
+}
+
+bool ok16(const void *ptr) { return (uintptr_t)ptr % 16 == 0; }
+
+}  // namespace
+
+int launch_delta_fwd_tiled(const DeltaFwdParams &p, hipStream_t s) {
+    if (p.E != p.M) return -1;
+    if (!ok16(p.Q, p.qs) || !ok16(p.K, p.ks) || !ok16(p.V, p.vs) || !ok16(p.vold) || !ok16(p.vins) ||
+        !ok16(p.out) || !ok16(p.W))
+        return -1;
+    switch (p.E) {
+        case 128: return launch_f<128, 8, 16, 8>(p, s);
+        case 64: return launch_f<64, 4, 8, 16>(p, s);
+        case 32: return launch_f<32, 2, 4, 16>(p, s);
+        case 16: return launch_f<16, 1, 2, 16>(p, s);
+        case 8: return launch_f<8, 1, 1, 32>(p, s);
+        default: return -1;
+    }
+}
+
+int launch_delta_bwd_tiled(const DeltaBwdParams &p, hipStream_t s) {
+    if (p.E != p.M) return -1;
+    if (!ok16(p.Q, p.qs) || !ok16(p.K, p.ks) || !ok16(p.V, p.vs) || !ok16(p.go, p.gs) || !ok16(p.vold) ||
+        !ok16(p.vins) || !ok16(p.W) || !ok16(p.gV) || (p.gW && !ok16(p.gW)))
+        return -1;
+    switch (p.E) {
+        case 128: return launch_b<128, 8, 16, 8>(p, s);
+        case 64: return launch_b<64, 4, 8, 8>(p, s);
+        case 32: return launch_b<32, 2, 4, 16>(p, s);
+        case 16: return launch_b<16, 1, 2, 16>(p, s);
+        case 8: return launch_b<8, 1, 1, 32>(p, s);
+        default: return -1;
+    }
+}
+
 }  // namespace fw
