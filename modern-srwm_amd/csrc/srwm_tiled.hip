@@ -105,9 +105,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     // tile loader: thread -> (step tid / (E/4), 4 consecutive elements)
     const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
     auto load_tile = [&](int tile) -> float4 {
-        const int t = tile * TT + ld_row;
-        if (t < p.L) return *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col);
-        return make_float4(0.f, 0.f, 0.f, 0.f);
+        const int t = min(tile * TT + ld_row, p.L - 1);  // rows past the end: loaded, never used
+        return *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col);
     };
     const int ntiles = (p.L + TT - 1) / TT;
     *reinterpret_cast<float4 *>(&xt[0][ld_row][ld_col]) = load_tile(0);
@@ -269,49 +268,46 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     float gbe = (has_b && p.grad_state_mode) ? p.gwb[sE4 + el * 4 + jb] : 0.f;
 
     const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
-    struct TileRegs {
-        float4 v[NVEC];
-        float4 b, bd;
-    };
-    auto load_tile = [&](int tile) -> TileRegs {
-        TileRegs r;
-        const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
-        const int t = tile * TT + ld_row;
-        const bool ok = t < p.L;
-        const int64_t o = (seq * p.L + t) * E + ld_col;
-        r.v[VX] = ok ? *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col) : z;
-        r.v[VGO] = ok ? *reinterpret_cast<const float4 *>(gobase + t * p.gs_l + ld_col) : z;
-        r.v[VQ] = ok ? *reinterpret_cast<const float4 *>(p.q + o) : z;
-        r.v[VK] = ok ? *reinterpret_cast<const float4 *>(p.k + o) : z;
-        r.v[VYD] = ok ? *reinterpret_cast<const float4 *>(p.ydiff + o) : z;
-        r.v[VQD] = ok ? *reinterpret_cast<const float4 *>(p.qdiff + o) : z;
-        r.v[VKD] = ok ? *reinterpret_cast<const float4 *>(p.kdiff + o) : z;
-        r.b = z;
-        r.bd = z;
-        const int tb_t = tile * TT + tid;
-        if (tid < TT && tb_t < p.L) {
-            r.b = *reinterpret_cast<const float4 *>(p.beta + (seq * p.L + tb_t) * 4);
-            r.bd = *reinterpret_cast<const float4 *>(p.bdiff + (seq * p.L + tb_t) * 4);
-        }
-        return r;
-    };
-    auto store_tile = [&](const TileRegs &r) {
-#pragma unroll
-        for (int v = 0; v < NVEC; ++v) *reinterpret_cast<float4 *>(&tl[v][ld_row][ld_col]) = r.v[v];
-        if (tid < TT) {
-            *reinterpret_cast<float4 *>(&tb[0][tid][0]) = r.b;
-            *reinterpret_cast<float4 *>(&tb[1][tid][0]) = r.bd;
-        }
-    };
+    // next tile, staged in registers
+    float4 n_x, n_go, n_q, n_k, n_yd, n_qd, n_kd, n_bt, n_bd;
+#define SRWM_BWD_LOAD_TILE(tile_)                                                                  \
+    do { /* rows past the end of the sequence are clamped: they are loaded but never used */       \
+        const int t_ = min((tile_) * TT + ld_row, p.L - 1);                                        \
+        const int64_t o_ = (seq * p.L + t_) * E + ld_col;                                          \
+        n_x = *reinterpret_cast<const float4 *>(xbase + t_ * p.xs_l + ld_col);                     \
+        n_go = *reinterpret_cast<const float4 *>(gobase + t_ * p.gs_l + ld_col);                   \
+        n_q = *reinterpret_cast<const float4 *>(p.q + o_);                                         \
+        n_k = *reinterpret_cast<const float4 *>(p.k + o_);                                         \
+        n_yd = *reinterpret_cast<const float4 *>(p.ydiff + o_);                                    \
+        n_qd = *reinterpret_cast<const float4 *>(p.qdiff + o_);                                    \
+        n_kd = *reinterpret_cast<const float4 *>(p.kdiff + o_);                                    \
+        const int64_t ob_ = (seq * p.L + min((tile_) * TT + (tid % TT), p.L - 1)) * 4;             \
+        n_bt = *reinterpret_cast<const float4 *>(p.beta + ob_);                                    \
+        n_bd = *reinterpret_cast<const float4 *>(p.bdiff + ob_);                                   \
+    } while (0)
+#define SRWM_BWD_STORE_TILE()                                                                      \
+    do {                                                                                           \
+        *reinterpret_cast<float4 *>(&tl[VX][ld_row][ld_col]) = n_x;                                \
+        *reinterpret_cast<float4 *>(&tl[VGO][ld_row][ld_col]) = n_go;                              \
+        *reinterpret_cast<float4 *>(&tl[VQ][ld_row][ld_col]) = n_q;                                \
+        *reinterpret_cast<float4 *>(&tl[VK][ld_row][ld_col]) = n_k;                                \
+        *reinterpret_cast<float4 *>(&tl[VYD][ld_row][ld_col]) = n_yd;                              \
+        *reinterpret_cast<float4 *>(&tl[VQD][ld_row][ld_col]) = n_qd;                              \
+        *reinterpret_cast<float4 *>(&tl[VKD][ld_row][ld_col]) = n_kd;                              \
+        if (tid < TT) {                                                                            \
+            *reinterpret_cast<float4 *>(&tb[0][tid][0]) = n_bt;                                    \
+            *reinterpret_cast<float4 *>(&tb[1][tid][0]) = n_bd;                                    \
+        }                                                                                          \
+    } while (0)
 
     const int ntiles = (p.L + TT - 1) / TT;
-    store_tile(load_tile(ntiles - 1));
+    SRWM_BWD_LOAD_TILE(ntiles - 1);
+    SRWM_BWD_STORE_TILE();
     __syncthreads();
 
     for (int tile = ntiles - 1; tile >= 0; --tile) {
         const int tlen = min(TT, p.L - tile * TT);
-        TileRegs nxt;
-        if (tile > 0) nxt = load_tile(tile - 1);
+        if (tile > 0) SRWM_BWD_LOAD_TILE(tile - 1);
 
         for (int tt = tlen - 1; tt >= 0; --tt) {
             const int t = tile * TT + tt;
@@ -454,7 +450,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             if (tt == 0 && tile > 0) {
                 // every wave is past its last read of this tile (all reads precede the
                 // first barrier of the step)
-                store_tile(nxt);
+                SRWM_BWD_STORE_TILE();
                 __syncthreads();
             }
         }
