@@ -38,6 +38,7 @@ WORKLOADS = {
     "srwm_c3": ("srwm", 32, 8, 100, 32),
     "delta_c2": ("delta", 32, 8, 256, 64),
     "delta_c5f32": ("delta", 8, 16, 4096, 128),
+    "delta_c5": ("delta_bf16", 8, 16, 4096, 128),     # bf16 q/k/v/beta/out/grads, fp32 memory
 }
 
 
@@ -74,8 +75,9 @@ def srwm_step(t, ev=None):
         ev[2].record()
 
 
-def delta_setup(N, H, L, E, dev):
+def delta_setup(N, H, L, E, dev, io=None):
     import torch
+    io = io or torch.float32
     g = torch.Generator().manual_seed(0)
     M = E
     if E >= 128:
@@ -88,13 +90,13 @@ def delta_setup(N, H, L, E, dev):
     v = torch.randn(N, H, L, M, generator=g)
     beta = torch.sigmoid(torch.randn(N, H, L, 1, generator=g))
     go = torch.randn(N, H, L, M, generator=g)
-    t = dict(q=q.to(dev), k=k.to(dev), v=v.to(dev), beta=beta.to(dev), go=go.to(dev))
+    t = dict(q=q.to(dev, io), k=k.to(dev, io), v=v.to(dev, io), beta=beta.to(dev, io), go=go.to(dev, io))
     t["W"] = torch.empty(N, H, E, M, device=dev)
-    bigm = lambda: torch.empty(N, H, L, M, device=dev)
-    bige = lambda: torch.empty(N, H, L, E, device=dev)
-    t["vold"], t["vins"], t["out"] = bigm(), bigm(), bigm()
-    t["gq"], t["gk"], t["gv"] = bige(), bige(), bigm()
-    t["gb"] = torch.empty(N, H, L, 1, device=dev)
+    bigm = lambda dt=torch.float32: torch.empty(N, H, L, M, device=dev, dtype=dt)
+    bige = lambda: torch.empty(N, H, L, E, device=dev, dtype=io)
+    t["vold"], t["vins"], t["out"] = bigm(), bigm(), bigm(io)
+    t["gq"], t["gk"], t["gv"] = bige(), bige(), bigm(io)
+    t["gb"] = torch.empty(N, H, L, 1, device=dev, dtype=io)
     return t
 
 
@@ -119,7 +121,11 @@ def algorithmic_bytes(op, N, H, L, E):
         S = E * (3 * E + 4)
         return 3 * S * 4 * hs, 6 * S * 4 * hs, (15 * E + 16) * 4 * hs + 4 * S * 4 * N * H
     S = E * E
-    return 2 * S * 4 * hs, 4 * S * 4 * hs, (6 * E + 9 * E + 3) * 4 * hs + 3 * S * 4 * N * H
+    # per (sequence, step): q,k,v,beta in (fwd and bwd), out + grad_out, 3 E-wide grads in the I/O
+    # type; v_old, v_insert written and read back in fp32
+    b = 2 if op == "delta_bf16" else 4
+    io_elems = 2 * (3 * E + 1) + 2 * E + 3 * E + 1
+    return 2 * S * 4 * hs, 4 * S * 4 * hs, (io_elems * b + 4 * E * 4) * hs + 3 * S * 4 * N * H
 
 
 def cpu_baseline(op, N, H, L, E, budget_s=20.0):
@@ -181,8 +187,11 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     op, N, H, L, E = WORKLOADS[a.workload]
-    setup, step = (srwm_setup, srwm_step) if op == "srwm" else (delta_setup, delta_step)
-    t = setup(N, H, L, E, dev)
+    if op == "srwm":
+        step, t = srwm_step, srwm_setup(N, H, L, E, dev)
+    else:
+        step = delta_step
+        t = delta_setup(N, H, L, E, dev, torch.bfloat16 if op == "delta_bf16" else torch.float32)
 
     for _ in range(a.warmup):
         step(t)
@@ -211,16 +220,17 @@ def main():
                   if a.workload == "srwm_c4" else f"fwd+bwd tokens/sec {a.workload}",
         "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{a.workload}: {op} fwd+bwd N={N} H={H} L={L} E={E} fp32, "
-                               "state re-initialised per step, x~N(0,1), W0~N(0,0.02), grad~N(0,1)"},
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32" if op != "delta_bf16" else "f32 (bf16 I/O)",
+        "data": "synthetic",
+        "config": {"workload": f"{a.workload}: {op} fwd+bwd N={N} H={H} L={L} E={E}, fp32 state, "
+                               "state re-initialised per step, seeded synthetic inputs"},
         "kernel_ms": {"forward": round(fwd_ms, 4), "backward": round(bwd_ms, 4)},
         "roofline": dict(roof("lds", lds_b, bwd_ms, LDS_PEAK_GBS), kernel="backward"),
         "roofline_fwd_bwd": roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS),
         "roofline_hbm": roof("hbm", hbm, fwd_ms + bwd_ms, HBM_PEAK_GBS),
     }
     if not a.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline(op, N, H, L, E, a.cpu_budget)
+        res["cpu_baseline"] = cpu_baseline("srwm" if op == "srwm" else "delta", N, H, L, E, a.cpu_budget)
     print(json.dumps(res))
 
 

@@ -35,6 +35,8 @@ extern "C" {
 #define SRWM_EINVAL (-1)   /* null pointer, non-positive size, bad flag combination */
 #define SRWM_ESIZE (-2)    /* E / M not supported by any kernel (state does not fit in LDS) */
 #define SRWM_ESTRIDE (-3)  /* stride makes an access misaligned or overflows 32-bit indexing */
+#define SRWM_ENOKERNEL (-4) /* no kernel for this combination (bf16 I/O needs E == M in {8,16,32,64,128}
+                               and rows aligned to 8 bytes) */
 
 /* backward: what the grad-state buffers hold on entry / exit */
 #define SRWM_GRAD_STATE_ZERO 0u   /* entry contents ignored (dL/dW_L = 0); exit: dL/dW_0 */
@@ -119,6 +121,31 @@ SRWM_API int delta_backward_f32(const float *Q, const int64_t q_strides[3],
                        float *W,
                        float *gQ, float *gK, float *gV, float *gbeta, float *gW,
                        int N, int H, int L, int E, int M, unsigned flags, void *stream);
+
+/*
+ * Delta rule with bf16 inputs/outputs and fp32 memory.  No counterpart in the reference
+ * (its kernels are float-only, fast_weight_cuda.cu:12-14); same recurrence as
+ * delta_forward_f32 / delta_backward_f32 with
+ *   Q, K, V, beta, out, grad_out, gQ, gK, gV, gbeta    bf16 (raw 16-bit patterns)
+ *   W, gW, v_old, v_insert                              fp32
+ * All arithmetic is fp32; inputs are widened on load, outputs rounded to nearest even.
+ */
+SRWM_API int delta_forward_bf16(const uint16_t *Q, const int64_t q_strides[3],
+                       const uint16_t *K, const int64_t k_strides[3],
+                       const uint16_t *V, const int64_t v_strides[3],
+                       const uint16_t *beta, const int64_t beta_strides[3],
+                       float *v_old, float *v_insert, float *W, uint16_t *out,
+                       int N, int H, int L, int E, int M, unsigned flags, void *stream);
+
+SRWM_API int delta_backward_bf16(const uint16_t *Q, const int64_t q_strides[3],
+                        const uint16_t *K, const int64_t k_strides[3],
+                        const uint16_t *V, const int64_t v_strides[3],
+                        const uint16_t *beta, const int64_t beta_strides[3],
+                        const float *v_old, const float *v_insert,
+                        const uint16_t *grad_out, const int64_t grad_out_strides[3],
+                        float *W,
+                        uint16_t *gQ, uint16_t *gK, uint16_t *gV, uint16_t *gbeta, float *gW,
+                        int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
 /* Largest E the SRWM entry points accept (forward / backward), and the largest
  * E == M the delta entry points accept, on the current device. */

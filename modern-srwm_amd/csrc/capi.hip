@@ -52,6 +52,7 @@ const char *srwm_hip_strerror(int code) {
         case SRWM_EINVAL: return "invalid argument (null pointer, non-positive size or bad flags)";
         case SRWM_ESIZE: return "head size not supported: the state does not fit in the CU's LDS";
         case SRWM_ESTRIDE: return "unsupported stride";
+        case SRWM_ENOKERNEL: return "no kernel for this dtype / size / alignment combination";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown srwm_hip error";
     }
 }
@@ -160,6 +161,46 @@ int delta_backward_f32(const float *Q, const int64_t qs[3], const float *K, cons
     }
     if (delta_bwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_delta_bwd_generic(p, s);
+}
+
+int delta_forward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K, const int64_t ks[3],
+                       const uint16_t *V, const int64_t vs[3], const uint16_t *beta, const int64_t bs[3],
+                       float *v_old, float *v_insert, float *W, uint16_t *out, int N, int H, int L,
+                       int E, int M, unsigned flags, void *stream) {
+    if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
+        return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || flags) return SRWM_EINVAL;
+    if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
+        !stride_ok(bs, N, H, L, 1))
+        return SRWM_ESTRIDE;
+    DeltaFwdParamsBf16 p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
+                         {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
+                         N, H, L, E, M};
+    const int r = launch_delta_fwd_tiled_bf16(p, (hipStream_t)stream);
+    return r >= 0 ? r : SRWM_ENOKERNEL;
+}
+
+int delta_backward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K, const int64_t ks[3],
+                        const uint16_t *V, const int64_t vs[3], const uint16_t *beta,
+                        const int64_t bs[3], const float *v_old, const float *v_insert,
+                        const uint16_t *grad_out, const int64_t gs[3], float *W, uint16_t *gQ,
+                        uint16_t *gK, uint16_t *gV, uint16_t *gbeta, float *gW, int N, int H, int L,
+                        int E, int M, unsigned flags, void *stream) {
+    if (!Q || !K || !V || !beta || !v_old || !v_insert || !grad_out || !W || !gQ || !gK || !gV ||
+        !gbeta || !qs || !ks || !vs || !bs || !gs)
+        return SRWM_EINVAL;
+    const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u || (flags & ~SRWM_GRAD_STATE_MASK))
+        return SRWM_EINVAL;
+    if (!gW && mode != SRWM_GRAD_STATE_ZERO) return SRWM_EINVAL;
+    if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
+        !stride_ok(bs, N, H, L, 1) || !stride_ok(gs, N, H, L, M))
+        return SRWM_ESTRIDE;
+    DeltaBwdParamsBf16 p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
+                         {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, grad_out,
+                         {gs[0], gs[1], gs[2]}, W, gQ, gK, gV, gbeta, gW, N, H, L, E, M, mode};
+    const int r = launch_delta_bwd_tiled_bf16(p, (hipStream_t)stream);
+    return r >= 0 ? r : SRWM_ENOKERNEL;
 }
 
 }  // extern "C"

@@ -50,6 +50,28 @@ struct DeltaBwdParams {
     unsigned grad_state_mode;
 };
 
+// bf16 I/O (16-bit patterns), fp32 memory / saved vectors
+struct DeltaFwdParamsBf16 {
+    const uint16_t *Q, *K, *V, *beta;
+    Strided3 qs, ks, vs, bs;
+    float *vold, *vins, *W;
+    uint16_t *out;
+    int N, H, L, E, M;
+};
+
+struct DeltaBwdParamsBf16 {
+    const uint16_t *Q, *K, *V, *beta;
+    Strided3 qs, ks, vs, bs;
+    const float *vold, *vins;
+    const uint16_t *go;
+    Strided3 gs;
+    float *W;
+    uint16_t *gQ, *gK, *gV, *gbeta;
+    float *gW;
+    int N, H, L, E, M;
+    unsigned grad_state_mode;
+};
+
 // ---- wave64 all-reduce helpers (every lane receives the result) -----------------
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
@@ -79,6 +101,8 @@ int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s);
 int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s);
 int launch_delta_fwd_tiled(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_bwd_tiled(const DeltaBwdParams &p, hipStream_t s);
+int launch_delta_fwd_tiled_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s);
+int launch_delta_bwd_tiled_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s);
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // gfx950: 160 KB of LDS per CU / workgroup
 

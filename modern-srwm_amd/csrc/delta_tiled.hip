@@ -66,18 +66,48 @@ __device__ __forceinline__ void wr(float *dst, const float (&src)[N]) {
     }
 }
 
-// One tile vector (TT steps x D floats) moved global -> registers -> LDS as float4s.
+// bf16 <-> fp32 (round to nearest even); bf16 travels as its 16-bit pattern
+typedef uint16_t bf16_t;
+__device__ __forceinline__ float bf2f(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ uint32_t f2bf(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float ld1(const float *p) { return *p; }
+__device__ __forceinline__ float ld1(const bf16_t *p) { return bf2f(*p); }
+__device__ __forceinline__ void st1(float *p, float v) { *p = v; }
+__device__ __forceinline__ void st1(bf16_t *p, float v) { *p = (bf16_t)f2bf(v); }
+__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ __forceinline__ float4 ld4(const bf16_t *p) {
+    const uint2 u = *reinterpret_cast<const uint2 *>(p);
+    return make_float4(bf2f(u.x & 0xFFFFu), bf2f(u.x >> 16), bf2f(u.y & 0xFFFFu), bf2f(u.y >> 16));
+}
+
+template <int N>
+__device__ __forceinline__ void wr(bf16_t *dst, const float (&src)[N]) {
+    if constexpr (N == 4) {
+        *reinterpret_cast<uint2 *>(dst) =
+            make_uint2(f2bf(src[0]) | (f2bf(src[1]) << 16), f2bf(src[2]) | (f2bf(src[3]) << 16));
+    } else if constexpr (N == 2) {
+        *reinterpret_cast<uint32_t *>(dst) = f2bf(src[0]) | (f2bf(src[1]) << 16);
+    } else {
+#pragma unroll
+        for (int i = 0; i < N; ++i) dst[i] = (bf16_t)f2bf(src[i]);
+    }
+}
+
+// One tile vector (TT steps x D elements) moved global -> registers (as fp32) -> LDS as float4s.
+// Rows past the end of the sequence are clamped to the last one: loaded, never used.
 template <class T>
 struct TileVec {
     float4 r[T::LD];
-    __device__ __forceinline__ void load(const float *base, int64_t step_stride, int t0, int L, int tid) {
+    template <class TI>
+    __device__ __forceinline__ void load(const TI *base, int64_t step_stride, int t0, int L, int tid) {
 #pragma unroll
         for (int j = 0; j < T::LD; ++j) {
-            const int f = tid + j * T::NT;
-            const int row = f / (T::NV4 / T::TT), col = (f % (T::NV4 / T::TT)) * 4;
-            const bool ok = f < T::NV4 && t0 + row < L;
-            r[j] = ok ? *reinterpret_cast<const float4 *>(base + (int64_t)(t0 + row) * step_stride + col)
-                      : make_float4(0.f, 0.f, 0.f, 0.f);
+            const int f = min(tid + j * T::NT, T::NV4 - 1);
+            const int row = min(t0 + f / (T::NV4 / T::TT), L - 1), col = (f % (T::NV4 / T::TT)) * 4;
+            r[j] = ld4(base + (int64_t)row * step_stride + col);
         }
     }
     __device__ __forceinline__ void store(float *lds, int tid) const {
@@ -89,8 +119,32 @@ struct TileVec {
     }
 };
 
-template <int D, int NW, int R, int TT>
-__global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(DeltaFwdParams p) {
+// Parameter blocks with the I/O element type TI (float or bf16_t) made explicit.  The memory
+// W, its gradient and the saved v_old / v_insert are always fp32.
+template <class TI>
+struct FwdP {
+    const TI *Q, *K, *V, *beta;
+    Strided3 qs, ks, vs, bs;
+    float *vold, *vins, *W;
+    TI *out;
+    int N, H, L;
+};
+template <class TI>
+struct BwdP {
+    const TI *Q, *K, *V, *beta;
+    Strided3 qs, ks, vs, bs;
+    const float *vold, *vins;
+    const TI *go;
+    Strided3 gs;
+    float *W;
+    TI *gQ, *gK, *gV, *gbeta;
+    float *gW;
+    int N, H, L;
+    unsigned grad_state_mode;
+};
+
+template <class TI, int D, int NW, int R, int TT>
+__global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) {
     using T = DTiling<D, NW, R, TT>;
     constexpr int RG = T::RG, CGW = T::CGW, CC = T::CC;
     enum { VQ, VK, VV, NVEC };
@@ -102,10 +156,10 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(DeltaFwdPara
     const int r0 = rg * R, c0 = cg * CC;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
-    const float *qb = p.Q + n * p.qs.n + h * p.qs.h;
-    const float *kb = p.K + n * p.ks.n + h * p.ks.h;
-    const float *vb = p.V + n * p.vs.n + h * p.vs.h;
-    const float *bb = p.beta + n * p.bs.n + h * p.bs.h;
+    const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;
+    const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
+    const TI *vb = p.V + n * p.vs.n + h * p.vs.h;
+    const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
     float *Wg = p.W + seq * D * D;
 
     float w[R][CC];
@@ -119,7 +173,7 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(DeltaFwdPara
         nq.load(qb, p.qs.l, t0, p.L, tid);
         nk.load(kb, p.ks.l, t0, p.L, tid);
         nv.load(vb, p.vs.l, t0, p.L, tid);
-        nb = (tid < TT && t0 + tid < p.L) ? bb[(int64_t)(t0 + tid) * p.bs.l] : 0.f;
+        nb = ld1(bb + (int64_t)min(t0 + (tid % TT), p.L - 1) * p.bs.l);
     };
     auto store_tile = [&](int buf) {
         nq.store(&tl[buf][VQ][0][0], tid);
@@ -185,8 +239,8 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(DeltaFwdPara
     for (int i = 0; i < R; ++i) wr<CC>(Wg + (r0 + i) * D + c0, w[i]);
 }
 
-template <int D, int NW, int R, int TT>
-__global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(DeltaBwdParams p) {
+template <class TI, int D, int NW, int R, int TT>
+__global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) {
     using T = DTiling<D, NW, R, TT>;
     constexpr int RG = T::RG, CGW = T::CGW, NCG = T::NCG, CC = T::CC, NT = T::NT;
     enum { VQ, VK, VV, VVO, VVI, VGO, NVEC };
@@ -201,11 +255,11 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(DeltaBwdPara
     const int r0 = rg * R, c0 = cg * CC;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
-    const float *qb = p.Q + n * p.qs.n + h * p.qs.h;
-    const float *kb = p.K + n * p.ks.n + h * p.ks.h;
-    const float *vb = p.V + n * p.vs.n + h * p.vs.h;
-    const float *gob = p.go + n * p.gs.n + h * p.gs.h;
-    const float *bb = p.beta + n * p.bs.n + h * p.bs.h;
+    const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;
+    const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
+    const TI *vb = p.V + n * p.vs.n + h * p.vs.h;
+    const TI *gob = p.go + n * p.gs.n + h * p.gs.h;
+    const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
     const float *vob = p.vold + seq * p.L * D;
     const float *vib = p.vins + seq * p.L * D;
     float *Wg = p.W + seq * D * D;
@@ -234,7 +288,7 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(DeltaBwdPara
         nv[VVO].load(vob, D, t0, p.L, tid);
         nv[VVI].load(vib, D, t0, p.L, tid);
         nv[VGO].load(gob, p.gs.l, t0, p.L, tid);
-        nb = (tid < TT && t0 + tid < p.L) ? bb[(int64_t)(t0 + tid) * p.bs.l] : 0.f;
+        nb = ld1(bb + (int64_t)min(t0 + (tid % TT), p.L - 1) * p.bs.l);
     };
     auto store_tile = [&](int buf) {
 #pragma unroll
@@ -314,14 +368,14 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(DeltaBwdPara
                 sk += rowk[tt][wv][e];
             }
             const int64_t oe = (seq * p.L + tile * TT + tt) * D + e;
-            p.gQ[oe] = sq;
-            p.gK[oe] = sk;
+            st1(p.gQ + oe, sq);
+            st1(p.gK + oe, sk);
         }
         if (tid < tlen) {
             float s = 0.f;
 #pragma unroll
             for (int c = 0; c < NCG; ++c) s += gbp[tid][c];
-            p.gbeta[seq * p.L + tile * TT + tid] = s;
+            st1(p.gbeta + seq * p.L + tile * TT + tid, s);
         }
         if (tile > 0) store_tile(buf ^ 1);
         __syncthreads();
@@ -339,54 +393,82 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(DeltaBwdPara
     }
 }
 
-template <int D, int NW, int R, int TT>
-int launch_f(const DeltaFwdParams &p, hipStream_t s) {
-    hipLaunchKernelGGL((delta_fwd_tiled_kernel<D, NW, R, TT>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+template <class TI, int D, int NW, int R, int TT>
+int launch_f(const FwdP<TI> &p, hipStream_t s) {
+    hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, NW, R, TT>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
-template <int D, int NW, int R, int TT>
-int launch_b(const DeltaBwdParams &p, hipStream_t s) {
-    hipLaunchKernelGGL((delta_bwd_tiled_kernel<D, NW, R, TT>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+template <class TI, int D, int NW, int R, int TT>
+int launch_b(const BwdP<TI> &p, hipStream_t s) {
+    hipLaunchKernelGGL((delta_bwd_tiled_kernel<TI, D, NW, R, TT>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
-bool ok16(const void *ptr, const Strided3 &s) {
-    return ((uintptr_t)ptr % 16 == 0) && s.n % 4 == 0 && s.h % 4 == 0 && s.l % 4 == 0;
+// rows are read as 4-element vectors: 16-byte aligned for fp32, 8-byte for bf16
+template <class TI>
+bool row_ok(const TI *ptr, const Strided3 &s) {
+    return ((uintptr_t)ptr % (4 * sizeof(TI)) == 0) && s.n % 4 == 0 && s.h % 4 == 0 && s.l % 4 == 0;
 }
-
 bool ok16(const void *ptr) { return (uintptr_t)ptr % 16 == 0; }
+
+template <class TI>
+int dispatch_fwd(const FwdP<TI> &p, int D, hipStream_t s) {
+    if (!row_ok(p.Q, p.qs) || !row_ok(p.K, p.ks) || !row_ok(p.V, p.vs) || !ok16(p.vold) || !ok16(p.vins) ||
+        !ok16(p.out) || !ok16(p.W))
+        return -1;
+    switch (D) {
+        case 128: return launch_f<TI, 128, 8, 16, 8>(p, s);
+        case 64: return launch_f<TI, 64, 4, 8, 16>(p, s);
+        case 32: return launch_f<TI, 32, 2, 4, 16>(p, s);
+        case 16: return launch_f<TI, 16, 1, 2, 16>(p, s);
+        case 8: return launch_f<TI, 8, 1, 1, 32>(p, s);
+        default: return -1;
+    }
+}
+
+template <class TI>
+int dispatch_bwd(const BwdP<TI> &p, int D, hipStream_t s) {
+    if (!row_ok(p.Q, p.qs) || !row_ok(p.K, p.ks) || !row_ok(p.V, p.vs) || !row_ok(p.go, p.gs) ||
+        !ok16(p.vold) || !ok16(p.vins) || !ok16(p.W) || !ok16(p.gV) || !ok16(p.gQ) || !ok16(p.gK) ||
+        (p.gW && !ok16(p.gW)))
+        return -1;
+    switch (D) {
+        case 128: return launch_b<TI, 128, 8, 16, 8>(p, s);
+        case 64: return launch_b<TI, 64, 4, 8, 8>(p, s);
+        case 32: return launch_b<TI, 32, 2, 4, 16>(p, s);
+        case 16: return launch_b<TI, 16, 1, 2, 16>(p, s);
+        case 8: return launch_b<TI, 8, 1, 1, 32>(p, s);
+        default: return -1;
+    }
+}
 
 }  // namespace
 
 int launch_delta_fwd_tiled(const DeltaFwdParams &p, hipStream_t s) {
     if (p.E != p.M) return -1;
-    if (!ok16(p.Q, p.qs) || !ok16(p.K, p.ks) || !ok16(p.V, p.vs) || !ok16(p.vold) || !ok16(p.vins) ||
-        !ok16(p.out) || !ok16(p.W))
-        return -1;
-    switch (p.E) {
-        case 128: return launch_f<128, 8, 16, 8>(p, s);
-        case 64: return launch_f<64, 4, 8, 16>(p, s);
-        case 32: return launch_f<32, 2, 4, 16>(p, s);
-        case 16: return launch_f<16, 1, 2, 16>(p, s);
-        case 8: return launch_f<8, 1, 1, 32>(p, s);
-        default: return -1;
-    }
+    const FwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.N, p.H, p.L};
+    return dispatch_fwd(q, p.E, s);
 }
 
 int launch_delta_bwd_tiled(const DeltaBwdParams &p, hipStream_t s) {
     if (p.E != p.M) return -1;
-    if (!ok16(p.Q, p.qs) || !ok16(p.K, p.ks) || !ok16(p.V, p.vs) || !ok16(p.go, p.gs) || !ok16(p.vold) ||
-        !ok16(p.vins) || !ok16(p.W) || !ok16(p.gV) || (p.gW && !ok16(p.gW)))
-        return -1;
-    switch (p.E) {
-        case 128: return launch_b<128, 8, 16, 8>(p, s);
-        case 64: return launch_b<64, 4, 8, 8>(p, s);
-        case 32: return launch_b<32, 2, 4, 16>(p, s);
-        case 16: return launch_b<16, 1, 2, 16>(p, s);
-        case 8: return launch_b<8, 1, 1, 32>(p, s);
-        default: return -1;
-    }
+    const BwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
+                        p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode};
+    return dispatch_bwd(q, p.E, s);
+}
+
+int launch_delta_fwd_tiled_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s) {
+    if (p.E != p.M) return -1;
+    const FwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.N, p.H, p.L};
+    return dispatch_fwd(q, p.E, s);
+}
+
+int launch_delta_bwd_tiled_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s) {
+    if (p.E != p.M) return -1;
+    const BwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
+                         p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode};
+    return dispatch_bwd(q, p.E, s);
 }
 
 }  // namespace fw

@@ -5,7 +5,8 @@ signature, same in-place semantics -- backed by libsrwm_hip.so.
     out = fast_weight_delta(Q, K, V, beta, W)
 
 Q, K: (N, H, L, E); V: (N, H, L, M); beta: (N, H, L, 1) (already sigmoid-ed); W: (N, H, E, M);
-float32 on the GPU.  W is OVERWRITTEN with the memory after the last step; the backward
+float32 on the GPU (bfloat16 Q, K, V, beta with a float32 W are accepted as well: outputs and
+gradients then come back in bfloat16, arithmetic and memory stay fp32).  W is OVERWRITTEN with the memory after the last step; the backward
 starts from it and leaves it reverted to its initial value, like the reference's kernels.
 No gradient is returned for W (the reference returns None).
 """
@@ -30,8 +31,8 @@ class DeltaFastWeight(torch.autograd.Function):
         N, H, L, E = Q.shape
         _, _, _, M = V.shape
         out = torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
-        V_old = torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
-        V_insert = torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
+        V_old = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
+        V_insert = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
         DeltaFastWeight.dot[device.type](Q.data, K.data, V.data, beta.data, V_old, V_insert, W, out)
         ctx.save_for_backward(Q, K, V, beta, V_old, V_insert, W)
         return out
@@ -43,6 +44,8 @@ class DeltaFastWeight(torch.autograd.Function):
         grad_K = torch.empty(K.shape, device=Q.device, dtype=Q.dtype)
         grad_V = torch.empty(V.shape, device=Q.device, dtype=Q.dtype)
         grad_beta = torch.empty(beta.shape, device=Q.device, dtype=Q.dtype)
+        if grad_out.dtype != Q.dtype:
+            grad_out = grad_out.to(Q.dtype)
         DeltaFastWeight.dot_backward[Q.device.type](
             Q.data, K.data, V.data, beta.data, V_old.data, V_insert.data, grad_out, W.data,
             grad_Q, grad_K, grad_V, grad_beta)

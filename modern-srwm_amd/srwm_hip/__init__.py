@@ -44,6 +44,8 @@ _SIGNATURES = {
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
     "delta_forward_f32": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_backward_f32": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_forward_bf16": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_backward_bf16": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
 }
 
 
@@ -92,13 +94,13 @@ def _check(code, what):
         raise RuntimeError(f"{what} failed with code {code}: {msg}")
 
 
-def _require(t, name, shape=None):
+def _require(t, name, shape=None, dtype=torch.float32):
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor")
     if t.device.type != "cuda":
         raise RuntimeError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
-    if t.dtype != torch.float32:
-        raise TypeError(f"{name} must be float32 (got {t.dtype})")
+    if t.dtype != dtype:
+        raise TypeError(f"{name} must be {dtype} (got {t.dtype})")
     if shape is not None and tuple(t.shape) != tuple(shape):
         raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
 
@@ -112,7 +114,7 @@ def _strided(t):
     16-byte aligned.  Anything else is copied."""
     ok = t.stride(-1) == 1 or t.shape[-1] == 1
     if ok and t.shape[-1] % 4 == 0:
-        ok = t.data_ptr() % 16 == 0 and all(s % 4 == 0 for s in t.stride()[:3])
+        ok = t.data_ptr() % (4 * t.element_size()) == 0 and all(s % 4 == 0 for s in t.stride()[:3])
     if not ok:
         t = t.contiguous()
     return t, (ctypes.c_int64 * 3)(*t.stride()[:3])
@@ -136,6 +138,10 @@ class _Dense:
                 if o is not w:
                     o.copy_(w)
         return False
+
+
+def _has_bf16_kernel(E, M):
+    return E == M and E in (8, 16, 32, 64, 128)
 
 
 def _stream(device):
@@ -200,25 +206,34 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
 
 
 def fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=0):
-    """Delta-rule forward.  kv ([N,H,E,M]) is overwritten with the final memory."""
-    _require(q, "q")
+    """Delta-rule forward.  kv ([N,H,E,M], fp32) is overwritten with the final memory.
+    q, k, v, beta and out are all float32 or all bfloat16; v_old, v_insert and kv are float32."""
+    io = q.dtype if isinstance(q, torch.Tensor) and q.dtype == torch.bfloat16 else torch.float32
+    _require(q, "q", None, io)
     N, H, L, E = q.shape
-    _require(k, "k", (N, H, L, E))
-    _require(v, "v")
+    _require(k, "k", (N, H, L, E), io)
+    _require(v, "v", None, io)
     M = v.shape[-1]
-    _require(v, "v", (N, H, L, M))
-    _require(beta, "beta", (N, H, L, 1))
-    for t, nm in ((v_old, "v_old"), (v_insert, "v_insert"), (out, "out")):
+    _require(v, "v", (N, H, L, M), io)
+    _require(beta, "beta", (N, H, L, 1), io)
+    _require(out, "out", (N, H, L, M), io)
+    for t, nm in ((v_old, "v_old"), (v_insert, "v_insert")):
         _require(t, nm, (N, H, L, M))
     _require(kv, "kv", (N, H, E, M))
     if q.numel() == 0 or v.numel() == 0:
         return
+    if io == torch.bfloat16 and not _has_bf16_kernel(E, M):
+        # no bf16 kernel for this size: widen, run the fp32 kernels, round the output
+        o32 = torch.empty(out.shape, device=out.device, dtype=torch.float32)
+        fast_weight_forward(q.float(), k.float(), v.float(), beta.float(), v_old, v_insert, kv, o32, flags)
+        out.copy_(o32)
+        return
+    fn = lib().delta_forward_bf16 if io == torch.bfloat16 else lib().delta_forward_f32
     (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr) = (_strided(t) for t in (q, k, v, beta))
     with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv, out], True) as d:
-        code = lib().delta_forward_f32(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
-                                       *[_ptr(t) for t in d], N, H, L, E, M, flags,
-                                       _stream(q.device))
-    _check(code, "delta_forward_f32")
+        code = fn(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
+                  *[_ptr(t) for t in d], N, H, L, E, M, flags, _stream(q.device))
+    _check(code, fn.__name__)
 
 
 def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v,
@@ -226,29 +241,40 @@ def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, g
     """Delta-rule backward.  kv must hold the final memory and is reverted to the initial
     one.  grad_kv (optional, beyond the reference's list): gradient of the memory, see
     the SRWM_GRAD_STATE_* flags."""
-    _require(q, "q")
+    io = q.dtype if isinstance(q, torch.Tensor) and q.dtype == torch.bfloat16 else torch.float32
+    _require(q, "q", None, io)
     N, H, L, E = q.shape
-    _require(k, "k", (N, H, L, E))
-    _require(v, "v")
+    _require(k, "k", (N, H, L, E), io)
+    _require(v, "v", None, io)
     M = v.shape[-1]
-    _require(beta, "beta", (N, H, L, 1))
-    for t, nm in ((v_old, "v_old"), (v_insert, "v_insert"), (grad_out, "grad_out"), (grad_v, "grad_v")):
+    _require(beta, "beta", (N, H, L, 1), io)
+    for t, nm in ((v_old, "v_old"), (v_insert, "v_insert")):
         _require(t, nm, (N, H, L, M))
+    for t, nm in ((grad_out, "grad_out"), (grad_v, "grad_v")):
+        _require(t, nm, (N, H, L, M), io)
     _require(kv, "kv", (N, H, E, M))
-    _require(grad_q, "grad_q", (N, H, L, E))
-    _require(grad_k, "grad_k", (N, H, L, E))
-    _require(grad_beta, "grad_beta", (N, H, L, 1))
+    _require(grad_q, "grad_q", (N, H, L, E), io)
+    _require(grad_k, "grad_k", (N, H, L, E), io)
+    _require(grad_beta, "grad_beta", (N, H, L, 1), io)
     if grad_kv is not None:
         _require(grad_kv, "grad_kv", (N, H, E, M))
     if q.numel() == 0 or v.numel() == 0:
         return
+    if io == torch.bfloat16 and not _has_bf16_kernel(E, M):
+        g32 = [torch.empty(t.shape, device=t.device, dtype=torch.float32)
+               for t in (grad_q, grad_k, grad_v, grad_beta)]
+        fast_weight_backward(q.float(), k.float(), v.float(), beta.float(), v_old, v_insert,
+                             grad_out.float(), kv, *g32, grad_kv=grad_kv, flags=flags)
+        for dst, src in zip((grad_q, grad_k, grad_v, grad_beta), g32):
+            dst.copy_(src)
+        return
+    fn = lib().delta_backward_bf16 if io == torch.bfloat16 else lib().delta_backward_f32
     (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr), (gos, gstr) = (
         _strided(t) for t in (q, k, v, beta, grad_out))
     outs = [kv, grad_q, grad_k, grad_v, grad_beta] + ([grad_kv] if grad_kv is not None else [])
     with torch.cuda.device(q.device), _Dense([v_old, v_insert], False) as sv, _Dense(outs, True) as d:
         gkv = _ptr(d[5]) if grad_kv is not None else ctypes.c_void_p(None)
-        code = lib().delta_backward_f32(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
-                                        _ptr(sv[0]), _ptr(sv[1]), _ptr(gos), gstr,
-                                        *[_ptr(t) for t in d[:5]], gkv, N, H, L, E, M, flags,
-                                        _stream(q.device))
-    _check(code, "delta_backward_f32")
+        code = fn(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
+                  _ptr(sv[0]), _ptr(sv[1]), _ptr(gos), gstr,
+                  *[_ptr(t) for t in d[:5]], gkv, N, H, L, E, M, flags, _stream(q.device))
+    _check(code, fn.__name__)

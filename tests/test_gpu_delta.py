@@ -141,3 +141,38 @@ def test_full_config2_properties():
     assert rel_err(f["out"][rows].cpu().numpy(), of["out"]) < TOL
     for n in ("grad_Q", "grad_K", "grad_V", "grad_beta"):
         assert rel_err(b[n][rows].cpu().numpy(), ob[n]) < TOL, n
+
+
+# ------------------------------------------------------------------ bf16 I/O, fp32 memory
+
+BF16_TOL = 2e-2   # bf16 inputs, fp32 state: bar stated for this mode
+
+
+@pytest.mark.parametrize("shape,qk", [
+    ((2, 3, 64, 16, 16), "softmax"),
+    ((2, 2, 200, 64, 64), "softmax"),
+    ((1, 2, 1024, 128, 128), "l2"),      # BASELINE config 5's state size and input style, shorter
+    ((1, 2, 40, 24, 24), "l2"),          # no bf16 kernel for D=24: widened on the host side
+])
+def test_bf16_io_matches_oracle_on_rounded_inputs(shape, qk):
+    """Oracle (fp64) on the bf16-rounded inputs vs the bf16-I/O kernel, through the autograd op."""
+    print(f"case bf16 shape={shape}", flush=True)
+    from fast_weight import fast_weight_delta
+    dev = _dev()
+    q, k, v, beta, W0, go = delta_inputs(*shape, seed=11, qk=qk)
+    rb = lambda t: t.to(torch.bfloat16)
+    qb, kb, vb, bb, gob = (rb(t) for t in (q, k, v, beta, go))
+    base = [t.to(torch.float64).numpy() for t in (qb, kb, vb, bb)] + [W0.numpy()]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, gob.to(torch.float64).numpy())
+    leaves = [t.to(dev).requires_grad_(True) for t in (qb, kb, vb, bb)]
+    W = W0.to(dev, torch.float32).contiguous()
+    out = fast_weight_delta(*leaves, W)
+    assert out.dtype == torch.bfloat16
+    assert rel_err(W.cpu().numpy(), of["W"]) < BF16_TOL
+    out.backward(gob.to(dev))
+    assert rel_err(out.detach().float().cpu().numpy(), of["out"]) < BF16_TOL
+    for leaf, n in zip(leaves, ("grad_Q", "grad_K", "grad_V", "grad_beta")):
+        assert leaf.grad.dtype == torch.bfloat16
+        assert rel_err(leaf.grad.float().cpu().numpy(), ob[n]) < BF16_TOL, n
+    assert W.abs().max().item() < 1e-4 * max(1.0, float(np.abs(of["W"]).max()))   # reverted to W_0 = 0
