@@ -212,12 +212,25 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
                     oq[c] = fmaf(w[i][c], qr[i], oq[c]);
                 }
             }
-            kq = group_sum<RG>(kq);
+            {
+                float red[2 * CC + 1];
+#pragma unroll
+                for (int c = 0; c < CC; ++c) {
+                    red[c] = vo[c];
+                    red[CC + c] = oq[c];
+                }
+                red[2 * CC] = kq;
+                group_sum_n<RG, 2 * CC + 1>(red);
+#pragma unroll
+                for (int c = 0; c < CC; ++c) {
+                    vo[c] = red[c];
+                    oq[c] = red[CC + c];
+                }
+                kq = red[2 * CC];
+            }
             float ins[CC], out[CC];
 #pragma unroll
             for (int c = 0; c < CC; ++c) {
-                vo[c] = group_sum<RG>(vo[c]);
-                oq[c] = group_sum<RG>(oq[c]);
                 ins[c] = b * (vc[c] - vo[c]);
                 out[c] = fmaf(kq, ins[c], oq[c]);  // (W + k (x) ins)^T q
             }
@@ -333,10 +346,10 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
                     ak[i] = fmaf(g[i][c], vi[c], ak[i]);    // grad_k, part through the write
                 }
             }
+            group_sum_n<RG, CC>(r);
             float gvo[CC], gv[CC], pb = 0.f;
 #pragma unroll
             for (int c = 0; c < CC; ++c) {
-                r[c] = group_sum<RG>(r[c]);
                 gv[c] = b * r[c];
                 gvo[c] = -gv[c];                            // dL/dv_old
                 pb = fmaf(r[c], dvv[c] - vo[c], pb);

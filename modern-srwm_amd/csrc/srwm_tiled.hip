@@ -133,8 +133,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < NC; ++c) acc[c] = fmaf(w[i][c], xr[i], acc[c]);
-#pragma unroll
-            for (int c = 0; c < NC; ++c) acc[c] = group_sum<RG>(acc[c]);
+            group_sum_n<RG, NC>(acc);
             const float pb = group_sum<E>(wbe * xb);
             if (rg == 0) {
                 store_vec<CB>(p.out + o + c0, &acc[0]);
@@ -148,11 +147,14 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 
             // ---- activations, redundantly in every wave, lane <-> element el
             const float qraw = raw[par][0][el], kraw = raw[par][1][el], braw = rawb[par][lane & 3];
-            const float mq = group_max<E>(qraw), mk = group_max<E>(kraw);
-            const float eq = expf(qraw - mq), ek = expf(kraw - mk);
-            const float sq = group_sum<E>(eq), sk = group_sum<E>(ek);
-            const float qn = eq * fast_rcp(sq), kn = ek * fast_rcp(sk);
-            const float sg = fast_rcp(1.f + expf(-braw));
+            float mx[2] = {qraw, kraw};
+            group_max_n<E, 2>(mx);
+            const float eq = exp_2ulp(qraw - mx[0]), ek = exp_2ulp(kraw - mx[1]);
+            float sm[2] = {eq, ek};
+            group_sum_n<E, 2>(sm);
+            const float qn = eq * fast_rcp(sm[0]), kn = ek * fast_rcp(sm[1]);
+            // sigmoid saturates to 0 / 1 in fp32 well inside +-80; the clamp keeps exp finite
+            const float sg = fast_rcp(1.f + exp_2ulp(-fminf(fmaxf(braw, -80.f), 80.f)));
             const float bt[4] = {quad_broadcast<0>(sg), quad_broadcast<1>(sg), quad_broadcast<2>(sg),
                                  quad_broadcast<3>(sg)};
             const float dv = qn - kn;
@@ -178,8 +180,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < NC; ++c) dif[c] = fmaf(w[i][c], dvr[i], dif[c]);
-#pragma unroll
-            for (int c = 0; c < NC; ++c) dif[c] = group_sum<RG>(dif[c]);
+            group_sum_n<RG, NC>(dif);
             const float pbd = group_sum<E>(wbe * dv);
             if (rg == 0) {
                 store_vec<CB>(p.ydiff + o + c0, &dif[0]);
@@ -350,12 +351,12 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < NC; ++c) gdif[c] = fmaf(g[i][c], kr[i], gdif[c]);
+            group_sum_n<RG, NC>(gdif);
             float pg[3] = {0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                const float gi = group_sum<RG>(gdif[c]);
-                pg[c / CB] = fmaf(gi, dif[c], pg[c / CB]);
-                gdif[c] = bt[c / CB] * gi;
+                pg[c / CB] = fmaf(gdif[c], dif[c], pg[c / CB]);
+                gdif[c] *= bt[c / CB];
             }
             const float ginsb = group_sum<E>(gbe * kb);
             const float gdifb = bt[3] * ginsb;
@@ -395,14 +396,17 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 gq += rowb[1][j][el];
             }
             gk -= gq;
-            const float dq = group_sum<E>(gq * qb), dk = group_sum<E>(gk * kb);
-            const float gpq = qb * (gq - dq), gpk = kb * (gk - dk);
+            float dqk[2] = {gq * qb, gk * kb};
+            group_sum_n<E, 2>(dqk);
+            const float gpq = qb * (gq - dqk[0]), gpk = kb * (gk - dqk[1]);
             float gb[4];
             {
                 float part[4];
                 lds_read_vec<4>(part, &gbp[lane % NCG][0]);
+                float p012[3] = {part[0], part[1], part[2]};
+                group_sum_n<NCG, 3>(p012);
 #pragma unroll
-                for (int j = 0; j < 3; ++j) gb[j] = group_sum<NCG>(part[j]);
+                for (int j = 0; j < 3; ++j) gb[j] = p012[j];
                 float p3[4];
                 lds_read_vec<4>(p3, &gbp3[0]);
                 gb[3] = (p3[0] + p3[1]) + (p3[2] + p3[3]);

@@ -24,37 +24,85 @@ __device__ __forceinline__ float readlane(float v, int lane) {
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
 
+constexpr int kDppBcast15 = 0x142;    // lane 15 of each row -> all lanes of the next row
+constexpr int kDppBcast31 = 0x143;    // lane 31 -> all lanes of rows 2 and 3
+
+// DPP move that only updates the rows selected by ROWMASK; the other rows receive `old`.
+template <int CTRL, int ROWMASK>
+__device__ __forceinline__ float dpp_mov_rows(float old, float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old),
+                                                                 __builtin_bit_cast(int, v), CTRL,
+                                                                 ROWMASK, 0xF, false));
+}
+
 struct OpSum {
     static __device__ __forceinline__ float f(float a, float b) { return a + b; }
+    static __device__ __forceinline__ float neutral(float) { return 0.f; }
 };
 struct OpMax {
     static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); }
+    static __device__ __forceinline__ float neutral(float v) { return v; }
 };
 
-// All-reduce over aligned groups of G consecutive lanes (G = 1, 2, 4, 8, 16, 32 or 64):
-// every lane of a group ends up with the group's result.  The mirror steps are valid
-// because the sub-groups they exchange are already uniform.
+// All-reduce of N independent values over aligned groups of G consecutive lanes (G = 1, 2,
+// 4, 8, 16, 32 or 64): every lane of a group ends up with the group's results.  Written
+// step-major so the N dependency chains interleave.  Inside a 16-lane row the steps are
+// xor-1, xor-2 and two mirror exchanges (valid because the halves they exchange are already
+// uniform); rows are joined with row_bcast:15 / row_bcast:31 and one v_readlane per half.
+template <int G, class Op, int N>
+__device__ __forceinline__ void group_allreduce_n(float (&v)[N]) {
+    static_assert(G == 1 || G == 2 || G == 4 || G == 8 || G == 16 || G == 32 || G == 64, "group size");
+    if constexpr (G >= 2) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) v[n] = Op::f(v[n], dpp_mov<kDppXor1>(v[n]));
+    }
+    if constexpr (G >= 4) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) v[n] = Op::f(v[n], dpp_mov<kDppXor2>(v[n]));
+    }
+    if constexpr (G >= 8) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) v[n] = Op::f(v[n], dpp_mov<kDppHalfMirror>(v[n]));
+    }
+    if constexpr (G >= 16) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) v[n] = Op::f(v[n], dpp_mov<kDppMirror>(v[n]));
+    }
+    if constexpr (G >= 32) {  // rows 1 and 3 += rows 0 and 2
+#pragma unroll
+        for (int n = 0; n < N; ++n)
+            v[n] = Op::f(v[n], dpp_mov_rows<kDppBcast15, 0xA>(Op::neutral(v[n]), v[n]));
+    }
+    if constexpr (G == 64) {  // rows 2 and 3 += row 1; lane 63 then holds the total
+#pragma unroll
+        for (int n = 0; n < N; ++n)
+            v[n] = Op::f(v[n], dpp_mov_rows<kDppBcast31, 0xC>(Op::neutral(v[n]), v[n]));
+#pragma unroll
+        for (int n = 0; n < N; ++n) v[n] = readlane(v[n], 63);
+    } else if constexpr (G == 32) {
+#pragma unroll
+        for (int n = 0; n < N; ++n) {
+            const float lo = readlane(v[n], 31), hi = readlane(v[n], 63);
+            v[n] = (threadIdx.x & 32) ? hi : lo;
+        }
+    }
+}
+
 template <int G, class Op>
 __device__ __forceinline__ float group_allreduce(float v) {
-    static_assert(G == 1 || G == 2 || G == 4 || G == 8 || G == 16 || G == 32 || G == 64, "group size");
-    if constexpr (G >= 2) v = Op::f(v, dpp_mov<kDppXor1>(v));
-    if constexpr (G >= 4) v = Op::f(v, dpp_mov<kDppXor2>(v));
-    if constexpr (G >= 8) v = Op::f(v, dpp_mov<kDppHalfMirror>(v));
-    if constexpr (G >= 16) v = Op::f(v, dpp_mov<kDppMirror>(v));
-    if constexpr (G == 64) {
-        v = Op::f(Op::f(readlane(v, 0), readlane(v, 16)), Op::f(readlane(v, 32), readlane(v, 48)));
-    } else if constexpr (G == 32) {
-        const float lo = Op::f(readlane(v, 0), readlane(v, 16));
-        const float hi = Op::f(readlane(v, 32), readlane(v, 48));
-        v = (threadIdx.x & 32) ? hi : lo;
-    }
-    return v;
+    float a[1] = {v};
+    group_allreduce_n<G, Op, 1>(a);
+    return a[0];
 }
 
 template <int G>
 __device__ __forceinline__ float group_sum(float v) { return group_allreduce<G, OpSum>(v); }
 template <int G>
 __device__ __forceinline__ float group_max(float v) { return group_allreduce<G, OpMax>(v); }
+template <int G, int N>
+__device__ __forceinline__ void group_sum_n(float (&v)[N]) { group_allreduce_n<G, OpSum, N>(v); }
+template <int G, int N>
+__device__ __forceinline__ void group_max_n(float (&v)[N]) { group_allreduce_n<G, OpMax, N>(v); }
 
 // Value of lane (4*(lane/4) + J) for every lane of the quad.
 template <int J>
@@ -70,43 +118,81 @@ __device__ __forceinline__ void wave_lds_fence() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-// Sum over the lane pairs (l, l^32) of x and of y: lanes 0..31 receive x[l] + x[l+32], lanes
-// 32..63 receive y[l-32] + y[l].  With x == y this is an all-reduce over the pair.
-// (Inline assembly because the compiler builtin returns the first result twice; the
-// s_nop pairs cover the VALU-write -> permlane-swap and permlane-swap -> VALU-read wait
-// states that the compiler's hazard recogniser cannot insert inside an asm block.)
-__device__ __forceinline__ float swap_add32(float x, float y) {
-    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
-    return x + y;
+// v_permlane32_swap x, y exchanges the upper 32 lanes of x with the lower 32 lanes of y;
+// v_permlane16_swap x, y exchanges the odd 16-lane rows of x with the even rows of y.  After
+// either one x + y holds, in the lower half / even rows, the pair sums of the old x and, in
+// the upper half / odd rows, the pair sums of the old y: a reduce-scatter step that halves
+// the number of live values.  With x == y it is an all-reduce over the pair.
+// (Inline assembly because the compiler builtin of this toolchain returns the first result
+// twice.  The s_nop pairs cover the VALU-write -> swap and swap -> VALU-read wait states the
+// compiler's hazard recogniser cannot insert inside an asm block; swaps on distinct registers
+// need nothing between them, so they are issued in batches.)
+template <int W>
+__device__ __forceinline__ void swap_pairs(float &x0, float &y0) {
+    if constexpr (W == 32)
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x0), "+v"(y0));
+    else
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x0), "+v"(y0));
+}
+template <int W>
+__device__ __forceinline__ void swap_pairs(float &x0, float &y0, float &x1, float &y1) {
+    if constexpr (W == 32)
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\ts_nop 1"
+                     : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1));
+    else
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\ts_nop 1"
+                     : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1));
+}
+template <int W>
+__device__ __forceinline__ void swap_pairs(float &x0, float &y0, float &x1, float &y1, float &x2,
+                                           float &y2, float &x3, float &y3) {
+    if constexpr (W == 32)
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\t"
+                     "v_permlane32_swap_b32 %4, %5\n\tv_permlane32_swap_b32 %6, %7\n\ts_nop 1"
+                     : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1), "+v"(x2), "+v"(y2), "+v"(x3), "+v"(y3));
+    else
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\t"
+                     "v_permlane16_swap_b32 %4, %5\n\tv_permlane16_swap_b32 %6, %7\n\ts_nop 1"
+                     : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1), "+v"(x2), "+v"(y2), "+v"(x3), "+v"(y3));
 }
 
-// Same for the row pairs (l, l^16): even 16-lane rows receive the pair sum of x, odd rows
-// the pair sum of y.
-__device__ __forceinline__ float swap_add16(float x, float y) {
-    asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x), "+v"(y));
-    return x + y;
+// One reduce-scatter step over lane distance W (32 or 16): out[i] = pair sums of v[i] in the
+// lower half / even rows and of v[i + N/2] in the upper half / odd rows (N >= 2); for N == 1
+// an all-reduce of v[0].
+template <int W, int N>
+__device__ __forceinline__ void swap_halve(const float (&v)[N], float (&out)[(N >= 2 ? N / 2 : 1)]) {
+    constexpr int H = N >= 2 ? N / 2 : 1;
+    float x[H], y[H];
+#pragma unroll
+    for (int i = 0; i < H; ++i) {
+        x[i] = v[i];
+        y[i] = N >= 2 ? v[i + H] : v[i];
+    }
+    if constexpr (H == 1) {
+        swap_pairs<W>(x[0], y[0]);
+    } else if constexpr (H == 2) {
+        swap_pairs<W>(x[0], y[0], x[1], y[1]);
+    } else if constexpr (H == 4) {
+        swap_pairs<W>(x[0], y[0], x[1], y[1], x[2], y[2], x[3], y[3]);
+    } else {
+        static_assert(H == 8, "swap_halve: unsupported width");
+        swap_pairs<W>(x[0], y[0], x[1], y[1], x[2], y[2], x[3], y[3]);
+        swap_pairs<W>(x[4], y[4], x[5], y[5], x[6], y[6], x[7], y[7]);
+    }
+#pragma unroll
+    for (int i = 0; i < H; ++i) out[i] = x[i] + y[i];
 }
 
 // Sums R per-lane values over the 8 lanes {l, l^8, l^16, l^32, ...} (same l % 8) and stores
 // the R results once: dst[i] = sum of v[i].  The 32- and 16-lane steps halve the number of
-// live values (reduce-scatter), so the whole reduction costs about R + R/2 + R/4 adds.
+// live values, so the whole reduction costs about R/2 + R/4 swaps and R adds.
 template <int R>
 __device__ __forceinline__ void stride8_reduce_store(const float (&v)[R], float *dst, int lane) {
     constexpr int NA = R >= 2 ? R / 2 : 1;
     constexpr int NB = NA >= 2 ? NA / 2 : 1;
     float a[NA], b[NB];
-    if constexpr (R >= 2) {
-#pragma unroll
-        for (int i = 0; i < NA; ++i) a[i] = swap_add32(v[i], v[i + NA]);
-    } else {
-        a[0] = swap_add32(v[0], v[0]);
-    }
-    if constexpr (NA >= 2) {
-#pragma unroll
-        for (int i = 0; i < NB; ++i) b[i] = swap_add16(a[i], a[i + NB]);
-    } else {
-        b[0] = swap_add16(a[0], a[0]);
-    }
+    swap_halve<32, R>(v, a);
+    swap_halve<16, NA>(a, b);
 #pragma unroll
     for (int i = 0; i < NB; ++i) b[i] += dpp_mov<kDppRor8>(b[i]);
     const int b5 = (lane >> 5) & 1, b4 = (lane >> 4) & 1, b3 = (lane >> 3) & 1;
@@ -115,11 +201,35 @@ __device__ __forceinline__ void stride8_reduce_store(const float (&v)[R], float 
     if (writer) {
         if constexpr (NB == 2) {
             *reinterpret_cast<float2 *>(dst + idx) = make_float2(b[0], b[1]);
+        } else if constexpr (NB == 4) {
+            *reinterpret_cast<float4 *>(dst + idx) = make_float4(b[0], b[1], b[2], b[3]);
         } else {
 #pragma unroll
             for (int i = 0; i < NB; ++i) dst[idx + i] = b[i];
         }
     }
+}
+
+// Sum over the lane pair (l, l^32) / (l, l^16), result in both lanes.
+__device__ __forceinline__ float swap_add32(float x, float y) {
+    swap_pairs<32>(x, y);
+    return x + y;
+}
+__device__ __forceinline__ float swap_add16(float x, float y) {
+    swap_pairs<16>(x, y);
+    return x + y;
+}
+
+// exp(x) to about 2 ulp with one v_exp_f32: x*log2(e) is formed in two pieces (product
+// rounding error via fma, low bits of log2(e)) and the small remainder r is applied as
+// 2^r ~ 1 + r ln 2.  Meant for softmax arguments (x <= 0) and clamped sigmoid arguments.
+__device__ __forceinline__ float exp_2ulp(float x) {
+    const float kL2eHi = 1.44269502162933349609375f, kL2eLo = 1.925963033500011e-8f;
+    const float t = x * kL2eHi;
+    float r = fmaf(x, kL2eHi, -t);
+    r = fmaf(x, kL2eLo, r);
+    const float e = __builtin_amdgcn_exp2f(t);
+    return fmaf(e, r * 0.693147180559945309f, e);
 }
 
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
