@@ -119,6 +119,17 @@ struct TileVec {
     }
 };
 
+// Stores one staged tile vector (rows x D floats in LDS) to global memory, 4 elements per
+// thread and store: full rows, consecutive lanes -> consecutive addresses.
+template <class T, int D, class TO>
+__device__ __forceinline__ void flush_rows(const float *lds, TO *gbase, int rows, int tid) {
+    for (int f = tid; f < rows * (D / 4); f += T::NT) {
+        const float4 v = reinterpret_cast<const float4 *>(lds)[f];
+        const float a[4] = {v.x, v.y, v.z, v.w};
+        wr<4>(gbase + (int64_t)f * 4, a);
+    }
+}
+
 // Parameter blocks with the I/O element type TI (float or bf16_t) made explicit.  The memory
 // W, its gradient and the saved v_old / v_insert are always fp32.
 template <class TI>
@@ -148,8 +159,13 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
     using T = DTiling<D, NW, R, TT>;
     constexpr int RG = T::RG, CGW = T::CGW, CC = T::CC;
     enum { VQ, VK, VV, NVEC };
+    enum { OVO, OVI, OOUT, NOUT };
     __shared__ __attribute__((aligned(16))) float tl[2][NVEC][TT][D];
     __shared__ float tbeta[2][TT];
+    // Outputs of a tile are parked here and written out after the step loop: the loop then
+    // contains no global memory instruction, so the prefetch of the next tile stays in
+    // flight across it, and the stores are full coalesced rows.
+    __shared__ __attribute__((aligned(16))) float ot[2][NOUT][TT][D];
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int rg = lane % RG, cg = wave * CGW + lane / RG;
@@ -192,60 +208,73 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
         const int tlen = min(TT, p.L - tile * TT);
         if (tile + 1 < ntiles) load_tile(tile + 1);
 
-        for (int tt = 0; tt < tlen; ++tt) {
-            const int64_t om = (seq * p.L + tile * TT + tt) * D + c0;
-            float kr[R], qr[R], vc[CC];
-            rd<R>(kr, &tl[buf][VK][tt][r0]);
-            rd<R>(qr, &tl[buf][VQ][tt][r0]);
-            rd<CC>(vc, &tl[buf][VV][tt][c0]);
-            const float b = tbeta[buf][tt];
-            // v_old = W^T k and W^T q in one pass over the tile, plus k.q
+        // Operands of a step are read from LDS one step ahead (software pipelining), and the
+        // step body is branch-free so that the compiler can interleave neighbouring steps.
+        struct Ops {
+            float kr[R], qr[R], vc[CC], b;
+        };
+        auto fetch = [&](Ops &o, int tt) __attribute__((always_inline)) {
+            rd<R>(o.kr, &tl[buf][VK][tt][r0]);
+            rd<R>(o.qr, &tl[buf][VQ][tt][r0]);
+            rd<CC>(o.vc, &tl[buf][VV][tt][c0]);
+            o.b = tbeta[buf][tt];
+        };
+        auto step = [&](const Ops &o, int tt) __attribute__((always_inline)) {
+            // v_old = W^T k and W^T q in one pass over the tile, plus this lane's part of k.q
             float vo[CC], oq[CC], kq = 0.f;
 #pragma unroll
             for (int c = 0; c < CC; ++c) vo[c] = oq[c] = 0.f;
 #pragma unroll
             for (int i = 0; i < R; ++i) {
-                kq = fmaf(kr[i], qr[i], kq);
+                kq = fmaf(o.kr[i], o.qr[i], kq);
 #pragma unroll
                 for (int c = 0; c < CC; ++c) {
-                    vo[c] = fmaf(w[i][c], kr[i], vo[c]);
-                    oq[c] = fmaf(w[i][c], qr[i], oq[c]);
+                    vo[c] = fmaf(w[i][c], o.kr[i], vo[c]);
+                    oq[c] = fmaf(w[i][c], o.qr[i], oq[c]);
                 }
             }
-            {
-                float red[2 * CC + 1];
-#pragma unroll
-                for (int c = 0; c < CC; ++c) {
-                    red[c] = vo[c];
-                    red[CC + c] = oq[c];
-                }
-                red[2 * CC] = kq;
-                group_sum_n<RG, 2 * CC + 1>(red);
-#pragma unroll
-                for (int c = 0; c < CC; ++c) {
-                    vo[c] = red[c];
-                    oq[c] = red[CC + c];
-                }
-                kq = red[2 * CC];
-            }
+            group_sum_n<RG, CC>(vo);
             float ins[CC], out[CC];
 #pragma unroll
             for (int c = 0; c < CC; ++c) {
-                ins[c] = b * (vc[c] - vo[c]);
-                out[c] = fmaf(kq, ins[c], oq[c]);  // (W + k (x) ins)^T q
+                ins[c] = o.b * (o.vc[c] - vo[c]);
+                // (W + k (x) ins)^T q = W^T q + (k.q) ins, summed over the lanes of the column group
+                out[c] = fmaf(kq, ins[c], oq[c]);
             }
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
-                for (int c = 0; c < CC; ++c) w[i][c] = fmaf(kr[i], ins[c], w[i][c]);
-            if (rg == 0) {
-                wr<CC>(p.vold + om, vo);
-                wr<CC>(p.vins + om, ins);
-                wr<CC>(p.out + om, out);
+                for (int c = 0; c < CC; ++c) w[i][c] = fmaf(o.kr[i], ins[c], w[i][c]);
+            group_sum_n<RG, CC>(out);   // off the recurrence's critical path
+            // all 8 lanes of the column group hold the same values and write them to the same
+            // words: no branch, no divergence
+            wr<CC>(&ot[buf][OVO][tt][c0], vo);
+            wr<CC>(&ot[buf][OVI][tt][c0], ins);
+            wr<CC>(&ot[buf][OOUT][tt][c0], out);
+        };
+        if (tlen == TT) {
+            Ops a, b;
+            fetch(a, 0);
+#pragma unroll
+            for (int tt = 0; tt < TT; tt += 2) {
+                fetch(b, tt + 1);
+                step(a, tt);
+                fetch(a, tt + 2 < TT ? tt + 2 : TT - 1);
+                step(b, tt + 1);
+            }
+        } else {
+            Ops a;
+            for (int tt = 0; tt < tlen; ++tt) {
+                fetch(a, tt);
+                step(a, tt);
             }
         }
         if (tile + 1 < ntiles) store_tile(buf ^ 1);
         __syncthreads();
+        const int64_t om = (seq * p.L + tile * TT) * D;
+        flush_rows<T, D>(&ot[buf][OVO][0][0], p.vold + om, tlen, tid);
+        flush_rows<T, D>(&ot[buf][OVI][0][0], p.vins + om, tlen, tid);
+        flush_rows<T, D>(&ot[buf][OOUT][0][0], p.out + om, tlen, tid);
     }
 
 #pragma unroll
@@ -262,6 +291,7 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
     __shared__ __attribute__((aligned(16))) float rowq[TT][NW][D];  // per-wave parts of grad_q
     __shared__ __attribute__((aligned(16))) float rowk[TT][NW][D];  // per-wave parts of grad_k
     __shared__ float gbp[TT][NCG];                                  // per column group parts of grad_beta
+    __shared__ __attribute__((aligned(16))) float gvt[TT][D];       // grad_v of the tile
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int rg = lane % RG, cg = wave * CGW + lane / RG;
@@ -319,17 +349,19 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
         const int tlen = min(TT, p.L - tile * TT);
         if (tile > 0) load_tile(tile - 1);
 
-        for (int tt = tlen - 1; tt >= 0; --tt) {
-            const int64_t om = (seq * p.L + tile * TT + tt) * D + c0;
-            float kr[R], qr[R], go[CC], vi[CC], dvv[CC], vo[CC];
-            rd<R>(kr, &tl[buf][VK][tt][r0]);
-            rd<R>(qr, &tl[buf][VQ][tt][r0]);
-            rd<CC>(go, &tl[buf][VGO][tt][c0]);
-            rd<CC>(vi, &tl[buf][VVI][tt][c0]);
-            rd<CC>(dvv, &tl[buf][VV][tt][c0]);
-            rd<CC>(vo, &tl[buf][VVO][tt][c0]);
-            const float b = tbeta[buf][tt];
-
+        struct Ops {
+            float kr[R], qr[R], go[CC], vi[CC], vv[CC], vo[CC], b;
+        };
+        auto fetch = [&](Ops &o, int tt) __attribute__((always_inline)) {
+            rd<R>(o.kr, &tl[buf][VK][tt][r0]);
+            rd<R>(o.qr, &tl[buf][VQ][tt][r0]);
+            rd<CC>(o.go, &tl[buf][VGO][tt][c0]);
+            rd<CC>(o.vi, &tl[buf][VVI][tt][c0]);
+            rd<CC>(o.vv, &tl[buf][VV][tt][c0]);
+            rd<CC>(o.vo, &tl[buf][VVO][tt][c0]);
+            o.b = tbeta[buf][tt];
+        };
+        auto step = [&](const Ops &o, int tt) __attribute__((always_inline)) {
             // out_t = W_t^T q_t :  G += q (x) go ;  grad_q = W_t go
             float aq[R], ak[R], r[CC];
 #pragma unroll
@@ -340,34 +372,61 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
                 ak[i] = 0.f;
 #pragma unroll
                 for (int c = 0; c < CC; ++c) {
-                    g[i][c] = fmaf(qr[i], go[c], g[i][c]);
-                    aq[i] = fmaf(w[i][c], go[c], aq[i]);
-                    r[c] = fmaf(g[i][c], kr[i], r[c]);      // dL/d ins = G^T k
-                    ak[i] = fmaf(g[i][c], vi[c], ak[i]);    // grad_k, part through the write
+                    g[i][c] = fmaf(o.qr[i], o.go[c], g[i][c]);
+                    aq[i] = fmaf(w[i][c], o.go[c], aq[i]);
+                    r[c] = fmaf(g[i][c], o.kr[i], r[c]);      // dL/d ins = G^T k
+                    ak[i] = fmaf(g[i][c], o.vi[c], ak[i]);    // grad_k, part through the write
                 }
             }
             group_sum_n<RG, CC>(r);
             float gvo[CC], gv[CC], pb = 0.f;
 #pragma unroll
             for (int c = 0; c < CC; ++c) {
-                gv[c] = b * r[c];
-                gvo[c] = -gv[c];                            // dL/dv_old
-                pb = fmaf(r[c], dvv[c] - vo[c], pb);
+                gv[c] = o.b * r[c];
+                gvo[c] = -gv[c];                              // dL/dv_old
+                pb = fmaf(r[c], o.vv[c] - o.vo[c], pb);
             }
             // revert the write, then the part of grad_k through v_old = W_{t-1}^T k
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < CC; ++c) {
-                    w[i][c] = fmaf(-kr[i], vi[c], w[i][c]);
+                    w[i][c] = fmaf(-o.kr[i], o.vi[c], w[i][c]);
                     ak[i] = fmaf(w[i][c], gvo[c], ak[i]);
-                    g[i][c] = fmaf(kr[i], gvo[c], g[i][c]);
+                    g[i][c] = fmaf(o.kr[i], gvo[c], g[i][c]);
                 }
-            stride8_reduce_store<R>(aq, &rowq[tt][wave][r0], lane);
-            stride8_reduce_store<R>(ak, &rowk[tt][wave][r0], lane);
-            if (rg == 0) {
-                wr<CC>(p.gV + om, gv);
-                gbp[tt][cg] = pb;
+            if constexpr (R >= 2) {
+                stride8_reduce_store2<R>(aq, ak, &rowq[tt][wave][r0], &rowk[tt][wave][r0], lane);
+            } else {
+                stride8_reduce_store<R>(aq, &rowq[tt][wave][r0], lane);
+                stride8_reduce_store<R>(ak, &rowk[tt][wave][r0], lane);
+            }
+            // the 8 lanes of a column group hold identical values: all write, no branch
+            wr<CC>(&gvt[tt][c0], gv);
+            gbp[tt][cg] = pb;
+        };
+        if constexpr (D >= 128) {   // no registers to spare: keep the steps rolled
+            Ops a;
+#pragma unroll 1
+            for (int tt = tlen - 1; tt >= 0; --tt) {
+                fetch(a, tt);
+                step(a, tt);
+            }
+        } else if (tlen == TT) {
+            Ops a, b;
+            fetch(a, TT - 1);
+#pragma unroll 1
+            for (int tt = TT - 1; tt >= 0; tt -= 2) {
+                fetch(b, tt - 1);
+                step(a, tt);
+                fetch(a, tt >= 2 ? tt - 2 : 0);
+                step(b, tt - 1);
+            }
+        } else {
+            Ops a;
+            for (int tt = tlen - 1; tt >= 0; --tt) {
+                fetch(a, tt);
+                step(a, tt);
             }
         }
         __syncthreads();
@@ -390,6 +449,7 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
             for (int c = 0; c < NCG; ++c) s += gbp[tid][c];
             st1(p.gbeta + seq * p.L + tile * TT + tid, s);
         }
+        flush_rows<T, D>(&gvt[0][0], p.gV + (seq * p.L + tile * TT) * D, tlen, tid);
         if (tile > 0) store_tile(buf ^ 1);
         __syncthreads();
     }

@@ -172,12 +172,11 @@ __device__ __forceinline__ void swap_halve(const float (&v)[N], float (&out)[(N 
         swap_pairs<W>(x[0], y[0]);
     } else if constexpr (H == 2) {
         swap_pairs<W>(x[0], y[0], x[1], y[1]);
-    } else if constexpr (H == 4) {
-        swap_pairs<W>(x[0], y[0], x[1], y[1], x[2], y[2], x[3], y[3]);
     } else {
-        static_assert(H == 8, "swap_halve: unsupported width");
-        swap_pairs<W>(x[0], y[0], x[1], y[1], x[2], y[2], x[3], y[3]);
-        swap_pairs<W>(x[4], y[4], x[5], y[5], x[6], y[6], x[7], y[7]);
+        static_assert(H % 4 == 0, "swap_halve: unsupported width");
+#pragma unroll
+        for (int i = 0; i < H; i += 4)
+            swap_pairs<W>(x[i], y[i], x[i + 1], y[i + 1], x[i + 2], y[i + 2], x[i + 3], y[i + 3]);
     }
 #pragma unroll
     for (int i = 0; i < H; ++i) out[i] = x[i] + y[i];
@@ -206,6 +205,39 @@ __device__ __forceinline__ void stride8_reduce_store(const float (&v)[R], float 
         } else {
 #pragma unroll
             for (int i = 0; i < NB; ++i) dst[idx + i] = b[i];
+        }
+    }
+}
+
+// Two such reductions at once (R >= 2): the 2R values travel through the swap steps together,
+// lanes 0..31 end up with results of `a` (stored to dst_a), lanes 32..63 with results of `b`.
+template <int R>
+__device__ __forceinline__ void stride8_reduce_store2(const float (&a)[R], const float (&b)[R],
+                                                      float *dst_a, float *dst_b, int lane) {
+    static_assert(R >= 2, "use stride8_reduce_store for single values");
+    constexpr int NB = R / 2;
+    float v[2 * R], h[R], q[NB];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        v[i] = a[i];
+        v[R + i] = b[i];
+    }
+    swap_halve<32, 2 * R>(v, h);   // lower half: a[i] pair sums, upper half: b[i]
+    swap_halve<16, R>(h, q);       // even rows: first NB of them, odd rows: last NB
+#pragma unroll
+    for (int i = 0; i < NB; ++i) q[i] += dpp_mov<kDppRor8>(q[i]);
+    const int b5 = (lane >> 5) & 1, b4 = (lane >> 4) & 1, b3 = (lane >> 3) & 1;
+    float *dst = (b5 ? dst_b : dst_a) + NB * b4;
+    if (b3 == 0) {
+        if constexpr (NB == 2) {
+            *reinterpret_cast<float2 *>(dst) = make_float2(q[0], q[1]);
+        } else if constexpr (NB % 4 == 0) {
+#pragma unroll
+            for (int i = 0; i < NB / 4; ++i)
+                reinterpret_cast<float4 *>(dst)[i] = make_float4(q[4 * i], q[4 * i + 1], q[4 * i + 2], q[4 * i + 3]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < NB; ++i) dst[i] = q[i];
         }
     }
 }
