@@ -1,0 +1,184 @@
+"""Layer modules over the HIP-backed operators, mirroring the callers of the reference:
+
+    SRWMlayer, FastFFlayer            supervised_learning/layer.py:112-210, :49-108
+    SRlayer, NoCarryOverSRlayer       reinforcement_learning/torchbeast/layer.py:340-421, :425-488
+    CarryFastFFlayer                  reinforcement_learning/torchbeast/layer.py:128-189 (the RL tree
+                                      calls it FastFFlayer too; it threads the memory as state)
+
+Same constructor arguments, parameter names and shapes (so state_dicts of the reference load
+unchanged: W_y, W_q, W_k: (1, H, d, d); w_b: (1, H, d, 4); slow_net / out_linear / layer_norm),
+same input/output conventions: activations are (len, batch, num_head * dim_head).  The carried
+SRWM state is the SHIFT from the slow weights, exactly as the reference keeps it.
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from fast_weight import fast_weight_delta
+from self_ref_v0 import self_ref_v0, stateful_self_ref_v0
+
+
+def elu_p1(x):
+    return F.elu(x, 1., False) + 1.
+
+
+def sum_norm(x):
+    return x / x.sum(-1, keepdim=True)
+
+
+def elu_p1_sum_norm_eps(x):
+    y = F.elu(x, 1., False) + 1.
+    return y / (y.sum(-1, keepdim=True) + 1e-5)
+
+
+def _heads_out(out, bsz, slen, width):
+    """(B, H, len, d) -> (len, B, H*d)"""
+    return out.transpose(1, 2).reshape(bsz, slen, width).transpose(0, 1)
+
+
+class _SRBase(nn.Module):
+    """Slow weights of a self-referential layer and the plumbing shared by its variants."""
+
+    def __init__(self, num_head, dim_head, in_dim, dropout, beta_mean):
+        super().__init__()
+        self.num_head = num_head
+        self.dim_head = dim_head
+        self.in_dim = in_dim
+        self.W_y = nn.Parameter(torch.empty(1, num_head, dim_head, dim_head))
+        self.W_q = nn.Parameter(torch.empty(1, num_head, dim_head, dim_head))
+        self.W_k = nn.Parameter(torch.empty(1, num_head, dim_head, dim_head))
+        self.w_b = nn.Parameter(torch.empty(1, num_head, dim_head, 4))
+        self.layer_norm = nn.LayerNorm(in_dim)
+        self.out_linear = nn.Linear(num_head * dim_head, in_dim, bias=False)
+        self.drop = nn.Dropout(dropout)
+        std = 1.0 / math.sqrt(dim_head)
+        for w in (self.W_y, self.W_q, self.W_k):
+            nn.init.normal_(w, mean=0., std=std)
+        nn.init.normal_(self.w_b, mean=beta_mean, std=std)
+
+    def _slow(self):
+        return (self.W_y, self.W_q, self.W_k, self.w_b)
+
+    def _split(self, h, softmax):
+        slen, bsz, _ = h.size()
+        x = h.reshape(slen, bsz, self.num_head, self.dim_head)
+        if softmax:
+            x = F.softmax(x, dim=-1)
+        return x.permute(1, 2, 0, 3), slen, bsz          # (B, H, len, d) view, no copy
+
+    def _fast(self, bsz, shift=None):
+        """Per-batch copies of the weights (the operator overwrites them with the final state)."""
+        if shift is None:
+            return [w.repeat(bsz, 1, 1, 1) for w in self._slow()]
+        return [s + w.repeat(bsz, 1, 1, 1) for s, w in zip(shift, self._slow())]
+
+    def _project(self, out, bsz, slen):
+        out = _heads_out(out, bsz, slen, self.num_head * self.dim_head)
+        return self.drop(self.out_linear(out))
+
+
+class SRWMlayer(_SRBase):
+    """Few-shot (supervised) SRWM layer."""
+
+    def __init__(self, num_head, dim_head, in_dim, dropout, use_ln=True, use_input_softmax=False,
+                 beta_init=-1.0, stateful=False):
+        super().__init__(num_head, dim_head, in_dim, dropout, beta_init)
+        self.use_ln = use_ln
+        self.use_input_softmax = use_input_softmax
+        self.stateful = stateful
+        self.sr_layer = stateful_self_ref_v0 if stateful else self_ref_v0
+        if not use_ln:
+            del self.layer_norm
+
+    def forward(self, h, state=None, get_state=False):
+        x, slen, bsz = self._split(h, self.use_input_softmax)
+        fast = self._fast(bsz, state)
+        if self.stateful:
+            out, *fast = self.sr_layer(x, *fast)
+        else:
+            out = self.sr_layer(x, *fast)
+        out = self._project(out, bsz, slen)
+        out = (self.layer_norm(h) if self.use_ln else h) + out
+        if get_state:
+            shift = tuple(f - w.repeat(bsz, 1, 1, 1) for f, w in zip(fast, self._slow()))
+            return out, shift
+        return out
+
+
+class SRlayer(_SRBase):
+    """RL SRWM layer: soft-maxed input, weights carried over segments as a detached shift."""
+
+    def __init__(self, num_head, dim_head, in_dim, dropout):
+        super().__init__(num_head, dim_head, in_dim, dropout, 0.)
+        self.fw_layer = self_ref_v0
+
+    def forward(self, h, state=None):
+        assert state is not None
+        x, slen, bsz = self._split(h, True)
+        fast = self._fast(bsz, state)
+        out = self.fw_layer(x, *fast)
+        out = h + self._project(out, bsz, slen)
+        new_state = tuple((f.detach() - w.repeat(bsz, 1, 1, 1)).detach()
+                          for f, w in zip(fast, self._slow()))
+        return out, new_state
+
+
+class NoCarryOverSRlayer(_SRBase):
+    """RL SRWM layer that restarts from the slow weights at every call."""
+
+    def __init__(self, num_head, dim_head, in_dim, dropout):
+        super().__init__(num_head, dim_head, in_dim, dropout, 0.)
+        self.fw_layer = self_ref_v0
+
+    def forward(self, h, state=None):
+        x, slen, bsz = self._split(h, True)
+        out = self.fw_layer(x, *self._fast(bsz))
+        return h + self._project(out, bsz, slen), state
+
+
+class _DeltaBase(nn.Module):
+    def __init__(self, num_head, dim_head, in_dim, dropout):
+        super().__init__()
+        self.num_head = num_head
+        self.dim_head = dim_head
+        self.in_dim = in_dim
+        self.fw_layer = fast_weight_delta
+        self.slow_net = nn.Linear(in_dim, num_head * (3 * dim_head + 1), bias=False)
+        self.layer_norm = nn.LayerNorm(in_dim)
+        self.out_linear = nn.Linear(num_head * dim_head, in_dim, bias=False)
+        self.drop = nn.Dropout(dropout)
+
+    def _qkvb(self, x, normalise):
+        slen, bsz, _ = x.size()
+        qkvb = self.slow_net(self.layer_norm(x)).view(slen, bsz, self.num_head, 3 * self.dim_head + 1)
+        q, k, v, beta = torch.split(qkvb, (self.dim_head,) * 3 + (1,), -1)
+        beta = torch.sigmoid(beta)
+        q, k, v, beta = (t.permute(1, 2, 0, 3) for t in (q, k, v, beta))
+        return normalise(q), normalise(k), v, beta, slen, bsz
+
+    def _finish(self, x, out, bsz, slen):
+        out = _heads_out(out, bsz, slen, self.num_head * self.dim_head)
+        return x + self.drop(self.out_linear(out))
+
+
+class FastFFlayer(_DeltaBase):
+    """Supervised delta-rule layer: the memory starts from zero at every call."""
+
+    def forward(self, x):
+        q, k, v, beta, slen, bsz = self._qkvb(x, lambda t: sum_norm(elu_p1(t)))
+        fast_weights = torch.zeros(bsz, self.num_head, self.dim_head, self.dim_head, device=k.device)
+        out = self.fw_layer(q, k, v, beta, fast_weights)
+        return self._finish(x, out, bsz, slen)
+
+
+class CarryFastFFlayer(_DeltaBase):
+    """RL delta-rule layer: the memory is passed in and the updated one returned."""
+
+    def forward(self, x, state=None):
+        assert state is not None
+        q, k, v, beta, slen, bsz = self._qkvb(x, elu_p1_sum_norm_eps)
+        fast_weights = state
+        out = self.fw_layer(q, k, v, beta, fast_weights)
+        return self._finish(x, out, bsz, slen), fast_weights.clone()

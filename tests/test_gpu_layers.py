@@ -1,0 +1,160 @@
+"""Layer modules (modern-srwm_amd/layer.py) on the GPU against an fp64 CPU statement built from
+the per-timestep torch recurrences: outputs, carried state and parameter gradients."""
+import copy
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import rel_err
+from oracle.recurrence import delta_recurrence, srwm_recurrence
+
+pytestmark = pytest.mark.gpu
+TOL = 5e-5   # fp32 LayerNorm / Linear around the 1e-5 operator
+
+
+def _dev():
+    return torch.device("cuda:0")
+
+
+def _ref_sr(layer, h, softmax, shift=None, use_ln_residual=None):
+    """fp64 CPU statement of an SRWM layer's forward; returns (out, final fast weights)."""
+    slen, bsz, _ = h.shape
+    H, d = layer.num_head, layer.dim_head
+    x = h.reshape(slen, bsz, H, d)
+    if softmax:
+        x = F.softmax(x, dim=-1)
+    x = x.permute(1, 2, 0, 3)
+    slow = [layer.W_y, layer.W_q, layer.W_k, layer.w_b]
+    fast = [w.repeat(bsz, 1, 1, 1) for w in slow]
+    if shift is not None:
+        fast = [s + f for s, f in zip(shift, fast)]
+    out, final = srwm_recurrence(x, *fast)
+    out = out.transpose(1, 2).reshape(bsz, slen, H * d).transpose(0, 1)
+    out = layer.out_linear(out)
+    res = layer.layer_norm(h) if use_ln_residual else h
+    return res + out, final
+
+
+def _pair(layer):
+    gpu = layer.to(_dev())
+    cpu = copy.deepcopy(layer).double().cpu()
+    return gpu, cpu
+
+
+def test_srwm_layer_supervised():
+    print("case SRWMlayer", flush=True)
+    from layer import SRWMlayer
+    torch.manual_seed(0)
+    L, B, H, d = 12, 3, 4, 16
+    gpu, cpu = _pair(SRWMlayer(H, d, H * d, 0.0, use_ln=True, use_input_softmax=True, beta_init=-1.0))
+    h = torch.randn(L, B, H * d, dtype=torch.float64)
+    go = torch.randn(L, B, H * d, dtype=torch.float64)
+    hg = h.to(_dev(), torch.float32).requires_grad_(True)
+    out, shift = gpu(hg, get_state=True)
+    (out * go.to(_dev(), torch.float32)).sum().backward()
+    hc = h.clone().requires_grad_(True)
+    ref, final = _ref_sr(cpu, hc, True, use_ln_residual=True)
+    (ref * go).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), ref.detach().numpy()) < TOL
+    assert rel_err(hg.grad.cpu().numpy(), hc.grad.numpy()) < TOL
+    for n in ("W_y", "W_q", "W_k", "w_b"):
+        assert rel_err(getattr(gpu, n).grad.cpu().numpy(), getattr(cpu, n).grad.numpy()) < TOL, n
+    assert rel_err(gpu.out_linear.weight.grad.cpu().numpy(), cpu.out_linear.weight.grad.numpy()) < TOL
+    # the shift is a small difference of O(1) fp32 numbers: compare it on the scale of the state
+    for s, f, w in zip(shift, final, (cpu.W_y, cpu.W_q, cpu.W_k, cpu.w_b)):
+        err = (s.detach().cpu().double() - (f - w).detach()).abs().max().item()
+        assert err < 1e-5 * f.abs().max().item()
+
+
+def test_srwm_layer_stateful_with_loss_on_state():
+    print("case SRWMlayer stateful", flush=True)
+    from layer import SRWMlayer
+    torch.manual_seed(1)
+    L, B, H, d = 7, 2, 2, 8
+    gpu, cpu = _pair(SRWMlayer(H, d, H * d, 0.0, use_ln=False, stateful=True, beta_init=0.0))
+    h = torch.randn(L, B, H * d, dtype=torch.float64)
+    hg = h.to(_dev(), torch.float32)
+    out1, st = gpu(hg, get_state=True)
+    out2, st2 = gpu(hg, state=st, get_state=True)      # second segment starts from the carried shift
+    loss = out2.sum() + sum((s * s).sum() for s in st2)
+    loss.backward()
+    r1, f1 = _ref_sr(cpu, h, False, use_ln_residual=False)
+    slow = (cpu.W_y, cpu.W_q, cpu.W_k, cpu.w_b)
+    sh1 = [f - w for f, w in zip(f1, slow)]
+    r2, f2 = _ref_sr(cpu, h, False, shift=sh1, use_ln_residual=False)
+    sh2 = [f - w for f, w in zip(f2, slow)]
+    (r2.sum() + sum((s * s).sum() for s in sh2)).backward()
+    assert rel_err(out2.detach().cpu().numpy(), r2.detach().numpy()) < TOL
+    for n in ("W_y", "W_q", "W_k", "w_b"):
+        assert rel_err(getattr(gpu, n).grad.cpu().numpy(), getattr(cpu, n).grad.numpy()) < 2e-4, n
+
+
+def test_rl_sr_layers_carry_and_restart():
+    print("case SRlayer / NoCarryOverSRlayer", flush=True)
+    from layer import NoCarryOverSRlayer, SRlayer
+    torch.manual_seed(2)
+    B, H, d = 4, 8, 16
+    gpu, cpu = _pair(SRlayer(H, d, H * d, 0.0))
+    state = tuple(torch.zeros(B, H, d, w, device=_dev()) for w in (d, d, d, 4))
+    ref_shift = None
+    for step in range(3):                                # one env step per call, as the actors do
+        h = torch.randn(1, B, H * d, dtype=torch.float64)
+        out, state = gpu(h.to(_dev(), torch.float32), state)
+        ref, final = _ref_sr(cpu, h, True, shift=ref_shift, use_ln_residual=False)
+        ref_shift = [(f - w).detach() for f, w in zip(final, (cpu.W_y, cpu.W_q, cpu.W_k, cpu.w_b))]
+        assert rel_err(out.detach().cpu().numpy(), ref.detach().numpy()) < TOL, step
+        assert all(not s.requires_grad for s in state)
+    for s, r, w in zip(state, ref_shift, (cpu.W_y, cpu.W_q, cpu.W_k, cpu.w_b)):
+        assert (s.cpu().double() - r).abs().max().item() < 1e-5 * max(1.0, w.abs().max().item())
+    gpu2, cpu2 = _pair(NoCarryOverSRlayer(H, d, H * d, 0.0))
+    h = torch.randn(5, B, H * d, dtype=torch.float64)
+    out, st = gpu2(h.to(_dev(), torch.float32), None)
+    ref, _ = _ref_sr(cpu2, h, True, use_ln_residual=False)
+    assert st is None and rel_err(out.detach().cpu().numpy(), ref.detach().numpy()) < TOL
+
+
+def test_delta_layers():
+    print("case FastFFlayer / CarryFastFFlayer", flush=True)
+    from layer import CarryFastFFlayer, FastFFlayer, elu_p1, elu_p1_sum_norm_eps, sum_norm
+    torch.manual_seed(3)
+    L, B, H, d = 9, 3, 4, 16
+
+    def ref_forward(cpu, x, normalise, W0):
+        qkvb = cpu.slow_net(cpu.layer_norm(x)).view(L, B, H, 3 * d + 1)
+        q, k, v, beta = torch.split(qkvb, (d,) * 3 + (1,), -1)
+        beta = torch.sigmoid(beta)
+        q, k, v, beta = (t.permute(1, 2, 0, 3) for t in (q, k, v, beta))
+        out, WL = delta_recurrence(normalise(q), normalise(k), v, beta, W0)
+        out = out.transpose(1, 2).reshape(B, L, H * d).transpose(0, 1)
+        return x + cpu.out_linear(out), WL
+
+    gpu, cpu = _pair(FastFFlayer(H, d, H * d, 0.0))
+    x = torch.randn(L, B, H * d, dtype=torch.float64)
+    go = torch.randn(L, B, H * d, dtype=torch.float64)
+    xg = x.to(_dev(), torch.float32).requires_grad_(True)
+    out = gpu(xg)
+    (out * go.to(_dev(), torch.float32)).sum().backward()
+    xc = x.clone().requires_grad_(True)
+    ref, _ = ref_forward(cpu, xc, lambda t: sum_norm(elu_p1(t)), torch.zeros(B, H, d, d, dtype=torch.float64))
+    (ref * go).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), ref.detach().numpy()) < TOL
+    assert rel_err(xg.grad.cpu().numpy(), xc.grad.numpy()) < TOL
+    assert rel_err(gpu.slow_net.weight.grad.cpu().numpy(), cpu.slow_net.weight.grad.numpy()) < TOL
+
+    gpu2, cpu2 = _pair(CarryFastFFlayer(H, d, H * d, 0.0))
+    W0 = torch.randn(B, H, d, d, dtype=torch.float64) * 0.1
+    out, new_state = gpu2(x.to(_dev(), torch.float32), W0.to(_dev(), torch.float32))
+    ref, WL = ref_forward(cpu2, x, elu_p1_sum_norm_eps, W0)
+    assert rel_err(out.detach().cpu().numpy(), ref.detach().numpy()) < TOL
+    assert rel_err(new_state.cpu().numpy(), WL.detach().numpy()) < TOL
+
+
+def test_state_dict_names_match_the_reference_layers():
+    from layer import FastFFlayer, SRWMlayer
+    sd = SRWMlayer(2, 8, 16, 0.0).state_dict()
+    assert {"W_y", "W_q", "W_k", "w_b", "layer_norm.weight", "layer_norm.bias",
+            "out_linear.weight"} == set(sd)
+    assert sd["W_y"].shape == (1, 2, 8, 8) and sd["w_b"].shape == (1, 2, 8, 4)
+    assert {"slow_net.weight", "layer_norm.weight", "layer_norm.bias", "out_linear.weight"} == \
+        set(FastFFlayer(2, 8, 16, 0.0).state_dict())
