@@ -126,8 +126,10 @@ SRWM_API int delta_backward_f32(const float *Q, const int64_t q_strides[3],
  * Delta rule with bf16 inputs/outputs and fp32 memory.  No counterpart in the reference
  * (its kernels are float-only, fast_weight_cuda.cu:12-14); same recurrence as
  * delta_forward_f32 / delta_backward_f32 with
- *   Q, K, V, beta, out, grad_out, gQ, gK, gV, gbeta    bf16 (raw 16-bit patterns)
- *   W, gW, v_old, v_insert                              fp32
+ *   Q, K, V, beta, out, grad_out, gV       bf16 (raw 16-bit patterns)
+ *   W, gW, v_old, v_insert, gQ, gK, gbeta  fp32 (gQ, gK, gbeta are sums over the value axis and
+ *                                          may be accumulated by several workgroups; the caller
+ *                                          rounds them to bf16 if it wants them in that type)
  * All arithmetic is fp32; inputs are widened on load, outputs rounded to nearest even.
  */
 SRWM_API int delta_forward_bf16(const uint16_t *Q, const int64_t q_strides[3],
@@ -144,7 +146,7 @@ SRWM_API int delta_backward_bf16(const uint16_t *Q, const int64_t q_strides[3],
                         const float *v_old, const float *v_insert,
                         const uint16_t *grad_out, const int64_t grad_out_strides[3],
                         float *W,
-                        uint16_t *gQ, uint16_t *gK, uint16_t *gV, uint16_t *gbeta, float *gW,
+                        float *gQ, float *gK, uint16_t *gV, float *gbeta, float *gW,
                         int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
 /* Largest E the SRWM entry points accept (forward / backward), and the largest

@@ -183,8 +183,8 @@ int delta_forward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K
 int delta_backward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K, const int64_t ks[3],
                         const uint16_t *V, const int64_t vs[3], const uint16_t *beta,
                         const int64_t bs[3], const float *v_old, const float *v_insert,
-                        const uint16_t *grad_out, const int64_t gs[3], float *W, uint16_t *gQ,
-                        uint16_t *gK, uint16_t *gV, uint16_t *gbeta, float *gW, int N, int H, int L,
+                        const uint16_t *grad_out, const int64_t gs[3], float *W, float *gQ,
+                        float *gK, uint16_t *gV, float *gbeta, float *gW, int N, int H, int L,
                         int E, int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !grad_out || !W || !gQ || !gK || !gV ||
         !gbeta || !qs || !ks || !vs || !bs || !gs)

@@ -66,7 +66,9 @@ struct DeltaBwdParamsBf16 {
     const uint16_t *go;
     Strided3 gs;
     float *W;
-    uint16_t *gQ, *gK, *gV, *gbeta;
+    float *gQ, *gK;
+    uint16_t *gV;
+    float *gbeta;
     float *gW;
     int N, H, L, E, M;
     unsigned grad_state_mode;

@@ -12,6 +12,10 @@
 //             reduces its part with v_permlane{32,16}_swap, parks it in LDS, and the
 //             workgroup adds the per-wave parts once per tile and stores them coalesced.
 // The backward is ONE reverse sweep (the reference needs two plus a [N,H,L,M] temporary).
+// When there are fewer sequences than compute units, MS workgroups share a sequence, each
+// owning D/MS columns of the memory (columns never interact); their grad_q / grad_k /
+// grad_beta parts then meet through fp32 atomic adds on zero-filled outputs -- with MS = 2
+// that is two addends per word, so the result does not depend on their order.
 //
 // Replaces fast_weight_forward_kernel, fast_weight_backward_value_beta_kernel and
 // fast_weight_backward_query_key_kernel of the reference
@@ -23,17 +27,18 @@ namespace fw {
 
 namespace {
 
-template <int D, int NW, int R, int TT_>
+// D x D memory, MS workgroups per sequence, each owning MC = D / MS columns.
+template <int D, int MS_, int NW, int R, int TT_>
 struct DTiling {
+    static constexpr int MS = MS_;
+    static constexpr int MC = D / MS;         // columns of the memory owned by one workgroup
     static constexpr int NT = NW * kWave;
     static constexpr int RG = D / R;          // lanes per column group
     static constexpr int CGW = kWave / RG;    // column groups per wave
     static constexpr int NCG = NW * CGW;      // column groups per workgroup
-    static constexpr int CC = D / NCG;        // columns per lane
+    static constexpr int CC = MC / NCG;       // columns per lane
     static constexpr int TT = TT_;            // steps per tile
-    static constexpr int NV4 = TT * D / 4;    // float4s per tile vector
-    static constexpr int LD = (NV4 + NT - 1) / NT;  // float4 loads per thread per vector
-    static_assert(RG == 8 && RG * R == D && CC * NCG == D && CC >= 1, "tiling");
+    static_assert(RG == 8 && RG * R == D && CC * NCG == MC && CC >= 1 && MC * MS == D, "tiling");
     static_assert(TT <= NT, "beta loader");
 };
 
@@ -96,37 +101,40 @@ __device__ __forceinline__ void wr(bf16_t *dst, const float (&src)[N]) {
     }
 }
 
-// One tile vector (TT steps x D elements) moved global -> registers (as fp32) -> LDS as float4s.
+// One tile vector (TT steps x W elements) moved global -> registers (as fp32) -> LDS as float4s.
 // Rows past the end of the sequence are clamped to the last one: loaded, never used.
-template <class T>
+template <int NT, int TT, int W>
 struct TileVec {
-    float4 r[T::LD];
+    static constexpr int NV4 = TT * W / 4;           // float4s per tile vector
+    static constexpr int LD = (NV4 + NT - 1) / NT;   // float4 loads per thread
+    float4 r[LD];
     template <class TI>
     __device__ __forceinline__ void load(const TI *base, int64_t step_stride, int t0, int L, int tid) {
 #pragma unroll
-        for (int j = 0; j < T::LD; ++j) {
-            const int f = min(tid + j * T::NT, T::NV4 - 1);
-            const int row = min(t0 + f / (T::NV4 / T::TT), L - 1), col = (f % (T::NV4 / T::TT)) * 4;
+        for (int j = 0; j < LD; ++j) {
+            const int f = min(tid + j * NT, NV4 - 1);
+            const int row = min(t0 + f / (W / 4), L - 1), col = (f % (W / 4)) * 4;
             r[j] = ld4(base + (int64_t)row * step_stride + col);
         }
     }
     __device__ __forceinline__ void store(float *lds, int tid) const {
 #pragma unroll
-        for (int j = 0; j < T::LD; ++j) {
-            const int f = tid + j * T::NT;
-            if (f < T::NV4) reinterpret_cast<float4 *>(lds)[f] = r[j];
+        for (int j = 0; j < LD; ++j) {
+            const int f = tid + j * NT;
+            if (f < NV4) reinterpret_cast<float4 *>(lds)[f] = r[j];
         }
     }
 };
 
-// Stores one staged tile vector (rows x D floats in LDS) to global memory, 4 elements per
-// thread and store: full rows, consecutive lanes -> consecutive addresses.
-template <class T, int D, class TO>
-__device__ __forceinline__ void flush_rows(const float *lds, TO *gbase, int rows, int tid) {
-    for (int f = tid; f < rows * (D / 4); f += T::NT) {
+// Stores one staged tile vector (rows x W floats in LDS) to rows of `row_stride` elements in
+// global memory, 4 elements per thread and store: consecutive lanes -> consecutive addresses.
+template <int NT, int W, class TO>
+__device__ __forceinline__ void flush_rows(const float *lds, TO *gbase, int64_t row_stride, int rows,
+                                           int tid) {
+    for (int f = tid; f < rows * (W / 4); f += NT) {
         const float4 v = reinterpret_cast<const float4 *>(lds)[f];
         const float a[4] = {v.x, v.y, v.z, v.w};
-        wr<4>(gbase + (int64_t)f * 4, a);
+        wr<4>(gbase + (int64_t)(f / (W / 4)) * row_stride + (f % (W / 4)) * 4, a);
     }
 }
 
@@ -148,41 +156,46 @@ struct BwdP {
     const TI *go;
     Strided3 gs;
     float *W;
-    TI *gQ, *gK, *gV, *gbeta;
+    float *gQ, *gK;   // fp32 whatever TI is (they may be accumulated across workgroups)
+    TI *gV;
+    float *gbeta;
     float *gW;
     int N, H, L;
     unsigned grad_state_mode;
 };
 
-template <class TI, int D, int NW, int R, int TT>
+template <class TI, int D, int MS, int NW, int R, int TT>
 __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) {
-    using T = DTiling<D, NW, R, TT>;
-    constexpr int RG = T::RG, CGW = T::CGW, CC = T::CC;
-    enum { VQ, VK, VV, NVEC };
+    using T = DTiling<D, MS, NW, R, TT>;
+    constexpr int RG = T::RG, CGW = T::CGW, CC = T::CC, MC = T::MC, NT = T::NT;
     enum { OVO, OVI, OOUT, NOUT };
-    __shared__ __attribute__((aligned(16))) float tl[2][NVEC][TT][D];
+    __shared__ __attribute__((aligned(16))) float tq[2][TT][D];
+    __shared__ __attribute__((aligned(16))) float tk[2][TT][D];
+    __shared__ __attribute__((aligned(16))) float tv[2][TT][MC];
     __shared__ float tbeta[2][TT];
     // Outputs of a tile are parked here and written out after the step loop: the loop then
     // contains no global memory instruction, so the prefetch of the next tile stays in
     // flight across it, and the stores are full coalesced rows.
-    __shared__ __attribute__((aligned(16))) float ot[2][NOUT][TT][D];
+    __shared__ __attribute__((aligned(16))) float ot[2][NOUT][TT][MC];
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int rg = lane % RG, cg = wave * CGW + lane / RG;
     const int r0 = rg * R, c0 = cg * CC;
-    const int64_t seq = blockIdx.x;
+    const int64_t seq = blockIdx.x / MS;
+    const int m0 = (int)(blockIdx.x % MS) * MC;   // first memory column of this workgroup
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
     const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;
     const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
-    const TI *vb = p.V + n * p.vs.n + h * p.vs.h;
+    const TI *vb = p.V + n * p.vs.n + h * p.vs.h + m0;
     const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
-    float *Wg = p.W + seq * D * D;
+    float *Wg = p.W + seq * D * D + m0;
 
     float w[R][CC];
 #pragma unroll
     for (int i = 0; i < R; ++i) rd<CC>(w[i], Wg + (r0 + i) * D + c0);
 
-    TileVec<T> nq, nk, nv;
+    TileVec<NT, TT, D> nq, nk;
+    TileVec<NT, TT, MC> nv;
     float nb = 0.f;
     auto load_tile = [&](int tile) {
         const int t0 = tile * TT;
@@ -192,9 +205,9 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
         nb = ld1(bb + (int64_t)min(t0 + (tid % TT), p.L - 1) * p.bs.l);
     };
     auto store_tile = [&](int buf) {
-        nq.store(&tl[buf][VQ][0][0], tid);
-        nk.store(&tl[buf][VK][0][0], tid);
-        nv.store(&tl[buf][VV][0][0], tid);
+        nq.store(&tq[buf][0][0], tid);
+        nk.store(&tk[buf][0][0], tid);
+        nv.store(&tv[buf][0][0], tid);
         if (tid < TT) tbeta[buf][tid] = nb;
     };
 
@@ -214,9 +227,9 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
             float kr[R], qr[R], vc[CC], b;
         };
         auto fetch = [&](Ops &o, int tt) __attribute__((always_inline)) {
-            rd<R>(o.kr, &tl[buf][VK][tt][r0]);
-            rd<R>(o.qr, &tl[buf][VQ][tt][r0]);
-            rd<CC>(o.vc, &tl[buf][VV][tt][c0]);
+            rd<R>(o.kr, &tk[buf][tt][r0]);
+            rd<R>(o.qr, &tq[buf][tt][r0]);
+            rd<CC>(o.vc, &tv[buf][tt][c0]);
             o.b = tbeta[buf][tt];
         };
         auto step = [&](const Ops &o, int tt) __attribute__((always_inline)) {
@@ -271,42 +284,45 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
         }
         if (tile + 1 < ntiles) store_tile(buf ^ 1);
         __syncthreads();
-        const int64_t om = (seq * p.L + tile * TT) * D;
-        flush_rows<T, D>(&ot[buf][OVO][0][0], p.vold + om, tlen, tid);
-        flush_rows<T, D>(&ot[buf][OVI][0][0], p.vins + om, tlen, tid);
-        flush_rows<T, D>(&ot[buf][OOUT][0][0], p.out + om, tlen, tid);
+        const int64_t om = (seq * p.L + tile * TT) * D + m0;
+        flush_rows<NT, MC>(&ot[buf][OVO][0][0], p.vold + om, D, tlen, tid);
+        flush_rows<NT, MC>(&ot[buf][OVI][0][0], p.vins + om, D, tlen, tid);
+        flush_rows<NT, MC>(&ot[buf][OOUT][0][0], p.out + om, D, tlen, tid);
     }
 
 #pragma unroll
     for (int i = 0; i < R; ++i) wr<CC>(Wg + (r0 + i) * D + c0, w[i]);
 }
 
-template <class TI, int D, int NW, int R, int TT>
+template <class TI, int D, int MS, int NW, int R, int TT>
 __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) {
-    using T = DTiling<D, NW, R, TT>;
-    constexpr int RG = T::RG, CGW = T::CGW, NCG = T::NCG, CC = T::CC, NT = T::NT;
-    enum { VQ, VK, VV, VVO, VVI, VGO, NVEC };
-    __shared__ __attribute__((aligned(16))) float tl[2][NVEC][TT][D];
+    using T = DTiling<D, MS, NW, R, TT>;
+    constexpr int RG = T::RG, CGW = T::CGW, NCG = T::NCG, CC = T::CC, MC = T::MC, NT = T::NT;
+    enum { CV, CVO, CVI, CGO, NCV };                                  // column-side vectors of a step
+    __shared__ __attribute__((aligned(16))) float tq[2][TT][D];
+    __shared__ __attribute__((aligned(16))) float tk[2][TT][D];
+    __shared__ __attribute__((aligned(16))) float tc[2][NCV][TT][MC];
     __shared__ float tbeta[2][TT];
     __shared__ __attribute__((aligned(16))) float rowq[TT][NW][D];  // per-wave parts of grad_q
     __shared__ __attribute__((aligned(16))) float rowk[TT][NW][D];  // per-wave parts of grad_k
     __shared__ float gbp[TT][NCG];                                  // per column group parts of grad_beta
-    __shared__ __attribute__((aligned(16))) float gvt[TT][D];       // grad_v of the tile
+    __shared__ __attribute__((aligned(16))) float gvt[TT][MC];      // grad_v of the tile
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int rg = lane % RG, cg = wave * CGW + lane / RG;
     const int r0 = rg * R, c0 = cg * CC;
-    const int64_t seq = blockIdx.x;
+    const int64_t seq = blockIdx.x / MS;
+    const int m0 = (int)(blockIdx.x % MS) * MC;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
     const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;
     const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
-    const TI *vb = p.V + n * p.vs.n + h * p.vs.h;
-    const TI *gob = p.go + n * p.gs.n + h * p.gs.h;
+    const TI *vb = p.V + n * p.vs.n + h * p.vs.h + m0;
+    const TI *gob = p.go + n * p.gs.n + h * p.gs.h + m0;
     const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
-    const float *vob = p.vold + seq * p.L * D;
-    const float *vib = p.vins + seq * p.L * D;
-    float *Wg = p.W + seq * D * D;
-    float *gWg = p.gW ? p.gW + seq * D * D : nullptr;
+    const float *vob = p.vold + seq * p.L * D + m0;
+    const float *vib = p.vins + seq * p.L * D + m0;
+    float *Wg = p.W + seq * D * D + m0;
+    float *gWg = p.gW ? p.gW + seq * D * D + m0 : nullptr;
     const bool g_in = gWg && p.grad_state_mode != 0u;
 
     float w[R][CC], g[R][CC];
@@ -321,21 +337,24 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
         }
     }
 
-    TileVec<T> nv[NVEC];
+    TileVec<NT, TT, D> nq, nk;
+    TileVec<NT, TT, MC> nc[NCV];
     float nb = 0.f;
     auto load_tile = [&](int tile) {
         const int t0 = tile * TT;
-        nv[VQ].load(qb, p.qs.l, t0, p.L, tid);
-        nv[VK].load(kb, p.ks.l, t0, p.L, tid);
-        nv[VV].load(vb, p.vs.l, t0, p.L, tid);
-        nv[VVO].load(vob, D, t0, p.L, tid);
-        nv[VVI].load(vib, D, t0, p.L, tid);
-        nv[VGO].load(gob, p.gs.l, t0, p.L, tid);
+        nq.load(qb, p.qs.l, t0, p.L, tid);
+        nk.load(kb, p.ks.l, t0, p.L, tid);
+        nc[CV].load(vb, p.vs.l, t0, p.L, tid);
+        nc[CVO].load(vob, D, t0, p.L, tid);
+        nc[CVI].load(vib, D, t0, p.L, tid);
+        nc[CGO].load(gob, p.gs.l, t0, p.L, tid);
         nb = ld1(bb + (int64_t)min(t0 + (tid % TT), p.L - 1) * p.bs.l);
     };
     auto store_tile = [&](int buf) {
+        nq.store(&tq[buf][0][0], tid);
+        nk.store(&tk[buf][0][0], tid);
 #pragma unroll
-        for (int v = 0; v < NVEC; ++v) nv[v].store(&tl[buf][v][0][0], tid);
+        for (int v = 0; v < NCV; ++v) nc[v].store(&tc[buf][v][0][0], tid);
         if (tid < TT) tbeta[buf][tid] = nb;
     };
 
@@ -353,12 +372,12 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
             float kr[R], qr[R], go[CC], vi[CC], vv[CC], vo[CC], b;
         };
         auto fetch = [&](Ops &o, int tt) __attribute__((always_inline)) {
-            rd<R>(o.kr, &tl[buf][VK][tt][r0]);
-            rd<R>(o.qr, &tl[buf][VQ][tt][r0]);
-            rd<CC>(o.go, &tl[buf][VGO][tt][c0]);
-            rd<CC>(o.vi, &tl[buf][VVI][tt][c0]);
-            rd<CC>(o.vv, &tl[buf][VV][tt][c0]);
-            rd<CC>(o.vo, &tl[buf][VVO][tt][c0]);
+            rd<R>(o.kr, &tk[buf][tt][r0]);
+            rd<R>(o.qr, &tq[buf][tt][r0]);
+            rd<CC>(o.go, &tc[buf][CGO][tt][c0]);
+            rd<CC>(o.vi, &tc[buf][CVI][tt][c0]);
+            rd<CC>(o.vv, &tc[buf][CV][tt][c0]);
+            rd<CC>(o.vo, &tc[buf][CVO][tt][c0]);
             o.b = tbeta[buf][tt];
         };
         auto step = [&](const Ops &o, int tt) __attribute__((always_inline)) {
@@ -405,7 +424,7 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
             wr<CC>(&gvt[tt][c0], gv);
             gbp[tt][cg] = pb;
         };
-        if constexpr (D >= 128) {   // no registers to spare: keep the steps rolled
+        if constexpr (R >= 16) {   // no registers to spare: keep the steps rolled
             Ops a;
 #pragma unroll 1
             for (int tt = tlen - 1; tt >= 0; --tt) {
@@ -430,7 +449,8 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
             }
         }
         __syncthreads();
-        // add the per-wave parts of this tile and store grad_q, grad_k, grad_beta coalesced
+        // add the per-wave parts of this tile and store grad_q, grad_k, grad_beta coalesced;
+        // with several workgroups per sequence the parts of all of them meet by atomic add
         for (int idx = tid; idx < tlen * D; idx += NT) {
             const int tt = idx / D, e = idx - tt * D;
             float sq = 0.f, sk = 0.f;
@@ -440,16 +460,25 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
                 sk += rowk[tt][wv][e];
             }
             const int64_t oe = (seq * p.L + tile * TT + tt) * D + e;
-            st1(p.gQ + oe, sq);
-            st1(p.gK + oe, sk);
+            if constexpr (MS == 1) {
+                p.gQ[oe] = sq;
+                p.gK[oe] = sk;
+            } else {
+                atomicAdd(p.gQ + oe, sq);
+                atomicAdd(p.gK + oe, sk);
+            }
         }
         if (tid < tlen) {
             float s = 0.f;
 #pragma unroll
             for (int c = 0; c < NCG; ++c) s += gbp[tid][c];
-            st1(p.gbeta + seq * p.L + tile * TT + tid, s);
+            if constexpr (MS == 1) {
+                p.gbeta[seq * p.L + tile * TT + tid] = s;
+            } else {
+                atomicAdd(p.gbeta + seq * p.L + tile * TT + tid, s);
+            }
         }
-        flush_rows<T, D>(&gvt[0][0], p.gV + (seq * p.L + tile * TT) * D, tlen, tid);
+        flush_rows<NT, MC>(&gvt[0][0], p.gV + (seq * p.L + tile * TT) * D + m0, D, tlen, tid);
         if (tile > 0) store_tile(buf ^ 1);
         __syncthreads();
     }
@@ -466,15 +495,29 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
     }
 }
 
-template <class TI, int D, int NW, int R, int TT>
+// zero fill for the outputs that several workgroups accumulate into
+__global__ void zero_fill_kernel(float *a, int64_t na, float *b, int64_t nb, float *c, int64_t nc) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t j = i; j < na; j += stride) a[j] = 0.f;
+    for (int64_t j = i; j < nb; j += stride) b[j] = 0.f;
+    for (int64_t j = i; j < nc; j += stride) c[j] = 0.f;
+}
+
+template <class TI, int D, int MS, int NW, int R, int TT>
 int launch_f(const FwdP<TI> &p, hipStream_t s) {
-    hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, NW, R, TT>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, MS, NW, R, TT>), dim3(p.N * p.H * MS),
+                       dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
-template <class TI, int D, int NW, int R, int TT>
+template <class TI, int D, int MS, int NW, int R, int TT>
 int launch_b(const BwdP<TI> &p, hipStream_t s) {
-    hipLaunchKernelGGL((delta_bwd_tiled_kernel<TI, D, NW, R, TT>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    if (MS > 1) {
+        const int64_t ne = (int64_t)p.N * p.H * p.L * D, nb = (int64_t)p.N * p.H * p.L;
+        hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, s, p.gQ, ne, p.gK, ne, p.gbeta, nb);
+    }
+    hipLaunchKernelGGL((delta_bwd_tiled_kernel<TI, D, MS, NW, R, TT>), dim3(p.N * p.H * MS),
+                       dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
@@ -485,17 +528,21 @@ bool row_ok(const TI *ptr, const Strided3 &s) {
 }
 bool ok16(const void *ptr) { return (uintptr_t)ptr % 16 == 0; }
 
+// Two workgroups per sequence pay off when one per sequence would leave compute units idle.
+constexpr int kSplitBelowSequences = 192;
+
 template <class TI>
 int dispatch_fwd(const FwdP<TI> &p, int D, hipStream_t s) {
     if (!row_ok(p.Q, p.qs) || !row_ok(p.K, p.ks) || !row_ok(p.V, p.vs) || !ok16(p.vold) || !ok16(p.vins) ||
         !ok16(p.out) || !ok16(p.W))
         return -1;
+    const bool split = p.N * p.H <= kSplitBelowSequences;
     switch (D) {
-        case 128: return launch_f<TI, 128, 8, 16, 8>(p, s);
-        case 64: return launch_f<TI, 64, 4, 8, 16>(p, s);
-        case 32: return launch_f<TI, 32, 2, 4, 16>(p, s);
-        case 16: return launch_f<TI, 16, 1, 2, 16>(p, s);
-        case 8: return launch_f<TI, 8, 1, 1, 32>(p, s);
+        case 128: return split ? launch_f<TI, 128, 2, 4, 16, 8>(p, s) : launch_f<TI, 128, 1, 8, 16, 8>(p, s);
+        case 64: return split ? launch_f<TI, 64, 2, 2, 8, 16>(p, s) : launch_f<TI, 64, 1, 4, 8, 16>(p, s);
+        case 32: return launch_f<TI, 32, 1, 2, 4, 16>(p, s);
+        case 16: return launch_f<TI, 16, 1, 1, 2, 16>(p, s);
+        case 8: return launch_f<TI, 8, 1, 1, 1, 32>(p, s);
         default: return -1;
     }
 }
@@ -506,12 +553,13 @@ int dispatch_bwd(const BwdP<TI> &p, int D, hipStream_t s) {
         !ok16(p.vold) || !ok16(p.vins) || !ok16(p.W) || !ok16(p.gV) || !ok16(p.gQ) || !ok16(p.gK) ||
         (p.gW && !ok16(p.gW)))
         return -1;
+    const bool split = p.N * p.H <= kSplitBelowSequences;
     switch (D) {
-        case 128: return launch_b<TI, 128, 8, 16, 8>(p, s);
-        case 64: return launch_b<TI, 64, 4, 8, 8>(p, s);
-        case 32: return launch_b<TI, 32, 2, 4, 16>(p, s);
-        case 16: return launch_b<TI, 16, 1, 2, 16>(p, s);
-        case 8: return launch_b<TI, 8, 1, 1, 32>(p, s);
+        case 128: return split ? launch_b<TI, 128, 2, 4, 16, 8>(p, s) : launch_b<TI, 128, 1, 8, 16, 8>(p, s);
+        case 64: return split ? launch_b<TI, 64, 2, 2, 8, 8>(p, s) : launch_b<TI, 64, 1, 4, 8, 8>(p, s);
+        case 32: return launch_b<TI, 32, 1, 2, 4, 16>(p, s);
+        case 16: return launch_b<TI, 16, 1, 1, 2, 16>(p, s);
+        case 8: return launch_b<TI, 8, 1, 1, 1, 32>(p, s);
         default: return -1;
     }
 }

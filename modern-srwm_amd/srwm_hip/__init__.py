@@ -271,6 +271,11 @@ def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, g
     fn = lib().delta_backward_bf16 if io == torch.bfloat16 else lib().delta_backward_f32
     (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr), (gos, gstr) = (
         _strided(t) for t in (q, k, v, beta, grad_out))
+    if io == torch.bfloat16:
+        # sums over the value axis come back in fp32 and are rounded here
+        bf_outs = (grad_q, grad_k, grad_beta)
+        grad_q, grad_k, grad_beta = (torch.empty(t.shape, device=t.device, dtype=torch.float32)
+                                     for t in bf_outs)
     outs = [kv, grad_q, grad_k, grad_v, grad_beta] + ([grad_kv] if grad_kv is not None else [])
     with torch.cuda.device(q.device), _Dense([v_old, v_insert], False) as sv, _Dense(outs, True) as d:
         gkv = _ptr(d[5]) if grad_kv is not None else ctypes.c_void_p(None)
@@ -278,3 +283,6 @@ def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, g
                   _ptr(sv[0]), _ptr(sv[1]), _ptr(gos), gstr,
                   *[_ptr(t) for t in d[:5]], gkv, N, H, L, E, M, flags, _stream(q.device))
     _check(code, fn.__name__)
+    if io == torch.bfloat16:
+        for dst, src in zip(bf_outs, (grad_q, grad_k, grad_beta)):
+            dst.copy_(src)
