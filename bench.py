@@ -165,6 +165,36 @@ def cpu_baseline(op, N, H, L, E, budget_s=20.0):
                       "sequences are independent so tokens/s does not depend on the slice"}
 
 
+def measure_lds_peak(dev):
+    """LDS read bandwidth of the device in GB/s from the library's probe kernel (2048 workgroups,
+    i.e. 8 per CU, each lane streaming 16-byte reads)."""
+    import ctypes
+    import torch
+    import srwm_hip
+    L = srwm_hip.lib()
+    L.srwm_hip_lds_probe.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                     ctypes.c_void_p, ctypes.POINTER(ctypes.c_double)]
+    L.srwm_hip_lds_probe.restype = ctypes.c_int
+    wgs, iters = 2048, 4000
+    out = torch.empty(wgs * 256, device=dev)
+    nbytes = ctypes.c_double()
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    best = 0.0
+    for width in (16, 8, 4):
+        for rep in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            rc = L.srwm_hip_lds_probe(ctypes.c_void_p(out.data_ptr()), wgs, iters, width, stream,
+                                      ctypes.byref(nbytes))
+            e1.record()
+            torch.cuda.synchronize()
+            if rc:
+                return None
+            if rep:
+                best = max(best, nbytes.value / (e0.elapsed_time(e1) * 1e-3) / 1e9)
+    return best
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -229,6 +259,11 @@ def main():
         "roofline_fwd_bwd": roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS),
         "roofline_hbm": roof("hbm", hbm, fwd_ms + bwd_ms, HBM_PEAK_GBS),
     }
+    lds_meas = measure_lds_peak(dev)
+    if lds_meas:
+        res["lds_peak_measured_GBs"] = round(lds_meas, 1)
+        res["roofline_fwd_bwd"]["frac_of_measured_lds_peak"] = round(
+            res["roofline_fwd_bwd"]["achieved"] / lds_meas, 4)
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline("srwm" if op == "srwm" else "delta", N, H, L, E, a.cpu_budget)
     print(json.dumps(res))

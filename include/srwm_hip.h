@@ -153,6 +153,14 @@ SRWM_API int delta_backward_bf16(const uint16_t *Q, const int64_t q_strides[3],
  * E == M the delta entry points accept, on the current device. */
 SRWM_API int srwm_hip_limits(int *srwm_fwd_max_E, int *srwm_bwd_max_E, int *delta_max_EM);
 
+/* Measurement aid, not part of the operator path: enqueues a kernel in which `workgroups`
+ * workgroups of 256 threads each issue `iters` x 8 conflict-free LDS reads of `bytes_per_lane`
+ * (4, 8 or 16) bytes per thread,
+ * writes workgroups*256 floats to `out` (device) and reports the LDS bytes read in
+ * *bytes_read (host).  The caller times it to obtain the LDS read bandwidth of the device. */
+SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes_per_lane, void *stream,
+                                double *bytes_read);
+
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 

@@ -503,7 +503,7 @@ int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
     for (const void *d : dense)
         if ((uintptr_t)d % 16) return -1;
     switch (p.E) {
-        case 64: return launch_fwd<64, 4, 8>(p, s);
+        case 64: return launch_fwd<64, 4, 16>(p, s);
         case 32: return launch_fwd<32, 4, 4>(p, s);
         case 16: return launch_fwd<16, 1, 2>(p, s);
         case 8: return launch_fwd<8, 1, 1>(p, s);
