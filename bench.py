@@ -39,6 +39,10 @@ WORKLOADS = {
     "delta_c2": ("delta", 32, 8, 256, 64),
     "delta_c5f32": ("delta", 8, 16, 4096, 128),
     "delta_c5": ("delta_bf16", 8, 16, 4096, 128),     # bf16 q/k/v/beta/out/grads, fp32 memory
+    # same shapes with the chunkwise (chunk = 64) MFMA forward; the backward is the step-by-step one
+    "delta_c2_chunk": ("delta", 32, 8, 256, 64),
+    "delta_c5f32_chunk": ("delta", 8, 16, 4096, 128),
+    "delta_c5_chunk": ("delta_bf16", 8, 16, 4096, 128),
 }
 
 
@@ -105,7 +109,8 @@ def delta_step(t, ev=None):
     t["W"].zero_()
     if ev:
         ev[0].record()
-    srwm_hip.fast_weight_forward(t["q"], t["k"], t["v"], t["beta"], t["vold"], t["vins"], t["W"], t["out"])
+    srwm_hip.fast_weight_forward(t["q"], t["k"], t["v"], t["beta"], t["vold"], t["vins"], t["W"], t["out"],
+                                 flags=t.get("fwd_flags", 0))
     if ev:
         ev[1].record()
     srwm_hip.fast_weight_backward(t["q"], t["k"], t["v"], t["beta"], t["vold"], t["vins"], t["go"],
@@ -222,6 +227,8 @@ def main():
     else:
         step = delta_step
         t = delta_setup(N, H, L, E, dev, torch.bfloat16 if op == "delta_bf16" else torch.float32)
+        if a.workload.endswith("_chunk"):
+            t["fwd_flags"] = srwm_hip.FLAG_CHUNKWISE
 
     for _ in range(a.warmup):
         step(t)

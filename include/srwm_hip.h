@@ -47,6 +47,8 @@ extern "C" {
                                      it, :1213-1229); equal to ZERO when the buffers arrive zeroed. */
 #define SRWM_GRAD_STATE_MASK 3u
 #define SRWM_FLAG_GENERIC 16u     /* force the any-size LDS-resident kernel (testing / comparison) */
+#define SRWM_FLAG_CHUNKWISE 32u   /* delta forward only: chunkwise (chunk = 64) MFMA kernel instead of the
+                                     step-by-step one; E == M in {64, 128}, else SRWM_ENOKERNEL */
 
 /*
  * SRWM forward.  Replaces self_ref_forward(), supervised_learning/self_ref_v0/

@@ -104,6 +104,9 @@ int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s);
 int launch_delta_fwd_tiled(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_bwd_tiled(const DeltaBwdParams &p, hipStream_t s);
 int launch_delta_fwd_tiled_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s);
+// Chunkwise (chunk = 64) forward on the matrix cores, E == M in {64, 128}; -1 otherwise.
+int launch_delta_fwd_chunk(const DeltaFwdParams &p, hipStream_t s);
+int launch_delta_fwd_chunk_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s);
 int launch_delta_bwd_tiled_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s);
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // gfx950: 160 KB of LDS per CU / workgroup

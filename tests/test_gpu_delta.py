@@ -176,3 +176,52 @@ def test_bf16_io_matches_oracle_on_rounded_inputs(shape, qk):
         assert leaf.grad.dtype == torch.bfloat16
         assert rel_err(leaf.grad.float().cpu().numpy(), ob[n]) < BF16_TOL, n
     assert W.abs().max().item() < 1e-4 * max(1.0, float(np.abs(of["W"]).max()))   # reverted to W_0 = 0
+
+
+# ------------------------------------------------------------------ chunkwise MFMA forward
+
+@pytest.mark.parametrize("shape,qk,w0,io", [
+    ((2, 3, 64, 64, 64), "softmax", 0.0, torch.float32),     # exactly one chunk
+    ((2, 2, 200, 64, 64), "softmax", 0.3, torch.float32),    # ragged last chunk, non-zero memory
+    ((1, 3, 256, 128, 128), "l2", 0.0, torch.float32),       # two workgroups per sequence
+    ((1, 2, 37, 128, 128), "l2", 0.2, torch.float32),        # shorter than a chunk
+    ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # BASELINE config 5 style, shorter
+])
+def test_chunkwise_forward_matches_oracle_and_feeds_the_sequential_backward(shape, qk, w0, io):
+    """Chunkwise (C = 64) MFMA forward vs the fp64 oracle, then the step-by-step backward run on
+    the v_old / v_insert it emitted."""
+    print(f"case chunkwise shape={shape} io={io}", flush=True)
+    import srwm_hip
+    dev = _dev()
+    tol = TOL if io == torch.float32 else BF16_TOL
+    q, k, v, beta, W0, go = delta_inputs(*shape, seed=13, qk=qk, w0_std=w0)
+    qi, ki, vi, bi, goi = (t.to(io) for t in (q, k, v, beta, go))
+    base = [t.to(torch.float64).numpy() for t in (qi, ki, vi, bi)] + [W0.numpy()]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, goi.to(torch.float64).numpy())
+    N, H, L, E = q.shape
+    qd, kd, vd, bd, god = (t.to(dev) for t in (qi, ki, vi, bi, goi))
+    W = W0.to(dev, torch.float32).contiguous()
+    nan = lambda *s, dt=torch.float32: torch.full(s, float("nan"), device=dev, dtype=dt)
+    vold, vins, out = nan(N, H, L, E), nan(N, H, L, E), nan(N, H, L, E, dt=io)
+    srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out, flags=srwm_hip.FLAG_CHUNKWISE)
+    errs = {"out": rel_err(out.float().cpu().numpy(), of["out"]),
+            "v_old": rel_err(vold.cpu().numpy(), of["v_old"]),
+            "v_insert": rel_err(vins.cpu().numpy(), of["v_insert"]),
+            "W": rel_err(W.cpu().numpy(), of["W"])}
+    gq, gk, gv, gb = nan(N, H, L, E, dt=io), nan(N, H, L, E, dt=io), nan(N, H, L, E, dt=io), nan(N, H, L, 1, dt=io)
+    srwm_hip.fast_weight_backward(qd, kd, vd, bd, vold, vins, god, W, gq, gk, gv, gb)
+    for n, t in (("grad_Q", gq), ("grad_K", gk), ("grad_V", gv), ("grad_beta", gb)):
+        errs[n] = rel_err(t.float().cpu().numpy(), ob[n])
+    bad = {n: e for n, e in errs.items() if not (e < tol)}
+    assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
+
+
+def test_chunkwise_flag_is_refused_where_there_is_no_kernel():
+    import srwm_hip
+    dev = _dev()
+    z = lambda *s: torch.zeros(*s, device=dev)
+    with pytest.raises(RuntimeError, match="no kernel"):
+        srwm_hip.fast_weight_forward(z(1, 1, 8, 32), z(1, 1, 8, 32), z(1, 1, 8, 32), z(1, 1, 8, 1),
+                                     z(1, 1, 8, 32), z(1, 1, 8, 32), z(1, 1, 32, 32), z(1, 1, 8, 32),
+                                     flags=srwm_hip.FLAG_CHUNKWISE)

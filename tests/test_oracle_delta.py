@@ -114,3 +114,19 @@ def test_f32_oracle_tracks_f64():
     b32 = oracle.delta_backward(*base[:4], f32, go.numpy(), dtype=np.float32)
     for n in ("grad_Q", "grad_K", "grad_V", "grad_beta"):
         assert rel_err(b32[n], b64[n]) < 1e-4, n
+
+
+# ---------------------------------------------------------- chunkwise restatement
+
+@pytest.mark.parametrize("chunk", [1, 5, 16, 64, 1000])
+@pytest.mark.parametrize("blocked", [False, True])
+def test_chunkwise_form_equals_the_sequential_recurrence(chunk, blocked):
+    """Any chunk size (1, not a divisor of L, a multiple of the 16-row block, >= L) and both
+    triangular solvers must reproduce the per-step oracle."""
+    from oracle.chunkwise import delta_forward_chunkwise
+    q, k, v, beta, W0, _ = delta_inputs(2, 2, 150, 12, 10, seed=9, qk="l2", w0_std=0.3)
+    base = _np((q, k, v, beta, W0))
+    seq = oracle.delta_forward(*base)
+    ch = delta_forward_chunkwise(*base, chunk=chunk, blocked=blocked)
+    for n in ("out", "v_old", "v_insert", "W"):
+        assert rel_err(ch[n], seq[n]) < 1e-11, n
