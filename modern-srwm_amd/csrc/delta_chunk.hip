@@ -111,28 +111,55 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
 #pragma unroll
         for (int r = 0; r < 4; ++r) s[eb][r] = Wg[(eb * 16 + 4 * lq + r) * D + ln];
 
+    // The chunk inputs are fetched one chunk ahead into registers (all loads in flight at
+    // once) and written to LDS as fp32 after the previous chunk is done with it.
+    constexpr int NKQ = kC * (D / 4) / kThreads;    // float4s of K (and of Q) per thread
+    constexpr int NV = kC * (kMC / 4) / kThreads;   // float4s of V per thread
+    float4 kreg[NKQ], qreg[NKQ], vreg[NV];
+    float breg = 0.f;
+    auto prefetch = [&](int ch) {   // rows past the end are clamped here and zeroed in commit()
+        const int t0 = ch * kC;
+#pragma unroll
+        for (int i = 0; i < NKQ; ++i) {
+            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const int t = min(t0 + row, p.L - 1);
+            kreg[i] = ld4(kb + (int64_t)t * p.ks.l + col);
+            qreg[i] = ld4(qb + (int64_t)t * p.qs.l + col);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int f = tid + i * kThreads, row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
+            vreg[i] = ld4(vb + (int64_t)min(t0 + row, p.L - 1) * p.vs.l + col);
+        }
+        breg = ld1(bb + (int64_t)min(t0 + (tid % kC), p.L - 1) * p.bs.l);
+    };
+    auto masked = [](const float4 &v, float m) { return make_float4(v.x * m, v.y * m, v.z * m, v.w * m); };
+    auto commit = [&](int ch) {
+        const int t0 = ch * kC;
+        const bool full = t0 + kC <= p.L;   // only the last chunk can be ragged
+#pragma unroll
+        for (int i = 0; i < NKQ; ++i) {
+            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const float m = (full || t0 + row < p.L) ? 1.f : 0.f;
+            *reinterpret_cast<float4 *>(Ks + row * LDK + col) = masked(kreg[i], m);
+            *reinterpret_cast<float4 *>(Qs + row * LDK + col) = masked(qreg[i], m);
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int f = tid + i * kThreads, row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
+            const float m = (full || t0 + row < p.L) ? 1.f : 0.f;
+            *reinterpret_cast<float4 *>(Vs + row * LDV + col) = masked(vreg[i], m);
+        }
+        if (tid < kC) bts[tid] = (t0 + tid < p.L) ? breg : 0.f;
+    };
+
     const int nchunks = (p.L + kC - 1) / kC;
+    prefetch(0);
+    commit(0);
+    __syncthreads();
     for (int ch = 0; ch < nchunks; ++ch) {
         const int t0 = ch * kC;
-        // ---- stage K, Q, V, beta of the chunk in LDS as fp32 (rows past the end: zeros)
-        for (int f = tid; f < kC * (D / 4); f += kThreads) {
-            const int row = f / (D / 4), col = (f % (D / 4)) * 4;
-            float4 kv = make_float4(0.f, 0.f, 0.f, 0.f), qv = kv;
-            if (t0 + row < p.L) {
-                kv = ld4(kb + (int64_t)(t0 + row) * p.ks.l + col);
-                qv = ld4(qb + (int64_t)(t0 + row) * p.qs.l + col);
-            }
-            *reinterpret_cast<float4 *>(Ks + row * LDK + col) = kv;
-            *reinterpret_cast<float4 *>(Qs + row * LDK + col) = qv;
-        }
-        for (int f = tid; f < kC * (kMC / 4); f += kThreads) {
-            const int row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
-            float4 vv = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (t0 + row < p.L) vv = ld4(vb + (int64_t)(t0 + row) * p.vs.l + col);
-            *reinterpret_cast<float4 *>(Vs + row * LDV + col) = vv;
-        }
-        if (tid < kC) bts[tid] = (t0 + tid < p.L) ? ld1(bb + (int64_t)(t0 + tid) * p.bs.l) : 0.f;
-        __syncthreads();
+        if (ch + 1 < nchunks) prefetch(ch + 1);
 
         // ---- A = K K^T (strict lower) and B = Q K^T (lower), 10 + 10 tiles over the 4 waves
         for (int tix = wave; tix < 20; tix += 4) {
@@ -141,7 +168,7 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
             const int cj = tri - (ci * (ci + 1)) / 2;
             const float *X = which ? Qs : Ks;
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+#pragma unroll
             for (int eb = 0; eb < EB; ++eb) {
                 const float4 a = *reinterpret_cast<const float4 *>(X + (ci * 16 + ln) * LDK + eb * 16 + 4 * lq);
                 const float4 b = *reinterpret_cast<const float4 *>(Ks + (cj * 16 + ln) * LDK + eb * 16 + 4 * lq);
@@ -170,14 +197,13 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
                 for (int j = 0; j < i; ++j) acc = fmaf(-bi * Ad[i * LDA + j], x[j], acc);
                 x[i] = acc;
             }
-            if (lane < 16) {
+            // lanes 16..63 hold copies of columns 0..15: everybody stores, no branch
 #pragma unroll
-                for (int i = 0; i < 16; ++i) Di[(wave * 16 + i) * LDD + ln] = x[i];
-            }
+            for (int i = 0; i < 16; ++i) Di[(wave * 16 + i) * LDD + ln] = x[i];
         }
-        __syncthreads();
 
-        // ---- everything below is per wave (its 16 columns), no synchronisation
+        // ---- P = K S and Q S for this wave's 16 columns: independent of the inversion above
+        //      (matrix-core work that can overlap its vector-ALU chain)
         f32x4 pt[kCB], ot[kCB], u[kCB];
 #pragma unroll
         for (int cb = 0; cb < kCB; ++cb) {
@@ -191,6 +217,9 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
                 ot[cb] = mma4(qa, s[eb], ot[cb]);   // Q S
             }
         }
+        __syncthreads();   // the four inverses are visible
+
+        // ---- everything below is per wave (its 16 columns), no synchronisation
         // block forward substitution, one 16-row block at a time
 #pragma unroll
         for (int a = 0; a < kCB; ++a) {
@@ -239,7 +268,11 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
                 kt.w = Ks[(cb * 16 + 4 * lq + 3) * LDK + eb * 16 + ln];
                 s[eb] = mma4(kt, u[cb], s[eb]);
             }
-        __syncthreads();   // the next chunk overwrites Ks, Qs, Vs, As, Bs
+        __syncthreads();   // every wave is done with Ks, Qs, Vs, As, Bs
+        if (ch + 1 < nchunks) {
+            commit(ch + 1);
+            __syncthreads();
+        }
     }
 
 #pragma unroll

@@ -14,7 +14,25 @@ import torch
 
 import srwm_hip
 
-causal_dot_product_cuda = srwm_hip.fast_weight_forward
+# Forward kernel choice: "auto" runs the chunkwise (chunk = 64) matrix-core kernel when it
+# exists for the shape (E == M in {64, 128}, at least one full chunk) and the step-by-step kernel
+# otherwise; True / False force one of them.  Both emit the same v_old / v_insert, so the
+# backward (always the step-by-step reverse sweep) is unaffected.
+CHUNKWISE_FORWARD = "auto"
+
+
+def _forward_flags(E, M, L):
+    has_kernel = E == M and E in (64, 128)
+    if CHUNKWISE_FORWARD is True or (CHUNKWISE_FORWARD == "auto" and has_kernel and L >= 64):
+        return srwm_hip.FLAG_CHUNKWISE
+    return 0
+
+
+def causal_dot_product_cuda(q, k, v, beta, v_old, v_insert, kv, out):
+    srwm_hip.fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out,
+                                 flags=_forward_flags(q.shape[-1], v.shape[-1], q.shape[2]))
+
+
 causal_dot_backward_cuda = srwm_hip.fast_weight_backward
 
 

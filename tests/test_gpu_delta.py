@@ -185,6 +185,8 @@ def test_bf16_io_matches_oracle_on_rounded_inputs(shape, qk):
     ((2, 2, 200, 64, 64), "softmax", 0.3, torch.float32),    # ragged last chunk, non-zero memory
     ((1, 3, 256, 128, 128), "l2", 0.0, torch.float32),       # two workgroups per sequence
     ((1, 2, 37, 128, 128), "l2", 0.2, torch.float32),        # shorter than a chunk
+    ((1, 2, 2048, 128, 128), "l2", 0.0, torch.float32),      # 32 chunks in a row
+    ((2, 8, 256, 64, 64), "softmax", 0.0, torch.float32),    # BASELINE config 2 style
     ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # BASELINE config 5 style, shorter
 ])
 def test_chunkwise_forward_matches_oracle_and_feeds_the_sequential_backward(shape, qk, w0, io):
