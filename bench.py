@@ -16,7 +16,7 @@ achieved HBM rate of the operator's I/O contract.  `cpu_baseline` is the per-tim
 PyTorch recurrence (oracle/recurrence.py) timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, delta_c2, delta_c5f32}.
+{srwm_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk}.
 """
 import argparse
 import json
@@ -31,6 +31,17 @@ for p in (ROOT, os.path.join(ROOT, "modern-srwm_amd")):
 
 LDS_PEAK_GBS = 256 * 128 * 2.4          # 256 CUs x 128 B/clk x 2.4 GHz = 78 643 GB/s
 HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch of the dominant (backward) kernel, measured with rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE (two runs; FETCH_SIZE scaled by the factor that makes a plain copy of known size
+# read its size).  Figures and commands: profiles/srwm_c4_kernels.txt, profiles/delta_kernels.txt.
+MEASURED_TRAFFIC_BYTES = {
+    "srwm_c4": (490477 + 90624) * 1024,
+    "delta_c2": (102444 + 53504) * 1024,
+    "delta_c2_chunk": (102444 + 53504) * 1024,
+    "delta_c5": (1316488 + 1191936) * 1024,
+    "delta_c5_chunk": (1316488 + 1191936) * 1024,
+}
 
 WORKLOADS = {
     # name: (op, N, H, L, E)
@@ -162,12 +173,17 @@ def cpu_baseline(op, N, H, L, E, budget_s=20.0):
 
     run(1)                                  # warm-up (thread pool, allocator)
     t1 = run(1)
-    n = max(1, min(N, int(budget_s / max(t1, 1e-3))))
-    tn = run(n) if n > 1 else t1
+    n = max(1, min(N, int(budget_s / 4 / max(t1, 1e-3))))
+    times = []
+    t_start = time.perf_counter()
+    while not times or (time.perf_counter() - t_start < budget_s * 0.6 and len(times) < 20):
+        times.append(run(n))
+    times.sort()
+    tn = times[len(times) // 2]
     return {"value": n * L / tn, "unit": "tokens/s", "cores": cores, "kind": "port",
             "sample": f"oracle/recurrence.py ({op}) fwd+autograd bwd, fp32, batch slice N={n} of {N} "
-                      f"(H={H}, L={L}, E={E}) in {tn:.2f}s, torch {cores} threads; "
-                      "sequences are independent so tokens/s does not depend on the slice"}
+                      f"(H={H}, L={L}, E={E}), median of {len(times)} runs of {tn:.2f}s, torch {cores} "
+                      "threads; sequences are independent so tokens/s does not depend on the slice"}
 
 
 def measure_lds_peak(dev):
@@ -208,6 +224,7 @@ def main():
     ap.add_argument("--workload", default="srwm_c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
+    ap.add_argument("--no-lds-probe", action="store_true")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this operator runs on ONE GPU (sequences shard over GPUs without any "
@@ -262,11 +279,12 @@ def main():
         "config": {"workload": f"{a.workload}: {op} fwd+bwd N={N} H={H} L={L} E={E}, fp32 state, "
                                "state re-initialised per step, seeded synthetic inputs"},
         "kernel_ms": {"forward": round(fwd_ms, 4), "backward": round(bwd_ms, 4)},
-        "roofline": dict(roof("lds", lds_b, bwd_ms, LDS_PEAK_GBS), kernel="backward"),
+        "roofline": dict(roof("lds", lds_b, bwd_ms, LDS_PEAK_GBS), kernel="backward",
+                         traffic=MEASURED_TRAFFIC_BYTES.get(a.workload)),
         "roofline_fwd_bwd": roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS),
         "roofline_hbm": roof("hbm", hbm, fwd_ms + bwd_ms, HBM_PEAK_GBS),
     }
-    lds_meas = measure_lds_peak(dev)
+    lds_meas = None if a.no_lds_probe else measure_lds_peak(dev)
     if lds_meas:
         res["lds_peak_measured_GBs"] = round(lds_meas, 1)
         res["roofline_fwd_bwd"]["frac_of_measured_lds_peak"] = round(
