@@ -3,9 +3,11 @@
 // One workgroup of NW wave64s owns one (batch, head) sequence for all L steps; the D x D
 // memory W (and its gradient G in the backward) lives in registers, cut into tiles of
 // R rows x CC columns: lane (rg, cg) holds rows [R*rg, R*rg+R) of columns [CC*cg, CC*cg+CC).
-// The 8 lanes of a column group are consecutive, so every column sum (W^T k, W^T q, G^T k)
-// -- the only reductions the recurrence itself depends on -- finishes with three DPP adds
-// inside the wave.  Columns of the delta rule evolve independently, so the waves never
+// The 8 or 16 lanes of a column group are consecutive, so every column sum (W^T k, W^T q,
+// G^T k) -- the only reductions the recurrence itself depends on -- finishes with three or
+// four DPP adds inside a 16-lane row.  (Tilings with 16-lane groups spread a sequence over
+// twice the waves: two waves per SIMD hide each other's dependency stalls, which pays in the
+// backward and for the 128 x 128 memory.)  Columns of the delta rule evolve independently, so the waves never
 // have to meet inside a step:
 //   forward   no workgroup barrier per step at all (one per input tile);
 //   backward  the row sums (grad_q, grad_k) and grad_beta are outputs only: each wave
@@ -38,7 +40,7 @@ struct DTiling {
     static constexpr int NCG = NW * CGW;      // column groups per workgroup
     static constexpr int CC = MC / NCG;       // columns per lane
     static constexpr int TT = TT_;            // steps per tile
-    static_assert(RG == 8 && RG * R == D && CC * NCG == MC && CC >= 1 && MC * MS == D, "tiling");
+    static_assert((RG == 8 || RG == 16) && RG * R == D && CC * NCG == MC && CC >= 1 && MC * MS == D, "tiling");
     static_assert(TT <= NT, "beta loader");
 };
 
@@ -414,7 +416,9 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
                     ak[i] = fmaf(w[i][c], gvo[c], ak[i]);
                     g[i][c] = fmaf(o.kr[i], gvo[c], g[i][c]);
                 }
-            if constexpr (R >= 2) {
+            if constexpr (RG == 16) {
+                stride16_reduce_store2<R>(aq, ak, &rowq[tt][wave][r0], &rowk[tt][wave][r0], lane);
+            } else if constexpr (R >= 2) {
                 stride8_reduce_store2<R>(aq, ak, &rowq[tt][wave][r0], &rowk[tt][wave][r0], lane);
             } else {
                 stride8_reduce_store<R>(aq, &rowq[tt][wave][r0], lane);
@@ -538,7 +542,7 @@ int dispatch_fwd(const FwdP<TI> &p, int D, hipStream_t s) {
         return -1;
     const bool split = p.N * p.H <= kSplitBelowSequences;
     switch (D) {
-        case 128: return split ? launch_f<TI, 128, 2, 4, 16, 8>(p, s) : launch_f<TI, 128, 1, 8, 16, 8>(p, s);
+        case 128: return split ? launch_f<TI, 128, 2, 8, 8, 8>(p, s) : launch_f<TI, 128, 1, 8, 16, 8>(p, s);
         case 64: return split ? launch_f<TI, 64, 2, 2, 8, 16>(p, s) : launch_f<TI, 64, 1, 4, 8, 16>(p, s);
         case 32: return launch_f<TI, 32, 1, 2, 4, 16>(p, s);
         case 16: return launch_f<TI, 16, 1, 1, 2, 16>(p, s);
@@ -555,8 +559,8 @@ int dispatch_bwd(const BwdP<TI> &p, int D, hipStream_t s) {
         return -1;
     const bool split = p.N * p.H <= kSplitBelowSequences;
     switch (D) {
-        case 128: return split ? launch_b<TI, 128, 2, 4, 16, 8>(p, s) : launch_b<TI, 128, 1, 8, 16, 8>(p, s);
-        case 64: return split ? launch_b<TI, 64, 2, 2, 8, 8>(p, s) : launch_b<TI, 64, 1, 4, 8, 8>(p, s);
+        case 128: return split ? launch_b<TI, 128, 2, 8, 8, 8>(p, s) : launch_b<TI, 128, 1, 8, 16, 8>(p, s);
+        case 64: return split ? launch_b<TI, 64, 2, 4, 4, 16>(p, s) : launch_b<TI, 64, 1, 8, 4, 16>(p, s);
         case 32: return launch_b<TI, 32, 1, 2, 4, 16>(p, s);
         case 16: return launch_b<TI, 16, 1, 1, 2, 16>(p, s);
         case 8: return launch_b<TI, 8, 1, 1, 1, 32>(p, s);

@@ -242,6 +242,36 @@ __device__ __forceinline__ void stride8_reduce_store2(const float (&a)[R], const
     }
 }
 
+// The same for column groups of 16 lanes: sums over the 4 lanes {l, l^16, l^32, l^48}.  Lanes
+// 0..31 end up with results of `a`, lanes 32..63 with results of `b`; even rows hold the first
+// R/2 of them, odd rows the rest, and every lane stores.
+template <int R>
+__device__ __forceinline__ void stride16_reduce_store2(const float (&a)[R], const float (&b)[R],
+                                                       float *dst_a, float *dst_b, int lane) {
+    static_assert(R >= 2, "needs at least two values per lane");
+    constexpr int NB = R / 2;
+    float v[2 * R], h[R], q[NB];
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+        v[i] = a[i];
+        v[R + i] = b[i];
+    }
+    swap_halve<32, 2 * R>(v, h);
+    swap_halve<16, R>(h, q);
+    const int b5 = (lane >> 5) & 1, b4 = (lane >> 4) & 1;
+    float *dst = (b5 ? dst_b : dst_a) + NB * b4;
+    if constexpr (NB == 2) {
+        *reinterpret_cast<float2 *>(dst) = make_float2(q[0], q[1]);
+    } else if constexpr (NB % 4 == 0) {
+#pragma unroll
+        for (int i = 0; i < NB / 4; ++i)
+            reinterpret_cast<float4 *>(dst)[i] = make_float4(q[4 * i], q[4 * i + 1], q[4 * i + 2], q[4 * i + 3]);
+    } else {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) dst[i] = q[i];
+    }
+}
+
 // Sum over the lane pair (l, l^32) / (l, l^16), result in both lanes.
 __device__ __forceinline__ float swap_add32(float x, float y) {
     swap_pairs<32>(x, y);

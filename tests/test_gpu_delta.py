@@ -219,6 +219,46 @@ def test_chunkwise_forward_matches_oracle_and_feeds_the_sequential_backward(shap
     assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
 
 
+def test_full_config5_properties():
+    """BASELINE config 5 at full size (N=8, H=16, L=4096, E=M=128, bf16 I/O, fp32 memory):
+    the step-by-step and the chunkwise forward agree with each other, the backward reverts the
+    memory to W_0 = 0, and sampled sequences match the fp64 oracle run on the rounded inputs."""
+    print("case full C5 properties", flush=True)
+    import srwm_hip
+    dev = _dev()
+    N, H, L, E = 8, 16, 4096, 128
+    q, k, v, beta, W0, go = delta_inputs(N, H, L, E, E, seed=0, qk="l2", dtype=torch.float32)
+    qd, kd, vd, bd, god = (t.to(dev, torch.bfloat16) for t in (q, k, v, beta, go))
+    new = lambda last, dt: torch.full((N, H, L, last), float("nan"), device=dev, dtype=dt)
+    res = {}
+    for name, flags in (("seq", 0), ("chunk", srwm_hip.FLAG_CHUNKWISE)):
+        W = torch.zeros(N, H, E, E, device=dev)
+        vold, vins, out = new(E, torch.float32), new(E, torch.float32), new(E, torch.bfloat16)
+        srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out, flags=flags)
+        res[name] = dict(W=W, v_old=vold, v_insert=vins, out=out)
+    for n in ("W", "v_old", "v_insert"):
+        a, b = res["seq"][n], res["chunk"][n]
+        assert torch.isfinite(a).all() and torch.isfinite(b).all(), n
+        assert (a - b).abs().max().item() < 1e-4 * b.abs().max().item(), n
+    assert (res["seq"]["out"].float() - res["chunk"]["out"].float()).abs().max().item() \
+        < 1e-2 * res["chunk"]["out"].float().abs().max().item()
+    r = res["chunk"]
+    WL = r["W"].clone()
+    gq, gk, gv, gb = new(E, torch.bfloat16), new(E, torch.bfloat16), new(E, torch.bfloat16), new(1, torch.bfloat16)
+    srwm_hip.fast_weight_backward(qd, kd, vd, bd, r["v_old"], r["v_insert"], god, r["W"], gq, gk, gv, gb)
+    torch.cuda.synchronize()
+    assert r["W"].abs().max().item() < 1e-4 * WL.abs().max().item()        # reverted to W_0 = 0
+    for (n_, h_) in ((0, 0), (7, 15)):
+        sl = (slice(n_, n_ + 1), slice(h_, h_ + 1))
+        base = [t[sl].float().cpu().to(torch.float64).numpy() for t in (qd, kd, vd, bd)] + [W0[sl].double().numpy()]
+        of = oracle.delta_forward(*base)
+        ob = oracle.delta_backward(*base[:4], of, god[sl].float().cpu().to(torch.float64).numpy())
+        assert rel_err(WL[sl].cpu().numpy(), of["W"]) < BF16_TOL
+        assert rel_err(r["out"][sl].float().cpu().numpy(), of["out"]) < BF16_TOL
+        for t, n in ((gq, "grad_Q"), (gk, "grad_K"), (gv, "grad_V"), (gb, "grad_beta")):
+            assert rel_err(t[sl].float().cpu().numpy(), ob[n]) < BF16_TOL, n
+
+
 def test_chunkwise_flag_is_refused_where_there_is_no_kernel():
     import srwm_hip
     dev = _dev()
