@@ -1,0 +1,221 @@
+// Matrix-core building blocks of the chunkwise delta-rule kernels: LDS operand matrices, operand
+// fragments and the product of one group of 16 contraction indices, in two precisions.
+//
+// Index conventions (verified on gfx950): with lane = 16*lq + ln,
+//   A fragment  row ln of the left operand, contraction slots 4*lq + j (j = 0..3) of the group
+//   B fragment  column ln of the right operand, the same contraction slots
+//   accumulator f32x4 register r  <->  row 4*lq + r, column ln of the 16 x 16 result tile
+// so an accumulator tile is directly a B fragment over its 16 rows.
+//
+//   PrecF32   operands fp32: one group = four v_mfma_f32_16x16x4f32 (128 cycles per SIMD).
+//   PrecBf16  operands bf16: one group = one v_mfma_f32_16x16x16_bf16 (16 cycles).  Values that
+//             are not exactly representable in bf16 travel as hi + lo (hi = the upper 16 bits,
+//             lo = bf16 of the exact remainder, 16 significant bits together) and a product
+//             takes the passes hi*hi, hi*lo, lo*hi as needed; accumulation is fp32 either way.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fw {
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+struct PrecF32 {
+    static constexpr bool kBf = false;
+    static constexpr int kPad = 4;        // row padding of LDS matrices, in elements
+    static constexpr int kPlanes = 1;
+    typedef float elem;
+    // LDS matrix with rows of LD elements; SPLIT is ignored (fp32 holds everything)
+    template <int LD, bool SPLIT>
+    struct Mat {
+        float *p;
+        static constexpr int kLd = LD;
+        __host__ __device__ static constexpr int bytes(int rows) { return rows * LD * 4; }
+        __device__ explicit Mat(void *base, int /*rows*/) : p(static_cast<float *>(base)) {}
+    };
+    struct A { float4 v; };
+    struct B { f32x4 v; };
+
+    // left-operand fragment: m[row][k .. k+3]          (k already includes 4*lq)
+    template <int LD, bool SP>
+    __device__ static __forceinline__ A lda(const Mat<LD, SP> &m, int row, int k) {
+        return A{*reinterpret_cast<const float4 *>(m.p + row * LD + k)};
+    }
+    // left-operand fragment of the transposed matrix: m[k .. k+3][col]
+    template <int LD, bool SP>
+    __device__ static __forceinline__ A lda_t(const Mat<LD, SP> &m, int k, int col) {
+        const float *q = m.p + k * LD + col;
+        return A{make_float4(q[0], q[LD], q[2 * LD], q[3 * LD])};
+    }
+    // right-operand fragment from a matrix stored [n][k]: m[n][k .. k+3]
+    template <int LD, bool SP>
+    __device__ static __forceinline__ B ldb(const Mat<LD, SP> &m, int n, int k) {
+        const float4 v = *reinterpret_cast<const float4 *>(m.p + n * LD + k);
+        return B{f32x4{v.x, v.y, v.z, v.w}};
+    }
+    // right-operand fragment from a matrix stored [k][n]: m[k .. k+3][n]
+    template <int LD, bool SP>
+    __device__ static __forceinline__ B ldb_t(const Mat<LD, SP> &m, int k, int n) {
+        const float *q = m.p + k * LD + n;
+        return B{f32x4{q[0], q[LD], q[2 * LD], q[3 * LD]}};
+    }
+    __device__ static __forceinline__ B accb(const f32x4 &x) { return B{x}; }
+    template <bool SA, bool SB>
+    __device__ static __forceinline__ f32x4 mma(const A &a, const B &b, f32x4 acc) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v.x, b.v[0], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v.y, b.v[1], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v.z, b.v[2], acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v.w, b.v[3], acc, 0, 0, 0);
+        return acc;
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ void st(const Mat<LD, SP> &m, int row, int col, float v) {
+        m.p[row * LD + col] = v;
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ void st4(const Mat<LD, SP> &m, int row, int col, const float4 &v) {
+        *reinterpret_cast<float4 *>(m.p + row * LD + col) = v;
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ float ld(const Mat<LD, SP> &m, int row, int col) {
+        return m.p[row * LD + col];
+    }
+    // four consecutive input elements as they come from global memory
+    typedef float4 Raw4;
+    __device__ static __forceinline__ Raw4 ld_raw(const float *g) { return *reinterpret_cast<const float4 *>(g); }
+    __device__ static __forceinline__ Raw4 keep_raw(const Raw4 &v, bool keep) {
+        const float m = keep ? 1.f : 0.f;
+        return make_float4(v.x * m, v.y * m, v.z * m, v.w * m);
+    }
+    __device__ static __forceinline__ float4 raw_f32(const Raw4 &v) { return v; }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ void st_raw(const Mat<LD, SP> &m, int row, int col, const Raw4 &v) {
+        *reinterpret_cast<float4 *>(m.p + row * LD + col) = v;
+    }
+};
+
+__device__ __forceinline__ uint32_t bf_hi_bits(float x) { return __float_as_uint(x) >> 16; }
+__device__ __forceinline__ float bf_hi_part(float x) { return __uint_as_float(__float_as_uint(x) & 0xFFFF0000u); }
+// upper halves of two words packed into one: (a >> 16) | (b & 0xFFFF0000)
+__device__ __forceinline__ uint32_t pack_hi16(uint32_t a, uint32_t b) {
+    return __builtin_amdgcn_perm(b, a, 0x07060302u);
+}
+
+struct PrecBf16 {
+    static constexpr bool kBf = true;
+    static constexpr int kPad = 4;        // rows of (LD * 2) bytes: LD = 4 (mod 64) keeps 8-byte reads conflict free
+    typedef uint16_t elem;
+    // Two planes (hi, lo) of LD bf16 per row; matrices whose values are exact in bf16 (SPLIT
+    // false) have no lo plane.
+    template <int LD, bool SPLIT>
+    struct Mat {
+        uint16_t *hi, *lo;
+        static constexpr int kLd = LD;
+        static constexpr bool kSplit = SPLIT;
+        __host__ __device__ static constexpr int bytes(int rows) { return rows * LD * 2 * (SPLIT ? 2 : 1); }
+        __device__ explicit Mat(void *base, int rows)
+            : hi(static_cast<uint16_t *>(base)), lo(static_cast<uint16_t *>(base) + (SPLIT ? rows * LD : 0)) {}
+    };
+    struct A { s16x4 hi, lo; };
+    struct B { s16x4 hi, lo; };
+
+    __device__ static __forceinline__ s16x4 rd4(const uint16_t *p) {
+        const uint2 u = *reinterpret_cast<const uint2 *>(p);
+        return __builtin_bit_cast(s16x4, u);
+    }
+    __device__ static __forceinline__ s16x4 rd4s(const uint16_t *q, int stride) {
+        const uint32_t a = q[0], b = q[stride], c = q[2 * stride], d = q[3 * stride];
+        const uint2 u = make_uint2(a | (b << 16), c | (d << 16));
+        return __builtin_bit_cast(s16x4, u);
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ A lda(const Mat<LD, SP> &m, int row, int k) {
+        A a;
+        a.hi = rd4(m.hi + row * LD + k);
+        a.lo = SP ? rd4(m.lo + row * LD + k) : a.hi;
+        return a;
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ A lda_t(const Mat<LD, SP> &m, int k, int col) {
+        A a;
+        a.hi = rd4s(m.hi + k * LD + col, LD);
+        a.lo = SP ? rd4s(m.lo + k * LD + col, LD) : a.hi;
+        return a;
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ B ldb(const Mat<LD, SP> &m, int n, int k) {
+        B b;
+        b.hi = rd4(m.hi + n * LD + k);
+        b.lo = SP ? rd4(m.lo + n * LD + k) : b.hi;
+        return b;
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ B ldb_t(const Mat<LD, SP> &m, int k, int n) {
+        B b;
+        b.hi = rd4s(m.hi + k * LD + n, LD);
+        b.lo = SP ? rd4s(m.lo + k * LD + n, LD) : b.hi;
+        return b;
+    }
+    // accumulator tile -> right operand: hi = upper 16 bits, lo = upper 16 bits of the remainder
+    __device__ static __forceinline__ B accb(const f32x4 &x) {
+        uint32_t xb[4], lb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            xb[j] = __float_as_uint(x[j]);
+            lb[j] = __float_as_uint(x[j] - bf_hi_part(x[j]));
+        }
+        B b;
+        b.hi = __builtin_bit_cast(s16x4, make_uint2(pack_hi16(xb[0], xb[1]), pack_hi16(xb[2], xb[3])));
+        b.lo = __builtin_bit_cast(s16x4, make_uint2(pack_hi16(lb[0], lb[1]), pack_hi16(lb[2], lb[3])));
+        return b;
+    }
+    // SA / SB: the left / right operand carries a lo part that matters
+    template <bool SA, bool SB>
+    __device__ static __forceinline__ f32x4 mma(const A &a, const B &b, f32x4 acc) {
+        if constexpr (SA) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.lo, b.hi, acc, 0, 0, 0);
+        if constexpr (SB) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.hi, b.lo, acc, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.hi, b.hi, acc, 0, 0, 0);
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ void st(const Mat<LD, SP> &m, int row, int col, float v) {
+        m.hi[row * LD + col] = (uint16_t)bf_hi_bits(v);
+        if constexpr (SP) m.lo[row * LD + col] = (uint16_t)bf_hi_bits(v - bf_hi_part(v));
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ void st4(const Mat<LD, SP> &m, int row, int col, const float4 &v) {
+        const uint32_t a = __float_as_uint(v.x), b = __float_as_uint(v.y), c = __float_as_uint(v.z),
+                       d = __float_as_uint(v.w);
+        *reinterpret_cast<uint2 *>(m.hi + row * LD + col) = make_uint2(pack_hi16(a, b), pack_hi16(c, d));
+        if constexpr (SP) {
+            const uint32_t la = __float_as_uint(v.x - bf_hi_part(v.x)), lb = __float_as_uint(v.y - bf_hi_part(v.y)),
+                           lc = __float_as_uint(v.z - bf_hi_part(v.z)), ld_ = __float_as_uint(v.w - bf_hi_part(v.w));
+            *reinterpret_cast<uint2 *>(m.lo + row * LD + col) = make_uint2(pack_hi16(la, lb), pack_hi16(lc, ld_));
+        }
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ float ld(const Mat<LD, SP> &m, int row, int col) {
+        float v = __uint_as_float((uint32_t)m.hi[row * LD + col] << 16);
+        if constexpr (SP) v += __uint_as_float((uint32_t)m.lo[row * LD + col] << 16);
+        return v;
+    }
+    typedef uint2 Raw4;   // four bf16 bit patterns
+    __device__ static __forceinline__ Raw4 ld_raw(const uint16_t *g) { return *reinterpret_cast<const uint2 *>(g); }
+    __device__ static __forceinline__ Raw4 keep_raw(const Raw4 &v, bool keep) {
+        const uint32_t m = keep ? 0xFFFFFFFFu : 0u;
+        return make_uint2(v.x & m, v.y & m);
+    }
+    __device__ static __forceinline__ float4 raw_f32(const Raw4 &v) {
+        return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xFFFF0000u),
+                           __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xFFFF0000u));
+    }
+    // exact matrices only: the bit patterns go to the hi plane as they are
+    template <int LD, bool SP>
+    __device__ static __forceinline__ void st_raw(const Mat<LD, SP> &m, int row, int col, const Raw4 &v) {
+        static_assert(!SP, "raw bf16 rows have no lo part");
+        *reinterpret_cast<uint2 *>(m.hi + row * LD + col) = v;
+    }
+};
+
+}  // namespace fw

@@ -22,6 +22,7 @@
 //
 // The backward of a chunkwise forward is the sequential reverse sweep of delta_tiled.hip (it
 // only needs v_old and v_insert, which this kernel emits).
+#include "chunk_mma.h"
 #include "common.h"
 #include "xlane.h"
 
@@ -29,42 +30,26 @@ namespace fw {
 
 namespace {
 
-typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint16_t bf16_t;
 
 constexpr int kC = 64;        // chunk length
 constexpr int kCB = kC / 16;  // 16-row blocks per chunk
 constexpr int kMC = 64;       // memory columns per workgroup (16 per wave)
-constexpr int kPad = 4;       // row padding (floats) of the LDS matrices
 constexpr int kThreads = 256;
 
-__device__ __forceinline__ float bf2f(uint32_t h) { return __uint_as_float(h << 16); }
 __device__ __forceinline__ uint32_t f2bf(float f) {
     const uint32_t u = __float_as_uint(f);
     return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
 }
-__device__ __forceinline__ float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
-__device__ __forceinline__ float4 ld4(const bf16_t *p) {
-    const uint2 u = *reinterpret_cast<const uint2 *>(p);
-    return make_float4(bf2f(u.x & 0xFFFFu), bf2f(u.x >> 16), bf2f(u.y & 0xFFFFu), bf2f(u.y >> 16));
-}
 __device__ __forceinline__ float ld1(const float *p) { return *p; }
-__device__ __forceinline__ float ld1(const bf16_t *p) { return bf2f(*p); }
+__device__ __forceinline__ float ld1(const bf16_t *p) { return __uint_as_float((uint32_t)*p << 16); }
 __device__ __forceinline__ void st1(float *p, float v) { *p = v; }
 __device__ __forceinline__ void st1(bf16_t *p, float v) { *p = (bf16_t)f2bf(v); }
 
-// acc += sum_j a[j] * b[j] as four MFMAs (k-slot of lane l in the j-th one: 4*(l/16)+j)
-__device__ __forceinline__ f32x4 mma4(const float4 &a, const f32x4 &b, f32x4 acc) {
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.x, b[0], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.y, b[1], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.z, b[2], acc, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.w, b[3], acc, 0, 0, 0);
-    return acc;
-}
-__device__ __forceinline__ f32x4 mma4(const float4 &a, const float4 &b, f32x4 acc) {
-    const f32x4 bv = {b.x, b.y, b.z, b.w};
-    return mma4(a, bv, acc);
-}
+// fp32 inputs multiply in fp32; bf16 inputs multiply in bf16 (hi + lo where a value is not
+// exactly a bf16 number) -- see chunk_mma.h
+template <class TI> struct PrecOf { typedef PrecF32 type; };
+template <> struct PrecOf<bf16_t> { typedef PrecBf16 type; };
 
 template <class TI>
 struct ChunkFwdP {
@@ -75,22 +60,41 @@ struct ChunkFwdP {
     int N, H, L;
 };
 
+// LDS carve-up shared by the kernel and the launcher
+template <class TI, int D>
+struct FwdLds {
+    typedef typename PrecOf<TI>::type X;
+    static constexpr int LDK = D + X::kPad, LDA = kC + X::kPad, LDD = 16 + X::kPad, LDV = kMC + 4;
+    typedef typename X::template Mat<LDK, false> MatK;   // K, Q: the inputs themselves
+    typedef typename X::template Mat<LDA, true> MatA;    // A, B: computed
+    typedef typename X::template Mat<LDD, true> MatD;    // inverses of the diagonal blocks
+    static constexpr int oK = 0;
+    static constexpr int oQ = oK + MatK::bytes(kC);
+    static constexpr int oA = oQ + MatK::bytes(kC);
+    static constexpr int oB = oA + MatA::bytes(kC);
+    static constexpr int oD = oB + MatA::bytes(kC);
+    static constexpr int oV = oD + MatD::bytes(kC);            // fp32 [C][LDV]
+    static constexpr int oAd = oV + kC * LDV * 4;              // fp32 [C][LDD]: diagonal blocks of A
+    static constexpr int oBt = oAd + kC * LDD * 4;             // fp32 [C]: beta
+    static constexpr int kBytes = oBt + kC * 4;
+    static_assert(MatK::bytes(kC) % 16 == 0 && MatA::bytes(kC) % 16 == 0 && MatD::bytes(kC) % 16 == 0, "alignment");
+};
+
 template <class TI, int D, int MS>
 __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI> p) {
+    typedef FwdLds<TI, D> Lds;
+    typedef typename Lds::X X;
     constexpr int EB = D / 16;          // 16-row blocks of the memory
-    constexpr int LDK = D + kPad;       // row stride of Ks / Qs
-    constexpr int LDV = kMC + kPad;
-    constexpr int LDA = kC + kPad;
-    constexpr int LDD = 16 + kPad;
+    constexpr int LDV = Lds::LDV, LDD = Lds::LDD;
     static_assert(MS * kMC == D, "column split");
-    extern __shared__ __attribute__((aligned(16))) float smem[];
-    float *Ks = smem;                   // [C][LDK]
-    float *Qs = Ks + kC * LDK;          // [C][LDK]
-    float *Vs = Qs + kC * LDK;          // [C][LDV]
-    float *As = Vs + kC * LDV;          // [C][LDA]  strict lower triangle of K K^T
-    float *Bs = As + kC * LDA;          // [C][LDA]  lower triangle (with diagonal) of Q K^T
-    float *Di = Bs + kC * LDA;          // [4][16][LDD]  inverses of the diagonal blocks of I + L
-    float *bts = Di + kCB * 16 * LDD;   // [C] beta
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const typename Lds::MatK Ks(smem + Lds::oK, kC), Qs(smem + Lds::oQ, kC);
+    const typename Lds::MatA As(smem + Lds::oA, kC);   // strict lower triangle of K K^T
+    const typename Lds::MatA Bs(smem + Lds::oB, kC);   // lower triangle (with diagonal) of Q K^T
+    const typename Lds::MatD Di(smem + Lds::oD, kC);   // [4][16] inverses of the diagonal blocks of I + L
+    float *Vs = reinterpret_cast<float *>(smem + Lds::oV);
+    float *Ad = reinterpret_cast<float *>(smem + Lds::oAd);
+    float *bts = reinterpret_cast<float *>(smem + Lds::oBt);
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int ln = lane & 15, lq = lane >> 4;        // accumulator layout: column ln, rows 4*lq + r
@@ -112,10 +116,10 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
         for (int r = 0; r < 4; ++r) s[eb][r] = Wg[(eb * 16 + 4 * lq + r) * D + ln];
 
     // The chunk inputs are fetched one chunk ahead into registers (all loads in flight at
-    // once) and written to LDS as fp32 after the previous chunk is done with it.
-    constexpr int NKQ = kC * (D / 4) / kThreads;    // float4s of K (and of Q) per thread
-    constexpr int NV = kC * (kMC / 4) / kThreads;   // float4s of V per thread
-    float4 kreg[NKQ], qreg[NKQ], vreg[NV];
+    // once) and written to LDS after the previous chunk is done with it.
+    constexpr int NKQ = kC * (D / 4) / kThreads;    // 4-element groups of K (and of Q) per thread
+    constexpr int NV = kC * (kMC / 4) / kThreads;   // 4-element groups of V per thread
+    typename X::Raw4 kreg[NKQ], qreg[NKQ], vreg[NV];
     float breg = 0.f;
     auto prefetch = [&](int ch) {   // rows past the end are clamped here and zeroed in commit()
         const int t0 = ch * kC;
@@ -123,32 +127,31 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
         for (int i = 0; i < NKQ; ++i) {
             const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
             const int t = min(t0 + row, p.L - 1);
-            kreg[i] = ld4(kb + (int64_t)t * p.ks.l + col);
-            qreg[i] = ld4(qb + (int64_t)t * p.qs.l + col);
+            kreg[i] = X::ld_raw(kb + (int64_t)t * p.ks.l + col);
+            qreg[i] = X::ld_raw(qb + (int64_t)t * p.qs.l + col);
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int f = tid + i * kThreads, row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
-            vreg[i] = ld4(vb + (int64_t)min(t0 + row, p.L - 1) * p.vs.l + col);
+            vreg[i] = X::ld_raw(vb + (int64_t)min(t0 + row, p.L - 1) * p.vs.l + col);
         }
         breg = ld1(bb + (int64_t)min(t0 + (tid % kC), p.L - 1) * p.bs.l);
     };
-    auto masked = [](const float4 &v, float m) { return make_float4(v.x * m, v.y * m, v.z * m, v.w * m); };
     auto commit = [&](int ch) {
         const int t0 = ch * kC;
         const bool full = t0 + kC <= p.L;   // only the last chunk can be ragged
 #pragma unroll
         for (int i = 0; i < NKQ; ++i) {
             const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
-            const float m = (full || t0 + row < p.L) ? 1.f : 0.f;
-            *reinterpret_cast<float4 *>(Ks + row * LDK + col) = masked(kreg[i], m);
-            *reinterpret_cast<float4 *>(Qs + row * LDK + col) = masked(qreg[i], m);
+            const bool keep = full || t0 + row < p.L;
+            X::st_raw(Ks, row, col, X::keep_raw(kreg[i], keep));
+            X::st_raw(Qs, row, col, X::keep_raw(qreg[i], keep));
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int f = tid + i * kThreads, row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
-            const float m = (full || t0 + row < p.L) ? 1.f : 0.f;
-            *reinterpret_cast<float4 *>(Vs + row * LDV + col) = masked(vreg[i], m);
+            const bool keep = full || t0 + row < p.L;
+            *reinterpret_cast<float4 *>(Vs + row * LDV + col) = X::raw_f32(X::keep_raw(vreg[i], keep));
         }
         if (tid < kC) bts[tid] = (t0 + tid < p.L) ? breg : 0.f;
     };
@@ -166,20 +169,20 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
             const int which = tix / 10, tri = tix % 10;     // tri -> (ci, cj), cj <= ci
             const int ci = tri < 1 ? 0 : tri < 3 ? 1 : tri < 6 ? 2 : 3;
             const int cj = tri - (ci * (ci + 1)) / 2;
-            const float *X = which ? Qs : Ks;
+            const typename Lds::MatK &Xm = which ? Qs : Ks;
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int eb = 0; eb < EB; ++eb) {
-                const float4 a = *reinterpret_cast<const float4 *>(X + (ci * 16 + ln) * LDK + eb * 16 + 4 * lq);
-                const float4 b = *reinterpret_cast<const float4 *>(Ks + (cj * 16 + ln) * LDK + eb * 16 + 4 * lq);
-                acc = mma4(a, b, acc);
-            }
-            float *T = which ? Bs : As;
+            for (int eb = 0; eb < EB; ++eb)
+                acc = X::template mma<false, false>(X::lda(Xm, ci * 16 + ln, eb * 16 + 4 * lq),
+                                                    X::ldb(Ks, cj * 16 + ln, eb * 16 + 4 * lq), acc);
+            const typename Lds::MatA &T = which ? Bs : As;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = ci * 16 + 4 * lq + r, col = cj * 16 + ln;
                 const bool keep = which ? col <= row : col < row;
-                T[row * LDA + col] = keep ? acc[r] : 0.f;
+                const float v = keep ? acc[r] : 0.f;
+                X::st(T, row, col, v);
+                if (!which && ci == cj) Ad[row * LDD + ln] = v;
             }
         }
         __syncthreads();
@@ -188,63 +191,63 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
         //      column ln of X, x_i = [i == ln] - sum_{j<i} beta_i A_ij x_j
         {
             float x[16];
-            const float *Ad = As + (wave * 16) * LDA + wave * 16;
+            const float *ad = Ad + (wave * 16) * LDD;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 float acc = (i == ln) ? 1.f : 0.f;
                 const float bi = bts[wave * 16 + i];
 #pragma unroll
-                for (int j = 0; j < i; ++j) acc = fmaf(-bi * Ad[i * LDA + j], x[j], acc);
+                for (int j = 0; j < i; ++j) acc = fmaf(-bi * ad[i * LDD + j], x[j], acc);
                 x[i] = acc;
             }
             // lanes 16..63 hold copies of columns 0..15: everybody stores, no branch
 #pragma unroll
-            for (int i = 0; i < 16; ++i) Di[(wave * 16 + i) * LDD + ln] = x[i];
+            for (int i = 0; i < 16; ++i) X::st(Di, wave * 16 + i, ln, x[i]);
         }
 
         // ---- P = K S and Q S for this wave's 16 columns: independent of the inversion above
         //      (matrix-core work that can overlap its vector-ALU chain)
         f32x4 pt[kCB], ot[kCB], u[kCB];
+        {
+            typename X::B sb[EB];
 #pragma unroll
-        for (int cb = 0; cb < kCB; ++cb) {
-            pt[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
-            ot[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+            for (int eb = 0; eb < EB; ++eb) sb[eb] = X::accb(s[eb]);
 #pragma unroll
-            for (int eb = 0; eb < EB; ++eb) {
-                const float4 ka = *reinterpret_cast<const float4 *>(Ks + (cb * 16 + ln) * LDK + eb * 16 + 4 * lq);
-                const float4 qa = *reinterpret_cast<const float4 *>(Qs + (cb * 16 + ln) * LDK + eb * 16 + 4 * lq);
-                pt[cb] = mma4(ka, s[eb], pt[cb]);   // P = K S
-                ot[cb] = mma4(qa, s[eb], ot[cb]);   // Q S
+            for (int cb = 0; cb < kCB; ++cb) {
+                pt[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+                ot[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int eb = 0; eb < EB; ++eb) {
+                    pt[cb] = X::template mma<false, true>(X::lda(Ks, cb * 16 + ln, eb * 16 + 4 * lq), sb[eb], pt[cb]);
+                    ot[cb] = X::template mma<false, true>(X::lda(Qs, cb * 16 + ln, eb * 16 + 4 * lq), sb[eb], ot[cb]);
+                }
             }
         }
         __syncthreads();   // the four inverses are visible
 
         // ---- everything below is per wave (its 16 columns), no synchronisation
         // block forward substitution, one 16-row block at a time
+        typename X::B ub[kCB];
 #pragma unroll
         for (int a = 0; a < kCB; ++a) {
             f32x4 y = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int b = 0; b < a; ++b) {
-                const float4 aa = *reinterpret_cast<const float4 *>(As + (a * 16 + ln) * LDA + b * 16 + 4 * lq);
-                y = mma4(aa, u[b], y);
-            }
+            for (int b = 0; b < a; ++b)
+                y = X::template mma<true, true>(X::lda(As, a * 16 + ln, b * 16 + 4 * lq), ub[b], y);
             f32x4 rhs;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = a * 16 + 4 * lq + r;
                 rhs[r] = bts[row] * (Vs[row * LDV + cw + ln] - pt[a][r] - y[r]);
             }
-            const float4 da = *reinterpret_cast<const float4 *>(Di + (a * 16 + ln) * LDD + 4 * lq);
-            u[a] = mma4(da, rhs, f32x4{0.f, 0.f, 0.f, 0.f});
-            const float4 ad = *reinterpret_cast<const float4 *>(As + (a * 16 + ln) * LDA + a * 16 + 4 * lq);
-            y = mma4(ad, u[a], y);                  // + strict_lower(A_aa) U_a
+            u[a] = X::template mma<true, true>(X::lda(Di, a * 16 + ln, 4 * lq), X::accb(rhs),
+                                               f32x4{0.f, 0.f, 0.f, 0.f});
+            ub[a] = X::accb(u[a]);
+            y = X::template mma<true, true>(X::lda(As, a * 16 + ln, a * 16 + 4 * lq), ub[a], y);   // + strict_lower(A_aa) U_a
             // out = Q S + tril(B) U
 #pragma unroll
-            for (int b = 0; b <= a; ++b) {
-                const float4 ba = *reinterpret_cast<const float4 *>(Bs + (a * 16 + ln) * LDA + b * 16 + 4 * lq);
-                ot[a] = mma4(ba, u[b], ot[a]);
-            }
+            for (int b = 0; b <= a; ++b)
+                ot[a] = X::template mma<true, true>(X::lda(Bs, a * 16 + ln, b * 16 + 4 * lq), ub[b], ot[a]);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int t = t0 + a * 16 + 4 * lq + r;
@@ -260,14 +263,8 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
 #pragma unroll
         for (int eb = 0; eb < EB; ++eb)
 #pragma unroll
-            for (int cb = 0; cb < kCB; ++cb) {
-                float4 kt;
-                kt.x = Ks[(cb * 16 + 4 * lq + 0) * LDK + eb * 16 + ln];
-                kt.y = Ks[(cb * 16 + 4 * lq + 1) * LDK + eb * 16 + ln];
-                kt.z = Ks[(cb * 16 + 4 * lq + 2) * LDK + eb * 16 + ln];
-                kt.w = Ks[(cb * 16 + 4 * lq + 3) * LDK + eb * 16 + ln];
-                s[eb] = mma4(kt, u[cb], s[eb]);
-            }
+            for (int cb = 0; cb < kCB; ++cb)
+                s[eb] = X::template mma<false, true>(X::lda_t(Ks, cb * 16 + 4 * lq, eb * 16 + ln), ub[cb], s[eb]);
         __syncthreads();   // every wave is done with Ks, Qs, Vs, As, Bs
         if (ch + 1 < nchunks) {
             commit(ch + 1);
@@ -281,15 +278,9 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
         for (int r = 0; r < 4; ++r) Wg[(eb * 16 + 4 * lq + r) * D + ln] = s[eb][r];
 }
 
-template <int D>
-constexpr size_t chunk_lds_bytes() {
-    return sizeof(float) * (2 * kC * (D + kPad) + kC * (kMC + kPad) + 2 * kC * (kC + kPad) +
-                            kCB * 16 * (16 + kPad) + kC);
-}
-
 template <class TI, int D, int MS>
 int launch_chunk(const ChunkFwdP<TI> &p, hipStream_t s) {
-    constexpr size_t lds = chunk_lds_bytes<D>();
+    constexpr size_t lds = FwdLds<TI, D>::kBytes;
     hipError_t err = hipFuncSetAttribute((const void *)delta_fwd_chunk_kernel<TI, D, MS>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return (int)err;
