@@ -108,10 +108,10 @@ def delta_setup(N, H, L, E, dev, io=None):
     t = dict(q=q.to(dev, io), k=k.to(dev, io), v=v.to(dev, io), beta=beta.to(dev, io), go=go.to(dev, io))
     t["W"] = torch.empty(N, H, E, M, device=dev)
     bigm = lambda dt=torch.float32: torch.empty(N, H, L, M, device=dev, dtype=dt)
-    bige = lambda: torch.empty(N, H, L, E, device=dev, dtype=io)
+    bige = lambda: torch.empty(N, H, L, E, device=dev)
     t["vold"], t["vins"], t["out"] = bigm(), bigm(), bigm(io)
-    t["gq"], t["gk"], t["gv"] = bige(), bige(), bigm(io)
-    t["gb"] = torch.empty(N, H, L, 1, device=dev, dtype=io)
+    t["gq"], t["gk"], t["gv"] = bige(), bige(), bigm()       # the library's gradients are fp32
+    t["gb"] = torch.empty(N, H, L, 1, device=dev)
     return t
 
 
@@ -125,7 +125,7 @@ def delta_step(t, ev=None):
     if ev:
         ev[1].record()
     srwm_hip.fast_weight_backward(t["q"], t["k"], t["v"], t["beta"], t["vold"], t["vins"], t["go"],
-                                  t["W"], t["gq"], t["gk"], t["gv"], t["gb"])
+                                  t["W"], t["gq"], t["gk"], t["gv"], t["gb"], flags=t.get("bwd_flags", 0))
     if ev:
         ev[2].record()
 
@@ -137,11 +137,11 @@ def algorithmic_bytes(op, N, H, L, E):
         S = E * (3 * E + 4)
         return 3 * S * 4 * hs, 6 * S * 4 * hs, (15 * E + 16) * 4 * hs + 4 * S * 4 * N * H
     S = E * E
-    # per (sequence, step): q,k,v,beta in (fwd and bwd), out + grad_out, 3 E-wide grads in the I/O
-    # type; v_old, v_insert written and read back in fp32
+    # per (sequence, step): q,k,v,beta in (fwd and bwd), out + grad_out in the I/O type; v_old,
+    # v_insert written and read back, and the 3 E-wide gradients + grad_beta written, in fp32
     b = 2 if op == "delta_bf16" else 4
-    io_elems = 2 * (3 * E + 1) + 2 * E + 3 * E + 1
-    return 2 * S * 4 * hs, 4 * S * 4 * hs, (io_elems * b + 4 * E * 4) * hs + 3 * S * 4 * N * H
+    io_elems = 2 * (3 * E + 1) + 2 * E
+    return 2 * S * 4 * hs, 4 * S * 4 * hs, (io_elems * b + (4 * E + 3 * E + 1) * 4) * hs + 3 * S * 4 * N * H
 
 
 def cpu_baseline(op, N, H, L, E, budget_s=20.0):
@@ -246,6 +246,7 @@ def main():
         t = delta_setup(N, H, L, E, dev, torch.bfloat16 if op == "delta_bf16" else torch.float32)
         if a.workload.endswith("_chunk"):
             t["fwd_flags"] = srwm_hip.FLAG_CHUNKWISE
+            t["bwd_flags"] = srwm_hip.FLAG_CHUNKWISE
 
     for _ in range(a.warmup):
         step(t)

@@ -47,8 +47,10 @@ extern "C" {
                                      it, :1213-1229); equal to ZERO when the buffers arrive zeroed. */
 #define SRWM_GRAD_STATE_MASK 3u
 #define SRWM_FLAG_GENERIC 16u     /* force the any-size LDS-resident kernel (testing / comparison) */
-#define SRWM_FLAG_CHUNKWISE 32u   /* delta forward only: chunkwise (chunk = 64) MFMA kernel instead of the
-                                     step-by-step one; E == M in {64, 128}, else SRWM_ENOKERNEL */
+#define SRWM_FLAG_CHUNKWISE 32u   /* delta rule only: chunkwise matrix-core kernels instead of the step-by-step
+                                     ones (forward: chunks of 64 steps; backward: a sweep over memory columns and
+                                     one over memory rows); E == M in {64, 128}, else SRWM_ENOKERNEL.  Forward and
+                                     backward may be mixed freely: both forms emit / consume the same v_old, v_insert */
 
 /*
  * SRWM forward.  Replaces self_ref_forward(), supervised_learning/self_ref_v0/
@@ -128,11 +130,12 @@ SRWM_API int delta_backward_f32(const float *Q, const int64_t q_strides[3],
  * Delta rule with bf16 inputs/outputs and fp32 memory.  No counterpart in the reference
  * (its kernels are float-only, fast_weight_cuda.cu:12-14); same recurrence as
  * delta_forward_f32 / delta_backward_f32 with
- *   Q, K, V, beta, out, grad_out, gV       bf16 (raw 16-bit patterns)
- *   W, gW, v_old, v_insert, gQ, gK, gbeta  fp32 (gQ, gK, gbeta are sums over the value axis and
- *                                          may be accumulated by several workgroups; the caller
- *                                          rounds them to bf16 if it wants them in that type)
- * All arithmetic is fp32; inputs are widened on load, outputs rounded to nearest even.
+ *   Q, K, V, beta, out, grad_out               bf16 (raw 16-bit patterns)
+ *   W, gW, v_old, v_insert, gQ, gK, gV, gbeta  fp32 (every gradient comes back in fp32: gQ, gK,
+ *                                              gbeta may be accumulated by several workgroups
+ *                                              and gV is re-read by the chunkwise backward;
+ *                                              the caller rounds them if it wants bf16)
+ * The memory and all accumulation are fp32; `out` is rounded to nearest even.
  */
 SRWM_API int delta_forward_bf16(const uint16_t *Q, const int64_t q_strides[3],
                        const uint16_t *K, const int64_t k_strides[3],
@@ -148,7 +151,7 @@ SRWM_API int delta_backward_bf16(const uint16_t *Q, const int64_t q_strides[3],
                         const float *v_old, const float *v_insert,
                         const uint16_t *grad_out, const int64_t grad_out_strides[3],
                         float *W,
-                        float *gQ, float *gK, uint16_t *gV, float *gbeta, float *gW,
+                        float *gQ, float *gK, float *gV, float *gbeta, float *gW,
                         int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
 /* Largest E the SRWM entry points accept (forward / backward), and the largest

@@ -150,7 +150,8 @@ int delta_backward_f32(const float *Q, const int64_t qs[3], const float *K, cons
         return SRWM_EINVAL;
     const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u ||
-        (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)))
+        (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE | SRWM_GRAD_STATE_MASK)) ||
+        (flags & (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE)) == (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE))
         return SRWM_EINVAL;
     if (!gW && mode != SRWM_GRAD_STATE_ZERO) return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
@@ -160,6 +161,10 @@ int delta_backward_f32(const float *Q, const int64_t qs[3], const float *K, cons
                      {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, grad_out,
                      {gs[0], gs[1], gs[2]}, W, gQ, gK, gV, gbeta, gW, N, H, L, E, M, mode};
     hipStream_t s = (hipStream_t)stream;
+    if (flags & SRWM_FLAG_CHUNKWISE) {
+        const int r = launch_delta_bwd_chunk(p, s);
+        return r >= 0 ? r : SRWM_ENOKERNEL;
+    }
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_delta_bwd_tiled(p, s);
         if (r >= 0) return r;
@@ -190,13 +195,14 @@ int delta_backward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *
                         const uint16_t *V, const int64_t vs[3], const uint16_t *beta,
                         const int64_t bs[3], const float *v_old, const float *v_insert,
                         const uint16_t *grad_out, const int64_t gs[3], float *W, float *gQ,
-                        float *gK, uint16_t *gV, float *gbeta, float *gW, int N, int H, int L,
+                        float *gK, float *gV, float *gbeta, float *gW, int N, int H, int L,
                         int E, int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !grad_out || !W || !gQ || !gK || !gV ||
         !gbeta || !qs || !ks || !vs || !bs || !gs)
         return SRWM_EINVAL;
     const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u || (flags & ~SRWM_GRAD_STATE_MASK))
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u ||
+        (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_GRAD_STATE_MASK)))
         return SRWM_EINVAL;
     if (!gW && mode != SRWM_GRAD_STATE_ZERO) return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
@@ -205,7 +211,8 @@ int delta_backward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *
     DeltaBwdParamsBf16 p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
                          {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, grad_out,
                          {gs[0], gs[1], gs[2]}, W, gQ, gK, gV, gbeta, gW, N, H, L, E, M, mode};
-    const int r = launch_delta_bwd_tiled_bf16(p, (hipStream_t)stream);
+    const int r = (flags & SRWM_FLAG_CHUNKWISE) ? launch_delta_bwd_chunk_bf16(p, (hipStream_t)stream)
+                                                : launch_delta_bwd_tiled_bf16(p, (hipStream_t)stream);
     return r >= 0 ? r : SRWM_ENOKERNEL;
 }
 

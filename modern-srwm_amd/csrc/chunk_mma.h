@@ -8,7 +8,7 @@
 // so an accumulator tile is directly a B fragment over its 16 rows.
 //
 //   PrecF32   operands fp32: one group = four v_mfma_f32_16x16x4f32 (128 cycles per SIMD).
-//   PrecBf16  operands bf16: one group = one v_mfma_f32_16x16x16_bf16 (16 cycles).  Values that
+//   PrecBf16  operands bf16: two groups = one v_mfma_f32_16x16x32_bf16 (16 cycles).  Values that
 //             are not exactly representable in bf16 travel as hi + lo (hi = the upper 16 bits,
 //             lo = bf16 of the exact remainder, 16 significant bits together) and a product
 //             takes the passes hi*hi, hi*lo, lo*hi as needed; accumulation is fp32 either way.
@@ -21,6 +21,7 @@ namespace fw {
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 struct PrecF32 {
     static constexpr bool kBf = false;
@@ -62,6 +63,8 @@ struct PrecF32 {
         return B{f32x4{q[0], q[LD], q[2 * LD], q[3 * LD]}};
     }
     __device__ static __forceinline__ B accb(const f32x4 &x) { return B{x}; }
+    __device__ static __forceinline__ B accb_exact(const f32x4 &x) { return B{x}; }
+    __device__ static __forceinline__ B negb(const B &b) { return B{-b.v}; }
     template <bool SA, bool SB>
     __device__ static __forceinline__ f32x4 mma(const A &a, const B &b, f32x4 acc) {
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v.x, b.v[0], acc, 0, 0, 0);
@@ -69,6 +72,11 @@ struct PrecF32 {
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v.z, b.v[2], acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a.v.w, b.v[3], acc, 0, 0, 0);
         return acc;
+    }
+    // two groups of 16 contraction indices at once
+    template <bool SA, bool SB>
+    __device__ static __forceinline__ f32x4 mma2(const A &a0, const A &a1, const B &b0, const B &b1, f32x4 acc) {
+        return mma<SA, SB>(a1, b1, mma<SA, SB>(a0, b0, acc));
     }
     template <int LD, bool SP>
     __device__ static __forceinline__ void st(const Mat<LD, SP> &m, int row, int col, float v) {
@@ -121,14 +129,25 @@ struct PrecBf16 {
     struct A { s16x4 hi, lo; };
     struct B { s16x4 hi, lo; };
 
+    __device__ static __forceinline__ bf16x8 cat(const s16x4 &x, const s16x4 &y) {
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        const s16x8 v = __builtin_shufflevector(x, y, 0, 1, 2, 3, 4, 5, 6, 7);
+        return __builtin_bit_cast(bf16x8, v);
+    }
     __device__ static __forceinline__ s16x4 rd4(const uint16_t *p) {
         const uint2 u = *reinterpret_cast<const uint2 *>(p);
         return __builtin_bit_cast(s16x4, u);
     }
-    __device__ static __forceinline__ s16x4 rd4s(const uint16_t *q, int stride) {
-        const uint32_t a = q[0], b = q[stride], c = q[2 * stride], d = q[3 * stride];
-        const uint2 u = make_uint2(a | (b << 16), c | (d << 16));
-        return __builtin_bit_cast(s16x4, u);
+    // Transposed fragment: element j of the calling lane = base[(k + j) * LD + col0 + (lane % 16)],
+    // in ONE ds_read_b64_tr_b16.  In each group of 16 lanes that instruction hands lane L, element
+    // j, the (L % 4)-th 16-bit word of the 8 bytes addressed by lane 4*j + L/4 (verified on
+    // gfx950), so lane s points at row k + s/4, columns col0 + 4*(s % 4) .. +3.
+    template <int LD>
+    __device__ static __forceinline__ s16x4 rd4t(const uint16_t *base, int k, int col) {
+        const int l = threadIdx.x & 15;
+        const uint16_t *q = base + (k + (l >> 2)) * LD + (col - l) + 4 * (l & 3);
+        typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+        return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(q));
     }
     template <int LD, bool SP>
     __device__ static __forceinline__ A lda(const Mat<LD, SP> &m, int row, int k) {
@@ -140,8 +159,8 @@ struct PrecBf16 {
     template <int LD, bool SP>
     __device__ static __forceinline__ A lda_t(const Mat<LD, SP> &m, int k, int col) {
         A a;
-        a.hi = rd4s(m.hi + k * LD + col, LD);
-        a.lo = SP ? rd4s(m.lo + k * LD + col, LD) : a.hi;
+        a.hi = rd4t<LD>(m.hi, k, col);
+        a.lo = SP ? rd4t<LD>(m.lo, k, col) : a.hi;
         return a;
     }
     template <int LD, bool SP>
@@ -154,8 +173,8 @@ struct PrecBf16 {
     template <int LD, bool SP>
     __device__ static __forceinline__ B ldb_t(const Mat<LD, SP> &m, int k, int n) {
         B b;
-        b.hi = rd4s(m.hi + k * LD + n, LD);
-        b.lo = SP ? rd4s(m.lo + k * LD + n, LD) : b.hi;
+        b.hi = rd4t<LD>(m.hi, k, n);
+        b.lo = SP ? rd4t<LD>(m.lo, k, n) : b.hi;
         return b;
     }
     // accumulator tile -> right operand: hi = upper 16 bits, lo = upper 16 bits of the remainder
@@ -171,12 +190,42 @@ struct PrecBf16 {
         b.lo = __builtin_bit_cast(s16x4, make_uint2(pack_hi16(lb[0], lb[1]), pack_hi16(lb[2], lb[3])));
         return b;
     }
-    // SA / SB: the left / right operand carries a lo part that matters
+    // the same for values that are exactly bf16 numbers (no lo part)
+    __device__ static __forceinline__ B accb_exact(const f32x4 &x) {
+        B b;
+        b.hi = __builtin_bit_cast(s16x4, make_uint2(pack_hi16(__float_as_uint(x[0]), __float_as_uint(x[1])),
+                                                    pack_hi16(__float_as_uint(x[2]), __float_as_uint(x[3]))));
+        b.lo = b.hi;
+        return b;
+    }
+    __device__ static __forceinline__ B negb(const B &b) {
+        const uint2 h = __builtin_bit_cast(uint2, b.hi), l = __builtin_bit_cast(uint2, b.lo);
+        B r;
+        r.hi = __builtin_bit_cast(s16x4, make_uint2(h.x ^ 0x80008000u, h.y ^ 0x80008000u));
+        r.lo = __builtin_bit_cast(s16x4, make_uint2(l.x ^ 0x80008000u, l.y ^ 0x80008000u));
+        return r;
+    }
+    // SA / SB: the left / right operand carries a lo part that matters.
+    // A single group is issued as the 32-index instruction with its second half zero, so that every
+    // matrix instruction of these kernels is the same opcode: a 16-index MFMA that accumulates
+    // onto the result of a 32-index one (or the reverse) a few instructions later was observed
+    // to read the accumulator before it was written.
     template <bool SA, bool SB>
     __device__ static __forceinline__ f32x4 mma(const A &a, const B &b, f32x4 acc) {
-        if constexpr (SA) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.lo, b.hi, acc, 0, 0, 0);
-        if constexpr (SB) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.hi, b.lo, acc, 0, 0, 0);
-        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a.hi, b.hi, acc, 0, 0, 0);
+        const s16x4 z = {0, 0, 0, 0};
+        const bf16x8 ah = cat(a.hi, z), bh = cat(b.hi, z);
+        if constexpr (SA) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cat(a.lo, z), bh, acc, 0, 0, 0);
+        if constexpr (SB) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, cat(b.lo, z), acc, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, bh, acc, 0, 0, 0);
+    }
+    // two groups of 16 contraction indices in one v_mfma_f32_16x16x32_bf16 (same 16 cycles as the
+    // 16-index instruction): lane l supplies slots 4*(l/16) + j of the first group and of the second
+    template <bool SA, bool SB>
+    __device__ static __forceinline__ f32x4 mma2(const A &a0, const A &a1, const B &b0, const B &b1, f32x4 acc) {
+        const bf16x8 ah = cat(a0.hi, a1.hi), bh = cat(b0.hi, b1.hi);
+        if constexpr (SA) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cat(a0.lo, a1.lo), bh, acc, 0, 0, 0);
+        if constexpr (SB) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, cat(b0.lo, b1.lo), acc, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, bh, acc, 0, 0, 0);
     }
     template <int LD, bool SP>
     __device__ static __forceinline__ void st(const Mat<LD, SP> &m, int row, int col, float v) {
@@ -217,5 +266,46 @@ struct PrecBf16 {
         *reinterpret_cast<uint2 *>(m.hi + row * LD + col) = v;
     }
 };
+
+// Raw bits of one input element and their fp32 value: loads keep the bits, the conversion is
+// done where the value is used, so that a prefetch does not wait for its own loads.
+__device__ __forceinline__ uint32_t ld_bits(const float *p) { return __float_as_uint(*p); }
+__device__ __forceinline__ uint32_t ld_bits(const uint16_t *p) { return *p; }
+template <class TI>
+__device__ __forceinline__ float bits_f32(uint32_t b) {
+    if constexpr (sizeof(TI) == 2) return __uint_as_float(b << 16);
+    else return __uint_as_float(b);
+}
+
+// fp32 inputs multiply in fp32; bf16 inputs (16-bit patterns) multiply in bf16
+template <class TI> struct PrecOf { typedef PrecF32 type; };
+template <> struct PrecOf<uint16_t> { typedef PrecBf16 type; };
+
+__device__ __forceinline__ uint32_t f2bf_rne(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float ld_in(const float *p) { return *p; }
+__device__ __forceinline__ float ld_in(const uint16_t *p) { return __uint_as_float((uint32_t)*p << 16); }
+__device__ __forceinline__ void st_out(float *p, float v) { *p = v; }
+__device__ __forceinline__ void st_out(uint16_t *p, float v) { *p = (uint16_t)f2bf_rne(v); }
+
+// acc += sum over g in [lo, hi) of fa(g) * fb(g), g numbering groups of 16 contraction indices;
+// two groups per instruction where they pair up.  Meant to be inlined into unrolled code (lo
+// and hi compile-time constants there).
+template <class X, bool SA, bool SB, class FA, class FB>
+__device__ __forceinline__ f32x4 mma_range(int lo, int hi, FA fa, FB fb, f32x4 acc) {
+#pragma unroll
+    for (int g = lo; g + 1 < hi; g += 2)
+        acc = X::template mma2<SA, SB>(fa(g), fa(g + 1), fb(g), fb(g + 1), acc);
+    if ((hi - lo) & 1) acc = X::template mma<SA, SB>(fa(hi - 1), fb(hi - 1), acc);
+    return acc;
+}
+
+// tile number of the lower triangle of a block matrix -> (block row, block column)
+__device__ __forceinline__ void tri_index(int tri, int &ci, int &cj) {
+    ci = tri < 1 ? 0 : tri < 3 ? 1 : tri < 6 ? 2 : 3;
+    cj = tri - (ci * (ci + 1)) / 2;
+}
 
 }  // namespace fw

@@ -66,9 +66,7 @@ struct DeltaBwdParamsBf16 {
     const uint16_t *go;
     Strided3 gs;
     float *W;
-    float *gQ, *gK;
-    uint16_t *gV;
-    float *gbeta;
+    float *gQ, *gK, *gV, *gbeta;   // every gradient is fp32
     float *gW;
     int N, H, L, E, M;
     unsigned grad_state_mode;
@@ -108,6 +106,9 @@ int launch_delta_fwd_tiled_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s);
 int launch_delta_fwd_chunk(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_fwd_chunk_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s);
 int launch_delta_bwd_tiled_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s);
+// Chunkwise backward on the matrix cores (two sweeps), E == M in {64, 128}; -1 otherwise.
+int launch_delta_bwd_chunk(const DeltaBwdParams &p, hipStream_t s);
+int launch_delta_bwd_chunk_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s);
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // gfx950: 160 KB of LDS per CU / workgroup
 

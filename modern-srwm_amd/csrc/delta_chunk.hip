@@ -37,20 +37,6 @@ constexpr int kCB = kC / 16;  // 16-row blocks per chunk
 constexpr int kMC = 64;       // memory columns per workgroup (16 per wave)
 constexpr int kThreads = 256;
 
-__device__ __forceinline__ uint32_t f2bf(float f) {
-    const uint32_t u = __float_as_uint(f);
-    return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
-}
-__device__ __forceinline__ float ld1(const float *p) { return *p; }
-__device__ __forceinline__ float ld1(const bf16_t *p) { return __uint_as_float((uint32_t)*p << 16); }
-__device__ __forceinline__ void st1(float *p, float v) { *p = v; }
-__device__ __forceinline__ void st1(bf16_t *p, float v) { *p = (bf16_t)f2bf(v); }
-
-// fp32 inputs multiply in fp32; bf16 inputs multiply in bf16 (hi + lo where a value is not
-// exactly a bf16 number) -- see chunk_mma.h
-template <class TI> struct PrecOf { typedef PrecF32 type; };
-template <> struct PrecOf<bf16_t> { typedef PrecBf16 type; };
-
 template <class TI>
 struct ChunkFwdP {
     const TI *Q, *K, *V, *beta;
@@ -120,7 +106,7 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
     constexpr int NKQ = kC * (D / 4) / kThreads;    // 4-element groups of K (and of Q) per thread
     constexpr int NV = kC * (kMC / 4) / kThreads;   // 4-element groups of V per thread
     typename X::Raw4 kreg[NKQ], qreg[NKQ], vreg[NV];
-    float breg = 0.f;
+    uint32_t breg = 0u;   // raw bits, converted in commit()
     auto prefetch = [&](int ch) {   // rows past the end are clamped here and zeroed in commit()
         const int t0 = ch * kC;
 #pragma unroll
@@ -135,7 +121,7 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
             const int f = tid + i * kThreads, row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
             vreg[i] = X::ld_raw(vb + (int64_t)min(t0 + row, p.L - 1) * p.vs.l + col);
         }
-        breg = ld1(bb + (int64_t)min(t0 + (tid % kC), p.L - 1) * p.bs.l);
+        breg = ld_bits(bb + (int64_t)min(t0 + (tid % kC), p.L - 1) * p.bs.l);
     };
     auto commit = [&](int ch) {
         const int t0 = ch * kC;
@@ -153,7 +139,7 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
             const bool keep = full || t0 + row < p.L;
             *reinterpret_cast<float4 *>(Vs + row * LDV + col) = X::raw_f32(X::keep_raw(vreg[i], keep));
         }
-        if (tid < kC) bts[tid] = (t0 + tid < p.L) ? breg : 0.f;
+        if (tid < kC) bts[tid] = (t0 + tid < p.L) ? bits_f32<TI>(breg) : 0.f;
     };
 
     const int nchunks = (p.L + kC - 1) / kC;
@@ -164,25 +150,24 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
         const int t0 = ch * kC;
         if (ch + 1 < nchunks) prefetch(ch + 1);
 
-        // ---- A = K K^T (strict lower) and B = Q K^T (lower), 10 + 10 tiles over the 4 waves
-        for (int tix = wave; tix < 20; tix += 4) {
-            const int which = tix / 10, tri = tix % 10;     // tri -> (ci, cj), cj <= ci
-            const int ci = tri < 1 ? 0 : tri < 3 ? 1 : tri < 6 ? 2 : 3;
-            const int cj = tri - (ci * (ci + 1)) / 2;
-            const typename Lds::MatK &Xm = which ? Qs : Ks;
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int eb = 0; eb < EB; ++eb)
-                acc = X::template mma<false, false>(X::lda(Xm, ci * 16 + ln, eb * 16 + 4 * lq),
-                                                    X::ldb(Ks, cj * 16 + ln, eb * 16 + 4 * lq), acc);
-            const typename Lds::MatA &T = which ? Bs : As;
+        // ---- A = K K^T (strict lower) and B = Q K^T (lower): 10 pairs of tiles over the 4 waves
+        //      (the two tiles of a pair share their right operand)
+        for (int pix = wave; pix < 10; pix += 4) {
+            int ci, cj;
+            tri_index(pix, ci, cj);
+            const auto fb = [&](int eb) { return X::ldb(Ks, cj * 16 + ln, eb * 16 + 4 * lq); };
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            const f32x4 accA = mma_range<X, false, false>(
+                0, EB, [&](int eb) { return X::lda(Ks, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
+            const f32x4 accB = mma_range<X, false, false>(
+                0, EB, [&](int eb) { return X::lda(Qs, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = ci * 16 + 4 * lq + r, col = cj * 16 + ln;
-                const bool keep = which ? col <= row : col < row;
-                const float v = keep ? acc[r] : 0.f;
-                X::st(T, row, col, v);
-                if (!which && ci == cj) Ad[row * LDD + ln] = v;
+                const float va = col < row ? accA[r] : 0.f;
+                X::st(As, row, col, va);
+                X::st(Bs, row, col, col <= row ? accB[r] : 0.f);
+                if (ci == cj) Ad[row * LDD + ln] = va;
             }
         }
         __syncthreads();
@@ -214,13 +199,13 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
             for (int eb = 0; eb < EB; ++eb) sb[eb] = X::accb(s[eb]);
 #pragma unroll
             for (int cb = 0; cb < kCB; ++cb) {
-                pt[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
-                ot[cb] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-                for (int eb = 0; eb < EB; ++eb) {
-                    pt[cb] = X::template mma<false, true>(X::lda(Ks, cb * 16 + ln, eb * 16 + 4 * lq), sb[eb], pt[cb]);
-                    ot[cb] = X::template mma<false, true>(X::lda(Qs, cb * 16 + ln, eb * 16 + 4 * lq), sb[eb], ot[cb]);
-                }
+                const auto fb = [&](int eb) { return sb[eb]; };
+                pt[cb] = mma_range<X, false, true>(
+                    0, EB, [&](int eb) { return X::lda(Ks, cb * 16 + ln, eb * 16 + 4 * lq); }, fb,
+                    f32x4{0.f, 0.f, 0.f, 0.f});
+                ot[cb] = mma_range<X, false, true>(
+                    0, EB, [&](int eb) { return X::lda(Qs, cb * 16 + ln, eb * 16 + 4 * lq); }, fb,
+                    f32x4{0.f, 0.f, 0.f, 0.f});
             }
         }
         __syncthreads();   // the four inverses are visible
@@ -230,10 +215,9 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
         typename X::B ub[kCB];
 #pragma unroll
         for (int a = 0; a < kCB; ++a) {
-            f32x4 y = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int b = 0; b < a; ++b)
-                y = X::template mma<true, true>(X::lda(As, a * 16 + ln, b * 16 + 4 * lq), ub[b], y);
+            const auto fu = [&](int b) { return ub[b]; };
+            f32x4 y = mma_range<X, true, true>(
+                0, a, [&](int b) { return X::lda(As, a * 16 + ln, b * 16 + 4 * lq); }, fu, f32x4{0.f, 0.f, 0.f, 0.f});
             f32x4 rhs;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -245,9 +229,8 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
             ub[a] = X::accb(u[a]);
             y = X::template mma<true, true>(X::lda(As, a * 16 + ln, a * 16 + 4 * lq), ub[a], y);   // + strict_lower(A_aa) U_a
             // out = Q S + tril(B) U
-#pragma unroll
-            for (int b = 0; b <= a; ++b)
-                ot[a] = X::template mma<true, true>(X::lda(Bs, a * 16 + ln, b * 16 + 4 * lq), ub[b], ot[a]);
+            ot[a] = mma_range<X, true, true>(
+                0, a + 1, [&](int b) { return X::lda(Bs, a * 16 + ln, b * 16 + 4 * lq); }, fu, ot[a]);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int t = t0 + a * 16 + 4 * lq + r;
@@ -255,16 +238,16 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
                     const int64_t o = (seq * p.L + t) * D + m0 + cw + ln;
                     p.vold[o] = pt[a][r] + y[r];
                     p.vins[o] = u[a][r];
-                    st1(p.out + o, ot[a][r]);
+                    st_out(p.out + o, ot[a][r]);
                 }
             }
         }
         // S += K^T U
 #pragma unroll
         for (int eb = 0; eb < EB; ++eb)
-#pragma unroll
-            for (int cb = 0; cb < kCB; ++cb)
-                s[eb] = X::template mma<false, true>(X::lda_t(Ks, cb * 16 + 4 * lq, eb * 16 + ln), ub[cb], s[eb]);
+            s[eb] = mma_range<X, false, true>(
+                0, kCB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, eb * 16 + ln); },
+                [&](int cb) { return ub[cb]; }, s[eb]);
         __syncthreads();   // every wave is done with Ks, Qs, Vs, As, Bs
         if (ch + 1 < nchunks) {
             commit(ch + 1);

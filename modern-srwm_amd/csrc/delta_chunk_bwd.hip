@@ -1,0 +1,585 @@
+// Chunkwise delta-rule BACKWARD on the matrix cores (E == M = D in {64, 128}).
+//
+// Per chunk, last chunk first, with S the memory at the chunk's entry (obtained by reverting
+// its exit value S'), dS' the gradient with respect to S', U = v_insert (saved by the forward):
+//     S  = S' - K^T U
+//     dU = tril(Q K^T)^T dOut + K dS'
+//     (I + strict_lower(K K^T)^T diag(beta)) dR = dU         dR: gradient of the inserts
+//     Y  = diag(beta) dR = grad_V,    grad_beta = rowsum(dR * (V - v_old))
+//     dS = dS' + Q^T dOut - K^T Y
+//     G1 = tril(dOut U^T),   X = strict_lower(Y U^T)
+//     grad_Q = dOut S^T + G1 K
+//     grad_K = G1^T Q + U dS'^T - Y S^T - (X + X^T) K
+// An MFMA contracts over the index that runs along lane/16 and the register number, and a
+// register tile of the memory has one fixed axis there.  The first five lines contract over
+// memory rows or chunk steps, the last three over memory COLUMNS, so the work is split into
+// two sweeps with the memory tiled the other way round:
+//   column sweep  a wave owns 16 columns of S and dS (rows in the registers); it solves the
+//                 upper triangular system by 16-row block back substitution (diagonal blocks
+//                 inverted on the vector ALUs, one per wave) and writes grad_V and grad_beta;
+//   row sweep     a wave owns 16 rows of S and dS, held transposed (columns in the registers);
+//                 it reads grad_V back, forms G1 and X cooperatively and writes grad_Q, grad_K,
+//                 the reverted memory and the gradient of the initial memory.  Every word of
+//                 grad_Q / grad_K has one writer: no atomics.
+// Both sweeps revert S and accumulate dS on their own (one extra product each, cheaper than
+// moving the memory between the two layouts every chunk).  With fp32 inputs every product is
+// v_mfma_f32_16x16x4f32; with bf16 inputs it is v_mfma_f32_16x16x32_bf16 on hi/lo split
+// operands (chunk_mma.h), accumulation in fp32 either way.
+//
+// Replaces fast_weight_backward_value_beta_kernel and fast_weight_backward_query_key_kernel of
+// the reference (supervised_learning/fast_weight/fast_weight_cuda.cu:397-560, :244-393) for
+// callers that ask for the chunkwise form.
+#include "chunk_mma.h"
+#include "common.h"
+#include "xlane.h"
+
+namespace fw {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWC = 64;   // memory columns (column sweep) or rows (row sweep) per workgroup
+
+template <class TI>
+struct ChunkBwdP {
+    const TI *Q, *K, *V, *beta;
+    Strided3 qs, ks, vs, bs;
+    const float *vold, *vins;
+    const TI *go;
+    Strided3 gs;
+    float *W;
+    float *gQ, *gK, *gV, *gbeta;
+    float *gW;
+    int N, H, L;
+    unsigned grad_state_mode;
+};
+
+// ------------------------------------------------------------------------------------------
+// Column sweep
+// ------------------------------------------------------------------------------------------
+template <class TI, int D>
+struct ColLds {
+    typedef typename PrecOf<TI>::type X;
+    static constexpr int C = 64;
+    static constexpr int LDK = D + X::kPad, LDA = C + X::kPad, LDD = 16 + X::kPad;
+    typedef typename X::template Mat<LDK, false> MatK;
+    typedef typename X::template Mat<LDA, true> MatA;
+    typedef typename X::template Mat<LDD, true> MatD;
+    static constexpr int oK = 0;
+    static constexpr int oQ = oK + MatK::bytes(C);
+    static constexpr int oAT = oQ + MatK::bytes(C);
+    static constexpr int oBT = oAT + MatA::bytes(C);
+    static constexpr int oD = oBT + MatA::bytes(C);
+    static constexpr int oAd = oD + MatD::bytes(C);            // fp32 [C][LDD]: diagonal blocks of A^T
+    static constexpr int oBt = oAd + C * LDD * 4;              // fp32 [C]: beta
+    static constexpr int oGb = oBt + C * 4;                    // fp32 [4][C]: per-wave parts of grad_beta
+    static constexpr int kBytes = oGb + 4 * C * 4;
+    static_assert(MatK::bytes(C) % 16 == 0 && MatA::bytes(C) % 16 == 0 && MatD::bytes(C) % 16 == 0, "alignment");
+};
+
+template <class TI, int D, int MS>
+__global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP<TI> p) {
+    typedef ColLds<TI, D> Lds;
+    typedef typename Lds::X X;
+    constexpr int C = Lds::C, CB = C / 16, EB = D / 16, LDD = Lds::LDD;
+    static_assert(MS * kWC == D, "column split");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const typename Lds::MatK Ks(smem + Lds::oK, C), Qs(smem + Lds::oQ, C);
+    const typename Lds::MatA AT(smem + Lds::oAT, C);   // strict upper triangle: (K K^T)^T
+    const typename Lds::MatA BT(smem + Lds::oBT, C);   // upper triangle with diagonal: tril(Q K^T)^T
+    const typename Lds::MatD Di(smem + Lds::oD, C);    // inverses of the diagonal blocks of I + A^T diag(beta)
+    float *Ad = reinterpret_cast<float *>(smem + Lds::oAd);
+    float *bts = reinterpret_cast<float *>(smem + Lds::oBt);
+    float *gbp = reinterpret_cast<float *>(smem + Lds::oGb);
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int ln = lane & 15, lq = lane >> 4;
+    const int64_t seq = blockIdx.x / MS;
+    const int m0 = (int)(blockIdx.x % MS) * kWC + 16 * wave;   // first memory column of this wave
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;
+    const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
+    const TI *vb = p.V + n * p.vs.n + h * p.vs.h + m0 + ln;
+    const TI *gob = p.go + n * p.gs.n + h * p.gs.h + m0 + ln;
+    const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
+    const float *vob = p.vold + seq * p.L * D + m0 + ln;
+    const float *vib = p.vins + seq * p.L * D + m0 + ln;
+    const float *Wg = p.W + seq * D * D + m0 + ln;
+    const float *gWg = (p.gW && p.grad_state_mode != 0u) ? p.gW + seq * D * D + m0 + ln : nullptr;
+
+    // 16 columns of the memory (exit value of the last chunk) and of its gradient
+    f32x4 s[EB], ds[EB];
+#pragma unroll
+    for (int eb = 0; eb < EB; ++eb)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int o = (eb * 16 + 4 * lq + r) * D;
+            s[eb][r] = Wg[o];
+            ds[eb][r] = gWg ? gWg[o] : 0.f;
+        }
+
+    // next chunk's inputs: K, Q rows for LDS; U, dOut, V, v_old directly in accumulator layout
+    constexpr int NKQ = C * (D / 4) / kThreads;
+    typename X::Raw4 kreg[NKQ], qreg[NKQ];
+    f32x4 pu[CB], po[CB];
+    uint32_t pg[CB][4], pv[CB][4], breg = 0u;   // raw bits, converted in commit()
+    auto prefetch = [&](int ch) {
+        const int t0 = ch * C;
+#pragma unroll
+        for (int i = 0; i < NKQ; ++i) {
+            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const int t = min(t0 + row, p.L - 1);
+            kreg[i] = X::ld_raw(kb + (int64_t)t * p.ks.l + col);
+            qreg[i] = X::ld_raw(qb + (int64_t)t * p.qs.l + col);
+        }
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t t = min(t0 + cb * 16 + 4 * lq + r, p.L - 1);
+                pu[cb][r] = vib[t * D];
+                po[cb][r] = vob[t * D];
+                pg[cb][r] = ld_bits(gob + t * p.gs.l);
+                pv[cb][r] = ld_bits(vb + t * p.vs.l);
+            }
+        breg = ld_bits(bb + (int64_t)min(t0 + (tid % C), p.L - 1) * p.bs.l);
+    };
+    f32x4 u[CB], g[CB], vd[CB];   // this chunk: U, dOut, V - v_old (rows past the end zeroed)
+    auto commit = [&](int ch) {
+        const int t0 = ch * C;
+        const bool full = t0 + C <= p.L;
+#pragma unroll
+        for (int i = 0; i < NKQ; ++i) {
+            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const bool keep = full || t0 + row < p.L;
+            X::st_raw(Ks, row, col, X::keep_raw(kreg[i], keep));
+            X::st_raw(Qs, row, col, X::keep_raw(qreg[i], keep));
+        }
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float m = (full || t0 + cb * 16 + 4 * lq + r < p.L) ? 1.f : 0.f;
+                u[cb][r] = pu[cb][r] * m;
+                g[cb][r] = bits_f32<TI>(pg[cb][r]) * m;
+                vd[cb][r] = (bits_f32<TI>(pv[cb][r]) - po[cb][r]) * m;
+            }
+        if (tid < C) bts[tid] = (t0 + tid < p.L) ? bits_f32<TI>(breg) : 0.f;
+    };
+
+    const int nchunks = (p.L + C - 1) / C;
+    prefetch(nchunks - 1);
+    commit(nchunks - 1);
+    __syncthreads();
+    for (int ch = nchunks - 1; ch >= 0; --ch) {
+        const int t0 = ch * C;
+        if (ch > 0) prefetch(ch - 1);
+
+        // ---- (K K^T)^T strict upper and tril(Q K^T)^T: 10 pairs of tiles (a pair shares its right
+        //      operand), stored transposed
+        for (int pix = wave; pix < 10; pix += 4) {
+            int ci, cj;
+            tri_index(pix, ci, cj);
+            const auto fb = [&](int eb) { return X::ldb(Ks, cj * 16 + ln, eb * 16 + 4 * lq); };
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            const f32x4 accA = mma_range<X, false, false>(
+                0, EB, [&](int eb) { return X::lda(Ks, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
+            const f32x4 accB = mma_range<X, false, false>(
+                0, EB, [&](int eb) { return X::lda(Qs, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
+            float va[4], vb_[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = ci * 16 + 4 * lq + r, col = cj * 16 + ln;
+                va[r] = col < row ? accA[r] : 0.f;
+                vb_[r] = col <= row ? accB[r] : 0.f;
+            }
+            X::st4(AT, cj * 16 + ln, ci * 16 + 4 * lq, make_float4(va[0], va[1], va[2], va[3]));
+            X::st4(BT, cj * 16 + ln, ci * 16 + 4 * lq, make_float4(vb_[0], vb_[1], vb_[2], vb_[3]));
+            if (ci == cj)
+                *reinterpret_cast<float4 *>(Ad + (ci * 16 + ln) * LDD + 4 * lq) = make_float4(va[0], va[1], va[2], va[3]);
+        }
+        __syncthreads();
+
+        // ---- inverse of the diagonal block `wave` of I + A^T diag(beta) (unit upper triangular):
+        //      column ln, x_i = [i == ln] - sum_{j>i} A^T_ij beta_j x_j, from the bottom row up
+        {
+            float x[16];
+            const float *ad = Ad + (wave * 16) * LDD;
+#pragma unroll
+            for (int i = 15; i >= 0; --i) {
+                float acc = (i == ln) ? 1.f : 0.f;
+#pragma unroll
+                for (int j = i + 1; j < 16; ++j) acc = fmaf(-bts[wave * 16 + j] * ad[i * LDD + j], x[j], acc);
+                x[i] = acc;
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) X::st(Di, wave * 16 + i, ln, x[i]);
+        }
+
+        // ---- independent of the inversion: revert S, dU = K dS' + tril(Q K^T)^T dOut
+        typename X::B gob_[CB];
+        f32x4 du[CB];
+        {
+            typename X::B nub[CB], dsb[EB];
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                nub[cb] = X::accb(-u[cb]);
+                gob_[cb] = X::accb_exact(g[cb]);
+            }
+#pragma unroll
+            for (int eb = 0; eb < EB; ++eb) dsb[eb] = X::accb(ds[eb]);
+#pragma unroll
+            for (int eb = 0; eb < EB; ++eb)
+                s[eb] = mma_range<X, false, true>(
+                    0, CB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, eb * 16 + ln); },
+                    [&](int cb) { return nub[cb]; }, s[eb]);
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                du[cb] = mma_range<X, false, true>(
+                    0, EB, [&](int eb) { return X::lda(Ks, cb * 16 + ln, eb * 16 + 4 * lq); },
+                    [&](int eb) { return dsb[eb]; }, f32x4{0.f, 0.f, 0.f, 0.f});
+                du[cb] = mma_range<X, true, false>(
+                    cb, CB, [&](int b) { return X::lda(BT, cb * 16 + ln, b * 16 + 4 * lq); },
+                    [&](int b) { return gob_[b]; }, du[cb]);
+            }
+        }
+        __syncthreads();   // the four inverses are visible
+
+        // ---- block back substitution, last 16-row block first
+        typename X::B nyb[CB];
+#pragma unroll
+        for (int a = CB - 1; a >= 0; --a) {
+            const f32x4 rhs = mma_range<X, true, true>(
+                a + 1, CB, [&](int b) { return X::lda(AT, a * 16 + ln, b * 16 + 4 * lq); },
+                [&](int b) { return nyb[b]; }, du[a]);
+            const f32x4 dr = X::template mma<true, true>(X::lda(Di, a * 16 + ln, 4 * lq), X::accb(rhs),
+                                                         f32x4{0.f, 0.f, 0.f, 0.f});
+            f32x4 y;
+            float pb[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                y[r] = bts[a * 16 + 4 * lq + r] * dr[r];
+                pb[r] = dr[r] * vd[a][r];
+            }
+            nyb[a] = X::accb(-y);
+            group_sum_n<16, 4>(pb);   // over the wave's 16 columns
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = t0 + a * 16 + 4 * lq + r;
+                if (t < p.L) p.gV[(seq * p.L + t) * D + m0 + ln] = y[r];
+                gbp[wave * C + a * 16 + 4 * lq + r] = pb[r];   // 16 lanes, same value, same word
+            }
+        }
+        // ---- dS = dS' + Q^T dOut - K^T Y
+#pragma unroll
+        for (int eb = 0; eb < EB; ++eb) {
+            ds[eb] = mma_range<X, false, false>(
+                0, CB, [&](int cb) { return X::lda_t(Qs, cb * 16 + 4 * lq, eb * 16 + ln); },
+                [&](int cb) { return gob_[cb]; }, ds[eb]);
+            ds[eb] = mma_range<X, false, true>(
+                0, CB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, eb * 16 + ln); },
+                [&](int cb) { return nyb[cb]; }, ds[eb]);
+        }
+        __syncthreads();   // every wave is done with the chunk's LDS; grad_beta parts are visible
+        if (tid < C && t0 + tid < p.L) {
+            const float sum = gbp[tid] + gbp[C + tid] + gbp[2 * C + tid] + gbp[3 * C + tid];
+            if constexpr (MS == 1) {
+                p.gbeta[seq * p.L + t0 + tid] = sum;
+            } else {
+                atomicAdd(p.gbeta + seq * p.L + t0 + tid, sum);
+            }
+        }
+        if (ch > 0) {
+            commit(ch - 1);
+            __syncthreads();
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Row sweep
+// ------------------------------------------------------------------------------------------
+template <class TI, int D, int C>
+struct RowLds {
+    typedef typename PrecOf<TI>::type X;
+    static constexpr int LDM = D + X::kPad, LDW = kWC + X::kPad, LDC = C + X::kPad;
+    typedef typename X::template Mat<LDM, false> MatG;   // dOut: an input
+    typedef typename X::template Mat<LDM, true> MatU;    // U, Y: computed
+    typedef typename X::template Mat<LDW, false> MatK;   // this workgroup's 64 columns of K, Q
+    typedef typename X::template Mat<LDC, true> MatC;    // G1, X + X^T
+    static constexpr int oG = 0;
+    static constexpr int oU = oG + MatG::bytes(C);
+    static constexpr int oY = oU + MatU::bytes(C);
+    static constexpr int oK = oY + MatU::bytes(C);
+    static constexpr int oQ = oK + MatK::bytes(C);
+    static constexpr int oG1 = oQ + MatK::bytes(C);
+    static constexpr int oZ = oG1 + MatC::bytes(C);
+    static constexpr int kBytes = oZ + MatC::bytes(C);
+    static_assert(MatG::bytes(C) % 16 == 0 && MatU::bytes(C) % 16 == 0 && MatK::bytes(C) % 16 == 0 &&
+                      MatC::bytes(C) % 16 == 0, "alignment");
+};
+
+template <class TI, int D, int MS, int C>
+__global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP<TI> p) {
+    typedef RowLds<TI, D, C> Lds;
+    typedef typename Lds::X X;
+    constexpr int CB = C / 16, MB = D / 16, NTRI = CB * (CB + 1) / 2;
+    static_assert(MS * kWC == D, "row split");
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const typename Lds::MatG Gs(smem + Lds::oG, C);
+    const typename Lds::MatU Us(smem + Lds::oU, C), Ys(smem + Lds::oY, C);
+    const typename Lds::MatK Kw(smem + Lds::oK, C), Qw(smem + Lds::oQ, C);
+    const typename Lds::MatC G1(smem + Lds::oG1, C), Z(smem + Lds::oZ, C);
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int ln = lane & 15, lq = lane >> 4;
+    const int64_t seq = blockIdx.x / MS;
+    const int e0 = (int)(blockIdx.x % MS) * kWC;     // first memory row of this workgroup
+    const int cw = 16 * wave;                        // this wave's rows inside it
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const TI *qb = p.Q + n * p.qs.n + h * p.qs.h + e0;
+    const TI *kb = p.K + n * p.ks.n + h * p.ks.h + e0;
+    const TI *gob = p.go + n * p.gs.n + h * p.gs.h;
+    const float *yb = p.gV + seq * p.L * D;
+    const float *ub = p.vins + seq * p.L * D;
+    float *Wg = p.W + seq * D * D + (e0 + cw + ln) * D;            // row e0 + cw + ln of the memory
+    float *gWg = p.gW ? p.gW + seq * D * D + (e0 + cw + ln) * D : nullptr;
+    const bool g_in = gWg && p.grad_state_mode != 0u;
+
+    // 16 rows of the memory and of its gradient, transposed: tile mb, register r <-> column
+    // 16*mb + 4*lq + r, lane ln <-> row
+    f32x4 st[MB], dst[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const float4 w = *reinterpret_cast<const float4 *>(Wg + mb * 16 + 4 * lq);
+        st[mb] = f32x4{w.x, w.y, w.z, w.w};
+        if (g_in) {
+            const float4 gw = *reinterpret_cast<const float4 *>(gWg + mb * 16 + 4 * lq);
+            dst[mb] = f32x4{gw.x, gw.y, gw.z, gw.w};
+        } else {
+            dst[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    }
+
+    constexpr int NG = C * (D / 4) / kThreads;      // 4-element groups per thread of dOut, U, Y
+    constexpr int NK = C * (kWC / 4) / kThreads;    // ... of the K and Q slices
+    static_assert(NG >= 1 && NK >= 1, "chunk too short for 256 threads");
+    typename X::Raw4 greg[NG], kreg[NK], qreg[NK];
+    float4 ureg[NG], yreg[NG];
+    auto prefetch = [&](int ch) {
+        const int t0 = ch * C;
+#pragma unroll
+        for (int i = 0; i < NG; ++i) {
+            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const int64_t t = min(t0 + row, p.L - 1);
+            greg[i] = X::ld_raw(gob + t * p.gs.l + col);
+            ureg[i] = *reinterpret_cast<const float4 *>(ub + t * D + col);
+            yreg[i] = *reinterpret_cast<const float4 *>(yb + t * D + col);
+        }
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int f = tid + i * kThreads, row = f / (kWC / 4), col = (f % (kWC / 4)) * 4;
+            const int64_t t = min(t0 + row, p.L - 1);
+            kreg[i] = X::ld_raw(kb + t * p.ks.l + col);
+            qreg[i] = X::ld_raw(qb + t * p.qs.l + col);
+        }
+    };
+    auto commit = [&](int ch) {
+        const int t0 = ch * C;
+        const bool full = t0 + C <= p.L;
+#pragma unroll
+        for (int i = 0; i < NG; ++i) {
+            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const bool keep = full || t0 + row < p.L;
+            const float m = keep ? 1.f : 0.f;
+            X::st_raw(Gs, row, col, X::keep_raw(greg[i], keep));
+            X::st4(Us, row, col, make_float4(ureg[i].x * m, ureg[i].y * m, ureg[i].z * m, ureg[i].w * m));
+            X::st4(Ys, row, col, make_float4(yreg[i].x * m, yreg[i].y * m, yreg[i].z * m, yreg[i].w * m));
+        }
+#pragma unroll
+        for (int i = 0; i < NK; ++i) {
+            const int f = tid + i * kThreads, row = f / (kWC / 4), col = (f % (kWC / 4)) * 4;
+            const bool keep = full || t0 + row < p.L;
+            X::st_raw(Kw, row, col, X::keep_raw(kreg[i], keep));
+            X::st_raw(Qw, row, col, X::keep_raw(qreg[i], keep));
+        }
+    };
+
+    const int nchunks = (p.L + C - 1) / C;
+    prefetch(nchunks - 1);
+    commit(nchunks - 1);
+    __syncthreads();
+    for (int ch = nchunks - 1; ch >= 0; --ch) {
+        const int t0 = ch * C;
+        if (ch > 0) prefetch(ch - 1);
+
+        // ---- G1 = tril(dOut U^T) and Z = X + X^T with X = strict_lower(Y U^T): NTRI pairs of tiles
+        //      (a pair shares its right operand)
+        for (int pix = wave; pix < NTRI; pix += 4) {
+            int ci, cj;
+            tri_index(pix, ci, cj);
+            const auto fb = [&](int mb) { return X::ldb(Us, cj * 16 + ln, mb * 16 + 4 * lq); };
+            const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+            const f32x4 accG = mma_range<X, false, true>(
+                0, MB, [&](int mb) { return X::lda(Gs, ci * 16 + ln, mb * 16 + 4 * lq); }, fb, zero);
+            const f32x4 accX = mma_range<X, true, true>(
+                0, MB, [&](int mb) { return X::lda(Ys, ci * 16 + ln, mb * 16 + 4 * lq); }, fb, zero);
+            const int col = cj * 16 + ln;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int row = ci * 16 + 4 * lq + r;
+                X::st(G1, row, col, col <= row ? accG[r] : 0.f);
+            }
+            if (ci != cj) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) X::st(Z, ci * 16 + 4 * lq + r, col, accX[r]);
+                X::st4(Z, col, ci * 16 + 4 * lq, make_float4(accX[0], accX[1], accX[2], accX[3]));
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int row = ci * 16 + 4 * lq + r;
+                    if (col <= row) X::st(Z, row, col, col < row ? accX[r] : 0.f);
+                    if (col < row) X::st(Z, col, row, accX[r]);
+                }
+            }
+        }
+
+        // ---- independent of the tiles: operand fragments, revert S^T
+        typename X::B nkb[CB], qbf[CB], nstb[MB], dstb[MB];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            nkb[cb] = X::negb(X::ldb_t(Kw, cb * 16 + 4 * lq, cw + ln));
+            qbf[cb] = X::ldb_t(Qw, cb * 16 + 4 * lq, cw + ln);
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            dstb[mb] = X::accb(dst[mb]);   // dS' (before this chunk's update)
+            st[mb] = mma_range<X, true, false>(
+                0, CB, [&](int cb) { return X::lda_t(Us, cb * 16 + 4 * lq, mb * 16 + ln); },
+                [&](int cb) { return nkb[cb]; }, st[mb]);
+            nstb[mb] = X::accb(-st[mb]);   // -S (entry value)
+        }
+        __syncthreads();   // G1 and Z are visible
+
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            const auto fns = [&](int mb) { return nstb[mb]; };
+            const auto fnk = [&](int b) { return nkb[b]; };
+            f32x4 dqn = mma_range<X, false, true>(
+                0, MB, [&](int mb) { return X::lda(Gs, cb * 16 + ln, mb * 16 + 4 * lq); }, fns, f32x4{0.f, 0.f, 0.f, 0.f});
+            dqn = mma_range<X, true, false>(
+                0, cb + 1, [&](int b) { return X::lda(G1, cb * 16 + ln, b * 16 + 4 * lq); }, fnk, dqn);
+            f32x4 dk = mma_range<X, true, true>(
+                0, MB, [&](int mb) { return X::lda(Us, cb * 16 + ln, mb * 16 + 4 * lq); },
+                [&](int mb) { return dstb[mb]; }, f32x4{0.f, 0.f, 0.f, 0.f});
+            dk = mma_range<X, true, true>(
+                0, MB, [&](int mb) { return X::lda(Ys, cb * 16 + ln, mb * 16 + 4 * lq); }, fns, dk);
+            dk = mma_range<X, true, false>(
+                cb, CB, [&](int b) { return X::lda_t(G1, b * 16 + 4 * lq, cb * 16 + ln); },
+                [&](int b) { return qbf[b]; }, dk);
+            dk = mma_range<X, true, false>(
+                0, CB, [&](int b) { return X::lda(Z, cb * 16 + ln, b * 16 + 4 * lq); }, fnk, dk);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = t0 + cb * 16 + 4 * lq + r;
+                if (t < p.L) {
+                    const int64_t o = (seq * p.L + t) * D + e0 + cw + ln;
+                    p.gQ[o] = -dqn[r];
+                    p.gK[o] = dk[r];
+                }
+            }
+        }
+        // ---- dS^T += dOut^T Q - Y^T K
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            dst[mb] = mma_range<X, false, false>(
+                0, CB, [&](int cb) { return X::lda_t(Gs, cb * 16 + 4 * lq, mb * 16 + ln); },
+                [&](int cb) { return qbf[cb]; }, dst[mb]);
+            dst[mb] = mma_range<X, true, false>(
+                0, CB, [&](int cb) { return X::lda_t(Ys, cb * 16 + 4 * lq, mb * 16 + ln); },
+                [&](int cb) { return nkb[cb]; }, dst[mb]);
+        }
+        __syncthreads();
+        if (ch > 0) {
+            commit(ch - 1);
+            __syncthreads();
+        }
+    }
+
+    // the memory is back at its initial value; its gradient goes out if asked for
+    const bool accum = gWg && p.grad_state_mode == 2u;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        *reinterpret_cast<float4 *>(Wg + mb * 16 + 4 * lq) = make_float4(st[mb][0], st[mb][1], st[mb][2], st[mb][3]);
+        if (gWg) {
+            float4 *d = reinterpret_cast<float4 *>(gWg + mb * 16 + 4 * lq);
+            float4 o = make_float4(dst[mb][0], dst[mb][1], dst[mb][2], dst[mb][3]);
+            if (accum) {
+                const float4 in = *d;
+                o = make_float4(o.x + in.x, o.y + in.y, o.z + in.z, o.w + in.w);
+            }
+            *d = o;
+        }
+    }
+}
+
+__global__ void zero_words_kernel(float *a, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t j = i; j < n; j += stride) a[j] = 0.f;
+}
+
+template <class TI, int D, int MS, int C2>
+int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
+    constexpr int lds1 = ColLds<TI, D>::kBytes, lds2 = RowLds<TI, D, C2>::kBytes;
+    static_assert(lds1 <= (int)kMaxLdsBytes && lds2 <= (int)kMaxLdsBytes, "LDS budget");
+    hipError_t err = hipFuncSetAttribute((const void *)delta_bwd_chunk_col_kernel<TI, D, MS>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds1);
+    if (err != hipSuccess) return (int)err;
+    err = hipFuncSetAttribute((const void *)delta_bwd_chunk_row_kernel<TI, D, MS, C2>,
+                              hipFuncAttributeMaxDynamicSharedMemorySize, lds2);
+    if (err != hipSuccess) return (int)err;
+    const int grid = p.N * p.H * MS;
+    if (MS > 1)   // two workgroups of the column sweep add their parts of grad_beta
+        hipLaunchKernelGGL(zero_words_kernel, dim3(256), dim3(256), 0, s, p.gbeta, (int64_t)p.N * p.H * p.L);
+    hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS>), dim3(grid), dim3(kThreads), lds1, s, p);
+    hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2>), dim3(grid), dim3(kThreads), lds2, s, p);
+    return (int)hipGetLastError();
+}
+
+template <class TI>
+bool rows_ok(const TI *ptr, const Strided3 &s) {
+    return ((uintptr_t)ptr % (4 * sizeof(TI)) == 0) && s.n % 4 == 0 && s.h % 4 == 0 && s.l % 4 == 0;
+}
+bool ok16(const void *ptr) { return (uintptr_t)ptr % 16 == 0; }
+
+template <class TI>
+int dispatch_chunk_bwd(const ChunkBwdP<TI> &p, int D, hipStream_t s) {
+    if (!rows_ok(p.Q, p.qs) || !rows_ok(p.K, p.ks) || !rows_ok(p.V, p.vs) || !rows_ok(p.go, p.gs) ||
+        !ok16(p.vold) || !ok16(p.vins) || !ok16(p.W) || !ok16(p.gV) || !ok16(p.gQ) || !ok16(p.gK) ||
+        (p.gW && !ok16(p.gW)))
+        return -1;
+    constexpr bool bf = PrecOf<TI>::type::kBf;
+    switch (D) {
+        case 128: return launch_chunk_bwd<TI, 128, 2, bf ? 64 : 32>(p, s);
+        case 64: return launch_chunk_bwd<TI, 64, 1, 64>(p, s);
+        default: return -1;
+    }
+}
+
+}  // namespace
+
+int launch_delta_bwd_chunk(const DeltaBwdParams &p, hipStream_t s) {
+    if (p.E != p.M) return -1;
+    const ChunkBwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
+                             p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode};
+    return dispatch_chunk_bwd(q, p.E, s);
+}
+
+int launch_delta_bwd_chunk_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s) {
+    if (p.E != p.M) return -1;
+    const ChunkBwdP<uint16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
+                                p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode};
+    return dispatch_chunk_bwd(q, p.E, s);
+}
+
+}  // namespace fw

@@ -158,9 +158,8 @@ struct BwdP {
     const TI *go;
     Strided3 gs;
     float *W;
-    float *gQ, *gK;   // fp32 whatever TI is (they may be accumulated across workgroups)
-    TI *gV;
-    float *gbeta;
+    float *gQ, *gK, *gV, *gbeta;   // fp32 whatever TI is
+
     float *gW;
     int N, H, L;
     unsigned grad_state_mode;

@@ -251,12 +251,15 @@ def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, g
     _require(beta, "beta", (N, H, L, 1), io)
     for t, nm in ((v_old, "v_old"), (v_insert, "v_insert")):
         _require(t, nm, (N, H, L, M))
-    for t, nm in ((grad_out, "grad_out"), (grad_v, "grad_v")):
-        _require(t, nm, (N, H, L, M), io)
+    _require(grad_out, "grad_out", (N, H, L, M), io)
     _require(kv, "kv", (N, H, E, M))
-    _require(grad_q, "grad_q", (N, H, L, E), io)
-    _require(grad_k, "grad_k", (N, H, L, E), io)
-    _require(grad_beta, "grad_beta", (N, H, L, 1), io)
+    # the library writes fp32 gradients; with bf16 inputs the caller may pass fp32 tensors
+    # (used as they are) or bf16 ones (filled through an fp32 temporary)
+    gdt = lambda t: torch.float32 if (isinstance(t, torch.Tensor) and t.dtype == torch.float32) else io
+    _require(grad_q, "grad_q", (N, H, L, E), gdt(grad_q))
+    _require(grad_k, "grad_k", (N, H, L, E), gdt(grad_k))
+    _require(grad_v, "grad_v", (N, H, L, M), gdt(grad_v))
+    _require(grad_beta, "grad_beta", (N, H, L, 1), gdt(grad_beta))
     if grad_kv is not None:
         _require(grad_kv, "grad_kv", (N, H, E, M))
     if q.numel() == 0 or v.numel() == 0:
@@ -273,10 +276,11 @@ def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, g
     (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr), (gos, gstr) = (
         _strided(t) for t in (q, k, v, beta, grad_out))
     if io == torch.bfloat16:
-        # sums over the value axis come back in fp32 and are rounded here
-        bf_outs = (grad_q, grad_k, grad_beta)
-        grad_q, grad_k, grad_beta = (torch.empty(t.shape, device=t.device, dtype=torch.float32)
-                                     for t in bf_outs)
+        # the library returns every gradient in fp32; bf16 destinations are rounded here
+        bf_outs = (grad_q, grad_k, grad_v, grad_beta)
+        grad_q, grad_k, grad_v, grad_beta = (
+            t if t.dtype == torch.float32 else torch.empty(t.shape, device=t.device, dtype=torch.float32)
+            for t in bf_outs)
     outs = [kv, grad_q, grad_k, grad_v, grad_beta] + ([grad_kv] if grad_kv is not None else [])
     with torch.cuda.device(q.device), _Dense([v_old, v_insert], False) as sv, _Dense(outs, True) as d:
         gkv = _ptr(d[5]) if grad_kv is not None else ctypes.c_void_p(None)
@@ -285,5 +289,6 @@ def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, g
                   *[_ptr(t) for t in d[:5]], gkv, N, H, L, E, M, flags, _stream(q.device))
     _check(code, fn.__name__)
     if io == torch.bfloat16:
-        for dst, src in zip(bf_outs, (grad_q, grad_k, grad_beta)):
-            dst.copy_(src)
+        for dst, src in zip(bf_outs, (grad_q, grad_k, grad_v, grad_beta)):
+            if dst is not src:
+                dst.copy_(src)

@@ -219,6 +219,54 @@ def test_chunkwise_forward_matches_oracle_and_feeds_the_sequential_backward(shap
     assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
 
 
+@pytest.mark.parametrize("shape,qk,w0,io", [
+    ((2, 3, 64, 64, 64), "softmax", 0.0, torch.float32),     # exactly one chunk
+    ((2, 2, 200, 64, 64), "softmax", 0.3, torch.float32),    # ragged last chunk, non-zero memory
+    ((1, 3, 256, 128, 128), "l2", 0.0, torch.float32),       # two workgroups per sequence, row sweep in chunks of 32
+    ((1, 2, 37, 128, 128), "l2", 0.2, torch.float32),        # shorter than a chunk
+    ((1, 2, 1100, 128, 128), "l2", 0.0, torch.float32),      # many chunks, ragged
+    ((2, 8, 256, 64, 64), "softmax", 0.0, torch.float32),    # BASELINE config 2 style
+    ((2, 2, 300, 64, 64), "softmax", 0.2, torch.bfloat16),
+    ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # BASELINE config 5 style, shorter
+    ((1, 2, 150, 128, 128), "l2", 0.3, torch.bfloat16),
+])
+@pytest.mark.parametrize("state_grad", [False, True])
+def test_chunkwise_backward_matches_oracle(shape, qk, w0, io, state_grad):
+    """Chunkwise backward (column sweep + row sweep on the matrix cores) vs the fp64 oracle, fed by
+    the step-by-step forward; with and without an incoming gradient of the final memory."""
+    print(f"case chunkwise backward shape={shape} io={io} state_grad={state_grad}", flush=True)
+    import srwm_hip
+    dev = _dev()
+    tol = TOL if io == torch.float32 else BF16_TOL
+    q, k, v, beta, W0, go = delta_inputs(*shape, seed=17, qk=qk, w0_std=w0)
+    qi, ki, vi, bi, goi = (t.to(io) for t in (q, k, v, beta, go))
+    base = [t.to(torch.float64).numpy() for t in (qi, ki, vi, bi)] + [W0.numpy()]
+    gs = torch.randn(W0.shape, generator=torch.Generator().manual_seed(5), dtype=torch.float64) if state_grad else None
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, goi.to(torch.float64).numpy(),
+                               grad_state=None if gs is None else gs.numpy(), want_grad_W=True)
+    N, H, L, E = q.shape
+    qd, kd, vd, bd, god = (t.to(dev) for t in (qi, ki, vi, bi, goi))
+    W = W0.to(dev, torch.float32).contiguous()
+    nan = lambda *s_: torch.full(s_, float("nan"), device=dev)
+    vold, vins = nan(N, H, L, E), nan(N, H, L, E)
+    out = torch.empty(N, H, L, E, device=dev, dtype=io)
+    srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out)
+    gq, gk, gv, gb = nan(N, H, L, E), nan(N, H, L, E), nan(N, H, L, E), nan(N, H, L, 1)
+    if gs is None:
+        gW, mode = nan(N, H, E, E), srwm_hip.GRAD_STATE_ZERO
+    else:
+        gW, mode = gs.to(dev, torch.float32).contiguous(), srwm_hip.GRAD_STATE_IN
+    srwm_hip.fast_weight_backward(qd, kd, vd, bd, vold, vins, god, W, gq, gk, gv, gb, grad_kv=gW,
+                                  flags=srwm_hip.FLAG_CHUNKWISE | mode)
+    torch.cuda.synchronize()
+    errs = {n: rel_err(t.cpu().numpy(), ob[n]) for n, t in
+            (("grad_Q", gq), ("grad_K", gk), ("grad_V", gv), ("grad_beta", gb), ("grad_W", gW))}
+    errs["W0"] = float(np.abs(W.cpu().numpy() - W0.numpy()).max() / max(1e-30, np.abs(of["W"]).max()))
+    bad = {n: e for n, e in errs.items() if not (e < tol)}
+    assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
+
+
 def test_full_config5_properties():
     """BASELINE config 5 at full size (N=8, H=16, L=4096, E=M=128, bf16 I/O, fp32 memory):
     the step-by-step and the chunkwise forward agree with each other, the backward reverts the

@@ -130,3 +130,21 @@ def test_chunkwise_form_equals_the_sequential_recurrence(chunk, blocked):
     ch = delta_forward_chunkwise(*base, chunk=chunk, blocked=blocked)
     for n in ("out", "v_old", "v_insert", "W"):
         assert rel_err(ch[n], seq[n]) < 1e-11, n
+
+
+@pytest.mark.parametrize("chunks", [(1, 1), (5, 7), (16, 32), (64, 32), (64, 64), (1000, 1000)])
+@pytest.mark.parametrize("blocked", [False, True])
+def test_chunkwise_backward_equals_the_sequential_reverse_sweep(chunks, blocked):
+    """The chunkwise backward (column sweep + row sweep, any pair of chunk sizes, both
+    triangular solvers) must reproduce the per-step oracle, including the gradient of the
+    initial memory and an incoming gradient of the final one."""
+    from oracle.chunkwise import delta_backward_chunkwise
+    q, k, v, beta, W0, go = delta_inputs(2, 2, 150, 12, 10, seed=10, qk="l2", w0_std=0.3)
+    gs = np.random.default_rng(3).standard_normal(W0.shape)
+    base = _np((q, k, v, beta, W0))
+    f = oracle.delta_forward(*base)
+    seq = oracle.delta_backward(*base[:4], f, go.numpy(), grad_state=gs)
+    ch = delta_backward_chunkwise(*base[:4], f, go.numpy(), grad_state=gs, chunk_col=chunks[0],
+                                  chunk_row=chunks[1], blocked=blocked)
+    for n in ("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W", "W0"):
+        assert rel_err(ch[n], seq[n]) < 1e-10, n
