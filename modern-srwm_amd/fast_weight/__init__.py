@@ -14,18 +14,23 @@ import torch
 
 import srwm_hip
 
-# Forward kernel choice: "auto" runs the chunkwise (chunk = 64) matrix-core kernel when it
-# exists for the shape (E == M in {64, 128}, at least one full chunk) and the step-by-step kernel
-# otherwise; True / False force one of them.  Both emit the same v_old / v_insert, so the
-# backward (always the step-by-step reverse sweep) is unaffected.
+# Kernel choice: "auto" runs the chunkwise matrix-core kernels when they exist for the shape
+# (E == M in {64, 128}, at least one full chunk of 64 steps) and the step-by-step kernels
+# otherwise; True / False force one of them.  The two forms emit and consume the same v_old /
+# v_insert, so forward and backward can be chosen independently.
 CHUNKWISE_FORWARD = "auto"
+CHUNKWISE_BACKWARD = "auto"
+
+
+def _chunk_flags(choice, E, M, L):
+    has_kernel = E == M and E in (64, 128)
+    if choice is True or (choice == "auto" and has_kernel and L >= 64):
+        return srwm_hip.FLAG_CHUNKWISE
+    return 0
 
 
 def _forward_flags(E, M, L):
-    has_kernel = E == M and E in (64, 128)
-    if CHUNKWISE_FORWARD is True or (CHUNKWISE_FORWARD == "auto" and has_kernel and L >= 64):
-        return srwm_hip.FLAG_CHUNKWISE
-    return 0
+    return _chunk_flags(CHUNKWISE_FORWARD, E, M, L)
 
 
 def causal_dot_product_cuda(q, k, v, beta, v_old, v_insert, kv, out):
@@ -33,7 +38,10 @@ def causal_dot_product_cuda(q, k, v, beta, v_old, v_insert, kv, out):
                                  flags=_forward_flags(q.shape[-1], v.shape[-1], q.shape[2]))
 
 
-causal_dot_backward_cuda = srwm_hip.fast_weight_backward
+def causal_dot_backward_cuda(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v, grad_beta):
+    srwm_hip.fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v,
+                                  grad_beta,
+                                  flags=_chunk_flags(CHUNKWISE_BACKWARD, q.shape[-1], v.shape[-1], q.shape[2]))
 
 
 class DeltaFastWeight(torch.autograd.Function):

@@ -121,6 +121,32 @@ def test_autograd_function_drop_in_with_layer_style_views():
     assert W.abs().max().item() < 1e-5 * WL.abs().max().item()
 
 
+@pytest.mark.parametrize("chunkwise", [False, True, "auto"])
+def test_autograd_function_with_either_kernel_family(chunkwise):
+    """The operator gives the same results whichever kernels it is told to use."""
+    print(f"case autograd op, chunkwise={chunkwise}", flush=True)
+    import fast_weight
+    from oracle.recurrence import delta_recurrence
+    dev = _dev()
+    q, k, v, beta, W0, go = delta_inputs(2, 2, 130, 64, 64, seed=23, w0_std=0.1)
+    ref = [t.clone().requires_grad_(True) for t in (q, k, v, beta)]
+    ref_out, _ = delta_recurrence(*ref, W0.clone())
+    (ref_out * go).sum().backward()
+    old = fast_weight.CHUNKWISE_FORWARD, fast_weight.CHUNKWISE_BACKWARD
+    fast_weight.CHUNKWISE_FORWARD = fast_weight.CHUNKWISE_BACKWARD = chunkwise
+    try:
+        leaves = [t.to(dev, torch.float32).requires_grad_(True) for t in (q, k, v, beta)]
+        W = W0.to(dev, torch.float32).contiguous()
+        out = fast_weight.fast_weight_delta(*leaves, W)
+        (out * go.to(dev, torch.float32)).sum().backward()
+    finally:
+        fast_weight.CHUNKWISE_FORWARD, fast_weight.CHUNKWISE_BACKWARD = old
+    assert rel_err(out.detach().cpu().numpy(), ref_out.detach().numpy()) < TOL
+    for a, b in zip(leaves, ref):
+        assert rel_err(a.grad.cpu().numpy(), b.grad.numpy()) < TOL
+    assert rel_err(W.cpu().numpy(), W0.numpy()) < TOL          # reverted to the initial memory
+
+
 def test_full_config2_properties():
     """BASELINE config 2 at full size: finite outputs, revert-to-W0 round trip, linearity in
     grad_out, oracle on a sample of sequences."""
@@ -292,10 +318,19 @@ def test_full_config5_properties():
         < 1e-2 * res["chunk"]["out"].float().abs().max().item()
     r = res["chunk"]
     WL = r["W"].clone()
-    gq, gk, gv, gb = new(E, torch.bfloat16), new(E, torch.bfloat16), new(E, torch.bfloat16), new(1, torch.bfloat16)
-    srwm_hip.fast_weight_backward(qd, kd, vd, bd, r["v_old"], r["v_insert"], god, r["W"], gq, gk, gv, gb)
+    f32 = torch.float32
+    gq, gk, gv, gb = new(E, f32), new(E, f32), new(E, f32), new(1, f32)
+    srwm_hip.fast_weight_backward(qd, kd, vd, bd, r["v_old"], r["v_insert"], god, r["W"], gq, gk, gv, gb,
+                                  flags=srwm_hip.FLAG_CHUNKWISE)
     torch.cuda.synchronize()
     assert r["W"].abs().max().item() < 1e-4 * WL.abs().max().item()        # reverted to W_0 = 0
+    # the step-by-step backward on the same saved vectors agrees with the chunkwise one
+    W2 = WL.clone()
+    sq, sk, sv, sb = new(E, f32), new(E, f32), new(E, f32), new(1, f32)
+    srwm_hip.fast_weight_backward(qd, kd, vd, bd, r["v_old"], r["v_insert"], god, W2, sq, sk, sv, sb)
+    for a, b, n in ((gq, sq, "grad_Q"), (gk, sk, "grad_K"), (gv, sv, "grad_V"), (gb, sb, "grad_beta")):
+        assert torch.isfinite(a).all(), n
+        assert (a - b).abs().max().item() < 2e-3 * b.abs().max().item(), n
     for (n_, h_) in ((0, 0), (7, 15)):
         sl = (slice(n_, n_ + 1), slice(h_, h_ + 1))
         base = [t[sl].float().cpu().to(torch.float64).numpy() for t in (qd, kd, vd, bd)] + [W0[sl].double().numpy()]
