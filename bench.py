@@ -34,13 +34,14 @@ HBM_PEAK_GBS = 8000.0
 
 # HBM bytes per launch of the dominant (backward) kernel, measured with rocprofv3 --pmc FETCH_SIZE and
 # --pmc WRITE_SIZE (two runs; FETCH_SIZE scaled by the factor that makes a plain copy of known size
-# read its size).  Figures and commands: profiles/srwm_c4_kernels.txt, profiles/delta_kernels.txt.
+# read its size).  Figures and commands: profiles/srwm_c4_kernels.txt, profiles/delta_kernels.txt,
+# profiles/delta_chunk_kernels.txt (backward kernels of the workload: fetch + write).
 MEASURED_TRAFFIC_BYTES = {
     "srwm_c4": (490477 + 90624) * 1024,
     "delta_c2": (102444 + 53504) * 1024,
-    "delta_c2_chunk": (102444 + 53504) * 1024,
-    "delta_c5": (1316488 + 1191936) * 1024,
-    "delta_c5_chunk": (1316488 + 1191936) * 1024,
+    "delta_c2_chunk": (82217 + 85992 + 16640 + 36864) * 1024,
+    "delta_c5": (1316522 + 1323008) * 1024,
+    "delta_c5_chunk": (1047345 + 1575915 + 266240 + 532480) * 1024,
 }
 
 WORKLOADS = {

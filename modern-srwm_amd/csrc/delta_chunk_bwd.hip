@@ -459,8 +459,10 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
                 [&](int cb) { return nkb[cb]; }, st[mb]);
             nstb[mb] = X::accb(-st[mb]);   // -S (entry value)
         }
-        __syncthreads();   // G1 and Z are visible
+        // ---- G1 and Z become visible
+        __syncthreads();
 
+        // ---- grad_Q = dOut S^T + G1 K,  grad_K = G1^T Q + U dS'^T - Y S^T - Z K
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
             const auto fns = [&](int mb) { return nstb[mb]; };
