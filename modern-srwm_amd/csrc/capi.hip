@@ -44,7 +44,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 1; }
+int srwm_hip_abi_version(void) { return 2; }
 
 const char *srwm_hip_strerror(int code) {
     switch (code) {

@@ -31,7 +31,7 @@ GRAD_STATE_ACCUM = 2
 FLAG_GENERIC = 16
 FLAG_CHUNKWISE = 32     # delta forward: chunkwise MFMA kernel (E == M in {64, 128})
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lib = None
 
