@@ -93,6 +93,38 @@ SRWM_API int srwm_backward_f32(const float *x, const int64_t x_strides[3],
                       int N, int H, int L, int E, unsigned flags, void *stream);
 
 /*
+ * SRWM forward over all steps of an unroll with per-step resets.  No counterpart function in the
+ * reference: it fuses the loop in which its RL learner calls the L = 1 operator once per time
+ * step, multiplying the carried shift by `notdone` first (reinforcement_learning/
+ * torchbeast_procgen/model.py:1176-1196, torchbeast/layer.py:377-421).  Same contract as
+ * srwm_forward_f32, plus
+ *   keep     dense [N,L] (or NULL = never reset): where keep[n][t] == 0 the state of batch row n
+ *            is replaced, before step t, by the shared weights of its head
+ *   sW_y, sW_q, sW_k  dense [H,E,E];  sw_b dense [H,E,4]   (the layer's parameters)
+ */
+SRWM_API int srwm_forward_steps_f32(const float *x, const int64_t x_strides[3], const float *keep,
+                           const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
+                           float *W_y, float *W_q, float *W_k, float *w_b,
+                           float *q, float *k, float *beta,
+                           float *y_diff, float *q_diff, float *k_diff, float *beta_diff,
+                           float *out, int N, int H, int L, int E, unsigned flags, void *stream);
+
+/*
+ * Gradient of that unroll with respect to x when the carried state is detached between steps
+ * (what the per-step calls of the reference compute, layer.py:412-418: the new state is
+ * `.detach()`-ed): grad_x[n][h][t] = W_y,t-1 grad_out[n][h][t], with W_y replayed forward from
+ * W_y_entry (the [N,H,E,E] tensor handed to srwm_forward_steps_f32, before that call) through
+ * the saved k, beta, y_diff and the same resets.  The gradient of the shared W_y is
+ * sum over n, t of x (x) grad_out, which the caller forms with a batched matrix product; the
+ * other shared weights receive no gradient in this regime.
+ */
+SRWM_API int srwm_readout_grad_f32(const float *k, const float *beta, const float *y_diff,
+                          const float *keep, const float *sW_y,
+                          const float *grad_out, const int64_t grad_out_strides[3],
+                          const float *W_y_entry, float *grad_x,
+                          int N, int H, int L, int E, unsigned flags, void *stream);
+
+/*
  * Delta-rule forward.  Replaces fast_weight_forward(), supervised_learning/
  * fast_weight/fast_weight_cuda.cu:182-240 (kernel :17-178).  Per sequence, W is E x M:
  *     v_old = W^T k_t;  ins = beta_t (v_t - v_old);  W += k_t (x) ins;  out_t = W^T q_t

@@ -88,6 +88,40 @@ int srwm_forward_f32(const float *x, const int64_t xs[3], float *Wy, float *Wq, 
     return launch_srwm_fwd_generic(p, s);
 }
 
+int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
+                           const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
+                           float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
+                           float *qdiff, float *kdiff, float *bdiff, float *out, int N, int H, int L,
+                           int E, unsigned flags, void *stream) {
+    if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
+        !out || !xs)
+        return SRWM_EINVAL;
+    if (keep && (!sWy || !sWq || !sWk || !swb)) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || (flags & ~(SRWM_FLAG_GENERIC))) return SRWM_EINVAL;
+    if (!stride_ok(xs, N, H, L, E)) return SRWM_ESTRIDE;
+    SrwmFwdParams p{x, xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff,
+                    out, N, H, L, E, keep, sWy, sWq, sWk, swb};
+    hipStream_t s = (hipStream_t)stream;
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_srwm_fwd_tiled(p, s);
+        if (r >= 0) return r;
+    }
+    if (srwm_fwd_generic_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
+    return launch_srwm_fwd_generic(p, s);
+}
+
+int srwm_readout_grad_f32(const float *k, const float *beta, const float *ydiff, const float *keep,
+                          const float *sWy, const float *grad_out, const int64_t gs[3],
+                          const float *Wy_entry, float *grad_x, int N, int H, int L, int E,
+                          unsigned flags, void *stream) {
+    if (!k || !beta || !ydiff || !grad_out || !gs || !Wy_entry || !grad_x || (keep && !sWy)) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || flags) return SRWM_EINVAL;
+    if (!stride_ok(gs, N, H, L, E)) return SRWM_ESTRIDE;
+    if (srwm_readout_grad_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
+    SrwmReadoutGradParams p{k, beta, ydiff, keep, grad_out, gs[0], gs[1], gs[2], Wy_entry, sWy, grad_x, N, H, L, E};
+    return launch_srwm_readout_grad(p, (hipStream_t)stream);
+}
+
 int srwm_backward_f32(const float *x, const int64_t xs[3], const float *q, const float *k,
                       const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
                       const float *bdiff, const float *grad_out, const int64_t gs[3], const float *Wy,

@@ -15,6 +15,22 @@ struct SrwmFwdParams {
     float *Wy, *Wq, *Wk, *wb;
     float *q, *k, *beta, *ydiff, *qdiff, *kdiff, *bdiff, *out;
     int N, H, L, E;
+    // optional per-step reset: before step t of batch row n the state is replaced by the shared
+    // weights of its head wherever keep[n*L + t] == 0 (keep == nullptr: never)
+    const float *keep;
+    const float *sWy, *sWq, *sWk, *swb;   // [H,E,E] x 3, [H,E,4]
+};
+
+// Gradient of the readout alone, for callers that detach the carried state between steps:
+// grad_x_t = W_y,t-1 grad_out_t with W_y replayed from its entry value and the saved k, beta_y, y_diff.
+struct SrwmReadoutGradParams {
+    const float *k, *beta, *ydiff, *keep;
+    const float *go;
+    int64_t gs_n, gs_h, gs_l;
+    const float *Wy0;    // [N,H,E,E] y block before step 0
+    const float *sWy;    // [H,E,E], used where keep == 0 (may be nullptr when keep is)
+    float *gx;
+    int N, H, L, E;
 };
 
 struct SrwmBwdParams {
@@ -91,6 +107,8 @@ size_t srwm_bwd_generic_lds_bytes(int E);
 size_t delta_fwd_generic_lds_bytes(int E, int M);
 size_t delta_bwd_generic_lds_bytes(int E, int M);
 int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s);
+size_t srwm_readout_grad_lds_bytes(int E);
+int launch_srwm_readout_grad(const SrwmReadoutGradParams &p, hipStream_t s);
 int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s);
 int launch_delta_fwd_generic(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_bwd_generic(const DeltaBwdParams &p, hipStream_t s);

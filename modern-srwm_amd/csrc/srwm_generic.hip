@@ -49,6 +49,10 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
     for (int t = 0; t < p.L; ++t) {
         const float *xt = p.x + n * p.xs_n + h * p.xs_h + t * p.xs_l;
         const int64_t o = (seq * p.L + t) * E, ob = (seq * p.L + t) * 4;
+        if (p.keep && p.keep[(int64_t)n * p.L + t] == 0.f) {   // uniform: per-step reset to the shared weights
+            load_state(W, Cp, p.sWy + (int64_t)h * E * E, p.sWq + (int64_t)h * E * E, p.sWk + (int64_t)h * E * E,
+                       p.swb + (int64_t)h * E * 4, E, tid);
+        }
         for (int e = tid; e < E; e += kThreads) xs[e] = xt[e];
         __syncthreads();
         // main readout: pre = W^T x

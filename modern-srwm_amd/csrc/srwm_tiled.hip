@@ -74,6 +74,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     constexpr int RG = T::RG, CGW = T::CGW, CB = T::CB, NC = T::NC, TT = T::TT;
 
     __shared__ __attribute__((aligned(16))) float xt[2][TT][E];   // input tiles, double buffered
+    __shared__ float kt[2][TT];                                   // keep flags of the tile's steps
     __shared__ __attribute__((aligned(16))) float raw[2][2][E];   // q~ | k~ of the step, by parity
     __shared__ float rawb[2][4];                                  // b~
     __shared__ __attribute__((aligned(16))) float exch[NW][2][E]; // per wave: q-k | k
@@ -101,6 +102,17 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
                 for (int c = 0; c < CB; ++c) w[i][b * CB + c] = src[b][(r0 + i) * E + c0 + c];
     }
     float wbe = has_b ? p.wb[sE4 + el * 4 + jb] : 0.f;
+    // replaces the state by the weights all batch rows of this head share (per-step reset)
+    auto reset_state = [&]() {
+        const float *src[3] = {p.sWy + (int64_t)h * E * E, p.sWq + (int64_t)h * E * E, p.sWk + (int64_t)h * E * E};
+#pragma unroll
+        for (int b = 0; b < 3; ++b)
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < CB; ++c) w[i][b * CB + c] = src[b][(r0 + i) * E + c0 + c];
+        wbe = has_b ? p.swb[(int64_t)h * E * 4 + el * 4 + jb] : 0.f;
+    };
 
     // tile loader: thread -> (step tid / (E/4), 4 consecutive elements)
     const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
@@ -108,19 +120,28 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         const int t = min(tile * TT + ld_row, p.L - 1);  // rows past the end: loaded, never used
         return *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col);
     };
+    auto load_keep = [&](int tile) -> float {
+        return (p.keep && tid < TT) ? p.keep[(int64_t)n * p.L + min(tile * TT + tid, p.L - 1)] : 1.f;
+    };
     const int ntiles = (p.L + TT - 1) / TT;
     *reinterpret_cast<float4 *>(&xt[0][ld_row][ld_col]) = load_tile(0);
+    if (tid < TT) kt[0][tid] = load_keep(0);
     __syncthreads();
 
     for (int tile = 0; tile < ntiles; ++tile) {
         const int buf = tile & 1;
         const int tlen = min(TT, p.L - tile * TT);
         float4 xnext = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (tile + 1 < ntiles) xnext = load_tile(tile + 1);
+        float knext = 1.f;
+        if (tile + 1 < ntiles) {
+            xnext = load_tile(tile + 1);
+            knext = load_keep(tile + 1);
+        }
 
         for (int tt = 0; tt < tlen; ++tt) {
             const int t = tile * TT + tt, par = t & 1;
             const int64_t o = (seq * p.L + t) * E, ob = (seq * p.L + t) * 4;
+            if (p.keep && kt[buf][tt] == 0.f) reset_state();   // uniform over the workgroup
 
             // ---- main readout: [y | q~ | k~ | b~] = W^T x_t
             float xr[R];
@@ -141,8 +162,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
                 store_vec<CB>(&raw[par][1][c0], &acc[2 * CB]);
             }
             if (has_b && el == 0) rawb[par][jb] = pb;
-            if (tt == tlen - 1 && tile + 1 < ntiles)
+            if (tt == tlen - 1 && tile + 1 < ntiles) {
                 *reinterpret_cast<float4 *>(&xt[buf ^ 1][ld_row][ld_col]) = xnext;
+                if (tid < TT) kt[buf ^ 1][tid] = knext;
+            }
             __syncthreads();
 
             // ---- activations, redundantly in every wave, lane <-> element el

@@ -17,7 +17,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from fast_weight import fast_weight_delta
-from self_ref_v0 import self_ref_v0, stateful_self_ref_v0
+from self_ref_v0 import self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
 
 
 def elu_p1(x):
@@ -122,6 +122,20 @@ class SRlayer(_SRBase):
         out = h + self._project(out, bsz, slen)
         new_state = tuple((f.detach() - w.repeat(bsz, 1, 1, 1)).detach()
                           for f, w in zip(fast, self._slow()))
+        return out, new_state
+
+    def forward_steps(self, h, notdone, state):
+        """The whole unroll at once: equivalent to calling forward() once per time step on
+        h[t:t+1] with the carried state multiplied by notdone[t] first (what the learner's loop
+        does, reinforcement_learning/torchbeast_procgen/model.py:1176-1196), in one kernel launch
+        forward and one backward.  h: (T, B, H*d); notdone: (T, B), 0 where an episode ended."""
+        assert state is not None
+        x, slen, bsz = self._split(h, True)
+        keep = notdone.to(h.dtype).transpose(0, 1).contiguous()            # (B, T)
+        fast = [s.detach() + w.detach().repeat(bsz, 1, 1, 1) for s, w in zip(state, self._slow())]
+        out = self_ref_v0_steps(x, keep, *fast, *self._slow())
+        out = h + self._project(out, bsz, slen)
+        new_state = tuple(f - w.detach().repeat(bsz, 1, 1, 1) for f, w in zip(fast, self._slow()))
         return out, new_state
 
 

@@ -5,6 +5,8 @@ same call signatures, same in-place final-state semantics -- backed by libsrwm_h
     out = self_ref_v0(x, W_y, W_q, W_k, w_b)
     out, W_y, W_q, W_k, w_b = stateful_self_ref_v0(x, W_y, W_q, W_k, w_b)
 
+    out = self_ref_v0_steps(x, keep, W_y, W_q, W_k, w_b, sW_y, sW_q, sW_k, sw_b)   # see SelfRefv0Steps
+
 x: (N, H, L, E); W_y, W_q, W_k: (N, H, E, E); w_b: (N, H, E, 4); float32 on the GPU.
 The weight tensors are OVERWRITTEN with the state after the last step (the layers read
 them back as the carried state); the backward starts from that mutated tensor.
@@ -99,3 +101,49 @@ class StatefulSelfRefv0(torch.autograd.Function):
 # Alias the autograd functions to python style snake case naming
 self_ref_v0 = SelfRefv0.apply
 stateful_self_ref_v0 = StatefulSelfRefv0.apply
+
+
+class SelfRefv0Steps(torch.autograd.Function):
+    """All time steps of an RL unroll in one launch, with the semantics of calling `self_ref_v0`
+    once per step on `carried shift (detached) + shared weights`, the shift zeroed where an
+    episode ended (reinforcement_learning/torchbeast_procgen/model.py:1176-1196,
+    torchbeast/layer.py:377-421).
+
+        out = self_ref_v0_steps(x, keep, W_y, W_q, W_k, w_b, sW_y, sW_q, sW_k, sw_b)
+
+    x: (N, H, L, E); keep: (N, L) float, 0 where the state is reset before the step (None: never);
+    W_*: (N, H, E, .) weights at entry (shift + shared), OVERWRITTEN with the weights after the
+    last step; sW_*: (1, H, E, .) shared weights (the layer's parameters).
+    Gradients are those of the per-step calls: the carried state is detached, so grad_x_t =
+    W_y,t-1 grad_out_t, the shared W_y receives sum_t x_t (x) grad_out_t and the other shared
+    weights receive zeros.
+    """
+
+    @staticmethod
+    def forward(ctx, x, keep, W_y, W_q, W_k, w_b, sW_y, sW_q, sW_k, sw_b):
+        for t in (x, W_y, W_q, W_k, w_b):
+            assert t.device.type != "cpu"
+        N, H, L, E = _check_shapes(x, W_y, W_q, W_k, w_b)
+        device = x.device
+        big = lambda: torch.empty((N, H, L, E), device=device, dtype=x.dtype)
+        small = lambda: torch.empty((N, H, L, 4), device=device, dtype=x.dtype)
+        out, q_main, k_main, beta_main = big(), big(), big(), small()
+        y_diff, q_diff, k_diff, beta_diff = big(), big(), big(), small()
+        W_y_entry = W_y.detach().clone()
+        srwm_hip.self_ref_forward_steps(x.data, keep, (sW_y, sW_q, sW_k, sw_b), W_y.data, W_q.data, W_k.data,
+                                        w_b.data, q_main, k_main, beta_main, y_diff, q_diff, k_diff,
+                                        beta_diff, out)
+        ctx.save_for_backward(x, keep, k_main, beta_main, y_diff, W_y_entry, sW_y, sW_q, sW_k, sw_b)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, keep, k, beta, y_diff, W_y_entry, sW_y, sW_q, sW_k, sw_b = ctx.saved_tensors
+        grad_x = torch.empty_like(x)
+        srwm_hip.self_ref_readout_grad(k, beta, y_diff, keep, sW_y, grad_out, W_y_entry, grad_x)
+        g_sWy = torch.einsum("nhle,nhlm->hem", x, grad_out).reshape(sW_y.shape)
+        return (grad_x, None, None, None, None, None,
+                g_sWy, torch.zeros_like(sW_q), torch.zeros_like(sW_k), torch.zeros_like(sw_b))
+
+
+self_ref_v0_steps = SelfRefv0Steps.apply

@@ -42,6 +42,8 @@ _U = ctypes.c_uint
 
 _SIGNATURES = {
     "srwm_forward_f32": [_F, _S] + [_F] * 12 + [_I] * 4 + [_U, ctypes.c_void_p],
+    "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
+    "srwm_readout_grad_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
     "delta_forward_f32": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_backward_f32": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -171,6 +173,73 @@ def self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, 
         code = lib().srwm_forward_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
                                       _stream(x.device))
     _check(code, "srwm_forward_f32")
+
+
+def self_ref_forward_steps(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff,
+                           beta_diff, out, flags=0):
+    """SRWM forward over all steps of an unroll with per-step resets: where keep[n, t] == 0 the
+    state of batch row n is replaced, before step t, by the shared weights `slow` = (W_y, W_q,
+    W_k: (1 or no batch axis, H, E, E), w_b: (..., H, E, 4)).  keep: (N, L) float32 or None.
+    Otherwise as self_ref_forward."""
+    _require(x, "x")
+    N, H, L, E = x.shape
+    for t, nm in ((W_y, "W_y"), (W_q, "W_q"), (W_k, "W_k")):
+        _require(t, nm, (N, H, E, E))
+    _require(w_b, "w_b", (N, H, E, 4))
+    for t, nm in ((q, "q"), (k, "k"), (y_diff, "y_diff"), (q_diff, "q_diff"), (k_diff, "k_diff"),
+                  (out, "out")):
+        _require(t, nm, (N, H, L, E))
+    _require(beta, "beta", (N, H, L, 4))
+    _require(beta_diff, "beta_diff", (N, H, L, 4))
+    null = ctypes.c_void_p(None)
+    sl = [null] * 4
+    if keep is not None:
+        _require(keep, "keep", (N, L))
+        keep = keep.contiguous()
+        shapes = ((H, E, E),) * 3 + ((H, E, 4),)
+        sl = []
+        for t, shp, nm in zip(slow, shapes, ("slow W_y", "slow W_q", "slow W_k", "slow w_b")):
+            t = t.detach().reshape(shp) if isinstance(t, torch.Tensor) and t.numel() == H * E * shp[-1] else t
+            _require(t, nm, shp)
+            sl.append(t.contiguous())
+    if x.numel() == 0:
+        return
+    xs, xstr = _strided(x)
+    with torch.cuda.device(x.device), \
+            _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out], True) as d:
+        code = lib().srwm_forward_steps_f32(
+            _ptr(xs), xstr, _ptr(keep) if keep is not None else null,
+            *[(_ptr(t) if keep is not None else t) for t in sl],
+            *[_ptr(t) for t in d], N, H, L, E, flags, _stream(x.device))
+    _check(code, "srwm_forward_steps_f32")
+
+
+def self_ref_readout_grad(k, beta, y_diff, keep, slow_W_y, grad_out, W_y_entry, grad_x):
+    """grad_x[n, h, t] = W_y,t-1 grad_out[n, h, t] for an unroll whose carried state is detached
+    between steps; W_y_entry is the (N, H, E, E) y block as it was before self_ref_forward_steps."""
+    _require(k, "k")
+    N, H, L, E = k.shape
+    _require(beta, "beta", (N, H, L, 4))
+    _require(y_diff, "y_diff", (N, H, L, E))
+    _require(grad_out, "grad_out", (N, H, L, E))
+    _require(W_y_entry, "W_y_entry", (N, H, E, E))
+    _require(grad_x, "grad_x", (N, H, L, E))
+    null = ctypes.c_void_p(None)
+    if keep is not None:
+        _require(keep, "keep", (N, L))
+        keep = keep.contiguous()
+        slow_W_y = slow_W_y.detach().reshape(H, E, E).contiguous()
+        _require(slow_W_y, "slow W_y", (H, E, E))
+    if k.numel() == 0:
+        return
+    gos, gstr = _strided(grad_out)
+    with torch.cuda.device(k.device), _Dense([k, beta, y_diff, W_y_entry], False) as sv, \
+            _Dense([grad_x], True) as gr:
+        code = lib().srwm_readout_grad_f32(
+            _ptr(sv[0]), _ptr(sv[1]), _ptr(sv[2]), _ptr(keep) if keep is not None else null,
+            _ptr(slow_W_y) if keep is not None else null, _ptr(gos), gstr, _ptr(sv[3]), _ptr(gr[0]),
+            N, H, L, E, 0, _stream(k.device))
+    _check(code, "srwm_readout_grad_f32")
 
 
 def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out,

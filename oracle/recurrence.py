@@ -67,3 +67,23 @@ def delta_recurrence(Q, K, V, beta, W0):
         outs.append(torch.bmm(W, qs[t].unsqueeze(2)).squeeze(2))
     out = torch.stack(outs).view(L, N, H, M).permute(1, 2, 0, 3)
     return out, W.transpose(1, 2).reshape(N, H, E, M)
+
+
+def srwm_steps_reference(x, keep, shift, slow):
+    """The RL learner's call pattern, literally (reinforcement_learning/torchbeast_procgen/
+    model.py:1176-1196 with torchbeast/layer.py:377-421): one L = 1 call of the recurrence per time
+    step on `shift * keep_t + shared weights`, the new shift DETACHED after every step.
+    x: (N, H, L, E); keep: (N, L) or None; shift: 4 tensors (N, H, E, .); slow: 4 tensors (1, H, E, .).
+    Returns (out (N, H, L, E), final shift (4 tensors))."""
+    N, H, L, E = x.shape
+    outs = []
+    shift = [s.detach() for s in shift]
+    for t in range(L):
+        if keep is not None:
+            kt = keep[:, t].reshape(N, 1, 1, 1)
+            shift = [s * kt for s in shift]
+        W = [s + w.repeat(N, 1, 1, 1) for s, w in zip(shift, slow)]
+        out, final = srwm_recurrence(x[:, :, t:t + 1], *W)
+        outs.append(out)
+        shift = [(f.detach() - w.repeat(N, 1, 1, 1)).detach() for f, w in zip(final, slow)]
+    return torch.cat(outs, dim=2), shift

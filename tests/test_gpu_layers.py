@@ -158,3 +158,45 @@ def test_state_dict_names_match_the_reference_layers():
     assert sd["W_y"].shape == (1, 2, 8, 8) and sd["w_b"].shape == (1, 2, 8, 4)
     assert {"slow_net.weight", "layer_norm.weight", "layer_norm.bias", "out_linear.weight"} == \
         set(FastFFlayer(2, 8, 16, 0.0).state_dict())
+
+
+def test_rl_sr_layer_whole_unroll_equals_the_per_step_loop():
+    """SRlayer.forward_steps (one launch) vs the learner's loop: state * notdone, then forward on
+    one time step, for every step -- outputs, carried state and parameter gradients."""
+    print("case SRlayer.forward_steps", flush=True)
+    from layer import SRlayer
+    dev = torch.device("cuda:0")
+    torch.manual_seed(5)
+    T, B, H, d = 23, 5, 4, 16
+    lay = SRlayer(H, d, H * d, 0.0).to(dev)
+    h = torch.randn(T, B, H * d, device=dev)
+    notdone = (torch.rand(T, B, device=dev) > 0.2).float()
+    state0 = tuple(0.1 * torch.randn(B, H, d, c, device=dev) for c in (d, d, d, 4))
+    go = torch.randn(T, B, H * d, device=dev)
+
+    hl = h.clone().requires_grad_(True)
+    outs, state = [], state0
+    for t in range(T):
+        nd = notdone[t].view(B, 1, 1, 1)
+        state = tuple(s * nd for s in state)
+        o, state = lay(hl[t:t + 1], state)
+        outs.append(o)
+    loop_out = torch.cat(outs)
+    (loop_out * go).sum().backward()
+    loop_grads = {n: p.grad.clone() for n, p in lay.named_parameters() if p.grad is not None}
+    loop_gh = hl.grad.clone()
+    lay.zero_grad()
+
+    hs = h.clone().requires_grad_(True)
+    out, new_state = lay.forward_steps(hs, notdone, state0)
+    (out * go).sum().backward()
+    scale = loop_out.abs().max().item()
+    assert (out - loop_out).abs().max().item() < 2e-5 * scale
+    for a, b in zip(new_state, state):
+        assert (a - b).abs().max().item() < 2e-5 * max(1.0, b.abs().max().item())
+    assert (hs.grad - loop_gh).abs().max().item() < 2e-5 * loop_gh.abs().max().item()
+    for n, p in lay.named_parameters():
+        if n in loop_grads:
+            ref = loop_grads[n]
+            got = p.grad if p.grad is not None else torch.zeros_like(ref)
+            assert (got - ref).abs().max().item() < 2e-5 * max(1e-6, ref.abs().max().item()), n

@@ -222,3 +222,41 @@ def test_errors_are_reported_not_swallowed():
          [torch.zeros(1, 1, 1, big, device=dev)]
     with pytest.raises(RuntimeError, match="not supported"):
         srwm_hip.self_ref_forward(xb, *Wb, *ob)
+
+
+# ---------------------------------------------------------- step-wise (RL learner) call pattern
+
+@pytest.mark.parametrize("shape,resets", [
+    ((4, 8, 100, 32), True),      # BASELINE config 3 shape (batch slice): register-resident kernel
+    ((2, 2, 37, 64), True),
+    ((3, 2, 20, 12), True),       # generic kernel
+    ((2, 3, 15, 16), False),      # keep = None
+])
+def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
+    """self_ref_v0_steps (one launch for the unroll, resets inside the kernel, gradient cut at the
+    carried state) vs the literal per-step loop in fp64."""
+    print(f"case stepwise shape={shape} resets={resets}", flush=True)
+    from oracle.recurrence import srwm_steps_reference
+    from self_ref_v0 import self_ref_v0_steps
+    from test_oracle_srwm import _steps_inputs
+    dev = _dev()
+    N, H, L, E = shape
+    x, keep, shift, slow, go = _steps_inputs(N, H, L, E, seed=41, resets=resets)
+    xr = x.clone().requires_grad_(True)
+    sr = [w.clone().requires_grad_(True) for w in slow]
+    ref_out, ref_shift = srwm_steps_reference(xr, keep, shift, sr)
+    (ref_out * go).sum().backward()
+
+    f32 = lambda t: t.to(dev, torch.float32)
+    xd = f32(x).requires_grad_(True)
+    sd = [f32(w).requires_grad_(True) for w in slow]
+    fast = [f32(s_) + f32(w).repeat(N, 1, 1, 1) for s_, w in zip(shift, slow)]
+    out = self_ref_v0_steps(xd, None if keep is None else f32(keep), *fast, *sd)
+    (out * f32(go)).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), ref_out.detach().numpy()) < TOL
+    for fw_, rs, w in zip(fast, ref_shift, slow):            # the weights after the last step
+        assert rel_err(fw_.cpu().numpy(), (rs + w).numpy()) < TOL
+    assert rel_err(xd.grad.cpu().numpy(), xr.grad.numpy()) < TOL
+    assert rel_err(sd[0].grad.cpu().numpy(), sr[0].grad.numpy()) < TOL
+    for w in sd[1:]:
+        assert float(w.grad.abs().max()) == 0.0

@@ -210,3 +210,67 @@ def test_f32_oracle_tracks_f64():
     b32 = oracle.srwm_backward(x.numpy(), f32, go.numpy(), dtype=np.float32)
     for n in ("grad_x", "grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"):
         assert rel_err(b32[n], b64[n]) < 1e-4, n
+
+
+# ---------------------------------------------------------- step-wise (RL learner) call pattern
+
+def _steps_inputs(N, H, L, E, seed, resets=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.softmax(torch.randn(N, H, L, E, generator=g, dtype=torch.float64), -1)
+    slow = [torch.randn(1, H, E, E, generator=g, dtype=torch.float64) * 0.4 for _ in range(3)]
+    slow.append(torch.randn(1, H, E, 4, generator=g, dtype=torch.float64) * 0.4)
+    shift = [torch.randn(N, H, E, E, generator=g, dtype=torch.float64) * 0.2 for _ in range(3)]
+    shift.append(torch.randn(N, H, E, 4, generator=g, dtype=torch.float64) * 0.2)
+    keep = None
+    if resets:
+        keep = (torch.rand(N, L, generator=g) > 0.25).to(torch.float64)
+        keep[0, 0] = 0.0                        # a reset before the very first step
+        keep[-1, :] = 1.0                       # and one row without any
+    go = torch.randn(N, H, L, E, generator=g, dtype=torch.float64)
+    return x, keep, shift, slow, go
+
+
+def test_stepwise_reference_values_are_those_of_restarted_recurrences():
+    """Detaching the carried state changes no value: without resets the per-step calls reproduce
+    the single full-length recurrence, and a reset restarts it from the shared weights."""
+    from oracle.recurrence import srwm_recurrence, srwm_steps_reference
+    N, H, L, E = 3, 2, 9, 4
+    x, keep, shift, slow, _ = _steps_inputs(N, H, L, E, seed=31)
+    out, fin = srwm_steps_reference(x, None, shift, slow)
+    ref, fin_ref = srwm_recurrence(x, *[s + w for s, w in zip(shift, slow)])
+    assert rel_err(out.numpy(), ref.numpy()) < 1e-13
+    for a, b, w in zip(fin, fin_ref, slow):
+        assert rel_err((a + w).numpy(), b.numpy()) < 1e-13
+    out, fin = srwm_steps_reference(x, keep, shift, slow)
+    for n in range(N):
+        W = [s[n:n + 1] + w for s, w in zip(shift, slow)]
+        t0 = 0
+        bounds = [t for t in range(L) if keep[n, t] == 0] + [L]
+        for t1 in bounds:
+            if t1 > t0:
+                seg, W = srwm_recurrence(x[n:n + 1, :, t0:t1], *W)
+                assert rel_err(out[n:n + 1, :, t0:t1].numpy(), seg.numpy()) < 1e-13
+            W = list(slow)
+            t0 = t1
+
+
+def test_stepwise_reference_gradients_have_the_closed_form():
+    """With the state detached between steps only the readout carries gradient:
+    grad_x_t = W_y,t-1 g_t, grad of the shared W_y = sum x_t (x) g_t, nothing for W_q, W_k, w_b."""
+    from oracle.recurrence import srwm_steps_reference
+    N, H, L, E = 2, 2, 7, 4
+    x, keep, shift, slow, go = _steps_inputs(N, H, L, E, seed=32, resets=False)
+    xl = x.clone().requires_grad_(True)
+    sl = [w.clone().requires_grad_(True) for w in slow]
+    out, _ = srwm_steps_reference(xl, None, shift, sl)
+    (out * go).sum().backward()
+    assert rel_err(sl[0].grad.numpy(), torch.einsum("nhle,nhlm->hem", x, go)[None].numpy()) < 1e-13
+    for w in sl[1:]:
+        assert w.grad is None or float(w.grad.abs().max()) == 0.0
+    W0 = [(s + w).numpy() for s, w in zip(shift, slow)]
+    f = oracle.srwm_forward(x.numpy(), *W0)
+    Wy = W0[0].copy()                                    # W_y trajectory from the saved vectors
+    for t in range(L):
+        gx = np.einsum("nhem,nhm->nhe", Wy, go[:, :, t].numpy())
+        assert rel_err(xl.grad[:, :, t].numpy(), gx) < 1e-12
+        Wy = Wy + np.einsum("nhe,nhm->nhem", f["k"][:, :, t], f["beta"][:, :, t, :1] * f["y_diff"][:, :, t])
