@@ -16,7 +16,7 @@ achieved HBM rate of the operator's I/O contract.  `cpu_baseline` is the per-tim
 PyTorch recurrence (oracle/recurrence.py) timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk}.
+{srwm_c3, srwm_c3_steps, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk}.
 """
 import argparse
 import json
@@ -48,6 +48,9 @@ WORKLOADS = {
     # name: (op, N, H, L, E)
     "srwm_c4": ("srwm", 32, 16, 512, 64),
     "srwm_c3": ("srwm", 32, 8, 100, 32),
+    # the RL learner's regime on the same shape: gradient cut at the carried state, 5 % resets;
+    # one launch for the unroll (forward) + readout-gradient replay + the batched x (x) g product
+    "srwm_c3_steps": ("srwm_steps", 32, 8, 100, 32),
     "delta_c2": ("delta", 32, 8, 256, 64),
     "delta_c5f32": ("delta", 8, 16, 4096, 128),
     "delta_c5": ("delta_bf16", 8, 16, 4096, 128),     # bf16 q/k/v/beta/out/grads, fp32 memory
@@ -89,6 +92,71 @@ def srwm_step(t, ev=None):
                                flags=srwm_hip.GRAD_STATE_ZERO)
     if ev:
         ev[2].record()
+
+
+def srwm_steps_setup(N, H, L, E, dev):
+    import torch
+    t = srwm_setup(N, H, L, E, dev)
+    g = torch.Generator().manual_seed(1)
+    t["x"] = torch.softmax(t["x"], -1)
+    t["keep"] = (torch.rand(N, L, generator=g) > 0.05).float().to(dev)
+    t["slow"] = [w[0].contiguous() for w in t["W0"]]
+    t["Wy_entry"] = torch.empty_like(t["W0"][0])
+    t["gWy"] = torch.empty(H, E, E, device=dev)
+    return t
+
+
+def srwm_steps_step(t, ev=None):
+    import torch
+    import srwm_hip
+    for w, w0 in zip(t["W"], t["W0"]):
+        w.copy_(w0)
+    t["Wy_entry"].copy_(t["W0"][0])
+    if ev:
+        ev[0].record()
+    srwm_hip.self_ref_forward_steps(t["x"], t["keep"], t["slow"], *t["W"], *t["saved"], t["out"])
+    if ev:
+        ev[1].record()
+    sv = t["saved"]
+    srwm_hip.self_ref_readout_grad(sv[1], sv[2], sv[3], t["keep"], t["slow"][0], t["go"], t["Wy_entry"], t["gx"])
+    t["gWy"].copy_(torch.einsum("nhle,nhlm->hem", t["x"], t["go"]))
+    if ev:
+        ev[2].record()
+
+
+def srwm_per_step_loop_ms(t, N, H, L, E, dev, reps=3):
+    """The same unroll issued the way the reference's learner issues it: per time step, weights =
+    carried shift * notdone + shared weights (new tensors), one L = 1 forward; then one L = 1
+    backward per step.  Wall time in ms, best of `reps`."""
+    import time
+    import torch
+    import srwm_hip
+    best = None
+    for _ in range(reps):
+        shift = [torch.zeros_like(w) for w in t["W0"]]
+        steps = []
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for s_ in range(L):
+            kp = t["keep"][:, s_].view(N, 1, 1, 1)
+            W = [sh * kp + w0 for sh, w0 in zip(shift, t["W0"])]
+            saved = [torch.empty(N, H, 1, E, device=dev) for _ in range(2)] + [torch.empty(N, H, 1, 4, device=dev)] + \
+                    [torch.empty(N, H, 1, E, device=dev) for _ in range(3)] + [torch.empty(N, H, 1, 4, device=dev)]
+            out = torch.empty(N, H, 1, E, device=dev)
+            xs = t["x"][:, :, s_:s_ + 1]
+            srwm_hip.self_ref_forward(xs, *W, *saved, out)
+            shift = [w - w0 for w, w0 in zip(W, t["W0"])]
+            steps.append((xs, saved, W))
+        for s_ in reversed(range(L)):
+            xs, saved, W = steps[s_]
+            gx = torch.empty(N, H, 1, E, device=dev)
+            gW = [torch.empty_like(w) for w in W]
+            srwm_hip.self_ref_backward(xs, *saved, t["go"][:, :, s_:s_ + 1], *W, gx, *gW,
+                                       flags=srwm_hip.GRAD_STATE_ZERO)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) * 1e3
+        best = dt if best is None else min(best, dt)
+    return best
 
 
 def delta_setup(N, H, L, E, dev, io=None):
@@ -137,6 +205,9 @@ def algorithmic_bytes(op, N, H, L, E):
     if op == "srwm":
         S = E * (3 * E + 4)
         return 3 * S * 4 * hs, 6 * S * 4 * hs, (15 * E + 16) * 4 * hs + 4 * S * 4 * N * H
+    if op == "srwm_steps":   # forward as above; the replay reads and writes the E x E y block once per step
+        S = E * (3 * E + 4)
+        return 3 * S * 4 * hs, 2 * E * E * 4 * hs, ((7 * E + 8) + (4 * E + 4)) * 4 * hs + (2 * S + E * E) * 4 * N * H
     S = E * E
     # per (sequence, step): q,k,v,beta in (fwd and bwd), out + grad_out in the I/O type; v_old,
     # v_insert written and read back, and the 3 E-wide gradients + grad_beta written, in fp32
@@ -242,6 +313,8 @@ def main():
     op, N, H, L, E = WORKLOADS[a.workload]
     if op == "srwm":
         step, t = srwm_step, srwm_setup(N, H, L, E, dev)
+    elif op == "srwm_steps":
+        step, t = srwm_steps_step, srwm_steps_setup(N, H, L, E, dev)
     else:
         step = delta_step
         t = delta_setup(N, H, L, E, dev, torch.bfloat16 if op == "delta_bf16" else torch.float32)
@@ -286,13 +359,17 @@ def main():
         "roofline_fwd_bwd": roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS),
         "roofline_hbm": roof("hbm", hbm, fwd_ms + bwd_ms, HBM_PEAK_GBS),
     }
+    if op == "srwm_steps":
+        res["per_step_loop_ms"] = round(srwm_per_step_loop_ms(t, N, H, L, E, dev), 3)
+        res["config"]["workload"] += ("; gradient cut at the carried state, 5 % resets; per_step_loop_ms = the same "
+                                      "unroll as L launches of the L = 1 operator (forward + backward)")
     lds_meas = None if a.no_lds_probe else measure_lds_peak(dev)
     if lds_meas:
         res["lds_peak_measured_GBs"] = round(lds_meas, 1)
         res["roofline_fwd_bwd"]["frac_of_measured_lds_peak"] = round(
             res["roofline_fwd_bwd"]["achieved"] / lds_meas, 4)
     if not a.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline("srwm" if op == "srwm" else "delta", N, H, L, E, a.cpu_budget)
+        res["cpu_baseline"] = cpu_baseline("srwm" if op.startswith("srwm") else "delta", N, H, L, E, a.cpu_budget)
     print(json.dumps(res))
 
 

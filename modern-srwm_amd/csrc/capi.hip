@@ -117,7 +117,7 @@ int srwm_readout_grad_f32(const float *k, const float *beta, const float *ydiff,
     if (!k || !beta || !ydiff || !grad_out || !gs || !Wy_entry || !grad_x || (keep && !sWy)) return SRWM_EINVAL;
     if (!dims_ok(N, H, L, E) || flags) return SRWM_EINVAL;
     if (!stride_ok(gs, N, H, L, E)) return SRWM_ESTRIDE;
-    if (srwm_readout_grad_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
+    if (E > 256 || srwm_readout_grad_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
     SrwmReadoutGradParams p{k, beta, ydiff, keep, grad_out, gs[0], gs[1], gs[2], Wy_entry, sWy, grad_x, N, H, L, E};
     return launch_srwm_readout_grad(p, (hipStream_t)stream);
 }

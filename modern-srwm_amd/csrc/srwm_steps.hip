@@ -37,17 +37,30 @@ __global__ __launch_bounds__(kThreads) void srwm_readout_grad_kernel(SrwmReadout
     for (int i = tid; i < E * E; i += kThreads) W[(i / E) * Ep + i % E] = p.Wy0[seq * E * E + i];
     __syncthreads();
 
+    // the vectors of a step are fetched one step ahead (thread e < E holds element e; E <= 256)
+    float nk = 0.f, ny = 0.f, ng = 0.f, nb = 0.f, nkeep = 1.f;
+    auto fetch = [&](int t) {
+        const int64_t o = (seq * p.L + t) * E;
+        nb = p.beta[(seq * p.L + t) * 4];
+        nkeep = p.keep ? p.keep[(int64_t)n * p.L + t] : 1.f;
+        if (tid < E) {
+            nk = p.k[o + tid];
+            ny = p.ydiff[o + tid];
+            ng = gob[t * p.gs_l + tid];
+        }
+    };
+    fetch(0);
     for (int t = 0; t < p.L; ++t) {
         const int64_t o = (seq * p.L + t) * E;
-        if (p.keep && p.keep[(int64_t)n * p.L + t] == 0.f) {   // uniform over the workgroup
+        if (nkeep == 0.f) {   // uniform over the workgroup
             for (int i = tid; i < E * E; i += kThreads) W[(i / E) * Ep + i % E] = p.sWy[(int64_t)h * E * E + i];
         }
-        const float by = p.beta[(seq * p.L + t) * 4];
-        for (int e = tid; e < E; e += kThreads) {
-            kv[e] = p.k[o + e];
-            iv[e] = by * p.ydiff[o + e];
-            gv[e] = gob[t * p.gs_l + e];
+        if (tid < E) {
+            kv[tid] = nk;
+            iv[tid] = nb * ny;
+            gv[tid] = ng;
         }
+        if (t + 1 < p.L) fetch(t + 1);
         __syncthreads();
         // grad_x[e] = sum_m W[e][m] grad_out[m]: 16 lanes per row, then a DPP sum inside the row
         for (int e = grp; e < E; e += kThreads / 16) {
