@@ -68,7 +68,8 @@ __device__ __forceinline__ void store_vec(float *dst, const float *src) {
     }
 }
 
-template <int E, int NW, int R>
+// RESET: the per-step reset to the shared weights is compiled in (p.keep != nullptr)
+template <int E, int NW, int R, bool RESET>
 __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams p) {
     using T = Tiling<E, NW, R>;
     constexpr int RG = T::RG, CGW = T::CGW, CB = T::CB, NC = T::NC, TT = T::TT;
@@ -121,11 +122,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         return *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col);
     };
     auto load_keep = [&](int tile) -> float {
-        return (p.keep && tid < TT) ? p.keep[(int64_t)n * p.L + min(tile * TT + tid, p.L - 1)] : 1.f;
+        return (RESET && tid < TT) ? p.keep[(int64_t)n * p.L + min(tile * TT + tid, p.L - 1)] : 1.f;
     };
     const int ntiles = (p.L + TT - 1) / TT;
     *reinterpret_cast<float4 *>(&xt[0][ld_row][ld_col]) = load_tile(0);
-    if (tid < TT) kt[0][tid] = load_keep(0);
+    if (RESET && tid < TT) kt[0][tid] = load_keep(0);
     __syncthreads();
 
     for (int tile = 0; tile < ntiles; ++tile) {
@@ -141,7 +142,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         for (int tt = 0; tt < tlen; ++tt) {
             const int t = tile * TT + tt, par = t & 1;
             const int64_t o = (seq * p.L + t) * E, ob = (seq * p.L + t) * 4;
-            if (p.keep && kt[buf][tt] == 0.f) reset_state();   // uniform over the workgroup
+            if constexpr (RESET) {
+                if (kt[buf][tt] == 0.f) reset_state();   // uniform over the workgroup
+            }
 
             // ---- main readout: [y | q~ | k~ | b~] = W^T x_t
             float xr[R];
@@ -164,7 +167,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             if (has_b && el == 0) rawb[par][jb] = pb;
             if (tt == tlen - 1 && tile + 1 < ntiles) {
                 *reinterpret_cast<float4 *>(&xt[buf ^ 1][ld_row][ld_col]) = xnext;
-                if (tid < TT) kt[buf ^ 1][tid] = knext;
+                if (RESET && tid < TT) kt[buf ^ 1][tid] = knext;
             }
             __syncthreads();
 
@@ -510,7 +513,10 @@ int launch_bwd(const SrwmBwdParams &p, hipStream_t s) {
 
 template <int E, int NW, int R>
 int launch_fwd(const SrwmFwdParams &p, hipStream_t s) {
-    hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    if (p.keep)
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, true>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    else
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, false>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
