@@ -159,6 +159,36 @@ SRWM_API int delta_backward_f32(const float *Q, const int64_t q_strides[3],
                        int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
 /*
+ * Delta rule over all steps of an unroll with per-step resets, and the product its detached-state
+ * gradient needs.  No counterpart functions in the reference: they fuse the loop in which its RL
+ * learner calls the L = 1 operator once per time step on `state * notdone`
+ * (reinforcement_learning/torchbeast_procgen/model.py:1176-1196, torchbeast/layer.py:128-189),
+ * where the memory receives no gradient (fast_weight/__init__.py:95-100 returns None for it).
+ *
+ * delta_forward_steps_f32: as delta_forward_f32, the memory zeroed before step t of batch row n
+ * where keep[n][t] == 0 (keep: dense [N,L] or NULL).
+ *
+ * delta_readout_replay_f32: u[n][h][t] = W_{t-1} grad_out[n][h][t] (dense [N,H,L,E]) with W
+ * replayed from W_entry (the memory handed to delta_forward_steps_f32, before that call) through
+ * W += k (x) v_insert and the same resets.  With kq = k.q, ig = v_insert.grad_out the per-step
+ * gradients are  grad_q = u + ig k,  grad_k = ig q - beta kq u,  grad_v = beta kq grad_out,
+ * grad_beta = kq grad_out.(v - v_old), which the caller forms elementwise.
+ */
+SRWM_API int delta_forward_steps_f32(const float *Q, const int64_t q_strides[3],
+                            const float *K, const int64_t k_strides[3],
+                            const float *V, const int64_t v_strides[3],
+                            const float *beta, const int64_t beta_strides[3],
+                            const float *keep,
+                            float *v_old, float *v_insert, float *W, float *out,
+                            int N, int H, int L, int E, int M, unsigned flags, void *stream);
+
+SRWM_API int delta_readout_replay_f32(const float *K, const int64_t k_strides[3],
+                             const float *v_insert, const float *keep,
+                             const float *grad_out, const int64_t grad_out_strides[3],
+                             const float *W_entry, float *u,
+                             int N, int H, int L, int E, int M, unsigned flags, void *stream);
+
+/*
  * Delta rule with bf16 inputs/outputs and fp32 memory.  No counterpart in the reference
  * (its kernels are float-only, fast_weight_cuda.cu:12-14); same recurrence as
  * delta_forward_f32 / delta_backward_f32 with

@@ -117,9 +117,44 @@ int srwm_readout_grad_f32(const float *k, const float *beta, const float *ydiff,
     if (!k || !beta || !ydiff || !grad_out || !gs || !Wy_entry || !grad_x || (keep && !sWy)) return SRWM_EINVAL;
     if (!dims_ok(N, H, L, E) || flags) return SRWM_EINVAL;
     if (!stride_ok(gs, N, H, L, E)) return SRWM_ESTRIDE;
-    if (E > 256 || srwm_readout_grad_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
-    SrwmReadoutGradParams p{k, beta, ydiff, keep, grad_out, gs[0], gs[1], gs[2], Wy_entry, sWy, grad_x, N, H, L, E};
-    return launch_srwm_readout_grad(p, (hipStream_t)stream);
+    if (E > 256 || replay_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
+    ReplayParams p{k, {(int64_t)H * L * E, (int64_t)L * E, E}, ydiff, beta, 4, keep, grad_out,
+                   {gs[0], gs[1], gs[2]}, Wy_entry, keep ? sWy : nullptr, grad_x, N, H, L, E, E};
+    return launch_replay(p, (hipStream_t)stream);
+}
+
+int delta_forward_steps_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],
+                            const float *V, const int64_t vs[3], const float *beta, const int64_t bs[3],
+                            const float *keep, float *v_old, float *v_insert, float *W, float *out, int N,
+                            int H, int L, int E, int M, unsigned flags, void *stream) {
+    if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
+        return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
+        !stride_ok(bs, N, H, L, 1))
+        return SRWM_ESTRIDE;
+    DeltaFwdParams p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
+                     {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
+                     N, H, L, E, M, keep};
+    hipStream_t s = (hipStream_t)stream;
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_delta_fwd_tiled(p, s);
+        if (r >= 0) return r;
+    }
+    if (delta_fwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
+    return launch_delta_fwd_generic(p, s);
+}
+
+int delta_readout_replay_f32(const float *K, const int64_t ks[3], const float *v_insert, const float *keep,
+                             const float *grad_out, const int64_t gs[3], const float *W_entry, float *u,
+                             int N, int H, int L, int E, int M, unsigned flags, void *stream) {
+    if (!K || !ks || !v_insert || !grad_out || !gs || !W_entry || !u) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || flags) return SRWM_EINVAL;
+    if (!stride_ok(ks, N, H, L, E) || !stride_ok(gs, N, H, L, M)) return SRWM_ESTRIDE;
+    if (E > 256 || M > 256 || replay_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
+    ReplayParams p{K, {ks[0], ks[1], ks[2]}, v_insert, nullptr, 0, keep, grad_out, {gs[0], gs[1], gs[2]},
+                   W_entry, nullptr, u, N, H, L, E, M};
+    return launch_replay(p, (hipStream_t)stream);
 }
 
 int srwm_backward_f32(const float *x, const int64_t xs[3], const float *q, const float *k,

@@ -21,18 +21,6 @@ struct SrwmFwdParams {
     const float *sWy, *sWq, *sWk, *swb;   // [H,E,E] x 3, [H,E,4]
 };
 
-// Gradient of the readout alone, for callers that detach the carried state between steps:
-// grad_x_t = W_y,t-1 grad_out_t with W_y replayed from its entry value and the saved k, beta_y, y_diff.
-struct SrwmReadoutGradParams {
-    const float *k, *beta, *ydiff, *keep;
-    const float *go;
-    int64_t gs_n, gs_h, gs_l;
-    const float *Wy0;    // [N,H,E,E] y block before step 0
-    const float *sWy;    // [H,E,E], used where keep == 0 (may be nullptr when keep is)
-    float *gx;
-    int N, H, L, E;
-};
-
 struct SrwmBwdParams {
     const float *x;
     int64_t xs_n, xs_h, xs_l;
@@ -49,11 +37,32 @@ struct Strided3 {
     int64_t n, h, l;
 };
 
+// Replay of a rank-1 recurrence with a row-sum readout BEFORE each write, for callers that cut
+// the gradient at the carried state:   u_t = W_{t-1} g_t;   W_t = W_{t-1} + a_t (x) (s_t * b_t),
+// W reset (to Wreset of the head, or to zero) before step t where keep[n][t] == 0.
+//   SRWM readout:  W = y block, a = k, b = y_diff, s = beta_y           -> u = grad_x
+//   delta rule:    W = memory,  a = k, b = v_insert, s = 1              -> u = W_{t-1} grad_out_t
+struct ReplayParams {
+    const float *a;        // [N,H,L,E], strided
+    Strided3 as;
+    const float *b;        // dense [N,H,L,M]
+    const float *bscale;   // element (n,h,t) at bscale[((n*H+h)*L+t) * bscale_stride], or nullptr
+    int bscale_stride;
+    const float *keep;     // dense [N,L] or nullptr
+    const float *g;        // [N,H,L,M], strided
+    Strided3 gs;
+    const float *W0;       // dense [N,H,E,M]: W before step 0
+    const float *Wreset;   // dense [H,E,M] or nullptr (reset to zero)
+    float *u;              // dense [N,H,L,E]
+    int N, H, L, E, M;
+};
+
 struct DeltaFwdParams {
     const float *Q, *K, *V, *beta;
     Strided3 qs, ks, vs, bs;
     float *vold, *vins, *W, *out;
     int N, H, L, E, M;
+    const float *keep;   // optional dense [N,L]: the memory is zeroed before step t where keep[n][t] == 0
 };
 
 struct DeltaBwdParams {
@@ -107,8 +116,8 @@ size_t srwm_bwd_generic_lds_bytes(int E);
 size_t delta_fwd_generic_lds_bytes(int E, int M);
 size_t delta_bwd_generic_lds_bytes(int E, int M);
 int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s);
-size_t srwm_readout_grad_lds_bytes(int E);
-int launch_srwm_readout_grad(const SrwmReadoutGradParams &p, hipStream_t s);
+size_t replay_lds_bytes(int E, int M);
+int launch_replay(const ReplayParams &p, hipStream_t s);
 int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s);
 int launch_delta_fwd_generic(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_bwd_generic(const DeltaBwdParams &p, hipStream_t s);

@@ -36,6 +36,9 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_generic_kernel(DeltaFwdPar
         const float b = p.beta[n * p.bs.n + h * p.bs.h + t * p.bs.l];
         const int64_t om = (seq * p.L + t) * M;
         __syncthreads();  // previous step's readers of ks/qs are done (and W is loaded)
+        if (p.keep && p.keep[(int64_t)n * p.L + t] == 0.f) {   // uniform: the memory restarts from zero
+            for (int i = tid; i < E * Mp; i += kThreads) W[i] = 0.f;
+        }
         for (int e = tid; e < E; e += kThreads) {
             ks[e] = kt[e];
             qs[e] = qt[e];

@@ -149,6 +149,7 @@ struct FwdP {
     float *vold, *vins, *W;
     TI *out;
     int N, H, L;
+    const float *keep;   // optional [N,L]: zero the memory before step t where keep[n][t] == 0
 };
 template <class TI>
 struct BwdP {
@@ -165,7 +166,7 @@ struct BwdP {
     unsigned grad_state_mode;
 };
 
-template <class TI, int D, int MS, int NW, int R, int TT>
+template <class TI, int D, int MS, int NW, int R, int TT, bool RESET>
 __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) {
     using T = DTiling<D, MS, NW, R, TT>;
     constexpr int RG = T::RG, CGW = T::CGW, CC = T::CC, MC = T::MC, NT = T::NT;
@@ -174,6 +175,7 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
     __shared__ __attribute__((aligned(16))) float tk[2][TT][D];
     __shared__ __attribute__((aligned(16))) float tv[2][TT][MC];
     __shared__ float tbeta[2][TT];
+    __shared__ float tkeep[2][TT];   // RESET only: keep flags of the tile's steps
     // Outputs of a tile are parked here and written out after the step loop: the loop then
     // contains no global memory instruction, so the prefetch of the next tile stays in
     // flight across it, and the stores are full coalesced rows.
@@ -197,19 +199,21 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
 
     TileVec<NT, TT, D> nq, nk;
     TileVec<NT, TT, MC> nv;
-    float nb = 0.f;
+    float nb = 0.f, nkeep = 1.f;
     auto load_tile = [&](int tile) {
         const int t0 = tile * TT;
         nq.load(qb, p.qs.l, t0, p.L, tid);
         nk.load(kb, p.ks.l, t0, p.L, tid);
         nv.load(vb, p.vs.l, t0, p.L, tid);
         nb = ld1(bb + (int64_t)min(t0 + (tid % TT), p.L - 1) * p.bs.l);
+        if constexpr (RESET) nkeep = p.keep[(int64_t)n * p.L + min(t0 + (tid % TT), p.L - 1)];
     };
     auto store_tile = [&](int buf) {
         nq.store(&tq[buf][0][0], tid);
         nk.store(&tk[buf][0][0], tid);
         nv.store(&tv[buf][0][0], tid);
         if (tid < TT) tbeta[buf][tid] = nb;
+        if (RESET && tid < TT) tkeep[buf][tid] = nkeep;
     };
 
     const int ntiles = (p.L + TT - 1) / TT;
@@ -234,6 +238,14 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
             o.b = tbeta[buf][tt];
         };
         auto step = [&](const Ops &o, int tt) __attribute__((always_inline)) {
+            if constexpr (RESET) {
+                if (tkeep[buf][tt] == 0.f) {   // uniform over the workgroup: the memory restarts from zero
+#pragma unroll
+                    for (int i = 0; i < R; ++i)
+#pragma unroll
+                        for (int c = 0; c < CC; ++c) w[i][c] = 0.f;
+                }
+            }
             // v_old = W^T k and W^T q in one pass over the tile, plus this lane's part of k.q
             float vo[CC], oq[CC], kq = 0.f;
 #pragma unroll
@@ -508,8 +520,12 @@ __global__ void zero_fill_kernel(float *a, int64_t na, float *b, int64_t nb, flo
 
 template <class TI, int D, int MS, int NW, int R, int TT>
 int launch_f(const FwdP<TI> &p, hipStream_t s) {
-    hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, MS, NW, R, TT>), dim3(p.N * p.H * MS),
-                       dim3(NW * kWave), 0, s, p);
+    if (p.keep)
+        hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, MS, NW, R, TT, true>), dim3(p.N * p.H * MS),
+                           dim3(NW * kWave), 0, s, p);
+    else
+        hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, MS, NW, R, TT, false>), dim3(p.N * p.H * MS),
+                           dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
@@ -571,7 +587,8 @@ int dispatch_bwd(const BwdP<TI> &p, int D, hipStream_t s) {
 
 int launch_delta_fwd_tiled(const DeltaFwdParams &p, hipStream_t s) {
     if (p.E != p.M) return -1;
-    const FwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.N, p.H, p.L};
+    const FwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.N, p.H, p.L,
+                        p.keep};
     return dispatch_fwd(q, p.E, s);
 }
 
@@ -584,7 +601,8 @@ int launch_delta_bwd_tiled(const DeltaBwdParams &p, hipStream_t s) {
 
 int launch_delta_fwd_tiled_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s) {
     if (p.E != p.M) return -1;
-    const FwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.N, p.H, p.L};
+    const FwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.N, p.H, p.L,
+                         nullptr};
     return dispatch_fwd(q, p.E, s);
 }
 

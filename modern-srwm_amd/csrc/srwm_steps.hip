@@ -1,17 +1,19 @@
-// Gradient of the SRWM readout for callers that cut the gradient at the carried state.
+// Step-mode support: gradients for callers that cut the gradient at the carried state.
 //
-// The RL learner of the reference runs the operator once per time step (L = 1) on
-// weights = detached carried shift + shared parameters (reinforcement_learning/torchbeast/
-// layer.py:377-421, torchbeast_procgen/model.py:1176-1196): the output of step t is
-// y_t = W_y,t-1^T x_t and nothing after it in the graph depends on the weights again, so
-//     grad_x_t = W_y,t-1 grad_out_t         (and grad of the shared W_y = sum_t x_t (x) grad_out_t,
-//                                            a plain batched product the caller forms itself).
-// When all steps of an unroll run in ONE forward launch (srwm_forward_steps_f32), this kernel
-// supplies grad_x: it replays the y block forward in time from its entry value with the saved
-// k_t, beta_y,t, y_diff_t (W_y += k (x) beta_y y_diff, reset to the shared block where keep == 0).
+// The RL learner of the reference runs its fast-weight operators once per time step (L = 1) on a
+// carried state that is detached (SRWM: reinforcement_learning/torchbeast/layer.py:412-418) or
+// receives no gradient (delta rule: fast_weight/__init__.py:95-100 returns None for W), zeroing
+// the carried part where an episode ended (torchbeast_procgen/model.py:1176-1196).  The output of
+// step t then depends on the state only through one read of W_{t-1}, and its gradient needs a
+// single product with that matrix:
+//     SRWM        y_t = W_y,t-1^T x_t                  grad_x_t = W_y,t-1 g_t
+//     delta rule  out_t = W^T q + (k.q) ins,  W = W_{t-1}:  u_t = W_{t-1} g_t enters grad_q, grad_k
+// When all steps of an unroll run in ONE forward launch, this kernel supplies u_t for all t: it
+// replays W forward in time from its entry value with the saved write vectors
+// (W += a (x) (s b)), applies the same resets, and reads W g before each write.
 //
-// One workgroup per (batch, head) sequence, the E x E block in LDS (odd row stride), 16-lane
-// groups own rows: any E whose block fits in LDS.
+// One workgroup per (batch, head) sequence, the E x M matrix in LDS (odd row stride), 16-lane
+// groups own rows; the vectors of a step are fetched one step ahead.
 #include "common.h"
 #include "xlane.h"
 
@@ -21,59 +23,59 @@ namespace {
 
 constexpr int kThreads = 256;
 
-__global__ __launch_bounds__(kThreads) void srwm_readout_grad_kernel(SrwmReadoutGradParams p) {
+__global__ __launch_bounds__(kThreads) void replay_kernel(ReplayParams p) {
     extern __shared__ float smem[];
-    const int E = p.E, Ep = E | 1;
-    float *W = smem;          // [E][Ep]
-    float *kv = W + E * Ep;   // [E]  k_t
-    float *iv = kv + E;       // [E]  beta_y,t * y_diff_t
-    float *gv = iv + E;       // [E]  grad_out_t
+    const int E = p.E, M = p.M, Mp = M | 1;
+    float *W = smem;          // [E][Mp]
+    float *av = W + E * Mp;   // [E]  a_t
+    float *bv = av + E;       // [M]  s_t * b_t
+    float *gv = bv + M;       // [M]  g_t
 
     const int tid = threadIdx.x, grp = tid >> 4, gl = tid & 15;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
-    const float *gob = p.go + n * p.gs_n + h * p.gs_h;
+    const float *ab = p.a + n * p.as.n + h * p.as.h;
+    const float *gb = p.g + n * p.gs.n + h * p.gs.h;
 
-    for (int i = tid; i < E * E; i += kThreads) W[(i / E) * Ep + i % E] = p.Wy0[seq * E * E + i];
-    __syncthreads();
+    for (int i = tid; i < E * M; i += kThreads) W[(i / M) * Mp + i % M] = p.W0[seq * E * M + i];
 
-    // the vectors of a step are fetched one step ahead (thread e < E holds element e; E <= 256)
-    float nk = 0.f, ny = 0.f, ng = 0.f, nb = 0.f, nkeep = 1.f;
+    // thread e < E holds a[e], thread m < M holds b[m], g[m] of the next step (E, M <= 256)
+    float na = 0.f, nb = 0.f, ng = 0.f, ns = 1.f, nkeep = 1.f;
     auto fetch = [&](int t) {
-        const int64_t o = (seq * p.L + t) * E;
-        nb = p.beta[(seq * p.L + t) * 4];
+        if (p.bscale) ns = p.bscale[(seq * p.L + t) * p.bscale_stride];
         nkeep = p.keep ? p.keep[(int64_t)n * p.L + t] : 1.f;
-        if (tid < E) {
-            nk = p.k[o + tid];
-            ny = p.ydiff[o + tid];
-            ng = gob[t * p.gs_l + tid];
+        if (tid < E) na = ab[t * p.as.l + tid];
+        if (tid < M) {
+            nb = p.b[(seq * p.L + t) * M + tid];
+            ng = gb[t * p.gs.l + tid];
         }
     };
     fetch(0);
+    __syncthreads();
     for (int t = 0; t < p.L; ++t) {
-        const int64_t o = (seq * p.L + t) * E;
         if (nkeep == 0.f) {   // uniform over the workgroup
-            for (int i = tid; i < E * E; i += kThreads) W[(i / E) * Ep + i % E] = p.sWy[(int64_t)h * E * E + i];
+            for (int i = tid; i < E * M; i += kThreads)
+                W[(i / M) * Mp + i % M] = p.Wreset ? p.Wreset[(int64_t)h * E * M + i] : 0.f;
         }
-        if (tid < E) {
-            kv[tid] = nk;
-            iv[tid] = nb * ny;
+        if (tid < E) av[tid] = na;
+        if (tid < M) {
+            bv[tid] = ns * nb;
             gv[tid] = ng;
         }
         if (t + 1 < p.L) fetch(t + 1);
         __syncthreads();
-        // grad_x[e] = sum_m W[e][m] grad_out[m]: 16 lanes per row, then a DPP sum inside the row
+        // u[e] = sum_m W[e][m] g[m]: 16 lanes per row, then a DPP sum inside the 16-lane row
         for (int e = grp; e < E; e += kThreads / 16) {
-            float a = 0.f;
-            for (int m = gl; m < E; m += 16) a = fmaf(W[e * Ep + m], gv[m], a);
-            a = group_sum<16>(a);
-            if (gl == 0) p.gx[o + e] = a;
+            float acc = 0.f;
+            for (int m = gl; m < M; m += 16) acc = fmaf(W[e * Mp + m], gv[m], acc);
+            acc = group_sum<16>(acc);
+            if (gl == 0) p.u[(seq * p.L + t) * E + e] = acc;
         }
         __syncthreads();
-        // the step's write: W += k (x) (beta_y y_diff)
-        for (int i = tid; i < E * E; i += kThreads) {
-            const int e = i / E, m = i - e * E;
-            W[e * Ep + m] = fmaf(kv[e], iv[m], W[e * Ep + m]);
+        // the step's write
+        for (int i = tid; i < E * M; i += kThreads) {
+            const int e = i / M, m = i - e * M;
+            W[e * Mp + m] = fmaf(av[e], bv[m], W[e * Mp + m]);
         }
         __syncthreads();
     }
@@ -81,14 +83,14 @@ __global__ __launch_bounds__(kThreads) void srwm_readout_grad_kernel(SrwmReadout
 
 }  // namespace
 
-size_t srwm_readout_grad_lds_bytes(int E) { return sizeof(float) * ((size_t)E * (E | 1) + 3 * (size_t)E); }
+size_t replay_lds_bytes(int E, int M) { return sizeof(float) * ((size_t)E * (M | 1) + E + 2 * (size_t)M); }
 
-int launch_srwm_readout_grad(const SrwmReadoutGradParams &p, hipStream_t s) {
-    const size_t lds = srwm_readout_grad_lds_bytes(p.E);
-    hipError_t err = hipFuncSetAttribute((const void *)srwm_readout_grad_kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+int launch_replay(const ReplayParams &p, hipStream_t s) {
+    const size_t lds = replay_lds_bytes(p.E, p.M);
+    hipError_t err = hipFuncSetAttribute((const void *)replay_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)lds);
     if (err != hipSuccess) return (int)err;
-    hipLaunchKernelGGL(srwm_readout_grad_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
+    hipLaunchKernelGGL(replay_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
     return (int)hipGetLastError();
 }
 

@@ -80,3 +80,44 @@ class DeltaFastWeight(torch.autograd.Function):
 
 # Alias the autograd functions to python style snake case naming
 fast_weight_delta = DeltaFastWeight.apply
+
+
+class DeltaFastWeightSteps(torch.autograd.Function):
+    """All time steps of an RL unroll in one launch, with the semantics of calling
+    `fast_weight_delta` once per step on `memory * notdone` (reinforcement_learning/
+    torchbeast_procgen/model.py:1176-1196, torchbeast/layer.py:128-189): the memory receives no
+    gradient, so each step's gradient sees W_{t-1} as a constant.
+
+        out = fast_weight_delta_steps(Q, K, V, beta, keep, W)
+
+    keep: (N, L) float, 0 where the memory is zeroed before the step (None: never).  W is
+    OVERWRITTEN with the memory after the last step (the carried state)."""
+
+    @staticmethod
+    def forward(ctx, Q, K, V, beta, keep, W):
+        for t in (Q, K, V, beta, W):
+            assert t.device.type != "cpu"
+        N, H, L, E = Q.shape
+        M = V.shape[-1]
+        new = lambda: torch.empty((N, H, L, M), device=Q.device, dtype=Q.dtype)
+        out, V_old, V_insert = new(), new(), new()
+        W_entry = W.detach().clone()
+        srwm_hip.fast_weight_forward_steps(Q.data, K.data, V.data, beta.data, keep, V_old, V_insert, W.data, out)
+        ctx.save_for_backward(Q, K, V, beta, keep, V_old, V_insert, W_entry)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        Q, K, V, beta, keep, V_old, V_insert, W_entry = ctx.saved_tensors
+        u = torch.empty(Q.shape, device=Q.device, dtype=Q.dtype)
+        srwm_hip.fast_weight_readout_replay(K, V_insert, keep, grad_out, W_entry, u)
+        kq = (K * Q).sum(-1, keepdim=True)
+        ig = (V_insert * grad_out).sum(-1, keepdim=True)
+        grad_Q = u + ig * K
+        grad_K = ig * Q - (beta * kq) * u
+        grad_V = (beta * kq) * grad_out
+        grad_beta = kq * (grad_out * (V - V_old)).sum(-1, keepdim=True)
+        return grad_Q, grad_K, grad_V, grad_beta, None, None
+
+
+fast_weight_delta_steps = DeltaFastWeightSteps.apply

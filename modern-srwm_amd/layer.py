@@ -16,7 +16,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from fast_weight import fast_weight_delta
+from fast_weight import fast_weight_delta, fast_weight_delta_steps
 from self_ref_v0 import self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
 
 
@@ -196,3 +196,14 @@ class CarryFastFFlayer(_DeltaBase):
         fast_weights = state
         out = self.fw_layer(q, k, v, beta, fast_weights)
         return self._finish(x, out, bsz, slen), fast_weights.clone()
+
+    def forward_steps(self, x, notdone, state):
+        """The whole unroll at once: equivalent to calling forward() once per time step on
+        x[t:t+1] with the memory multiplied by notdone[t] first (the learner's loop,
+        reinforcement_learning/torchbeast_procgen/model.py:1176-1196).  x: (T, B, D); notdone: (T, B)."""
+        assert state is not None
+        q, k, v, beta, slen, bsz = self._qkvb(x, elu_p1_sum_norm_eps)
+        keep = notdone.to(x.dtype).transpose(0, 1).contiguous()
+        fast_weights = state.detach().clone()
+        out = fast_weight_delta_steps(q, k, v, beta, keep, fast_weights)
+        return self._finish(x, out, bsz, slen), fast_weights

@@ -45,6 +45,8 @@ _SIGNATURES = {
     "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
+    "delta_forward_steps_f32": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_readout_replay_f32": [_F, _S] + [_F, _F] + [_F, _S] + [_F, _F] + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_forward_f32": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_backward_f32": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_forward_bf16": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -304,6 +306,58 @@ def fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=0):
         code = fn(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
                   *[_ptr(t) for t in d], N, H, L, E, M, flags, _stream(q.device))
     _check(code, fn.__name__)
+
+
+def fast_weight_forward_steps(q, k, v, beta, keep, v_old, v_insert, kv, out, flags=0):
+    """Delta-rule forward over all steps of an unroll; the memory is zeroed before step t of batch
+    row n where keep[n, t] == 0 (keep: (N, L) float32 or None).  float32 only."""
+    _require(q, "q")
+    N, H, L, E = q.shape
+    _require(k, "k", (N, H, L, E))
+    _require(v, "v")
+    M = v.shape[-1]
+    _require(v, "v", (N, H, L, M))
+    _require(beta, "beta", (N, H, L, 1))
+    for t, nm in ((v_old, "v_old"), (v_insert, "v_insert"), (out, "out")):
+        _require(t, nm, (N, H, L, M))
+    _require(kv, "kv", (N, H, E, M))
+    null = ctypes.c_void_p(None)
+    if keep is not None:
+        _require(keep, "keep", (N, L))
+        keep = keep.contiguous()
+    if q.numel() == 0 or v.numel() == 0:
+        return
+    (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr) = (_strided(t) for t in (q, k, v, beta))
+    with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv, out], True) as d:
+        code = lib().delta_forward_steps_f32(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
+                                             _ptr(keep) if keep is not None else null,
+                                             *[_ptr(t) for t in d], N, H, L, E, M, flags, _stream(q.device))
+    _check(code, "delta_forward_steps_f32")
+
+
+def fast_weight_readout_replay(k, v_insert, keep, grad_out, kv_entry, u):
+    """u[n, h, t] = W_{t-1} grad_out[n, h, t] for an unroll whose memory carries no gradient;
+    kv_entry is the (N, H, E, M) memory as it was before fast_weight_forward_steps."""
+    _require(k, "k")
+    N, H, L, E = k.shape
+    _require(v_insert, "v_insert")
+    M = v_insert.shape[-1]
+    _require(v_insert, "v_insert", (N, H, L, M))
+    _require(grad_out, "grad_out", (N, H, L, M))
+    _require(kv_entry, "kv_entry", (N, H, E, M))
+    _require(u, "u", (N, H, L, E))
+    null = ctypes.c_void_p(None)
+    if keep is not None:
+        _require(keep, "keep", (N, L))
+        keep = keep.contiguous()
+    if k.numel() == 0:
+        return
+    (ks, kstr), (gos, gstr) = _strided(k), _strided(grad_out)
+    with torch.cuda.device(k.device), _Dense([v_insert, kv_entry], False) as sv, _Dense([u], True) as d:
+        code = lib().delta_readout_replay_f32(_ptr(ks), kstr, _ptr(sv[0]), _ptr(keep) if keep is not None else null,
+                                              _ptr(gos), gstr, _ptr(sv[1]), _ptr(d[0]), N, H, L, E, M, 0,
+                                              _stream(k.device))
+    _check(code, "delta_readout_replay_f32")
 
 
 def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v,

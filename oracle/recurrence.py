@@ -87,3 +87,21 @@ def srwm_steps_reference(x, keep, shift, slow):
         outs.append(out)
         shift = [(f.detach() - w.repeat(N, 1, 1, 1)).detach() for f, w in zip(final, slow)]
     return torch.cat(outs, dim=2), shift
+
+
+def delta_steps_reference(Q, K, V, beta, keep, W0):
+    """The RL learner's call pattern for the delta rule, literally: one L = 1 call per time step on
+    `memory * keep_t`; the operator returns no gradient for its memory argument
+    (supervised_learning/fast_weight/__init__.py:95-100), which the detach reproduces.
+    Returns (out (N, H, L, M), final memory)."""
+    N, H, L, E = Q.shape
+    W = W0.detach()
+    outs = []
+    for t in range(L):
+        if keep is not None:
+            W = W * keep[:, t].reshape(N, 1, 1, 1)
+        sl = slice(t, t + 1)
+        out, W = delta_recurrence(Q[:, :, sl], K[:, :, sl], V[:, :, sl], beta[:, :, sl], W)
+        W = W.detach()
+        outs.append(out)
+    return torch.cat(outs, dim=2), W

@@ -350,3 +350,37 @@ def test_chunkwise_flag_is_refused_where_there_is_no_kernel():
         srwm_hip.fast_weight_forward(z(1, 1, 8, 32), z(1, 1, 8, 32), z(1, 1, 8, 32), z(1, 1, 8, 1),
                                      z(1, 1, 8, 32), z(1, 1, 8, 32), z(1, 1, 32, 32), z(1, 1, 8, 32),
                                      flags=srwm_hip.FLAG_CHUNKWISE)
+
+
+# ------------------------------------------------------------------ step-wise (RL learner) call pattern
+
+@pytest.mark.parametrize("shape,resets", [
+    ((4, 8, 100, 32, 32), True),     # RL-sized heads, register-resident forward
+    ((2, 2, 40, 64, 64), True),
+    ((2, 3, 25, 12, 20), True),      # E != M: generic forward
+    ((2, 2, 30, 16, 16), False),     # keep = None
+])
+def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
+    print(f"case delta stepwise shape={shape} resets={resets}", flush=True)
+    from oracle.recurrence import delta_steps_reference
+    from fast_weight import fast_weight_delta_steps
+    dev = _dev()
+    N, H, L, E, M = shape
+    q, k, v, beta, W0, go = delta_inputs(N, H, L, E, M, seed=29, qk="softmax", w0_std=0.3)
+    keep = None
+    if resets:
+        keep = (torch.rand(N, L, generator=torch.Generator().manual_seed(3)) > 0.2).to(torch.float64)
+        keep[0, 0] = 0.0
+        keep[-1, :] = 1.0
+    ref_leaves = [t.clone().requires_grad_(True) for t in (q, k, v, beta)]
+    ref_out, ref_W = delta_steps_reference(*ref_leaves, keep, W0)
+    (ref_out * go).sum().backward()
+    f32 = lambda t: t.to(dev, torch.float32)
+    leaves = [f32(t).requires_grad_(True) for t in (q, k, v, beta)]
+    W = f32(W0).contiguous()
+    out = fast_weight_delta_steps(*leaves, None if keep is None else f32(keep), W)
+    (out * f32(go)).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), ref_out.detach().numpy()) < TOL
+    assert rel_err(W.cpu().numpy(), ref_W.numpy()) < TOL
+    for a, b, nm in zip(leaves, ref_leaves, ("grad_Q", "grad_K", "grad_V", "grad_beta")):
+        assert rel_err(a.grad.cpu().numpy(), b.grad.numpy()) < TOL, nm

@@ -200,3 +200,38 @@ def test_rl_sr_layer_whole_unroll_equals_the_per_step_loop():
             ref = loop_grads[n]
             got = p.grad if p.grad is not None else torch.zeros_like(ref)
             assert (got - ref).abs().max().item() < 2e-5 * max(1e-6, ref.abs().max().item()), n
+
+
+def test_rl_delta_layer_whole_unroll_equals_the_per_step_loop():
+    print("case CarryFastFFlayer.forward_steps", flush=True)
+    from layer import CarryFastFFlayer
+    dev = torch.device("cuda:0")
+    torch.manual_seed(6)
+    T, B, H, d = 19, 4, 4, 16
+    lay = CarryFastFFlayer(H, d, H * d, 0.0).to(dev)
+    x = torch.randn(T, B, H * d, device=dev)
+    notdone = (torch.rand(T, B, device=dev) > 0.2).float()
+    state0 = 0.1 * torch.randn(B, H, d, d, device=dev)
+    go = torch.randn(T, B, H * d, device=dev)
+
+    xl = x.clone().requires_grad_(True)
+    outs, state = [], state0.clone()
+    for t in range(T):
+        state = state * notdone[t].view(B, 1, 1, 1)
+        o, state = lay(xl[t:t + 1], state)
+        outs.append(o)
+    loop_out = torch.cat(outs)
+    (loop_out * go).sum().backward()
+    loop_grads = {n: p.grad.clone() for n, p in lay.named_parameters() if p.grad is not None}
+    loop_gx = xl.grad.clone()
+    lay.zero_grad()
+
+    xs = x.clone().requires_grad_(True)
+    out, new_state = lay.forward_steps(xs, notdone, state0)
+    (out * go).sum().backward()
+    assert (out - loop_out).abs().max().item() < 2e-5 * loop_out.abs().max().item()
+    assert (new_state - state).abs().max().item() < 2e-5 * max(1.0, state.abs().max().item())
+    assert (xs.grad - loop_gx).abs().max().item() < 2e-5 * loop_gx.abs().max().item()
+    for n, p in lay.named_parameters():
+        if n in loop_grads:
+            assert (p.grad - loop_grads[n]).abs().max().item() < 2e-5 * max(1e-6, loop_grads[n].abs().max().item()), n

@@ -148,3 +148,38 @@ def test_chunkwise_backward_equals_the_sequential_reverse_sweep(chunks, blocked)
                                   chunk_row=chunks[1], blocked=blocked)
     for n in ("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W", "W0"):
         assert rel_err(ch[n], seq[n]) < 1e-10, n
+
+
+# ---------------------------------------------------------- step-wise (RL learner) call pattern
+
+def test_stepwise_reference_values_and_closed_form_gradients():
+    """Per-step calls with a memory that carries no gradient: values equal the full recurrence
+    (restarted from zero at resets); gradients follow from one product with W_{t-1}:
+    grad_q = u + ig k, grad_k = ig q - beta kq u, grad_v = beta kq g, grad_beta = kq g.(v - v_old)
+    with u = W_{t-1} g, kq = k.q, ig = v_insert.g."""
+    from oracle.recurrence import delta_steps_reference
+    N, H, L, E, M = 3, 2, 8, 5, 4
+    q, k, v, beta, W0, go = delta_inputs(N, H, L, E, M, seed=12, qk="l2", w0_std=0.4)
+    out, WL = delta_steps_reference(q, k, v, beta, None, W0)
+    ref, WL_ref = delta_recurrence(q, k, v, beta, W0)
+    assert rel_err(out.numpy(), ref.numpy()) < 1e-13 and rel_err(WL.numpy(), WL_ref.numpy()) < 1e-13
+
+    keep = torch.ones(N, L, dtype=torch.float64)
+    keep[0, 0] = keep[0, 5] = keep[1, 3] = 0.0
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, beta)]
+    out, _ = delta_steps_reference(*leaves, keep, W0)
+    (out * go).sum().backward()
+    W = W0.clone()
+    for t in range(L):
+        W = W * keep[:, t].reshape(N, 1, 1, 1)
+        qt, kt, vt, bt, gt = (a[:, :, t] for a in (q, k, v, beta, go))
+        vold = torch.einsum("nhem,nhe->nhm", W, kt)
+        ins = bt * (vt - vold)
+        assert rel_err(out[:, :, t].detach().numpy(),
+                       (torch.einsum("nhem,nhe->nhm", W, qt) + (kt * qt).sum(-1, keepdim=True) * ins).numpy()) < 1e-13
+        u = torch.einsum("nhem,nhm->nhe", W, gt)
+        kq, ig = (kt * qt).sum(-1, keepdim=True), (ins * gt).sum(-1, keepdim=True)
+        for leaf, formula in zip(leaves, (u + ig * kt, ig * qt - bt * kq * u, bt * kq * gt,
+                                          kq * (gt * (vt - vold)).sum(-1, keepdim=True))):
+            assert rel_err(leaf.grad[:, :, t].numpy(), formula.numpy()) < 1e-12
+        W = W + torch.einsum("nhe,nhm->nhem", kt, ins)
