@@ -50,6 +50,37 @@ def main():
                  W0=base[4], grad_out=go.numpy(), out=f["out"], v_old=f["v_old"],
                  v_insert=f["v_insert"], W_final=f["W"],
                  **{k: v for k, v in b.items() if k.startswith("grad")})
+    # chunk-sized delta case (one full chunk of 64 steps + a ragged one): exercises the chunkwise kernels
+    q, k, v, beta, W0, go = delta_inputs(1, 1, 66, 64, 64, seed=204, qk="l2", w0_std=0.1)
+    base = [t.numpy() for t in (q, k, v, beta, W0)]
+    f = oracle.delta_forward(*base)
+    b = oracle.delta_backward(*base[:4], f, go.numpy(), want_grad_W=True)
+    np.savez(os.path.join(HERE, "delta_n1h1l66e64m64.npz"), Q=base[0], K=base[1], V=base[2], beta=base[3],
+             W0=base[4], grad_out=go.numpy(), out=f["out"], v_old=f["v_old"], v_insert=f["v_insert"],
+             W_final=f["W"], **{k_: v_ for k_, v_ in b.items() if k_.startswith("grad")})
+    # step-wise (RL learner) call pattern: per-step calls with resets, gradient cut at the carried state
+    from oracle.recurrence import delta_steps_reference, srwm_steps_reference
+    from test_oracle_srwm import _steps_inputs
+    x, keep, shift, slow, go = _steps_inputs(2, 2, 7, 8, seed=301)
+    xl = x.clone().requires_grad_(True)
+    sl = [w.clone().requires_grad_(True) for w in slow]
+    out, fin = srwm_steps_reference(xl, keep, shift, sl)
+    (out * go).sum().backward()
+    np.savez(os.path.join(HERE, "steps_srwm_n2h2l7e8.npz"), x=x.numpy(), keep=keep.numpy(), grad_out=go.numpy(),
+             **{f"shift{i}": t.numpy() for i, t in enumerate(shift)},
+             **{f"slow{i}": t.numpy() for i, t in enumerate(slow)},
+             out=out.detach().numpy(), grad_x=xl.grad.numpy(), grad_slow0=sl[0].grad.numpy(),
+             **{f"final_shift{i}": t.numpy() for i, t in enumerate(fin)})
+    q, k, v, beta, W0, go = delta_inputs(2, 2, 7, 8, 8, seed=302, qk="softmax", w0_std=0.3)
+    keep = torch.ones(2, 7, dtype=torch.float64)
+    keep[0, 0] = keep[1, 4] = 0.0
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v, beta)]
+    out, WL = delta_steps_reference(*leaves, keep, W0)
+    (out * go).sum().backward()
+    np.savez(os.path.join(HERE, "steps_delta_n2h2l7e8m8.npz"), Q=q.numpy(), K=k.numpy(), V=v.numpy(),
+             beta=beta.numpy(), keep=keep.numpy(), W0=W0.numpy(), grad_out=go.numpy(),
+             out=out.detach().numpy(), W_final=WL.numpy(),
+             **{n: t.grad.numpy() for n, t in zip(("grad_Q", "grad_K", "grad_V", "grad_beta"), leaves)})
     print("wrote", sorted(n for n in os.listdir(HERE) if n.endswith(".npz")))
 
 

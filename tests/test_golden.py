@@ -14,11 +14,32 @@ from helpers import rel_err
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 SRWM = sorted(glob.glob(os.path.join(GOLD, "srwm_*.npz")))
 DELTA = sorted(glob.glob(os.path.join(GOLD, "delta_*.npz")))
+STEPS_SRWM = os.path.join(GOLD, "steps_srwm_n2h2l7e8.npz")
+STEPS_DELTA = os.path.join(GOLD, "steps_delta_n2h2l7e8m8.npz")
 TOL = 1e-5
 
 
 def test_fixtures_exist():
-    assert len(SRWM) >= 3 and len(DELTA) >= 3
+    assert len(SRWM) >= 3 and len(DELTA) >= 4 and os.path.exists(STEPS_SRWM) and os.path.exists(STEPS_DELTA)
+
+
+def test_stepwise_references_reproduce_their_fixtures():
+    from oracle.recurrence import delta_steps_reference, srwm_steps_reference
+    g = np.load(STEPS_SRWM)
+    t = torch.from_numpy
+    x = t(g["x"]).requires_grad_(True)
+    slow = [t(g[f"slow{i}"]).requires_grad_(True) for i in range(4)]
+    out, fin = srwm_steps_reference(x, t(g["keep"]), [t(g[f"shift{i}"]) for i in range(4)], slow)
+    (out * t(g["grad_out"])).sum().backward()
+    assert rel_err(out.detach().numpy(), g["out"]) < 1e-13
+    assert rel_err(x.grad.numpy(), g["grad_x"]) < 1e-12 and rel_err(slow[0].grad.numpy(), g["grad_slow0"]) < 1e-12
+    g = np.load(STEPS_DELTA)
+    leaves = [t(g[n]).requires_grad_(True) for n in ("Q", "K", "V", "beta")]
+    out, WL = delta_steps_reference(*leaves, t(g["keep"]), t(g["W0"]))
+    (out * t(g["grad_out"])).sum().backward()
+    assert rel_err(out.detach().numpy(), g["out"]) < 1e-13 and rel_err(WL.numpy(), g["W_final"]) < 1e-13
+    for leaf, n in zip(leaves, ("grad_Q", "grad_K", "grad_V", "grad_beta")):
+        assert rel_err(leaf.grad.numpy(), g[n]) < 1e-12, n
 
 
 @pytest.mark.parametrize("path", SRWM, ids=os.path.basename)
@@ -81,3 +102,53 @@ def test_hip_matches_delta_fixture(path):
     for leaf, n in zip(leaves, ("grad_Q", "grad_K", "grad_V", "grad_beta")):
         assert rel_err(leaf.grad.cpu().numpy(), g[n]) < TOL, n
     assert np.abs(W.cpu().numpy() - g["W0"]).max() < TOL * max(1.0, np.abs(g["W_final"]).max())
+
+
+@pytest.mark.gpu
+def test_hip_chunkwise_kernels_match_the_chunk_sized_fixture():
+    """The fixture with E = M = 64 and L = 66 through the chunkwise forward and backward (fp32)."""
+    print("case chunkwise fixture", flush=True)
+    import srwm_hip
+    g = np.load(os.path.join(GOLD, "delta_n1h1l66e64m64.npz"))
+    dev = torch.device("cuda:0")
+    t = lambda a: torch.from_numpy(a).to(dev, torch.float32).contiguous()
+    q, k, v, beta, go = (t(g[n]) for n in ("Q", "K", "V", "beta", "grad_out"))
+    W = t(g["W0"]).clone()
+    new = lambda *s_: torch.empty(*s_, device=dev)
+    vold, vins, out = new(*v.shape), new(*v.shape), new(*v.shape)
+    srwm_hip.fast_weight_forward(q, k, v, beta, vold, vins, W, out, flags=srwm_hip.FLAG_CHUNKWISE)
+    assert rel_err(out.cpu().numpy(), g["out"]) < TOL and rel_err(W.cpu().numpy(), g["W_final"]) < TOL
+    gq, gk, gv, gb, gW = new(*q.shape), new(*q.shape), new(*v.shape), new(*beta.shape), new(*W.shape)
+    srwm_hip.fast_weight_backward(q, k, v, beta, vold, vins, go, W, gq, gk, gv, gb, grad_kv=gW,
+                                  flags=srwm_hip.FLAG_CHUNKWISE)
+    for a, n in ((gq, "grad_Q"), (gk, "grad_K"), (gv, "grad_V"), (gb, "grad_beta"), (gW, "grad_W")):
+        assert rel_err(a.cpu().numpy(), g[n]) < TOL, n
+
+
+@pytest.mark.gpu
+def test_hip_stepwise_operators_match_their_fixtures():
+    print("case stepwise fixtures", flush=True)
+    from fast_weight import fast_weight_delta_steps
+    from self_ref_v0 import self_ref_v0_steps
+    dev = torch.device("cuda:0")
+    t = lambda a: torch.from_numpy(a).to(dev, torch.float32).contiguous()
+    g = np.load(STEPS_SRWM)
+    x = t(g["x"]).requires_grad_(True)
+    slow = [t(g[f"slow{i}"]).requires_grad_(True) for i in range(4)]
+    N = x.shape[0]
+    fast = [t(g[f"shift{i}"]) + w.detach().repeat(N, 1, 1, 1) for i, w in enumerate(slow)]
+    out = self_ref_v0_steps(x, t(g["keep"]), *fast, *slow)
+    (out * t(g["grad_out"])).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), g["out"]) < TOL
+    assert rel_err(x.grad.cpu().numpy(), g["grad_x"]) < TOL
+    assert rel_err(slow[0].grad.cpu().numpy(), g["grad_slow0"]) < TOL
+    for i, (f_, w) in enumerate(zip(fast, slow)):
+        assert rel_err((f_ - w.detach().repeat(N, 1, 1, 1)).cpu().numpy(), g[f"final_shift{i}"]) < 5 * TOL
+    g = np.load(STEPS_DELTA)
+    leaves = [t(g[n]).requires_grad_(True) for n in ("Q", "K", "V", "beta")]
+    W = t(g["W0"]).clone()
+    out = fast_weight_delta_steps(*leaves, t(g["keep"]), W)
+    (out * t(g["grad_out"])).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), g["out"]) < TOL and rel_err(W.cpu().numpy(), g["W_final"]) < TOL
+    for leaf, n in zip(leaves, ("grad_Q", "grad_K", "grad_V", "grad_beta")):
+        assert rel_err(leaf.grad.cpu().numpy(), g[n]) < TOL, n
