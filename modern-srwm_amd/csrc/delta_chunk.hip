@@ -47,7 +47,10 @@ struct ChunkFwdP {
 };
 
 // LDS carve-up shared by the kernel and the launcher
-template <class TI, int D>
+// KS = 2: the rows of the memory are split over two groups of four waves (8 waves per workgroup,
+// two per SIMD); a pair of waves owns the same 16 columns, each half of the rows, and exchanges
+// its partial K S and Q S through LDS.
+template <class TI, int D, int KS>
 struct FwdLds {
     typedef typename PrecOf<TI>::type X;
     static constexpr int LDK = D + X::kPad, LDA = kC + X::kPad, LDD = 16 + X::kPad, LDV = kMC + 4;
@@ -62,15 +65,17 @@ struct FwdLds {
     static constexpr int oV = oD + MatD::bytes(kC);            // fp32 [C][LDV]
     static constexpr int oAd = oV + kC * LDV * 4;              // fp32 [C][LDD]: diagonal blocks of A
     static constexpr int oBt = oAd + kC * LDD * 4;             // fp32 [C]: beta
-    static constexpr int kBytes = oBt + kC * 4;
+    static constexpr int oX = oBt + kC * 4;                    // KS == 2: [8 waves][2 * kCB tiles][64 lanes] f32x4
+    static constexpr int kBytes = oX + (KS == 2 ? 8 * 2 * kCB * 64 * 16 : 0);
     static_assert(MatK::bytes(kC) % 16 == 0 && MatA::bytes(kC) % 16 == 0 && MatD::bytes(kC) % 16 == 0, "alignment");
 };
 
-template <class TI, int D, int MS>
-__global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI> p) {
-    typedef FwdLds<TI, D> Lds;
+template <class TI, int D, int MS, int KS>
+__global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP<TI> p) {
+    typedef FwdLds<TI, D, KS> Lds;
     typedef typename Lds::X X;
-    constexpr int EB = D / 16;          // 16-row blocks of the memory
+    constexpr int NT = kThreads * KS;
+    constexpr int EB = D / 16 / KS;     // 16-row blocks of the memory held by this wave
     constexpr int LDV = Lds::LDV, LDD = Lds::LDD;
     static_assert(MS * kMC == D, "column split");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -82,7 +87,11 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
     float *Ad = reinterpret_cast<float *>(smem + Lds::oAd);
     float *bts = reinterpret_cast<float *>(smem + Lds::oBt);
 
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    f32x4 *Xs = reinterpret_cast<f32x4 *>(smem + Lds::oX);
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    const int wave = wv & 3, hf = wv >> 2;           // column tile, row half
+    const int e0 = hf * EB * 16;                     // first memory row held by this wave
     const int ln = lane & 15, lq = lane >> 4;        // accumulator layout: column ln, rows 4*lq + r
     const int64_t seq = blockIdx.x / MS;
     const int m0 = (int)(blockIdx.x % MS) * kMC;     // first memory column of this workgroup
@@ -99,26 +108,27 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
 #pragma unroll
     for (int eb = 0; eb < EB; ++eb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) s[eb][r] = Wg[(eb * 16 + 4 * lq + r) * D + ln];
+        for (int r = 0; r < 4; ++r) s[eb][r] = Wg[(e0 + eb * 16 + 4 * lq + r) * D + ln];
 
     // The chunk inputs are fetched one chunk ahead into registers (all loads in flight at
     // once) and written to LDS after the previous chunk is done with it.
-    constexpr int NKQ = kC * (D / 4) / kThreads;    // 4-element groups of K (and of Q) per thread
-    constexpr int NV = kC * (kMC / 4) / kThreads;   // 4-element groups of V per thread
+    constexpr int NKQ = kC * (D / 4) / NT;    // 4-element groups of K (and of Q) per thread
+    constexpr int NV = kC * (kMC / 4) / NT;   // 4-element groups of V per thread
+    static_assert(NKQ >= 1 && NV >= 1, "too many threads for the chunk loaders");
     typename X::Raw4 kreg[NKQ], qreg[NKQ], vreg[NV];
     uint32_t breg = 0u;   // raw bits, converted in commit()
     auto prefetch = [&](int ch) {   // rows past the end are clamped here and zeroed in commit()
         const int t0 = ch * kC;
 #pragma unroll
         for (int i = 0; i < NKQ; ++i) {
-            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const int f = tid + i * NT, row = f / (D / 4), col = (f % (D / 4)) * 4;
             const int t = min(t0 + row, p.L - 1);
             kreg[i] = X::ld_raw(kb + (int64_t)t * p.ks.l + col);
             qreg[i] = X::ld_raw(qb + (int64_t)t * p.qs.l + col);
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int f = tid + i * kThreads, row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
+            const int f = tid + i * NT, row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
             vreg[i] = X::ld_raw(vb + (int64_t)min(t0 + row, p.L - 1) * p.vs.l + col);
         }
         breg = ld_bits(bb + (int64_t)min(t0 + (tid % kC), p.L - 1) * p.bs.l);
@@ -128,14 +138,14 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
         const bool full = t0 + kC <= p.L;   // only the last chunk can be ragged
 #pragma unroll
         for (int i = 0; i < NKQ; ++i) {
-            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const int f = tid + i * NT, row = f / (D / 4), col = (f % (D / 4)) * 4;
             const bool keep = full || t0 + row < p.L;
             X::st_raw(Ks, row, col, X::keep_raw(kreg[i], keep));
             X::st_raw(Qs, row, col, X::keep_raw(qreg[i], keep));
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
-            const int f = tid + i * kThreads, row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
+            const int f = tid + i * NT, row = f / (kMC / 4), col = (f % (kMC / 4)) * 4;
             const bool keep = full || t0 + row < p.L;
             *reinterpret_cast<float4 *>(Vs + row * LDV + col) = X::raw_f32(X::keep_raw(vreg[i], keep));
         }
@@ -152,15 +162,15 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
 
         // ---- A = K K^T (strict lower) and B = Q K^T (lower): 10 pairs of tiles over the 4 waves
         //      (the two tiles of a pair share their right operand)
-        for (int pix = wave; pix < 10; pix += 4) {
+        for (int pix = wv; pix < 10; pix += 4 * KS) {
             int ci, cj;
             tri_index(pix, ci, cj);
             const auto fb = [&](int eb) { return X::ldb(Ks, cj * 16 + ln, eb * 16 + 4 * lq); };
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             const f32x4 accA = mma_range<X, false, false>(
-                0, EB, [&](int eb) { return X::lda(Ks, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
+                0, D / 16, [&](int eb) { return X::lda(Ks, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
             const f32x4 accB = mma_range<X, false, false>(
-                0, EB, [&](int eb) { return X::lda(Qs, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
+                0, D / 16, [&](int eb) { return X::lda(Qs, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int row = ci * 16 + 4 * lq + r, col = cj * 16 + ln;
@@ -174,7 +184,7 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
 
         // ---- inverse of the diagonal block `wave` of I + diag(beta) strict_lower(A):
         //      column ln of X, x_i = [i == ln] - sum_{j<i} beta_i A_ij x_j
-        {
+        if (hf == 0) {
             float x[16];
             const float *ad = Ad + (wave * 16) * LDD;
 #pragma unroll
@@ -201,14 +211,31 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
             for (int cb = 0; cb < kCB; ++cb) {
                 const auto fb = [&](int eb) { return sb[eb]; };
                 pt[cb] = mma_range<X, false, true>(
-                    0, EB, [&](int eb) { return X::lda(Ks, cb * 16 + ln, eb * 16 + 4 * lq); }, fb,
+                    0, EB, [&](int eb) { return X::lda(Ks, cb * 16 + ln, e0 + eb * 16 + 4 * lq); }, fb,
                     f32x4{0.f, 0.f, 0.f, 0.f});
                 ot[cb] = mma_range<X, false, true>(
-                    0, EB, [&](int eb) { return X::lda(Qs, cb * 16 + ln, eb * 16 + 4 * lq); }, fb,
+                    0, EB, [&](int eb) { return X::lda(Qs, cb * 16 + ln, e0 + eb * 16 + 4 * lq); }, fb,
                     f32x4{0.f, 0.f, 0.f, 0.f});
             }
         }
-        __syncthreads();   // the four inverses are visible
+        if constexpr (KS == 2) {   // hand the partial products to the wave that holds the other rows
+#pragma unroll
+            for (int cb = 0; cb < kCB; ++cb) {
+                Xs[(wv * 2 * kCB + cb) * 64 + lane] = pt[cb];
+                Xs[(wv * 2 * kCB + kCB + cb) * 64 + lane] = ot[cb];
+            }
+        }
+        __syncthreads();   // the four inverses (and the partial products) are visible
+        if constexpr (KS == 2) {
+            const int ow = wv ^ 4;
+#pragma unroll
+            for (int cb = 0; cb < kCB; ++cb) {
+                // both waves of a pair add in the same order (lower rows first): identical results
+                const f32x4 a = Xs[(ow * 2 * kCB + cb) * 64 + lane], b = Xs[(ow * 2 * kCB + kCB + cb) * 64 + lane];
+                pt[cb] = hf == 0 ? pt[cb] + a : a + pt[cb];
+                ot[cb] = hf == 0 ? ot[cb] + b : b + ot[cb];
+            }
+        }
 
         // ---- everything below is per wave (its 16 columns), no synchronisation
         // block forward substitution, one 16-row block at a time
@@ -231,6 +258,7 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
             // out = Q S + tril(B) U
             ot[a] = mma_range<X, true, true>(
                 0, a + 1, [&](int b) { return X::lda(Bs, a * 16 + ln, b * 16 + 4 * lq); }, fu, ot[a]);
+            if (a % KS == hf)   // the two waves of a pair share the stores
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int t = t0 + a * 16 + 4 * lq + r;
@@ -246,7 +274,7 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
 #pragma unroll
         for (int eb = 0; eb < EB; ++eb)
             s[eb] = mma_range<X, false, true>(
-                0, kCB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, eb * 16 + ln); },
+                0, kCB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, e0 + eb * 16 + ln); },
                 [&](int cb) { return ub[cb]; }, s[eb]);
         __syncthreads();   // every wave is done with Ks, Qs, Vs, As, Bs
         if (ch + 1 < nchunks) {
@@ -258,16 +286,17 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_chunk_kernel(ChunkFwdP<TI>
 #pragma unroll
     for (int eb = 0; eb < EB; ++eb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) Wg[(eb * 16 + 4 * lq + r) * D + ln] = s[eb][r];
+        for (int r = 0; r < 4; ++r) Wg[(e0 + eb * 16 + 4 * lq + r) * D + ln] = s[eb][r];
 }
 
-template <class TI, int D, int MS>
+template <class TI, int D, int MS, int KS>
 int launch_chunk(const ChunkFwdP<TI> &p, hipStream_t s) {
-    constexpr size_t lds = FwdLds<TI, D>::kBytes;
-    hipError_t err = hipFuncSetAttribute((const void *)delta_fwd_chunk_kernel<TI, D, MS>,
+    constexpr size_t lds = FwdLds<TI, D, KS>::kBytes;
+    static_assert(lds <= kMaxLdsBytes, "LDS budget");
+    hipError_t err = hipFuncSetAttribute((const void *)delta_fwd_chunk_kernel<TI, D, MS, KS>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return (int)err;
-    hipLaunchKernelGGL((delta_fwd_chunk_kernel<TI, D, MS>), dim3(p.N * p.H * MS), dim3(kThreads), lds, s, p);
+    hipLaunchKernelGGL((delta_fwd_chunk_kernel<TI, D, MS, KS>), dim3(p.N * p.H * MS), dim3(kThreads * KS), lds, s, p);
     return (int)hipGetLastError();
 }
 
@@ -280,8 +309,8 @@ template <class TI>
 int dispatch_chunk(const ChunkFwdP<TI> &p, int D, hipStream_t s) {
     if (!rows_ok(p.Q, p.qs) || !rows_ok(p.K, p.ks) || !rows_ok(p.V, p.vs)) return -1;
     switch (D) {
-        case 128: return launch_chunk<TI, 128, 2>(p, s);
-        case 64: return launch_chunk<TI, 64, 1>(p, s);
+        case 128: return launch_chunk<TI, 128, 2, PrecOf<TI>::type::kBf ? 2 : 1>(p, s);
+        case 64: return launch_chunk<TI, 64, 1, 1>(p, s);
         default: return -1;
     }
 }
