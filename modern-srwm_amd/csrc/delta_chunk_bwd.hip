@@ -57,7 +57,10 @@ struct ChunkBwdP {
 // ------------------------------------------------------------------------------------------
 // Column sweep
 // ------------------------------------------------------------------------------------------
-template <class TI, int D>
+// KS = 2: the rows of S and dS are split over two groups of four waves (8 waves per workgroup, two
+// per SIMD); a pair of waves owns the same 16 columns, each half of the rows, and exchanges its
+// partial K dS' through LDS.
+template <class TI, int D, int KS>
 struct ColLds {
     typedef typename PrecOf<TI>::type X;
     static constexpr int C = 64;
@@ -73,15 +76,17 @@ struct ColLds {
     static constexpr int oAd = oD + MatD::bytes(C);            // fp32 [C][LDD]: diagonal blocks of A^T
     static constexpr int oBt = oAd + C * LDD * 4;              // fp32 [C]: beta
     static constexpr int oGb = oBt + C * 4;                    // fp32 [4][C]: per-wave parts of grad_beta
-    static constexpr int kBytes = oGb + 4 * C * 4;
+    static constexpr int oX = oGb + 4 * C * 4;                 // KS == 2: [8 waves][C/16 tiles][64 lanes] f32x4
+    static constexpr int kBytes = oX + (KS == 2 ? 8 * (C / 16) * 64 * 16 : 0);
     static_assert(MatK::bytes(C) % 16 == 0 && MatA::bytes(C) % 16 == 0 && MatD::bytes(C) % 16 == 0, "alignment");
 };
 
-template <class TI, int D, int MS>
-__global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP<TI> p) {
-    typedef ColLds<TI, D> Lds;
+template <class TI, int D, int MS, int KS>
+__global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(ChunkBwdP<TI> p) {
+    typedef ColLds<TI, D, KS> Lds;
     typedef typename Lds::X X;
-    constexpr int C = Lds::C, CB = C / 16, EB = D / 16, LDD = Lds::LDD;
+    constexpr int NT = kThreads * KS;
+    constexpr int C = Lds::C, CB = C / 16, EB = D / 16 / KS, LDD = Lds::LDD;   // EB: row blocks held by this wave
     static_assert(MS * kWC == D, "column split");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const typename Lds::MatK Ks(smem + Lds::oK, C), Qs(smem + Lds::oQ, C);
@@ -91,8 +96,11 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP
     float *Ad = reinterpret_cast<float *>(smem + Lds::oAd);
     float *bts = reinterpret_cast<float *>(smem + Lds::oBt);
     float *gbp = reinterpret_cast<float *>(smem + Lds::oGb);
+    f32x4 *Xs = reinterpret_cast<f32x4 *>(smem + Lds::oX);
 
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    const int wave = wv & 3, hf = wv >> 2;          // column tile, row half
+    const int e0 = hf * EB * 16;                    // first memory row held by this wave
     const int ln = lane & 15, lq = lane >> 4;
     const int64_t seq = blockIdx.x / MS;
     const int m0 = (int)(blockIdx.x % MS) * kWC + 16 * wave;   // first memory column of this wave
@@ -113,21 +121,22 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP
     for (int eb = 0; eb < EB; ++eb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            const int o = (eb * 16 + 4 * lq + r) * D;
+            const int o = (e0 + eb * 16 + 4 * lq + r) * D;
             s[eb][r] = Wg[o];
             ds[eb][r] = gWg ? gWg[o] : 0.f;
         }
 
     // next chunk's inputs: K, Q rows for LDS; U, dOut, V, v_old directly in accumulator layout
-    constexpr int NKQ = C * (D / 4) / kThreads;
+    constexpr int NKQ = C * (D / 4) / NT;
     typename X::Raw4 kreg[NKQ], qreg[NKQ];
-    f32x4 pu[CB], po[CB];
-    uint32_t pg[CB][4], pv[CB][4], breg = 0u;   // raw bits, converted in commit()
+    // V and v_old only enter grad_beta: a wave loads them for the row blocks whose results it stores
+    f32x4 pu[CB], po[CB / KS];
+    uint32_t pg[CB][4], pv[CB / KS][4], breg = 0u;   // raw bits, converted in commit()
     auto prefetch = [&](int ch) {
         const int t0 = ch * C;
 #pragma unroll
         for (int i = 0; i < NKQ; ++i) {
-            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const int f = tid + i * NT, row = f / (D / 4), col = (f % (D / 4)) * 4;
             const int t = min(t0 + row, p.L - 1);
             kreg[i] = X::ld_raw(kb + (int64_t)t * p.ks.l + col);
             qreg[i] = X::ld_raw(qb + (int64_t)t * p.qs.l + col);
@@ -138,19 +147,25 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP
             for (int r = 0; r < 4; ++r) {
                 const int64_t t = min(t0 + cb * 16 + 4 * lq + r, p.L - 1);
                 pu[cb][r] = vib[t * D];
-                po[cb][r] = vob[t * D];
                 pg[cb][r] = ld_bits(gob + t * p.gs.l);
-                pv[cb][r] = ld_bits(vb + t * p.vs.l);
+            }
+#pragma unroll
+        for (int j = 0; j < CB / KS; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int64_t t = min(t0 + (j * KS + hf) * 16 + 4 * lq + r, p.L - 1);
+                po[j][r] = vob[t * D];
+                pv[j][r] = ld_bits(vb + t * p.vs.l);
             }
         breg = ld_bits(bb + (int64_t)min(t0 + (tid % C), p.L - 1) * p.bs.l);
     };
-    f32x4 u[CB], g[CB], vd[CB];   // this chunk: U, dOut, V - v_old (rows past the end zeroed)
+    f32x4 u[CB], g[CB], vd[CB / KS];   // this chunk: U, dOut, V - v_old (rows past the end zeroed)
     auto commit = [&](int ch) {
         const int t0 = ch * C;
         const bool full = t0 + C <= p.L;
 #pragma unroll
         for (int i = 0; i < NKQ; ++i) {
-            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const int f = tid + i * NT, row = f / (D / 4), col = (f % (D / 4)) * 4;
             const bool keep = full || t0 + row < p.L;
             X::st_raw(Ks, row, col, X::keep_raw(kreg[i], keep));
             X::st_raw(Qs, row, col, X::keep_raw(qreg[i], keep));
@@ -162,7 +177,13 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP
                 const float m = (full || t0 + cb * 16 + 4 * lq + r < p.L) ? 1.f : 0.f;
                 u[cb][r] = pu[cb][r] * m;
                 g[cb][r] = bits_f32<TI>(pg[cb][r]) * m;
-                vd[cb][r] = (bits_f32<TI>(pv[cb][r]) - po[cb][r]) * m;
+            }
+#pragma unroll
+        for (int j = 0; j < CB / KS; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float m = (full || t0 + (j * KS + hf) * 16 + 4 * lq + r < p.L) ? 1.f : 0.f;
+                vd[j][r] = (bits_f32<TI>(pv[j][r]) - po[j][r]) * m;
             }
         if (tid < C) bts[tid] = (t0 + tid < p.L) ? bits_f32<TI>(breg) : 0.f;
     };
@@ -177,15 +198,15 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP
 
         // ---- (K K^T)^T strict upper and tril(Q K^T)^T: 10 pairs of tiles (a pair shares its right
         //      operand), stored transposed
-        for (int pix = wave; pix < 10; pix += 4) {
+        for (int pix = wv; pix < 10; pix += 4 * KS) {
             int ci, cj;
             tri_index(pix, ci, cj);
             const auto fb = [&](int eb) { return X::ldb(Ks, cj * 16 + ln, eb * 16 + 4 * lq); };
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             const f32x4 accA = mma_range<X, false, false>(
-                0, EB, [&](int eb) { return X::lda(Ks, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
+                0, D / 16, [&](int eb) { return X::lda(Ks, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
             const f32x4 accB = mma_range<X, false, false>(
-                0, EB, [&](int eb) { return X::lda(Qs, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
+                0, D / 16, [&](int eb) { return X::lda(Qs, ci * 16 + ln, eb * 16 + 4 * lq); }, fb, zero);
             float va[4], vb_[4];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -202,7 +223,7 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP
 
         // ---- inverse of the diagonal block `wave` of I + A^T diag(beta) (unit upper triangular):
         //      column ln, x_i = [i == ln] - sum_{j>i} A^T_ij beta_j x_j, from the bottom row up
-        {
+        if (hf == 0) {
             float x[16];
             const float *ad = Ad + (wave * 16) * LDD;
 #pragma unroll
@@ -231,19 +252,27 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP
 #pragma unroll
             for (int eb = 0; eb < EB; ++eb)
                 s[eb] = mma_range<X, false, true>(
-                    0, CB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, eb * 16 + ln); },
+                    0, CB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, e0 + eb * 16 + ln); },
                     [&](int cb) { return nub[cb]; }, s[eb]);
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 du[cb] = mma_range<X, false, true>(
-                    0, EB, [&](int eb) { return X::lda(Ks, cb * 16 + ln, eb * 16 + 4 * lq); },
+                    0, EB, [&](int eb) { return X::lda(Ks, cb * 16 + ln, e0 + eb * 16 + 4 * lq); },
                     [&](int eb) { return dsb[eb]; }, f32x4{0.f, 0.f, 0.f, 0.f});
-                du[cb] = mma_range<X, true, false>(
-                    cb, CB, [&](int b) { return X::lda(BT, cb * 16 + ln, b * 16 + 4 * lq); },
-                    [&](int b) { return gob_[b]; }, du[cb]);
+                if constexpr (KS == 2) Xs[(wv * CB + cb) * 64 + lane] = du[cb];   // partial K dS' of this half
             }
         }
-        __syncthreads();   // the four inverses are visible
+        __syncthreads();   // the four inverses (and the partial products) are visible
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            if constexpr (KS == 2) {   // both waves of a pair add in the same order: identical results
+                const f32x4 o = Xs[((wv ^ 4) * CB + cb) * 64 + lane];
+                du[cb] = hf == 0 ? du[cb] + o : o + du[cb];
+            }
+            du[cb] = mma_range<X, true, false>(
+                cb, CB, [&](int b) { return X::lda(BT, cb * 16 + ln, b * 16 + 4 * lq); },
+                [&](int b) { return gob_[b]; }, du[cb]);
+        }
 
         // ---- block back substitution, last 16-row block first
         typename X::B nyb[CB];
@@ -255,29 +284,30 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_col_kernel(ChunkBwdP
             const f32x4 dr = X::template mma<true, true>(X::lda(Di, a * 16 + ln, 4 * lq), X::accb(rhs),
                                                          f32x4{0.f, 0.f, 0.f, 0.f});
             f32x4 y;
-            float pb[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                y[r] = bts[a * 16 + 4 * lq + r] * dr[r];
-                pb[r] = dr[r] * vd[a][r];
-            }
+            for (int r = 0; r < 4; ++r) y[r] = bts[a * 16 + 4 * lq + r] * dr[r];
             nyb[a] = X::accb(-y);
-            group_sum_n<16, 4>(pb);   // over the wave's 16 columns
+            if (a % KS == hf) {   // wave-uniform: the two waves of a pair share the stores
+                float pb[4];
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int t = t0 + a * 16 + 4 * lq + r;
-                if (t < p.L) p.gV[(seq * p.L + t) * D + m0 + ln] = y[r];
-                gbp[wave * C + a * 16 + 4 * lq + r] = pb[r];   // 16 lanes, same value, same word
+                for (int r = 0; r < 4; ++r) pb[r] = dr[r] * vd[a / KS][r];
+                group_sum_n<16, 4>(pb);   // over the wave's 16 columns
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int t = t0 + a * 16 + 4 * lq + r;
+                    if (t < p.L) p.gV[(seq * p.L + t) * D + m0 + ln] = y[r];
+                    gbp[wave * C + a * 16 + 4 * lq + r] = pb[r];   // 16 lanes, same value, same word
+                }
             }
         }
         // ---- dS = dS' + Q^T dOut - K^T Y
 #pragma unroll
         for (int eb = 0; eb < EB; ++eb) {
             ds[eb] = mma_range<X, false, false>(
-                0, CB, [&](int cb) { return X::lda_t(Qs, cb * 16 + 4 * lq, eb * 16 + ln); },
+                0, CB, [&](int cb) { return X::lda_t(Qs, cb * 16 + 4 * lq, e0 + eb * 16 + ln); },
                 [&](int cb) { return gob_[cb]; }, ds[eb]);
             ds[eb] = mma_range<X, false, true>(
-                0, CB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, eb * 16 + ln); },
+                0, CB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, e0 + eb * 16 + ln); },
                 [&](int cb) { return nyb[cb]; }, ds[eb]);
         }
         __syncthreads();   // every wave is done with the chunk's LDS; grad_beta parts are visible
@@ -530,11 +560,11 @@ __global__ void zero_words_kernel(float *a, int64_t n) {
     for (int64_t j = i; j < n; j += stride) a[j] = 0.f;
 }
 
-template <class TI, int D, int MS, int C2>
+template <class TI, int D, int MS, int C2, int KS>
 int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
-    constexpr int lds1 = ColLds<TI, D>::kBytes, lds2 = RowLds<TI, D, C2>::kBytes;
+    constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2>::kBytes;
     static_assert(lds1 <= (int)kMaxLdsBytes && lds2 <= (int)kMaxLdsBytes, "LDS budget");
-    hipError_t err = hipFuncSetAttribute((const void *)delta_bwd_chunk_col_kernel<TI, D, MS>,
+    hipError_t err = hipFuncSetAttribute((const void *)delta_bwd_chunk_col_kernel<TI, D, MS, KS>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds1);
     if (err != hipSuccess) return (int)err;
     err = hipFuncSetAttribute((const void *)delta_bwd_chunk_row_kernel<TI, D, MS, C2>,
@@ -543,7 +573,7 @@ int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
     const int grid = p.N * p.H * MS;
     if (MS > 1)   // two workgroups of the column sweep add their parts of grad_beta
         hipLaunchKernelGGL(zero_words_kernel, dim3(256), dim3(256), 0, s, p.gbeta, (int64_t)p.N * p.H * p.L);
-    hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS>), dim3(grid), dim3(kThreads), lds1, s, p);
+    hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS, KS>), dim3(grid), dim3(kThreads * KS), lds1, s, p);
     hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2>), dim3(grid), dim3(kThreads), lds2, s, p);
     return (int)hipGetLastError();
 }
@@ -562,8 +592,8 @@ int dispatch_chunk_bwd(const ChunkBwdP<TI> &p, int D, hipStream_t s) {
         return -1;
     constexpr bool bf = PrecOf<TI>::type::kBf;
     switch (D) {
-        case 128: return launch_chunk_bwd<TI, 128, 2, bf ? 64 : 32>(p, s);
-        case 64: return launch_chunk_bwd<TI, 64, 1, 64>(p, s);
+        case 128: return launch_chunk_bwd<TI, 128, 2, bf ? 64 : 32, bf ? 2 : 1>(p, s);
+        case 64: return launch_chunk_bwd<TI, 64, 1, 64, 1>(p, s);
         default: return -1;
     }
 }
