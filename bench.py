@@ -16,7 +16,7 @@ achieved HBM rate of the operator's I/O contract.  `cpu_baseline` is the per-tim
 PyTorch recurrence (oracle/recurrence.py) timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, srwm_c3_steps, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk}.
+{srwm_c3, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk}.
 """
 import argparse
 import json
@@ -51,6 +51,8 @@ WORKLOADS = {
     # the RL learner's regime on the same shape: gradient cut at the carried state, 5 % resets;
     # one launch for the unroll (forward) + readout-gradient replay + the batched x (x) g product
     "srwm_c3_steps": ("srwm_steps", 32, 8, 100, 32),
+    # the same shape with the output block 3E+1 = 97 columns wide (the self_ref_v1 operator)
+    "srwm_wide_c3": ("srwm_wide", 32, 8, 100, 32),
     "delta_c2": ("delta", 32, 8, 256, 64),
     "delta_c5f32": ("delta", 8, 16, 4096, 128),
     "delta_c5": ("delta_bf16", 8, 16, 4096, 128),     # bf16 q/k/v/beta/out/grads, fp32 memory
@@ -61,19 +63,21 @@ WORKLOADS = {
 }
 
 
-def srwm_setup(N, H, L, E, dev):
+def srwm_setup(N, H, L, E, dev, Y=None):
     import torch
+    Y = E if Y is None else Y
     g = torch.Generator().manual_seed(0)
     x = torch.randn(N, H, L, E, generator=g)
-    W0 = [torch.randn(1, H, E, E, generator=g) * 0.02 for _ in range(3)]
+    W0 = [torch.randn(1, H, E, w, generator=g) * 0.02 for w in (Y, E, E)]
     W0.append(torch.randn(1, H, E, 4, generator=g) * 0.02)
-    go = torch.randn(N, H, L, E, generator=g)
+    go = torch.randn(N, H, L, Y, generator=g)
     t = dict(x=x.to(dev), go=go.to(dev), W0=[w.repeat(N, 1, 1, 1).to(dev) for w in W0])
     t["W"] = [torch.empty_like(w) for w in t["W0"]]
     big = lambda: torch.empty(N, H, L, E, device=dev)
+    wide = lambda: torch.empty(N, H, L, Y, device=dev)
     small = lambda: torch.empty(N, H, L, 4, device=dev)
-    t["saved"] = [big(), big(), small(), big(), big(), big(), small()]
-    t["out"] = big()
+    t["saved"] = [big(), big(), small(), wide(), big(), big(), small()]
+    t["out"] = wide()
     t["gx"] = big()
     t["gW"] = [torch.empty_like(w) for w in t["W0"]]
     return t
@@ -205,6 +209,10 @@ def algorithmic_bytes(op, N, H, L, E):
     if op == "srwm":
         S = E * (3 * E + 4)
         return 3 * S * 4 * hs, 6 * S * 4 * hs, (15 * E + 16) * 4 * hs + 4 * S * 4 * N * H
+    if op == "srwm_wide":    # as above with Y = 3E+1 output columns: y, y_diff, grad_out are Y wide
+        Y = 3 * E + 1
+        S = E * (Y + 2 * E + 4)
+        return 3 * S * 4 * hs, 6 * S * 4 * hs, (11 * E + 4 * Y + 16) * 4 * hs + 4 * S * 4 * N * H
     if op == "srwm_steps":   # forward as above; the replay reads and writes the E x E y block once per step
         S = E * (3 * E + 4)
         return 3 * S * 4 * hs, 2 * E * E * 4 * hs, ((7 * E + 8) + (4 * E + 4)) * 4 * hs + (2 * S + E * E) * 4 * N * H
@@ -225,11 +233,12 @@ def cpu_baseline(op, N, H, L, E, budget_s=20.0):
     g = torch.Generator().manual_seed(0)
 
     def run(n):
-        if op == "srwm":
+        if op in ("srwm", "srwm_wide"):
+            Y = E if op == "srwm" else 3 * E + 1
             x = torch.randn(n, H, L, E, generator=g).requires_grad_(True)
-            W = [(torch.randn(n, H, E, E, generator=g) * 0.02).requires_grad_(True) for _ in range(3)]
+            W = [(torch.randn(n, H, E, w, generator=g) * 0.02).requires_grad_(True) for w in (Y, E, E)]
             W.append((torch.randn(n, H, E, 4, generator=g) * 0.02).requires_grad_(True))
-            go = torch.randn(n, H, L, E, generator=g)
+            go = torch.randn(n, H, L, Y, generator=g)
             t0 = time.perf_counter()
             out, _ = srwm_recurrence(x, *W)
         else:
@@ -313,6 +322,8 @@ def main():
     op, N, H, L, E = WORKLOADS[a.workload]
     if op == "srwm":
         step, t = srwm_step, srwm_setup(N, H, L, E, dev)
+    elif op == "srwm_wide":
+        step, t = srwm_step, srwm_setup(N, H, L, E, dev, 3 * E + 1)
     elif op == "srwm_steps":
         step, t = srwm_steps_step, srwm_steps_setup(N, H, L, E, dev)
     else:
@@ -369,7 +380,8 @@ def main():
         res["roofline_fwd_bwd"]["frac_of_measured_lds_peak"] = round(
             res["roofline_fwd_bwd"]["achieved"] / lds_meas, 4)
     if not a.no_cpu_baseline:
-        res["cpu_baseline"] = cpu_baseline("srwm" if op.startswith("srwm") else "delta", N, H, L, E, a.cpu_budget)
+        res["cpu_baseline"] = cpu_baseline("srwm_wide" if op == "srwm_wide" else "srwm" if op.startswith("srwm") else "delta",
+                                           N, H, L, E, a.cpu_budget)
     print(json.dumps(res))
 
 

@@ -93,6 +93,35 @@ SRWM_API int srwm_backward_f32(const float *x, const int64_t x_strides[3],
                       int N, int H, int L, int E, unsigned flags, void *stream);
 
 /*
+ * SRWM forward / backward with an output block Y columns wide.  Replace self_ref_forward_v1() and
+ * self_ref_backward_v1(), reinforcement_learning/torchbeast/self_ref_v1/self_ref_v1.cu:538-635
+ * (kernel :27-534) and :1551-1656 (kernel :639-1547), where Y = 3E+1: the readout supplies the
+ * query | key | value | beta pre-activations of a following fast-weight layer.  The recurrence is
+ * the one of srwm_forward_f32 with the state W = [W_y | W_q | W_k | w_b]  (E x (Y+2E+4)); every
+ * column of the y block is written with the first of the four learning rates.
+ *   Wy, gWy                 dense [N,H,E,Y]
+ *   out, ydiff              dense [N,H,L,Y];  grad_out strided [N,H,L,Y]
+ *   everything else         as in srwm_forward_f32 / srwm_backward_f32
+ * Any Y >= 1 is accepted; Y == E is the plain operator.  SRWM_ESIZE when E x (Y+2E+4) floats (twice
+ * that in the backward) do not fit in the CU's LDS.
+ */
+SRWM_API int srwm_forward_wide_f32(const float *x, const int64_t x_strides[3],
+                     float *Wy, float *Wq, float *Wk, float *wb,
+                     float *q, float *k, float *beta,
+                     float *ydiff, float *qdiff, float *kdiff, float *bdiff,
+                     float *out,
+                     int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+
+SRWM_API int srwm_backward_wide_f32(const float *x, const int64_t x_strides[3],
+                      const float *q, const float *k, const float *beta,
+                      const float *ydiff, const float *qdiff, const float *kdiff,
+                      const float *bdiff,
+                      const float *grad_out, const int64_t grad_out_strides[3],
+                      const float *Wy, const float *Wq, const float *Wk, const float *wb,
+                      float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb,
+                      int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+
+/*
  * SRWM forward over all steps of an unroll with per-step resets.  No counterpart function in the
  * reference: it fuses the loop in which its RL learner calls the L = 1 operator once per time
  * step, multiplying the carried shift by `notdone` first (reinforcement_learning/

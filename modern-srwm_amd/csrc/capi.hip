@@ -37,6 +37,8 @@ int max_E_for(size_t (*bytes)(int), size_t limit) {
     return e;
 }
 
+size_t srwm_fwd_sq(int e) { return srwm_fwd_generic_lds_bytes(e, e); }
+size_t srwm_bwd_sq(int e) { return srwm_bwd_generic_lds_bytes(e, e); }
 size_t delta_fwd_sq(int e) { return delta_fwd_generic_lds_bytes(e, e); }
 size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
@@ -59,8 +61,8 @@ const char *srwm_hip_strerror(int code) {
 
 int srwm_hip_limits(int *srwm_fwd_max_E, int *srwm_bwd_max_E, int *delta_max_EM) {
     const size_t lim = lds_limit();
-    if (srwm_fwd_max_E) *srwm_fwd_max_E = max_E_for(srwm_fwd_generic_lds_bytes, lim);
-    if (srwm_bwd_max_E) *srwm_bwd_max_E = max_E_for(srwm_bwd_generic_lds_bytes, lim);
+    if (srwm_fwd_max_E) *srwm_fwd_max_E = max_E_for(srwm_fwd_sq, lim);
+    if (srwm_bwd_max_E) *srwm_bwd_max_E = max_E_for(srwm_bwd_sq, lim);
     if (delta_max_EM) {
         const int f = max_E_for(delta_fwd_sq, lim), b = max_E_for(delta_bwd_sq, lim);
         *delta_max_EM = f < b ? f : b;
@@ -68,24 +70,33 @@ int srwm_hip_limits(int *srwm_fwd_max_E, int *srwm_bwd_max_E, int *delta_max_EM)
     return SRWM_OK;
 }
 
-int srwm_forward_f32(const float *x, const int64_t xs[3], float *Wy, float *Wq, float *Wk, float *wb,
-                     float *q, float *k, float *beta, float *ydiff, float *qdiff, float *kdiff,
-                     float *bdiff, float *out, int N, int H, int L, int E, unsigned flags,
-                     void *stream) {
+int srwm_forward_wide_f32(const float *x, const int64_t xs[3], float *Wy, float *Wq, float *Wk,
+                          float *wb, float *q, float *k, float *beta, float *ydiff, float *qdiff,
+                          float *kdiff, float *bdiff, float *out, int N, int H, int L, int E, int Y,
+                          unsigned flags, void *stream) {
     if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
         !out || !xs)
         return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || (flags & ~(SRWM_FLAG_GENERIC))) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || (flags & ~(SRWM_FLAG_GENERIC))) return SRWM_EINVAL;
     if (!stride_ok(xs, N, H, L, E)) return SRWM_ESTRIDE;
     SrwmFwdParams p{x, xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff,
                     out, N, H, L, E};
+    p.Y = Y;
     hipStream_t s = (hipStream_t)stream;
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_fwd_tiled(p, s);
         if (r >= 0) return r;
     }
-    if (srwm_fwd_generic_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
+    if (srwm_fwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_srwm_fwd_generic(p, s);
+}
+
+int srwm_forward_f32(const float *x, const int64_t xs[3], float *Wy, float *Wq, float *Wk, float *wb,
+                     float *q, float *k, float *beta, float *ydiff, float *qdiff, float *kdiff,
+                     float *bdiff, float *out, int N, int H, int L, int E, unsigned flags,
+                     void *stream) {
+    return srwm_forward_wide_f32(x, xs, Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff, out, N, H,
+                                 L, E, E, flags, stream);
 }
 
 int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
@@ -100,13 +111,13 @@ int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *kee
     if (!dims_ok(N, H, L, E) || (flags & ~(SRWM_FLAG_GENERIC))) return SRWM_EINVAL;
     if (!stride_ok(xs, N, H, L, E)) return SRWM_ESTRIDE;
     SrwmFwdParams p{x, xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff,
-                    out, N, H, L, E, keep, sWy, sWq, sWk, swb};
+                    out, N, H, L, E, keep, sWy, sWq, sWk, swb, E};
     hipStream_t s = (hipStream_t)stream;
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_fwd_tiled(p, s);
         if (r >= 0) return r;
     }
-    if (srwm_fwd_generic_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
+    if (srwm_fwd_generic_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
     return launch_srwm_fwd_generic(p, s);
 }
 
@@ -157,28 +168,39 @@ int delta_readout_replay_f32(const float *K, const int64_t ks[3], const float *v
     return launch_replay(p, (hipStream_t)stream);
 }
 
+int srwm_backward_wide_f32(const float *x, const int64_t xs[3], const float *q, const float *k,
+                           const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
+                           const float *bdiff, const float *grad_out, const int64_t gs[3],
+                           const float *Wy, const float *Wq, const float *Wk, const float *wb,
+                           float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, int N, int H,
+                           int L, int E, int Y, unsigned flags, void *stream) {
+    if (!x || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff || !grad_out || !Wy || !Wq ||
+        !Wk || !wb || !grad_x || !gWy || !gWq || !gWk || !gwb || !xs || !gs)
+        return SRWM_EINVAL;
+    const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || mode == 3u ||
+        (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)))
+        return SRWM_EINVAL;
+    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, Y)) return SRWM_ESTRIDE;
+    SrwmBwdParams p{x, xs[0], xs[1], xs[2], q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out,
+                    gs[0], gs[1], gs[2], Wy, Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, N, H, L, E, mode, Y};
+    hipStream_t s = (hipStream_t)stream;
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_srwm_bwd_tiled(p, s);
+        if (r >= 0) return r;
+    }
+    if (srwm_bwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
+    return launch_srwm_bwd_generic(p, s);
+}
+
 int srwm_backward_f32(const float *x, const int64_t xs[3], const float *q, const float *k,
                       const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
                       const float *bdiff, const float *grad_out, const int64_t gs[3], const float *Wy,
                       const float *Wq, const float *Wk, const float *wb, float *grad_x, float *gWy,
                       float *gWq, float *gWk, float *gwb, int N, int H, int L, int E, unsigned flags,
                       void *stream) {
-    if (!x || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff || !grad_out || !Wy || !Wq ||
-        !Wk || !wb || !grad_x || !gWy || !gWq || !gWk || !gwb || !xs || !gs)
-        return SRWM_EINVAL;
-    const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
-    if (!dims_ok(N, H, L, E) || mode == 3u || (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)))
-        return SRWM_EINVAL;
-    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, E)) return SRWM_ESTRIDE;
-    SrwmBwdParams p{x, xs[0], xs[1], xs[2], q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out,
-                    gs[0], gs[1], gs[2], Wy, Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, N, H, L, E, mode};
-    hipStream_t s = (hipStream_t)stream;
-    if (!(flags & SRWM_FLAG_GENERIC)) {
-        const int r = launch_srwm_bwd_tiled(p, s);
-        if (r >= 0) return r;
-    }
-    if (srwm_bwd_generic_lds_bytes(E) > lds_limit()) return SRWM_ESIZE;
-    return launch_srwm_bwd_generic(p, s);
+    return srwm_backward_wide_f32(x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, Wy, Wq, Wk,
+                                  wb, grad_x, gWy, gWq, gWk, gwb, N, H, L, E, E, flags, stream);
 }
 
 int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],

@@ -18,7 +18,8 @@ struct SrwmFwdParams {
     // optional per-step reset: before step t of batch row n the state is replaced by the shared
     // weights of its head wherever keep[n*L + t] == 0 (keep == nullptr: never)
     const float *keep;
-    const float *sWy, *sWq, *sWk, *swb;   // [H,E,E] x 3, [H,E,4]
+    const float *sWy, *sWq, *sWk, *swb;   // [H,E,Y], [H,E,E] x 2, [H,E,4]
+    int Y;   // columns of W_y, out and ydiff (E for the plain operator)
 };
 
 struct SrwmBwdParams {
@@ -31,6 +32,7 @@ struct SrwmBwdParams {
     float *gx, *gWy, *gWq, *gWk, *gwb;
     int N, H, L, E;
     unsigned grad_state_mode;  // SRWM_GRAD_STATE_*
+    int Y;   // columns of W_y, grad_out, ydiff and gWy (E for the plain operator)
 };
 
 struct Strided3 {
@@ -111,8 +113,8 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // ---- launchers (each returns a hipError_t as int, 0 = launched) -----------------
 // LDS-resident kernels that accept any E (M) whose state fits in the CU's LDS.
-size_t srwm_fwd_generic_lds_bytes(int E);
-size_t srwm_bwd_generic_lds_bytes(int E);
+size_t srwm_fwd_generic_lds_bytes(int E, int Y);
+size_t srwm_bwd_generic_lds_bytes(int E, int Y);
 size_t delta_fwd_generic_lds_bytes(int E, int M);
 size_t delta_bwd_generic_lds_bytes(int E, int M);
 int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s);

@@ -1,6 +1,8 @@
 // SRWM forward / backward for ANY head size: one workgroup per (batch, head) sequence,
-// the packed state W = [W_y | W_q | W_k | w_b] (E x (3E+4), plus the gradient G in the
-// backward) resident in LDS for the whole sequence, one launch for all L steps.
+// the packed state W = [W_y | W_q | W_k | w_b] (E x (Y+2E+4), plus the gradient G in the
+// backward) resident in LDS for the whole sequence, one launch for all L steps.  Y, the
+// width of the output block, is E for the plain operator and 3E+1 for the variant whose
+// readout feeds a following fast-weight layer.
 //
 // This is the fallback behind the register-resident kernels of srwm_tiled.hip: column
 // passes give one thread one column (bank-conflict free: consecutive lanes read
@@ -8,7 +10,8 @@
 // shuffle reduction.  No atomics anywhere; every output element is written once.
 //
 // Replaces self_ref_forward_kernel / self_ref_backward_kernel of the reference
-// (supervised_learning/self_ref_v0/self_ref_v0.cu:24-432, :534-1234).
+// (supervised_learning/self_ref_v0/self_ref_v0.cu:24-432, :534-1234) and their wide-output
+// siblings (reinforcement_learning/torchbeast/self_ref_v1/self_ref_v1.cu:27-534, :639-1547).
 #include "common.h"
 
 namespace fw {
@@ -21,19 +24,28 @@ constexpr int kWaves = kThreads / kWave;
 __device__ __forceinline__ int padded_cols(int C) { return C | 1; }
 
 __device__ __forceinline__ void load_state(float *W, int Cp, const float *Wy, const float *Wq,
-                                           const float *Wk, const float *wb, int E, int tid) {
+                                           const float *Wk, const float *wb, int E, int Y, int tid) {
+    for (int i = tid; i < E * Y; i += kThreads) {
+        const int e = i / Y, m = i - e * Y;
+        W[e * Cp + m] = Wy[i];
+    }
     for (int i = tid; i < E * E; i += kThreads) {
         const int e = i / E, m = i - e * E;
-        W[e * Cp + m] = Wy[i];
-        W[e * Cp + E + m] = Wq[i];
-        W[e * Cp + 2 * E + m] = Wk[i];
+        W[e * Cp + Y + m] = Wq[i];
+        W[e * Cp + Y + E + m] = Wk[i];
     }
-    for (int i = tid; i < E * 4; i += kThreads) W[(i >> 2) * Cp + 3 * E + (i & 3)] = wb[i];
+    for (int i = tid; i < E * 4; i += kThreads) W[(i >> 2) * Cp + Y + 2 * E + (i & 3)] = wb[i];
+}
+
+// column of the packed state -> its block: 0 = y, 1 = q, 2 = k, 3 = b (also the index of its beta)
+__device__ __forceinline__ int col_block(int m, int E, int Y) {
+    return m < Y ? 0 : m < Y + E ? 1 : m < Y + 2 * E ? 2 : 3;
 }
 
 __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParams p) {
     extern __shared__ float smem[];
-    const int E = p.E, C = 3 * E + 4, Cp = padded_cols(C);
+    const int E = p.E, Y = p.Y, C = Y + 2 * E + 4, Cp = padded_cols(C);
+    const int oq = Y, ok = Y + E, ob4 = Y + 2 * E;   // first column of the q, k, b blocks
     float *W = smem;         // [E][Cp]
     float *xs = W + E * Cp;  // [E]
     float *pre = xs + E;     // [C]: y | q | k | beta (activated in place)
@@ -41,17 +53,17 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
-    const int64_t sEE = seq * E * E, sE4 = seq * E * 4;
+    const int64_t sEE = seq * E * E, sEY = seq * E * Y, sE4 = seq * E * 4;
 
-    load_state(W, Cp, p.Wy + sEE, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, E, tid);
+    load_state(W, Cp, p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, E, Y, tid);
     __syncthreads();
 
     for (int t = 0; t < p.L; ++t) {
         const float *xt = p.x + n * p.xs_n + h * p.xs_h + t * p.xs_l;
-        const int64_t o = (seq * p.L + t) * E, ob = (seq * p.L + t) * 4;
+        const int64_t o = (seq * p.L + t) * E, oy = (seq * p.L + t) * Y, ob = (seq * p.L + t) * 4;
         if (p.keep && p.keep[(int64_t)n * p.L + t] == 0.f) {   // uniform: per-step reset to the shared weights
-            load_state(W, Cp, p.sWy + (int64_t)h * E * E, p.sWq + (int64_t)h * E * E, p.sWk + (int64_t)h * E * E,
-                       p.swb + (int64_t)h * E * 4, E, tid);
+            load_state(W, Cp, p.sWy + (int64_t)h * E * Y, p.sWq + (int64_t)h * E * E, p.sWk + (int64_t)h * E * E,
+                       p.swb + (int64_t)h * E * 4, E, Y, tid);
         }
         for (int e = tid; e < E; e += kThreads) xs[e] = xt[e];
         __syncthreads();
@@ -60,12 +72,12 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
             float a = 0.f;
             for (int e = 0; e < E; ++e) a = fmaf(W[e * Cp + m], xs[e], a);
             pre[m] = a;
-            if (m < E) p.out[o + m] = a;
+            if (m < Y) p.out[oy + m] = a;
         }
         __syncthreads();
         // activations: wave 0 -> softmax(q~), wave 1 -> softmax(k~), wave 2 -> sigmoid(b~)
         if (wave < 2) {
-            float *v = pre + E + wave * E;
+            float *v = pre + oq + wave * E;
             float mx = -INFINITY;
             for (int i = lane; i < E; i += kWave) mx = fmaxf(mx, v[i]);
             mx = wave_max(mx);
@@ -83,38 +95,42 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
                 dst[i] = r;
             }
         } else if (wave == 2 && lane < 4) {
-            const float b = 1.f / (1.f + expf(-pre[3 * E + lane]));
-            pre[3 * E + lane] = b;
+            const float b = 1.f / (1.f + expf(-pre[ob4 + lane]));
+            pre[ob4 + lane] = b;
             p.beta[ob + lane] = b;
         }
         __syncthreads();
         // diff = W^T (q - k), then the rank-1 write of the thread's own column
         for (int m = tid; m < C; m += kThreads) {
             float a = 0.f;
-            for (int e = 0; e < E; ++e) a = fmaf(W[e * Cp + m], pre[E + e] - pre[2 * E + e], a);
-            const int blk = m < 3 * E ? m / E : 3;
-            if (blk == 0) p.ydiff[o + m] = a;
-            else if (blk == 1) p.qdiff[o + m - E] = a;
-            else if (blk == 2) p.kdiff[o + m - 2 * E] = a;
-            else p.bdiff[ob + m - 3 * E] = a;
-            const float ins = pre[3 * E + blk] * a;
-            for (int e = 0; e < E; ++e) W[e * Cp + m] = fmaf(pre[2 * E + e], ins, W[e * Cp + m]);
+            for (int e = 0; e < E; ++e) a = fmaf(W[e * Cp + m], pre[oq + e] - pre[ok + e], a);
+            const int blk = col_block(m, E, Y);
+            if (blk == 0) p.ydiff[oy + m] = a;
+            else if (blk == 1) p.qdiff[o + m - oq] = a;
+            else if (blk == 2) p.kdiff[o + m - ok] = a;
+            else p.bdiff[ob + m - ob4] = a;
+            const float ins = pre[ob4 + blk] * a;
+            for (int e = 0; e < E; ++e) W[e * Cp + m] = fmaf(pre[ok + e], ins, W[e * Cp + m]);
         }
         __syncthreads();
     }
 
+    for (int i = tid; i < E * Y; i += kThreads) {
+        const int e = i / Y, m = i - e * Y;
+        p.Wy[sEY + i] = W[e * Cp + m];
+    }
     for (int i = tid; i < E * E; i += kThreads) {
         const int e = i / E, m = i - e * E;
-        p.Wy[sEE + i] = W[e * Cp + m];
-        p.Wq[sEE + i] = W[e * Cp + E + m];
-        p.Wk[sEE + i] = W[e * Cp + 2 * E + m];
+        p.Wq[sEE + i] = W[e * Cp + oq + m];
+        p.Wk[sEE + i] = W[e * Cp + ok + m];
     }
-    for (int i = tid; i < E * 4; i += kThreads) p.wb[sE4 + i] = W[(i >> 2) * Cp + 3 * E + (i & 3)];
+    for (int i = tid; i < E * 4; i += kThreads) p.wb[sE4 + i] = W[(i >> 2) * Cp + ob4 + (i & 3)];
 }
 
 __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParams p) {
     extern __shared__ float smem[];
-    const int E = p.E, C = 3 * E + 4, Cp = padded_cols(C);
+    const int E = p.E, Y = p.Y, C = Y + 2 * E + 4, Cp = padded_cols(C);
+    const int oq = Y, ok = Y + E, ob4 = Y + 2 * E;
     float *W = smem;             // [E][Cp]  state, reverted step by step
     float *G = W + E * Cp;       // [E][Cp]  dL/dW
     float *xs = G + E * Cp;      // [E]
@@ -132,37 +148,39 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
-    const int64_t sEE = seq * E * E, sE4 = seq * E * 4;
+    const int64_t sEE = seq * E * E, sEY = seq * E * Y, sE4 = seq * E * 4;
 
-    load_state(W, Cp, p.Wy + sEE, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, E, tid);
+    load_state(W, Cp, p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, E, Y, tid);
     if (p.grad_state_mode == 0u) {
         for (int i = tid; i < E * Cp; i += kThreads) G[i] = 0.f;
     } else {
-        load_state(G, Cp, p.gWy + sEE, p.gWq + sEE, p.gWk + sEE, p.gwb + sE4, E, tid);
+        load_state(G, Cp, p.gWy + sEY, p.gWq + sEE, p.gWk + sEE, p.gwb + sE4, E, Y, tid);
     }
     __syncthreads();
 
     for (int t = p.L - 1; t >= 0; --t) {
         const float *xt = p.x + n * p.xs_n + h * p.xs_h + t * p.xs_l;
         const float *got = p.go + n * p.gs_n + h * p.gs_h + t * p.gs_l;
-        const int64_t o = (seq * p.L + t) * E, ob = (seq * p.L + t) * 4;
+        const int64_t o = (seq * p.L + t) * E, oy = (seq * p.L + t) * Y, ob = (seq * p.L + t) * 4;
         for (int e = tid; e < E; e += kThreads) {
             xs[e] = xt[e];
             qs[e] = p.q[o + e];
             ks[e] = p.k[o + e];
-            diff[e] = p.ydiff[o + e];
-            diff[E + e] = p.qdiff[o + e];
-            diff[2 * E + e] = p.kdiff[o + e];
-            gpre[e] = got[e];
+            diff[oq + e] = p.qdiff[o + e];
+            diff[ok + e] = p.kdiff[o + e];
+        }
+        for (int m = tid; m < Y; m += kThreads) {
+            diff[m] = p.ydiff[oy + m];
+            gpre[m] = got[m];
         }
         if (tid < 4) {
             bt[tid] = p.beta[ob + tid];
-            diff[3 * E + tid] = p.bdiff[ob + tid];
+            diff[ob4 + tid] = p.bdiff[ob + tid];
         }
         __syncthreads();
         // column pass: revert W, g_ins = G^T k
         for (int m = tid; m < C; m += kThreads) {
-            const float b = bt[m < 3 * E ? m / E : 3];
+            const float b = bt[col_block(m, E, Y)];
             const float im = b * diff[m];
             float gi = 0.f;
             for (int e = 0; e < E; ++e) {
@@ -197,14 +215,14 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
             float d = 0.f;
             for (int i = lane; i < E; i += kWave) d = fmaf(g[i], s[i], d);
             d = wave_sum(d);
-            for (int i = lane; i < E; i += kWave) gpre[(1 + wave) * E + i] = s[i] * (g[i] - d);
+            for (int i = lane; i < E; i += kWave) gpre[oq + wave * E + i] = s[i] * (g[i] - d);
         } else if (wave == 2) {
             for (int j = 0; j < 4; ++j) {
-                const int lo = j * E, hi = j < 3 ? lo + E : lo + 4;
+                const int lo = j == 0 ? 0 : Y + (j - 1) * E, hi = j == 0 ? Y : j < 3 ? lo + E : lo + 4;
                 float a = 0.f;
                 for (int m = lo + lane; m < hi; m += kWave) a += prod[m];
                 a = wave_sum(a);
-                if (lane == 0) gpre[3 * E + j] = a * bt[j] * (1.f - bt[j]);
+                if (lane == 0) gpre[ob4 + j] = a * bt[j] * (1.f - bt[j]);
             }
         }
         __syncthreads();
@@ -225,33 +243,37 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
     }
 
     const bool accum = p.grad_state_mode == 2u;
+    for (int i = tid; i < E * Y; i += kThreads) {
+        const int e = i / Y, m = i - e * Y;
+        const float gy = G[e * Cp + m];
+        p.gWy[sEY + i] = accum ? p.gWy[sEY + i] + gy : gy;
+    }
     for (int i = tid; i < E * E; i += kThreads) {
         const int e = i / E, m = i - e * E;
-        const float gy = G[e * Cp + m], gqv = G[e * Cp + E + m], gkv = G[e * Cp + 2 * E + m];
-        p.gWy[sEE + i] = accum ? p.gWy[sEE + i] + gy : gy;
+        const float gqv = G[e * Cp + oq + m], gkv = G[e * Cp + ok + m];
         p.gWq[sEE + i] = accum ? p.gWq[sEE + i] + gqv : gqv;
         p.gWk[sEE + i] = accum ? p.gWk[sEE + i] + gkv : gkv;
     }
     for (int i = tid; i < E * 4; i += kThreads) {
-        const float g = G[(i >> 2) * Cp + 3 * E + (i & 3)];
+        const float g = G[(i >> 2) * Cp + ob4 + (i & 3)];
         p.gwb[sE4 + i] = accum ? p.gwb[sE4 + i] + g : g;
     }
 }
 
 }  // namespace
 
-size_t srwm_fwd_generic_lds_bytes(int E) {
-    const size_t C = 3 * (size_t)E + 4, Cp = C | 1;
+size_t srwm_fwd_generic_lds_bytes(int E, int Y) {
+    const size_t C = (size_t)Y + 2 * (size_t)E + 4, Cp = C | 1;
     return sizeof(float) * (E * Cp + E + C);
 }
 
-size_t srwm_bwd_generic_lds_bytes(int E) {
-    const size_t C = 3 * (size_t)E + 4, Cp = C | 1;
+size_t srwm_bwd_generic_lds_bytes(int E, int Y) {
+    const size_t C = (size_t)Y + 2 * (size_t)E + 4, Cp = C | 1;
     return sizeof(float) * (2 * E * Cp + 5 * E + 5 * C + 4);
 }
 
 int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s) {
-    const size_t lds = srwm_fwd_generic_lds_bytes(p.E);
+    const size_t lds = srwm_fwd_generic_lds_bytes(p.E, p.Y);
     hipError_t err = hipFuncSetAttribute((const void *)srwm_fwd_generic_kernel,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return (int)err;
@@ -260,7 +282,7 @@ int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s) {
 }
 
 int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s) {
-    const size_t lds = srwm_bwd_generic_lds_bytes(p.E);
+    const size_t lds = srwm_bwd_generic_lds_bytes(p.E, p.Y);
     hipError_t err = hipFuncSetAttribute((const void *)srwm_bwd_generic_kernel,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (err != hipSuccess) return (int)err;

@@ -527,6 +527,7 @@ bool aligned16(const void *ptr, int64_t a, int64_t b, int64_t c) {
 }  // namespace
 
 int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
+    if (p.Y != p.E) return -1;   // the lane tiling assumes three E x E blocks
     if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l)) return -1;
     const void *dense[] = {p.q, p.k, p.beta, p.ydiff, p.qdiff, p.kdiff, p.bdiff, p.out};
     for (const void *d : dense)
@@ -541,6 +542,7 @@ int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
 }
 
 int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s) {
+    if (p.Y != p.E) return -1;
     if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l) || !aligned16(p.go, p.gs_n, p.gs_h, p.gs_l)) return -1;
     const void *dense[] = {p.q, p.k, p.beta, p.ydiff, p.qdiff, p.kdiff, p.bdiff, p.gx};
     for (const void *d : dense)

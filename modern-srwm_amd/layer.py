@@ -4,6 +4,7 @@
     SRlayer, NoCarryOverSRlayer       reinforcement_learning/torchbeast/layer.py:340-421, :425-488
     CarryFastFFlayer                  reinforcement_learning/torchbeast/layer.py:128-189 (the RL tree
                                       calls it FastFFlayer too; it threads the memory as state)
+    SMFWPlayer                        reinforcement_learning/torchbeast/layer.py:492-586
 
 Same constructor arguments, parameter names and shapes (so state_dicts of the reference load
 unchanged: W_y, W_q, W_k: (1, H, d, d); w_b: (1, H, d, 4); slow_net / out_linear / layer_norm),
@@ -18,6 +19,7 @@ import torch.nn.functional as F
 
 from fast_weight import fast_weight_delta, fast_weight_delta_steps
 from self_ref_v0 import self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
+from self_ref_v1 import self_ref_v1
 
 
 def elu_p1(x):
@@ -150,6 +152,54 @@ class NoCarryOverSRlayer(_SRBase):
         x, slen, bsz = self._split(h, True)
         out = self.fw_layer(x, *self._fast(bsz))
         return h + self._project(out, bsz, slen), state
+
+
+class SMFWPlayer(nn.Module):
+    """Self-modifying fast-weight-programmer layer: an SRWM whose readout is 3d+1 wide and
+    supplies query | key | value | beta of a delta-rule memory.  State: the four SRWM shifts and
+    the memory, (W_y (B,H,d,3d+1), W_q, W_k (B,H,d,d), w_b (B,H,d,4), fast_weights (B,H,d,d)).
+
+    The reference's forward names the memory operator `fast_weight_memory`, which none of its
+    files define (reinforcement_learning/torchbeast/layer.py:562); its arguments (q, k, v, beta,
+    memory) are those of the delta-rule operator, which is what runs here."""
+
+    def __init__(self, num_head, dim_head, in_dim, dropout):
+        super().__init__()
+        self.num_head = num_head
+        self.dim_head = dim_head
+        self.in_dim = in_dim
+        self.fw_layer = self_ref_v1
+        self.y_d_head = 3 * dim_head + 1
+        self.W_y = nn.Parameter(torch.empty(1, num_head, dim_head, self.y_d_head))
+        self.W_q = nn.Parameter(torch.empty(1, num_head, dim_head, dim_head))
+        self.W_k = nn.Parameter(torch.empty(1, num_head, dim_head, dim_head))
+        self.w_b = nn.Parameter(torch.empty(1, num_head, dim_head, 4))
+        self.layer_norm = nn.LayerNorm(in_dim)
+        self.out_linear = nn.Linear(num_head * dim_head, in_dim, bias=False)
+        self.drop = nn.Dropout(dropout)
+        self.reset_rec_parameters()
+
+    def reset_rec_parameters(self):
+        std = 1.0 / math.sqrt(self.dim_head)
+        for w in (self.W_y, self.W_q, self.W_k, self.w_b):
+            nn.init.normal_(w, mean=0., std=std)
+
+    def forward(self, h, state=None):
+        assert state is not None
+        slen, bsz, _ = h.size()
+        x = F.softmax(h.reshape(slen, bsz, self.num_head, self.dim_head), dim=-1).permute(1, 2, 0, 3)
+        slow = (self.W_y, self.W_q, self.W_k, self.w_b)
+        *shift, fast_weights = state
+        fast = [s + w.repeat(bsz, 1, 1, 1) for s, w in zip(shift, slow)]
+        qkvb = self.fw_layer(x, *fast)
+        q, k, v, beta = torch.split(qkvb, (self.dim_head,) * 3 + (1,), -1)
+        out = fast_weight_delta(F.softmax(q, dim=-1), F.softmax(k, dim=-1), v, torch.sigmoid(beta),
+                                fast_weights)
+        out = _heads_out(out, bsz, slen, self.num_head * self.dim_head)
+        out = h + self.drop(self.out_linear(out))
+        new_state = tuple((f.detach() - w.repeat(bsz, 1, 1, 1)).detach() for f, w in zip(fast, slow))
+        # a copy: the delta-rule backward reverts `fast_weights` in place to its value at entry
+        return out, new_state + (fast_weights.detach().clone(),)
 
 
 class _DeltaBase(nn.Module):

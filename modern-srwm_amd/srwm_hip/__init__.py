@@ -42,6 +42,8 @@ _U = ctypes.c_uint
 
 _SIGNATURES = {
     "srwm_forward_f32": [_F, _S] + [_F] * 12 + [_I] * 4 + [_U, ctypes.c_void_p],
+    "srwm_forward_wide_f32": [_F, _S] + [_F] * 12 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_backward_wide_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
@@ -156,25 +158,37 @@ def _stream(device):
 def self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out,
                      flags=0):
     """SRWM forward over the whole sequence.  W_y, W_q, W_k, w_b are overwritten with the
-    final state; q ... out are overwritten with the per-step vectors."""
+    final state; q ... out are overwritten with the per-step vectors.  W_y is (N, H, E, Y):
+    Y = E for the plain operator, any other width (3E+1 in the reference's second variant)
+    makes out and y_diff (N, H, L, Y)."""
     _require(x, "x")
     N, H, L, E = x.shape
-    for t, nm in ((W_y, "W_y"), (W_q, "W_q"), (W_k, "W_k")):
+    _require(W_y, "W_y")
+    Y = W_y.shape[-1]
+    _require(W_y, "W_y", (N, H, E, Y))
+    for t, nm in ((W_q, "W_q"), (W_k, "W_k")):
         _require(t, nm, (N, H, E, E))
     _require(w_b, "w_b", (N, H, E, 4))
-    for t, nm in ((q, "q"), (k, "k"), (y_diff, "y_diff"), (q_diff, "q_diff"), (k_diff, "k_diff"),
-                  (out, "out")):
+    for t, nm in ((q, "q"), (k, "k"), (q_diff, "q_diff"), (k_diff, "k_diff")):
         _require(t, nm, (N, H, L, E))
+    for t, nm in ((y_diff, "y_diff"), (out, "out")):
+        _require(t, nm, (N, H, L, Y))
     _require(beta, "beta", (N, H, L, 4))
     _require(beta_diff, "beta_diff", (N, H, L, 4))
-    if x.numel() == 0:
+    if x.numel() == 0 or Y == 0:
         return
     xs, xstr = _strided(x)
     with torch.cuda.device(x.device), \
             _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out], True) as d:
-        code = lib().srwm_forward_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
-                                      _stream(x.device))
-    _check(code, "srwm_forward_f32")
+        if Y == E:
+            name = "srwm_forward_f32"
+            code = lib().srwm_forward_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
+                                          _stream(x.device))
+        else:
+            name = "srwm_forward_wide_f32"
+            code = lib().srwm_forward_wide_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, Y,
+                                               flags, _stream(x.device))
+    _check(code, name)
 
 
 def self_ref_forward_steps(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff,
@@ -250,20 +264,25 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
     """SRWM backward.  W_* must hold the final state the forward left behind.  By default
     behaves like the reference extension function: the grad_W buffers are read as the
     gradient w.r.t. the final state and the result is added to them (identical to a plain
-    overwrite when they arrive zero-filled, which is how SelfRefv0.backward calls it)."""
+    overwrite when they arrive zero-filled, which is how SelfRefv0.backward calls it).
+    W_y (N, H, E, Y) fixes the width of y_diff, grad_out and grad_W_y."""
     _require(x, "x")
     N, H, L, E = x.shape
-    for t, nm in ((q, "q"), (k, "k"), (y_diff, "y_diff"), (q_diff, "q_diff"), (k_diff, "k_diff"),
-                  (grad_out, "grad_out"), (grad_x, "grad_x")):
+    _require(W_y, "W_y")
+    Y = W_y.shape[-1]
+    for t, nm in ((q, "q"), (k, "k"), (q_diff, "q_diff"), (k_diff, "k_diff"), (grad_x, "grad_x")):
         _require(t, nm, (N, H, L, E))
+    for t, nm in ((y_diff, "y_diff"), (grad_out, "grad_out")):
+        _require(t, nm, (N, H, L, Y))
     _require(beta, "beta", (N, H, L, 4))
     _require(beta_diff, "beta_diff", (N, H, L, 4))
-    for t, nm in ((W_y, "W_y"), (W_q, "W_q"), (W_k, "W_k"), (grad_W_y, "grad_W_y"),
-                  (grad_W_q, "grad_W_q"), (grad_W_k, "grad_W_k")):
+    for t, nm in ((W_y, "W_y"), (grad_W_y, "grad_W_y")):
+        _require(t, nm, (N, H, E, Y))
+    for t, nm in ((W_q, "W_q"), (W_k, "W_k"), (grad_W_q, "grad_W_q"), (grad_W_k, "grad_W_k")):
         _require(t, nm, (N, H, E, E))
     _require(w_b, "w_b", (N, H, E, 4))
     _require(grad_w_b, "grad_w_b", (N, H, E, 4))
-    if x.numel() == 0:
+    if x.numel() == 0 or Y == 0:
         return
     xs, xstr = _strided(x)
     gos, gstr = _strided(grad_out)
@@ -271,10 +290,23 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
             _Dense([q, k, beta, y_diff, q_diff, k_diff, beta_diff], False) as sv, \
             _Dense([W_y, W_q, W_k, w_b], False) as st, \
             _Dense([grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b], True) as gr:
-        code = lib().srwm_backward_f32(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
-                                       *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
-                                       N, H, L, E, flags, _stream(x.device))
-    _check(code, "srwm_backward_f32")
+        if Y == E:
+            name = "srwm_backward_f32"
+            code = lib().srwm_backward_f32(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
+                                           *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
+                                           N, H, L, E, flags, _stream(x.device))
+        else:
+            name = "srwm_backward_wide_f32"
+            code = lib().srwm_backward_wide_f32(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
+                                                *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
+                                                N, H, L, E, Y, flags, _stream(x.device))
+    _check(code, name)
+
+
+# names of the extension functions of the reference's wide-output variant
+# (reinforcement_learning/torchbeast/self_ref_v1/__init__.py:31-32): same call, W_y is (N,H,E,3E+1)
+self_ref_forward_v1 = self_ref_forward
+self_ref_backward_v1 = self_ref_backward
 
 
 def fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=0):

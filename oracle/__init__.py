@@ -62,25 +62,28 @@ def _c(a, dtype):
 
 
 def srwm_forward(x, W_y, W_q, W_k, w_b, dtype=np.float64):
-    """x [N,H,L,E]; W_y/W_q/W_k [N,H,E,E]; w_b [N,H,E,4].
+    """x [N,H,L,E]; W_y [N,H,E,Y]; W_q/W_k [N,H,E,E]; w_b [N,H,E,4].
 
-    Returns a dict with ``out,q,k,beta,y_diff,q_diff,k_diff,beta_diff`` and the
+    Y = E is the reference's first variant, Y = 3E+1 its second (self_ref_v1); ``out`` and
+    ``y_diff`` are [N,H,L,Y].  Returns a dict with ``out,q,k,beta,y_diff,q_diff,k_diff,beta_diff`` and the
     final state ``W_y,W_q,W_k,w_b`` (inputs are not modified).
     """
     sfx, ct = _dt(dtype)
     x = _c(x, dtype)
     N, H, L, E = x.shape
     st = [_c(a, dtype).copy() for a in (W_y, W_q, W_k, w_b)]
-    assert st[0].shape == (N, H, E, E) and st[3].shape == (N, H, E, 4)
+    Y = st[0].shape[-1]
+    assert st[0].shape == (N, H, E, Y) and st[1].shape == (N, H, E, E) and st[3].shape == (N, H, E, 4)
     big = lambda: np.zeros((N, H, L, E), dtype=dtype)
+    wide = lambda: np.zeros((N, H, L, Y), dtype=dtype)
     small = lambda: np.zeros((N, H, L, 4), dtype=dtype)
-    r = dict(q=big(), k=big(), beta=small(), y_diff=big(), q_diff=big(), k_diff=big(),
-             beta_diff=small(), out=big())
-    fn = getattr(lib(), "srwm_oracle_forward_" + sfx)
+    r = dict(q=big(), k=big(), beta=small(), y_diff=wide(), q_diff=big(), k_diff=big(),
+             beta_diff=small(), out=wide())
+    fn = getattr(lib(), "srwm_oracle_forward_wide_" + sfx)
     fn.restype = None
     fn(_p(x, ct), *[_p(a, ct) for a in st],
        *[_p(r[n], ct) for n in ("q", "k", "beta", "y_diff", "q_diff", "k_diff", "beta_diff", "out")],
-       ctypes.c_int(N * H), ctypes.c_int(L), ctypes.c_int(E))
+       ctypes.c_int(N * H), ctypes.c_int(L), ctypes.c_int(E), ctypes.c_int(Y))
     r.update(W_y=st[0], W_q=st[1], W_k=st[2], w_b=st[3])
     return r
 
@@ -104,11 +107,13 @@ def srwm_backward(x, fwd, grad_out, grad_state=None, dtype=np.float64):
         g = [_c(a, dtype).copy() for a in grad_state]
     gx = np.zeros_like(x)
     W0 = [np.zeros_like(a) for a in Wl]
-    fn = getattr(lib(), "srwm_oracle_backward_" + sfx)
+    Y = Wl[0].shape[-1]
+    assert go.shape == (N, H, L, Y)
+    fn = getattr(lib(), "srwm_oracle_backward_wide_" + sfx)
     fn.restype = None
     fn(_p(x, ct), *[_p(a, ct) for a in saved], _p(go, ct), *[_p(a, ct) for a in Wl], _p(gx, ct),
        *[_p(a, ct) for a in g], *[_p(a, ct) for a in W0],
-       ctypes.c_int(N * H), ctypes.c_int(L), ctypes.c_int(E))
+       ctypes.c_int(N * H), ctypes.c_int(L), ctypes.c_int(E), ctypes.c_int(Y))
     return dict(grad_x=gx, grad_W_y=g[0], grad_W_q=g[1], grad_W_k=g[2], grad_w_b=g[3],
                 W0_y=W0[0], W0_q=W0[1], W0_k=W0[2], w0_b=W0[3])
 

@@ -17,6 +17,11 @@
  *                  state written back in place)
  *   SRWM backward  supervised_learning/self_ref_v0/self_ref_v0.cu:689-1233
  *                  (reverse-time sweep that reverts W and carries dL/dW)
+ *   SRWM with a wide output block (W_y is E x Y; Y = 3E+1 in the reference's second
+ *                  variant, whose readout feeds q, k, v, beta of a following layer):
+ *                  reinforcement_learning/torchbeast/self_ref_v1/__init__.py:246-296 (loop),
+ *                  reinforcement_learning/torchbeast/self_ref_v1/self_ref_v1.cu:181-534, 834-1547;
+ *                  the same recurrence with column blocks y (Y wide) | q | k | b
  *   delta forward  supervised_learning/fast_weight/__init__.py:186-191,
  *                  supervised_learning/fast_weight/fast_weight_cuda.cu:101-177
  *   delta backward supervised_learning/fast_weight/fast_weight_cuda.cu:336-392, 489-559
@@ -40,50 +45,57 @@ static void FN(softmax_inplace)(REAL *v, int n) {
     for (int i = 0; i < n; i++) v[i] /= s;
 }
 
-/* Packs the four state tensors of one sequence into W[E][C], C = 3E+4,
- * column blocks y | q | k | b.  (self_ref_v0.cu:146-157 loads the same four.) */
+/* Packs the four state tensors of one sequence into W[E][C], C = Y+2E+4,
+ * column blocks y (Y wide) | q | k | b.  (self_ref_v0.cu:146-157 loads the same four.) */
 static void FN(pack_state)(REAL *W, const REAL *Wy, const REAL *Wq, const REAL *Wk,
-                           const REAL *wb, int E) {
-    const int C = 3 * E + 4;
+                           const REAL *wb, int E, int Y) {
+    const int C = Y + 2 * E + 4;
     for (int e = 0; e < E; e++) {
+        for (int m = 0; m < Y; m++) W[e * C + m] = Wy[e * Y + m];
         for (int m = 0; m < E; m++) {
-            W[e * C + m] = Wy[e * E + m];
-            W[e * C + E + m] = Wq[e * E + m];
-            W[e * C + 2 * E + m] = Wk[e * E + m];
+            W[e * C + Y + m] = Wq[e * E + m];
+            W[e * C + Y + E + m] = Wk[e * E + m];
         }
-        for (int j = 0; j < 4; j++) W[e * C + 3 * E + j] = wb[e * 4 + j];
+        for (int j = 0; j < 4; j++) W[e * C + Y + 2 * E + j] = wb[e * 4 + j];
     }
 }
 
-static void FN(unpack_state)(const REAL *W, REAL *Wy, REAL *Wq, REAL *Wk, REAL *wb, int E) {
-    const int C = 3 * E + 4;
+static void FN(unpack_state)(const REAL *W, REAL *Wy, REAL *Wq, REAL *Wk, REAL *wb, int E, int Y) {
+    const int C = Y + 2 * E + 4;
     for (int e = 0; e < E; e++) {
+        for (int m = 0; m < Y; m++) Wy[e * Y + m] = W[e * C + m];
         for (int m = 0; m < E; m++) {
-            Wy[e * E + m] = W[e * C + m];
-            Wq[e * E + m] = W[e * C + E + m];
-            Wk[e * E + m] = W[e * C + 2 * E + m];
+            Wq[e * E + m] = W[e * C + Y + m];
+            Wk[e * E + m] = W[e * C + Y + E + m];
         }
-        for (int j = 0; j < 4; j++) wb[e * 4 + j] = W[e * C + 3 * E + j];
+        for (int j = 0; j < 4; j++) wb[e * 4 + j] = W[e * C + Y + 2 * E + j];
     }
+}
+
+/* column -> index of its beta: y block 0, q block 1, k block 2, b block 3 */
+static int FN(col_block)(int m, int E, int Y) {
+    return m < Y ? 0 : m < Y + E ? 1 : m < Y + 2 * E ? 2 : 3;
 }
 
 /*
- * SRWM forward.  x,out,q,k,ydiff,qdiff,kdiff: [NH,L,E]; beta,bdiff: [NH,L,4];
- * Wy,Wq,Wk: [NH,E,E]; wb: [NH,E,4] -- overwritten with the final state W_L.
+ * SRWM forward, output block Y columns wide.  x,q,k,qdiff,kdiff: [NH,L,E]; out,ydiff:
+ * [NH,L,Y]; beta,bdiff: [NH,L,4]; Wy: [NH,E,Y]; Wq,Wk: [NH,E,E]; wb: [NH,E,4] --
+ * overwritten with the final state W_L.
  */
-void FN(srwm_oracle_forward)(const REAL *x, REAL *Wy, REAL *Wq, REAL *Wk, REAL *wb,
-                             REAL *q, REAL *k, REAL *beta, REAL *ydiff, REAL *qdiff,
-                             REAL *kdiff, REAL *bdiff, REAL *out, int NH, int L, int E) {
-    const int C = 3 * E + 4;
+void FN(srwm_oracle_forward_wide)(const REAL *x, REAL *Wy, REAL *Wq, REAL *Wk, REAL *wb,
+                                  REAL *q, REAL *k, REAL *beta, REAL *ydiff, REAL *qdiff,
+                                  REAL *kdiff, REAL *bdiff, REAL *out, int NH, int L, int E, int Y) {
+    const int C = Y + 2 * E + 4;
     REAL *W = (REAL *)malloc(sizeof(REAL) * E * C);
     REAL *pre = (REAL *)malloc(sizeof(REAL) * C);
     REAL *diff = (REAL *)malloc(sizeof(REAL) * C);
     REAL *dv = (REAL *)malloc(sizeof(REAL) * E);
     for (int s = 0; s < NH; s++) {
-        FN(pack_state)(W, Wy + (size_t)s * E * E, Wq + (size_t)s * E * E,
-                       Wk + (size_t)s * E * E, wb + (size_t)s * E * 4, E);
+        FN(pack_state)(W, Wy + (size_t)s * E * Y, Wq + (size_t)s * E * E,
+                       Wk + (size_t)s * E * E, wb + (size_t)s * E * 4, E, Y);
         for (int t = 0; t < L; t++) {
-            const size_t o = ((size_t)s * L + t) * E, ob = ((size_t)s * L + t) * 4;
+            const size_t o = ((size_t)s * L + t) * E, oy = ((size_t)s * L + t) * Y,
+                         ob = ((size_t)s * L + t) * 4;
             const REAL *xt = x + o;
             /* main readout: pre = W^T x  (self_ref_v0.cu:164-194) */
             for (int m = 0; m < C; m++) {
@@ -91,16 +103,16 @@ void FN(srwm_oracle_forward)(const REAL *x, REAL *Wy, REAL *Wq, REAL *Wk, REAL *
                 for (int e = 0; e < E; e++) a += W[e * C + m] * xt[e];
                 pre[m] = a;
             }
-            for (int m = 0; m < E; m++) out[o + m] = pre[m];           /* y, no activation */
-            FN(softmax_inplace)(pre + E, E);                            /* q  (:200-239) */
-            FN(softmax_inplace)(pre + 2 * E, E);                        /* k */
+            for (int m = 0; m < Y; m++) out[oy + m] = pre[m];          /* y, no activation */
+            FN(softmax_inplace)(pre + Y, E);                            /* q  (:200-239) */
+            FN(softmax_inplace)(pre + Y + E, E);                        /* k */
             REAL bt[4];
             for (int j = 0; j < 4; j++)                                 /* sigmoid (:196-198) */
-                bt[j] = (REAL)(1.0 / (1.0 + exp(-(double)pre[3 * E + j])));
+                bt[j] = (REAL)(1.0 / (1.0 + exp(-(double)pre[Y + 2 * E + j])));
             for (int e = 0; e < E; e++) {
-                q[o + e] = pre[E + e];
-                k[o + e] = pre[2 * E + e];
-                dv[e] = pre[E + e] - pre[2 * E + e];
+                q[o + e] = pre[Y + e];
+                k[o + e] = pre[Y + E + e];
+                dv[e] = pre[Y + e] - pre[Y + E + e];
             }
             for (int j = 0; j < 4; j++) beta[ob + j] = bt[j];
             /* diff = W^T q - W^T k (:245-313), here as one readout of (q - k) */
@@ -109,28 +121,35 @@ void FN(srwm_oracle_forward)(const REAL *x, REAL *Wy, REAL *Wq, REAL *Wk, REAL *
                 for (int e = 0; e < E; e++) a += W[e * C + m] * dv[e];
                 diff[m] = a;
             }
+            for (int m = 0; m < Y; m++) ydiff[oy + m] = diff[m];
             for (int m = 0; m < E; m++) {
-                ydiff[o + m] = diff[m];
-                qdiff[o + m] = diff[E + m];
-                kdiff[o + m] = diff[2 * E + m];
+                qdiff[o + m] = diff[Y + m];
+                kdiff[o + m] = diff[Y + E + m];
             }
-            for (int j = 0; j < 4; j++) bdiff[ob + j] = diff[3 * E + j];
+            for (int j = 0; j < 4; j++) bdiff[ob + j] = diff[Y + 2 * E + j];
             /* rank-1 write into all four blocks (:317-350), also at the last step */
             for (int m = 0; m < C; m++) {
-                const int blk = m < 3 * E ? m / E : 3;
-                const REAL ins = bt[blk] * diff[m];
+                const REAL ins = bt[FN(col_block)(m, E, Y)] * diff[m];
                 for (int e = 0; e < E; e++) W[e * C + m] += k[o + e] * ins;
             }
         }
-        FN(unpack_state)(W, Wy + (size_t)s * E * E, Wq + (size_t)s * E * E,
-                         Wk + (size_t)s * E * E, wb + (size_t)s * E * 4, E);
+        FN(unpack_state)(W, Wy + (size_t)s * E * Y, Wq + (size_t)s * E * E,
+                         Wk + (size_t)s * E * E, wb + (size_t)s * E * 4, E, Y);
     }
     free(W); free(pre); free(diff); free(dv);
 }
 
+/* The reference's first variant: W_y is E x E. */
+void FN(srwm_oracle_forward)(const REAL *x, REAL *Wy, REAL *Wq, REAL *Wk, REAL *wb,
+                             REAL *q, REAL *k, REAL *beta, REAL *ydiff, REAL *qdiff,
+                             REAL *kdiff, REAL *bdiff, REAL *out, int NH, int L, int E) {
+    FN(srwm_oracle_forward_wide)(x, Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff, out,
+                                 NH, L, E, E);
+}
+
 /*
- * SRWM backward.  Inputs: x and everything the forward emitted, grad_out
- * [NH,L,E], and Wy..wb holding the FINAL state W_L (read only here, as in the
+ * SRWM backward, output block Y columns wide.  Inputs: x and everything the forward
+ * emitted, grad_out [NH,L,Y], and Wy..wb holding the FINAL state W_L (read only here, as in the
  * reference: self_ref_v0.cu:1208-1233 writes only gradients).
  * gWy,gWq,gWk,gwb: on entry the gradient w.r.t. the final state (zeros for the
  * plain operator; the incoming grads for the stateful one), on exit the
@@ -138,13 +157,13 @@ void FN(srwm_oracle_forward)(const REAL *x, REAL *Wy, REAL *Wq, REAL *Wk, REAL *
  * If W0_out* are non-NULL the fully reverted state is stored there (it must
  * equal the W_0 the forward started from).
  */
-void FN(srwm_oracle_backward)(const REAL *x, const REAL *q, const REAL *k, const REAL *beta,
-                              const REAL *ydiff, const REAL *qdiff, const REAL *kdiff,
-                              const REAL *bdiff, const REAL *gout, const REAL *Wy,
-                              const REAL *Wq, const REAL *Wk, const REAL *wb, REAL *gx,
-                              REAL *gWy, REAL *gWq, REAL *gWk, REAL *gwb, REAL *W0y,
-                              REAL *W0q, REAL *W0k, REAL *w0b, int NH, int L, int E) {
-    const int C = 3 * E + 4;
+void FN(srwm_oracle_backward_wide)(const REAL *x, const REAL *q, const REAL *k, const REAL *beta,
+                                   const REAL *ydiff, const REAL *qdiff, const REAL *kdiff,
+                                   const REAL *bdiff, const REAL *gout, const REAL *Wy,
+                                   const REAL *Wq, const REAL *Wk, const REAL *wb, REAL *gx,
+                                   REAL *gWy, REAL *gWq, REAL *gWk, REAL *gwb, REAL *W0y,
+                                   REAL *W0q, REAL *W0k, REAL *w0b, int NH, int L, int E, int Y) {
+    const int C = Y + 2 * E + 4;
     REAL *W = (REAL *)malloc(sizeof(REAL) * E * C);
     REAL *G = (REAL *)malloc(sizeof(REAL) * E * C);
     REAL *ins = (REAL *)malloc(sizeof(REAL) * C);
@@ -155,19 +174,20 @@ void FN(srwm_oracle_backward)(const REAL *x, const REAL *q, const REAL *k, const
     REAL *gq = (REAL *)malloc(sizeof(REAL) * E);
     REAL *gk = (REAL *)malloc(sizeof(REAL) * E);
     for (int s = 0; s < NH; s++) {
-        const size_t ow = (size_t)s * E * E, owb = (size_t)s * E * 4;
-        FN(pack_state)(W, Wy + ow, Wq + ow, Wk + ow, wb + owb, E);
-        FN(pack_state)(G, gWy + ow, gWq + ow, gWk + ow, gwb + owb, E);
+        const size_t ow = (size_t)s * E * E, owy = (size_t)s * E * Y, owb = (size_t)s * E * 4;
+        FN(pack_state)(W, Wy + owy, Wq + ow, Wk + ow, wb + owb, E, Y);
+        FN(pack_state)(G, gWy + owy, gWq + ow, gWk + ow, gwb + owb, E, Y);
         for (int t = L - 1; t >= 0; t--) {
-            const size_t o = ((size_t)s * L + t) * E, ob = ((size_t)s * L + t) * 4;
-            const REAL *xt = x + o, *qt = q + o, *kt = k + o, *bt = beta + ob, *go = gout + o;
+            const size_t o = ((size_t)s * L + t) * E, oy = ((size_t)s * L + t) * Y,
+                         ob = ((size_t)s * L + t) * 4;
+            const REAL *xt = x + o, *qt = q + o, *kt = k + o, *bt = beta + ob, *go = gout + oy;
+            for (int m = 0; m < Y; m++) diff[m] = ydiff[oy + m];
             for (int m = 0; m < E; m++) {
-                diff[m] = ydiff[o + m];
-                diff[E + m] = qdiff[o + m];
-                diff[2 * E + m] = kdiff[o + m];
+                diff[Y + m] = qdiff[o + m];
+                diff[Y + E + m] = kdiff[o + m];
             }
-            for (int j = 0; j < 4; j++) diff[3 * E + j] = bdiff[ob + j];
-            for (int m = 0; m < C; m++) ins[m] = bt[m < 3 * E ? m / E : 3] * diff[m];
+            for (int j = 0; j < 4; j++) diff[Y + 2 * E + j] = bdiff[ob + j];
+            for (int m = 0; m < C; m++) ins[m] = bt[FN(col_block)(m, E, Y)] * diff[m];
             /* revert the write: W_{t-1} = W_t - k (x) ins  (:701-709 and siblings) */
             for (int e = 0; e < E; e++)
                 for (int m = 0; m < C; m++) W[e * C + m] -= kt[e] * ins[m];
@@ -185,7 +205,7 @@ void FN(srwm_oracle_backward)(const REAL *x, const REAL *q, const REAL *k, const
             /* through ins = beta_blk * diff */
             REAL gb[4] = {0, 0, 0, 0};
             for (int m = 0; m < C; m++) {
-                const int blk = m < 3 * E ? m / E : 3;
+                const int blk = FN(col_block)(m, E, Y);
                 gdiff[m] = bt[blk] * gins[m];
                 gb[blk] += gins[m] * diff[m];
             }
@@ -201,12 +221,12 @@ void FN(srwm_oracle_backward)(const REAL *x, const REAL *q, const REAL *k, const
             /* softmax / sigmoid backward -> gradient of the main readout */
             REAL dq = 0, dk = 0;
             for (int e = 0; e < E; e++) { dq += gq[e] * qt[e]; dk += gk[e] * kt[e]; }
+            for (int m = 0; m < Y; m++) gpre[m] = go[m];
             for (int m = 0; m < E; m++) {
-                gpre[m] = go[m];
-                gpre[E + m] = qt[m] * (gq[m] - dq);
-                gpre[2 * E + m] = kt[m] * (gk[m] - dk);
+                gpre[Y + m] = qt[m] * (gq[m] - dq);
+                gpre[Y + E + m] = kt[m] * (gk[m] - dk);
             }
-            for (int j = 0; j < 4; j++) gpre[3 * E + j] = gb[j] * bt[j] * (1 - bt[j]);
+            for (int j = 0; j < 4; j++) gpre[Y + 2 * E + j] = gb[j] * bt[j] * (1 - bt[j]);
             /* through pre = W_{t-1}^T x */
             for (int e = 0; e < E; e++) {
                 REAL a = 0;
@@ -216,11 +236,22 @@ void FN(srwm_oracle_backward)(const REAL *x, const REAL *q, const REAL *k, const
             for (int e = 0; e < E; e++)
                 for (int m = 0; m < C; m++) G[e * C + m] += xt[e] * gpre[m];
         }
-        FN(unpack_state)(G, gWy + ow, gWq + ow, gWk + ow, gwb + owb, E);
-        if (W0y) FN(unpack_state)(W, W0y + ow, W0q + ow, W0k + ow, w0b + owb, E);
+        FN(unpack_state)(G, gWy + owy, gWq + ow, gWk + ow, gwb + owb, E, Y);
+        if (W0y) FN(unpack_state)(W, W0y + owy, W0q + ow, W0k + ow, w0b + owb, E, Y);
     }
     free(W); free(G); free(ins); free(diff); free(gins); free(gdiff); free(gpre);
     free(gq); free(gk);
+}
+
+/* The reference's first variant: W_y is E x E. */
+void FN(srwm_oracle_backward)(const REAL *x, const REAL *q, const REAL *k, const REAL *beta,
+                              const REAL *ydiff, const REAL *qdiff, const REAL *kdiff,
+                              const REAL *bdiff, const REAL *gout, const REAL *Wy,
+                              const REAL *Wq, const REAL *Wk, const REAL *wb, REAL *gx,
+                              REAL *gWy, REAL *gWq, REAL *gWk, REAL *gwb, REAL *W0y,
+                              REAL *W0q, REAL *W0k, REAL *w0b, int NH, int L, int E) {
+    FN(srwm_oracle_backward_wide)(x, q, k, beta, ydiff, qdiff, kdiff, bdiff, gout, Wy, Wq, Wk, wb,
+                                  gx, gWy, gWq, gWk, gwb, W0y, W0q, W0k, w0b, NH, L, E, E);
 }
 
 /*

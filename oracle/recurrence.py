@@ -20,10 +20,14 @@ import torch.nn.functional as F
 
 
 def srwm_recurrence(x, W_y, W_q, W_k, w_b):
-    """x [N,H,L,E]; W_* [N,H,E,E]; w_b [N,H,E,4] -> (out [N,H,L,E], final 4-state)."""
+    """x [N,H,L,E]; W_y [N,H,E,Y]; W_q,W_k [N,H,E,E]; w_b [N,H,E,4] -> (out [N,H,L,Y], final 4-state).
+
+    Y = E: self_ref_v0; Y = 3E+1: the same loop as the reference writes it for self_ref_v1
+    (reinforcement_learning/torchbeast/self_ref_v1/__init__.py:246-296)."""
     N, H, L, E = x.shape
+    Y = W_y.shape[-1]
     xs = x.permute(2, 0, 1, 3).reshape(L, N * H, E)
-    Wy = W_y.reshape(N * H, E, E)
+    Wy = W_y.reshape(N * H, E, Y)
     Wq = W_q.reshape(N * H, E, E)
     Wk = W_k.reshape(N * H, E, E)
     wb = w_b.reshape(N * H, E, 4)
@@ -45,8 +49,8 @@ def srwm_recurrence(x, W_y, W_q, W_k, w_b):
         Wq = Wq + torch.bmm(kc, q_ins.unsqueeze(1))
         Wk = Wk + torch.bmm(kc, k_ins.unsqueeze(1))
         wb = wb + torch.bmm(kc, b_ins.unsqueeze(1))
-    out = torch.stack(outs).view(L, N, H, E).permute(1, 2, 0, 3)
-    final = (Wy.view(N, H, E, E), Wq.view(N, H, E, E), Wk.view(N, H, E, E), wb.view(N, H, E, 4))
+    out = torch.stack(outs).view(L, N, H, Y).permute(1, 2, 0, 3)
+    final = (Wy.view(N, H, E, Y), Wq.view(N, H, E, E), Wk.view(N, H, E, E), wb.view(N, H, E, 4))
     return out, final
 
 

@@ -25,6 +25,9 @@ SRWM_CASES = {  # name: (N, H, L, E, seed, w_std, x_softmax)
     "srwm_n2h2l5e4": (2, 2, 5, 4, 101, 0.7, False),
     "srwm_n1h2l9e8": (1, 2, 9, 8, 102, 0.5, True),
     "srwm_n1h1l6e16": (1, 1, 6, 16, 103, 0.2, False),
+    # output block 3E+1 columns wide (the self_ref_v1 shape)
+    "srwm_wide_n2h2l7e4y13": (2, 2, 7, 4, 104, 0.7, True, 13),
+    "srwm_wide_n1h2l5e8y25": (1, 2, 5, 8, 105, 0.5, False, 25),
 }
 DELTA_CASES = {  # name: (N, H, L, E, M, seed, qk, w0_std)
     "delta_n2h2l5e4m4": (2, 2, 5, 4, 4, 201, "softmax", 0.3),
@@ -34,8 +37,9 @@ DELTA_CASES = {  # name: (N, H, L, E, M, seed, qk, w0_std)
 
 
 def main():
-    for name, (N, H, L, E, seed, w_std, xsm) in SRWM_CASES.items():
-        x, W, go = srwm_inputs(N, H, L, E, seed=seed, w_std=w_std, x_softmax=xsm, per_batch_state=True)
+    for name, (N, H, L, E, seed, w_std, xsm, *yw) in SRWM_CASES.items():
+        x, W, go = srwm_inputs(N, H, L, E, seed=seed, w_std=w_std, x_softmax=xsm, per_batch_state=True,
+                               y_width=yw[0] if yw else None)
         f = oracle.srwm_forward(x.numpy(), *[w.numpy() for w in W])
         b = oracle.srwm_backward(x.numpy(), f, go.numpy())
         np.savez(os.path.join(HERE, name + ".npz"), x=x.numpy(), W_y0=W[0].numpy(), W_q0=W[1].numpy(),

@@ -14,9 +14,10 @@ def rel_err(a, b):
 
 
 def srwm_inputs(N, H, L, E, seed=0, w_std=0.02, x_softmax=False, per_batch_state=False,
-                dtype=torch.float64):
+                dtype=torch.float64, y_width=None):
     """x ~ N(0,1) (optionally soft-maxed); W_0 = [W_y|W_q|W_k|w_b] ~ N(0, w_std) per head,
-    broadcast over the batch the way the layers do with .repeat()."""
+    broadcast over the batch the way the layers do with .repeat().  y_width: columns of W_y
+    (and of the upstream gradient) when they differ from E."""
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(N, H, L, E, generator=g, dtype=torch.float64)
     if x_softmax:
@@ -27,6 +28,10 @@ def srwm_inputs(N, H, L, E, seed=0, w_std=0.02, x_softmax=False, per_batch_state
     if not per_batch_state:
         W = [w.repeat(N, 1, 1, 1) for w in W]
     go = torch.randn(N, H, L, E, generator=g, dtype=torch.float64)
+    if y_width is not None and y_width != E:
+        wy = torch.randn(nb, H, E, y_width, generator=g, dtype=torch.float64) * w_std
+        W[0] = wy if per_batch_state else wy.repeat(N, 1, 1, 1)
+        go = torch.randn(N, H, L, y_width, generator=g, dtype=torch.float64)
     return x.to(dtype), [w.to(dtype).contiguous() for w in W], go.to(dtype)
 
 

@@ -20,7 +20,7 @@ TOL = 1e-5
 
 
 def test_fixtures_exist():
-    assert len(SRWM) >= 3 and len(DELTA) >= 4 and os.path.exists(STEPS_SRWM) and os.path.exists(STEPS_DELTA)
+    assert len(SRWM) >= 5 and len(DELTA) >= 4 and os.path.exists(STEPS_SRWM) and os.path.exists(STEPS_DELTA)
 
 
 def test_stepwise_references_reproduce_their_fixtures():
@@ -69,13 +69,15 @@ def test_oracle_reproduces_delta_fixture(path):
 def test_hip_matches_srwm_fixture(path):
     print("case", os.path.basename(path), flush=True)
     from self_ref_v0 import self_ref_v0
+    from self_ref_v1 import self_ref_v1
     g = np.load(path)
     dev = torch.device("cuda:0")
     t = lambda a: torch.from_numpy(a).to(dev, torch.float32)
     x = t(g["x"]).requires_grad_(True)
     W = [t(g[n]).requires_grad_(True) for n in ("W_y0", "W_q0", "W_k0", "w_b0")]
     Wc = [w.clone() for w in W]
-    out = self_ref_v0(x, *Wc)
+    op = self_ref_v0 if g["W_y0"].shape[-1] == g["x"].shape[-1] else self_ref_v1
+    out = op(x, *Wc)
     (out * t(g["grad_out"])).sum().backward()
     assert rel_err(out.detach().cpu().numpy(), g["out"]) < TOL
     assert rel_err(x.grad.cpu().numpy(), g["grad_x"]) < TOL

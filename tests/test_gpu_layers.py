@@ -235,3 +235,44 @@ def test_rl_delta_layer_whole_unroll_equals_the_per_step_loop():
     for n, p in lay.named_parameters():
         if n in loop_grads:
             assert (p.grad - loop_grads[n]).abs().max().item() < 2e-5 * max(1e-6, loop_grads[n].abs().max().item()), n
+
+
+def test_self_modifying_fwp_layer():
+    """SMFWPlayer: wide SRWM readout -> softmax / sigmoid -> delta-rule memory, two segments with
+    carried state; outputs, carried state and parameter gradients against the fp64 recurrences."""
+    print("case SMFWPlayer", flush=True)
+    from layer import SMFWPlayer
+    torch.manual_seed(5)
+    L, B, H, d = 6, 3, 4, 16
+    gpu, cpu = _pair(SMFWPlayer(H, d, H * d, 0.0))
+    assert gpu.W_y.shape == (1, H, d, 3 * d + 1)
+    widths = (3 * d + 1, d, d, 4, d)
+    state = tuple(torch.zeros(B, H, d, w, device=_dev()) for w in widths)
+    ref_state = tuple(torch.zeros(B, H, d, w, dtype=torch.float64) for w in widths)
+    slow_c = (cpu.W_y, cpu.W_q, cpu.W_k, cpu.w_b)
+    for seg in range(2):
+        h = torch.randn(L, B, H * d, dtype=torch.float64)
+        go = torch.randn(L, B, H * d, dtype=torch.float64)
+        hg = h.to(_dev(), torch.float32).requires_grad_(True)
+        gpu.zero_grad()
+        out, state = gpu(hg, state)
+        (out * go.to(_dev(), torch.float32)).sum().backward()
+        # fp64 statement
+        cpu.zero_grad()
+        hc = h.clone().requires_grad_(True)
+        x = F.softmax(hc.reshape(L, B, H, d), dim=-1).permute(1, 2, 0, 3)
+        fast = [s + w.repeat(B, 1, 1, 1) for s, w in zip(ref_state[:4], slow_c)]
+        qkvb, final = srwm_recurrence(x, *fast)
+        q, k, v, beta = torch.split(qkvb, (d,) * 3 + (1,), -1)
+        mem_out, WL = delta_recurrence(F.softmax(q, -1), F.softmax(k, -1), v, torch.sigmoid(beta), ref_state[4])
+        ref = hc + cpu.out_linear(mem_out.transpose(1, 2).reshape(B, L, H * d).transpose(0, 1))
+        (ref * go).sum().backward()
+        ref_state = tuple((f - w).detach() for f, w in zip(final, slow_c)) + (WL.detach(),)
+        assert rel_err(out.detach().cpu().numpy(), ref.detach().numpy()) < TOL, seg
+        assert rel_err(hg.grad.cpu().numpy(), hc.grad.numpy()) < TOL, seg
+        for n in ("W_y", "W_q", "W_k", "w_b"):
+            assert rel_err(getattr(gpu, n).grad.cpu().numpy(), getattr(cpu, n).grad.numpy()) < TOL, (seg, n)
+        assert rel_err(gpu.out_linear.weight.grad.cpu().numpy(), cpu.out_linear.weight.grad.numpy()) < TOL
+        assert all(not s.requires_grad for s in state)
+        for s, r in zip(state, ref_state):
+            assert (s.cpu().double() - r).abs().max().item() < 2e-5 * max(1.0, r.abs().max().item())

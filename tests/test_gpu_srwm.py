@@ -27,12 +27,14 @@ def run_hip(x, W, go, flags=0, grad_state=None, mode=None):
     import srwm_hip
     dev = _dev()
     N, H, L, E = x.shape
+    Y = W[0].shape[-1]
     xd = x.to(dev, torch.float32)
     Wd = [w.to(dev, torch.float32).contiguous() for w in W]
     big = lambda: torch.full((N, H, L, E), float("nan"), device=dev)
+    wide = lambda: torch.full((N, H, L, Y), float("nan"), device=dev)
     small = lambda: torch.full((N, H, L, 4), float("nan"), device=dev)
-    f = dict(q=big(), k=big(), beta=small(), y_diff=big(), q_diff=big(), k_diff=big(),
-             beta_diff=small(), out=big())
+    f = dict(q=big(), k=big(), beta=small(), y_diff=wide(), q_diff=big(), k_diff=big(),
+             beta_diff=small(), out=wide())
     srwm_hip.self_ref_forward(xd, *Wd, *[f[n] for n in FWD_NAMES], flags=flags)
     f.update(W_y=Wd[0], W_q=Wd[1], W_k=Wd[2], w_b=Wd[3])
     if go is None:
@@ -260,3 +262,93 @@ def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
     assert rel_err(sd[0].grad.cpu().numpy(), sr[0].grad.numpy()) < TOL
     for w in sd[1:]:
         assert float(w.grad.abs().max()) == 0.0
+
+
+# ---------------------------------------------------------------- wide output block (self_ref_v1)
+
+@pytest.mark.parametrize("shape,Y,w_std,xsm,per_batch", [
+    ((3, 5, 11, 8), 25, 0.6, True, True),                    # the reference self-test's shape for this variant
+    ((4, 8, 100, 32), 97, 1 / math.sqrt(32), True, False),   # RL learner shape: 8 heads of 32, Y = 3E+1
+    ((2, 4, 40, 16), 49, 0.25, True, True),
+    ((1, 2, 20, 48), 145, 0.1, True, True),                  # largest multiple of 16 whose backward fits in LDS
+    ((1, 3, 7, 5), 16, 0.8, False, True),                    # odd head size
+    ((2, 2, 1, 16), 49, 0.3, True, True),                    # L = 1
+    ((1, 2, 9, 8), 3, 0.7, False, True),                     # narrower than E
+])
+def test_wide_matches_fp64_oracle(shape, Y, w_std, xsm, per_batch):
+    print(f"case wide shape={shape} Y={Y}", flush=True)
+    x, W, go = srwm_inputs(*shape, seed=0, w_std=w_std, x_softmax=xsm, per_batch_state=per_batch, y_width=Y)
+    check_against_oracle(x, W, go, 0)
+
+
+def test_wide_grad_state_modes_and_strided_views():
+    import srwm_hip
+    print("case wide grad_state + strided", flush=True)
+    N, H, L, E, Y = 2, 3, 9, 16, 49
+    x, W, go = srwm_inputs(N, H, L, E, seed=3, w_std=0.5, per_batch_state=True, y_width=Y)
+    g = torch.Generator().manual_seed(7)
+    gs = [torch.randn(w.shape, generator=g, dtype=torch.float64) for w in W]
+    of = oracle.srwm_forward(x.numpy(), *[w.numpy() for w in W])
+    ob = oracle.srwm_backward(x.numpy(), of, go.numpy(), grad_state=[s.numpy() for s in gs])
+    _, b_in = run_hip(x, W, go, 0, grad_state=gs, mode=srwm_hip.GRAD_STATE_IN)
+    _, b_acc = run_hip(x, W, go, 0, grad_state=gs, mode=srwm_hip.GRAD_STATE_ACCUM)
+    assert rel_err(b_in["grad_x"].cpu().numpy(), ob["grad_x"]) < TOL
+    for n, s in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), gs):
+        assert rel_err(b_in[n].cpu().numpy(), ob[n]) < TOL, n
+        assert rel_err(b_acc[n].cpu().numpy(), ob[n] + s.numpy()) < TOL, n
+    # permuted views of (L, N, H, .) storage, as a layer passes them
+    dev = _dev()
+    xv = x.permute(2, 0, 1, 3).contiguous().to(dev, torch.float32).permute(1, 2, 0, 3)
+    gov = go.permute(2, 0, 1, 3).contiguous().to(dev, torch.float32).permute(1, 2, 0, 3)
+    Wd = [w.to(dev, torch.float32).contiguous() for w in W]
+    big = lambda: torch.empty((N, H, L, E), device=dev)
+    wide = lambda: torch.empty((N, H, L, Y), device=dev)
+    small = lambda: torch.empty((N, H, L, 4), device=dev)
+    f = [big(), big(), small(), wide(), big(), big(), small(), wide()]
+    srwm_hip.self_ref_forward_v1(xv, *Wd, *f)
+    gx = big()
+    gw = [torch.empty_like(w) for w in Wd]
+    srwm_hip.self_ref_backward_v1(xv, *f[:-1], gov, *Wd, gx, *gw, flags=srwm_hip.GRAD_STATE_ZERO)
+    ob0 = oracle.srwm_backward(x.numpy(), of, go.numpy())
+    assert rel_err(f[-1].cpu().numpy(), of["out"]) < TOL
+    assert rel_err(gx.cpu().numpy(), ob0["grad_x"]) < TOL
+    assert rel_err(gw[0].cpu().numpy(), ob0["grad_W_y"]) < TOL
+
+
+def test_wide_autograd_function_drop_in():
+    """self_ref_v1 as the reference calls it: repeat()-ed weights, out.sum().backward(); checked
+    against fp64 autograd of the per-step recurrence."""
+    print("case wide autograd drop-in", flush=True)
+    from oracle.recurrence import srwm_recurrence
+    from self_ref_v1 import self_ref_v1
+    N, H, L, E = 3, 5, 11, 8
+    Y = 3 * E + 1
+    x, W, go = srwm_inputs(N, H, L, E, seed=111, w_std=0.6, x_softmax=True, y_width=Y)
+    dev = _dev()
+    slow = [w[:1].to(dev, torch.float32).clone().requires_grad_(True) for w in W]
+    xd = x.to(dev, torch.float32).requires_grad_(True)
+    out = self_ref_v1(xd, *[w.repeat(N, 1, 1, 1) for w in slow])
+    assert out.shape == (N, H, L, Y)
+    (out * go.to(dev, torch.float32)).sum().backward()
+    xr = x.clone().requires_grad_(True)
+    slow_r = [w[:1].clone().requires_grad_(True) for w in W]
+    out_r, _ = srwm_recurrence(xr, *[w.repeat(N, 1, 1, 1) for w in slow_r])
+    (out_r * go).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), out_r.detach().numpy()) < TOL
+    assert rel_err(xd.grad.cpu().numpy(), xr.grad.numpy()) < TOL
+    for a, b in zip(slow, slow_r):
+        assert rel_err(a.grad.cpu().numpy(), b.grad.numpy()) < TOL
+
+
+def test_wide_rejects_a_state_that_does_not_fit():
+    import srwm_hip
+    dev = _dev()
+    N, H, L, E, Y = 1, 1, 2, 64, 1000   # 64 x 1132 floats = 290 KB
+    x = torch.zeros(N, H, L, E, device=dev)
+    W = [torch.zeros(N, H, E, Y, device=dev), torch.zeros(N, H, E, E, device=dev),
+         torch.zeros(N, H, E, E, device=dev), torch.zeros(N, H, E, 4, device=dev)]
+    big = lambda: torch.empty((N, H, L, E), device=dev)
+    wide = lambda: torch.empty((N, H, L, Y), device=dev)
+    small = lambda: torch.empty((N, H, L, 4), device=dev)
+    with pytest.raises(RuntimeError, match="LDS"):
+        srwm_hip.self_ref_forward_v1(x, *W, big(), big(), small(), wide(), big(), big(), small(), wide())

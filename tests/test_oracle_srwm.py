@@ -212,6 +212,107 @@ def test_f32_oracle_tracks_f64():
         assert rel_err(b32[n], b64[n]) < 1e-4, n
 
 
+# ---------------------------------------------------------- wide output block (self_ref_v1: Y = 3E+1)
+
+def _brute_force_step_wide(x, Wy, Wq, Wk, wb):
+    """One step with Python floats; the width of each block is read off the nested lists."""
+    E = len(x)
+    col = lambda W, v, m: sum(W[e][m] * v[e] for e in range(E))
+    y = [col(Wy, x, m) for m in range(len(Wy[0]))]
+    sm = lambda v: [math.exp(a - max(v)) / sum(math.exp(b - max(v)) for b in v) for a in v]
+    q, k = sm([col(Wq, x, m) for m in range(E)]), sm([col(Wk, x, m) for m in range(E)])
+    beta = [1.0 / (1.0 + math.exp(-col(wb, x, j))) for j in range(4)]
+    new = []
+    for W, b in ((Wy, beta[0]), (Wq, beta[1]), (Wk, beta[2]), (wb, beta[3])):
+        n = len(W[0])
+        ins = [b * (col(W, q, m) - col(W, k, m)) for m in range(n)]
+        new.append([[W[e][m] + k[e] * ins[m] for m in range(n)] for e in range(E)])
+    return y, q, k, beta, new
+
+
+@pytest.mark.parametrize("E", [2, 3])
+def test_wide_brute_force_three_steps(E):
+    Y = 3 * E + 1
+    x, W, _ = srwm_inputs(1, 1, 3, E, seed=20 + E, w_std=1.0, y_width=Y)
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    assert f["out"].shape == (1, 1, 3, Y) and f["y_diff"].shape == (1, 1, 3, Y)
+    st = [w[0, 0].tolist() for w in W]
+    for t in range(3):
+        y, q, k, beta, st = _brute_force_step_wide(x[0, 0, t].tolist(), *st)
+        assert np.allclose(f["out"][0, 0, t], y, rtol=1e-13, atol=1e-15)
+        assert np.allclose(f["q"][0, 0, t], q, rtol=1e-13)
+        assert np.allclose(f["k"][0, 0, t], k, rtol=1e-13)
+        assert np.allclose(f["beta"][0, 0, t], beta, rtol=1e-13)
+    for name, s in zip(("W_y", "W_q", "W_k", "w_b"), st):
+        assert np.allclose(f[name][0, 0], np.array(s), rtol=1e-12, atol=1e-15)
+
+
+def test_wide_beta_zero_is_a_plain_matmul():
+    E, Y = 8, 25
+    x, W, go = srwm_inputs(2, 3, 9, E, seed=21, w_std=0.5, x_softmax=True, y_width=Y)
+    W[3] = torch.full_like(W[3], -60.0)
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    assert rel_err(f["out"], torch.matmul(x, W[0]).numpy()) < 1e-14
+    b = oracle.srwm_backward(x.numpy(), f, go.numpy())
+    assert rel_err(b["grad_W_y"], torch.matmul(x.transpose(-1, -2), go).numpy()) < 1e-13
+    assert rel_err(b["grad_x"], torch.matmul(go, W[0].transpose(-1, -2)).numpy()) < 1e-13
+
+
+def test_wide_equals_narrow_when_the_extra_columns_are_cut():
+    """The first E columns of a wide W_y evolve exactly like a narrow W_y: the columns of
+    the output block do not interact (q, k, beta come from the other three blocks)."""
+    E, Y = 6, 19
+    x, W, _ = srwm_inputs(2, 2, 12, E, seed=22, w_std=0.8, y_width=Y)
+    wide = oracle.srwm_forward(x.numpy(), *_np(W))
+    narrow = oracle.srwm_forward(x.numpy(), W[0][..., :E].numpy(), *_np(W[1:]))
+    assert rel_err(wide["out"][..., :E], narrow["out"]) < 1e-14
+    assert rel_err(wide["W_y"][..., :E], narrow["W_y"]) < 1e-14
+    for n in ("q", "k", "beta", "q_diff", "k_diff", "beta_diff", "W_q", "W_k", "w_b"):
+        assert rel_err(wide[n], narrow[n]) < 1e-14, n
+
+
+@pytest.mark.parametrize("shape,Y,w_std,xsm", [
+    ((3, 5, 11, 8), 25, 0.6, True),     # the shape of the reference's self-test for this variant
+    ((2, 2, 20, 16), 49, 0.25, True),
+    ((1, 3, 5, 7), 22, 1.0, False),     # odd head dim
+    ((1, 2, 6, 4), 2, 0.9, False),      # narrower than E
+])
+def test_wide_c_oracle_matches_autograd_of_the_torch_recurrence(shape, Y, w_std, xsm):
+    x, W, go = srwm_inputs(*shape, seed=23, w_std=w_std, x_softmax=xsm, per_batch_state=True, y_width=Y)
+    g = torch.Generator().manual_seed(61)
+    gs = [torch.randn(w.shape, generator=g, dtype=torch.float64) for w in W]
+    xt = x.clone().requires_grad_(True)
+    Wt = [w.clone().requires_grad_(True) for w in W]
+    out, final = srwm_recurrence(xt, *Wt)
+    ((out * go).sum() + sum((f * s).sum() for f, s in zip(final, gs))).backward()
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    assert rel_err(f["out"], out.detach().numpy()) < 1e-12
+    for name, fw in zip(("W_y", "W_q", "W_k", "w_b"), final):
+        assert rel_err(f[name], fw.detach().numpy()) < 1e-12
+    b = oracle.srwm_backward(x.numpy(), f, go.numpy(), grad_state=_np(gs))
+    assert rel_err(b["grad_x"], xt.grad.numpy()) < 1e-10
+    for name, w in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), Wt):
+        assert rel_err(b[name], w.grad.numpy()) < 1e-10, name
+    for name, w0 in zip(("W0_y", "W0_q", "W0_k", "w0_b"), W):
+        assert rel_err(b[name], w0.numpy()) < 1e-12
+
+
+def test_wide_c_oracle_backward_against_central_differences():
+    E, Y = 4, 13
+    x, W, go = srwm_inputs(1, 2, 5, E, seed=24, w_std=0.9, per_batch_state=True, y_width=Y)
+    rng = np.random.default_rng(1)
+    dirs = [rng.standard_normal(t.shape) for t in [x] + W]
+    loss = lambda xs, Ws: float((oracle.srwm_forward(xs, *Ws)["out"] * go.numpy()).sum())
+    h = 1e-6
+    fd = (loss(x.numpy() + h * dirs[0], [w.numpy() + h * d for w, d in zip(W, dirs[1:])])
+          - loss(x.numpy() - h * dirs[0], [w.numpy() - h * d for w, d in zip(W, dirs[1:])])) / (2 * h)
+    f = oracle.srwm_forward(x.numpy(), *_np(W))
+    b = oracle.srwm_backward(x.numpy(), f, go.numpy())
+    an = sum((b[n] * d).sum() for n, d in
+             zip(("grad_x", "grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), dirs))
+    assert abs(fd - an) < 1e-7 * max(1.0, abs(an))
+
+
 # ---------------------------------------------------------- step-wise (RL learner) call pattern
 
 def _steps_inputs(N, H, L, E, seed, resets=True):
