@@ -15,8 +15,14 @@
 // the R-row operand slices to the tile lanes through a wave-private LDS strip.
 // x is streamed through LDS in tiles of TT steps, fetched one tile ahead.
 //
+// YB > 1 is the wide-output variant: W_y is E x (YB*E + 1), i.e. YB blocks of E columns, tiled
+// like the others (a lane then holds YB + 2 blocks), plus one last column that is kept like a
+// fifth column of w_b: one element per thread of the first E threads.  All y columns use
+// beta_y.  Rows of the wide tensors are not 16-byte aligned, so they are accessed word by word.
+//
 // Replaces self_ref_forward_kernel / self_ref_backward_kernel of the reference
-// (supervised_learning/self_ref_v0/self_ref_v0.cu:24-432, :534-1234).
+// (supervised_learning/self_ref_v0/self_ref_v0.cu:24-432, :534-1234) and, with YB = 3, those of
+// reinforcement_learning/torchbeast/self_ref_v1/self_ref_v1.cu:27-534, :639-1547.
 #include "common.h"
 #include "xlane.h"
 
@@ -69,10 +75,14 @@ __device__ __forceinline__ void store_vec(float *dst, const float *src) {
 }
 
 // RESET: the per-step reset to the shared weights is compiled in (p.keep != nullptr)
-template <int E, int NW, int R, bool RESET>
+template <int E, int NW, int R, bool RESET, int YB>
 __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams p) {
     using T = Tiling<E, NW, R>;
-    constexpr int RG = T::RG, CGW = T::CGW, CB = T::CB, NC = T::NC, TT = T::TT;
+    constexpr int RG = T::RG, CGW = T::CGW, CB = T::CB, TT = T::TT;
+    constexpr int NB = YB + 2, NC = NB * CB;          // blocks of E columns: y (YB of them) | q | k
+    constexpr bool XC = YB > 1;                       // one more y column, held like a column of w_b
+    constexpr int Y = XC ? YB * E + 1 : E;            // row length of W_y, out, y_diff
+    constexpr int QB = YB * CB, KB = (YB + 1) * CB;   // first lane column of the q / k block
 
     __shared__ __attribute__((aligned(16))) float xt[2][TT][E];   // input tiles, double buffered
     __shared__ float kt[2][TT];                                   // keep flags of the tile's steps
@@ -89,30 +99,41 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
-    const int64_t sEE = seq * E * E, sE4 = seq * E * 4;
+    const int64_t sEE = seq * E * E, sEY = seq * E * Y, sE4 = seq * E * 4;
     const float *xbase = p.x + n * p.xs_n + h * p.xs_h;
+    const bool has_y = XC && jb == 0;        // thread holds row el of the last y column
 
     float w[R][NC];
-    {
-        const float *src[3] = {p.Wy + sEE, p.Wq + sEE, p.Wk + sEE};
+    float wbe, wye = 0.f;
+    auto load_state = [&](const float *Wy, const float *Wq, const float *Wk, const float *wb) {
 #pragma unroll
-        for (int b = 0; b < 3; ++b)
+        for (int b = 0; b < NB; ++b) {
+            const float *src = b < YB ? Wy + b * E : b == YB ? Wq : Wk;
+            const int ld = b < YB ? Y : E;
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
-                for (int c = 0; c < CB; ++c) w[i][b * CB + c] = src[b][(r0 + i) * E + c0 + c];
-    }
-    float wbe = has_b ? p.wb[sE4 + el * 4 + jb] : 0.f;
+                for (int c = 0; c < CB; ++c) w[i][b * CB + c] = src[(r0 + i) * ld + c0 + c];
+        }
+        wbe = has_b ? wb[el * 4 + jb] : 0.f;
+        if constexpr (XC) wye = has_y ? Wy[el * Y + YB * E] : 0.f;
+    };
+    load_state(p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4);
     // replaces the state by the weights all batch rows of this head share (per-step reset)
     auto reset_state = [&]() {
-        const float *src[3] = {p.sWy + (int64_t)h * E * E, p.sWq + (int64_t)h * E * E, p.sWk + (int64_t)h * E * E};
+        load_state(p.sWy + (int64_t)h * E * Y, p.sWq + (int64_t)h * E * E, p.sWk + (int64_t)h * E * E,
+                   p.swb + (int64_t)h * E * 4);
+    };
+    // rows of the Y-wide tensors start at any word: no vector stores there
+    auto store_y = [&](float *dst, const float *v) {
+        if constexpr (XC) {
 #pragma unroll
-        for (int b = 0; b < 3; ++b)
+            for (int b = 0; b < YB; ++b)
 #pragma unroll
-            for (int i = 0; i < R; ++i)
-#pragma unroll
-                for (int c = 0; c < CB; ++c) w[i][b * CB + c] = src[b][(r0 + i) * E + c0 + c];
-        wbe = has_b ? p.swb[(int64_t)h * E * 4 + el * 4 + jb] : 0.f;
+                for (int c = 0; c < CB; ++c) dst[b * E + c0 + c] = v[b * CB + c];
+        } else {
+            store_vec<CB>(dst + c0, v);
+        }
     };
 
     // tile loader: thread -> (step tid / (E/4), 4 consecutive elements)
@@ -141,7 +162,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 
         for (int tt = 0; tt < tlen; ++tt) {
             const int t = tile * TT + tt, par = t & 1;
-            const int64_t o = (seq * p.L + t) * E, ob = (seq * p.L + t) * 4;
+            const int64_t o = (seq * p.L + t) * E, oy = (seq * p.L + t) * Y, ob = (seq * p.L + t) * 4;
             if constexpr (RESET) {
                 if (kt[buf][tt] == 0.f) reset_state();   // uniform over the workgroup
             }
@@ -160,11 +181,15 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             group_sum_n<RG, NC>(acc);
             const float pb = group_sum<E>(wbe * xb);
             if (rg == 0) {
-                store_vec<CB>(p.out + o + c0, &acc[0]);
-                store_vec<CB>(&raw[par][0][c0], &acc[CB]);
-                store_vec<CB>(&raw[par][1][c0], &acc[2 * CB]);
+                store_y(p.out + oy, &acc[0]);
+                store_vec<CB>(&raw[par][0][c0], &acc[QB]);
+                store_vec<CB>(&raw[par][1][c0], &acc[KB]);
             }
             if (has_b && el == 0) rawb[par][jb] = pb;
+            if constexpr (XC) {
+                const float py = group_sum<E>(wye * xb);
+                if (has_y && el == 0) p.out[oy + YB * E] = py;
+            }
             if (tt == tlen - 1 && tile + 1 < ntiles) {
                 *reinterpret_cast<float4 *>(&xt[buf ^ 1][ld_row][ld_col]) = xnext;
                 if (RESET && tid < TT) kt[buf ^ 1][tid] = knext;
@@ -209,34 +234,42 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             group_sum_n<RG, NC>(dif);
             const float pbd = group_sum<E>(wbe * dv);
             if (rg == 0) {
-                store_vec<CB>(p.ydiff + o + c0, &dif[0]);
-                store_vec<CB>(p.qdiff + o + c0, &dif[CB]);
-                store_vec<CB>(p.kdiff + o + c0, &dif[2 * CB]);
+                store_y(p.ydiff + oy, &dif[0]);
+                store_vec<CB>(p.qdiff + o + c0, &dif[QB]);
+                store_vec<CB>(p.kdiff + o + c0, &dif[KB]);
             }
             if (has_b && el == 0) p.bdiff[ob + jb] = pbd;
 
-            // ---- rank-1 write W += k (x) (beta_blk * diff)
+            // ---- rank-1 write W += k (x) (beta_blk * diff); every y block uses beta_y
             float ins[NC];
 #pragma unroll
-            for (int c = 0; c < NC; ++c) ins[c] = bt[c / CB] * dif[c];
+            for (int c = 0; c < NC; ++c) ins[c] = bt[c / CB < YB ? 0 : c / CB - YB + 1] * dif[c];
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < NC; ++c) w[i][c] = fmaf(kr[i], ins[c], w[i][c]);
             wbe = fmaf(kn, bt[3] * pbd, wbe);
+            if constexpr (XC) {
+                const float pyd = group_sum<E>(wye * dv);
+                if (has_y && el == 0) p.ydiff[oy + YB * E] = pyd;
+                wye = fmaf(kn, bt[0] * pyd, wye);
+            }
         }
     }
 
-    {
-        float *dst[3] = {p.Wy + sEE, p.Wq + sEE, p.Wk + sEE};
 #pragma unroll
-        for (int b = 0; b < 3; ++b)
+    for (int b = 0; b < NB; ++b) {
+        float *dst = b < YB ? p.Wy + sEY + b * E : b == YB ? p.Wq + sEE : p.Wk + sEE;
+        const int ld = b < YB ? Y : E;
 #pragma unroll
-            for (int i = 0; i < R; ++i)
+        for (int i = 0; i < R; ++i)
 #pragma unroll
-                for (int c = 0; c < CB; ++c) dst[b][(r0 + i) * E + c0 + c] = w[i][b * CB + c];
+            for (int c = 0; c < CB; ++c) dst[(r0 + i) * ld + c0 + c] = w[i][b * CB + c];
     }
     if (has_b) p.wb[sE4 + el * 4 + jb] = wbe;
+    if constexpr (XC) {
+        if (has_y) p.Wy[sEY + el * Y + YB * E] = wye;
+    }
 }
 
 // ---------------------------------------------------------------------------------------
@@ -249,19 +282,28 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 // and two workgroup barriers (after the first pair of row sums, after the grad_x row sum).
 // The seven per-step vectors and beta are streamed through a single LDS tile of TT steps;
 // the next tile is fetched into registers one tile ahead.
-template <int E, int NW, int R>
+template <int E, int NW, int R, int YB>
 __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams p) {
     using T = Tiling<E, NW, R>;
-    constexpr int RG = T::RG, CGW = T::CGW, NCG = T::NCG, CB = T::CB, NC = T::NC, TT = T::TT;
+    constexpr int RG = T::RG, CGW = T::CGW, NCG = T::NCG, CB = T::CB, TT = T::TT, NT = T::NT;
     static_assert(RG == 8, "row-sum reduction assumes column groups 8 lanes apart");
-    enum { VX, VQ, VK, VYD, VQD, VKD, VGO, NVEC };
+    constexpr int NB = YB + 2, NC = NB * CB;          // blocks of E columns: y (YB of them) | q | k
+    constexpr bool XC = YB > 1;                       // one more y column, held like a column of w_b
+    constexpr int Y = XC ? YB * E + 1 : E;            // row length of W_y, grad_out, y_diff
+    constexpr int YS = (Y + 3) & ~3;                  // its row stride in LDS
+    constexpr int QB = YB * CB, KB = (YB + 1) * CB;   // first lane column of the q / k block
+    constexpr int NXS = XC ? 5 : 4;                   // narrow columns: w_b and the last y column
+    constexpr int NWL = XC ? (TT * Y + NT - 1) / NT : 1;   // words per thread of a wide tile
+    enum { VX, VQ, VK, VQD, VKD, NVEC };
 
     __shared__ __attribute__((aligned(16))) float tl[NVEC][TT][E];  // per-step vectors of the tile
+    __shared__ __attribute__((aligned(16))) float tyd[TT][YS];      // y_diff of the tile
+    __shared__ __attribute__((aligned(16))) float tgo[TT][YS];      // grad_out of the tile
     __shared__ __attribute__((aligned(16))) float tb[2][TT][4];     // beta | beta_diff
     __shared__ __attribute__((aligned(16))) float rowm[3][NW][E];   // row sums per wave: G ins | W gdiff | W gpre
-    __shared__ __attribute__((aligned(16))) float rowb[3][4][E];    // same, contribution of the w_b block
-    __shared__ __attribute__((aligned(16))) float gbp[NCG][4];      // per column group: sum gins*diff per block
-    __shared__ __attribute__((aligned(16))) float gbp3[4];          // same for the four w_b columns
+    __shared__ __attribute__((aligned(16))) float rowb[3][NXS][E];  // same, contribution of the narrow columns
+    __shared__ __attribute__((aligned(16))) float gbp[NCG][4];      // per column group: sum gins*diff per beta
+    __shared__ __attribute__((aligned(16))) float gbp3[8];          // same for the narrow columns
     __shared__ __attribute__((aligned(16))) float exch[NW][2][E];   // per wave: g_pre of the q | k block
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -273,41 +315,57 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
-    const int64_t sEE = seq * E * E, sE4 = seq * E * 4;
+    const int64_t sEE = seq * E * E, sEY = seq * E * Y, sE4 = seq * E * 4;
     const float *xbase = p.x + n * p.xs_n + h * p.xs_h;
     const float *gobase = p.go + n * p.gs_n + h * p.gs_h;
+    const bool has_y = XC && jb == 0;        // thread holds row el of the last y column
 
     float w[R][NC], g[R][NC];
-    {
-        const float *src[3] = {p.Wy + sEE, p.Wq + sEE, p.Wk + sEE};
-        const float *gsrc[3] = {p.gWy + sEE, p.gWq + sEE, p.gWk + sEE};
 #pragma unroll
-        for (int b = 0; b < 3; ++b)
+    for (int b = 0; b < NB; ++b) {
+        const float *src = b < YB ? p.Wy + sEY + b * E : b == YB ? p.Wq + sEE : p.Wk + sEE;
+        const float *gsrc = b < YB ? p.gWy + sEY + b * E : b == YB ? p.gWq + sEE : p.gWk + sEE;
+        const int ld = b < YB ? Y : E;
 #pragma unroll
-            for (int i = 0; i < R; ++i)
+        for (int i = 0; i < R; ++i)
 #pragma unroll
-                for (int c = 0; c < CB; ++c) {
-                    w[i][b * CB + c] = src[b][(r0 + i) * E + c0 + c];
-                    g[i][b * CB + c] = p.grad_state_mode ? gsrc[b][(r0 + i) * E + c0 + c] : 0.f;
-                }
+            for (int c = 0; c < CB; ++c) {
+                w[i][b * CB + c] = src[(r0 + i) * ld + c0 + c];
+                g[i][b * CB + c] = p.grad_state_mode ? gsrc[(r0 + i) * ld + c0 + c] : 0.f;
+            }
     }
     float wbe = has_b ? p.wb[sE4 + el * 4 + jb] : 0.f;
     float gbe = (has_b && p.grad_state_mode) ? p.gwb[sE4 + el * 4 + jb] : 0.f;
+    float wye = 0.f, gye = 0.f;
+    if constexpr (XC) {
+        wye = has_y ? p.Wy[sEY + el * Y + YB * E] : 0.f;
+        gye = (has_y && p.grad_state_mode) ? p.gWy[sEY + el * Y + YB * E] : 0.f;
+    }
 
     const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
     // next tile, staged in registers
     float4 n_x, n_go, n_q, n_k, n_yd, n_qd, n_kd, n_bt, n_bd;
+    float n_ydw[NWL], n_gow[NWL];   // wide rows start at any word: fetched word by word
 #define SRWM_BWD_LOAD_TILE(tile_)                                                                  \
     do { /* rows past the end of the sequence are clamped: they are loaded but never used */       \
         const int t_ = min((tile_) * TT + ld_row, p.L - 1);                                        \
         const int64_t o_ = (seq * p.L + t_) * E + ld_col;                                          \
         n_x = *reinterpret_cast<const float4 *>(xbase + t_ * p.xs_l + ld_col);                     \
-        n_go = *reinterpret_cast<const float4 *>(gobase + t_ * p.gs_l + ld_col);                   \
         n_q = *reinterpret_cast<const float4 *>(p.q + o_);                                         \
         n_k = *reinterpret_cast<const float4 *>(p.k + o_);                                         \
-        n_yd = *reinterpret_cast<const float4 *>(p.ydiff + o_);                                    \
         n_qd = *reinterpret_cast<const float4 *>(p.qdiff + o_);                                    \
         n_kd = *reinterpret_cast<const float4 *>(p.kdiff + o_);                                    \
+        if constexpr (XC) {                                                                        \
+            _Pragma("unroll") for (int i_ = 0; i_ < NWL; ++i_) {                                   \
+                const int f_ = min(tid + i_ * NT, TT * Y - 1), r_ = f_ / Y, m_ = f_ - r_ * Y;      \
+                const int64_t tw_ = min((tile_) * TT + r_, p.L - 1);                               \
+                n_ydw[i_] = p.ydiff[(seq * p.L + tw_) * Y + m_];                                   \
+                n_gow[i_] = gobase[tw_ * p.gs_l + m_];                                             \
+            }                                                                                      \
+        } else {                                                                                   \
+            n_go = *reinterpret_cast<const float4 *>(gobase + t_ * p.gs_l + ld_col);               \
+            n_yd = *reinterpret_cast<const float4 *>(p.ydiff + o_);                                \
+        }                                                                                          \
         const int64_t ob_ = (seq * p.L + min((tile_) * TT + (tid % TT), p.L - 1)) * 4;             \
         n_bt = *reinterpret_cast<const float4 *>(p.beta + ob_);                                    \
         n_bd = *reinterpret_cast<const float4 *>(p.bdiff + ob_);                                   \
@@ -315,12 +373,22 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 #define SRWM_BWD_STORE_TILE()                                                                      \
     do {                                                                                           \
         *reinterpret_cast<float4 *>(&tl[VX][ld_row][ld_col]) = n_x;                                \
-        *reinterpret_cast<float4 *>(&tl[VGO][ld_row][ld_col]) = n_go;                              \
         *reinterpret_cast<float4 *>(&tl[VQ][ld_row][ld_col]) = n_q;                                \
         *reinterpret_cast<float4 *>(&tl[VK][ld_row][ld_col]) = n_k;                                \
-        *reinterpret_cast<float4 *>(&tl[VYD][ld_row][ld_col]) = n_yd;                              \
         *reinterpret_cast<float4 *>(&tl[VQD][ld_row][ld_col]) = n_qd;                              \
         *reinterpret_cast<float4 *>(&tl[VKD][ld_row][ld_col]) = n_kd;                              \
+        if constexpr (XC) {                                                                        \
+            _Pragma("unroll") for (int i_ = 0; i_ < NWL; ++i_) {                                   \
+                const int f_ = tid + i_ * NT, r_ = f_ / Y, m_ = f_ - r_ * Y;                       \
+                if (f_ < TT * Y) {                                                                 \
+                    tyd[r_][m_] = n_ydw[i_];                                                       \
+                    tgo[r_][m_] = n_gow[i_];                                                       \
+                }                                                                                  \
+            }                                                                                      \
+        } else {                                                                                   \
+            *reinterpret_cast<float4 *>(&tgo[ld_row][ld_col]) = n_go;                              \
+            *reinterpret_cast<float4 *>(&tyd[ld_row][ld_col]) = n_yd;                              \
+        }                                                                                          \
         if (tid < TT) {                                                                            \
             *reinterpret_cast<float4 *>(&tb[0][tid][0]) = n_bt;                                    \
             *reinterpret_cast<float4 *>(&tb[1][tid][0]) = n_bd;                                    \
@@ -348,10 +416,13 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 #pragma unroll
             for (int i = 0; i < R; ++i) dvr[i] -= kr[i];
             float dif[NC], gpre[NC];
-            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[0]), &tl[VYD][tt][c0]);
-            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[CB]), &tl[VQD][tt][c0]);
-            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[2 * CB]), &tl[VKD][tt][c0]);
-            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[0]), &tl[VGO][tt][c0]);
+#pragma unroll
+            for (int b = 0; b < YB; ++b) {
+                lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[b * CB]), &tyd[tt][b * E + c0]);
+                lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[b * CB]), &tgo[tt][b * E + c0]);
+            }
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[QB]), &tl[VQD][tt][c0]);
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[KB]), &tl[VKD][tt][c0]);
             float bt[4];
             lds_read_vec<4>(bt, &tb[0][tt][0]);
             const float bd = tb[1][tt][jb & 3];
@@ -359,15 +430,23 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             const float dvb = qb - kb;
 
             // ---- revert the write: W_{t-1} = W_t - k (x) ins
+            constexpr auto beta_of = [](int c) { return c / CB < YB ? 0 : c / CB - YB + 1; };
             float ins[NC];
 #pragma unroll
-            for (int c = 0; c < NC; ++c) ins[c] = bt[c / CB] * dif[c];
+            for (int c = 0; c < NC; ++c) ins[c] = bt[beta_of(c)] * dif[c];
             const float insb = bt[3] * bd;
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < NC; ++c) w[i][c] = fmaf(-kr[i], ins[c], w[i][c]);
             wbe = fmaf(-kb, insb, wbe);
+            float ydl = 0.f, insy = 0.f, gprey = 0.f;   // last y column: its diff, insert and upstream gradient
+            if constexpr (XC) {
+                ydl = tyd[tt][YB * E];
+                gprey = tgo[tt][YB * E];
+                insy = bt[0] * ydl;
+                wye = fmaf(-kb, insy, wye);
+            }
 
             // ---- g_ins = G^T k (column sums), g_diff = beta_blk * g_ins
             float gdif[NC];
@@ -381,11 +460,16 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             float pg[3] = {0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
-                pg[c / CB] = fmaf(gdif[c], dif[c], pg[c / CB]);
-                gdif[c] *= bt[c / CB];
+                pg[beta_of(c)] = fmaf(gdif[c], dif[c], pg[beta_of(c)]);
+                gdif[c] *= bt[beta_of(c)];
             }
             const float ginsb = group_sum<E>(gbe * kb);
             const float gdifb = bt[3] * ginsb;
+            float ginsy = 0.f, gdify = 0.f;
+            if constexpr (XC) {
+                ginsy = group_sum<E>(gye * kb);
+                gdify = bt[0] * ginsy;
+            }
 
             // ---- row sums  a = G ins,  u = W_{t-1} g_diff
             float a[R], u[R];
@@ -406,6 +490,13 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 rowb[1][jb][el] = wbe * gdifb;
                 if (el == 0) gbp3[jb] = ginsb * bd;
             }
+            if constexpr (XC) {
+                if (has_y) {
+                    rowb[0][4][el] = gye * insy;
+                    rowb[1][4][el] = wye * gdify;
+                    if (el == 0) gbp3[4] = ginsy * ydl;
+                }
+            }
             if (rg == 0) *reinterpret_cast<float4 *>(&gbp[cg][0]) = make_float4(pg[0], pg[1], pg[2], 0.f);
             __syncthreads();
 
@@ -417,7 +508,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 gq += rowm[1][wv][el];
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int j = 0; j < NXS; ++j) {
                 gk += rowb[0][j][el];
                 gq += rowb[1][j][el];
             }
@@ -436,6 +527,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 float p3[4];
                 lds_read_vec<4>(p3, &gbp3[0]);
                 gb[3] = (p3[0] + p3[1]) + (p3[2] + p3[3]);
+                if constexpr (XC) gb[0] += gbp3[4];
             }
             float gpb[4];
 #pragma unroll
@@ -446,8 +538,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 exch[wave][1][lane] = gpk;
             }
             wave_lds_fence();
-            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[CB]), &exch[wave][0][c0]);
-            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[2 * CB]), &exch[wave][1][c0]);
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[QB]), &exch[wave][0][c0]);
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[KB]), &exch[wave][1][c0]);
 
             // ---- grad_x = W_{t-1} g_pre (row sums)
             float sx[R];
@@ -459,13 +551,16 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             }
             stride8_reduce_store<R>(sx, &rowm[2][wave][r0], lane);
             if (has_b) rowb[2][jb][el] = wbe * gpreb;
+            if constexpr (XC) {
+                if (has_y) rowb[2][4][el] = wye * gprey;
+            }
             __syncthreads();
             if (tid < E) {
                 float s = 0.f;
 #pragma unroll
                 for (int wv = 0; wv < NW; ++wv) s += rowm[2][wv][tid];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) s += rowb[2][j][tid];
+                for (int j = 0; j < NXS; ++j) s += rowb[2][j][tid];
                 p.gx[o + tid] = s;
             }
 
@@ -476,6 +571,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 for (int c = 0; c < NC; ++c)
                     g[i][c] = fmaf(dvr[i], gdif[c], fmaf(xr[i], gpre[c], g[i][c]));
             gbe = fmaf(dvb, gdifb, fmaf(xb, gpreb, gbe));
+            if constexpr (XC) gye = fmaf(dvb, gdify, fmaf(xb, gprey, gye));
 
             if (tt == 0 && tile > 0) {
                 // every wave is past its last read of this tile (all reads precede the
@@ -487,36 +583,44 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     }
 
     {
-        float *dst[3] = {p.gWy + sEE, p.gWq + sEE, p.gWk + sEE};
         const bool accum = p.grad_state_mode == 2u;
 #pragma unroll
-        for (int b = 0; b < 3; ++b)
+        for (int b = 0; b < NB; ++b) {
+            float *dst = b < YB ? p.gWy + sEY + b * E : b == YB ? p.gWq + sEE : p.gWk + sEE;
+            const int ld = b < YB ? Y : E;
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < CB; ++c) {
-                    float *d = &dst[b][(r0 + i) * E + c0 + c];
+                    float *d = &dst[(r0 + i) * ld + c0 + c];
                     *d = accum ? *d + g[i][b * CB + c] : g[i][b * CB + c];
                 }
+        }
         if (has_b) {
             float *d = &p.gwb[sE4 + el * 4 + jb];
             *d = accum ? *d + gbe : gbe;
         }
+        if constexpr (XC) {
+            if (has_y) {
+                float *d = &p.gWy[sEY + el * Y + YB * E];
+                *d = accum ? *d + gye : gye;
+            }
+        }
     }
 }
 
-template <int E, int NW, int R>
+template <int E, int NW, int R, int YB = 1>
 int launch_bwd(const SrwmBwdParams &p, hipStream_t s) {
-    hipLaunchKernelGGL((srwm_bwd_tiled_kernel<E, NW, R>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    hipLaunchKernelGGL((srwm_bwd_tiled_kernel<E, NW, R, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
-template <int E, int NW, int R>
+template <int E, int NW, int R, int YB = 1>
 int launch_fwd(const SrwmFwdParams &p, hipStream_t s) {
     if (p.keep)
-        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, true>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, true, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
     else
-        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, false>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, false, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
@@ -527,11 +631,20 @@ bool aligned16(const void *ptr, int64_t a, int64_t b, int64_t c) {
 }  // namespace
 
 int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
-    if (p.Y != p.E) return -1;   // the lane tiling assumes three E x E blocks
     if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l)) return -1;
     const void *dense[] = {p.q, p.k, p.beta, p.ydiff, p.qdiff, p.kdiff, p.bdiff, p.out};
     for (const void *d : dense)
         if ((uintptr_t)d % 16) return -1;
+    if (p.Y == 3 * p.E + 1) {   // wide output block: three tiled blocks of E columns and one more column
+        switch (p.E) {
+            case 64: return launch_fwd<64, 4, 16, 3>(p, s);
+            case 32: return launch_fwd<32, 4, 4, 3>(p, s);
+            case 16: return launch_fwd<16, 1, 2, 3>(p, s);
+            case 8: return launch_fwd<8, 1, 1, 3>(p, s);
+            default: return -1;
+        }
+    }
+    if (p.Y != p.E) return -1;
     switch (p.E) {
         case 64: return launch_fwd<64, 4, 16>(p, s);
         case 32: return launch_fwd<32, 4, 4>(p, s);
@@ -542,11 +655,20 @@ int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
 }
 
 int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s) {
-    if (p.Y != p.E) return -1;
-    if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l) || !aligned16(p.go, p.gs_n, p.gs_h, p.gs_l)) return -1;
-    const void *dense[] = {p.q, p.k, p.beta, p.ydiff, p.qdiff, p.kdiff, p.bdiff, p.gx};
+    if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l)) return -1;
+    const void *dense[] = {p.q, p.k, p.beta, p.qdiff, p.kdiff, p.bdiff, p.gx};
     for (const void *d : dense)
         if ((uintptr_t)d % 16) return -1;
+    if (p.Y == 3 * p.E + 1) {   // grad_out and y_diff rows are read word by word: any alignment
+        switch (p.E) {
+            case 64: return launch_bwd<64, 4, 8, 3>(p, s);
+            case 32: return launch_bwd<32, 4, 4, 3>(p, s);
+            case 16: return launch_bwd<16, 1, 2, 3>(p, s);
+            case 8: return launch_bwd<8, 1, 1, 3>(p, s);
+            default: return -1;
+        }
+    }
+    if (p.Y != p.E || (uintptr_t)p.ydiff % 16 || !aligned16(p.go, p.gs_n, p.gs_h, p.gs_l)) return -1;
     switch (p.E) {
         case 64: return launch_bwd<64, 4, 8>(p, s);
         case 32: return launch_bwd<32, 4, 4>(p, s);

@@ -270,7 +270,9 @@ def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
     ((3, 5, 11, 8), 25, 0.6, True, True),                    # the reference self-test's shape for this variant
     ((4, 8, 100, 32), 97, 1 / math.sqrt(32), True, False),   # RL learner shape: 8 heads of 32, Y = 3E+1
     ((2, 4, 40, 16), 49, 0.25, True, True),
-    ((1, 2, 20, 48), 145, 0.1, True, True),                  # largest multiple of 16 whose backward fits in LDS
+    ((1, 2, 20, 48), 145, 0.1, True, True),                  # LDS-resident kernels, large state
+    ((2, 2, 40, 64), 193, 0.1, True, True),                  # E = 64: only the register-resident backward can hold it
+    ((2, 3, 37, 32), 50, 0.3, False, True),                  # a width that is not 3E+1 (LDS-resident kernels)
     ((1, 3, 7, 5), 16, 0.8, False, True),                    # odd head size
     ((2, 2, 1, 16), 49, 0.3, True, True),                    # L = 1
     ((1, 2, 9, 8), 3, 0.7, False, True),                     # narrower than E
