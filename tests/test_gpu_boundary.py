@@ -1,0 +1,134 @@
+"""The C-ABI boundary under the calling conditions of the reference's RL learner: several Python
+threads, each on its own HIP stream (reinforcement_learning/torchbeast_procgen/polybeast_learner.py
+runs inference and learner threads side by side), work enqueued on the caller's current stream
+without any synchronisation inside the library, and argument errors reported as negative codes
+before anything is launched."""
+import ctypes
+import threading
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import delta_inputs, rel_err, srwm_inputs
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def _dev():
+    return torch.device("cuda:0")
+
+
+def test_two_threads_on_their_own_streams():
+    """Each thread runs SRWM and delta-rule forward+backward through the autograd operators a few
+    times on its own stream with its own inputs; every result must equal the oracle's."""
+    print("case two threads", flush=True)
+    from fast_weight import fast_weight_delta
+    from self_ref_v0 import self_ref_v0
+    dev = _dev()
+    results, errors = {}, []
+
+    def worker(idx):
+        try:
+            stream = torch.cuda.Stream(device=dev)
+            with torch.cuda.stream(stream):
+                for it in range(4):
+                    seed = 100 * idx + it
+                    x, W, go = srwm_inputs(3, 4, 40, 32, seed=seed, w_std=0.2, per_batch_state=True)
+                    xd = x.to(dev, torch.float32).requires_grad_(True)
+                    Wd = [w.to(dev, torch.float32).requires_grad_(True) for w in W]
+                    out = self_ref_v0(xd, *[w.clone() for w in Wd])
+                    (out * go.to(dev, torch.float32)).sum().backward()
+                    q, k, v, beta, W0, dgo = delta_inputs(2, 4, 70, 64, 64, seed=seed, qk="softmax", w0_std=0.1)
+                    leaves = [t.to(dev, torch.float32).requires_grad_(True) for t in (q, k, v, beta)]
+                    dout = fast_weight_delta(*leaves, W0.to(dev, torch.float32))
+                    (dout * dgo.to(dev, torch.float32)).sum().backward()
+                    stream.synchronize()
+                    results[(idx, it)] = (out.detach().cpu(), xd.grad.cpu(), Wd[0].grad.cpu(),
+                                          dout.detach().cpu(), leaves[1].grad.cpu())
+        except Exception as e:   # surfaced in the main thread
+            errors.append(e)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    assert len(results) == 8
+    for (idx, it), (out, gx, gwy, dout, gk) in results.items():
+        seed = 100 * idx + it
+        x, W, go = srwm_inputs(3, 4, 40, 32, seed=seed, w_std=0.2, per_batch_state=True)
+        f = oracle.srwm_forward(x.numpy(), *[w.numpy() for w in W])
+        b = oracle.srwm_backward(x.numpy(), f, go.numpy())
+        assert rel_err(out.numpy(), f["out"]) < TOL and rel_err(gx.numpy(), b["grad_x"]) < TOL
+        assert rel_err(gwy.numpy(), b["grad_W_y"]) < TOL
+        q, k, v, beta, W0, dgo = delta_inputs(2, 4, 70, 64, 64, seed=seed, qk="softmax", w0_std=0.1)
+        base = [t.numpy() for t in (q, k, v, beta, W0)]
+        df = oracle.delta_forward(*base)
+        db = oracle.delta_backward(*base[:4], df, dgo.numpy())
+        assert rel_err(dout.numpy(), df["out"]) < TOL and rel_err(gk.numpy(), db["grad_K"]) < TOL
+
+
+def test_work_is_ordered_on_the_callers_stream():
+    """Inputs are produced on a side stream right before the call and results consumed right
+    after it, with no synchronisation in between: correct only if the kernels are enqueued on
+    that stream."""
+    print("case stream order", flush=True)
+    import srwm_hip
+    dev = _dev()
+    N, H, L, E = 4, 8, 64, 32
+    x, W, go = srwm_inputs(N, H, L, E, seed=9, w_std=0.2, per_batch_state=True)
+    f = oracle.srwm_forward(x.numpy(), *[w.numpy() for w in W])
+    xh = x.to(torch.float32).pin_memory()
+    Wh = [w.to(torch.float32).pin_memory() for w in W]
+    side = torch.cuda.Stream(device=dev)
+    big = lambda: torch.empty((N, H, L, E), device=dev)
+    small = lambda: torch.empty((N, H, L, 4), device=dev)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        filler = torch.randn(4096, 4096, device=dev)
+        for _ in range(10):
+            filler = filler @ filler * 1e-4            # keeps the side stream busy before the copies
+        xd = xh.to(dev, non_blocking=True)
+        Wd = [w.to(dev, non_blocking=True) for w in Wh]
+        bufs = [big(), big(), small(), big(), big(), big(), small(), big()]
+        srwm_hip.self_ref_forward(xd, *Wd, *bufs)
+        out_h = bufs[-1].to("cpu", non_blocking=True)
+        wy_h = Wd[0].to("cpu", non_blocking=True)
+    side.synchronize()
+    assert rel_err(out_h.numpy(), f["out"]) < TOL
+    assert rel_err(wy_h.numpy(), f["W_y"]) < TOL
+
+
+def test_argument_errors_come_back_as_negative_codes():
+    """Straight through ctypes: null pointers, bad sizes, unknown flags and a state that cannot
+    fit return SRWM_E* codes and launch nothing (the output buffer keeps its fill value)."""
+    import srwm_hip
+    lib = srwm_hip.lib()
+    dev = _dev()
+    N, H, L, E = 1, 2, 3, 16
+    x = torch.zeros(N, H, L, E, device=dev)
+    W = [torch.zeros(N, H, E, E, device=dev) for _ in range(3)] + [torch.zeros(N, H, E, 4, device=dev)]
+    big = lambda: torch.full((N, H, L, E), 7.0, device=dev)
+    small = lambda: torch.full((N, H, L, 4), 7.0, device=dev)
+    outs = [big(), big(), small(), big(), big(), big(), small(), big()]
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    strides = (ctypes.c_int64 * 3)(*x.stride()[:3])
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    call = lambda xs, n, e, flags, xp=P(x): lib.srwm_forward_f32(
+        xp, xs, *[P(w) for w in W], *[P(o) for o in outs], n, H, L, e, flags, stream)
+    assert call(strides, N, E, 0, ctypes.c_void_p(None)) == -1      # SRWM_EINVAL: null input
+    assert call(None, N, E, 0) == -1                                 # null stride array
+    assert call(strides, 0, E, 0) == -1                              # empty batch
+    assert call(strides, N, E, 1 << 9) == -1                         # unknown flag bit
+    assert call(strides, N, 4096, 0) == -2                           # SRWM_ESIZE
+    torch.cuda.synchronize()
+    assert all(bool((o == 7.0).all()) for o in outs)
+    assert call(strides, N, E, 0) == 0
+    torch.cuda.synchronize()
+    assert bool((outs[-1] == 0.0).all())                             # x = 0 -> y = 0, and it did run
+    for code in (-1, -2, -3, -4):
+        assert len(lib.srwm_hip_strerror(code)) > 8
