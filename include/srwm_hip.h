@@ -51,6 +51,12 @@ extern "C" {
                                      ones (forward: chunks of 64 steps; backward: a sweep over memory columns and
                                      one over memory rows); E == M in {64, 128}, else SRWM_ENOKERNEL.  Forward and
                                      backward may be mixed freely: both forms emit / consume the same v_old, v_insert */
+/* srwm_layer_forward_f32 / srwm_layer_backward_f32 only: */
+#define SRWM_FLAG_STATE_SHIFT 64u    /* W_y..w_b hold the state MINUS the head's shared weights, on entry and on
+                                        exit (how the RL layers carry it, torchbeast/layer.py:389-418) */
+#define SRWM_FLAG_FRESH_STATE 128u   /* forward: start from the shared weights; W_y..w_b are outputs only */
+#define SRWM_FLAG_SOFTMAX_INPUT 256u /* x is the layer input BEFORE its softmax over the last axis
+                                        (layer.py:382-384); the kernels apply it and grad_x refers to that input */
 
 /*
  * SRWM forward.  Replaces self_ref_forward(), supervised_learning/self_ref_v0/
@@ -137,6 +143,46 @@ SRWM_API int srwm_forward_steps_f32(const float *x, const int64_t x_strides[3], 
                            float *q, float *k, float *beta,
                            float *y_diff, float *q_diff, float *k_diff, float *beta_diff,
                            float *out, int N, int H, int L, int E, unsigned flags, void *stream);
+
+/*
+ * The SRWM operator as the reference's layers use it, with their elementwise prologue and epilogue
+ * folded into the kernels.  No counterpart function in the reference: SRWMlayer.forward
+ * (supervised_learning/layer.py:156-195) and SRlayer.forward (reinforcement_learning/torchbeast/
+ * layer.py:377-421) build the per-row weights with `state + W.repeat(bsz, 1, 1, 1)`, soft-max the
+ * input, call the operator, and subtract `W.repeat(...)` again to obtain the carried shift; autograd
+ * sums the per-row weight gradients over the batch.  Here:
+ *   sW_y [H,E,Y], sW_q, sW_k [H,E,E], sw_b [H,E,4]   the shared weights, read directly (no repeat)
+ *   W_y .. w_b  dense [N,H,E,.]   SRWM_FLAG_FRESH_STATE: outputs only (start from the shared weights);
+ *                                 otherwise in: initial state, out: final state; with
+ *                                 SRWM_FLAG_STATE_SHIFT both as the difference from the shared weights
+ *   keep        as in srwm_forward_steps_f32 (NULL = no resets)
+ *   Y           columns of W_y (E, or 3E+1 for the wide variant)
+ * srwm_forward_steps_f32 is this function with Y = E and none of the three flags.
+ * Backward (full back-propagation through the sequence; keep must have been NULL):
+ *   W_y .. w_b  the final state as the forward left it (same SRWM_FLAG_STATE_SHIFT)
+ *   gW_y .. gw_b dense [N,H,E,.]  per batch row, SRWM_GRAD_STATE_* semantics: dL/d(initial state of the row)
+ *   gsW_y .. gsw_b dense [H,E,.] or all NULL: the sum of the former over the batch = the gradient the
+ *                                 shared weights receive through the initial state (second launch, fixed
+ *                                 summation order)
+ *   grad_x      with SRWM_FLAG_SOFTMAX_INPUT the gradient of the un-soft-maxed input
+ */
+SRWM_API int srwm_layer_forward_f32(const float *x, const int64_t x_strides[3], const float *keep,
+                           const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
+                           float *W_y, float *W_q, float *W_k, float *w_b,
+                           float *q, float *k, float *beta,
+                           float *y_diff, float *q_diff, float *k_diff, float *beta_diff,
+                           float *out, int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+
+SRWM_API int srwm_layer_backward_f32(const float *x, const int64_t x_strides[3],
+                            const float *q, const float *k, const float *beta,
+                            const float *y_diff, const float *q_diff, const float *k_diff,
+                            const float *beta_diff,
+                            const float *grad_out, const int64_t grad_out_strides[3],
+                            const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
+                            const float *W_y, const float *W_q, const float *W_k, const float *w_b,
+                            float *grad_x, float *gW_y, float *gW_q, float *gW_k, float *gw_b,
+                            float *gsW_y, float *gsW_q, float *gsW_k, float *gsw_b,
+                            int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
 /*
  * Gradient of that unroll with respect to x when the carried state is detached between steps
@@ -260,7 +306,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any signature change); currently 2. */
+/* ABI version of this header (bumped on any signature change); currently 3. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

@@ -46,7 +46,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 2; }
+int srwm_hip_abi_version(void) { return 3; }
 
 const char *srwm_hip_strerror(int code) {
     switch (code) {
@@ -99,26 +99,40 @@ int srwm_forward_f32(const float *x, const int64_t xs[3], float *Wy, float *Wq, 
                                  L, E, E, flags, stream);
 }
 
-int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
+int srwm_layer_forward_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
                            const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
                            float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
                            float *qdiff, float *kdiff, float *bdiff, float *out, int N, int H, int L,
-                           int E, unsigned flags, void *stream) {
+                           int E, int Y, unsigned flags, void *stream) {
     if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
         !out || !xs)
         return SRWM_EINVAL;
-    if (keep && (!sWy || !sWq || !sWk || !swb)) return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || (flags & ~(SRWM_FLAG_GENERIC))) return SRWM_EINVAL;
+    const unsigned known = SRWM_FLAG_GENERIC | SRWM_FLAG_STATE_SHIFT | SRWM_FLAG_FRESH_STATE | SRWM_FLAG_SOFTMAX_INPUT;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || (flags & ~known)) return SRWM_EINVAL;
+    const bool needs_shared = keep || (flags & (SRWM_FLAG_STATE_SHIFT | SRWM_FLAG_FRESH_STATE));
+    if (needs_shared && (!sWy || !sWq || !sWk || !swb)) return SRWM_EINVAL;
     if (!stride_ok(xs, N, H, L, E)) return SRWM_ESTRIDE;
     SrwmFwdParams p{x, xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff,
-                    out, N, H, L, E, keep, sWy, sWq, sWk, swb, E};
+                    out, N, H, L, E, keep, sWy, sWq, sWk, swb, Y};
+    p.mode = ((flags & SRWM_FLAG_STATE_SHIFT) ? kModeShift : 0u) | ((flags & SRWM_FLAG_FRESH_STATE) ? kModeFresh : 0u) |
+             ((flags & SRWM_FLAG_SOFTMAX_INPUT) ? kModeSoftmaxX : 0u);
     hipStream_t s = (hipStream_t)stream;
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_fwd_tiled(p, s);
         if (r >= 0) return r;
     }
-    if (srwm_fwd_generic_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
+    if (srwm_fwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_srwm_fwd_generic(p, s);
+}
+
+int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
+                           const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
+                           float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
+                           float *qdiff, float *kdiff, float *bdiff, float *out, int N, int H, int L,
+                           int E, unsigned flags, void *stream) {
+    if (flags & ~(SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    return srwm_layer_forward_f32(x, xs, keep, sWy, sWq, sWk, swb, Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff,
+                                  kdiff, bdiff, out, N, H, L, E, E, flags, stream);
 }
 
 int srwm_readout_grad_f32(const float *k, const float *beta, const float *ydiff, const float *keep,
@@ -201,6 +215,41 @@ int srwm_backward_f32(const float *x, const int64_t xs[3], const float *q, const
                       void *stream) {
     return srwm_backward_wide_f32(x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, Wy, Wq, Wk,
                                   wb, grad_x, gWy, gWq, gWk, gwb, N, H, L, E, E, flags, stream);
+}
+
+int srwm_layer_backward_f32(const float *x, const int64_t xs[3], const float *q, const float *k,
+                            const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
+                            const float *bdiff, const float *grad_out, const int64_t gs[3],
+                            const float *sWy, const float *sWq, const float *sWk, const float *swb,
+                            const float *Wy, const float *Wq, const float *Wk, const float *wb,
+                            float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, float *gsWy,
+                            float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
+                            unsigned flags, void *stream) {
+    if (!x || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff || !grad_out || !Wy || !Wq ||
+        !Wk || !wb || !grad_x || !gWy || !gWq || !gWk || !gwb || !xs || !gs)
+        return SRWM_EINVAL;
+    const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
+    const unsigned known = SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK | SRWM_FLAG_STATE_SHIFT | SRWM_FLAG_SOFTMAX_INPUT;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || mode == 3u || (flags & ~known)) return SRWM_EINVAL;
+    if ((flags & SRWM_FLAG_STATE_SHIFT) && (!sWy || !sWq || !sWk || !swb)) return SRWM_EINVAL;
+    const bool sums = gsWy || gsWq || gsWk || gswb;
+    if (sums && (!gsWy || !gsWq || !gsWk || !gswb)) return SRWM_EINVAL;
+    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, Y)) return SRWM_ESTRIDE;
+    SrwmBwdParams p{x, xs[0], xs[1], xs[2], q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out,
+                    gs[0], gs[1], gs[2], Wy, Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, N, H, L, E, mode, Y,
+                    sWy, sWq, sWk, swb};
+    p.mode = ((flags & SRWM_FLAG_STATE_SHIFT) ? kModeShift : 0u) | ((flags & SRWM_FLAG_SOFTMAX_INPUT) ? kModeSoftmaxX : 0u);
+    hipStream_t s = (hipStream_t)stream;
+    int r = -1;
+    if (!(flags & SRWM_FLAG_GENERIC)) r = launch_srwm_bwd_tiled(p, s);
+    if (r < 0) {
+        if (srwm_bwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
+        r = launch_srwm_bwd_generic(p, s);
+    }
+    if (r != 0 || !sums) return r;
+    const float *const src[4] = {gWy, gWq, gWk, gwb};
+    float *const dst[4] = {gsWy, gsWq, gsWk, gswb};
+    return launch_srwm_batch_sum(src, dst, N, H, E, Y, s);
 }
 
 int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],

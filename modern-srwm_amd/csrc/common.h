@@ -9,6 +9,11 @@ namespace fw {
 
 constexpr int kWave = 64;
 
+// How the SRWM kernels treat the state tensors and the input (bits of `mode`):
+constexpr unsigned kModeShift = 1u;     // Wy..wb hold W minus the head's shared weights sWy..swb (in and out)
+constexpr unsigned kModeFresh = 2u;     // forward: start from the shared weights, the incoming Wy..wb are not read
+constexpr unsigned kModeSoftmaxX = 4u;  // x is given before its softmax over the last axis; grad_x refers to that input
+
 struct SrwmFwdParams {
     const float *x;
     int64_t xs_n, xs_h, xs_l;
@@ -20,6 +25,7 @@ struct SrwmFwdParams {
     const float *keep;
     const float *sWy, *sWq, *sWk, *swb;   // [H,E,Y], [H,E,E] x 2, [H,E,4]
     int Y;   // columns of W_y, out and ydiff (E for the plain operator)
+    unsigned mode;   // kMode* bits
 };
 
 struct SrwmBwdParams {
@@ -33,6 +39,8 @@ struct SrwmBwdParams {
     int N, H, L, E;
     unsigned grad_state_mode;  // SRWM_GRAD_STATE_*
     int Y;   // columns of W_y, grad_out, ydiff and gWy (E for the plain operator)
+    const float *sWy, *sWq, *sWk, *swb;   // shared weights, read when mode has kModeShift
+    unsigned mode;   // kMode* bits
 };
 
 struct Strided3 {
@@ -121,6 +129,8 @@ int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s);
 size_t replay_lds_bytes(int E, int M);
 int launch_replay(const ReplayParams &p, hipStream_t s);
 int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s);
+// dst[j][h, :] = sum over n of src[j][n, h, :] for the four state tensors (y: E x Y, q, k: E x E, b: E x 4)
+int launch_srwm_batch_sum(const float *const src[4], float *const dst[4], int N, int H, int E, int Y, hipStream_t s);
 int launch_delta_fwd_generic(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_bwd_generic(const DeltaBwdParams &p, hipStream_t s);
 

@@ -23,18 +23,38 @@ constexpr int kWaves = kThreads / kWave;
 
 __device__ __forceinline__ int padded_cols(int C) { return C | 1; }
 
+// W = tensors (sign = 0), W += tensors (sign = 1) or W -= tensors (sign = -1); every thread touches
+// the same elements in each call, so consecutive calls need no barrier between them
 __device__ __forceinline__ void load_state(float *W, int Cp, const float *Wy, const float *Wq,
-                                           const float *Wk, const float *wb, int E, int Y, int tid) {
+                                           const float *Wk, const float *wb, int E, int Y, int tid,
+                                           int sign = 0) {
+    const float keep = sign ? 1.f : 0.f, sc = sign < 0 ? -1.f : 1.f;
+    auto put = [&](int idx, float v) { W[idx] = sign ? fmaf(sc, v, keep * W[idx]) : v; };
     for (int i = tid; i < E * Y; i += kThreads) {
         const int e = i / Y, m = i - e * Y;
-        W[e * Cp + m] = Wy[i];
+        put(e * Cp + m, Wy[i]);
     }
     for (int i = tid; i < E * E; i += kThreads) {
         const int e = i / E, m = i - e * E;
-        W[e * Cp + Y + m] = Wq[i];
-        W[e * Cp + Y + E + m] = Wk[i];
+        put(e * Cp + Y + m, Wq[i]);
+        put(e * Cp + Y + E + m, Wk[i]);
     }
-    for (int i = tid; i < E * 4; i += kThreads) W[(i >> 2) * Cp + Y + 2 * E + (i & 3)] = wb[i];
+    for (int i = tid; i < E * 4; i += kThreads) put((i >> 2) * Cp + Y + 2 * E + (i & 3), wb[i]);
+}
+
+// softmax of the E floats at v, by one wave
+__device__ __forceinline__ void wave_softmax(float *v, int E, int lane) {
+    float mx = -INFINITY;
+    for (int i = lane; i < E; i += kWave) mx = fmaxf(mx, v[i]);
+    mx = wave_max(mx);
+    float s = 0.f;
+    for (int i = lane; i < E; i += kWave) {
+        const float ex = expf(v[i] - mx);
+        v[i] = ex;
+        s += ex;
+    }
+    s = wave_sum(s);
+    for (int i = lane; i < E; i += kWave) v[i] = v[i] / s;
 }
 
 // column of the packed state -> its block: 0 = y, 1 = q, 2 = k, 3 = b (also the index of its beta)
@@ -55,18 +75,28 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
     const int64_t sEE = seq * E * E, sEY = seq * E * Y, sE4 = seq * E * 4;
 
-    load_state(W, Cp, p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, E, Y, tid);
+    const float *shWy = p.sWy + (int64_t)h * E * Y, *shWq = p.sWq + (int64_t)h * E * E,
+                *shWk = p.sWk + (int64_t)h * E * E, *shwb = p.swb + (int64_t)h * E * 4;
+    if (p.mode & kModeFresh) {
+        load_state(W, Cp, shWy, shWq, shWk, shwb, E, Y, tid);
+    } else {
+        load_state(W, Cp, p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, E, Y, tid);
+        if (p.mode & kModeShift) load_state(W, Cp, shWy, shWq, shWk, shwb, E, Y, tid, 1);
+    }
     __syncthreads();
 
     for (int t = 0; t < p.L; ++t) {
         const float *xt = p.x + n * p.xs_n + h * p.xs_h + t * p.xs_l;
         const int64_t o = (seq * p.L + t) * E, oy = (seq * p.L + t) * Y, ob = (seq * p.L + t) * 4;
         if (p.keep && p.keep[(int64_t)n * p.L + t] == 0.f) {   // uniform: per-step reset to the shared weights
-            load_state(W, Cp, p.sWy + (int64_t)h * E * Y, p.sWq + (int64_t)h * E * E, p.sWk + (int64_t)h * E * E,
-                       p.swb + (int64_t)h * E * 4, E, Y, tid);
+            load_state(W, Cp, shWy, shWq, shWk, shwb, E, Y, tid);
         }
         for (int e = tid; e < E; e += kThreads) xs[e] = xt[e];
         __syncthreads();
+        if (p.mode & kModeSoftmaxX) {
+            if (wave == 0) wave_softmax(xs, E, lane);
+            __syncthreads();
+        }
         // main readout: pre = W^T x
         for (int m = tid; m < C; m += kThreads) {
             float a = 0.f;
@@ -115,6 +145,7 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
         __syncthreads();
     }
 
+    if (p.mode & kModeShift) load_state(W, Cp, shWy, shWq, shWk, shwb, E, Y, tid, -1);   // stored as a shift
     for (int i = tid; i < E * Y; i += kThreads) {
         const int e = i / Y, m = i - e * Y;
         p.Wy[sEY + i] = W[e * Cp + m];
@@ -151,6 +182,9 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
     const int64_t sEE = seq * E * E, sEY = seq * E * Y, sE4 = seq * E * 4;
 
     load_state(W, Cp, p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, E, Y, tid);
+    if (p.mode & kModeShift)
+        load_state(W, Cp, p.sWy + (int64_t)h * E * Y, p.sWq + (int64_t)h * E * E, p.sWk + (int64_t)h * E * E,
+                   p.swb + (int64_t)h * E * 4, E, Y, tid, 1);
     if (p.grad_state_mode == 0u) {
         for (int i = tid; i < E * Cp; i += kThreads) G[i] = 0.f;
     } else {
@@ -178,6 +212,10 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
             diff[ob4 + tid] = p.bdiff[ob + tid];
         }
         __syncthreads();
+        if (p.mode & kModeSoftmaxX) {
+            if (wave == 0) wave_softmax(xs, E, lane);
+            __syncthreads();
+        }
         // column pass: revert W, g_ins = G^T k
         for (int m = tid; m < C; m += kThreads) {
             const float b = bt[col_block(m, E, Y)];
@@ -226,12 +264,25 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
             }
         }
         __syncthreads();
-        // row pass: grad_x = W_{t-1} g_pre
+        // row pass: grad_x = W_{t-1} g_pre (gq is free again: it holds grad_x until the softmax of the input is undone)
+        const bool smx = p.mode & kModeSoftmaxX;
         for (int e = wave; e < E; e += kWaves) {
             float a = 0.f;
             for (int m = lane; m < C; m += kWave) a = fmaf(W[e * Cp + m], gpre[m], a);
             a = wave_sum(a);
-            if (lane == 0) p.gx[o + e] = a;
+            if (lane == 0) {
+                if (smx) gq[e] = a;
+                else p.gx[o + e] = a;
+            }
+        }
+        if (smx) {
+            __syncthreads();
+            if (wave == 0) {
+                float d = 0.f;
+                for (int i = lane; i < E; i += kWave) d = fmaf(gq[i], xs[i], d);
+                d = wave_sum(d);
+                for (int i = lane; i < E; i += kWave) p.gx[o + i] = xs[i] * (gq[i] - d);
+            }
         }
         // column pass: G += (q - k) (x) g_diff + x (x) g_pre
         for (int m = tid; m < C; m += kThreads) {

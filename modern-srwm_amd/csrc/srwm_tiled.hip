@@ -23,6 +23,8 @@
 // Replaces self_ref_forward_kernel / self_ref_backward_kernel of the reference
 // (supervised_learning/self_ref_v0/self_ref_v0.cu:24-432, :534-1234) and, with YB = 3, those of
 // reinforcement_learning/torchbeast/self_ref_v1/self_ref_v1.cu:27-534, :639-1547.
+#include <type_traits>
+
 #include "common.h"
 #include "xlane.h"
 
@@ -74,7 +76,19 @@ __device__ __forceinline__ void store_vec(float *dst, const float *src) {
     }
 }
 
-// RESET: the per-step reset to the shared weights is compiled in (p.keep != nullptr)
+// Softmax over a row of E floats that E/4 consecutive lanes hold as one float4 each.
+template <int E>
+__device__ __forceinline__ float4 row_softmax4(float4 v) {
+    const float m = group_max<E / 4>(fmaxf(fmaxf(v.x, v.y), fmaxf(v.z, v.w)));
+    v.x = exp_2ulp(v.x - m); v.y = exp_2ulp(v.y - m); v.z = exp_2ulp(v.z - m); v.w = exp_2ulp(v.w - m);
+    const float inv = fast_rcp(group_sum<E / 4>((v.x + v.y) + (v.z + v.w)));
+    v.x *= inv; v.y *= inv; v.z *= inv; v.w *= inv;
+    return v;
+}
+
+// RESET: the layer-level extras are compiled in -- the per-step reset to the shared weights
+// (p.keep), the state kept as a shift from them or started from them, the softmax of the input
+// (p.mode).  The plain operator runs the instantiation without them.
 template <int E, int NW, int R, bool RESET, int YB>
 __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams p) {
     using T = Tiling<E, NW, R>;
@@ -104,8 +118,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     const bool has_y = XC && jb == 0;        // thread holds row el of the last y column
 
     float w[R][NC];
-    float wbe, wye = 0.f;
-    auto load_state = [&](const float *Wy, const float *Wq, const float *Wk, const float *wb) {
+    float wbe = 0.f, wye = 0.f;
+    // state = tensors, or state += tensors when `add` is std::true_type
+    auto load_state = [&](const float *Wy, const float *Wq, const float *Wk, const float *wb, auto add) {
+        constexpr bool ADD = decltype(add)::value;
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const float *src = b < YB ? Wy + b * E : b == YB ? Wq : Wk;
@@ -113,17 +129,27 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
-                for (int c = 0; c < CB; ++c) w[i][b * CB + c] = src[(r0 + i) * ld + c0 + c];
+                for (int c = 0; c < CB; ++c) {
+                    const float v = src[(r0 + i) * ld + c0 + c];
+                    w[i][b * CB + c] = ADD ? w[i][b * CB + c] + v : v;
+                }
         }
-        wbe = has_b ? wb[el * 4 + jb] : 0.f;
-        if constexpr (XC) wye = has_y ? Wy[el * Y + YB * E] : 0.f;
+        if (has_b) wbe = ADD ? wbe + wb[el * 4 + jb] : wb[el * 4 + jb];
+        if constexpr (XC) {
+            if (has_y) wye = ADD ? wye + Wy[el * Y + YB * E] : Wy[el * Y + YB * E];
+        }
     };
-    load_state(p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4);
+    const float *shWy = p.sWy + (int64_t)h * E * Y, *shWq = p.sWq + (int64_t)h * E * E,
+                *shWk = p.sWk + (int64_t)h * E * E, *shwb = p.swb + (int64_t)h * E * 4;
+    if (RESET && (p.mode & kModeFresh)) {
+        load_state(shWy, shWq, shWk, shwb, std::false_type{});
+    } else {
+        load_state(p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, std::false_type{});
+        if (RESET && (p.mode & kModeShift)) load_state(shWy, shWq, shWk, shwb, std::true_type{});   // incoming state is a shift
+    }
     // replaces the state by the weights all batch rows of this head share (per-step reset)
-    auto reset_state = [&]() {
-        load_state(p.sWy + (int64_t)h * E * Y, p.sWq + (int64_t)h * E * E, p.sWk + (int64_t)h * E * E,
-                   p.swb + (int64_t)h * E * 4);
-    };
+    auto reset_state = [&]() { load_state(shWy, shWq, shWk, shwb, std::false_type{}); };
+    const bool softmax_x = RESET && (p.mode & kModeSoftmaxX);
     // rows of the Y-wide tensors start at any word: no vector stores there
     auto store_y = [&](float *dst, const float *v) {
         if constexpr (XC) {
@@ -143,10 +169,13 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         return *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col);
     };
     auto load_keep = [&](int tile) -> float {
-        return (RESET && tid < TT) ? p.keep[(int64_t)n * p.L + min(tile * TT + tid, p.L - 1)] : 1.f;
+        return (RESET && p.keep && tid < TT) ? p.keep[(int64_t)n * p.L + min(tile * TT + tid, p.L - 1)] : 1.f;
     };
     const int ntiles = (p.L + TT - 1) / TT;
-    *reinterpret_cast<float4 *>(&xt[0][ld_row][ld_col]) = load_tile(0);
+    {
+        const float4 x0 = load_tile(0);
+        *reinterpret_cast<float4 *>(&xt[0][ld_row][ld_col]) = softmax_x ? row_softmax4<E>(x0) : x0;
+    }
     if (RESET && tid < TT) kt[0][tid] = load_keep(0);
     __syncthreads();
 
@@ -191,7 +220,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
                 if (has_y && el == 0) p.out[oy + YB * E] = py;
             }
             if (tt == tlen - 1 && tile + 1 < ntiles) {
-                *reinterpret_cast<float4 *>(&xt[buf ^ 1][ld_row][ld_col]) = xnext;
+                *reinterpret_cast<float4 *>(&xt[buf ^ 1][ld_row][ld_col]) =
+                    softmax_x ? row_softmax4<E>(xnext) : xnext;
                 if (RESET && tid < TT) kt[buf ^ 1][tid] = knext;
             }
             __syncthreads();
@@ -257,18 +287,24 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         }
     }
 
+    // the final state, as the shift from the shared weights if that is how the caller keeps it
+    const bool as_shift = RESET && (p.mode & kModeShift);
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         float *dst = b < YB ? p.Wy + sEY + b * E : b == YB ? p.Wq + sEE : p.Wk + sEE;
+        const float *base = b < YB ? shWy + b * E : b == YB ? shWq : shWk;
         const int ld = b < YB ? Y : E;
 #pragma unroll
         for (int i = 0; i < R; ++i)
 #pragma unroll
-            for (int c = 0; c < CB; ++c) dst[(r0 + i) * ld + c0 + c] = w[i][b * CB + c];
+            for (int c = 0; c < CB; ++c) {
+                const int o = (r0 + i) * ld + c0 + c;
+                dst[o] = as_shift ? w[i][b * CB + c] - base[o] : w[i][b * CB + c];
+            }
     }
-    if (has_b) p.wb[sE4 + el * 4 + jb] = wbe;
+    if (has_b) p.wb[sE4 + el * 4 + jb] = as_shift ? wbe - shwb[el * 4 + jb] : wbe;
     if constexpr (XC) {
-        if (has_y) p.Wy[sEY + el * Y + YB * E] = wye;
+        if (has_y) p.Wy[sEY + el * Y + YB * E] = as_shift ? wye - shWy[el * Y + YB * E] : wye;
     }
 }
 
@@ -320,27 +356,36 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     const float *gobase = p.go + n * p.gs_n + h * p.gs_h;
     const bool has_y = XC && jb == 0;        // thread holds row el of the last y column
 
+    // the final state; given as its shift from the head's shared weights when the caller keeps it so
+    const bool as_shift = p.mode & kModeShift;
+    const float *shWy = p.sWy + (int64_t)h * E * Y, *shWq = p.sWq + (int64_t)h * E * E,
+                *shWk = p.sWk + (int64_t)h * E * E, *shwb = p.swb + (int64_t)h * E * 4;
     float w[R][NC], g[R][NC];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         const float *src = b < YB ? p.Wy + sEY + b * E : b == YB ? p.Wq + sEE : p.Wk + sEE;
+        const float *base = b < YB ? shWy + b * E : b == YB ? shWq : shWk;
         const float *gsrc = b < YB ? p.gWy + sEY + b * E : b == YB ? p.gWq + sEE : p.gWk + sEE;
         const int ld = b < YB ? Y : E;
 #pragma unroll
         for (int i = 0; i < R; ++i)
 #pragma unroll
             for (int c = 0; c < CB; ++c) {
-                w[i][b * CB + c] = src[(r0 + i) * ld + c0 + c];
-                g[i][b * CB + c] = p.grad_state_mode ? gsrc[(r0 + i) * ld + c0 + c] : 0.f;
+                const int o = (r0 + i) * ld + c0 + c;
+                w[i][b * CB + c] = as_shift ? src[o] + base[o] : src[o];
+                g[i][b * CB + c] = p.grad_state_mode ? gsrc[o] : 0.f;
             }
     }
     float wbe = has_b ? p.wb[sE4 + el * 4 + jb] : 0.f;
+    if (has_b && as_shift) wbe += shwb[el * 4 + jb];
     float gbe = (has_b && p.grad_state_mode) ? p.gwb[sE4 + el * 4 + jb] : 0.f;
     float wye = 0.f, gye = 0.f;
     if constexpr (XC) {
         wye = has_y ? p.Wy[sEY + el * Y + YB * E] : 0.f;
+        if (has_y && as_shift) wye += shWy[el * Y + YB * E];
         gye = (has_y && p.grad_state_mode) ? p.gWy[sEY + el * Y + YB * E] : 0.f;
     }
+    const bool softmax_x = p.mode & kModeSoftmaxX;
 
     const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
     // next tile, staged in registers
@@ -372,7 +417,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     } while (0)
 #define SRWM_BWD_STORE_TILE()                                                                      \
     do {                                                                                           \
-        *reinterpret_cast<float4 *>(&tl[VX][ld_row][ld_col]) = n_x;                                \
+        *reinterpret_cast<float4 *>(&tl[VX][ld_row][ld_col]) = softmax_x ? row_softmax4<E>(n_x) : n_x; \
         *reinterpret_cast<float4 *>(&tl[VQ][ld_row][ld_col]) = n_q;                                \
         *reinterpret_cast<float4 *>(&tl[VK][ld_row][ld_col]) = n_k;                                \
         *reinterpret_cast<float4 *>(&tl[VQD][ld_row][ld_col]) = n_qd;                              \
@@ -561,6 +606,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 for (int wv = 0; wv < NW; ++wv) s += rowm[2][wv][tid];
 #pragma unroll
                 for (int j = 0; j < NXS; ++j) s += rowb[2][j][tid];
+                if (softmax_x) {   // through the softmax of the input: sx (s - <s, sx>); tid < E covers whole lane groups
+                    const float sx = tl[VX][tt][tid];
+                    s = sx * (s - group_sum<E>(s * sx));
+                }
                 p.gx[o + tid] = s;
             }
 
@@ -617,7 +666,7 @@ int launch_bwd(const SrwmBwdParams &p, hipStream_t s) {
 
 template <int E, int NW, int R, int YB = 1>
 int launch_fwd(const SrwmFwdParams &p, hipStream_t s) {
-    if (p.keep)
+    if (p.keep || p.mode)
         hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, true, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
     else
         hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, false, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);

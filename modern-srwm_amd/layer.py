@@ -18,8 +18,14 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from fast_weight import fast_weight_delta, fast_weight_delta_steps
-from self_ref_v0 import self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
+from self_ref_v0 import self_ref_layer, self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
 from self_ref_v1 import self_ref_v1
+
+
+# True: the SRWM layers run the fused layer operator (shared weights read directly, input softmax,
+# carried shift and batch-summed weight gradients inside the kernels).  False: they spell the
+# reference's tensor operations out around the plain operator; both give the same results.
+FUSED_SRWM_LAYER = True
 
 
 def elu_p1(x):
@@ -80,6 +86,13 @@ class _SRBase(nn.Module):
         out = _heads_out(out, bsz, slen, self.num_head * self.dim_head)
         return self.drop(self.out_linear(out))
 
+    def _fused(self, h, softmax, shift):
+        """(operator output, new shift) from the layer input, everything inside the kernels."""
+        slen, bsz, _ = h.size()
+        x = h.reshape(slen, bsz, self.num_head, self.dim_head).permute(1, 2, 0, 3)
+        out, *new_shift = self_ref_layer(x, *self._slow(), *(shift if shift is not None else (None,) * 4), softmax)
+        return out, tuple(new_shift), slen, bsz
+
 
 class SRWMlayer(_SRBase):
     """Few-shot (supervised) SRWM layer."""
@@ -95,6 +108,12 @@ class SRWMlayer(_SRBase):
             del self.layer_norm
 
     def forward(self, h, state=None, get_state=False):
+        if FUSED_SRWM_LAYER:
+            out, shift, slen, bsz = self._fused(h, self.use_input_softmax, state)
+            if not self.stateful:   # the plain operator's state carries no gradient (layer.py:179-182 of the reference)
+                shift = tuple(s.detach() for s in shift)
+            out = (self.layer_norm(h) if self.use_ln else h) + self._project(out, bsz, slen)
+            return (out, shift) if get_state else out
         x, slen, bsz = self._split(h, self.use_input_softmax)
         fast = self._fast(bsz, state)
         if self.stateful:
@@ -118,6 +137,9 @@ class SRlayer(_SRBase):
 
     def forward(self, h, state=None):
         assert state is not None
+        if FUSED_SRWM_LAYER:
+            out, shift, slen, bsz = self._fused(h, True, tuple(s.detach() for s in state))
+            return h + self._project(out, bsz, slen), tuple(s.detach() for s in shift)
         x, slen, bsz = self._split(h, True)
         fast = self._fast(bsz, state)
         out = self.fw_layer(x, *fast)
@@ -149,6 +171,9 @@ class NoCarryOverSRlayer(_SRBase):
         self.fw_layer = self_ref_v0
 
     def forward(self, h, state=None):
+        if FUSED_SRWM_LAYER:
+            out, _, slen, bsz = self._fused(h, True, None)
+            return h + self._project(out, bsz, slen), state
         x, slen, bsz = self._split(h, True)
         out = self.fw_layer(x, *self._fast(bsz))
         return h + self._project(out, bsz, slen), state

@@ -147,3 +147,81 @@ class SelfRefv0Steps(torch.autograd.Function):
 
 
 self_ref_v0_steps = SelfRefv0Steps.apply
+
+
+class SelfRefLayerFn(torch.autograd.Function):
+    """The SRWM operator as the layers call it, with `state + W.repeat(bsz, 1, 1, 1)`, the softmax
+    of the input, the final `- W.repeat(...)` and the batch sum of the weight gradients done inside
+    the kernels (supervised_learning/layer.py:156-195, reinforcement_learning/torchbeast/
+    layer.py:377-421 spell them out as separate tensor operations).
+
+        out, dW_y, dW_q, dW_k, dw_b = self_ref_layer(x, sW_y, sW_q, sW_k, sw_b,
+                                                     shift_y, shift_q, shift_k, shift_b, softmax_input)
+
+    x: (N, H, L, E), any strides (a permuted view of the layer input is fine), before its softmax
+    when `softmax_input`; sW_*: the shared weights (1, H, E, .); shift_*: (N, H, E, .) carried
+    shift from the shared weights, or all None to start from them.  Returns the output and the NEW
+    shift (freshly allocated; the inputs are not modified).  Gradients: x, the shared weights
+    (through the initial state and, if the returned shift is used in the loss, through it), the
+    incoming shift.
+    """
+
+    @staticmethod
+    def forward(ctx, x, sW_y, sW_q, sW_k, sw_b, shift_y, shift_q, shift_k, shift_b, softmax_input):
+        N, H, L, E = x.shape
+        Y = sW_y.shape[-1]
+        dev = x.device
+        shifts = (shift_y, shift_q, shift_k, shift_b)
+        fresh = shift_y is None
+        assert all((s is None) == fresh for s in shifts), "give all four shifts or none"
+        widths = (Y, E, E, 4)
+        if fresh:
+            state = [torch.empty((N, H, E, w), device=dev, dtype=x.dtype) for w in widths]
+        else:
+            state = [s.detach().clone(memory_format=torch.contiguous_format) for s in shifts]
+        big = lambda: torch.empty((N, H, L, E), device=dev, dtype=x.dtype)
+        wide = lambda: torch.empty((N, H, L, Y), device=dev, dtype=x.dtype)
+        small = lambda: torch.empty((N, H, L, 4), device=dev, dtype=x.dtype)
+        out = wide()
+        saved = [big(), big(), small(), wide(), big(), big(), small()]
+        flags = srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_FRESH_STATE if fresh else 0) | \
+            (srwm_hip.FLAG_SOFTMAX_INPUT if softmax_input else 0)
+        slow = (sW_y, sW_q, sW_k, sw_b)
+        srwm_hip.self_ref_layer_forward(x.detach(), None, slow, *state, *saved, out, flags=flags)
+        ctx.save_for_backward(x, *saved, *slow, *state)
+        ctx.softmax_input = softmax_input
+        ctx.fresh = fresh
+        return (out, *state)
+
+    @staticmethod
+    def backward(ctx, grad_out, g_y, g_q, g_k, g_b):
+        x, *rest = ctx.saved_tensors
+        saved, slow, state = rest[:7], rest[7:11], rest[11:15]
+        N, H, L, E = x.shape
+        Y = slow[0].shape[-1]
+        g_state = (g_y, g_q, g_k, g_b)
+        has_gs = any(g is not None for g in g_state)
+        if has_gs:   # the loss also depends on the returned shift: private contiguous copies, zeros where unused
+            grad_W = [torch.zeros_like(s) if g is None else g.clone(memory_format=torch.contiguous_format)
+                      for g, s in zip(g_state, state)]
+            mode = srwm_hip.GRAD_STATE_IN
+        else:
+            grad_W = [torch.empty_like(s) for s in state]
+            mode = srwm_hip.GRAD_STATE_ZERO
+        need_slow = any(ctx.needs_input_grad[1:5])
+        grad_slow = [torch.empty((H, E, w), device=x.device, dtype=x.dtype) for w in (Y, E, E, 4)] \
+            if need_slow else None
+        # d(shift_out)/d(shared) = dW_L/d(shared) - 1: the incoming state gradient is taken off again
+        minus = [g.sum(0) for g in grad_W] if (has_gs and need_slow) else None
+        grad_x = torch.empty(x.shape, device=x.device, dtype=x.dtype)
+        flags = mode | srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_SOFTMAX_INPUT if ctx.softmax_input else 0)
+        srwm_hip.self_ref_layer_backward(x, *saved, grad_out, slow, *state, grad_x, grad_W, grad_slow, flags=flags)
+        gs = [None] * 4
+        if need_slow:
+            gs = [(g - m if minus is not None else g).reshape(s.shape) for g, m, s in
+                  zip(grad_slow, minus or [None] * 4, slow)]
+        gshift = [None] * 4 if ctx.fresh else grad_W
+        return (grad_x, *gs, *gshift, None)
+
+
+self_ref_layer = SelfRefLayerFn.apply

@@ -30,8 +30,11 @@ GRAD_STATE_IN = 1
 GRAD_STATE_ACCUM = 2
 FLAG_GENERIC = 16
 FLAG_CHUNKWISE = 32     # delta forward: chunkwise MFMA kernel (E == M in {64, 128})
+FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus the shared weights
+FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
+FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 
@@ -44,6 +47,8 @@ _SIGNATURES = {
     "srwm_forward_f32": [_F, _S] + [_F] * 12 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_forward_wide_f32": [_F, _S] + [_F] * 12 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_backward_wide_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_forward_f32": [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
@@ -301,6 +306,100 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
                                                 *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
                                                 N, H, L, E, Y, flags, _stream(x.device))
     _check(code, name)
+
+
+def _shared(slow, H, E, Y):
+    """The layer's parameters as dense (H, E, .) tensors; a leading batch axis of 1 is dropped."""
+    shapes = ((H, E, Y), (H, E, E), (H, E, E), (H, E, 4))
+    out = []
+    for t, shp, nm in zip(slow, shapes, ("shared W_y", "shared W_q", "shared W_k", "shared w_b")):
+        _require(t, nm)
+        if t.dim() == 4 and t.shape[0] == 1:
+            t = t[0]
+        _require(t, nm, shp)
+        out.append(t.detach().contiguous())
+    return out
+
+
+def self_ref_layer_forward(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff,
+                           beta_diff, out, flags=0):
+    """SRWM forward with the layers' prologue and epilogue inside the kernel: `slow` = the shared
+    weights (W_y: (1, H, E, Y) or (H, E, Y), ...), read without a repeat(); flags FLAG_FRESH_STATE
+    (start from them, W_* are outputs), FLAG_STATE_SHIFT (W_* hold the state minus the shared
+    weights, in and out), FLAG_SOFTMAX_INPUT (x is soft-maxed by the kernel); keep as in
+    self_ref_forward_steps."""
+    _require(x, "x")
+    N, H, L, E = x.shape
+    _require(W_y, "W_y")
+    Y = W_y.shape[-1]
+    _require(W_y, "W_y", (N, H, E, Y))
+    for t, nm in ((W_q, "W_q"), (W_k, "W_k")):
+        _require(t, nm, (N, H, E, E))
+    _require(w_b, "w_b", (N, H, E, 4))
+    for t, nm in ((q, "q"), (k, "k"), (q_diff, "q_diff"), (k_diff, "k_diff")):
+        _require(t, nm, (N, H, L, E))
+    for t, nm in ((y_diff, "y_diff"), (out, "out")):
+        _require(t, nm, (N, H, L, Y))
+    _require(beta, "beta", (N, H, L, 4))
+    _require(beta_diff, "beta_diff", (N, H, L, 4))
+    sl = _shared(slow, H, E, Y)
+    null = ctypes.c_void_p(None)
+    if keep is not None:
+        _require(keep, "keep", (N, L))
+        keep = keep.contiguous()
+    if x.numel() == 0:
+        return
+    xs, xstr = _strided(x)
+    with torch.cuda.device(x.device), \
+            _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out], True) as d:
+        code = lib().srwm_layer_forward_f32(
+            _ptr(xs), xstr, _ptr(keep) if keep is not None else null, *[_ptr(t) for t in sl],
+            *[_ptr(t) for t in d], N, H, L, E, Y, flags, _stream(x.device))
+    _check(code, "srwm_layer_forward_f32")
+
+
+def self_ref_layer_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out, slow,
+                            W_y, W_q, W_k, w_b, grad_x, grad_W, grad_slow, flags=GRAD_STATE_ZERO):
+    """Backward of self_ref_layer_forward (without resets).  W_*: the final state as the forward
+    left it; grad_W: four (N, H, E, .) tensors (SRWM_GRAD_STATE_* semantics, per batch row);
+    grad_slow: four (H, E, .) tensors receiving the sum of grad_W over the batch, or None."""
+    _require(x, "x")
+    N, H, L, E = x.shape
+    _require(W_y, "W_y")
+    Y = W_y.shape[-1]
+    for t, nm in ((q, "q"), (k, "k"), (q_diff, "q_diff"), (k_diff, "k_diff"), (grad_x, "grad_x")):
+        _require(t, nm, (N, H, L, E))
+    for t, nm in ((y_diff, "y_diff"), (grad_out, "grad_out")):
+        _require(t, nm, (N, H, L, Y))
+    _require(beta, "beta", (N, H, L, 4))
+    _require(beta_diff, "beta_diff", (N, H, L, 4))
+    shapes = ((N, H, E, Y), (N, H, E, E), (N, H, E, E), (N, H, E, 4))
+    for t, g, shp in zip((W_y, W_q, W_k, w_b), grad_W, shapes):
+        _require(t, "state", shp)
+        _require(g, "grad_W", shp)
+        if not g.is_contiguous():
+            raise ValueError("grad_W tensors must be contiguous")
+    sl = _shared(slow, H, E, Y)
+    null = ctypes.c_void_p(None)
+    gsl = [null] * 4
+    if grad_slow is not None:
+        for g, shp in zip(grad_slow, ((H, E, Y), (H, E, E), (H, E, E), (H, E, 4))):
+            _require(g, "grad_slow", shp)
+            if not g.is_contiguous():
+                raise ValueError("grad_slow tensors must be contiguous")
+        gsl = [_ptr(g) for g in grad_slow]
+    if x.numel() == 0:
+        return
+    xs, xstr = _strided(x)
+    gos, gstr = _strided(grad_out)
+    with torch.cuda.device(x.device), \
+            _Dense([q, k, beta, y_diff, q_diff, k_diff, beta_diff], False) as sv, \
+            _Dense([W_y, W_q, W_k, w_b], False) as st, _Dense([grad_x], True) as gx:
+        code = lib().srwm_layer_backward_f32(
+            _ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr, *[_ptr(t) for t in sl],
+            *[_ptr(t) for t in st], _ptr(gx[0]), *[_ptr(g) for g in grad_W], *gsl,
+            N, H, L, E, Y, flags, _stream(x.device))
+    _check(code, "srwm_layer_backward_f32")
 
 
 # names of the extension functions of the reference's wide-output variant

@@ -17,6 +17,17 @@ def _dev():
     return torch.device("cuda:0")
 
 
+@pytest.fixture(params=[True, False], ids=["fused", "spelled-out"])
+def srwm_layer_path(request):
+    """Runs a test once with the fused layer operator and once with the reference's tensor
+    operations around the plain operator."""
+    import layer
+    old = layer.FUSED_SRWM_LAYER
+    layer.FUSED_SRWM_LAYER = request.param
+    yield request.param
+    layer.FUSED_SRWM_LAYER = old
+
+
 def _ref_sr(layer, h, softmax, shift=None, use_ln_residual=None):
     """fp64 CPU statement of an SRWM layer's forward; returns (out, final fast weights)."""
     slen, bsz, _ = h.shape
@@ -42,7 +53,7 @@ def _pair(layer):
     return gpu, cpu
 
 
-def test_srwm_layer_supervised():
+def test_srwm_layer_supervised(srwm_layer_path):
     print("case SRWMlayer", flush=True)
     from layer import SRWMlayer
     torch.manual_seed(0)
@@ -67,7 +78,7 @@ def test_srwm_layer_supervised():
         assert err < 1e-5 * f.abs().max().item()
 
 
-def test_srwm_layer_stateful_with_loss_on_state():
+def test_srwm_layer_stateful_with_loss_on_state(srwm_layer_path):
     print("case SRWMlayer stateful", flush=True)
     from layer import SRWMlayer
     torch.manual_seed(1)
@@ -90,7 +101,7 @@ def test_srwm_layer_stateful_with_loss_on_state():
         assert rel_err(getattr(gpu, n).grad.cpu().numpy(), getattr(cpu, n).grad.numpy()) < 2e-4, n
 
 
-def test_rl_sr_layers_carry_and_restart():
+def test_rl_sr_layers_carry_and_restart(srwm_layer_path):
     print("case SRlayer / NoCarryOverSRlayer", flush=True)
     from layer import NoCarryOverSRlayer, SRlayer
     torch.manual_seed(2)

@@ -354,3 +354,57 @@ def test_wide_rejects_a_state_that_does_not_fit():
     small = lambda: torch.empty((N, H, L, 4), device=dev)
     with pytest.raises(RuntimeError, match="LDS"):
         srwm_hip.self_ref_forward_v1(x, *W, big(), big(), small(), wide(), big(), big(), small(), wide())
+
+
+# ---------------------------------------------------------------- fused layer operator
+
+@pytest.mark.parametrize("shape,Y,generic", [
+    ((3, 4, 20, 32), 32, False),
+    ((2, 16, 70, 64), 64, False),      # headline head size
+    ((3, 4, 20, 32), 97, False),       # wide output block
+    ((2, 3, 9, 12), 12, True),         # LDS-resident kernels (no register tiling for E = 12)
+    ((2, 2, 6, 8), 11, True),
+])
+@pytest.mark.parametrize("with_shift", [False, True], ids=["fresh", "shift"])
+def test_fused_layer_operator_matches_fp64_autograd(shape, Y, generic, with_shift):
+    """self_ref_layer: raw input soft-maxed in the kernel, shared weights read directly, state kept
+    as a shift, weight gradients summed over the batch; the loss also uses the returned shift."""
+    print(f"case fused layer op shape={shape} Y={Y} shift={with_shift}", flush=True)
+    from oracle.recurrence import srwm_recurrence
+    from self_ref_v0 import self_ref_layer
+    N, H, L, E = shape
+    g = torch.Generator().manual_seed(17)
+    std = 1.0 / math.sqrt(E)
+    xr = torch.randn(N, H, L, E, generator=g, dtype=torch.float64)
+    slow = [torch.randn(1, H, E, w, generator=g, dtype=torch.float64) * std for w in (Y, E, E, 4)]
+    shift = [torch.randn(N, H, E, w, generator=g, dtype=torch.float64) * 0.1 for w in (Y, E, E, 4)]
+    go = torch.randn(N, H, L, Y, generator=g, dtype=torch.float64)
+    # weight of the returned shift in the loss; kept small because the gradient of the shared weights is
+    # sum_n (dL/dW_0[n] - gs[n]), a difference of nearly equal fp32 numbers when gs dominates
+    gs = [torch.randn(N, H, E, w, generator=g, dtype=torch.float64) * 0.03 for w in (Y, E, E, 4)]
+    dev = _dev()
+    # GPU
+    x_lnhe = xr.permute(2, 0, 1, 3).contiguous().to(dev, torch.float32).requires_grad_(True)   # layer storage order
+    slow_d = [w.to(dev, torch.float32).requires_grad_(True) for w in slow]
+    shift_d = [s.to(dev, torch.float32).requires_grad_(True) for s in shift] if with_shift else [None] * 4
+    out, *new = self_ref_layer(x_lnhe.permute(1, 2, 0, 3), *slow_d, *shift_d, True)
+    loss = (out * go.to(dev, torch.float32)).sum() + sum((n * s.to(dev, torch.float32)).sum() for n, s in zip(new, gs))
+    loss.backward()
+    # fp64 statement with the tensor operations spelled out
+    xc = xr.clone().requires_grad_(True)
+    slow_c = [w.clone().requires_grad_(True) for w in slow]
+    shift_c = [s.clone().requires_grad_(True) for s in shift]
+    fast = [w.repeat(N, 1, 1, 1) + (s if with_shift else 0.0) for w, s in zip(slow_c, shift_c)]
+    out_c, final = srwm_recurrence(torch.softmax(xc, -1), *fast)
+    new_c = [f - w.repeat(N, 1, 1, 1) for f, w in zip(final, slow_c)]
+    ((out_c * go).sum() + sum((n * s).sum() for n, s in zip(new_c, gs))).backward()
+    assert rel_err(out.detach().cpu().numpy(), out_c.detach().numpy()) < TOL
+    for a, b in zip(new, new_c):
+        assert (a.detach().cpu().double() - b.detach()).abs().max().item() < TOL * max(1.0, b.abs().max().item())
+    assert rel_err(x_lnhe.grad.permute(1, 2, 0, 3).cpu().numpy(), xc.grad.numpy()) < TOL
+    for a, b, s_ in zip(slow_d, slow_c, gs):   # error measured against the larger of the two terms of that difference
+        scale = max(b.grad.abs().max().item(), s_.sum(0).abs().max().item())
+        assert (a.grad.cpu().double() - b.grad).abs().max().item() < TOL * scale
+    if with_shift:
+        for a, b in zip(shift_d, shift_c):
+            assert rel_err(a.grad.cpu().numpy(), b.grad.numpy()) < TOL
