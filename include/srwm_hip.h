@@ -99,6 +99,30 @@ SRWM_API int srwm_backward_f32(const float *x, const int64_t x_strides[3],
                       int N, int H, int L, int E, unsigned flags, void *stream);
 
 /*
+ * SRWM with bf16 input and output, fp32 state.  No counterpart in the reference (its kernels are
+ * float-only, self_ref_v0.cu:14): same recurrence as srwm_forward_f32 / srwm_backward_f32 with
+ *   x, out, grad_out                                       bf16 (raw 16-bit patterns; strides in bf16 elements)
+ *   the state, q, k, beta, the diffs, grad_x and the state gradients   fp32
+ * All arithmetic and the state are fp32; `out` is rounded to nearest even; grad_x comes back in
+ * fp32 (the caller rounds it if it wants bf16).
+ */
+SRWM_API int srwm_forward_bf16(const uint16_t *x, const int64_t x_strides[3],
+                      float *Wy, float *Wq, float *Wk, float *wb,
+                      float *q, float *k, float *beta,
+                      float *ydiff, float *qdiff, float *kdiff, float *bdiff,
+                      uint16_t *out,
+                      int N, int H, int L, int E, unsigned flags, void *stream);
+
+SRWM_API int srwm_backward_bf16(const uint16_t *x, const int64_t x_strides[3],
+                       const float *q, const float *k, const float *beta,
+                       const float *ydiff, const float *qdiff, const float *kdiff,
+                       const float *bdiff,
+                       const uint16_t *grad_out, const int64_t grad_out_strides[3],
+                       const float *Wy, const float *Wq, const float *Wk, const float *wb,
+                       float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb,
+                       int N, int H, int L, int E, unsigned flags, void *stream);
+
+/*
  * SRWM forward / backward with an output block Y columns wide.  Replace self_ref_forward_v1() and
  * self_ref_backward_v1(), reinforcement_learning/torchbeast/self_ref_v1/self_ref_v1.cu:538-635
  * (kernel :27-534) and :1551-1656 (kernel :639-1547), where Y = 3E+1: the readout supplies the

@@ -125,6 +125,54 @@ int srwm_layer_forward_f32(const float *x, const int64_t xs[3], const float *kee
     return launch_srwm_fwd_generic(p, s);
 }
 
+int srwm_forward_bf16(const uint16_t *x, const int64_t xs[3], float *Wy, float *Wq, float *Wk, float *wb,
+                      float *q, float *k, float *beta, float *ydiff, float *qdiff, float *kdiff,
+                      float *bdiff, uint16_t *out, int N, int H, int L, int E, unsigned flags,
+                      void *stream) {
+    if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
+        !out || !xs)
+        return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || (flags & ~(SRWM_FLAG_GENERIC))) return SRWM_EINVAL;
+    if (!stride_ok(xs, N, H, L, E)) return SRWM_ESTRIDE;
+    SrwmFwdParams p{reinterpret_cast<const float *>(x), xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta,
+                    ydiff, qdiff, kdiff, bdiff, reinterpret_cast<float *>(out), N, H, L, E};
+    p.Y = E;
+    p.mode = kModeBf16;
+    hipStream_t s = (hipStream_t)stream;
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_srwm_fwd_tiled(p, s);
+        if (r >= 0) return r;
+    }
+    if (srwm_fwd_generic_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
+    return launch_srwm_fwd_generic(p, s);
+}
+
+int srwm_backward_bf16(const uint16_t *x, const int64_t xs[3], const float *q, const float *k,
+                       const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
+                       const float *bdiff, const uint16_t *grad_out, const int64_t gs[3], const float *Wy,
+                       const float *Wq, const float *Wk, const float *wb, float *grad_x, float *gWy,
+                       float *gWq, float *gWk, float *gwb, int N, int H, int L, int E, unsigned flags,
+                       void *stream) {
+    if (!x || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff || !grad_out || !Wy || !Wq ||
+        !Wk || !wb || !grad_x || !gWy || !gWq || !gWk || !gwb || !xs || !gs)
+        return SRWM_EINVAL;
+    const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
+    if (!dims_ok(N, H, L, E) || mode == 3u || (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)))
+        return SRWM_EINVAL;
+    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, E)) return SRWM_ESTRIDE;
+    SrwmBwdParams p{reinterpret_cast<const float *>(x), xs[0], xs[1], xs[2], q, k, beta, ydiff, qdiff, kdiff,
+                    bdiff, reinterpret_cast<const float *>(grad_out), gs[0], gs[1], gs[2], Wy, Wq, Wk, wb,
+                    grad_x, gWy, gWq, gWk, gwb, N, H, L, E, mode, E};
+    p.mode = kModeBf16;
+    hipStream_t s = (hipStream_t)stream;
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_srwm_bwd_tiled(p, s);
+        if (r >= 0) return r;
+    }
+    if (srwm_bwd_generic_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
+    return launch_srwm_bwd_generic(p, s);
+}
+
 int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
                            const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
                            float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,

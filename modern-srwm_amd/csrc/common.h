@@ -13,6 +13,8 @@ constexpr int kWave = 64;
 constexpr unsigned kModeShift = 1u;     // Wy..wb hold W minus the head's shared weights sWy..swb (in and out)
 constexpr unsigned kModeFresh = 2u;     // forward: start from the shared weights, the incoming Wy..wb are not read
 constexpr unsigned kModeSoftmaxX = 4u;  // x is given before its softmax over the last axis; grad_x refers to that input
+constexpr unsigned kModeBf16 = 8u;      // x, out (forward) and x, grad_out (backward) are bf16 behind the float pointers;
+                                        // their strides count bf16 elements; everything else stays fp32
 
 struct SrwmFwdParams {
     const float *x;
@@ -106,6 +108,17 @@ struct DeltaBwdParamsBf16 {
     int N, H, L, E, M;
     unsigned grad_state_mode;
 };
+
+// ---- bf16 <-> fp32 (16-bit patterns; round to nearest even on the way down)
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ float4 bf16x4_to_f32(uint2 u) {
+    return make_float4(bf16_bits_to_f32(u.x & 0xFFFFu), bf16_bits_to_f32(u.x >> 16), bf16_bits_to_f32(u.y & 0xFFFFu),
+                       bf16_bits_to_f32(u.y >> 16));
+}
 
 // ---- wave64 all-reduce helpers (every lane receives the result) -----------------
 __device__ __forceinline__ float wave_sum(float v) {

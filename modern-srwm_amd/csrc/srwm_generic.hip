@@ -85,13 +85,15 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
     }
     __syncthreads();
 
+    const bool bf16_io = p.mode & kModeBf16;
     for (int t = 0; t < p.L; ++t) {
         const float *xt = p.x + n * p.xs_n + h * p.xs_h + t * p.xs_l;
+        const uint16_t *xt16 = reinterpret_cast<const uint16_t *>(p.x) + n * p.xs_n + h * p.xs_h + t * p.xs_l;
         const int64_t o = (seq * p.L + t) * E, oy = (seq * p.L + t) * Y, ob = (seq * p.L + t) * 4;
         if (p.keep && p.keep[(int64_t)n * p.L + t] == 0.f) {   // uniform: per-step reset to the shared weights
             load_state(W, Cp, shWy, shWq, shWk, shwb, E, Y, tid);
         }
-        for (int e = tid; e < E; e += kThreads) xs[e] = xt[e];
+        for (int e = tid; e < E; e += kThreads) xs[e] = bf16_io ? bf16_bits_to_f32(xt16[e]) : xt[e];
         __syncthreads();
         if (p.mode & kModeSoftmaxX) {
             if (wave == 0) wave_softmax(xs, E, lane);
@@ -102,7 +104,10 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
             float a = 0.f;
             for (int e = 0; e < E; ++e) a = fmaf(W[e * Cp + m], xs[e], a);
             pre[m] = a;
-            if (m < Y) p.out[oy + m] = a;
+            if (m < Y) {
+                if (bf16_io) reinterpret_cast<uint16_t *>(p.out)[oy + m] = f32_to_bf16_bits(a);
+                else p.out[oy + m] = a;
+            }
         }
         __syncthreads();
         // activations: wave 0 -> softmax(q~), wave 1 -> softmax(k~), wave 2 -> sigmoid(b~)
@@ -192,12 +197,15 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
     }
     __syncthreads();
 
+    const bool bf16_io = p.mode & kModeBf16;
     for (int t = p.L - 1; t >= 0; --t) {
         const float *xt = p.x + n * p.xs_n + h * p.xs_h + t * p.xs_l;
         const float *got = p.go + n * p.gs_n + h * p.gs_h + t * p.gs_l;
+        const uint16_t *xt16 = reinterpret_cast<const uint16_t *>(p.x) + n * p.xs_n + h * p.xs_h + t * p.xs_l;
+        const uint16_t *got16 = reinterpret_cast<const uint16_t *>(p.go) + n * p.gs_n + h * p.gs_h + t * p.gs_l;
         const int64_t o = (seq * p.L + t) * E, oy = (seq * p.L + t) * Y, ob = (seq * p.L + t) * 4;
         for (int e = tid; e < E; e += kThreads) {
-            xs[e] = xt[e];
+            xs[e] = bf16_io ? bf16_bits_to_f32(xt16[e]) : xt[e];
             qs[e] = p.q[o + e];
             ks[e] = p.k[o + e];
             diff[oq + e] = p.qdiff[o + e];
@@ -205,7 +213,7 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
         }
         for (int m = tid; m < Y; m += kThreads) {
             diff[m] = p.ydiff[oy + m];
-            gpre[m] = got[m];
+            gpre[m] = bf16_io ? bf16_bits_to_f32(got16[m]) : got[m];
         }
         if (tid < 4) {
             bt[tid] = p.beta[ob + tid];

@@ -150,6 +150,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     // replaces the state by the weights all batch rows of this head share (per-step reset)
     auto reset_state = [&]() { load_state(shWy, shWq, shWk, shwb, std::false_type{}); };
     const bool softmax_x = RESET && (p.mode & kModeSoftmaxX);
+    const bool bf16_io = RESET && (p.mode & kModeBf16);
     // rows of the Y-wide tensors start at any word: no vector stores there
     auto store_y = [&](float *dst, const float *v) {
         if constexpr (XC) {
@@ -164,8 +165,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 
     // tile loader: thread -> (step tid / (E/4), 4 consecutive elements)
     const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
+    const uint16_t *xbase16 = reinterpret_cast<const uint16_t *>(p.x) + n * p.xs_n + h * p.xs_h;
     auto load_tile = [&](int tile) -> float4 {
         const int t = min(tile * TT + ld_row, p.L - 1);  // rows past the end: loaded, never used
+        if (bf16_io) return bf16x4_to_f32(*reinterpret_cast<const uint2 *>(xbase16 + t * p.xs_l + ld_col));
         return *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col);
     };
     auto load_keep = [&](int tile) -> float {
@@ -210,14 +213,25 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             group_sum_n<RG, NC>(acc);
             const float pb = group_sum<E>(wbe * xb);
             if (rg == 0) {
-                store_y(p.out + oy, &acc[0]);
+                if (bf16_io) {
+                    uint16_t *o16 = reinterpret_cast<uint16_t *>(p.out) + oy;
+#pragma unroll
+                    for (int b = 0; b < YB; ++b)
+#pragma unroll
+                        for (int c = 0; c < CB; ++c) o16[b * E + c0 + c] = f32_to_bf16_bits(acc[b * CB + c]);
+                } else {
+                    store_y(p.out + oy, &acc[0]);
+                }
                 store_vec<CB>(&raw[par][0][c0], &acc[QB]);
                 store_vec<CB>(&raw[par][1][c0], &acc[KB]);
             }
             if (has_b && el == 0) rawb[par][jb] = pb;
             if constexpr (XC) {
                 const float py = group_sum<E>(wye * xb);
-                if (has_y && el == 0) p.out[oy + YB * E] = py;
+                if (has_y && el == 0) {
+                    if (bf16_io) reinterpret_cast<uint16_t *>(p.out)[oy + YB * E] = f32_to_bf16_bits(py);
+                    else p.out[oy + YB * E] = py;
+                }
             }
             if (tt == tlen - 1 && tile + 1 < ntiles) {
                 *reinterpret_cast<float4 *>(&xt[buf ^ 1][ld_row][ld_col]) =
@@ -386,6 +400,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
         gye = (has_y && p.grad_state_mode) ? p.gWy[sEY + el * Y + YB * E] : 0.f;
     }
     const bool softmax_x = p.mode & kModeSoftmaxX;
+    const bool bf16_io = p.mode & kModeBf16;
+    const uint16_t *xbase16 = reinterpret_cast<const uint16_t *>(p.x) + n * p.xs_n + h * p.xs_h;
+    const uint16_t *gobase16 = reinterpret_cast<const uint16_t *>(p.go) + n * p.gs_n + h * p.gs_h;
 
     const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
     // next tile, staged in registers
@@ -395,7 +412,13 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     do { /* rows past the end of the sequence are clamped: they are loaded but never used */       \
         const int t_ = min((tile_) * TT + ld_row, p.L - 1);                                        \
         const int64_t o_ = (seq * p.L + t_) * E + ld_col;                                          \
-        n_x = *reinterpret_cast<const float4 *>(xbase + t_ * p.xs_l + ld_col);                     \
+        if (bf16_io) { /* raw bits: widened when the tile is committed, so the fetch is not waited for */ \
+            const uint2 u_ = *reinterpret_cast<const uint2 *>(xbase16 + t_ * p.xs_l + ld_col);     \
+            n_x.x = __uint_as_float(u_.x);                                                         \
+            n_x.y = __uint_as_float(u_.y);                                                         \
+        } else {                                                                                   \
+            n_x = *reinterpret_cast<const float4 *>(xbase + t_ * p.xs_l + ld_col);                 \
+        }                                                                                          \
         n_q = *reinterpret_cast<const float4 *>(p.q + o_);                                         \
         n_k = *reinterpret_cast<const float4 *>(p.k + o_);                                         \
         n_qd = *reinterpret_cast<const float4 *>(p.qdiff + o_);                                    \
@@ -405,10 +428,17 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 const int f_ = min(tid + i_ * NT, TT * Y - 1), r_ = f_ / Y, m_ = f_ - r_ * Y;      \
                 const int64_t tw_ = min((tile_) * TT + r_, p.L - 1);                               \
                 n_ydw[i_] = p.ydiff[(seq * p.L + tw_) * Y + m_];                                   \
-                n_gow[i_] = gobase[tw_ * p.gs_l + m_];                                             \
+                n_gow[i_] = bf16_io ? __uint_as_float((uint32_t)gobase16[tw_ * p.gs_l + m_])       \
+                                    : gobase[tw_ * p.gs_l + m_];                                   \
             }                                                                                      \
         } else {                                                                                   \
-            n_go = *reinterpret_cast<const float4 *>(gobase + t_ * p.gs_l + ld_col);               \
+            if (bf16_io) {                                                                         \
+                const uint2 u_ = *reinterpret_cast<const uint2 *>(gobase16 + t_ * p.gs_l + ld_col); \
+                n_go.x = __uint_as_float(u_.x);                                                    \
+                n_go.y = __uint_as_float(u_.y);                                                    \
+            } else {                                                                               \
+                n_go = *reinterpret_cast<const float4 *>(gobase + t_ * p.gs_l + ld_col);           \
+            }                                                                                      \
             n_yd = *reinterpret_cast<const float4 *>(p.ydiff + o_);                                \
         }                                                                                          \
         const int64_t ob_ = (seq * p.L + min((tile_) * TT + (tid % TT), p.L - 1)) * 4;             \
@@ -417,6 +447,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     } while (0)
 #define SRWM_BWD_STORE_TILE()                                                                      \
     do {                                                                                           \
+        if (bf16_io) n_x = bf16x4_to_f32(make_uint2(__float_as_uint(n_x.x), __float_as_uint(n_x.y))); \
         *reinterpret_cast<float4 *>(&tl[VX][ld_row][ld_col]) = softmax_x ? row_softmax4<E>(n_x) : n_x; \
         *reinterpret_cast<float4 *>(&tl[VQ][ld_row][ld_col]) = n_q;                                \
         *reinterpret_cast<float4 *>(&tl[VK][ld_row][ld_col]) = n_k;                                \
@@ -427,10 +458,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 const int f_ = tid + i_ * NT, r_ = f_ / Y, m_ = f_ - r_ * Y;                       \
                 if (f_ < TT * Y) {                                                                 \
                     tyd[r_][m_] = n_ydw[i_];                                                       \
-                    tgo[r_][m_] = n_gow[i_];                                                       \
+                    tgo[r_][m_] = bf16_io ? bf16_bits_to_f32(__float_as_uint(n_gow[i_])) : n_gow[i_]; \
                 }                                                                                  \
             }                                                                                      \
         } else {                                                                                   \
+            if (bf16_io) n_go = bf16x4_to_f32(make_uint2(__float_as_uint(n_go.x), __float_as_uint(n_go.y))); \
             *reinterpret_cast<float4 *>(&tgo[ld_row][ld_col]) = n_go;                              \
             *reinterpret_cast<float4 *>(&tyd[ld_row][ld_col]) = n_yd;                              \
         }                                                                                          \

@@ -7,7 +7,9 @@ same call signatures, same in-place final-state semantics -- backed by libsrwm_h
 
     out = self_ref_v0_steps(x, keep, W_y, W_q, W_k, w_b, sW_y, sW_q, sW_k, sw_b)   # see SelfRefv0Steps
 
-x: (N, H, L, E); W_y, W_q, W_k: (N, H, E, E); w_b: (N, H, E, 4); float32 on the GPU.
+x: (N, H, L, E); W_y, W_q, W_k: (N, H, E, E); w_b: (N, H, E, 4); float32 on the GPU.  x may also
+be bfloat16: the output (and the gradient handed back for x) is then bfloat16 too, while the
+weights, everything saved for the backward and all arithmetic stay float32.
 The weight tensors are OVERWRITTEN with the state after the last step (the layers read
 them back as the carried state); the backward starts from that mutated tensor.
 """
@@ -40,9 +42,9 @@ def _forward(dot, ctx, x, W_y, W_q, W_k, w_b):
     N, H, L, E = _check_shapes(x, W_y, W_q, W_k, w_b)
     fn = dot[device.type]
     # every element is written by the kernel, so no zero-fill is needed
-    big = lambda: torch.empty((N, H, L, E), device=device, dtype=x.dtype)
-    small = lambda: torch.empty((N, H, L, 4), device=device, dtype=x.dtype)
-    out = big()
+    big = lambda: torch.empty((N, H, L, E), device=device, dtype=torch.float32)
+    small = lambda: torch.empty((N, H, L, 4), device=device, dtype=torch.float32)
+    out = torch.empty((N, H, L, E), device=device, dtype=x.dtype)
     q_main, k_main, beta_main = big(), big(), small()
     y_diff, q_diff, k_diff, beta_diff = big(), big(), big(), small()
     fn(x, W_y, W_q, W_k, w_b, q_main, k_main, beta_main, y_diff, q_diff, k_diff, beta_diff, out)
@@ -63,7 +65,7 @@ class SelfRefv0(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         (x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, W_y, W_q, W_k, w_b) = ctx.saved_tensors
-        grad_x = torch.empty(x.shape, device=x.device, dtype=x.dtype)
+        grad_x = torch.empty(x.shape, device=x.device, dtype=torch.float32)
         grad_W_y = torch.empty_like(W_y, memory_format=torch.contiguous_format)
         grad_W_q = torch.empty_like(W_q, memory_format=torch.contiguous_format)
         grad_W_k = torch.empty_like(W_k, memory_format=torch.contiguous_format)
@@ -71,7 +73,7 @@ class SelfRefv0(torch.autograd.Function):
         SelfRefv0.dot_backward[x.device.type](
             x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out, W_y, W_q, W_k, w_b,
             grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b, flags=srwm_hip.GRAD_STATE_ZERO)
-        return grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b
+        return grad_x.to(x.dtype), grad_W_y, grad_W_q, grad_W_k, grad_w_b
 
 
 class StatefulSelfRefv0(torch.autograd.Function):
@@ -87,7 +89,7 @@ class StatefulSelfRefv0(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out, grad_W_y, grad_W_q, grad_W_k, grad_w_b):
         (x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, W_y, W_q, W_k, w_b) = ctx.saved_tensors
-        grad_x = torch.empty(x.shape, device=x.device, dtype=x.dtype)
+        grad_x = torch.empty(x.shape, device=x.device, dtype=torch.float32)
         # work on private contiguous copies: autograd may hand the same buffers elsewhere
         gs = [g.clone(memory_format=torch.contiguous_format) for g in
               (grad_W_y, grad_W_q, grad_W_k, grad_w_b)]
@@ -95,7 +97,7 @@ class StatefulSelfRefv0(torch.autograd.Function):
         StatefulSelfRefv0.dot_backward[x.device.type](
             x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out, W_y, W_q, W_k, w_b,
             grad_x, *gs, flags=mode)
-        return (grad_x, *gs)
+        return (grad_x.to(x.dtype), *gs)
 
 
 # Alias the autograd functions to python style snake case naming

@@ -45,6 +45,8 @@ _U = ctypes.c_uint
 
 _SIGNATURES = {
     "srwm_forward_f32": [_F, _S] + [_F] * 12 + [_I] * 4 + [_U, ctypes.c_void_p],
+    "srwm_forward_bf16": [_F, _S] + [_F] * 12 + [_I] * 4 + [_U, ctypes.c_void_p],
+    "srwm_backward_bf16": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_forward_wide_f32": [_F, _S] + [_F] * 12 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_backward_wide_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_layer_forward_f32": [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -165,8 +167,10 @@ def self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, 
     """SRWM forward over the whole sequence.  W_y, W_q, W_k, w_b are overwritten with the
     final state; q ... out are overwritten with the per-step vectors.  W_y is (N, H, E, Y):
     Y = E for the plain operator, any other width (3E+1 in the reference's second variant)
-    makes out and y_diff (N, H, L, Y)."""
-    _require(x, "x")
+    makes out and y_diff (N, H, L, Y).  x and out may both be bfloat16 (Y = E only); everything
+    else stays float32."""
+    io = x.dtype if isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 else torch.float32
+    _require(x, "x", None, io)
     N, H, L, E = x.shape
     _require(W_y, "W_y")
     Y = W_y.shape[-1]
@@ -176,16 +180,22 @@ def self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, 
     _require(w_b, "w_b", (N, H, E, 4))
     for t, nm in ((q, "q"), (k, "k"), (q_diff, "q_diff"), (k_diff, "k_diff")):
         _require(t, nm, (N, H, L, E))
-    for t, nm in ((y_diff, "y_diff"), (out, "out")):
-        _require(t, nm, (N, H, L, Y))
+    _require(y_diff, "y_diff", (N, H, L, Y))
+    _require(out, "out", (N, H, L, Y), io)
     _require(beta, "beta", (N, H, L, 4))
     _require(beta_diff, "beta_diff", (N, H, L, 4))
+    if io == torch.bfloat16 and Y != E:
+        raise ValueError("bfloat16 input is supported for W_y of shape (N, H, E, E) only")
     if x.numel() == 0 or Y == 0:
         return
     xs, xstr = _strided(x)
     with torch.cuda.device(x.device), \
             _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out], True) as d:
-        if Y == E:
+        if io == torch.bfloat16:
+            name = "srwm_forward_bf16"
+            code = lib().srwm_forward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
+                                           _stream(x.device))
+        elif Y == E:
             name = "srwm_forward_f32"
             code = lib().srwm_forward_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
                                           _stream(x.device))
@@ -270,15 +280,19 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
     behaves like the reference extension function: the grad_W buffers are read as the
     gradient w.r.t. the final state and the result is added to them (identical to a plain
     overwrite when they arrive zero-filled, which is how SelfRefv0.backward calls it).
-    W_y (N, H, E, Y) fixes the width of y_diff, grad_out and grad_W_y."""
-    _require(x, "x")
+    W_y (N, H, E, Y) fixes the width of y_diff, grad_out and grad_W_y.  x and grad_out may both be
+    bfloat16 (Y = E only); grad_x and everything else stay float32."""
+    io = x.dtype if isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 else torch.float32
+    _require(x, "x", None, io)
     N, H, L, E = x.shape
     _require(W_y, "W_y")
     Y = W_y.shape[-1]
     for t, nm in ((q, "q"), (k, "k"), (q_diff, "q_diff"), (k_diff, "k_diff"), (grad_x, "grad_x")):
         _require(t, nm, (N, H, L, E))
-    for t, nm in ((y_diff, "y_diff"), (grad_out, "grad_out")):
-        _require(t, nm, (N, H, L, Y))
+    _require(y_diff, "y_diff", (N, H, L, Y))
+    _require(grad_out, "grad_out", (N, H, L, Y), io)
+    if io == torch.bfloat16 and Y != E:
+        raise ValueError("bfloat16 input is supported for W_y of shape (N, H, E, E) only")
     _require(beta, "beta", (N, H, L, 4))
     _require(beta_diff, "beta_diff", (N, H, L, 4))
     for t, nm in ((W_y, "W_y"), (grad_W_y, "grad_W_y")):
@@ -295,7 +309,12 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
             _Dense([q, k, beta, y_diff, q_diff, k_diff, beta_diff], False) as sv, \
             _Dense([W_y, W_q, W_k, w_b], False) as st, \
             _Dense([grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b], True) as gr:
-        if Y == E:
+        if io == torch.bfloat16:
+            name = "srwm_backward_bf16"
+            code = lib().srwm_backward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
+                                            *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
+                                            N, H, L, E, flags, _stream(x.device))
+        elif Y == E:
             name = "srwm_backward_f32"
             code = lib().srwm_backward_f32(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
                                            *[_ptr(t) for t in st], *[_ptr(t) for t in gr],

@@ -408,3 +408,68 @@ def test_fused_layer_operator_matches_fp64_autograd(shape, Y, generic, with_shif
     if with_shift:
         for a, b in zip(shift_d, shift_c):
             assert rel_err(a.grad.cpu().numpy(), b.grad.numpy()) < TOL
+
+
+# ---------------------------------------------------------------- bf16 input / output, fp32 state
+
+BF16_TOL = 2e-2   # bf16 I/O with fp32 state: the output is rounded to 8 significant bits
+
+
+@pytest.mark.parametrize("flags", KERNELS)
+@pytest.mark.parametrize("shape,w_std,xsm", [
+    ((2, 16, 200, 64), 0.02, False),            # headline head size
+    ((4, 8, 100, 32), 1 / math.sqrt(32), True),  # RL shape
+    ((2, 2, 9, 16), 0.5, True),
+    ((1, 3, 7, 12), 0.5, False),                # LDS-resident kernels only
+])
+def test_bf16_io_matches_the_oracle_on_the_rounded_inputs(shape, w_std, xsm, flags):
+    """x and grad_out are rounded to bf16 first and the fp64 oracle runs on those values, so the only
+    differences left are fp32 arithmetic (1e-5) in the saved vectors and gradients and the final
+    rounding of `out` to bf16."""
+    print(f"case bf16 shape={shape} flags={flags}", flush=True)
+    import srwm_hip
+    x, W, go = srwm_inputs(*shape, seed=2, w_std=w_std, x_softmax=xsm, per_batch_state=True)
+    xb, gob = x.to(torch.bfloat16), go.to(torch.bfloat16)
+    N, H, L, E = shape
+    dev = _dev()
+    Wd = [w.to(dev, torch.float32).contiguous() for w in W]
+    big = lambda: torch.full((N, H, L, E), float("nan"), device=dev)
+    small = lambda: torch.full((N, H, L, 4), float("nan"), device=dev)
+    f = dict(q=big(), k=big(), beta=small(), y_diff=big(), q_diff=big(), k_diff=big(), beta_diff=small(),
+             out=torch.zeros((N, H, L, E), device=dev, dtype=torch.bfloat16))
+    srwm_hip.self_ref_forward(xb.to(dev), *Wd, *[f[n] for n in FWD_NAMES], flags=flags)
+    gx = torch.full((N, H, L, E), float("nan"), device=dev)
+    g = [torch.full_like(w, float("nan")) for w in Wd]
+    srwm_hip.self_ref_backward(xb.to(dev), *[f[n] for n in FWD_NAMES[:-1]], gob.to(dev), *Wd, gx, *g,
+                               flags=flags | srwm_hip.GRAD_STATE_ZERO)
+    of = oracle.srwm_forward(xb.double().numpy(), *[w.numpy() for w in W])
+    ob = oracle.srwm_backward(xb.double().numpy(), of, gob.double().numpy())
+    assert rel_err(f["out"].float().cpu().numpy(), of["out"]) < BF16_TOL
+    for n in FWD_NAMES[:-1]:
+        assert rel_err(f[n].cpu().numpy(), of[n]) < TOL, n            # fp32 all the way
+    for n, t in zip(("W_y", "W_q", "W_k", "w_b"), Wd):
+        assert rel_err(t.cpu().numpy(), of[n]) < TOL, n
+    assert rel_err(gx.cpu().numpy(), ob["grad_x"]) < TOL
+    for n, t in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), g):
+        assert rel_err(t.cpu().numpy(), ob[n]) < TOL, n
+
+
+def test_bf16_autograd_operator():
+    print("case bf16 autograd", flush=True)
+    from self_ref_v0 import self_ref_v0
+    N, H, L, E = 2, 4, 30, 32
+    x, W, go = srwm_inputs(N, H, L, E, seed=4, w_std=0.2, x_softmax=True, per_batch_state=True)
+    dev = _dev()
+    xb = x.to(dev, torch.bfloat16).requires_grad_(True)
+    Wd = [w.to(dev, torch.float32).requires_grad_(True) for w in W]
+    out = self_ref_v0(xb, *[w.clone() for w in Wd])
+    assert out.dtype == torch.bfloat16
+    (out * go.to(dev, torch.bfloat16)).sum().backward()
+    assert xb.grad.dtype == torch.bfloat16 and Wd[0].grad.dtype == torch.float32
+    xr = x.to(torch.bfloat16).double()
+    of = oracle.srwm_forward(xr.numpy(), *[w.numpy() for w in W])
+    # the upstream gradient autograd hands to the operator: d(sum(out*go))/d out = go, in bf16
+    ob = oracle.srwm_backward(xr.numpy(), of, go.to(torch.bfloat16).double().numpy())
+    assert rel_err(out.float().detach().cpu().numpy(), of["out"]) < BF16_TOL
+    assert rel_err(xb.grad.float().cpu().numpy(), ob["grad_x"]) < BF16_TOL
+    assert rel_err(Wd[0].grad.cpu().numpy(), ob["grad_W_y"]) < TOL
