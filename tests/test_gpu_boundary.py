@@ -132,3 +132,69 @@ def test_argument_errors_come_back_as_negative_codes():
     assert bool((outs[-1] == 0.0).all())                             # x = 0 -> y = 0, and it did run
     for code in (-1, -2, -3, -4):
         assert len(lib.srwm_hip_strerror(code)) > 8
+
+
+def test_operators_replay_from_a_captured_hip_graph():
+    """An actor's env step (L = 1 layer-operator forward) and a delta-rule forward+backward are
+    captured into one graph and replayed with new inputs in the static buffers; every replay must
+    equal the eager result on the same inputs.  The library launches only kernels (no memset
+    nodes, no allocation), which is what makes the capture legal."""
+    print("case graph replay", flush=True)
+    import srwm_hip
+    dev = _dev()
+    N, H, E = 8, 8, 32
+    g = torch.Generator().manual_seed(5)
+    slow = [(torch.randn(1, H, E, w, generator=g) * 0.2).to(dev) for w in (E, E, E, 4)]
+    x_static = torch.zeros(N, H, 1, E, device=dev)
+    shift = [torch.zeros(N, H, E, w, device=dev) for w in (E, E, E, 4)]
+    saved = [torch.empty(N, H, 1, w, device=dev) for w in (E, E, 4, E, E, E, 4)]
+    out = torch.empty(N, H, 1, E, device=dev)
+    D, L = 64, 70
+    q_s, k_s, v_s = (torch.zeros(2, 4, L, D, device=dev) for _ in range(3))
+    b_s = torch.zeros(2, 4, L, 1, device=dev)
+    go_s = torch.zeros(2, 4, L, D, device=dev)
+    W = torch.zeros(2, 4, D, D, device=dev)
+    dbuf = [torch.empty(2, 4, L, D, device=dev) for _ in range(3)]            # v_old, v_insert, out
+    dgr = [torch.empty(2, 4, L, D, device=dev) for _ in range(3)] + [torch.empty(2, 4, L, 1, device=dev)]
+    flags = srwm_hip.FLAG_STATE_SHIFT | srwm_hip.FLAG_SOFTMAX_INPUT
+
+    def work():
+        srwm_hip.self_ref_layer_forward(x_static, None, slow, *shift, *saved, out, flags=flags)
+        W.zero_()                                                               # a fill kernel, not a memset node
+        srwm_hip.fast_weight_forward(q_s, k_s, v_s, b_s, dbuf[0], dbuf[1], W, dbuf[2])
+        srwm_hip.fast_weight_backward(q_s, k_s, v_s, b_s, dbuf[0], dbuf[1], go_s, W, *dgr)
+
+    side = torch.cuda.Stream(device=dev)
+    with torch.cuda.stream(side):                # warm-up outside the capture (module loading, attributes)
+        work()
+    side.synchronize()
+    for s in shift:
+        s.zero_()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        work()
+    for s in shift:
+        s.zero_()
+    eager_shift = [torch.zeros_like(s) for s in shift]
+    for it in range(4):
+        xin = torch.randn(N, H, 1, E, generator=g).to(dev)
+        dq, dk = (torch.softmax(torch.randn(2, 4, L, D, generator=g), -1).to(dev) for _ in range(2))
+        dv, dgo = (torch.randn(2, 4, L, D, generator=g).to(dev) for _ in range(2))
+        db = torch.sigmoid(torch.randn(2, 4, L, 1, generator=g)).to(dev)
+        x_static.copy_(xin); q_s.copy_(dq); k_s.copy_(dk); v_s.copy_(dv); b_s.copy_(db); go_s.copy_(dgo)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [out.clone(), *[s.clone() for s in shift], dbuf[2].clone(), dgr[0].clone(), dgr[3].clone()]
+        # eager, on copies of the same inputs and the same carried state
+        e_saved = [torch.empty_like(t) for t in saved]
+        e_out = torch.empty_like(out)
+        srwm_hip.self_ref_layer_forward(xin, None, slow, *eager_shift, *e_saved, e_out, flags=flags)
+        eW = torch.zeros_like(W)
+        e_d = [torch.empty_like(t) for t in dbuf]
+        e_g = [torch.empty_like(t) for t in dgr]
+        srwm_hip.fast_weight_forward(dq, dk, dv, db, e_d[0], e_d[1], eW, e_d[2])
+        srwm_hip.fast_weight_backward(dq, dk, dv, db, e_d[0], e_d[1], dgo, eW, *e_g)
+        torch.cuda.synchronize()
+        want = [e_out, *eager_shift, e_d[2], e_g[0], e_g[3]]
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), it                 # same kernels, same inputs: bit-identical
