@@ -48,10 +48,10 @@ def run_hip(q, k, v, beta, W0, go, flags=0, grad_state=None, want_grad_W=False):
 @pytest.mark.parametrize("flags", KERNELS)
 @pytest.mark.parametrize("shape,qk,w0", [
     ((3, 5, 11, 64, 64), "sumnorm", 0.0),   # the reference self-test's shape / input style
-    ((4, 8, 256, 64, 64), "softmax", 0.0),  # BASELINE config 2, batch slice
+    ((4, 8, 256, 64, 64), "softmax", 0.0),  # benchmark configuration 2, batch slice
     ((2, 3, 50, 16, 16), "softmax", 0.3),
     ((2, 2, 40, 32, 32), "l2", 0.0),
-    ((1, 4, 300, 128, 128), "l2", 0.0),     # BASELINE config 5's state size, fp32 I/O, short
+    ((1, 4, 300, 128, 128), "l2", 0.0),     # benchmark configuration 5's state size, fp32 I/O, short
     ((2, 3, 17, 8, 12), "l2", 0.5),          # E != M -> generic kernel
     ((2, 2, 1, 16, 16), "softmax", 0.2),     # L = 1
 ])
@@ -148,7 +148,7 @@ def test_autograd_function_with_either_kernel_family(chunkwise):
 
 
 def test_full_config2_properties():
-    """BASELINE config 2 at full size: finite outputs, revert-to-W0 round trip, linearity in
+    """benchmark configuration 2 at full size: finite outputs, revert-to-W0 round trip, linearity in
     grad_out, oracle on a sample of sequences."""
     print("case full C2 properties", flush=True)
     q, k, v, beta, W0, go = delta_inputs(32, 8, 256, 64, 64, seed=0)
@@ -177,7 +177,7 @@ BF16_TOL = 2e-2   # bf16 inputs, fp32 state: bar stated for this mode
 @pytest.mark.parametrize("shape,qk", [
     ((2, 3, 64, 16, 16), "softmax"),
     ((2, 2, 200, 64, 64), "softmax"),
-    ((1, 2, 1024, 128, 128), "l2"),      # BASELINE config 5's state size and input style, shorter
+    ((1, 2, 1024, 128, 128), "l2"),      # benchmark configuration 5's state size and input style, shorter
     ((1, 2, 40, 24, 24), "l2"),          # no bf16 kernel for D=24: widened on the host side
 ])
 def test_bf16_io_matches_oracle_on_rounded_inputs(shape, qk):
@@ -212,8 +212,8 @@ def test_bf16_io_matches_oracle_on_rounded_inputs(shape, qk):
     ((1, 3, 256, 128, 128), "l2", 0.0, torch.float32),       # two workgroups per sequence
     ((1, 2, 37, 128, 128), "l2", 0.2, torch.float32),        # shorter than a chunk
     ((1, 2, 2048, 128, 128), "l2", 0.0, torch.float32),      # 32 chunks in a row
-    ((2, 8, 256, 64, 64), "softmax", 0.0, torch.float32),    # BASELINE config 2 style
-    ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # BASELINE config 5 style, shorter
+    ((2, 8, 256, 64, 64), "softmax", 0.0, torch.float32),    # benchmark configuration 2 style
+    ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # benchmark configuration 5 style, shorter
 ])
 def test_chunkwise_forward_matches_oracle_and_feeds_the_sequential_backward(shape, qk, w0, io):
     """Chunkwise (C = 64) MFMA forward vs the fp64 oracle, then the step-by-step backward run on
@@ -251,9 +251,9 @@ def test_chunkwise_forward_matches_oracle_and_feeds_the_sequential_backward(shap
     ((1, 3, 256, 128, 128), "l2", 0.0, torch.float32),       # two workgroups per sequence, row sweep in chunks of 32
     ((1, 2, 37, 128, 128), "l2", 0.2, torch.float32),        # shorter than a chunk
     ((1, 2, 1100, 128, 128), "l2", 0.0, torch.float32),      # many chunks, ragged
-    ((2, 8, 256, 64, 64), "softmax", 0.0, torch.float32),    # BASELINE config 2 style
+    ((2, 8, 256, 64, 64), "softmax", 0.0, torch.float32),    # benchmark configuration 2 style
     ((2, 2, 300, 64, 64), "softmax", 0.2, torch.bfloat16),
-    ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # BASELINE config 5 style, shorter
+    ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # benchmark configuration 5 style, shorter
     ((1, 2, 150, 128, 128), "l2", 0.3, torch.bfloat16),
 ])
 @pytest.mark.parametrize("state_grad", [False, True])
@@ -294,7 +294,7 @@ def test_chunkwise_backward_matches_oracle(shape, qk, w0, io, state_grad):
 
 
 def test_full_config5_properties():
-    """BASELINE config 5 at full size (N=8, H=16, L=4096, E=M=128, bf16 I/O, fp32 memory):
+    """benchmark configuration 5 at full size (N=8, H=16, L=4096, E=M=128, bf16 I/O, fp32 memory):
     the step-by-step and the chunkwise forward agree with each other, the backward reverts the
     memory to W_0 = 0, and sampled sequences match the fp64 oracle run on the rounded inputs."""
     print("case full C5 properties", flush=True)

@@ -73,9 +73,9 @@ KERNELS = [pytest.param(0, id="default"), pytest.param(16, id="generic")]
 @pytest.mark.parametrize("flags", KERNELS)
 @pytest.mark.parametrize("shape,w_std,xsm,per_batch", [
     ((3, 5, 11, 8), 0.6, True, True),                  # the reference self-test's shape / input style
-    ((2, 4, 64, 16), 0.02, False, False),              # BASELINE config 1
-    ((4, 8, 100, 32), 1 / math.sqrt(32), True, False),  # BASELINE config 3, batch slice
-    ((2, 16, 512, 64), 0.02, False, False),            # BASELINE config 4 (headline), batch slice
+    ((2, 4, 64, 16), 0.02, False, False),              # benchmark configuration 1
+    ((4, 8, 100, 32), 1 / math.sqrt(32), True, False),  # benchmark configuration 3, batch slice
+    ((2, 16, 512, 64), 0.02, False, False),            # benchmark configuration 4 (headline), batch slice
     ((1, 3, 7, 5), 0.8, False, True),                  # odd head size -> generic kernel
     ((2, 2, 1, 16), 0.3, True, True),                  # L = 1 (how the RL actors call it)
     ((1, 2, 33, 64), 0.1, True, True),                 # E = 64 with a stronger state
@@ -171,7 +171,7 @@ def test_autograd_function_drop_in():
 
 
 def test_full_headline_shape_properties():
-    """BASELINE config 4 at full size (N=32, H=16, L=512, E=64): size-independent properties
+    """benchmark configuration 4 at full size (N=32, H=16, L=512, E=64): size-independent properties
     plus the oracle on a sample of the 512 sequences."""
     print("case full C4 properties", flush=True)
     N, H, L, E = 32, 16, 512, 64
@@ -229,7 +229,7 @@ def test_errors_are_reported_not_swallowed():
 # ---------------------------------------------------------- step-wise (RL learner) call pattern
 
 @pytest.mark.parametrize("shape,resets", [
-    ((4, 8, 100, 32), True),      # BASELINE config 3 shape (batch slice): register-resident kernel
+    ((4, 8, 100, 32), True),      # benchmark configuration 3 shape (batch slice): register-resident kernel
     ((2, 2, 37, 64), True),
     ((3, 2, 20, 12), True),       # generic kernel
     ((2, 3, 15, 16), False),      # keep = None

@@ -126,7 +126,7 @@ def test_backward_reverts_the_state_to_W0():
 
 @pytest.mark.parametrize("shape,w_std,xsm", [
     ((3, 5, 11, 8), 0.6, True),     # the reference self-test's shape and input style
-    ((2, 4, 64, 16), 0.02, False),  # BASELINE config 1 (CPU parity anchor)
+    ((2, 4, 64, 16), 0.02, False),  # benchmark configuration 1 (CPU parity anchor)
     ((2, 2, 20, 32), 1 / math.sqrt(32), True),
     ((1, 3, 5, 7), 1.0, False),     # odd head dim
 ])
