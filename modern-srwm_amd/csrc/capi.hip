@@ -188,11 +188,15 @@ int srwm_readout_grad_f32(const float *k, const float *beta, const float *ydiff,
                           const float *Wy_entry, float *grad_x, int N, int H, int L, int E,
                           unsigned flags, void *stream) {
     if (!k || !beta || !ydiff || !grad_out || !gs || !Wy_entry || !grad_x || (keep && !sWy)) return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || flags) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
     if (!stride_ok(gs, N, H, L, E)) return SRWM_ESTRIDE;
-    if (E > 256 || replay_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
     ReplayParams p{k, {(int64_t)H * L * E, (int64_t)L * E, E}, ydiff, beta, 4, keep, grad_out,
                    {gs[0], gs[1], gs[2]}, Wy_entry, keep ? sWy : nullptr, grad_x, N, H, L, E, E};
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_replay_tiled(p, (hipStream_t)stream);
+        if (r >= 0) return r;
+    }
+    if (E > 256 || replay_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
     return launch_replay(p, (hipStream_t)stream);
 }
 
@@ -222,11 +226,15 @@ int delta_readout_replay_f32(const float *K, const int64_t ks[3], const float *v
                              const float *grad_out, const int64_t gs[3], const float *W_entry, float *u,
                              int N, int H, int L, int E, int M, unsigned flags, void *stream) {
     if (!K || !ks || !v_insert || !grad_out || !gs || !W_entry || !u) return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || flags) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
     if (!stride_ok(ks, N, H, L, E) || !stride_ok(gs, N, H, L, M)) return SRWM_ESTRIDE;
-    if (E > 256 || M > 256 || replay_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     ReplayParams p{K, {ks[0], ks[1], ks[2]}, v_insert, nullptr, 0, keep, grad_out, {gs[0], gs[1], gs[2]},
                    W_entry, nullptr, u, N, H, L, E, M};
+    if (!(flags & SRWM_FLAG_GENERIC)) {
+        const int r = launch_replay_tiled(p, (hipStream_t)stream);
+        if (r >= 0) return r;
+    }
+    if (E > 256 || M > 256 || replay_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_replay(p, (hipStream_t)stream);
 }
 

@@ -141,6 +141,7 @@ size_t delta_bwd_generic_lds_bytes(int E, int M);
 int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s);
 size_t replay_lds_bytes(int E, int M);
 int launch_replay(const ReplayParams &p, hipStream_t s);
+int launch_replay_tiled(const ReplayParams &p, hipStream_t s);   // -1: no register-resident instantiation
 int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s);
 // dst[j][h, :] = sum over n of src[j][n, h, :] for the four state tensors (y: E x Y, q, k: E x E, b: E x 4)
 int launch_srwm_batch_sum(const float *const src[4], float *const dst[4], int N, int H, int E, int Y, hipStream_t s);

@@ -12,8 +12,12 @@
 // replays W forward in time from its entry value with the saved write vectors
 // (W += a (x) (s b)), applies the same resets, and reads W g before each write.
 //
-// One workgroup per (batch, head) sequence, the E x M matrix in LDS (odd row stride), 16-lane
-// groups own rows; the vectors of a step are fetched one step ahead.
+// Two kernels.  replay_tiled_kernel (square matrices of 8..128 rows): the matrix lives in
+// registers, a wave owns a block of rows (all columns), so the row sums finish inside the wave
+// and the waves of a workgroup never meet -- no barrier in the whole kernel; the vectors of TT
+// steps are staged in a wave-private LDS tile, fetched one tile ahead.  replay_kernel (any
+// size that fits): the matrix in LDS (odd row stride), 16-lane groups own rows, the vectors of a
+// step fetched one step ahead.
 #include "common.h"
 #include "xlane.h"
 
@@ -81,7 +85,156 @@ __global__ __launch_bounds__(kThreads) void replay_kernel(ReplayParams p) {
     }
 }
 
+// Register-resident replay.  NWV waves per sequence; wave w owns rows [w*ER, (w+1)*ER), ER = E/NWV.
+// Inside a wave, CGL consecutive lanes share a block of R rows and split its M columns (CB each).
+template <int E, int M, int NWV, int CGL>
+__global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p) {
+    constexpr int ER = E / NWV, RGL = kWave / CGL, R = ER / RGL, CB = M / CGL;
+    constexpr int TT = M > 64 ? 8 : (256 / ER > 16 ? 256 / ER : 16);   // steps per tile
+    constexpr int NG = TT * M / 4 / kWave, NA = TT * ER / 4 / kWave;    // float4 per lane per tile
+    static_assert(ER * NWV == E && R * RGL == ER && CB * CGL == M && R >= 1 && CB >= 1, "tiling");
+    static_assert(NG * 4 * kWave == TT * M && NA * 4 * kWave == TT * ER && TT <= kWave, "tile loader");
+    static_assert(CGL <= 16, "row sums must stay inside a DPP row");
+
+    __shared__ __attribute__((aligned(16))) float tg[NWV][TT][M];    // g_t
+    __shared__ __attribute__((aligned(16))) float tb[NWV][TT][M];    // b_t
+    __shared__ __attribute__((aligned(16))) float ta[NWV][TT][ER];   // this wave's rows of a_t
+    __shared__ float tsk[NWV][2][TT];                                // s_t | keep_t
+
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int cgl = lane % CGL, rg = lane / CGL;
+    const int e0 = wave * ER, r0 = rg * R, c0 = cgl * CB;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const float *ab = p.a + n * p.as.n + h * p.as.h + e0;
+    const float *gb = p.g + n * p.gs.n + h * p.gs.h;
+    const float *bb = p.b + seq * p.L * M;
+
+    float w[R][CB];
+    auto load_w = [&](const float *src) {   // src: E x M of this sequence / head, or nullptr for zero
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int c = 0; c < CB; ++c) w[i][c] = src ? src[(e0 + r0 + i) * M + c0 + c] : 0.f;
+    };
+    load_w(p.W0 + seq * E * M);
+    const float *wreset = p.Wreset ? p.Wreset + (int64_t)h * E * M : nullptr;
+
+    // next tile, staged in registers: rows past the end are clamped (loaded, never used)
+    float4 ng[NG], nb[NG], na[NA];
+    float ns = 1.f, nk = 1.f;
+    auto fetch = [&](int tile) {
+#pragma unroll
+        for (int i = 0; i < NG; ++i) {
+            const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
+            const int64_t t = min(tile * TT + row, p.L - 1);
+            ng[i] = *reinterpret_cast<const float4 *>(gb + t * p.gs.l + col);
+            nb[i] = *reinterpret_cast<const float4 *>(bb + t * M + col);
+        }
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            const int f = lane + i * kWave, row = f / (ER / 4), col = (f % (ER / 4)) * 4;
+            const int64_t t = min(tile * TT + row, p.L - 1);
+            na[i] = *reinterpret_cast<const float4 *>(ab + t * p.as.l + col);
+        }
+        if (lane < TT) {
+            const int64_t t = min(tile * TT + lane, p.L - 1);
+            ns = p.bscale ? p.bscale[(seq * p.L + t) * p.bscale_stride] : 1.f;
+            nk = p.keep ? p.keep[(int64_t)n * p.L + t] : 1.f;
+        }
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int i = 0; i < NG; ++i) {
+            const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
+            *reinterpret_cast<float4 *>(&tg[wave][row][col]) = ng[i];
+            *reinterpret_cast<float4 *>(&tb[wave][row][col]) = nb[i];
+        }
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            const int f = lane + i * kWave, row = f / (ER / 4), col = (f % (ER / 4)) * 4;
+            *reinterpret_cast<float4 *>(&ta[wave][row][col]) = na[i];
+        }
+        if (lane < TT) {
+            tsk[wave][0][lane] = ns;
+            tsk[wave][1][lane] = nk;
+        }
+    };
+
+    const int ntiles = (p.L + TT - 1) / TT;
+    fetch(0);
+    commit();
+    wave_lds_fence();
+    for (int tile = 0; tile < ntiles; ++tile) {
+        const int tlen = min(TT, p.L - tile * TT);
+        if (tile + 1 < ntiles) fetch(tile + 1);
+        for (int tt = 0; tt < tlen; ++tt) {
+            const int t = tile * TT + tt;
+            if (tsk[wave][1][tt] == 0.f) load_w(wreset);   // uniform over the wave
+            float gv[CB], bv[CB], av[R];
+#pragma unroll
+            for (int c = 0; c < CB; ++c) {
+                gv[c] = tg[wave][tt][c0 + c];
+                bv[c] = tb[wave][tt][c0 + c];
+            }
+#pragma unroll
+            for (int i = 0; i < R; ++i) av[i] = ta[wave][tt][r0 + i];
+            const float sc = tsk[wave][0][tt];
+            // u = W g: the lane's R partial row sums, completed over the CGL lanes of the row block
+            float u[R];
+#pragma unroll
+            for (int i = 0; i < R; ++i) {
+                u[i] = 0.f;
+#pragma unroll
+                for (int c = 0; c < CB; ++c) u[i] = fmaf(w[i][c], gv[c], u[i]);
+            }
+            group_sum_n<CGL, R>(u);
+            if (cgl == 0) {
+                float *dst = p.u + (seq * p.L + t) * E + e0 + r0;
+#pragma unroll
+                for (int i = 0; i < R; ++i) dst[i] = u[i];
+            }
+            // the step's write
+#pragma unroll
+            for (int c = 0; c < CB; ++c) bv[c] *= sc;
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < CB; ++c) w[i][c] = fmaf(av[i], bv[c], w[i][c]);
+        }
+        if (tile + 1 < ntiles) {
+            wave_lds_fence();   // this wave's reads of the tile are done
+            commit();
+            wave_lds_fence();
+        }
+    }
+}
+
+template <int E, int NWV, int CGL>
+int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
+    hipLaunchKernelGGL((replay_tiled_kernel<E, E, NWV, CGL>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
+    return (int)hipGetLastError();
+}
+
+bool rows16(const void *ptr, const Strided3 &st) {
+    return (uintptr_t)ptr % 16 == 0 && st.n % 4 == 0 && st.h % 4 == 0 && st.l % 4 == 0;
+}
+
 }  // namespace
+
+// Register-resident replay for square matrices with aligned rows; -1 when there is no instantiation.
+int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
+    if (p.E != p.M || !rows16(p.a, p.as) || !rows16(p.g, p.gs) || (uintptr_t)p.b % 16 || (uintptr_t)p.u % 16)
+        return -1;
+    switch (p.E) {
+        case 128: return launch_replay_tiled<128, 4, 16>(p, s);
+        case 64: return launch_replay_tiled<64, 2, 8>(p, s);
+        case 32: return launch_replay_tiled<32, 1, 8>(p, s);
+        case 16: return launch_replay_tiled<16, 1, 8>(p, s);
+        case 8: return launch_replay_tiled<8, 1, 8>(p, s);
+        default: return -1;
+    }
+}
 
 size_t replay_lds_bytes(int E, int M) { return sizeof(float) * ((size_t)E * (M | 1) + E + 2 * (size_t)M); }
 

@@ -245,9 +245,10 @@ def self_ref_forward_steps(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff
     _check(code, "srwm_forward_steps_f32")
 
 
-def self_ref_readout_grad(k, beta, y_diff, keep, slow_W_y, grad_out, W_y_entry, grad_x):
+def self_ref_readout_grad(k, beta, y_diff, keep, slow_W_y, grad_out, W_y_entry, grad_x, flags=0):
     """grad_x[n, h, t] = W_y,t-1 grad_out[n, h, t] for an unroll whose carried state is detached
-    between steps; W_y_entry is the (N, H, E, E) y block as it was before self_ref_forward_steps."""
+    between steps; W_y_entry is the (N, H, E, E) y block as it was before self_ref_forward_steps.
+    flags: FLAG_GENERIC forces the LDS-resident kernel."""
     _require(k, "k")
     N, H, L, E = k.shape
     _require(beta, "beta", (N, H, L, 4))
@@ -269,7 +270,7 @@ def self_ref_readout_grad(k, beta, y_diff, keep, slow_W_y, grad_out, W_y_entry, 
         code = lib().srwm_readout_grad_f32(
             _ptr(sv[0]), _ptr(sv[1]), _ptr(sv[2]), _ptr(keep) if keep is not None else null,
             _ptr(slow_W_y) if keep is not None else null, _ptr(gos), gstr, _ptr(sv[3]), _ptr(gr[0]),
-            N, H, L, E, 0, _stream(k.device))
+            N, H, L, E, flags, _stream(k.device))
     _check(code, "srwm_readout_grad_f32")
 
 
@@ -485,9 +486,10 @@ def fast_weight_forward_steps(q, k, v, beta, keep, v_old, v_insert, kv, out, fla
     _check(code, "delta_forward_steps_f32")
 
 
-def fast_weight_readout_replay(k, v_insert, keep, grad_out, kv_entry, u):
+def fast_weight_readout_replay(k, v_insert, keep, grad_out, kv_entry, u, flags=0):
     """u[n, h, t] = W_{t-1} grad_out[n, h, t] for an unroll whose memory carries no gradient;
-    kv_entry is the (N, H, E, M) memory as it was before fast_weight_forward_steps."""
+    kv_entry is the (N, H, E, M) memory as it was before fast_weight_forward_steps.
+    flags: FLAG_GENERIC forces the LDS-resident kernel."""
     _require(k, "k")
     N, H, L, E = k.shape
     _require(v_insert, "v_insert")
@@ -505,7 +507,7 @@ def fast_weight_readout_replay(k, v_insert, keep, grad_out, kv_entry, u):
     (ks, kstr), (gos, gstr) = _strided(k), _strided(grad_out)
     with torch.cuda.device(k.device), _Dense([v_insert, kv_entry], False) as sv, _Dense([u], True) as d:
         code = lib().delta_readout_replay_f32(_ptr(ks), kstr, _ptr(sv[0]), _ptr(keep) if keep is not None else null,
-                                              _ptr(gos), gstr, _ptr(sv[1]), _ptr(d[0]), N, H, L, E, M, 0,
+                                              _ptr(gos), gstr, _ptr(sv[1]), _ptr(d[0]), N, H, L, E, M, flags,
                                               _stream(k.device))
     _check(code, "delta_readout_replay_f32")
 

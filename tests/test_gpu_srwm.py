@@ -473,3 +473,54 @@ def test_bf16_autograd_operator():
     assert rel_err(out.float().detach().cpu().numpy(), of["out"]) < BF16_TOL
     assert rel_err(xb.grad.float().cpu().numpy(), ob["grad_x"]) < BF16_TOL
     assert rel_err(Wd[0].grad.cpu().numpy(), ob["grad_W_y"]) < TOL
+
+
+# ---------------------------------------------------------------- readout-gradient replay kernels
+
+@pytest.mark.parametrize("E,NH,L", [(8, (2, 3), 70), (16, (2, 2), 33), (32, (4, 8), 100), (64, (2, 4), 50),
+                                    (128, (1, 2), 41)])
+def test_replay_kernels_agree_and_match_a_numpy_replay(E, NH, L):
+    """u_t = W_{t-1} g_t with W_t = W_{t-1} + a_t (x) (s_t b_t) and resets: the register-resident
+    kernel, the LDS-resident kernel and an fp64 numpy loop."""
+    print(f"case replay E={E} L={L}", flush=True)
+    import srwm_hip
+    N, H = NH
+    g = torch.Generator().manual_seed(E)
+    a = torch.softmax(torch.randn(N, H, L, E, generator=g, dtype=torch.float64), -1)
+    b = torch.randn(N, H, L, E, generator=g, dtype=torch.float64) * 0.5
+    beta = torch.sigmoid(torch.randn(N, H, L, 4, generator=g, dtype=torch.float64))
+    go = torch.randn(N, H, L, E, generator=g, dtype=torch.float64)
+    W0 = torch.randn(N, H, E, E, generator=g, dtype=torch.float64) * 0.3
+    Wr = torch.randn(H, E, E, generator=g, dtype=torch.float64) * 0.3
+    keep = (torch.rand(N, L, generator=g) > 0.1).double()
+    # fp64 loop
+    u_ref = np.zeros((N, H, L, E))
+    W = W0.numpy().copy()
+    for t in range(L):
+        for n in range(N):
+            if keep[n, t] == 0:
+                W[n] = Wr.numpy()
+        u_ref[:, :, t] = np.einsum("nhem,nhm->nhe", W, go[:, :, t].numpy())
+        W += np.einsum("nhe,nhm->nhem", a[:, :, t].numpy(), (beta[:, :, t, :1] * b[:, :, t]).numpy())
+    dev = _dev()
+    f32 = lambda t: t.to(dev, torch.float32).contiguous()
+    args = (f32(a), f32(beta), f32(b), f32(keep), f32(Wr), f32(go), f32(W0))
+    outs = []
+    for flags in (0, srwm_hip.FLAG_GENERIC):
+        u = torch.full((N, H, L, E), float("nan"), device=dev)
+        srwm_hip.self_ref_readout_grad(*args, u, flags=flags)
+        assert rel_err(u.cpu().numpy(), u_ref) < TOL, flags
+        outs.append(u)
+    # the delta-rule flavour (no scale, reset to zero) through the same kernels, strided g
+    go_l = f32(go.permute(2, 0, 1, 3)).permute(1, 2, 0, 3)
+    W = W0.numpy().copy()
+    for t in range(L):
+        for n in range(N):
+            if keep[n, t] == 0:
+                W[n] = 0.0
+        u_ref[:, :, t] = np.einsum("nhem,nhm->nhe", W, go[:, :, t].numpy())
+        W += np.einsum("nhe,nhm->nhem", a[:, :, t].numpy(), b[:, :, t].numpy())
+    for flags in (0, srwm_hip.FLAG_GENERIC):
+        u = torch.full((N, H, L, E), float("nan"), device=dev)
+        srwm_hip.fast_weight_readout_replay(f32(a), f32(b), f32(keep), go_l, f32(W0), u, flags=flags)
+        assert rel_err(u.cpu().numpy(), u_ref) < TOL, flags
