@@ -303,6 +303,10 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
     _require(w_b, "w_b", (N, H, E, 4))
     _require(grad_w_b, "grad_w_b", (N, H, E, 4))
     if x.numel() == 0 or Y == 0:
+        # no steps: the state gradient passes through unchanged (zero when none came in)
+        if (flags & 3) == GRAD_STATE_ZERO:
+            for g in (grad_W_y, grad_W_q, grad_W_k, grad_w_b):
+                g.zero_()
         return
     xs, xstr = _strided(x)
     gos, gstr = _strided(grad_out)
@@ -368,6 +372,12 @@ def self_ref_layer_forward(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff
         _require(keep, "keep", (N, L))
         keep = keep.contiguous()
     if x.numel() == 0:
+        if flags & FLAG_FRESH_STATE:   # no steps: the state is the shared weights (a zero shift)
+            for w, sw in zip((W_y, W_q, W_k, w_b), sl):
+                if flags & FLAG_STATE_SHIFT:
+                    w.zero_()
+                else:
+                    w.copy_(sw.unsqueeze(0).expand_as(w))
         return
     xs, xstr = _strided(x)
     with torch.cuda.device(x.device), \
@@ -409,6 +419,12 @@ def self_ref_layer_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, gr
                 raise ValueError("grad_slow tensors must be contiguous")
         gsl = [_ptr(g) for g in grad_slow]
     if x.numel() == 0:
+        if (flags & 3) == GRAD_STATE_ZERO:
+            for g in grad_W:
+                g.zero_()
+        if grad_slow is not None:
+            for gs_, g in zip(grad_slow, grad_W):
+                gs_.copy_(g.sum(0))
         return
     xs, xstr = _strided(x)
     gos, gstr = _strided(grad_out)
@@ -538,6 +554,8 @@ def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, g
     if grad_kv is not None:
         _require(grad_kv, "grad_kv", (N, H, E, M))
     if q.numel() == 0 or v.numel() == 0:
+        if grad_kv is not None and (flags & 3) == GRAD_STATE_ZERO:
+            grad_kv.zero_()
         return
     if io == torch.bfloat16 and not _has_bf16_kernel(E, M):
         g32 = [torch.empty(t.shape, device=t.device, dtype=torch.float32)

@@ -198,3 +198,34 @@ def test_operators_replay_from_a_captured_hip_graph():
         want = [e_out, *eager_shift, e_d[2], e_g[0], e_g[3]]
         for a, b in zip(got, want):
             assert torch.equal(a, b), it                 # same kernels, same inputs: bit-identical
+
+
+def test_empty_sequences_and_batches():
+    """L = 0 and N = 0 through the autograd operators: empty outputs, state untouched, zero weight
+    gradients (not uninitialised memory)."""
+    from fast_weight import fast_weight_delta
+    from self_ref_v0 import self_ref_layer, self_ref_v0
+    dev = _dev()
+    H, E = 2, 16
+    for N, L in ((3, 0), (0, 5)):
+        x = torch.zeros(N, H, L, E, device=dev, requires_grad=True)
+        W = [torch.randn(N, H, E, w, device=dev).requires_grad_(True) for w in (E, E, E, 4)]
+        Wc = [w.detach().clone() for w in W]
+        out = self_ref_v0(x, *[w.clone() for w in W])
+        assert out.shape == (N, H, L, E)
+        (out.sum() + 0.0 * sum(w.sum() for w in W)).backward()
+        for w, c in zip(W, Wc):
+            assert torch.equal(w.detach(), c) and bool((w.grad == 0).all())
+        q = torch.zeros(N, H, L, E, device=dev, requires_grad=True)
+        beta = torch.zeros(N, H, L, 1, device=dev, requires_grad=True)
+        mem = torch.randn(N, H, E, E, device=dev)
+        mc = mem.clone()
+        o = fast_weight_delta(q, q, q, beta, mem)
+        o.sum().backward()
+        assert o.shape == (N, H, L, E) and torch.equal(mem, mc) and q.grad.shape == q.shape
+    slow = [torch.randn(1, H, E, w, device=dev).requires_grad_(True) for w in (E, E, E, 4)]
+    x = torch.zeros(3, H, 0, E, device=dev, requires_grad=True)
+    out, *shift = self_ref_layer(x, *slow, None, None, None, None, True)
+    (out.sum() + sum(s.sum() for s in shift)).backward()
+    assert all(bool((s == 0).all()) for s in shift)            # no steps: the state stays at the shared weights
+    assert all(bool((w.grad == 0).all()) for w in slow)        # d(shift)/d(shared) = dW_L/d(shared) - 1 = 0
