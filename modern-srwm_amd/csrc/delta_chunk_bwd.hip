@@ -349,19 +349,31 @@ struct RowLds {
                       MatC::bytes(C) % 16 == 0, "alignment");
 };
 
-template <class TI, int D, int MS, int C>
-__global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP<TI> p) {
+// KS = 2: 8 waves; a pair of waves owns the same 16 memory rows and splits their columns (the
+// contraction index of dOut S^T, U dS'^T, Y S^T) in halves.  Each computes its half of those
+// products for the whole chunk, hands the part belonging to the other's half of the chunk over
+// through LDS (the K / Q slices are dead by then: their fragments sit in registers), and finishes
+// grad_Q, grad_K for its own half of the chunk.
+template <class TI, int D, int MS, int C, int KS>
+__global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(ChunkBwdP<TI> p) {
     typedef RowLds<TI, D, C> Lds;
     typedef typename Lds::X X;
-    constexpr int CB = C / 16, MB = D / 16, NTRI = CB * (CB + 1) / 2;
+    constexpr int NT = kThreads * KS;
+    constexpr int CB = C / 16, MBF = D / 16, MB = MBF / KS, NTRI = CB * (CB + 1) / 2;   // MB: column blocks held by a wave
+    constexpr int CBH = CB / KS;                                                         // chunk row blocks a wave finishes
     static_assert(MS * kWC == D, "row split");
+    static_assert(KS == 1 || (CB % KS == 0 && 8 * CBH * 64 * 16 <= 2 * Lds::MatK::bytes(C)), "exchange buffer");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const typename Lds::MatG Gs(smem + Lds::oG, C);
     const typename Lds::MatU Us(smem + Lds::oU, C), Ys(smem + Lds::oY, C);
     const typename Lds::MatK Kw(smem + Lds::oK, C), Qw(smem + Lds::oQ, C);
     const typename Lds::MatC G1(smem + Lds::oG1, C), Z(smem + Lds::oZ, C);
 
-    const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+    f32x4 *Xs = reinterpret_cast<f32x4 *>(smem + Lds::oK);   // KS == 2: [8 waves][CBH tiles][64 lanes]
+
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    const int wave = wv & 3, hf = wv >> 2;           // row block, column half
+    const int m0 = hf * MB * 16;                     // first memory column held by this wave
     const int ln = lane & 15, lq = lane >> 4;
     const int64_t seq = blockIdx.x / MS;
     const int e0 = (int)(blockIdx.x % MS) * kWC;     // first memory row of this workgroup
@@ -372,12 +384,12 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
     const TI *gob = p.go + n * p.gs.n + h * p.gs.h;
     const float *yb = p.gV + seq * p.L * D;
     const float *ub = p.vins + seq * p.L * D;
-    float *Wg = p.W + seq * D * D + (e0 + cw + ln) * D;            // row e0 + cw + ln of the memory
-    float *gWg = p.gW ? p.gW + seq * D * D + (e0 + cw + ln) * D : nullptr;
+    float *Wg = p.W + seq * D * D + (e0 + cw + ln) * D + m0;       // row e0 + cw + ln of the memory, from column m0
+    float *gWg = p.gW ? p.gW + seq * D * D + (e0 + cw + ln) * D + m0 : nullptr;
     const bool g_in = gWg && p.grad_state_mode != 0u;
 
     // 16 rows of the memory and of its gradient, transposed: tile mb, register r <-> column
-    // 16*mb + 4*lq + r, lane ln <-> row
+    // m0 + 16*mb + 4*lq + r, lane ln <-> row
     f32x4 st[MB], dst[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -391,16 +403,16 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
         }
     }
 
-    constexpr int NG = C * (D / 4) / kThreads;      // 4-element groups per thread of dOut, U, Y
-    constexpr int NK = C * (kWC / 4) / kThreads;    // ... of the K and Q slices
-    static_assert(NG >= 1 && NK >= 1, "chunk too short for 256 threads");
+    constexpr int NG = C * (D / 4) / NT;      // 4-element groups per thread of dOut, U, Y
+    constexpr int NK = C * (kWC / 4) / NT;    // ... of the K and Q slices
+    static_assert(NG >= 1 && NK >= 1, "chunk too short for the workgroup");
     typename X::Raw4 greg[NG], kreg[NK], qreg[NK];
     float4 ureg[NG], yreg[NG];
     auto prefetch = [&](int ch) {
         const int t0 = ch * C;
 #pragma unroll
         for (int i = 0; i < NG; ++i) {
-            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const int f = tid + i * NT, row = f / (D / 4), col = (f % (D / 4)) * 4;
             const int64_t t = min(t0 + row, p.L - 1);
             greg[i] = X::ld_raw(gob + t * p.gs.l + col);
             ureg[i] = *reinterpret_cast<const float4 *>(ub + t * D + col);
@@ -408,7 +420,7 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
         }
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
-            const int f = tid + i * kThreads, row = f / (kWC / 4), col = (f % (kWC / 4)) * 4;
+            const int f = tid + i * NT, row = f / (kWC / 4), col = (f % (kWC / 4)) * 4;
             const int64_t t = min(t0 + row, p.L - 1);
             kreg[i] = X::ld_raw(kb + t * p.ks.l + col);
             qreg[i] = X::ld_raw(qb + t * p.qs.l + col);
@@ -419,7 +431,7 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
         const bool full = t0 + C <= p.L;
 #pragma unroll
         for (int i = 0; i < NG; ++i) {
-            const int f = tid + i * kThreads, row = f / (D / 4), col = (f % (D / 4)) * 4;
+            const int f = tid + i * NT, row = f / (D / 4), col = (f % (D / 4)) * 4;
             const bool keep = full || t0 + row < p.L;
             const float m = keep ? 1.f : 0.f;
             X::st_raw(Gs, row, col, X::keep_raw(greg[i], keep));
@@ -428,7 +440,7 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
         }
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
-            const int f = tid + i * kThreads, row = f / (kWC / 4), col = (f % (kWC / 4)) * 4;
+            const int f = tid + i * NT, row = f / (kWC / 4), col = (f % (kWC / 4)) * 4;
             const bool keep = full || t0 + row < p.L;
             X::st_raw(Kw, row, col, X::keep_raw(kreg[i], keep));
             X::st_raw(Qw, row, col, X::keep_raw(qreg[i], keep));
@@ -445,15 +457,15 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
 
         // ---- G1 = tril(dOut U^T) and Z = X + X^T with X = strict_lower(Y U^T): NTRI pairs of tiles
         //      (a pair shares its right operand)
-        for (int pix = wave; pix < NTRI; pix += 4) {
+        for (int pix = wv; pix < NTRI; pix += 4 * KS) {
             int ci, cj;
             tri_index(pix, ci, cj);
             const auto fb = [&](int mb) { return X::ldb(Us, cj * 16 + ln, mb * 16 + 4 * lq); };
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
             const f32x4 accG = mma_range<X, false, true>(
-                0, MB, [&](int mb) { return X::lda(Gs, ci * 16 + ln, mb * 16 + 4 * lq); }, fb, zero);
+                0, MBF, [&](int mb) { return X::lda(Gs, ci * 16 + ln, mb * 16 + 4 * lq); }, fb, zero);
             const f32x4 accX = mma_range<X, true, true>(
-                0, MB, [&](int mb) { return X::lda(Ys, ci * 16 + ln, mb * 16 + 4 * lq); }, fb, zero);
+                0, MBF, [&](int mb) { return X::lda(Ys, ci * 16 + ln, mb * 16 + 4 * lq); }, fb, zero);
             const int col = cj * 16 + ln;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -485,7 +497,7 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
         for (int mb = 0; mb < MB; ++mb) {
             dstb[mb] = X::accb(dst[mb]);   // dS' (before this chunk's update)
             st[mb] = mma_range<X, true, false>(
-                0, CB, [&](int cb) { return X::lda_t(Us, cb * 16 + 4 * lq, mb * 16 + ln); },
+                0, CB, [&](int cb) { return X::lda_t(Us, cb * 16 + 4 * lq, m0 + mb * 16 + ln); },
                 [&](int cb) { return nkb[cb]; }, st[mb]);
             nstb[mb] = X::accb(-st[mb]);   // -S (entry value)
         }
@@ -493,19 +505,25 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
         __syncthreads();
 
         // ---- grad_Q = dOut S^T + G1 K,  grad_K = G1^T Q + U dS'^T - Y S^T - Z K
-#pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            const auto fns = [&](int mb) { return nstb[mb]; };
-            const auto fnk = [&](int b) { return nkb[b]; };
-            f32x4 dqn = mma_range<X, false, true>(
-                0, MB, [&](int mb) { return X::lda(Gs, cb * 16 + ln, mb * 16 + 4 * lq); }, fns, f32x4{0.f, 0.f, 0.f, 0.f});
+        const auto fns = [&](int mb) { return nstb[mb]; };
+        const auto fnk = [&](int b) { return nkb[b]; };
+        // the products over memory columns (this wave's columns), for row block cb of the chunk
+        const auto dq_state = [&](int cb) {
+            return mma_range<X, false, true>(
+                0, MB, [&](int mb) { return X::lda(Gs, cb * 16 + ln, m0 + mb * 16 + 4 * lq); }, fns,
+                f32x4{0.f, 0.f, 0.f, 0.f});
+        };
+        const auto dk_state = [&](int cb) {
+            const f32x4 a = mma_range<X, true, true>(
+                0, MB, [&](int mb) { return X::lda(Us, cb * 16 + ln, m0 + mb * 16 + 4 * lq); },
+                [&](int mb) { return dstb[mb]; }, f32x4{0.f, 0.f, 0.f, 0.f});
+            return mma_range<X, true, true>(
+                0, MB, [&](int mb) { return X::lda(Ys, cb * 16 + ln, m0 + mb * 16 + 4 * lq); }, fns, a);
+        };
+        // the products over the chunk's steps, added onto those, and the stores
+        const auto finish = [&](int cb, f32x4 dqn, f32x4 dk) {
             dqn = mma_range<X, true, false>(
                 0, cb + 1, [&](int b) { return X::lda(G1, cb * 16 + ln, b * 16 + 4 * lq); }, fnk, dqn);
-            f32x4 dk = mma_range<X, true, true>(
-                0, MB, [&](int mb) { return X::lda(Us, cb * 16 + ln, mb * 16 + 4 * lq); },
-                [&](int mb) { return dstb[mb]; }, f32x4{0.f, 0.f, 0.f, 0.f});
-            dk = mma_range<X, true, true>(
-                0, MB, [&](int mb) { return X::lda(Ys, cb * 16 + ln, mb * 16 + 4 * lq); }, fns, dk);
             dk = mma_range<X, true, false>(
                 cb, CB, [&](int b) { return X::lda_t(G1, b * 16 + 4 * lq, cb * 16 + ln); },
                 [&](int b) { return qbf[b]; }, dk);
@@ -520,15 +538,47 @@ __global__ __launch_bounds__(kThreads) void delta_bwd_chunk_row_kernel(ChunkBwdP
                     p.gK[o] = dk[r];
                 }
             }
+        };
+        if constexpr (KS == 1) {
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) finish(cb, dq_state(cb), dk_state(cb));
+        } else {
+            // wave hf finishes row blocks [hf*CBH, (hf+1)*CBH) of the chunk; `mine` / `theirs` are compile-time
+            // positions, the half they fall in is chosen by hf at run time
+            f32x4 pq[CB], pk[CB];
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) pq[cb] = dq_state(cb);
+#pragma unroll
+            for (int j = 0; j < CBH; ++j)   // partial grad_Q of the other wave's row blocks
+                Xs[(wv * CBH + j) * 64 + lane] = hf ? pq[j] : pq[CBH + j];
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) pk[cb] = dk_state(cb);
+            __syncthreads();
+            f32x4 oq[CBH];
+#pragma unroll
+            for (int j = 0; j < CBH; ++j) oq[j] = Xs[((wv ^ 4) * CBH + j) * 64 + lane];
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < CBH; ++j) Xs[(wv * CBH + j) * 64 + lane] = hf ? pk[j] : pk[CBH + j];
+            __syncthreads();
+            if (hf == 0) {
+#pragma unroll
+                for (int j = 0; j < CBH; ++j)
+                    finish(j, pq[j] + oq[j], pk[j] + Xs[((wv ^ 4) * CBH + j) * 64 + lane]);
+            } else {
+#pragma unroll
+                for (int j = 0; j < CBH; ++j)
+                    finish(CBH + j, pq[CBH + j] + oq[j], pk[CBH + j] + Xs[((wv ^ 4) * CBH + j) * 64 + lane]);
+            }
         }
         // ---- dS^T += dOut^T Q - Y^T K
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
             dst[mb] = mma_range<X, false, false>(
-                0, CB, [&](int cb) { return X::lda_t(Gs, cb * 16 + 4 * lq, mb * 16 + ln); },
+                0, CB, [&](int cb) { return X::lda_t(Gs, cb * 16 + 4 * lq, m0 + mb * 16 + ln); },
                 [&](int cb) { return qbf[cb]; }, dst[mb]);
             dst[mb] = mma_range<X, true, false>(
-                0, CB, [&](int cb) { return X::lda_t(Ys, cb * 16 + 4 * lq, mb * 16 + ln); },
+                0, CB, [&](int cb) { return X::lda_t(Ys, cb * 16 + 4 * lq, m0 + mb * 16 + ln); },
                 [&](int cb) { return nkb[cb]; }, dst[mb]);
         }
         __syncthreads();
@@ -567,14 +617,14 @@ int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
     hipError_t err = hipFuncSetAttribute((const void *)delta_bwd_chunk_col_kernel<TI, D, MS, KS>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds1);
     if (err != hipSuccess) return (int)err;
-    err = hipFuncSetAttribute((const void *)delta_bwd_chunk_row_kernel<TI, D, MS, C2>,
+    err = hipFuncSetAttribute((const void *)delta_bwd_chunk_row_kernel<TI, D, MS, C2, KS>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds2);
     if (err != hipSuccess) return (int)err;
     const int grid = p.N * p.H * MS;
     if (MS > 1)   // two workgroups of the column sweep add their parts of grad_beta
         hipLaunchKernelGGL(zero_words_kernel, dim3(256), dim3(256), 0, s, p.gbeta, (int64_t)p.N * p.H * p.L);
     hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS, KS>), dim3(grid), dim3(kThreads * KS), lds1, s, p);
-    hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2>), dim3(grid), dim3(kThreads), lds2, s, p);
+    hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2, KS>), dim3(grid), dim3(kThreads * KS), lds2, s, p);
     return (int)hipGetLastError();
 }
 
