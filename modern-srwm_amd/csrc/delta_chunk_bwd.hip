@@ -610,21 +610,22 @@ __global__ void zero_words_kernel(float *a, int64_t n) {
     for (int64_t j = i; j < n; j += stride) a[j] = 0.f;
 }
 
-template <class TI, int D, int MS, int C2, int KS>
+// KS: waves per memory row / column block in the column sweep, KSR: in the row sweep
+template <class TI, int D, int MS, int C2, int KS, int KSR>
 int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
     constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2>::kBytes;
     static_assert(lds1 <= (int)kMaxLdsBytes && lds2 <= (int)kMaxLdsBytes, "LDS budget");
     hipError_t err = hipFuncSetAttribute((const void *)delta_bwd_chunk_col_kernel<TI, D, MS, KS>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, lds1);
     if (err != hipSuccess) return (int)err;
-    err = hipFuncSetAttribute((const void *)delta_bwd_chunk_row_kernel<TI, D, MS, C2, KS>,
+    err = hipFuncSetAttribute((const void *)delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR>,
                               hipFuncAttributeMaxDynamicSharedMemorySize, lds2);
     if (err != hipSuccess) return (int)err;
     const int grid = p.N * p.H * MS;
     if (MS > 1)   // two workgroups of the column sweep add their parts of grad_beta
         hipLaunchKernelGGL(zero_words_kernel, dim3(256), dim3(256), 0, s, p.gbeta, (int64_t)p.N * p.H * p.L);
     hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS, KS>), dim3(grid), dim3(kThreads * KS), lds1, s, p);
-    hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2, KS>), dim3(grid), dim3(kThreads * KS), lds2, s, p);
+    hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR>), dim3(grid), dim3(kThreads * KSR), lds2, s, p);
     return (int)hipGetLastError();
 }
 
@@ -642,8 +643,8 @@ int dispatch_chunk_bwd(const ChunkBwdP<TI> &p, int D, hipStream_t s) {
         return -1;
     constexpr bool bf = PrecOf<TI>::type::kBf;
     switch (D) {
-        case 128: return launch_chunk_bwd<TI, 128, 2, bf ? 64 : 32, bf ? 2 : 1>(p, s);
-        case 64: return launch_chunk_bwd<TI, 64, 1, 64, 1>(p, s);
+        case 128: return launch_chunk_bwd<TI, 128, 2, bf ? 64 : 32, bf ? 2 : 1, 2>(p, s);
+        case 64: return launch_chunk_bwd<TI, 64, 1, 64, 1, 1>(p, s);
         default: return -1;
     }
 }
