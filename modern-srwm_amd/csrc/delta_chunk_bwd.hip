@@ -644,7 +644,7 @@ int dispatch_chunk_bwd(const ChunkBwdP<TI> &p, int D, hipStream_t s) {
     constexpr bool bf = PrecOf<TI>::type::kBf;
     switch (D) {
         case 128: return launch_chunk_bwd<TI, 128, 2, bf ? 64 : 32, bf ? 2 : 1, 2>(p, s);
-        case 64: return launch_chunk_bwd<TI, 64, 1, 64, 1, 1>(p, s);
+        case 64: return launch_chunk_bwd<TI, 64, 1, 64, 1, 2>(p, s);
         default: return -1;
     }
 }
