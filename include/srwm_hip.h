@@ -223,6 +223,14 @@ SRWM_API int srwm_readout_grad_f32(const float *k, const float *beta, const floa
                           const float *W_y_entry, float *grad_x,
                           int N, int H, int L, int E, unsigned flags, void *stream);
 
+/* The same for an output block Y columns wide (y_diff, grad_out: [N,H,L,Y]; W_y_entry: [N,H,E,Y];
+ * sW_y: [H,E,Y]); the forward of such an unroll is srwm_layer_forward_f32 with `keep`. */
+SRWM_API int srwm_readout_grad_wide_f32(const float *k, const float *beta, const float *y_diff,
+                               const float *keep, const float *sW_y,
+                               const float *grad_out, const int64_t grad_out_strides[3],
+                               const float *W_y_entry, float *grad_x,
+                               int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+
 /*
  * Delta-rule forward.  Replaces fast_weight_forward(), supervised_learning/
  * fast_weight/fast_weight_cuda.cu:182-240 (kernel :17-178).  Per sequence, W is E x M:

@@ -183,21 +183,29 @@ int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *kee
                                   kdiff, bdiff, out, N, H, L, E, E, flags, stream);
 }
 
-int srwm_readout_grad_f32(const float *k, const float *beta, const float *ydiff, const float *keep,
-                          const float *sWy, const float *grad_out, const int64_t gs[3],
-                          const float *Wy_entry, float *grad_x, int N, int H, int L, int E,
-                          unsigned flags, void *stream) {
+int srwm_readout_grad_wide_f32(const float *k, const float *beta, const float *ydiff, const float *keep,
+                               const float *sWy, const float *grad_out, const int64_t gs[3],
+                               const float *Wy_entry, float *grad_x, int N, int H, int L, int E, int Y,
+                               unsigned flags, void *stream) {
     if (!k || !beta || !ydiff || !grad_out || !gs || !Wy_entry || !grad_x || (keep && !sWy)) return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
-    if (!stride_ok(gs, N, H, L, E)) return SRWM_ESTRIDE;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    if (!stride_ok(gs, N, H, L, Y)) return SRWM_ESTRIDE;
     ReplayParams p{k, {(int64_t)H * L * E, (int64_t)L * E, E}, ydiff, beta, 4, keep, grad_out,
-                   {gs[0], gs[1], gs[2]}, Wy_entry, keep ? sWy : nullptr, grad_x, N, H, L, E, E};
+                   {gs[0], gs[1], gs[2]}, Wy_entry, keep ? sWy : nullptr, grad_x, N, H, L, E, Y};
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_replay_tiled(p, (hipStream_t)stream);
         if (r >= 0) return r;
     }
-    if (E > 256 || replay_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
+    if (E > 256 || Y > 256 || replay_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_replay(p, (hipStream_t)stream);
+}
+
+int srwm_readout_grad_f32(const float *k, const float *beta, const float *ydiff, const float *keep,
+                          const float *sWy, const float *grad_out, const int64_t gs[3],
+                          const float *Wy_entry, float *grad_x, int N, int H, int L, int E,
+                          unsigned flags, void *stream) {
+    return srwm_readout_grad_wide_f32(k, beta, ydiff, keep, sWy, grad_out, gs, Wy_entry, grad_x, N, H, L, E, E,
+                                      flags, stream);
 }
 
 int delta_forward_steps_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],

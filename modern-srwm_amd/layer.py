@@ -19,7 +19,7 @@ import torch.nn.functional as F
 
 from fast_weight import fast_weight_delta, fast_weight_delta_steps
 from self_ref_v0 import self_ref_layer, self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
-from self_ref_v1 import self_ref_v1
+from self_ref_v1 import self_ref_v1, self_ref_v1_steps
 
 
 # True: the SRWM layers run the fused layer operator (shared weights read directly, input softmax,
@@ -225,6 +225,27 @@ class SMFWPlayer(nn.Module):
         new_state = tuple((f.detach() - w.repeat(bsz, 1, 1, 1)).detach() for f, w in zip(fast, slow))
         # a copy: the delta-rule backward reverts `fast_weights` in place to its value at entry
         return out, new_state + (fast_weights.detach().clone(),)
+
+    def forward_steps(self, h, notdone, state):
+        """The whole unroll at once: equivalent to calling forward() once per time step on
+        h[t:t+1] with every part of the carried state multiplied by notdone[t] first, in one
+        launch per operator.  h: (T, B, H*d); notdone: (T, B), 0 where an episode ended."""
+        assert state is not None
+        slen, bsz, _ = h.size()
+        x = F.softmax(h.reshape(slen, bsz, self.num_head, self.dim_head), dim=-1).permute(1, 2, 0, 3)
+        keep = notdone.to(h.dtype).transpose(0, 1).contiguous()            # (B, T)
+        slow = (self.W_y, self.W_q, self.W_k, self.w_b)
+        *shift, fast_weights = state
+        fast = [s.detach() + w.detach().repeat(bsz, 1, 1, 1) for s, w in zip(shift, slow)]
+        qkvb = self_ref_v1_steps(x, keep, *fast, *slow)
+        q, k, v, beta = torch.split(qkvb, (self.dim_head,) * 3 + (1,), -1)
+        memory = fast_weights.detach().clone()
+        out = fast_weight_delta_steps(F.softmax(q, dim=-1), F.softmax(k, dim=-1), v, torch.sigmoid(beta),
+                                      keep, memory)
+        out = _heads_out(out, bsz, slen, self.num_head * self.dim_head)
+        out = h + self.drop(self.out_linear(out))
+        new_state = tuple(f - w.detach().repeat(bsz, 1, 1, 1) for f, w in zip(fast, slow))
+        return out, new_state + (memory,)
 
 
 class _DeltaBase(nn.Module):

@@ -125,12 +125,16 @@ class SelfRefv0Steps(torch.autograd.Function):
     def forward(ctx, x, keep, W_y, W_q, W_k, w_b, sW_y, sW_q, sW_k, sw_b):
         for t in (x, W_y, W_q, W_k, w_b):
             assert t.device.type != "cpu"
-        N, H, L, E = _check_shapes(x, W_y, W_q, W_k, w_b)
+        N, H, L, E = x.shape
+        Y = W_y.shape[-1]        # E, or 3E+1 for the wide-output variant
+        assert W_y.shape == (N, H, E, Y) and W_q.shape == (N, H, E, E) and W_k.shape == (N, H, E, E) \
+            and w_b.shape == (N, H, E, 4), "Reshape/unsqueeze if needed."
         device = x.device
         big = lambda: torch.empty((N, H, L, E), device=device, dtype=x.dtype)
+        wide = lambda: torch.empty((N, H, L, Y), device=device, dtype=x.dtype)
         small = lambda: torch.empty((N, H, L, 4), device=device, dtype=x.dtype)
-        out, q_main, k_main, beta_main = big(), big(), big(), small()
-        y_diff, q_diff, k_diff, beta_diff = big(), big(), big(), small()
+        out, q_main, k_main, beta_main = wide(), big(), big(), small()
+        y_diff, q_diff, k_diff, beta_diff = wide(), big(), big(), small()
         W_y_entry = W_y.detach().clone()
         srwm_hip.self_ref_forward_steps(x.data, keep, (sW_y, sW_q, sW_k, sw_b), W_y.data, W_q.data, W_k.data,
                                         w_b.data, q_main, k_main, beta_main, y_diff, q_diff, k_diff,

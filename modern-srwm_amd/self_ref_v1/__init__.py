@@ -62,3 +62,7 @@ class SelfRefv1(torch.autograd.Function):
 
 # Alias the autograd functions to python style snake case naming
 self_ref_v1 = SelfRefv1.apply
+
+# All time steps of an RL unroll in one launch (per-step resets, gradient cut at the carried state):
+# the step-mode operator of self_ref_v0 takes W_y of any width.
+from self_ref_v0 import self_ref_v0_steps as self_ref_v1_steps  # noqa: E402

@@ -52,6 +52,7 @@ _SIGNATURES = {
     "srwm_layer_forward_f32": [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_layer_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
+    "srwm_readout_grad_wide_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
     "delta_forward_steps_f32": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -211,9 +212,12 @@ def self_ref_forward_steps(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff
     """SRWM forward over all steps of an unroll with per-step resets: where keep[n, t] == 0 the
     state of batch row n is replaced, before step t, by the shared weights `slow` = (W_y, W_q,
     W_k: (1 or no batch axis, H, E, E), w_b: (..., H, E, 4)).  keep: (N, L) float32 or None.
-    Otherwise as self_ref_forward."""
+    Otherwise as self_ref_forward.  A W_y of another width (N, H, E, Y) selects the wide-output form."""
     _require(x, "x")
     N, H, L, E = x.shape
+    if isinstance(W_y, torch.Tensor) and W_y.dim() == 4 and W_y.shape[-1] != E:
+        return self_ref_layer_forward(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff,
+                                      beta_diff, out, flags=flags)
     for t, nm in ((W_y, "W_y"), (W_q, "W_q"), (W_k, "W_k")):
         _require(t, nm, (N, H, E, E))
     _require(w_b, "w_b", (N, H, E, 4))
@@ -251,27 +255,29 @@ def self_ref_readout_grad(k, beta, y_diff, keep, slow_W_y, grad_out, W_y_entry, 
     flags: FLAG_GENERIC forces the LDS-resident kernel."""
     _require(k, "k")
     N, H, L, E = k.shape
+    _require(y_diff, "y_diff")
+    Y = y_diff.shape[-1]                      # width of the output block (E, or 3E+1 for the wide variant)
     _require(beta, "beta", (N, H, L, 4))
-    _require(y_diff, "y_diff", (N, H, L, E))
-    _require(grad_out, "grad_out", (N, H, L, E))
-    _require(W_y_entry, "W_y_entry", (N, H, E, E))
+    _require(y_diff, "y_diff", (N, H, L, Y))
+    _require(grad_out, "grad_out", (N, H, L, Y))
+    _require(W_y_entry, "W_y_entry", (N, H, E, Y))
     _require(grad_x, "grad_x", (N, H, L, E))
     null = ctypes.c_void_p(None)
     if keep is not None:
         _require(keep, "keep", (N, L))
         keep = keep.contiguous()
-        slow_W_y = slow_W_y.detach().reshape(H, E, E).contiguous()
-        _require(slow_W_y, "slow W_y", (H, E, E))
+        slow_W_y = slow_W_y.detach().reshape(H, E, Y).contiguous()
+        _require(slow_W_y, "slow W_y", (H, E, Y))
     if k.numel() == 0:
         return
     gos, gstr = _strided(grad_out)
     with torch.cuda.device(k.device), _Dense([k, beta, y_diff, W_y_entry], False) as sv, \
             _Dense([grad_x], True) as gr:
-        code = lib().srwm_readout_grad_f32(
+        code = lib().srwm_readout_grad_wide_f32(
             _ptr(sv[0]), _ptr(sv[1]), _ptr(sv[2]), _ptr(keep) if keep is not None else null,
             _ptr(slow_W_y) if keep is not None else null, _ptr(gos), gstr, _ptr(sv[3]), _ptr(gr[0]),
-            N, H, L, E, flags, _stream(k.device))
-    _check(code, "srwm_readout_grad_f32")
+            N, H, L, E, Y, flags, _stream(k.device))
+    _check(code, "srwm_readout_grad_wide_f32")
 
 
 def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out,

@@ -287,3 +287,45 @@ def test_self_modifying_fwp_layer():
         assert all(not s.requires_grad for s in state)
         for s, r in zip(state, ref_state):
             assert (s.cpu().double() - r).abs().max().item() < 2e-5 * max(1.0, r.abs().max().item())
+
+
+def test_rl_self_modifying_layer_whole_unroll_equals_the_per_step_loop():
+    """SMFWPlayer.forward_steps (one launch per operator) vs the per-step loop over forward() with
+    every part of the state multiplied by notdone first."""
+    print("case SMFWPlayer.forward_steps", flush=True)
+    from layer import SMFWPlayer
+    dev = torch.device("cuda:0")
+    torch.manual_seed(8)
+    T, B, H, d = 17, 4, 4, 16
+    lay = SMFWPlayer(H, d, H * d, 0.0).to(dev)
+    h = torch.randn(T, B, H * d, device=dev)
+    notdone = (torch.rand(T, B, device=dev) > 0.2).float()
+    state0 = tuple(0.1 * torch.randn(B, H, d, c, device=dev) for c in (3 * d + 1, d, d, 4, d))
+    go = torch.randn(T, B, H * d, device=dev)
+
+    hl = h.clone().requires_grad_(True)
+    outs, state = [], state0
+    for t in range(T):
+        nd = notdone[t].view(B, 1, 1, 1)
+        state = tuple(s * nd for s in state)
+        o, state = lay(hl[t:t + 1], state)
+        outs.append(o)
+    loop_out = torch.cat(outs)
+    (loop_out * go).sum().backward()
+    loop_grads = {n: p.grad.clone() for n, p in lay.named_parameters() if p.grad is not None}
+    loop_gh = hl.grad.clone()
+    lay.zero_grad()
+
+    hs = h.clone().requires_grad_(True)
+    out, new_state = lay.forward_steps(hs, notdone, state0)
+    (out * go).sum().backward()
+    scale = loop_out.abs().max().item()
+    assert (out - loop_out).abs().max().item() < 2e-5 * scale
+    for a, b in zip(new_state, state):
+        assert (a - b).abs().max().item() < 2e-5 * max(1.0, b.abs().max().item())
+    assert (hs.grad - loop_gh).abs().max().item() < 2e-5 * loop_gh.abs().max().item()
+    for n, p in lay.named_parameters():
+        if n in loop_grads:
+            ref = loop_grads[n]
+            got = p.grad if p.grad is not None else torch.zeros_like(ref)
+            assert (got - ref).abs().max().item() < 2e-5 * max(1e-6, ref.abs().max().item()), n
