@@ -593,8 +593,21 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             float dqk[2] = {gq * qb, gk * kb};
             group_sum_n<E, 2>(dqk);
             const float gpq = qb * (gq - dqk[0]), gpk = kb * (gk - dqk[1]);
-            float gb[4];
-            {
+            float gpreb;
+            if constexpr (E == kWave && !XC) {
+                // jb == wave: a wave only needs the beta gradient of its own w_b column, one sum instead of three
+                float gbw;
+                if (jb < 3) {
+                    gbw = group_sum<NCG>(gbp[lane % NCG][jb]);
+                } else {
+                    float p3[4];
+                    lds_read_vec<4>(p3, &gbp3[0]);
+                    gbw = (p3[0] + p3[1]) + (p3[2] + p3[3]);
+                }
+                const float btw = bt[jb & 3];
+                gpreb = gbw * btw * (1.f - btw);
+            } else {
+                float gb[4];
                 float part[4];
                 lds_read_vec<4>(part, &gbp[lane % NCG][0]);
                 float p012[3] = {part[0], part[1], part[2]};
@@ -605,11 +618,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 lds_read_vec<4>(p3, &gbp3[0]);
                 gb[3] = (p3[0] + p3[1]) + (p3[2] + p3[3]);
                 if constexpr (XC) gb[0] += gbp3[4];
-            }
-            float gpb[4];
+                float gpb[4];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) gpb[j] = gb[j] * bt[j] * (1.f - bt[j]);
-            const float gpreb = jb == 0 ? gpb[0] : jb == 1 ? gpb[1] : jb == 2 ? gpb[2] : gpb[3];
+                for (int j = 0; j < 4; ++j) gpb[j] = gb[j] * bt[j] * (1.f - bt[j]);
+                gpreb = jb == 0 ? gpb[0] : jb == 1 ? gpb[1] : jb == 2 ? gpb[2] : gpb[3];
+            }
             if (lane < E) {
                 exch[wave][0][lane] = gpq;
                 exch[wave][1][lane] = gpk;
