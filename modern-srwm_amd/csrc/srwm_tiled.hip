@@ -174,6 +174,12 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     auto load_keep = [&](int tile) -> float {
         return (RESET && p.keep && tid < TT) ? p.keep[(int64_t)n * p.L + min(tile * TT + tid, p.L - 1)] : 1.f;
     };
+    // outputs of this sequence: uniform bases, 32-bit offsets per step
+    float *const out_s = p.out + seq * p.L * Y, *const ydiff_s = p.ydiff + seq * p.L * Y;
+    uint16_t *const out16_s = reinterpret_cast<uint16_t *>(p.out) + seq * p.L * Y;
+    float *const q_s = p.q + seq * p.L * E, *const k_s = p.k + seq * p.L * E;
+    float *const qdiff_s = p.qdiff + seq * p.L * E, *const kdiff_s = p.kdiff + seq * p.L * E;
+    float *const beta_s = p.beta + seq * p.L * 4, *const bdiff_s = p.bdiff + seq * p.L * 4;
     const int ntiles = (p.L + TT - 1) / TT;
     {
         const float4 x0 = load_tile(0);
@@ -194,7 +200,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 
         for (int tt = 0; tt < tlen; ++tt) {
             const int t = tile * TT + tt, par = t & 1;
-            const int64_t o = (seq * p.L + t) * E, oy = (seq * p.L + t) * Y, ob = (seq * p.L + t) * 4;
+            const int o = t * E, oy = t * Y, ob = t * 4;   // offsets inside the sequence (the launcher bounds L * Y)
             if constexpr (RESET) {
                 if (kt[buf][tt] == 0.f) reset_state();   // uniform over the workgroup
             }
@@ -214,13 +220,13 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             const float pb = group_sum<E>(wbe * xb);
             if (rg == 0) {
                 if (bf16_io) {
-                    uint16_t *o16 = reinterpret_cast<uint16_t *>(p.out) + oy;
+                    uint16_t *o16 = out16_s + oy;
 #pragma unroll
                     for (int b = 0; b < YB; ++b)
 #pragma unroll
                         for (int c = 0; c < CB; ++c) o16[b * E + c0 + c] = f32_to_bf16_bits(acc[b * CB + c]);
                 } else {
-                    store_y(p.out + oy, &acc[0]);
+                    store_y(out_s + oy, &acc[0]);
                 }
                 store_vec<CB>(&raw[par][0][c0], &acc[QB]);
                 store_vec<CB>(&raw[par][1][c0], &acc[KB]);
@@ -229,8 +235,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             if constexpr (XC) {
                 const float py = group_sum<E>(wye * xb);
                 if (has_y && el == 0) {
-                    if (bf16_io) reinterpret_cast<uint16_t *>(p.out)[oy + YB * E] = f32_to_bf16_bits(py);
-                    else p.out[oy + YB * E] = py;
+                    if (bf16_io) out16_s[oy + YB * E] = f32_to_bf16_bits(py);
+                    else out_s[oy + YB * E] = py;
                 }
             }
             if (tt == tlen - 1 && tile + 1 < ntiles) {
@@ -254,10 +260,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
                                  quad_broadcast<3>(sg)};
             const float dv = qn - kn;
             if (wave == 0 && lane < E) {
-                p.q[o + lane] = qn;
-                p.k[o + lane] = kn;
+                q_s[o + lane] = qn;
+                k_s[o + lane] = kn;
             }
-            if (wave == NW - 1 && lane < 4) p.beta[ob + lane] = sg;
+            if (wave == NW - 1 && lane < 4) beta_s[ob + lane] = sg;
             if (lane < E) {
                 exch[wave][0][lane] = dv;
                 exch[wave][1][lane] = kn;
@@ -278,11 +284,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             group_sum_n<RG, NC>(dif);
             const float pbd = group_sum<E>(wbe * dv);
             if (rg == 0) {
-                store_y(p.ydiff + oy, &dif[0]);
-                store_vec<CB>(p.qdiff + o + c0, &dif[QB]);
-                store_vec<CB>(p.kdiff + o + c0, &dif[KB]);
+                store_y(ydiff_s + oy, &dif[0]);
+                store_vec<CB>(qdiff_s + o + c0, &dif[QB]);
+                store_vec<CB>(kdiff_s + o + c0, &dif[KB]);
             }
-            if (has_b && el == 0) p.bdiff[ob + jb] = pbd;
+            if (has_b && el == 0) bdiff_s[ob + jb] = pbd;
 
             // ---- rank-1 write W += k (x) (beta_blk * diff); every y block uses beta_y
             float ins[NC];
@@ -295,7 +301,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             wbe = fmaf(kn, bt[3] * pbd, wbe);
             if constexpr (XC) {
                 const float pyd = group_sum<E>(wye * dv);
-                if (has_y && el == 0) p.ydiff[oy + YB * E] = pyd;
+                if (has_y && el == 0) ydiff_s[oy + YB * E] = pyd;
                 wye = fmaf(kn, bt[0] * pyd, wye);
             }
         }
@@ -725,6 +731,7 @@ bool aligned16(const void *ptr, int64_t a, int64_t b, int64_t c) {
 }  // namespace
 
 int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
+    if ((int64_t)p.L * (p.Y > p.E ? p.Y : p.E) >= ((int64_t)1 << 29)) return -1;   // 32-bit offsets inside a sequence
     if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l)) return -1;
     const void *dense[] = {p.q, p.k, p.beta, p.ydiff, p.qdiff, p.kdiff, p.bdiff, p.out};
     for (const void *d : dense)
