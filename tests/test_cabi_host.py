@@ -33,6 +33,36 @@ def test_library_exports_every_declared_symbol():
     assert srwm_hip.lib().srwm_hip_abi_version() == srwm_hip.ABI_VERSION
 
 
+def _prototypes():
+    """name -> list of parameter declarations, parsed from the header."""
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    text = "\n".join(line for line in text.split("\n") if not line.lstrip().startswith("#"))
+    out = {}
+    for m in re.finditer(r"SRWM_API\s+(?:const\s+)?\w+\s*\*?\s*(\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S):
+        params = [p.strip() for p in m.group(2).split(",")]
+        out[m.group(1)] = [] if params == ["void"] else params
+    return out
+
+
+def test_ctypes_signatures_match_the_header():
+    """The host layer binds every compute entry point with the parameter list the header declares:
+    same count, pointers where the header has pointers or arrays, ints where it has ints."""
+    import srwm_hip
+    protos = _prototypes()
+    aux = {"srwm_hip_abi_version", "srwm_hip_strerror", "srwm_hip_limits", "srwm_hip_lds_probe"}
+    assert set(protos) - aux == set(srwm_hip._SIGNATURES), set(protos) - aux ^ set(srwm_hip._SIGNATURES)
+    for name, args in srwm_hip._SIGNATURES.items():
+        params = protos[name]
+        assert len(params) == len(args), (name, len(params), len(args))
+        for decl, ct in zip(params, args):
+            if "*" in decl or "[" in decl:
+                assert ct in (ctypes.c_void_p, srwm_hip._S), (name, decl)
+            elif decl.startswith("unsigned"):
+                assert ct is ctypes.c_uint, (name, decl)
+            else:
+                assert decl.startswith("int ") and ct is ctypes.c_int, (name, decl)
+
+
 def test_error_strings():
     import srwm_hip
     L = srwm_hip.lib()
