@@ -87,6 +87,8 @@ __global__ __launch_bounds__(kThreads) void replay_kernel(ReplayParams p) {
 
 // Register-resident replay.  NWV waves per sequence; wave w owns rows [w*ER, (w+1)*ER), ER = E/NWV.
 // Inside a wave, CGL consecutive lanes share a block of R rows and split its M columns (CB each).
+typedef float v4f __attribute__((ext_vector_type(4)));
+
 template <int E, int M, int NWV, int CGL>
 __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p) {
     constexpr int ER = E / NWV, RGL = kWave / CGL, R = ER / RGL, CB = M / CGL;
@@ -120,54 +122,36 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
     load_w(p.W0 + seq * E * M);
     const float *wreset = p.Wreset ? p.Wreset + (int64_t)h * E * M : nullptr;
 
-    // next tile, staged in registers: rows past the end are clamped (loaded, never used)
-    float4 ng[NG], nb[NG], na[NA];
+    // Next tile, staged in registers; rows past the end are clamped (loaded, never used).  The loop
+    // starts one tile early so that fetch and commit each appear once in the code: with two call
+    // sites the staging arrays end up in scratch memory instead of registers.
+    v4f ng[NG], nb[NG], na[NA];   // native vectors: arrays of HIP float4 structs are not kept in registers here
     float ns = 1.f, nk = 1.f;
-    auto fetch = [&](int tile) {
-#pragma unroll
-        for (int i = 0; i < NG; ++i) {
-            const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
-            const int64_t t = min(tile * TT + row, p.L - 1);
-            ng[i] = *reinterpret_cast<const float4 *>(gb + t * p.gs.l + col);
-            nb[i] = *reinterpret_cast<const float4 *>(bb + t * M + col);
-        }
-#pragma unroll
-        for (int i = 0; i < NA; ++i) {
-            const int f = lane + i * kWave, row = f / (ER / 4), col = (f % (ER / 4)) * 4;
-            const int64_t t = min(tile * TT + row, p.L - 1);
-            na[i] = *reinterpret_cast<const float4 *>(ab + t * p.as.l + col);
-        }
-        if (lane < TT) {
-            const int64_t t = min(tile * TT + lane, p.L - 1);
-            ns = p.bscale ? p.bscale[(seq * p.L + t) * p.bscale_stride] : 1.f;
-            nk = p.keep ? p.keep[(int64_t)n * p.L + t] : 1.f;
-        }
-    };
-    auto commit = [&]() {
-#pragma unroll
-        for (int i = 0; i < NG; ++i) {
-            const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
-            *reinterpret_cast<float4 *>(&tg[wave][row][col]) = ng[i];
-            *reinterpret_cast<float4 *>(&tb[wave][row][col]) = nb[i];
-        }
-#pragma unroll
-        for (int i = 0; i < NA; ++i) {
-            const int f = lane + i * kWave, row = f / (ER / 4), col = (f % (ER / 4)) * 4;
-            *reinterpret_cast<float4 *>(&ta[wave][row][col]) = na[i];
-        }
-        if (lane < TT) {
-            tsk[wave][0][lane] = ns;
-            tsk[wave][1][lane] = nk;
-        }
-    };
-
     const int ntiles = (p.L + TT - 1) / TT;
-    fetch(0);
-    commit();
-    wave_lds_fence();
-    for (int tile = 0; tile < ntiles; ++tile) {
-        const int tlen = min(TT, p.L - tile * TT);
-        if (tile + 1 < ntiles) fetch(tile + 1);
+    for (int tile = -1; tile < ntiles; ++tile) {
+        const bool more = tile + 1 < ntiles;
+        if (more) {   // fetch tile + 1
+            const int tb0 = (tile + 1) * TT;
+#pragma unroll
+            for (int i = 0; i < NG; ++i) {
+                const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
+                const int64_t t = min(tb0 + row, p.L - 1);
+                ng[i] = *reinterpret_cast<const v4f *>(gb + t * p.gs.l + col);
+                nb[i] = *reinterpret_cast<const v4f *>(bb + t * M + col);
+            }
+#pragma unroll
+            for (int i = 0; i < NA; ++i) {
+                const int f = lane + i * kWave, row = f / (ER / 4), col = (f % (ER / 4)) * 4;
+                const int64_t t = min(tb0 + row, p.L - 1);
+                na[i] = *reinterpret_cast<const v4f *>(ab + t * p.as.l + col);
+            }
+            if (lane < TT) {
+                const int64_t t = min(tb0 + lane, p.L - 1);
+                ns = p.bscale ? p.bscale[(seq * p.L + t) * p.bscale_stride] : 1.f;
+                nk = p.keep ? p.keep[(int64_t)n * p.L + t] : 1.f;
+            }
+        }
+        const int tlen = tile < 0 ? 0 : min(TT, p.L - tile * TT);
         for (int tt = 0; tt < tlen; ++tt) {
             const int t = tile * TT + tt;
             if (tsk[wave][1][tt] == 0.f) load_w(wreset);   // uniform over the wave
@@ -202,9 +186,23 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
 #pragma unroll
                 for (int c = 0; c < CB; ++c) w[i][c] = fmaf(av[i], bv[c], w[i][c]);
         }
-        if (tile + 1 < ntiles) {
-            wave_lds_fence();   // this wave's reads of the tile are done
-            commit();
+        if (more) {   // commit tile + 1
+            wave_lds_fence();   // this wave's reads of the current tile are done
+#pragma unroll
+            for (int i = 0; i < NG; ++i) {
+                const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
+                *reinterpret_cast<v4f *>(&tg[wave][row][col]) = ng[i];
+                *reinterpret_cast<v4f *>(&tb[wave][row][col]) = nb[i];
+            }
+#pragma unroll
+            for (int i = 0; i < NA; ++i) {
+                const int f = lane + i * kWave, row = f / (ER / 4), col = (f % (ER / 4)) * 4;
+                *reinterpret_cast<v4f *>(&ta[wave][row][col]) = na[i];
+            }
+            if (lane < TT) {
+                tsk[wave][0][lane] = ns;
+                tsk[wave][1][lane] = nk;
+            }
             wave_lds_fence();
         }
     }
