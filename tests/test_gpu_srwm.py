@@ -524,3 +524,11 @@ def test_replay_kernels_agree_and_match_a_numpy_replay(E, NH, L):
         u = torch.full((N, H, L, E), float("nan"), device=dev)
         srwm_hip.fast_weight_readout_replay(f32(a), f32(b), f32(keep), go_l, f32(W0), u, flags=flags)
         assert rel_err(u.cpu().numpy(), u_ref) < TOL, flags
+
+
+def test_long_sequence_reversal_stays_within_tolerance():
+    """L = 4096 (8x the headline length): the backward reverts the state through 4096 fp32 rank-1
+    writes; outputs, final state and gradients must still meet the 1e-5 bar."""
+    print("case long sequence", flush=True)
+    x, W, go = srwm_inputs(1, 2, 4096, 64, seed=0, w_std=0.02, per_batch_state=True)
+    check_against_oracle(x, W, go, 0)
