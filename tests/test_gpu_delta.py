@@ -214,6 +214,7 @@ def test_bf16_io_matches_oracle_on_rounded_inputs(shape, qk):
     ((1, 2, 2048, 128, 128), "l2", 0.0, torch.float32),      # 32 chunks in a row
     ((2, 8, 256, 64, 64), "softmax", 0.0, torch.float32),    # benchmark configuration 2 style
     ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # benchmark configuration 5 style, shorter
+    ((2, 2, 200, 64, 64), "softmax", 0.2, torch.bfloat16),   # bf16 at D = 64 (four waves, one workgroup per sequence)
 ])
 def test_chunkwise_forward_matches_oracle_and_feeds_the_sequential_backward(shape, qk, w0, io):
     """Chunkwise (C = 64) MFMA forward vs the fp64 oracle, then the step-by-step backward run on
