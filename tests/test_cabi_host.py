@@ -109,3 +109,41 @@ def test_host_layer_uses_no_oracle_and_no_torch_math():
             if f.endswith((".py", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "import oracle" not in text and "from oracle" not in text, f
+
+
+def test_argument_validation_needs_no_gpu():
+    """Every entry point rejects bad arguments before it touches the device, so the checks can be
+    exercised here with placeholder pointers that are never dereferenced (all calls below return a
+    negative code; nothing is launched)."""
+    import srwm_hip
+    L = srwm_hip.lib()
+    P = ctypes.c_void_p
+    fake = lambda: P(0x1000)                      # non-null, 16-byte aligned, never read
+    ok_strides = (ctypes.c_int64 * 3)(64 * 16, 16, 16 * 8)
+    huge = (ctypes.c_int64 * 3)(1 << 41, 16, 16)
+    N, H, Ls, E = 2, 8, 4, 16
+    srwm_f = lambda x, xs, n, e, flags: L.srwm_forward_f32(x, xs, *[fake() for _ in range(12)], n, H, Ls, e, flags, P(None))
+    assert srwm_f(P(None), ok_strides, N, E, 0) == -1          # SRWM_EINVAL: null input
+    assert srwm_f(fake(), None, N, E, 0) == -1                 # null stride array
+    assert srwm_f(fake(), ok_strides, 0, E, 0) == -1           # empty batch
+    assert srwm_f(fake(), ok_strides, N, -3, 0) == -1          # negative head size
+    assert srwm_f(fake(), ok_strides, N, E, 32) == -1          # the chunkwise flag means nothing to the SRWM
+    assert srwm_f(fake(), ok_strides, N, E, 1 << 20) == -1     # unknown flag bit
+    assert srwm_f(fake(), huge, N, E, 0) == -3                 # SRWM_ESTRIDE: extent overflows the 2^40 bound
+    assert srwm_f(fake(), ok_strides, N, 4096, 0) == -2        # SRWM_ESIZE: 4096 x 12292 floats fit no CU
+    srwm_b = lambda flags: L.srwm_backward_f32(fake(), ok_strides, *[fake() for _ in range(7)], fake(), ok_strides,
+                                               *[fake() for _ in range(9)], N, H, Ls, E, flags, P(None))
+    assert srwm_b(3) == -1                                     # grad-state mode 3 does not exist
+    delta_f = lambda flags, m: L.delta_forward_f32(*[a for _ in range(4) for a in (fake(), ok_strides)],
+                                                   *[fake() for _ in range(4)], N, H, Ls, E, m, flags, P(None))
+    assert delta_f(16 | 32, E) == -1                           # generic and chunkwise exclude each other
+    assert delta_f(0, 0) == -1                                 # value width 0
+    assert delta_f(32, E) == -4                                # SRWM_ENOKERNEL: no chunkwise kernel for E = M = 16
+    delta_b = lambda gW, flags: L.delta_backward_f32(*[a for _ in range(4) for a in (fake(), ok_strides)],
+                                                     fake(), fake(), fake(), ok_strides, fake(), fake(), fake(), fake(),
+                                                     fake(), gW, N, H, Ls, E, E, flags, P(None))
+    assert delta_b(P(None), 1) == -1                           # an incoming state gradient needs the buffer
+    layer_f = lambda sw, flags: L.srwm_layer_forward_f32(fake(), ok_strides, P(None), sw, sw, sw, sw,
+                                                         *[fake() for _ in range(12)], N, H, Ls, E, E, flags, P(None))
+    assert layer_f(P(None), 64) == -1                          # the shift form needs the shared weights
+    assert layer_f(P(None), 128) == -1                         # so does a fresh start
