@@ -290,6 +290,35 @@ __device__ __forceinline__ float ld_in(const uint16_t *p) { return __uint_as_flo
 __device__ __forceinline__ void st_out(float *p, float v) { *p = v; }
 __device__ __forceinline__ void st_out(uint16_t *p, float v) { *p = (uint16_t)f2bf_rne(v); }
 
+// Inverse of a unit triangular 16 x 16 matrix T = I - M on the matrix cores.  M is strictly
+// triangular, so M^16 = 0 and T^-1 = I + M + ... + M^15 = (I + M)(I + M^2)(I + M^4)(I + M^8): three
+// squarings and three multiply-adds instead of a 16-step substitution.  An accumulator tile
+// converts directly into a right operand (accb); the same registers, read as a LEFT operand,
+// are the left operand of the TRANSPOSED matrix (lane <-> column of the tile <-> row of its
+// transpose).  So the powers P and the partial products R are carried together with their
+// transposes, and each stage is four products (two in the last one).
+// m, mt: accumulator tiles of M and M^T (register r <-> row 4*(lane/16) + r, lane % 16 <-> column).
+template <class X>
+__device__ __forceinline__ f32x4 tri_inverse16(const f32x4 &m, const f32x4 &mt) {
+    const int ln = threadIdx.x & 15, lq = (threadIdx.x & 63) >> 4;
+    const auto as_a = [](const typename X::B &b) { return __builtin_bit_cast(typename X::A, b); };
+    f32x4 id;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) id[r] = (4 * lq + r == ln) ? 1.f : 0.f;
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    f32x4 p = m, pt = mt, res = id + m, rest = id + mt;
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+        const typename X::B pb = X::accb(p), ptb = X::accb(pt);
+        p = X::template mma<true, true>(as_a(ptb), pb, zero);                    // P^2
+        if (s < 2) pt = X::template mma<true, true>(as_a(pb), ptb, zero);        // (P^T)^2
+        const typename X::B p2b = X::accb(p), rtb = X::accb(rest);
+        res = X::template mma<true, true>(as_a(rtb), p2b, res);                  // R += R P^2
+        if (s < 2) rest = X::template mma<true, true>(as_a(p2b), rtb, rest);     // R^T += (P^2)^T R^T
+    }
+    return res;
+}
+
 // acc += sum over g in [lo, hi) of fa(g) * fb(g), g numbering groups of 16 contraction indices;
 // two groups per instruction where they pair up.  Meant to be inlined into unrolled code (lo
 // and hi compile-time constants there).

@@ -185,19 +185,36 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
         // ---- inverse of the diagonal block `wave` of I + diag(beta) strict_lower(A):
         //      column ln of X, x_i = [i == ln] - sum_{j<i} beta_i A_ij x_j
         if (hf == 0) {
-            float x[16];
             const float *ad = Ad + (wave * 16) * LDD;
+            if constexpr (X::kBf) {
+                // on the matrix cores: T = I - M with M_ij = -beta_i A_ij for j < i
+                const float4 row = *reinterpret_cast<const float4 *>(ad + ln * LDD + 4 * lq);
+                const float rv[4] = {row.x, row.y, row.z, row.w};
+                const float bl = bts[wave * 16 + ln];
+                f32x4 m, mt;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float acc = (i == ln) ? 1.f : 0.f;
-                const float bi = bts[wave * 16 + i];
+                for (int r = 0; r < 4; ++r) {
+                    const int i = 4 * lq + r;
+                    m[r] = ln < i ? -bts[wave * 16 + i] * ad[i * LDD + ln] : 0.f;   // M[i][ln]
+                    mt[r] = i < ln ? -bl * rv[r] : 0.f;                             // M[ln][i]
+                }
+                const f32x4 inv = tri_inverse16<X>(m, mt);
 #pragma unroll
-                for (int j = 0; j < i; ++j) acc = fmaf(-bi * ad[i * LDD + j], x[j], acc);
-                x[i] = acc;
+                for (int r = 0; r < 4; ++r) X::st(Di, wave * 16 + 4 * lq + r, ln, inv[r]);
+            } else {
+                float x[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    float acc = (i == ln) ? 1.f : 0.f;
+                    const float bi = bts[wave * 16 + i];
+#pragma unroll
+                    for (int j = 0; j < i; ++j) acc = fmaf(-bi * ad[i * LDD + j], x[j], acc);
+                    x[i] = acc;
+                }
+                // lanes 16..63 hold copies of columns 0..15: everybody stores, no branch
+#pragma unroll
+                for (int i = 0; i < 16; ++i) X::st(Di, wave * 16 + i, ln, x[i]);
             }
-            // lanes 16..63 hold copies of columns 0..15: everybody stores, no branch
-#pragma unroll
-            for (int i = 0; i < 16; ++i) X::st(Di, wave * 16 + i, ln, x[i]);
         }
 
         // ---- P = K S and Q S for this wave's 16 columns: independent of the inversion above
