@@ -16,8 +16,8 @@
 // same assignment, which makes its four values one 16-byte LDS read.  So S, U and the right
 // hand sides go from accumulator to operand without touching LDS.
 // Per chunk: A and B tiles (lower triangle only) are produced cooperatively and shared through
-// LDS, the four 16x16 diagonal blocks of I + L are inverted by forward substitution (one per
-// wave), then each wave runs the block forward substitution and all products for its own
+// LDS, the four 16x16 diagonal blocks of I + L are inverted on the matrix cores (one per wave,
+// tri_inverse16), then each wave runs the block forward substitution and all products for its own
 // columns with no further synchronisation.
 //
 // The backward of a chunkwise forward is the sequential reverse sweep of delta_tiled.hip (it
@@ -182,43 +182,26 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
         }
         __syncthreads();
 
-        // ---- inverse of the diagonal block `wave` of I + diag(beta) strict_lower(A):
-        //      column ln of X, x_i = [i == ln] - sum_{j<i} beta_i A_ij x_j
+        // ---- inverse of the diagonal block `wave` of I + diag(beta) strict_lower(A), on the matrix
+        //      cores: T = I - M with M_ij = -beta_i A_ij for j < i
         if (hf == 0) {
             const float *ad = Ad + (wave * 16) * LDD;
-            if constexpr (X::kBf) {
-                // on the matrix cores: T = I - M with M_ij = -beta_i A_ij for j < i
-                const float4 row = *reinterpret_cast<const float4 *>(ad + ln * LDD + 4 * lq);
-                const float rv[4] = {row.x, row.y, row.z, row.w};
-                const float bl = bts[wave * 16 + ln];
-                f32x4 m, mt;
+            const float4 row = *reinterpret_cast<const float4 *>(ad + ln * LDD + 4 * lq);
+            const float rv[4] = {row.x, row.y, row.z, row.w};
+            const float bl = bts[wave * 16 + ln];
+            f32x4 m, mt;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 4 * lq + r;
-                    m[r] = ln < i ? -bts[wave * 16 + i] * ad[i * LDD + ln] : 0.f;   // M[i][ln]
-                    mt[r] = i < ln ? -bl * rv[r] : 0.f;                             // M[ln][i]
-                }
-                const f32x4 inv = tri_inverse16<X>(m, mt);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) X::st(Di, wave * 16 + 4 * lq + r, ln, inv[r]);
-            } else {
-                float x[16];
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    float acc = (i == ln) ? 1.f : 0.f;
-                    const float bi = bts[wave * 16 + i];
-#pragma unroll
-                    for (int j = 0; j < i; ++j) acc = fmaf(-bi * ad[i * LDD + j], x[j], acc);
-                    x[i] = acc;
-                }
-                // lanes 16..63 hold copies of columns 0..15: everybody stores, no branch
-#pragma unroll
-                for (int i = 0; i < 16; ++i) X::st(Di, wave * 16 + i, ln, x[i]);
+            for (int r = 0; r < 4; ++r) {
+                const int i = 4 * lq + r;
+                m[r] = ln < i ? -bts[wave * 16 + i] * ad[i * LDD + ln] : 0.f;   // M[i][ln]
+                mt[r] = i < ln ? -bl * rv[r] : 0.f;                             // M[ln][i]
             }
+            const f32x4 inv = tri_inverse16<X>(m, mt);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) X::st(Di, wave * 16 + 4 * lq + r, ln, inv[r]);
         }
 
         // ---- P = K S and Q S for this wave's 16 columns: independent of the inversion above
-        //      (matrix-core work that can overlap its vector-ALU chain)
         f32x4 pt[kCB], ot[kCB], u[kCB];
         {
             typename X::B sb[EB];

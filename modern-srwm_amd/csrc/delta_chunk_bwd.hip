@@ -16,7 +16,7 @@
 // two sweeps with the memory tiled the other way round:
 //   column sweep  a wave owns 16 columns of S and dS (rows in the registers); it solves the
 //                 upper triangular system by 16-row block back substitution (diagonal blocks
-//                 inverted on the vector ALUs, one per wave) and writes grad_V and grad_beta;
+//                 inverted on the matrix cores, one per wave) and writes grad_V and grad_beta;
 //   row sweep     a wave owns 16 rows of S and dS, held transposed (columns in the registers);
 //                 it reads grad_V back, forms G1 and X cooperatively and writes grad_Q, grad_K,
 //                 the reverted memory and the gradient of the initial memory.  Every word of
@@ -221,37 +221,23 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
         }
         __syncthreads();
 
-        // ---- inverse of the diagonal block `wave` of I + A^T diag(beta) (unit upper triangular):
-        //      column ln, x_i = [i == ln] - sum_{j>i} A^T_ij beta_j x_j, from the bottom row up
+        // ---- inverse of the diagonal block `wave` of I + A^T diag(beta) (unit upper triangular), on the
+        //      matrix cores: T = I - M with M_ij = -A^T_ij beta_j for j > i
         if (hf == 0) {
             const float *ad = Ad + (wave * 16) * LDD;
-            if constexpr (X::kBf) {
-                // on the matrix cores: T = I - M with M_ij = -A^T_ij beta_j for j > i
-                const float4 row = *reinterpret_cast<const float4 *>(ad + ln * LDD + 4 * lq);
-                const float rv[4] = {row.x, row.y, row.z, row.w};
-                const float bl = bts[wave * 16 + ln];
-                f32x4 m, mt;
+            const float4 row = *reinterpret_cast<const float4 *>(ad + ln * LDD + 4 * lq);
+            const float rv[4] = {row.x, row.y, row.z, row.w};
+            const float bl = bts[wave * 16 + ln];
+            f32x4 m, mt;
 #pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int i = 4 * lq + r;
-                    m[r] = ln > i ? -ad[i * LDD + ln] * bl : 0.f;                  // M[i][ln]
-                    mt[r] = i > ln ? -rv[r] * bts[wave * 16 + i] : 0.f;            // M[ln][i]
-                }
-                const f32x4 inv = tri_inverse16<X>(m, mt);
-#pragma unroll
-                for (int r = 0; r < 4; ++r) X::st(Di, wave * 16 + 4 * lq + r, ln, inv[r]);
-            } else {
-                float x[16];
-#pragma unroll
-                for (int i = 15; i >= 0; --i) {
-                    float acc = (i == ln) ? 1.f : 0.f;
-#pragma unroll
-                    for (int j = i + 1; j < 16; ++j) acc = fmaf(-bts[wave * 16 + j] * ad[i * LDD + j], x[j], acc);
-                    x[i] = acc;
-                }
-#pragma unroll
-                for (int i = 0; i < 16; ++i) X::st(Di, wave * 16 + i, ln, x[i]);
+            for (int r = 0; r < 4; ++r) {
+                const int i = 4 * lq + r;
+                m[r] = ln > i ? -ad[i * LDD + ln] * bl : 0.f;                  // M[i][ln]
+                mt[r] = i > ln ? -rv[r] * bts[wave * 16 + i] : 0.f;            // M[ln][i]
             }
+            const f32x4 inv = tri_inverse16<X>(m, mt);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) X::st(Di, wave * 16 + 4 * lq + r, ln, inv[r]);
         }
 
         // ---- independent of the inversion: revert S, dU = K dS' + tril(Q K^T)^T dOut
