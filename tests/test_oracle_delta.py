@@ -183,3 +183,23 @@ def test_stepwise_reference_values_and_closed_form_gradients():
                                           kq * (gt * (vt - vold)).sum(-1, keepdim=True))):
             assert rel_err(leaf.grad[:, :, t].numpy(), formula.numpy()) < 1e-12
         W = W + torch.einsum("nhe,nhm->nhem", kt, ins)
+
+
+def test_product_formula_of_the_triangular_block_inverse():
+    """The chunkwise kernels invert their 16 x 16 unit triangular diagonal blocks T = I - M as
+    (I + M)(I + M^2)(I + M^4)(I + M^8), valid because M is nilpotent (M^16 = 0).  Checked here
+    against numpy's inverse for both triangles, and the transposed recurrence the kernels carry
+    along (R^T <- R^T + (P^T)^2 R^T) against the transpose of the result."""
+    rng = np.random.default_rng(3)
+    eye = np.eye(16)
+    for lower in (True, False):
+        M = rng.standard_normal((16, 16))
+        M = np.tril(M, -1) if lower else np.triu(M, 1)
+        P, Pt, R, Rt = M.copy(), M.T.copy(), eye + M, eye + M.T
+        for _ in range(3):
+            P, Pt = P @ P, Pt @ Pt
+            R, Rt = R + R @ P, Rt + Pt @ Rt
+        ref = np.linalg.inv(eye - M)
+        assert np.allclose(R, ref, rtol=1e-10, atol=1e-10)
+        assert np.allclose(Rt, ref.T, rtol=1e-10, atol=1e-10)
+        assert np.abs(np.linalg.matrix_power(M, 16)).max() == 0.0
