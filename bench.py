@@ -41,7 +41,7 @@ MEASURED_TRAFFIC_BYTES = {
     "delta_c2": (102444 + 53504) * 1024,
     "delta_c2_chunk": (82217 + 85992 + 16640 + 36864) * 1024,
     "delta_c5": (1316522 + 1323008) * 1024,
-    "delta_c5_chunk": (1047417 + 1575763 + 267264 + 532480) * 1024,
+    "delta_c5_chunk": (1047391 + 1575757 + 267264 + 532480) * 1024,
 }
 
 WORKLOADS = {
