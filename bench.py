@@ -2,8 +2,8 @@
 """Headline benchmark: SRWM forward+backward tokens/s on one MI355X.
 
 A "step" is one forward + one backward pass of the SRWM operator over one batch of
-synthetic input (N=32, H=16, L=512, d_head=64, fp32 -- BASELINE.json configs[3], the
-configuration the metric is quoted on), including the re-initialisation of the per-batch
+synthetic input (N=32, H=16, L=512, d_head=64, fp32 -- the configuration the headline
+metric is quoted on), including the re-initialisation of the per-batch
 state copies that the layer's `.repeat()` performs every call.  All tensors are resident
 in HBM before the timed region; kernels are launched through the C ABI on torch's current
 stream, so torch.cuda.Event brackets exactly the stream the kernels run on.
@@ -56,7 +56,7 @@ WORKLOADS = {
     "delta_c2": ("delta", 32, 8, 256, 64),
     "delta_c5f32": ("delta", 8, 16, 4096, 128),
     "delta_c5": ("delta_bf16", 8, 16, 4096, 128),     # bf16 q/k/v/beta/out/grads, fp32 memory
-    # same shapes with the chunkwise (chunk = 64) MFMA forward; the backward is the step-by-step one
+    # same shapes with the chunkwise matrix-core kernels (forward, and the two backward sweeps)
     "delta_c2_chunk": ("delta", 32, 8, 256, 64),
     "delta_c5f32_chunk": ("delta", 8, 16, 4096, 128),
     "delta_c5_chunk": ("delta_bf16", 8, 16, 4096, 128),

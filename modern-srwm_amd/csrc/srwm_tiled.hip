@@ -540,6 +540,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 #pragma unroll
                 for (int c = 0; c < NC; ++c) gdif[c] = fmaf(g[i][c], kr[i], gdif[c]);
             group_sum_n<RG, NC>(gdif);
+            pin_here(gdif);   // the last add stays beside its DPP move
             float pg[3] = {0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < NC; ++c) {

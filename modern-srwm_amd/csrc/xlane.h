@@ -35,14 +35,43 @@ __device__ __forceinline__ float dpp_mov_rows(float old, float v) {
                                                                  ROWMASK, 0xF, false));
 }
 
+// Reduction operators.  rows_accumulate<15> folds lane 15 of the previous 16-lane row into rows 1
+// and 3, rows_accumulate<31> folds lane 31 into rows 2 and 3; the other rows keep their value.
+// One DPP instruction with a row mask each -- written as assembly because the compiler only
+// forms the masked DPP form for integer operators (it would emit a zero, a DPP move and an add).
+// The s_nop covers the two wait states a DPP read needs after a vector write of its source,
+// which the compiler's hazard recogniser cannot see inside an asm block.
 struct OpSum {
     static __device__ __forceinline__ float f(float a, float b) { return a + b; }
-    static __device__ __forceinline__ float neutral(float) { return 0.f; }
+    template <int LAST>
+    static __device__ __forceinline__ void rows_accumulate(float &v) {
+        static_assert(LAST == 15 || LAST == 31, "row_bcast:15 or row_bcast:31");
+        if constexpr (LAST == 15)
+            asm("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf" : "+v"(v));
+        else
+            asm("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf" : "+v"(v));
+    }
 };
 struct OpMax {
     static __device__ __forceinline__ float f(float a, float b) { return fmaxf(a, b); }
-    static __device__ __forceinline__ float neutral(float v) { return v; }
+    template <int LAST>
+    static __device__ __forceinline__ void rows_accumulate(float &v) {
+        static_assert(LAST == 15 || LAST == 31, "row_bcast:15 or row_bcast:31");
+        if constexpr (LAST == 15)
+            asm("s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf" : "+v"(v));
+        else
+            asm("s_nop 1\n\tv_max_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf" : "+v"(v));
+    }
 };
+
+// Makes the compiler finish computing v[] at this point of the program: an empty asm it can neither
+// remove nor move below a later branch.  Used where an add would otherwise be sunk away from the
+// DPP move that feeds it, which keeps the two from fusing into one DPP add.
+template <int N>
+__device__ __forceinline__ void pin_here(float (&v)[N]) {
+#pragma unroll
+    for (int n = 0; n < N; ++n) asm volatile("" : "+v"(v[n]));
+}
 
 // All-reduce of N independent values over aligned groups of G consecutive lanes (G = 1, 2,
 // 4, 8, 16, 32 or 64): every lane of a group ends up with the group's results.  Written
@@ -70,13 +99,11 @@ __device__ __forceinline__ void group_allreduce_n(float (&v)[N]) {
     }
     if constexpr (G >= 32) {  // rows 1 and 3 += rows 0 and 2
 #pragma unroll
-        for (int n = 0; n < N; ++n)
-            v[n] = Op::f(v[n], dpp_mov_rows<kDppBcast15, 0xA>(Op::neutral(v[n]), v[n]));
+        for (int n = 0; n < N; ++n) Op::template rows_accumulate<15>(v[n]);
     }
     if constexpr (G == 64) {  // rows 2 and 3 += row 1; lane 63 then holds the total
 #pragma unroll
-        for (int n = 0; n < N; ++n)
-            v[n] = Op::f(v[n], dpp_mov_rows<kDppBcast31, 0xC>(Op::neutral(v[n]), v[n]));
+        for (int n = 0; n < N; ++n) Op::template rows_accumulate<31>(v[n]);
 #pragma unroll
         for (int n = 0; n < N; ++n) v[n] = readlane(v[n], 63);
     } else if constexpr (G == 32) {
@@ -194,6 +221,7 @@ __device__ __forceinline__ void stride8_reduce_store(const float (&v)[R], float 
     swap_halve<16, NA>(a, b);
 #pragma unroll
     for (int i = 0; i < NB; ++i) b[i] += dpp_mov<kDppRor8>(b[i]);
+    pin_here(b);   // keeps the add beside its DPP move (one v_add_f32_dpp) instead of inside the store's branch
     const int b5 = (lane >> 5) & 1, b4 = (lane >> 4) & 1, b3 = (lane >> 3) & 1;
     const int idx = (R >= 2 ? NA * b5 : 0) + (NA >= 2 ? NB * b4 : 0);
     const bool writer = b3 == 0 && (R >= 2 || b5 == 0) && (NA >= 2 || b4 == 0);
