@@ -76,6 +76,13 @@ __device__ __forceinline__ void store_vec(float *dst, const float *src) {
     }
 }
 
+// base[idx] addressed as a uniform base plus a 32-bit byte offset per lane (one instruction-level
+// address operand each, no 64-bit vector arithmetic); idx * sizeof(T) must stay below 2^32.
+template <class T>
+__device__ __forceinline__ T *at32(T *base, unsigned idx) {
+    return reinterpret_cast<T *>(reinterpret_cast<char *>(base) + idx * (unsigned)sizeof(T));
+}
+
 // Softmax over a row of E floats that E/4 consecutive lanes hold as one float4 each.
 template <int E>
 __device__ __forceinline__ float4 row_softmax4(float4 v) {
@@ -152,14 +159,14 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     const bool softmax_x = RESET && (p.mode & kModeSoftmaxX);
     const bool bf16_io = RESET && (p.mode & kModeBf16);
     // rows of the Y-wide tensors start at any word: no vector stores there
-    auto store_y = [&](float *dst, const float *v) {
+    auto store_y = [&](float *base, unsigned row, const float *v) {   // row = offset of the step's row inside the sequence
         if constexpr (XC) {
 #pragma unroll
             for (int b = 0; b < YB; ++b)
 #pragma unroll
-                for (int c = 0; c < CB; ++c) dst[b * E + c0 + c] = v[b * CB + c];
+                for (int c = 0; c < CB; ++c) *at32(base, row + (unsigned)(b * E + c0 + c)) = v[b * CB + c];
         } else {
-            store_vec<CB>(dst + c0, v);
+            store_vec<CB>(at32(base, row + (unsigned)c0), v);
         }
     };
 
@@ -187,124 +194,191 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     }
     if (RESET && tid < TT) kt[0][tid] = load_keep(0);
     __syncthreads();
+    float4 xnext = make_float4(0.f, 0.f, 0.f, 0.f);   // the tile after the committed ones, staged in registers
+    float knext = 1.f;
+    if (ntiles > 1) {
+        xnext = load_tile(1);
+        knext = load_keep(1);
+    }
 
-    for (int tile = 0; tile < ntiles; ++tile) {
-        const int buf = tile & 1;
-        const int tlen = min(TT, p.L - tile * TT);
-        float4 xnext = make_float4(0.f, 0.f, 0.f, 0.f);
-        float knext = 1.f;
-        if (tile + 1 < ntiles) {
-            xnext = load_tile(tile + 1);
-            knext = load_keep(tile + 1);
+    // [y | q~ | k~ | b~] = W^T x of one step, straight from the state in registers
+    auto readout = [&](const float (&xr)[R], float xb, float (&acc)[NC], float &pb, float &py) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) acc[c] = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int c = 0; c < NC; ++c) acc[c] = fmaf(w[i][c], xr[i], acc[c]);
+        group_sum_n<RG, NC>(acc);
+        if constexpr (XC) {
+            float s[2] = {wbe * xb, wye * xb};
+            group_sum_n<E, 2>(s);
+            pb = s[0];
+            py = s[1];
+        } else {
+            pb = group_sum<E>(wbe * xb);
+        }
+    };
+    // hands the readout of step t to the output and, through LDS, to the activations of that step
+    auto publish = [&](int t, const float (&acc)[NC], float pb, float py) {
+        const unsigned oy = t * Y;           // offsets inside the sequence (the launcher bounds L * Y)
+        const int par = t & 1;
+        if (rg == 0) {
+            if (bf16_io) {
+#pragma unroll
+                for (int b = 0; b < YB; ++b)
+#pragma unroll
+                    for (int c = 0; c < CB; ++c)
+                        *at32(out16_s, oy + (unsigned)(b * E + c0 + c)) = f32_to_bf16_bits(acc[b * CB + c]);
+            } else {
+                store_y(out_s, oy, &acc[0]);
+            }
+            store_vec<CB>(&raw[par][0][c0], &acc[QB]);
+            store_vec<CB>(&raw[par][1][c0], &acc[KB]);
+        }
+        if (has_b && el == 0) rawb[par][jb] = pb;
+        if constexpr (XC) {
+            if (has_y && el == 0) {
+                if (bf16_io) *at32(out16_s, oy + YB * E) = f32_to_bf16_bits(py);
+                else *at32(out_s, oy + YB * E) = py;
+            }
+        }
+    };
+
+    // The loop is rotated by half a step: iteration t starts where the readout of step t is in LDS
+    // and ends with the readout of step t+1.  That readout is formed WITHOUT waiting for the write
+    // of step t:  W_t^T x' = W_{t-1}^T x' + ins (k . x'), so the pass over the state runs beside the
+    // softmax of step t, only the scalar correction depends on it, and the rank-1 write itself
+    // comes after the readout has been handed over.
+    {
+        if constexpr (RESET) {
+            if (kt[0][0] == 0.f) reset_state();   // uniform over the workgroup
+        }
+        float xr[R], acc[NC], pb, py = 0.f;
+        lds_read_vec<R>(xr, &xt[0][0][r0]);
+        readout(xr, xt[0][0][el], acc, pb, py);
+        publish(0, acc, pb, py);
+    }
+    __syncthreads();
+
+    for (int t = 0; t < p.L; ++t) {
+        const int par = t & 1, t1 = t + 1;
+        const unsigned o = t * E, oy = t * Y, ob = t * 4;   // unsigned: uniform base + 32-bit lane offset addressing
+        const int b1 = (t1 / TT) & 1, r1 = t1 % TT;   // where x of step t+1 sits (stale rows past the end: never published)
+        const bool have_next = t1 < p.L;
+
+        // ---- early part of the next readout: e = W_{t-1}^T x_{t+1}
+        float xr[R];
+        lds_read_vec<R>(xr, &xt[b1][r1][r0]);
+        const float xb = xt[b1][r1][el];
+        const bool reset_next = RESET && have_next && kt[b1][r1] == 0.f;   // uniform over the workgroup
+        const float qraw = raw[par][0][el], kraw = raw[par][1][el], braw = rawb[par][lane & 3];
+        float e[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) e[c] = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int c = 0; c < NC; ++c) e[c] = fmaf(w[i][c], xr[i], e[c]);
+        group_sum_n<RG, NC>(e);
+
+        // ---- activations of step t, redundantly in every wave, lane <-> element el
+        float mx[2] = {qraw, kraw};
+        group_max_n<E, 2>(mx);
+        const float eq = exp_2ulp(qraw - mx[0]), ek = exp_2ulp(kraw - mx[1]);
+        float sm[2] = {eq, ek};
+        group_sum_n<E, 2>(sm);
+        const float qn = eq * fast_rcp(sm[0]), kn = ek * fast_rcp(sm[1]);
+        // sigmoid saturates to 0 / 1 in fp32 well inside +-80; the clamp keeps exp finite
+        const float sg = fast_rcp(1.f + exp_2ulp(-fminf(fmaxf(braw, -80.f), 80.f)));
+        const float bt[4] = {quad_broadcast<0>(sg), quad_broadcast<1>(sg), quad_broadcast<2>(sg),
+                             quad_broadcast<3>(sg)};
+        const float dv = qn - kn;
+        if (wave == 0 && lane < E) {
+            *at32(q_s, o + lane) = qn;
+            *at32(k_s, o + lane) = kn;
+        }
+        if (wave == NW - 1 && lane < 4) *at32(beta_s, ob + lane) = sg;
+        if (lane < E) {
+            exch[wave][0][lane] = dv;
+            exch[wave][1][lane] = kn;
+        }
+        wave_lds_fence();
+        float dvr[R], kr[R];
+        lds_read_vec<R>(dvr, &exch[wave][0][r0]);
+        lds_read_vec<R>(kr, &exch[wave][1][r0]);
+
+        // ---- diff = W_{t-1}^T (q - k); with it, the narrow columns and k . x_{t+1}
+        float dif[NC];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) dif[c] = 0.f;
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int c = 0; c < NC; ++c) dif[c] = fmaf(w[i][c], dvr[i], dif[c]);
+        group_sum_n<RG, NC>(dif);
+        constexpr int NS = XC ? 5 : 3;
+        float s[NS];
+        s[0] = wbe * dv;   // -> b diff
+        s[1] = kn * xb;    // -> k . x_{t+1}
+        s[2] = wbe * xb;   // -> early b~ of step t+1
+        if constexpr (XC) {
+            s[3] = wye * dv;
+            s[4] = wye * xb;
+        }
+        group_sum_n<E, NS>(s);
+        const float pbd = s[0], kx = s[1];
+        if (rg == 0) {
+            store_y(ydiff_s, oy, &dif[0]);
+            store_vec<CB>(at32(qdiff_s, o + (unsigned)c0), &dif[QB]);
+            store_vec<CB>(at32(kdiff_s, o + (unsigned)c0), &dif[KB]);
+        }
+        if (has_b && el == 0) *at32(bdiff_s, ob + jb) = pbd;
+        if constexpr (XC) {
+            if (has_y && el == 0) *at32(ydiff_s, oy + YB * E) = s[3];
         }
 
-        for (int tt = 0; tt < tlen; ++tt) {
-            const int t = tile * TT + tt, par = t & 1;
-            const int o = t * E, oy = t * Y, ob = t * 4;   // offsets inside the sequence (the launcher bounds L * Y)
-            if constexpr (RESET) {
-                if (kt[buf][tt] == 0.f) reset_state();   // uniform over the workgroup
-            }
-
-            // ---- main readout: [y | q~ | k~ | b~] = W^T x_t
-            float xr[R];
-            lds_read_vec<R>(xr, &xt[buf][tt][r0]);
-            const float xb = xt[buf][tt][el];
-            float acc[NC];
+        // ---- the write of step t: W += k (x) (beta_blk * diff); every y block uses beta_y
+        float ins[NC];
 #pragma unroll
-            for (int c = 0; c < NC; ++c) acc[c] = 0.f;
-#pragma unroll
-            for (int i = 0; i < R; ++i)
-#pragma unroll
-                for (int c = 0; c < NC; ++c) acc[c] = fmaf(w[i][c], xr[i], acc[c]);
-            group_sum_n<RG, NC>(acc);
-            const float pb = group_sum<E>(wbe * xb);
-            if (rg == 0) {
-                if (bf16_io) {
-                    uint16_t *o16 = out16_s + oy;
-#pragma unroll
-                    for (int b = 0; b < YB; ++b)
-#pragma unroll
-                        for (int c = 0; c < CB; ++c) o16[b * E + c0 + c] = f32_to_bf16_bits(acc[b * CB + c]);
-                } else {
-                    store_y(out_s + oy, &acc[0]);
-                }
-                store_vec<CB>(&raw[par][0][c0], &acc[QB]);
-                store_vec<CB>(&raw[par][1][c0], &acc[KB]);
-            }
-            if (has_b && el == 0) rawb[par][jb] = pb;
-            if constexpr (XC) {
-                const float py = group_sum<E>(wye * xb);
-                if (has_y && el == 0) {
-                    if (bf16_io) out16_s[oy + YB * E] = f32_to_bf16_bits(py);
-                    else out_s[oy + YB * E] = py;
-                }
-            }
-            if (tt == tlen - 1 && tile + 1 < ntiles) {
-                *reinterpret_cast<float4 *>(&xt[buf ^ 1][ld_row][ld_col]) =
-                    softmax_x ? row_softmax4<E>(xnext) : xnext;
-                if (RESET && tid < TT) kt[buf ^ 1][tid] = knext;
-            }
-            __syncthreads();
-
-            // ---- activations, redundantly in every wave, lane <-> element el
-            const float qraw = raw[par][0][el], kraw = raw[par][1][el], braw = rawb[par][lane & 3];
-            float mx[2] = {qraw, kraw};
-            group_max_n<E, 2>(mx);
-            const float eq = exp_2ulp(qraw - mx[0]), ek = exp_2ulp(kraw - mx[1]);
-            float sm[2] = {eq, ek};
-            group_sum_n<E, 2>(sm);
-            const float qn = eq * fast_rcp(sm[0]), kn = ek * fast_rcp(sm[1]);
-            // sigmoid saturates to 0 / 1 in fp32 well inside +-80; the clamp keeps exp finite
-            const float sg = fast_rcp(1.f + exp_2ulp(-fminf(fmaxf(braw, -80.f), 80.f)));
-            const float bt[4] = {quad_broadcast<0>(sg), quad_broadcast<1>(sg), quad_broadcast<2>(sg),
-                                 quad_broadcast<3>(sg)};
-            const float dv = qn - kn;
-            if (wave == 0 && lane < E) {
-                q_s[o + lane] = qn;
-                k_s[o + lane] = kn;
-            }
-            if (wave == NW - 1 && lane < 4) beta_s[ob + lane] = sg;
-            if (lane < E) {
-                exch[wave][0][lane] = dv;
-                exch[wave][1][lane] = kn;
-            }
-            wave_lds_fence();
-            float dvr[R], kr[R];
-            lds_read_vec<R>(dvr, &exch[wave][0][r0]);
-            lds_read_vec<R>(kr, &exch[wave][1][r0]);
-
-            // ---- diff = W^T (q - k)
-            float dif[NC];
-#pragma unroll
-            for (int c = 0; c < NC; ++c) dif[c] = 0.f;
-#pragma unroll
-            for (int i = 0; i < R; ++i)
-#pragma unroll
-                for (int c = 0; c < NC; ++c) dif[c] = fmaf(w[i][c], dvr[i], dif[c]);
-            group_sum_n<RG, NC>(dif);
-            const float pbd = group_sum<E>(wbe * dv);
-            if (rg == 0) {
-                store_y(ydiff_s + oy, &dif[0]);
-                store_vec<CB>(qdiff_s + o + c0, &dif[QB]);
-                store_vec<CB>(kdiff_s + o + c0, &dif[KB]);
-            }
-            if (has_b && el == 0) bdiff_s[ob + jb] = pbd;
-
-            // ---- rank-1 write W += k (x) (beta_blk * diff); every y block uses beta_y
-            float ins[NC];
-#pragma unroll
-            for (int c = 0; c < NC; ++c) ins[c] = bt[c / CB < YB ? 0 : c / CB - YB + 1] * dif[c];
+        for (int c = 0; c < NC; ++c) ins[c] = bt[c / CB < YB ? 0 : c / CB - YB + 1] * dif[c];
+        const float insb = bt[3] * pbd;
+        float insy = 0.f;
+        if constexpr (XC) insy = bt[0] * s[3];
+        auto write_state = [&]() {
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < NC; ++c) w[i][c] = fmaf(kr[i], ins[c], w[i][c]);
-            wbe = fmaf(kn, bt[3] * pbd, wbe);
-            if constexpr (XC) {
-                const float pyd = group_sum<E>(wye * dv);
-                if (has_y && el == 0) ydiff_s[oy + YB * E] = pyd;
-                wye = fmaf(kn, bt[0] * pyd, wye);
+            wbe = fmaf(kn, insb, wbe);
+            if constexpr (XC) wye = fmaf(kn, insy, wye);
+        };
+
+        // ---- readout of step t+1, published before the write is carried out
+        if (RESET && reset_next) {
+            reset_state();   // the state of step t is dropped: the write is not needed
+            float acc[NC], pb, py = 0.f;
+            readout(xr, xb, acc, pb, py);
+            publish(t1, acc, pb, py);
+        } else {
+#pragma unroll
+            for (int c = 0; c < NC; ++c) e[c] = fmaf(ins[c], kx, e[c]);
+            float py = 0.f;
+            if constexpr (XC) py = fmaf(insy, kx, s[4]);
+            if (have_next) publish(t1, e, fmaf(insb, kx, s[2]), py);
+            write_state();
+        }
+
+        // x of step t+2 opens a new tile: commit the staged tile, fetch the one after it
+        if (r1 == TT - 1 && t1 / TT + 1 < ntiles) {
+            *reinterpret_cast<float4 *>(&xt[b1 ^ 1][ld_row][ld_col]) = softmax_x ? row_softmax4<E>(xnext) : xnext;
+            if (RESET && tid < TT) kt[b1 ^ 1][tid] = knext;
+            if (t1 / TT + 2 < ntiles) {
+                xnext = load_tile(t1 / TT + 2);
+                knext = load_keep(t1 / TT + 2);
             }
         }
+        __syncthreads();
     }
 
     // the final state, as the shift from the shared weights if that is how the caller keeps it
