@@ -409,7 +409,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 //   row sums     G ins, W_{t-1} g_diff, W_{t-1} g_pre (per lane R partial rows -> reduce-scatter
 //                over the wave's 8 column groups with v_permlane{32,16}_swap + one DPP step,
 //                then summed over the waves through LDS)
-// and two workgroup barriers (after the first pair of row sums, after the grad_x row sum).
+// and ONE workgroup barrier, after the first pair of row sums: the hand-over buffers exist once
+// per step parity, and the grad_x row sums of a step are added up behind the barrier of the
+// following step (the last ones after the loop), so they need no barrier of their own.
 // The seven per-step vectors and beta are streamed through a single LDS tile of TT steps;
 // the next tile is fetched into registers one tile ahead.
 template <int E, int NW, int R, int YB>
@@ -430,10 +432,12 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     __shared__ __attribute__((aligned(16))) float tyd[TT][YS];      // y_diff of the tile
     __shared__ __attribute__((aligned(16))) float tgo[TT][YS];      // grad_out of the tile
     __shared__ __attribute__((aligned(16))) float tb[2][TT][4];     // beta | beta_diff
-    __shared__ __attribute__((aligned(16))) float rowm[3][NW][E];   // row sums per wave: G ins | W gdiff | W gpre
-    __shared__ __attribute__((aligned(16))) float rowb[3][NXS][E];  // same, contribution of the narrow columns
-    __shared__ __attribute__((aligned(16))) float gbp[NCG][4];      // per column group: sum gins*diff per beta
-    __shared__ __attribute__((aligned(16))) float gbp3[8];          // same for the narrow columns
+    // cross-wave hand-over buffers, one set per step parity: a wave may start writing those of the
+    // next step while a slower wave still reads this step's
+    __shared__ __attribute__((aligned(16))) float rowm[2][3][NW][E];   // row sums per wave: G ins | W gdiff | W gpre
+    __shared__ __attribute__((aligned(16))) float rowb[2][3][NXS][E];  // same, contribution of the narrow columns
+    __shared__ __attribute__((aligned(16))) float gbp[2][NCG][4];      // per column group: sum gins*diff per beta
+    __shared__ __attribute__((aligned(16))) float gbp3[2][8];          // same for the narrow columns
     __shared__ __attribute__((aligned(16))) float exch[NW][2][E];   // per wave: g_pre of the q | k block
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -552,6 +556,22 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
         }                                                                                          \
     } while (0)
 
+    // grad_x of step t: the row sums W_{t-1} g_pre of all waves and of the narrow columns (buffers of
+    // parity pp), through the softmax of the input where the kernel applies it (xs = this thread's
+    // element of the softmaxed x_t)
+    auto finish_gx = [&](int t, int pp, float xs) {
+        if (tid < E) {
+            float s = 0.f;
+#pragma unroll
+            for (int wv = 0; wv < NW; ++wv) s += rowm[pp][2][wv][tid];
+#pragma unroll
+            for (int j = 0; j < NXS; ++j) s += rowb[pp][2][j][tid];
+            if (softmax_x) s = xs * (s - group_sum<E>(s * xs));   // tid < E covers whole lane groups
+            p.gx[(seq * p.L + t) * E + tid] = s;
+        }
+    };
+    float xb_prev = 0.f;
+
     const int ntiles = (p.L + TT - 1) / TT;
     SRWM_BWD_LOAD_TILE(ntiles - 1);
     SRWM_BWD_STORE_TILE();
@@ -562,8 +582,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
         if (tile > 0) SRWM_BWD_LOAD_TILE(tile - 1);
 
         for (int tt = tlen - 1; tt >= 0; --tt) {
-            const int t = tile * TT + tt;
-            const int64_t o = (seq * p.L + t) * E;
+            const int t = tile * TT + tt, par = t & 1;
 
             // ---- operands of the step
             float kr[R], dvr[R], xr[R];
@@ -641,34 +660,34 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                     u[i] = fmaf(w[i][c], gdif[c], u[i]);
                 }
             }
-            stride8_reduce_store<R>(a, &rowm[0][wave][r0], lane);
-            stride8_reduce_store<R>(u, &rowm[1][wave][r0], lane);
+            stride8_reduce_store<R>(a, &rowm[par][0][wave][r0], lane);
+            stride8_reduce_store<R>(u, &rowm[par][1][wave][r0], lane);
             if (has_b) {
-                rowb[0][jb][el] = gbe * insb;
-                rowb[1][jb][el] = wbe * gdifb;
-                if (el == 0) gbp3[jb] = ginsb * bd;
+                rowb[par][0][jb][el] = gbe * insb;
+                rowb[par][1][jb][el] = wbe * gdifb;
+                if (el == 0) gbp3[par][jb] = ginsb * bd;
             }
             if constexpr (XC) {
                 if (has_y) {
-                    rowb[0][4][el] = gye * insy;
-                    rowb[1][4][el] = wye * gdify;
-                    if (el == 0) gbp3[4] = ginsy * ydl;
+                    rowb[par][0][4][el] = gye * insy;
+                    rowb[par][1][4][el] = wye * gdify;
+                    if (el == 0) gbp3[par][4] = ginsy * ydl;
                 }
             }
-            if (rg == 0) *reinterpret_cast<float4 *>(&gbp[cg][0]) = make_float4(pg[0], pg[1], pg[2], 0.f);
+            if (rg == 0) *reinterpret_cast<float4 *>(&gbp[par][cg][0]) = make_float4(pg[0], pg[1], pg[2], 0.f);
             __syncthreads();
 
             // ---- every wave, lane <-> element el: gradients of q, k, beta before activation
             float gq = 0.f, gk = 0.f;
 #pragma unroll
             for (int wv = 0; wv < NW; ++wv) {
-                gk += rowm[0][wv][el];
-                gq += rowm[1][wv][el];
+                gk += rowm[par][0][wv][el];
+                gq += rowm[par][1][wv][el];
             }
 #pragma unroll
             for (int j = 0; j < NXS; ++j) {
-                gk += rowb[0][j][el];
-                gq += rowb[1][j][el];
+                gk += rowb[par][0][j][el];
+                gq += rowb[par][1][j][el];
             }
             gk -= gq;
             float dqk[2] = {gq * qb, gk * kb};
@@ -679,10 +698,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 // jb == wave: a wave only needs the beta gradient of its own w_b column, one sum instead of three
                 float gbw;
                 if (jb < 3) {
-                    gbw = group_sum<NCG>(gbp[lane % NCG][jb]);
+                    gbw = group_sum<NCG>(gbp[par][lane % NCG][jb]);
                 } else {
                     float p3[4];
-                    lds_read_vec<4>(p3, &gbp3[0]);
+                    lds_read_vec<4>(p3, &gbp3[par][0]);
                     gbw = (p3[0] + p3[1]) + (p3[2] + p3[3]);
                 }
                 const float btw = bt[jb & 3];
@@ -690,15 +709,15 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             } else {
                 float gb[4];
                 float part[4];
-                lds_read_vec<4>(part, &gbp[lane % NCG][0]);
+                lds_read_vec<4>(part, &gbp[par][lane % NCG][0]);
                 float p012[3] = {part[0], part[1], part[2]};
                 group_sum_n<NCG, 3>(p012);
 #pragma unroll
                 for (int j = 0; j < 3; ++j) gb[j] = p012[j];
                 float p3[4];
-                lds_read_vec<4>(p3, &gbp3[0]);
+                lds_read_vec<4>(p3, &gbp3[par][0]);
                 gb[3] = (p3[0] + p3[1]) + (p3[2] + p3[3]);
-                if constexpr (XC) gb[0] += gbp3[4];
+                if constexpr (XC) gb[0] += gbp3[par][4];
                 float gpb[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) gpb[j] = gb[j] * bt[j] * (1.f - bt[j]);
@@ -720,24 +739,14 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 #pragma unroll
                 for (int c = 0; c < NC; ++c) sx[i] = fmaf(w[i][c], gpre[c], sx[i]);
             }
-            stride8_reduce_store<R>(sx, &rowm[2][wave][r0], lane);
-            if (has_b) rowb[2][jb][el] = wbe * gpreb;
+            stride8_reduce_store<R>(sx, &rowm[par][2][wave][r0], lane);
+            if (has_b) rowb[par][2][jb][el] = wbe * gpreb;
             if constexpr (XC) {
-                if (has_y) rowb[2][4][el] = wye * gprey;
+                if (has_y) rowb[par][2][4][el] = wye * gprey;
             }
-            __syncthreads();
-            if (tid < E) {
-                float s = 0.f;
-#pragma unroll
-                for (int wv = 0; wv < NW; ++wv) s += rowm[2][wv][tid];
-#pragma unroll
-                for (int j = 0; j < NXS; ++j) s += rowb[2][j][tid];
-                if (softmax_x) {   // through the softmax of the input: sx (s - <s, sx>); tid < E covers whole lane groups
-                    const float sx = tl[VX][tt][tid];
-                    s = sx * (s - group_sum<E>(s * sx));
-                }
-                p.gx[o + tid] = s;
-            }
+            // the grad_x partials are summed one step later, behind the next step's barrier: no barrier of their own
+            if (t + 1 < p.L) finish_gx(t + 1, par ^ 1, xb_prev);
+            xb_prev = xb;
 
             // ---- G_{t-1} = G_t + (q - k) (x) g_diff + x (x) g_pre
 #pragma unroll
@@ -756,6 +765,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             }
         }
     }
+
+    __syncthreads();
+    finish_gx(0, 0, xb_prev);
 
     {
         const bool accum = p.grad_state_mode == 2u;
