@@ -561,9 +561,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     // element of the softmaxed x_t)
     auto finish_gx = [&](int t, int pp, float xs) {
         if (tid < E) {
-            float s = 0.f;
+            float s = rowm[pp][2][0][tid];
 #pragma unroll
-            for (int wv = 0; wv < NW; ++wv) s += rowm[pp][2][wv][tid];
+            for (int wv = 1; wv < NW; ++wv) s += rowm[pp][2][wv][tid];
 #pragma unroll
             for (int j = 0; j < NXS; ++j) s += rowb[pp][2][j][tid];
             if (softmax_x) s = xs * (s - group_sum<E>(s * xs));   // tid < E covers whole lane groups
@@ -601,7 +601,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[KB]), &tl[VKD][tt][c0]);
             float bt[4];
             lds_read_vec<4>(bt, &tb[0][tt][0]);
-            const float bd = tb[1][tt][jb & 3];
+            const float bd = tb[1][tt][jb & 3], btj = tb[0][tt][jb & 3];   // this thread's w_b column: beta_diff, beta
             const float kb = tl[VK][tt][el], qb = tl[VQ][tt][el], xb = tl[VX][tt][el];
             const float dvb = qb - kb;
 
@@ -678,9 +678,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             __syncthreads();
 
             // ---- every wave, lane <-> element el: gradients of q, k, beta before activation
-            float gq = 0.f, gk = 0.f;
+            float gk = rowm[par][0][0][el], gq = rowm[par][1][0][el];
 #pragma unroll
-            for (int wv = 0; wv < NW; ++wv) {
+            for (int wv = 1; wv < NW; ++wv) {
                 gk += rowm[par][0][wv][el];
                 gq += rowm[par][1][wv][el];
             }
@@ -704,8 +704,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                     lds_read_vec<4>(p3, &gbp3[par][0]);
                     gbw = (p3[0] + p3[1]) + (p3[2] + p3[3]);
                 }
-                const float btw = bt[jb & 3];
-                gpreb = gbw * btw * (1.f - btw);
+                gpreb = gbw * btj * (1.f - btj);
             } else {
                 float gb[4];
                 float part[4];
