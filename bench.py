@@ -37,7 +37,7 @@ HBM_PEAK_GBS = 8000.0
 # read its size).  Figures and commands: profiles/srwm_c4_kernels.txt, profiles/delta_kernels.txt,
 # profiles/delta_chunk_kernels.txt (backward kernels of the workload: fetch + write).
 MEASURED_TRAFFIC_BYTES = {
-    "srwm_c4": (490477 + 90624) * 1024,
+    "srwm_c4": (490413 + 90624) * 1024,
     "delta_c2": (102444 + 53504) * 1024,
     "delta_c2_chunk": (82217 + 85992 + 16640 + 36864) * 1024,
     "delta_c5": (1316522 + 1323008) * 1024,
