@@ -154,8 +154,34 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         load_state(p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, std::false_type{});
         if (RESET && (p.mode & kModeShift)) load_state(shWy, shWq, shWk, shwb, std::true_type{});   // incoming state is a shift
     }
-    // replaces the state by the weights all batch rows of this head share (per-step reset)
-    auto reset_state = [&]() { load_state(shWy, shWq, shWk, shwb, std::false_type{}); };
+    // Per-step reset: the state is replaced by the weights all batch rows of this head share.  A
+    // copy of this lane's part of them is kept in registers when the call can reset (fetching
+    // them again at every reset costs microseconds each).
+    float w0[R][NC];
+    float wbe0 = 0.f, wye0 = 0.f;
+    if (RESET && p.keep) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const float *src = b < YB ? shWy + b * E : b == YB ? shWq : shWk;
+            const int ld = b < YB ? Y : E;
+#pragma unroll
+            for (int i = 0; i < R; ++i)
+#pragma unroll
+                for (int c = 0; c < CB; ++c) w0[i][b * CB + c] = src[(r0 + i) * ld + c0 + c];
+        }
+        if (has_b) wbe0 = shwb[el * 4 + jb];
+        if constexpr (XC) {
+            if (has_y) wye0 = shWy[el * Y + YB * E];
+        }
+    }
+    auto reset_state = [&]() {
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int c = 0; c < NC; ++c) w[i][c] = w0[i][c];
+        wbe = wbe0;
+        if constexpr (XC) wye = wye0;
+    };
     const bool softmax_x = RESET && (p.mode & kModeSoftmaxX);
     const bool bf16_io = RESET && (p.mode & kModeBf16);
     // rows of the Y-wide tensors start at any word: no vector stores there
