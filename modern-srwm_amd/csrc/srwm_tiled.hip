@@ -435,9 +435,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 //   row sums     G ins, W_{t-1} g_diff, W_{t-1} g_pre (per lane R partial rows -> reduce-scatter
 //                over the wave's 8 column groups with v_permlane{32,16}_swap + one DPP step,
 //                then summed over the waves through LDS)
-// and ONE workgroup barrier, after the first pair of row sums: the hand-over buffers exist once
-// per step parity, and the grad_x row sums of a step are added up behind the barrier of the
-// following step (the last ones after the loop), so they need no barrier of their own.
+// At E = 64, ONE workgroup barrier per step, after the first pair of row sums: the hand-over
+// buffers exist once per step parity, and the grad_x row sums of a step are added up behind the
+// barrier of the following step (the last ones after the loop), so they need no barrier of their
+// own.  The smaller sizes use a second barrier before those sums instead.
 // The seven per-step vectors and beta are streamed through a single LDS tile of TT steps;
 // the next tile is fetched into registers one tile ahead.
 template <int E, int NW, int R, int YB>
@@ -458,12 +459,17 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     __shared__ __attribute__((aligned(16))) float tyd[TT][YS];      // y_diff of the tile
     __shared__ __attribute__((aligned(16))) float tgo[TT][YS];      // grad_out of the tile
     __shared__ __attribute__((aligned(16))) float tb[2][TT][4];     // beta | beta_diff
-    // cross-wave hand-over buffers, one set per step parity: a wave may start writing those of the
-    // next step while a slower wave still reads this step's
-    __shared__ __attribute__((aligned(16))) float rowm[2][3][NW][E];   // row sums per wave: G ins | W gdiff | W gpre
-    __shared__ __attribute__((aligned(16))) float rowb[2][3][NXS][E];  // same, contribution of the narrow columns
-    __shared__ __attribute__((aligned(16))) float gbp[2][NCG][4];      // per column group: sum gins*diff per beta
-    __shared__ __attribute__((aligned(16))) float gbp3[2][8];          // same for the narrow columns
+    // Cross-wave hand-over buffers.  ONEBAR (E = 64, where two workgroups share a CU and the step is
+    // bound by instruction issue): one set per step parity, so that a wave may start writing those of
+    // the next step while a slower wave still reads this step's, and one barrier per step.  The
+    // smaller sizes are bound by the latency of a single step; there the parity addressing costs
+    // more than the second barrier, which they keep.
+    constexpr bool ONEBAR = E == kWave;
+    constexpr int NPAR = ONEBAR ? 2 : 1;
+    __shared__ __attribute__((aligned(16))) float rowm[NPAR][3][NW][E];   // row sums per wave: G ins | W gdiff | W gpre
+    __shared__ __attribute__((aligned(16))) float rowb[NPAR][3][NXS][E];  // same, contribution of the narrow columns
+    __shared__ __attribute__((aligned(16))) float gbp[NPAR][NCG][4];      // per column group: sum gins*diff per beta
+    __shared__ __attribute__((aligned(16))) float gbp3[NPAR][8];          // same for the narrow columns
     __shared__ __attribute__((aligned(16))) float exch[NW][2][E];   // per wave: g_pre of the q | k block
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -608,7 +614,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
         if (tile > 0) SRWM_BWD_LOAD_TILE(tile - 1);
 
         for (int tt = tlen - 1; tt >= 0; --tt) {
-            const int t = tile * TT + tt, par = t & 1;
+            const int t = tile * TT + tt, par = ONEBAR ? (t & 1) : 0;
 
             // ---- operands of the step
             float kr[R], dvr[R], xr[R];
@@ -769,9 +775,14 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             if constexpr (XC) {
                 if (has_y) rowb[par][2][4][el] = wye * gprey;
             }
-            // the grad_x partials are summed one step later, behind the next step's barrier: no barrier of their own
-            if (t + 1 < p.L) finish_gx(t + 1, par ^ 1, xb_prev);
-            xb_prev = xb;
+            if constexpr (ONEBAR) {
+                // the grad_x partials are summed one step later, behind the next step's barrier: no barrier of their own
+                if (t + 1 < p.L) finish_gx(t + 1, par ^ 1, xb_prev);
+                xb_prev = xb;
+            } else {
+                __syncthreads();
+                finish_gx(t, 0, xb);
+            }
 
             // ---- G_{t-1} = G_t + (q - k) (x) g_diff + x (x) g_pre
 #pragma unroll
@@ -791,8 +802,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
         }
     }
 
-    __syncthreads();
-    finish_gx(0, 0, xb_prev);
+    if constexpr (ONEBAR) {
+        __syncthreads();
+        finish_gx(0, 0, xb_prev);
+    }
 
     {
         const bool accum = p.grad_state_mode == 2u;
