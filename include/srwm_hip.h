@@ -51,7 +51,7 @@ extern "C" {
                                      ones (forward: chunks of 64 steps; backward: a sweep over memory columns and
                                      one over memory rows); E == M in {64, 128}, else SRWM_ENOKERNEL.  Forward and
                                      backward may be mixed freely: both forms emit / consume the same v_old, v_insert */
-/* srwm_layer_forward_f32 / srwm_layer_backward_f32 only: */
+/* srwm_layer_forward_* / srwm_layer_backward_* only: */
 #define SRWM_FLAG_STATE_SHIFT 64u    /* W_y..w_b hold the state MINUS the head's shared weights, on entry and on
                                         exit (how the RL layers carry it, torchbeast/layer.py:389-418) */
 #define SRWM_FLAG_FRESH_STATE 128u   /* forward: start from the shared weights; W_y..w_b are outputs only */
@@ -209,6 +209,32 @@ SRWM_API int srwm_layer_backward_f32(const float *x, const int64_t x_strides[3],
                             int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
 /*
+ * The layer operator with bf16 input and output, fp32 state.  No counterpart in the reference (its
+ * kernels are float-only): same contract as srwm_layer_forward_f32 / srwm_layer_backward_f32 with
+ *   x, out, grad_out   bf16 (raw 16-bit patterns; strides in bf16 elements)
+ *   everything else    fp32, including grad_x and all state gradients
+ * With keep and the shared weights NULL and none of the three layer flags they are the plain operator
+ * for any width Y of the output block (srwm_forward_bf16 / srwm_backward_bf16 are that with Y = E).
+ */
+SRWM_API int srwm_layer_forward_bf16(const uint16_t *x, const int64_t x_strides[3], const float *keep,
+                            const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
+                            float *W_y, float *W_q, float *W_k, float *w_b,
+                            float *q, float *k, float *beta,
+                            float *y_diff, float *q_diff, float *k_diff, float *beta_diff,
+                            uint16_t *out, int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+
+SRWM_API int srwm_layer_backward_bf16(const uint16_t *x, const int64_t x_strides[3],
+                             const float *q, const float *k, const float *beta,
+                             const float *y_diff, const float *q_diff, const float *k_diff,
+                             const float *beta_diff,
+                             const uint16_t *grad_out, const int64_t grad_out_strides[3],
+                             const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
+                             const float *W_y, const float *W_q, const float *W_k, const float *w_b,
+                             float *grad_x, float *gW_y, float *gW_q, float *gW_k, float *gw_b,
+                             float *gsW_y, float *gsW_q, float *gsW_k, float *gsw_b,
+                             int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+
+/*
  * Gradient of that unroll with respect to x when the carried state is detached between steps
  * (what the per-step calls of the reference compute, layer.py:412-418: the new state is
  * `.detach()`-ed): grad_x[n][h][t] = W_y,t-1 grad_out[n][h][t], with W_y replayed forward from
@@ -338,7 +364,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any signature change); currently 3. */
+/* ABI version of this header (bumped on any signature change); currently 4. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

@@ -46,7 +46,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 3; }
+int srwm_hip_abi_version(void) { return 4; }
 
 const char *srwm_hip_strerror(int code) {
     switch (code) {
@@ -99,11 +99,13 @@ int srwm_forward_f32(const float *x, const int64_t xs[3], float *Wy, float *Wq, 
                                  L, E, E, flags, stream);
 }
 
-int srwm_layer_forward_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
-                           const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
-                           float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
-                           float *qdiff, float *kdiff, float *bdiff, float *out, int N, int H, int L,
-                           int E, int Y, unsigned flags, void *stream) {
+// body of the layer forward for both input / output types: `x` and `out` are float or bf16
+// (io16) behind the same pointer types, strides in elements of the actual type
+static int layer_forward(bool io16, const float *x, const int64_t xs[3], const float *keep, const float *sWy,
+                         const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
+                         float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
+                         float *qdiff, float *kdiff, float *bdiff, float *out, int N, int H, int L,
+                         int E, int Y, unsigned flags, void *stream) {
     if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
         !out || !xs)
         return SRWM_EINVAL;
@@ -115,7 +117,7 @@ int srwm_layer_forward_f32(const float *x, const int64_t xs[3], const float *kee
     SrwmFwdParams p{x, xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff,
                     out, N, H, L, E, keep, sWy, sWq, sWk, swb, Y};
     p.mode = ((flags & SRWM_FLAG_STATE_SHIFT) ? kModeShift : 0u) | ((flags & SRWM_FLAG_FRESH_STATE) ? kModeFresh : 0u) |
-             ((flags & SRWM_FLAG_SOFTMAX_INPUT) ? kModeSoftmaxX : 0u);
+             ((flags & SRWM_FLAG_SOFTMAX_INPUT) ? kModeSoftmaxX : 0u) | (io16 ? kModeBf16 : 0u);
     hipStream_t s = (hipStream_t)stream;
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_fwd_tiled(p, s);
@@ -125,52 +127,32 @@ int srwm_layer_forward_f32(const float *x, const int64_t xs[3], const float *kee
     return launch_srwm_fwd_generic(p, s);
 }
 
+int srwm_layer_forward_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
+                           const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
+                           float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
+                           float *qdiff, float *kdiff, float *bdiff, float *out, int N, int H, int L,
+                           int E, int Y, unsigned flags, void *stream) {
+    return layer_forward(false, x, xs, keep, sWy, sWq, sWk, swb, Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff,
+                         bdiff, out, N, H, L, E, Y, flags, stream);
+}
+
+int srwm_layer_forward_bf16(const uint16_t *x, const int64_t xs[3], const float *keep, const float *sWy,
+                            const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
+                            float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
+                            float *qdiff, float *kdiff, float *bdiff, uint16_t *out, int N, int H, int L,
+                            int E, int Y, unsigned flags, void *stream) {
+    return layer_forward(true, reinterpret_cast<const float *>(x), xs, keep, sWy, sWq, sWk, swb, Wy, Wq, Wk, wb, q,
+                         k, beta, ydiff, qdiff, kdiff, bdiff, reinterpret_cast<float *>(out), N, H, L, E, Y, flags,
+                         stream);
+}
+
 int srwm_forward_bf16(const uint16_t *x, const int64_t xs[3], float *Wy, float *Wq, float *Wk, float *wb,
                       float *q, float *k, float *beta, float *ydiff, float *qdiff, float *kdiff,
                       float *bdiff, uint16_t *out, int N, int H, int L, int E, unsigned flags,
                       void *stream) {
-    if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
-        !out || !xs)
-        return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || (flags & ~(SRWM_FLAG_GENERIC))) return SRWM_EINVAL;
-    if (!stride_ok(xs, N, H, L, E)) return SRWM_ESTRIDE;
-    SrwmFwdParams p{reinterpret_cast<const float *>(x), xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta,
-                    ydiff, qdiff, kdiff, bdiff, reinterpret_cast<float *>(out), N, H, L, E};
-    p.Y = E;
-    p.mode = kModeBf16;
-    hipStream_t s = (hipStream_t)stream;
-    if (!(flags & SRWM_FLAG_GENERIC)) {
-        const int r = launch_srwm_fwd_tiled(p, s);
-        if (r >= 0) return r;
-    }
-    if (srwm_fwd_generic_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
-    return launch_srwm_fwd_generic(p, s);
-}
-
-int srwm_backward_bf16(const uint16_t *x, const int64_t xs[3], const float *q, const float *k,
-                       const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
-                       const float *bdiff, const uint16_t *grad_out, const int64_t gs[3], const float *Wy,
-                       const float *Wq, const float *Wk, const float *wb, float *grad_x, float *gWy,
-                       float *gWq, float *gWk, float *gwb, int N, int H, int L, int E, unsigned flags,
-                       void *stream) {
-    if (!x || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff || !grad_out || !Wy || !Wq ||
-        !Wk || !wb || !grad_x || !gWy || !gWq || !gWk || !gwb || !xs || !gs)
-        return SRWM_EINVAL;
-    const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
-    if (!dims_ok(N, H, L, E) || mode == 3u || (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)))
-        return SRWM_EINVAL;
-    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, E)) return SRWM_ESTRIDE;
-    SrwmBwdParams p{reinterpret_cast<const float *>(x), xs[0], xs[1], xs[2], q, k, beta, ydiff, qdiff, kdiff,
-                    bdiff, reinterpret_cast<const float *>(grad_out), gs[0], gs[1], gs[2], Wy, Wq, Wk, wb,
-                    grad_x, gWy, gWq, gWk, gwb, N, H, L, E, mode, E};
-    p.mode = kModeBf16;
-    hipStream_t s = (hipStream_t)stream;
-    if (!(flags & SRWM_FLAG_GENERIC)) {
-        const int r = launch_srwm_bwd_tiled(p, s);
-        if (r >= 0) return r;
-    }
-    if (srwm_bwd_generic_lds_bytes(E, E) > lds_limit()) return SRWM_ESIZE;
-    return launch_srwm_bwd_generic(p, s);
+    if (flags & ~(SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    return srwm_layer_forward_bf16(x, xs, nullptr, nullptr, nullptr, nullptr, nullptr, Wy, Wq, Wk, wb, q, k, beta,
+                                   ydiff, qdiff, kdiff, bdiff, out, N, H, L, E, E, flags, stream);
 }
 
 int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
@@ -281,14 +263,15 @@ int srwm_backward_f32(const float *x, const int64_t xs[3], const float *q, const
                                   wb, grad_x, gWy, gWq, gWk, gwb, N, H, L, E, E, flags, stream);
 }
 
-int srwm_layer_backward_f32(const float *x, const int64_t xs[3], const float *q, const float *k,
-                            const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
-                            const float *bdiff, const float *grad_out, const int64_t gs[3],
-                            const float *sWy, const float *sWq, const float *sWk, const float *swb,
-                            const float *Wy, const float *Wq, const float *Wk, const float *wb,
-                            float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, float *gsWy,
-                            float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
-                            unsigned flags, void *stream) {
+// body of the layer backward for both input types: `x` and `grad_out` are float or bf16 (io16)
+static int layer_backward(bool io16, const float *x, const int64_t xs[3], const float *q, const float *k,
+                          const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
+                          const float *bdiff, const float *grad_out, const int64_t gs[3],
+                          const float *sWy, const float *sWq, const float *sWk, const float *swb,
+                          const float *Wy, const float *Wq, const float *Wk, const float *wb,
+                          float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, float *gsWy,
+                          float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
+                          unsigned flags, void *stream) {
     if (!x || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff || !grad_out || !Wy || !Wq ||
         !Wk || !wb || !grad_x || !gWy || !gWq || !gWk || !gwb || !xs || !gs)
         return SRWM_EINVAL;
@@ -302,7 +285,8 @@ int srwm_layer_backward_f32(const float *x, const int64_t xs[3], const float *q,
     SrwmBwdParams p{x, xs[0], xs[1], xs[2], q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out,
                     gs[0], gs[1], gs[2], Wy, Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, N, H, L, E, mode, Y,
                     sWy, sWq, sWk, swb};
-    p.mode = ((flags & SRWM_FLAG_STATE_SHIFT) ? kModeShift : 0u) | ((flags & SRWM_FLAG_SOFTMAX_INPUT) ? kModeSoftmaxX : 0u);
+    p.mode = ((flags & SRWM_FLAG_STATE_SHIFT) ? kModeShift : 0u) | ((flags & SRWM_FLAG_SOFTMAX_INPUT) ? kModeSoftmaxX : 0u) |
+             (io16 ? kModeBf16 : 0u);
     hipStream_t s = (hipStream_t)stream;
     int r = -1;
     if (!(flags & SRWM_FLAG_GENERIC)) r = launch_srwm_bwd_tiled(p, s);
@@ -314,6 +298,44 @@ int srwm_layer_backward_f32(const float *x, const int64_t xs[3], const float *q,
     const float *const src[4] = {gWy, gWq, gWk, gwb};
     float *const dst[4] = {gsWy, gsWq, gsWk, gswb};
     return launch_srwm_batch_sum(src, dst, N, H, E, Y, s);
+}
+
+int srwm_layer_backward_f32(const float *x, const int64_t xs[3], const float *q, const float *k,
+                            const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
+                            const float *bdiff, const float *grad_out, const int64_t gs[3],
+                            const float *sWy, const float *sWq, const float *sWk, const float *swb,
+                            const float *Wy, const float *Wq, const float *Wk, const float *wb,
+                            float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, float *gsWy,
+                            float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
+                            unsigned flags, void *stream) {
+    return layer_backward(false, x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, sWy, sWq, sWk, swb, Wy,
+                          Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags,
+                          stream);
+}
+
+int srwm_layer_backward_bf16(const uint16_t *x, const int64_t xs[3], const float *q, const float *k,
+                             const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
+                             const float *bdiff, const uint16_t *grad_out, const int64_t gs[3],
+                             const float *sWy, const float *sWq, const float *sWk, const float *swb,
+                             const float *Wy, const float *Wq, const float *Wk, const float *wb,
+                             float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, float *gsWy,
+                             float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
+                             unsigned flags, void *stream) {
+    return layer_backward(true, reinterpret_cast<const float *>(x), xs, q, k, beta, ydiff, qdiff, kdiff, bdiff,
+                          reinterpret_cast<const float *>(grad_out), gs, sWy, sWq, sWk, swb, Wy, Wq, Wk, wb, grad_x,
+                          gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags, stream);
+}
+
+int srwm_backward_bf16(const uint16_t *x, const int64_t xs[3], const float *q, const float *k,
+                       const float *beta, const float *ydiff, const float *qdiff, const float *kdiff,
+                       const float *bdiff, const uint16_t *grad_out, const int64_t gs[3], const float *Wy,
+                       const float *Wq, const float *Wk, const float *wb, float *grad_x, float *gWy,
+                       float *gWq, float *gWk, float *gwb, int N, int H, int L, int E, unsigned flags,
+                       void *stream) {
+    if (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)) return SRWM_EINVAL;
+    return srwm_layer_backward_bf16(x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, nullptr, nullptr,
+                                    nullptr, nullptr, Wy, Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, nullptr, nullptr,
+                                    nullptr, nullptr, N, H, L, E, E, flags, stream);
 }
 
 int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],

@@ -181,14 +181,15 @@ class SelfRefLayerFn(torch.autograd.Function):
         fresh = shift_y is None
         assert all((s is None) == fresh for s in shifts), "give all four shifts or none"
         widths = (Y, E, E, 4)
+        f32 = torch.float32   # x (and with it out and the gradient handed back for x) may be bfloat16; the rest is fp32
         if fresh:
-            state = [torch.empty((N, H, E, w), device=dev, dtype=x.dtype) for w in widths]
+            state = [torch.empty((N, H, E, w), device=dev, dtype=f32) for w in widths]
         else:
             state = [s.detach().clone(memory_format=torch.contiguous_format) for s in shifts]
-        big = lambda: torch.empty((N, H, L, E), device=dev, dtype=x.dtype)
-        wide = lambda: torch.empty((N, H, L, Y), device=dev, dtype=x.dtype)
-        small = lambda: torch.empty((N, H, L, 4), device=dev, dtype=x.dtype)
-        out = wide()
+        big = lambda: torch.empty((N, H, L, E), device=dev, dtype=f32)
+        wide = lambda: torch.empty((N, H, L, Y), device=dev, dtype=f32)
+        small = lambda: torch.empty((N, H, L, 4), device=dev, dtype=f32)
+        out = torch.empty((N, H, L, Y), device=dev, dtype=x.dtype)
         saved = [big(), big(), small(), wide(), big(), big(), small()]
         flags = srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_FRESH_STATE if fresh else 0) | \
             (srwm_hip.FLAG_SOFTMAX_INPUT if softmax_input else 0)
@@ -215,19 +216,20 @@ class SelfRefLayerFn(torch.autograd.Function):
             grad_W = [torch.empty_like(s) for s in state]
             mode = srwm_hip.GRAD_STATE_ZERO
         need_slow = any(ctx.needs_input_grad[1:5])
-        grad_slow = [torch.empty((H, E, w), device=x.device, dtype=x.dtype) for w in (Y, E, E, 4)] \
+        grad_slow = [torch.empty((H, E, w), device=x.device, dtype=torch.float32) for w in (Y, E, E, 4)] \
             if need_slow else None
         # d(shift_out)/d(shared) = dW_L/d(shared) - 1: the incoming state gradient is taken off again
         minus = [g.sum(0) for g in grad_W] if (has_gs and need_slow) else None
-        grad_x = torch.empty(x.shape, device=x.device, dtype=x.dtype)
+        grad_x = torch.empty(x.shape, device=x.device, dtype=torch.float32)
         flags = mode | srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_SOFTMAX_INPUT if ctx.softmax_input else 0)
-        srwm_hip.self_ref_layer_backward(x, *saved, grad_out, slow, *state, grad_x, grad_W, grad_slow, flags=flags)
+        srwm_hip.self_ref_layer_backward(x, *saved, grad_out.to(x.dtype), slow, *state, grad_x, grad_W, grad_slow,
+                                         flags=flags)
         gs = [None] * 4
         if need_slow:
             gs = [(g - m if minus is not None else g).reshape(s.shape) for g, m, s in
                   zip(grad_slow, minus or [None] * 4, slow)]
         gshift = [None] * 4 if ctx.fresh else grad_W
-        return (grad_x, *gs, *gshift, None)
+        return (grad_x.to(x.dtype), *gs, *gshift, None)
 
 
 self_ref_layer = SelfRefLayerFn.apply

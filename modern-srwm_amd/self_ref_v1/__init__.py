@@ -5,7 +5,7 @@ class, call signature and in-place final-state semantics -- backed by libsrwm_hi
     out = self_ref_v1(x, W_y, W_q, W_k, w_b)
 
 x: (N, H, L, E); W_y: (N, H, E, 3E+1); W_q, W_k: (N, H, E, E); w_b: (N, H, E, 4); float32 on the
-GPU.  out: (N, H, L, 3E+1), the query | key | value | beta pre-activations of a following
+GPU (x may also be bfloat16: out is then bfloat16, the state stays float32).  out: (N, H, L, 3E+1), the query | key | value | beta pre-activations of a following
 fast-weight layer.  The recurrence is that of `self_ref_v0` with more output columns: all of
 them share the first of the four learning rates.  The weight tensors are OVERWRITTEN with the
 state after the last step; the backward starts from that mutated tensor.  Any width of W_y is
@@ -34,10 +34,11 @@ class SelfRefv1(torch.autograd.Function):
         assert W_k.shape == (N, H, E, E), "Reshape/unsqueeze if needed."
         assert w_b.shape == (N, H, E, 4), "Reshape/unsqueeze if needed."
         # every element is written by the kernel, so no zero-fill is needed
-        big = lambda: torch.empty((N, H, L, E), device=device, dtype=x.dtype)
-        wide = lambda: torch.empty((N, H, L, Y), device=device, dtype=x.dtype)
-        small = lambda: torch.empty((N, H, L, 4), device=device, dtype=x.dtype)
-        out = wide()
+        f32 = torch.float32   # x may be bfloat16 (out and the gradient handed back for x then too); the rest is fp32
+        big = lambda: torch.empty((N, H, L, E), device=device, dtype=f32)
+        wide = lambda: torch.empty((N, H, L, Y), device=device, dtype=f32)
+        small = lambda: torch.empty((N, H, L, 4), device=device, dtype=f32)
+        out = torch.empty((N, H, L, Y), device=device, dtype=x.dtype)
         q_main, k_main, beta_main = big(), big(), small()
         y_diff, q_diff, k_diff, beta_diff = wide(), big(), big(), small()
         SelfRefv1.dot[device.type](x, W_y, W_q, W_k, w_b, q_main, k_main, beta_main, y_diff, q_diff,
@@ -49,15 +50,15 @@ class SelfRefv1(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         (x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, W_y, W_q, W_k, w_b) = ctx.saved_tensors
-        grad_x = torch.empty(x.shape, device=x.device, dtype=x.dtype)
+        grad_x = torch.empty(x.shape, device=x.device, dtype=torch.float32)
         grad_W_y = torch.empty_like(W_y, memory_format=torch.contiguous_format)
         grad_W_q = torch.empty_like(W_q, memory_format=torch.contiguous_format)
         grad_W_k = torch.empty_like(W_k, memory_format=torch.contiguous_format)
         grad_w_b = torch.empty_like(w_b, memory_format=torch.contiguous_format)
         SelfRefv1.dot_backward[x.device.type](
-            x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out, W_y, W_q, W_k, w_b,
+            x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out.to(x.dtype), W_y, W_q, W_k, w_b,
             grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b, flags=srwm_hip.GRAD_STATE_ZERO)
-        return grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b
+        return grad_x.to(x.dtype), grad_W_y, grad_W_q, grad_W_k, grad_w_b
 
 
 # Alias the autograd functions to python style snake case naming

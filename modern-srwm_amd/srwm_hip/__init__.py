@@ -34,7 +34,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _lib = None
 
@@ -51,6 +51,8 @@ _SIGNATURES = {
     "srwm_backward_wide_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_layer_forward_f32": [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_layer_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_forward_bf16": [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_backward_bf16": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_wide_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 4 + [_U, ctypes.c_void_p],
@@ -168,8 +170,8 @@ def self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, 
     """SRWM forward over the whole sequence.  W_y, W_q, W_k, w_b are overwritten with the
     final state; q ... out are overwritten with the per-step vectors.  W_y is (N, H, E, Y):
     Y = E for the plain operator, any other width (3E+1 in the reference's second variant)
-    makes out and y_diff (N, H, L, Y).  x and out may both be bfloat16 (Y = E only); everything
-    else stays float32."""
+    makes out and y_diff (N, H, L, Y).  x and out may both be bfloat16; everything else stays
+    float32."""
     io = x.dtype if isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 else torch.float32
     _require(x, "x", None, io)
     N, H, L, E = x.shape
@@ -185,17 +187,20 @@ def self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, 
     _require(out, "out", (N, H, L, Y), io)
     _require(beta, "beta", (N, H, L, 4))
     _require(beta_diff, "beta_diff", (N, H, L, 4))
-    if io == torch.bfloat16 and Y != E:
-        raise ValueError("bfloat16 input is supported for W_y of shape (N, H, E, E) only")
     if x.numel() == 0 or Y == 0:
         return
     xs, xstr = _strided(x)
+    null = ctypes.c_void_p(None)
     with torch.cuda.device(x.device), \
             _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out], True) as d:
-        if io == torch.bfloat16:
+        if io == torch.bfloat16 and Y == E:
             name = "srwm_forward_bf16"
             code = lib().srwm_forward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
                                            _stream(x.device))
+        elif io == torch.bfloat16:   # wide output block: the layer entry point without any of its extras
+            name = "srwm_layer_forward_bf16"
+            code = lib().srwm_layer_forward_bf16(_ptr(xs), xstr, null, null, null, null, null,
+                                                 *[_ptr(t) for t in d], N, H, L, E, Y, flags, _stream(x.device))
         elif Y == E:
             name = "srwm_forward_f32"
             code = lib().srwm_forward_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
@@ -288,7 +293,7 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
     gradient w.r.t. the final state and the result is added to them (identical to a plain
     overwrite when they arrive zero-filled, which is how SelfRefv0.backward calls it).
     W_y (N, H, E, Y) fixes the width of y_diff, grad_out and grad_W_y.  x and grad_out may both be
-    bfloat16 (Y = E only); grad_x and everything else stay float32."""
+    bfloat16; grad_x and everything else stay float32."""
     io = x.dtype if isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 else torch.float32
     _require(x, "x", None, io)
     N, H, L, E = x.shape
@@ -298,8 +303,6 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
         _require(t, nm, (N, H, L, E))
     _require(y_diff, "y_diff", (N, H, L, Y))
     _require(grad_out, "grad_out", (N, H, L, Y), io)
-    if io == torch.bfloat16 and Y != E:
-        raise ValueError("bfloat16 input is supported for W_y of shape (N, H, E, E) only")
     _require(beta, "beta", (N, H, L, 4))
     _require(beta_diff, "beta_diff", (N, H, L, 4))
     for t, nm in ((W_y, "W_y"), (grad_W_y, "grad_W_y")):
@@ -320,11 +323,18 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
             _Dense([q, k, beta, y_diff, q_diff, k_diff, beta_diff], False) as sv, \
             _Dense([W_y, W_q, W_k, w_b], False) as st, \
             _Dense([grad_x, grad_W_y, grad_W_q, grad_W_k, grad_w_b], True) as gr:
-        if io == torch.bfloat16:
+        if io == torch.bfloat16 and Y == E:
             name = "srwm_backward_bf16"
             code = lib().srwm_backward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
                                             *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
                                             N, H, L, E, flags, _stream(x.device))
+        elif io == torch.bfloat16:
+            null = ctypes.c_void_p(None)
+            name = "srwm_layer_backward_bf16"
+            code = lib().srwm_layer_backward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
+                                                  null, null, null, null, *[_ptr(t) for t in st],
+                                                  *[_ptr(t) for t in gr], null, null, null, null,
+                                                  N, H, L, E, Y, flags, _stream(x.device))
         elif Y == E:
             name = "srwm_backward_f32"
             code = lib().srwm_backward_f32(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
@@ -357,8 +367,9 @@ def self_ref_layer_forward(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff
     weights (W_y: (1, H, E, Y) or (H, E, Y), ...), read without a repeat(); flags FLAG_FRESH_STATE
     (start from them, W_* are outputs), FLAG_STATE_SHIFT (W_* hold the state minus the shared
     weights, in and out), FLAG_SOFTMAX_INPUT (x is soft-maxed by the kernel); keep as in
-    self_ref_forward_steps."""
-    _require(x, "x")
+    self_ref_forward_steps.  x and out may both be bfloat16."""
+    io = x.dtype if isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 else torch.float32
+    _require(x, "x", None, io)
     N, H, L, E = x.shape
     _require(W_y, "W_y")
     Y = W_y.shape[-1]
@@ -368,8 +379,8 @@ def self_ref_layer_forward(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff
     _require(w_b, "w_b", (N, H, E, 4))
     for t, nm in ((q, "q"), (k, "k"), (q_diff, "q_diff"), (k_diff, "k_diff")):
         _require(t, nm, (N, H, L, E))
-    for t, nm in ((y_diff, "y_diff"), (out, "out")):
-        _require(t, nm, (N, H, L, Y))
+    _require(y_diff, "y_diff", (N, H, L, Y))
+    _require(out, "out", (N, H, L, Y), io)
     _require(beta, "beta", (N, H, L, 4))
     _require(beta_diff, "beta_diff", (N, H, L, 4))
     sl = _shared(slow, H, E, Y)
@@ -388,25 +399,28 @@ def self_ref_layer_forward(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff
     xs, xstr = _strided(x)
     with torch.cuda.device(x.device), \
             _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out], True) as d:
-        code = lib().srwm_layer_forward_f32(
+        name = "srwm_layer_forward_bf16" if io == torch.bfloat16 else "srwm_layer_forward_f32"
+        code = getattr(lib(), name)(
             _ptr(xs), xstr, _ptr(keep) if keep is not None else null, *[_ptr(t) for t in sl],
             *[_ptr(t) for t in d], N, H, L, E, Y, flags, _stream(x.device))
-    _check(code, "srwm_layer_forward_f32")
+    _check(code, name)
 
 
 def self_ref_layer_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out, slow,
                             W_y, W_q, W_k, w_b, grad_x, grad_W, grad_slow, flags=GRAD_STATE_ZERO):
     """Backward of self_ref_layer_forward (without resets).  W_*: the final state as the forward
     left it; grad_W: four (N, H, E, .) tensors (SRWM_GRAD_STATE_* semantics, per batch row);
-    grad_slow: four (H, E, .) tensors receiving the sum of grad_W over the batch, or None."""
-    _require(x, "x")
+    grad_slow: four (H, E, .) tensors receiving the sum of grad_W over the batch, or None.
+    x and grad_out may both be bfloat16; every gradient comes back in float32."""
+    io = x.dtype if isinstance(x, torch.Tensor) and x.dtype == torch.bfloat16 else torch.float32
+    _require(x, "x", None, io)
     N, H, L, E = x.shape
     _require(W_y, "W_y")
     Y = W_y.shape[-1]
     for t, nm in ((q, "q"), (k, "k"), (q_diff, "q_diff"), (k_diff, "k_diff"), (grad_x, "grad_x")):
         _require(t, nm, (N, H, L, E))
-    for t, nm in ((y_diff, "y_diff"), (grad_out, "grad_out")):
-        _require(t, nm, (N, H, L, Y))
+    _require(y_diff, "y_diff", (N, H, L, Y))
+    _require(grad_out, "grad_out", (N, H, L, Y), io)
     _require(beta, "beta", (N, H, L, 4))
     _require(beta_diff, "beta_diff", (N, H, L, 4))
     shapes = ((N, H, E, Y), (N, H, E, E), (N, H, E, E), (N, H, E, 4))
@@ -437,11 +451,12 @@ def self_ref_layer_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, gr
     with torch.cuda.device(x.device), \
             _Dense([q, k, beta, y_diff, q_diff, k_diff, beta_diff], False) as sv, \
             _Dense([W_y, W_q, W_k, w_b], False) as st, _Dense([grad_x], True) as gx:
-        code = lib().srwm_layer_backward_f32(
+        name = "srwm_layer_backward_bf16" if io == torch.bfloat16 else "srwm_layer_backward_f32"
+        code = getattr(lib(), name)(
             _ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr, *[_ptr(t) for t in sl],
             *[_ptr(t) for t in st], _ptr(gx[0]), *[_ptr(g) for g in grad_W], *gsl,
             N, H, L, E, Y, flags, _stream(x.device))
-    _check(code, "srwm_layer_backward_f32")
+    _check(code, name)
 
 
 # names of the extension functions of the reference's wide-output variant

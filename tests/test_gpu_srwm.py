@@ -416,27 +416,32 @@ BF16_TOL = 2e-2   # bf16 I/O with fp32 state: the output is rounded to 8 signifi
 
 
 @pytest.mark.parametrize("flags", KERNELS)
-@pytest.mark.parametrize("shape,w_std,xsm", [
-    ((2, 16, 200, 64), 0.02, False),            # headline head size
-    ((4, 8, 100, 32), 1 / math.sqrt(32), True),  # RL shape
-    ((2, 2, 9, 16), 0.5, True),
-    ((1, 3, 7, 12), 0.5, False),                # LDS-resident kernels only
+@pytest.mark.parametrize("shape,w_std,xsm,Y", [
+    ((2, 16, 200, 64), 0.02, False, None),            # headline head size
+    ((4, 8, 100, 32), 1 / math.sqrt(32), True, None),  # RL shape
+    ((2, 2, 9, 16), 0.5, True, None),
+    ((1, 3, 7, 12), 0.5, False, None),                # LDS-resident kernels only
+    ((4, 8, 50, 32), 1 / math.sqrt(32), True, 97),    # wide output block, RL shape
+    ((2, 2, 9, 8), 0.5, True, 25),
+    ((2, 2, 9, 12), 0.5, False, 20),                  # any width: LDS-resident kernels
 ])
-def test_bf16_io_matches_the_oracle_on_the_rounded_inputs(shape, w_std, xsm, flags):
+def test_bf16_io_matches_the_oracle_on_the_rounded_inputs(shape, w_std, xsm, Y, flags):
     """x and grad_out are rounded to bf16 first and the fp64 oracle runs on those values, so the only
     differences left are fp32 arithmetic (1e-5) in the saved vectors and gradients and the final
     rounding of `out` to bf16."""
-    print(f"case bf16 shape={shape} flags={flags}", flush=True)
+    print(f"case bf16 shape={shape} Y={Y} flags={flags}", flush=True)
     import srwm_hip
-    x, W, go = srwm_inputs(*shape, seed=2, w_std=w_std, x_softmax=xsm, per_batch_state=True)
+    x, W, go = srwm_inputs(*shape, seed=2, w_std=w_std, x_softmax=xsm, per_batch_state=True, y_width=Y)
     xb, gob = x.to(torch.bfloat16), go.to(torch.bfloat16)
     N, H, L, E = shape
+    Y = E if Y is None else Y
     dev = _dev()
     Wd = [w.to(dev, torch.float32).contiguous() for w in W]
     big = lambda: torch.full((N, H, L, E), float("nan"), device=dev)
+    wide = lambda: torch.full((N, H, L, Y), float("nan"), device=dev)
     small = lambda: torch.full((N, H, L, 4), float("nan"), device=dev)
-    f = dict(q=big(), k=big(), beta=small(), y_diff=big(), q_diff=big(), k_diff=big(), beta_diff=small(),
-             out=torch.zeros((N, H, L, E), device=dev, dtype=torch.bfloat16))
+    f = dict(q=big(), k=big(), beta=small(), y_diff=wide(), q_diff=big(), k_diff=big(), beta_diff=small(),
+             out=torch.zeros((N, H, L, Y), device=dev, dtype=torch.bfloat16))
     srwm_hip.self_ref_forward(xb.to(dev), *Wd, *[f[n] for n in FWD_NAMES], flags=flags)
     gx = torch.full((N, H, L, E), float("nan"), device=dev)
     g = [torch.full_like(w, float("nan")) for w in Wd]
@@ -473,6 +478,39 @@ def test_bf16_autograd_operator():
     assert rel_err(out.float().detach().cpu().numpy(), of["out"]) < BF16_TOL
     assert rel_err(xb.grad.float().cpu().numpy(), ob["grad_x"]) < BF16_TOL
     assert rel_err(Wd[0].grad.cpu().numpy(), ob["grad_W_y"]) < TOL
+
+
+@pytest.mark.parametrize("shape,Y", [((3, 4, 20, 32), 32), ((2, 4, 30, 64), 64), ((3, 4, 20, 32), 97), ((2, 3, 9, 12), 12)])
+def test_bf16_fused_layer_operator(shape, Y):
+    """self_ref_layer with a bf16 layer input: softmax in the kernel on the widened input, fresh state
+    from the shared weights, batch-summed weight gradients -- against fp64 autograd on the rounded input."""
+    print(f"case bf16 fused layer op shape={shape} Y={Y}", flush=True)
+    from oracle.recurrence import srwm_recurrence
+    from self_ref_v0 import self_ref_layer
+    N, H, L, E = shape
+    g = torch.Generator().manual_seed(23)
+    std = 1.0 / math.sqrt(E)
+    xr = torch.randn(N, H, L, E, generator=g, dtype=torch.float64).to(torch.bfloat16)
+    slow = [torch.randn(1, H, E, w, generator=g, dtype=torch.float64) * std for w in (Y, E, E, 4)]
+    go = torch.randn(N, H, L, Y, generator=g, dtype=torch.float64).to(torch.bfloat16)
+    dev = _dev()
+    x_lnhe = xr.permute(2, 0, 1, 3).contiguous().to(dev).requires_grad_(True)   # layer storage order, bf16
+    slow_d = [w.to(dev, torch.float32).requires_grad_(True) for w in slow]
+    out, *new = self_ref_layer(x_lnhe.permute(1, 2, 0, 3), *slow_d, None, None, None, None, True)
+    assert out.dtype == torch.bfloat16 and new[0].dtype == torch.float32
+    (out * go.to(dev)).sum().backward()
+    xc = xr.double().requires_grad_(True)
+    slow_c = [w.clone().requires_grad_(True) for w in slow]
+    out_c, final = srwm_recurrence(torch.softmax(xc, -1), *[w.repeat(N, 1, 1, 1) for w in slow_c])
+    (out_c * go.double()).sum().backward()
+    assert rel_err(out.float().detach().cpu().numpy(), out_c.detach().numpy()) < BF16_TOL
+    for a, b, w in zip(new, final, slow):   # the returned shift: final state minus the shared weights, fp32
+        want = b.detach() - w.repeat(N, 1, 1, 1)
+        assert (a.detach().cpu().double() - want).abs().max().item() < TOL * max(1.0, b.abs().max().item())
+    assert x_lnhe.grad.dtype == torch.bfloat16
+    assert rel_err(x_lnhe.grad.float().permute(1, 2, 0, 3).cpu().numpy(), xc.grad.numpy()) < BF16_TOL
+    for a, b in zip(slow_d, slow_c):
+        assert rel_err(a.grad.cpu().numpy(), b.grad.numpy()) < TOL
 
 
 # ---------------------------------------------------------------- readout-gradient replay kernels
