@@ -86,20 +86,25 @@ __global__ __launch_bounds__(kThreads) void replay_kernel(ReplayParams p) {
 }
 
 // Register-resident replay.  NWV waves per sequence; wave w owns rows [w*ER, (w+1)*ER), ER = E/NWV.
-// Inside a wave, CGL consecutive lanes share a block of R rows and split its M columns (CB each).
+// Inside a wave, CGL consecutive lanes share a block of R rows and split its columns (CB each).
+// M need not be a multiple of CGL or of 4 (the wide output block of the SRWM has M = 3E+1): the
+// lanes then tile MP = M rounded up to a multiple of CGL columns, the surplus columns are zero
+// throughout, and the rows of g and b -- no longer 16-byte aligned -- are fetched word by word.
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 template <int E, int M, int NWV, int CGL>
 __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p) {
-    constexpr int ER = E / NWV, RGL = kWave / CGL, R = ER / RGL, CB = M / CGL;
+    constexpr int MP = (M + CGL - 1) / CGL * CGL;
+    constexpr bool WORDS = MP != M || M % 4 != 0;   // rows of g, b fetched word by word
+    constexpr int ER = E / NWV, RGL = kWave / CGL, R = ER / RGL, CB = MP / CGL;
     constexpr int TT = M > 64 ? 8 : (256 / ER > 16 ? 256 / ER : 16);   // steps per tile
-    constexpr int NG = TT * M / 4 / kWave, NA = TT * ER / 4 / kWave;    // float4 per lane per tile
-    static_assert(ER * NWV == E && R * RGL == ER && CB * CGL == M && R >= 1 && CB >= 1, "tiling");
-    static_assert(NG * 4 * kWave == TT * M && NA * 4 * kWave == TT * ER && TT <= kWave, "tile loader");
+    constexpr int NG = WORDS ? 1 : TT * M / 4 / kWave, NA = TT * ER / 4 / kWave;   // float4 per lane per tile
+    constexpr int NWL = WORDS ? (TT * M + kWave - 1) / kWave : 1;                  // words per lane per tile
+    static_assert(ER * NWV == E && R * RGL == ER && CB * CGL == MP && R >= 1 && CB >= 1, "tiling");
+    static_assert((WORDS || NG * 4 * kWave == TT * M) && NA * 4 * kWave == TT * ER && TT <= kWave, "tile loader");
     static_assert(CGL <= 16, "row sums must stay inside a DPP row");
-
-    __shared__ __attribute__((aligned(16))) float tg[NWV][TT][M];    // g_t
-    __shared__ __attribute__((aligned(16))) float tb[NWV][TT][M];    // b_t
+    __shared__ __attribute__((aligned(16))) float tg[NWV][TT][MP];   // g_t
+    __shared__ __attribute__((aligned(16))) float tb[NWV][TT][MP];   // b_t
     __shared__ __attribute__((aligned(16))) float ta[NWV][TT][ER];   // this wave's rows of a_t
     __shared__ float tsk[NWV][2][TT];                                // s_t | keep_t
 
@@ -112,12 +117,20 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
     const float *gb = p.g + n * p.gs.n + h * p.gs.h;
     const float *bb = p.b + seq * p.L * M;
 
+    if constexpr (MP != M) {   // the surplus columns of the tiles stay zero: commits only write m < M
+        for (int i = lane; i < TT * (MP - M); i += kWave) {
+            tg[wave][i / (MP - M)][M + i % (MP - M)] = 0.f;
+            tb[wave][i / (MP - M)][M + i % (MP - M)] = 0.f;
+        }
+    }
+
     float w[R][CB];
     auto load_w = [&](const float *src) {   // src: E x M of this sequence / head, or nullptr for zero
 #pragma unroll
         for (int i = 0; i < R; ++i)
 #pragma unroll
-            for (int c = 0; c < CB; ++c) w[i][c] = src ? src[(e0 + r0 + i) * M + c0 + c] : 0.f;
+            for (int c = 0; c < CB; ++c)
+                w[i][c] = (src && (MP == M || c0 + c < M)) ? src[(e0 + r0 + i) * M + c0 + c] : 0.f;
     };
     load_w(p.W0 + seq * E * M);
     const float *wreset = p.Wreset ? p.Wreset + (int64_t)h * E * M : nullptr;
@@ -126,18 +139,29 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
     // starts one tile early so that fetch and commit each appear once in the code: with two call
     // sites the staging arrays end up in scratch memory instead of registers.
     v4f ng[NG], nb[NG], na[NA];   // native vectors: arrays of HIP float4 structs are not kept in registers here
+    float ngw[NWL], nbw[NWL];
     float ns = 1.f, nk = 1.f;
     const int ntiles = (p.L + TT - 1) / TT;
     for (int tile = -1; tile < ntiles; ++tile) {
         const bool more = tile + 1 < ntiles;
         if (more) {   // fetch tile + 1
             const int tb0 = (tile + 1) * TT;
+            if constexpr (WORDS) {
 #pragma unroll
-            for (int i = 0; i < NG; ++i) {
-                const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
-                const int64_t t = min(tb0 + row, p.L - 1);
-                ng[i] = *reinterpret_cast<const v4f *>(gb + t * p.gs.l + col);
-                nb[i] = *reinterpret_cast<const v4f *>(bb + t * M + col);
+                for (int i = 0; i < NWL; ++i) {
+                    const int f = min(lane + i * kWave, TT * M - 1), row = f / M, col = f - row * M;
+                    const int64_t t = min(tb0 + row, p.L - 1);
+                    ngw[i] = gb[t * p.gs.l + col];
+                    nbw[i] = bb[t * M + col];
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NG; ++i) {
+                    const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
+                    const int64_t t = min(tb0 + row, p.L - 1);
+                    ng[i] = *reinterpret_cast<const v4f *>(gb + t * p.gs.l + col);
+                    nb[i] = *reinterpret_cast<const v4f *>(bb + t * M + col);
+                }
             }
 #pragma unroll
             for (int i = 0; i < NA; ++i) {
@@ -188,11 +212,22 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
         }
         if (more) {   // commit tile + 1
             wave_lds_fence();   // this wave's reads of the current tile are done
+            if constexpr (WORDS) {
 #pragma unroll
-            for (int i = 0; i < NG; ++i) {
-                const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
-                *reinterpret_cast<v4f *>(&tg[wave][row][col]) = ng[i];
-                *reinterpret_cast<v4f *>(&tb[wave][row][col]) = nb[i];
+                for (int i = 0; i < NWL; ++i) {
+                    const int f = lane + i * kWave, row = f / M, col = f - row * M;
+                    if (f < TT * M) {
+                        tg[wave][row][col] = ngw[i];
+                        tb[wave][row][col] = nbw[i];
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < NG; ++i) {
+                    const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
+                    *reinterpret_cast<v4f *>(&tg[wave][row][col]) = ng[i];
+                    *reinterpret_cast<v4f *>(&tb[wave][row][col]) = nb[i];
+                }
             }
 #pragma unroll
             for (int i = 0; i < NA; ++i) {
@@ -208,6 +243,12 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
     }
 }
 
+template <int E, int M, int NWV, int CGL>
+int launch_replay_tiled_as(const ReplayParams &p, hipStream_t s) {
+    hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
+    return (int)hipGetLastError();
+}
+
 template <int E, int NWV, int CGL>
 int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
     hipLaunchKernelGGL((replay_tiled_kernel<E, E, NWV, CGL>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
@@ -220,10 +261,20 @@ bool rows16(const void *ptr, const Strided3 &st) {
 
 }  // namespace
 
-// Register-resident replay for square matrices with aligned rows; -1 when there is no instantiation.
+// Register-resident replay for square matrices with aligned rows and for E x (3E+1) ones (rows of
+// g and b at any alignment); -1 when there is no instantiation.
 int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
-    if (p.E != p.M || !rows16(p.a, p.as) || !rows16(p.g, p.gs) || (uintptr_t)p.b % 16 || (uintptr_t)p.u % 16)
-        return -1;
+    if (!rows16(p.a, p.as)) return -1;
+    if (p.M == 3 * p.E + 1) {
+        switch (p.E) {
+            case 64: return launch_replay_tiled_as<64, 193, 2, 8>(p, s);
+            case 32: return launch_replay_tiled_as<32, 97, 1, 8>(p, s);
+            case 16: return launch_replay_tiled_as<16, 49, 1, 8>(p, s);
+            case 8: return launch_replay_tiled_as<8, 25, 1, 8>(p, s);
+            default: return -1;
+        }
+    }
+    if (p.E != p.M || !rows16(p.g, p.gs) || (uintptr_t)p.b % 16 || (uintptr_t)p.u % 16) return -1;
     switch (p.E) {
         case 128: return launch_replay_tiled<128, 4, 16>(p, s);
         case 64: return launch_replay_tiled<64, 2, 8>(p, s);

@@ -515,21 +515,24 @@ def test_bf16_fused_layer_operator(shape, Y):
 
 # ---------------------------------------------------------------- readout-gradient replay kernels
 
-@pytest.mark.parametrize("E,NH,L", [(8, (2, 3), 70), (16, (2, 2), 33), (32, (4, 8), 100), (64, (2, 4), 50),
-                                    (128, (1, 2), 41)])
-def test_replay_kernels_agree_and_match_a_numpy_replay(E, NH, L):
+@pytest.mark.parametrize("E,NH,L,M", [(8, (2, 3), 70, 8), (16, (2, 2), 33, 16), (32, (4, 8), 100, 32),
+                                      (64, (2, 4), 50, 64), (128, (1, 2), 41, 128),
+                                      # the wide output block, M = 3E+1 (rows of g and b at any alignment)
+                                      (8, (2, 3), 70, 25), (16, (2, 2), 33, 49), (32, (4, 8), 100, 97),
+                                      (64, (2, 2), 19, 193)])
+def test_replay_kernels_agree_and_match_a_numpy_replay(E, NH, L, M):
     """u_t = W_{t-1} g_t with W_t = W_{t-1} + a_t (x) (s_t b_t) and resets: the register-resident
     kernel, the LDS-resident kernel and an fp64 numpy loop."""
-    print(f"case replay E={E} L={L}", flush=True)
+    print(f"case replay E={E} M={M} L={L}", flush=True)
     import srwm_hip
     N, H = NH
     g = torch.Generator().manual_seed(E)
     a = torch.softmax(torch.randn(N, H, L, E, generator=g, dtype=torch.float64), -1)
-    b = torch.randn(N, H, L, E, generator=g, dtype=torch.float64) * 0.5
+    b = torch.randn(N, H, L, M, generator=g, dtype=torch.float64) * 0.5
     beta = torch.sigmoid(torch.randn(N, H, L, 4, generator=g, dtype=torch.float64))
-    go = torch.randn(N, H, L, E, generator=g, dtype=torch.float64)
-    W0 = torch.randn(N, H, E, E, generator=g, dtype=torch.float64) * 0.3
-    Wr = torch.randn(H, E, E, generator=g, dtype=torch.float64) * 0.3
+    go = torch.randn(N, H, L, M, generator=g, dtype=torch.float64)
+    W0 = torch.randn(N, H, E, M, generator=g, dtype=torch.float64) * 0.3
+    Wr = torch.randn(H, E, M, generator=g, dtype=torch.float64) * 0.3
     keep = (torch.rand(N, L, generator=g) > 0.1).double()
     # fp64 loop
     u_ref = np.zeros((N, H, L, E))
