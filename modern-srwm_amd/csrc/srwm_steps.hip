@@ -12,7 +12,7 @@
 // replays W forward in time from its entry value with the saved write vectors
 // (W += a (x) (s b)), applies the same resets, and reads W g before each write.
 //
-// Two kernels.  replay_tiled_kernel (square matrices of 8..128 rows): the matrix lives in
+// Two kernels.  replay_tiled_kernel (square matrices of 8..128 rows, and E x (3E+1)): the matrix lives in
 // registers, a wave owns a block of rows (all columns), so the row sums finish inside the wave
 // and the waves of a workgroup never meet -- no barrier in the whole kernel; the vectors of TT
 // steps are staged in a wave-private LDS tile, fetched one tile ahead.  replay_kernel (any
