@@ -16,7 +16,7 @@ achieved HBM rate of the operator's I/O contract.  `cpu_baseline` is the per-tim
 PyTorch recurrence (oracle/recurrence.py) timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk}.
+{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk}.
 """
 import argparse
 import json
@@ -48,6 +48,9 @@ WORKLOADS = {
     # name: (op, N, H, L, E)
     "srwm_c4": ("srwm", 32, 16, 512, 64),
     "srwm_c3": ("srwm", 32, 8, 100, 32),
+    # the headline shape through the layer operator: shared weights read directly (no per-row
+    # copies), softmax of the layer input inside the kernels, weight gradients summed over the batch
+    "srwm_layer_c4": ("srwm_layer", 32, 16, 512, 64),
     # the RL learner's regime on the same shape: gradient cut at the carried state, 5 % resets;
     # one launch for the unroll (forward) + readout-gradient replay + the batched x (x) g product
     "srwm_c3_steps": ("srwm_steps", 32, 8, 100, 32),
@@ -94,6 +97,21 @@ def srwm_step(t, ev=None):
         ev[1].record()
     srwm_hip.self_ref_backward(t["x"], *t["saved"], t["go"], *t["W"], t["gx"], *t["gW"],
                                flags=srwm_hip.GRAD_STATE_ZERO)
+    if ev:
+        ev[2].record()
+
+
+def srwm_layer_step(t, ev=None):
+    import srwm_hip
+    fl = srwm_hip.FLAG_STATE_SHIFT | srwm_hip.FLAG_SOFTMAX_INPUT
+    if ev:
+        ev[0].record()
+    srwm_hip.self_ref_layer_forward(t["x"], None, t["slow"], *t["W"], *t["saved"], t["out"],
+                                    flags=fl | srwm_hip.FLAG_FRESH_STATE)
+    if ev:
+        ev[1].record()
+    srwm_hip.self_ref_layer_backward(t["x"], *t["saved"], t["go"], t["slow"], *t["W"], t["gx"], t["gW"], t["gslow"],
+                                     flags=fl | srwm_hip.GRAD_STATE_ZERO)
     if ev:
         ev[2].record()
 
@@ -206,7 +224,7 @@ def delta_step(t, ev=None):
 def algorithmic_bytes(op, N, H, L, E):
     """(lds_fwd, lds_bwd, hbm_total) bytes per launch pair."""
     hs = N * H * L
-    if op == "srwm":
+    if op in ("srwm", "srwm_layer"):
         S = E * (3 * E + 4)
         return 3 * S * 4 * hs, 6 * S * 4 * hs, (15 * E + 16) * 4 * hs + 4 * S * 4 * N * H
     if op == "srwm_wide":    # as above with Y = 3E+1 output columns: y, y_diff, grad_out are Y wide
@@ -322,6 +340,10 @@ def main():
     op, N, H, L, E = WORKLOADS[a.workload]
     if op == "srwm":
         step, t = srwm_step, srwm_setup(N, H, L, E, dev)
+    elif op == "srwm_layer":
+        step, t = srwm_layer_step, srwm_setup(N, H, L, E, dev)
+        t["slow"] = [w[0].contiguous() for w in t["W0"]]
+        t["gslow"] = [torch.empty_like(w) for w in t["slow"]]
     elif op == "srwm_wide":
         step, t = srwm_step, srwm_setup(N, H, L, E, dev, 3 * E + 1)
     elif op == "srwm_steps":

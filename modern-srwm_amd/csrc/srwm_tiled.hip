@@ -96,7 +96,9 @@ __device__ __forceinline__ float4 row_softmax4(float4 v) {
 // RESET: the layer-level extras are compiled in -- the per-step reset to the shared weights
 // (p.keep), the state kept as a shift from them or started from them, the softmax of the input
 // (p.mode).  The plain operator runs the instantiation without them.
-template <int E, int NW, int R, bool RESET, int YB>
+// BF16: x and out are bf16 behind the float pointers (a compile-time switch: the output store
+// sits inside the step).
+template <int E, int NW, int R, bool RESET, int YB, bool BF16>
 __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams p) {
     using T = Tiling<E, NW, R>;
     constexpr int RG = T::RG, CGW = T::CGW, CB = T::CB, TT = T::TT;
@@ -183,7 +185,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         if constexpr (XC) wye = wye0;
     };
     const bool softmax_x = RESET && (p.mode & kModeSoftmaxX);
-    const bool bf16_io = RESET && (p.mode & kModeBf16);
+    constexpr bool bf16_io = BF16;
+    static_assert(RESET || !BF16, "bf16 input / output is compiled with the layer extras");
     // rows of the Y-wide tensors start at any word: no vector stores there
     auto store_y = [&](float *base, unsigned row, const float *v) {   // row = offset of the step's row inside the sequence
         if constexpr (XC) {
@@ -381,18 +384,21 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         };
 
         // ---- readout of step t+1, published before the write is carried out
-        if (RESET && reset_next) {
-            reset_state();   // the state of step t is dropped: the write is not needed
-            float acc[NC], pb, py = 0.f;
-            readout(xr, xb, acc, pb, py);
-            publish(t1, acc, pb, py);
-        } else {
+        {
 #pragma unroll
             for (int c = 0; c < NC; ++c) e[c] = fmaf(ins[c], kx, e[c]);
             float py = 0.f;
             if constexpr (XC) py = fmaf(insy, kx, s[4]);
             if (have_next) publish(t1, e, fmaf(insb, kx, s[2]), py);
             write_state();
+        }
+        if constexpr (RESET) {
+            if (__builtin_expect(reset_next, 0)) {   // rare: the state is replaced before step t+1, whose readout is redone and published again
+                reset_state();
+                float acc[NC], pb, py = 0.f;
+                readout(xr, xb, acc, pb, py);
+                publish(t1, acc, pb, py);
+            }
         }
 
         // x of step t+2 opens a new tile: commit the staged tile, fetch the one after it
@@ -842,10 +848,12 @@ int launch_bwd(const SrwmBwdParams &p, hipStream_t s) {
 
 template <int E, int NW, int R, int YB = 1>
 int launch_fwd(const SrwmFwdParams &p, hipStream_t s) {
-    if (p.keep || p.mode)
-        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, true, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    if (p.mode & kModeBf16)
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, true, YB, true>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    else if (p.keep || p.mode)
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, true, YB, false>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
     else
-        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, false, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, false, YB, false>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
