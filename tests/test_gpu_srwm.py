@@ -264,6 +264,44 @@ def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
         assert float(w.grad.abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("E,L", [(64, 15), (64, 16), (64, 17), (64, 32), (64, 33), (32, 31), (32, 32), (32, 33),
+                                 (32, 64), (16, 16), (16, 17), (8, 32), (8, 33)])
+def test_sequence_lengths_around_the_input_tile_size(E, L):
+    """The kernels stream the per-step vectors through LDS tiles of 16 or 32 steps and the forward
+    prepares the readout of step t+1 during step t: lengths one below, at and one above a whole
+    number of tiles, forward and backward."""
+    print(f"case tile boundary E={E} L={L}", flush=True)
+    x, W, go = srwm_inputs(2, 2, L, E, seed=L, w_std=0.3, x_softmax=True, per_batch_state=True)
+    check_against_oracle(x, W, go, 0)
+
+
+@pytest.mark.parametrize("E,L", [(64, 40), (32, 70)])
+def test_resets_at_tile_boundaries(E, L):
+    """Resets right before the first step, before the last step and on either side of every tile
+    boundary, in different batch rows and in the same one."""
+    print(f"case resets at tile boundaries E={E} L={L}", flush=True)
+    from oracle.recurrence import srwm_steps_reference
+    from self_ref_v0 import self_ref_v0_steps
+    from test_oracle_srwm import _steps_inputs
+    dev = _dev()
+    N, H = 4, 2
+    x, keep, shift, slow, go = _steps_inputs(N, H, L, E, seed=5, resets=True)
+    tile = 16 if E == 64 else 32
+    keep[:] = 1.0
+    keep[0, 0] = keep[0, L - 1] = 0.0
+    for b in range(tile, L, tile):
+        keep[1, b - 1] = 0.0          # last step of a tile
+        keep[2, b] = 0.0              # first step of the next
+        keep[3, b - 1] = keep[3, b] = keep[3, min(b + 1, L - 1)] = 0.0
+    ref_out, ref_shift = srwm_steps_reference(x, keep, shift, slow)
+    f32 = lambda t: t.to(dev, torch.float32)
+    fast = [f32(s_) + f32(w).repeat(N, 1, 1, 1) for s_, w in zip(shift, slow)]
+    out = self_ref_v0_steps(f32(x), f32(keep), *fast, *[f32(w) for w in slow])
+    assert rel_err(out.cpu().numpy(), ref_out.numpy()) < TOL
+    for fw_, rs, w in zip(fast, ref_shift, slow):
+        assert rel_err(fw_.cpu().numpy(), (rs + w).numpy()) < TOL
+
+
 # ---------------------------------------------------------------- wide output block (self_ref_v1)
 
 @pytest.mark.parametrize("shape,Y,w_std,xsm,per_batch", [
