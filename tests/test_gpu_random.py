@@ -1,0 +1,156 @@
+"""Seeded random shapes, strides, kernel families and gradient modes for both operators against the
+fp64 oracle, through the same host entry points as the fixed cases of the other GPU test files.
+
+Bar: 1e-5 relative to the largest element of each tensor (fp32 arithmetic on both sides of the
+comparison would meet it; the oracle is fp64).  One family of outputs is measured differently: the
+`*_diff` vectors the SRWM forward emits are W^T (q - k), sums with heavy cancellation when q and k
+are close, so their fp32 error is bounded by 1e-5 times |W|^T |q - k| (the size of the terms that
+cancel), not by 1e-5 times the result.  The test computes that scale from the oracle's own vectors.
+The gradient of w_b is, per step, a product with sum(g_ins * diff): it inherits the conditioning of
+the diffs and is allowed 1e-5 times the same amplification factor (about 2 to 4 in these cases).
+"""
+import math
+import random
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from helpers import delta_inputs, rel_err, srwm_inputs
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+
+def _cases(kind, count, seed):
+    rng = random.Random(seed)
+    out = []
+    for i in range(count):
+        if kind == "srwm":
+            E = rng.choice([8, 16, 32, 64, 5, 12, 20, 48])
+            wide = rng.random() < 0.35
+            Y = (3 * E + 1 if rng.random() < 0.7 else rng.randint(1, 2 * E)) if wide else E
+            if E > 32 and Y > 2 * E and Y != 3 * E + 1:
+                Y = 2 * E                                     # keeps the LDS-resident backward inside the CU's LDS
+            generic = rng.random() < 0.3
+            if E == 64 and Y == 3 * E + 1:
+                generic = False                               # that state only fits the register-resident kernels
+            out.append(dict(i=i, N=rng.randint(1, 3), H=rng.randint(1, 4), E=E, Y=Y,
+                            L=rng.choice([1, 2, 7, 15, 16, 17, 31, 33, 64, 65, 100, 129]),
+                            generic=generic, strided=rng.random() < 0.5, mode=rng.choice([0, 1, 2]),
+                            w_std=rng.choice([0.02, 0.3, 1 / math.sqrt(E)]), xsm=rng.random() < 0.5))
+        else:
+            D = rng.choice([8, 16, 32, 64, 128, 12, 40])
+            M = D if rng.random() < 0.8 else rng.choice([8, 24, 64])
+            chunkable = D == M and D in (64, 128)
+            out.append(dict(i=i, N=rng.randint(1, 2), H=rng.randint(1, 3), E=D, M=M,
+                            L=rng.choice([1, 3, 16, 63, 64, 65, 127, 130, 200]),
+                            fwd=rng.choice(["tiled", "tiled", "generic", "chunk"] if chunkable else ["tiled", "generic"]),
+                            bwd=rng.choice(["tiled", "generic", "chunk"] if chunkable else ["tiled", "generic"]),
+                            mode=rng.choice([0, 1]), strided=rng.random() < 0.5,
+                            qk=rng.choice(["softmax", "l2", "sumnorm"]), w0_std=rng.choice([0.0, 0.3])))
+    return out
+
+
+def _id(c):
+    return "-".join(f"{k}{v if not isinstance(v, float) else round(v, 3)}" for k, v in c.items())
+
+
+def _dev():
+    return torch.device("cuda:0")
+
+
+def _to_dev(t, strided):
+    """fp32 on the GPU; `strided`: a permuted view of (L, N, H, d) storage, as the layers pass it."""
+    if strided:
+        return t.permute(2, 0, 1, 3).contiguous().to(_dev(), torch.float32).permute(1, 2, 0, 3)
+    return t.to(_dev(), torch.float32)
+
+
+def _cancellation_scales(W0, of, L):
+    """max over steps and columns of (|W_{t-1}|^T |q_t - k_t|) for the four column blocks, the state
+    replayed from the oracle's own per-step vectors."""
+    W = [w.copy() for w in W0]
+    names = ("y_diff", "q_diff", "k_diff", "beta_diff")
+    scale = dict.fromkeys(names, 0.0)
+    for t in range(L):
+        dv = np.abs(of["q"][:, :, t] - of["k"][:, :, t])
+        k, beta = of["k"][:, :, t], of["beta"][:, :, t]
+        for j, (n, w) in enumerate(zip(names, W)):
+            scale[n] = max(scale[n], float(np.einsum("nhem,nhe->nhm", np.abs(w), dv).max()))
+            w += k[..., None] * (beta[..., j][..., None] * of[n][:, :, t])[:, :, None, :]
+    return scale
+
+
+@pytest.mark.parametrize("c", _cases("srwm", 64, 1234), ids=_id)
+def test_srwm_random_case(c):
+    print(f"case random srwm {c}", flush=True)
+    import srwm_hip
+    N, H, L, E, Y = c["N"], c["H"], c["L"], c["E"], c["Y"]
+    x, W, go = srwm_inputs(N, H, L, E, seed=1000 + c["i"], w_std=c["w_std"], x_softmax=c["xsm"],
+                           per_batch_state=True, y_width=Y)
+    gs = [torch.randn(w.shape, generator=torch.Generator().manual_seed(c["i"]), dtype=torch.float64) for w in W]
+    dev = _dev()
+    xd, god = _to_dev(x, c["strided"]), _to_dev(go, c["strided"])
+    Wd = [w.to(dev, torch.float32).contiguous() for w in W]
+    nan = lambda *shape: torch.full(shape, float("nan"), device=dev)
+    f = [nan(N, H, L, E), nan(N, H, L, E), nan(N, H, L, 4), nan(N, H, L, Y), nan(N, H, L, E), nan(N, H, L, E),
+         nan(N, H, L, 4), nan(N, H, L, Y)]
+    flags = srwm_hip.FLAG_GENERIC if c["generic"] else 0
+    srwm_hip.self_ref_forward(xd, *Wd, *f, flags=flags)
+    gx = nan(N, H, L, E)
+    mode = c["mode"]
+    gW = [s.to(dev, torch.float32).contiguous() for s in gs] if mode else [torch.full_like(w, float("nan")) for w in Wd]
+    srwm_hip.self_ref_backward(xd, *f[:-1], god, *Wd, gx, *gW, flags=flags | mode)
+
+    W0 = [w.numpy() for w in W]
+    of = oracle.srwm_forward(x.numpy(), *W0)
+    ob = oracle.srwm_backward(x.numpy(), of, go.numpy(), grad_state=[s.numpy() for s in gs] if mode else None)
+    scales = _cancellation_scales(W0, of, L)
+    names = ("q", "k", "beta", "y_diff", "q_diff", "k_diff", "beta_diff", "out")
+    for n, t in zip(names, f):
+        got = t.cpu().numpy()
+        if n.endswith("_diff"):
+            assert np.abs(got - of[n]).max() <= TOL * max(scales[n], np.abs(of[n]).max()), n
+        else:
+            assert rel_err(got, of[n]) < TOL, n
+    for n, t in zip(("W_y", "W_q", "W_k", "w_b"), Wd):
+        assert rel_err(t.cpu().numpy(), of[n]) < TOL, n
+    assert rel_err(gx.cpu().numpy(), ob["grad_x"]) < TOL
+    kappa = max(1.0, max(scales[n] / max(float(np.abs(of[n]).max()), 1e-300) for n in scales))
+    for n, t, s in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), gW, gs):
+        want = ob[n] + (s.numpy() if mode == 2 else 0.0)
+        assert rel_err(t.cpu().numpy(), want) < TOL * (kappa if n == "grad_w_b" else 1.0), n
+
+
+@pytest.mark.parametrize("c", _cases("delta", 64, 4321), ids=_id)
+def test_delta_random_case(c):
+    print(f"case random delta {c}", flush=True)
+    import srwm_hip
+    N, H, L, D, M = c["N"], c["H"], c["L"], c["E"], c["M"]
+    q, k, v, beta, W0, go = delta_inputs(N, H, L, D, M, seed=2000 + c["i"], qk=c["qk"], w0_std=c["w0_std"])
+    gsW = torch.randn(W0.shape, generator=torch.Generator().manual_seed(c["i"]), dtype=torch.float64)
+    dev = _dev()
+    flag = {"tiled": 0, "generic": srwm_hip.FLAG_GENERIC, "chunk": srwm_hip.FLAG_CHUNKWISE}
+    qd, kd, vd, bd, god = (_to_dev(t, c["strided"]) for t in (q, k, v, beta, go))
+    W = W0.to(dev, torch.float32).contiguous()
+    nan = lambda *shape: torch.full(shape, float("nan"), device=dev)
+    vo, vi, out = nan(N, H, L, M), nan(N, H, L, M), nan(N, H, L, M)
+    srwm_hip.fast_weight_forward(qd, kd, vd, bd, vo, vi, W, out, flags=flag[c["fwd"]])
+    W_L = W.clone()
+    gq, gk, gv, gb = nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, M), nan(N, H, L, 1)
+    mode = c["mode"]
+    gkv = gsW.to(dev, torch.float32).contiguous() if mode else torch.full_like(W, float("nan"))
+    srwm_hip.fast_weight_backward(qd, kd, vd, bd, vo, vi, god, W, gq, gk, gv, gb, grad_kv=gkv,
+                                  flags=flag[c["bwd"]] | mode)
+    base = [t.numpy() for t in (q, k, v, beta, W0)]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, go.numpy(), grad_state=gsW.numpy() if mode else None, want_grad_W=True)
+    assert rel_err(out.cpu().numpy(), of["out"]) < TOL
+    assert rel_err(vo.cpu().numpy(), of["v_old"]) < TOL
+    assert rel_err(W_L.cpu().numpy(), of["W"]) < TOL
+    # the backward leaves the memory reverted to its entry value: L fp32 rank-1 subtractions
+    assert np.abs(W.cpu().numpy() - W0.numpy()).max() < 2e-5 * max(1.0, float(np.abs(W0.numpy()).max()))
+    for n, t in (("grad_Q", gq), ("grad_K", gk), ("grad_V", gv), ("grad_beta", gb), ("grad_W", gkv)):
+        assert rel_err(t.cpu().numpy(), ob[n]) < TOL, n
