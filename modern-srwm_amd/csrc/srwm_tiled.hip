@@ -93,13 +93,16 @@ __device__ __forceinline__ float4 row_softmax4(float4 v) {
     return v;
 }
 
-// RESET: the layer-level extras are compiled in -- the per-step reset to the shared weights
-// (p.keep), the state kept as a shift from them or started from them, the softmax of the input
-// (p.mode).  The plain operator runs the instantiation without them.
+// XTRA selects how much of the layer-level extras is compiled in: 0 = the plain operator; 1 = the
+// mode bits of p.mode (state started from / kept as a shift from the shared weights, softmax of the
+// input), which cost nothing inside the step loop; 2 = also the per-step reset to the shared weights
+// (p.keep), which adds a check to every step and a register copy of the shared weights.
 // BF16: x and out are bf16 behind the float pointers (a compile-time switch: the output store
 // sits inside the step).
-template <int E, int NW, int R, bool RESET, int YB, bool BF16>
+template <int E, int NW, int R, int XTRA, int YB, bool BF16>
 __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams p) {
+    constexpr bool MODES = XTRA >= 1;   // p.mode: work outside the step loop only (entry / exit form of the state, input tiles)
+    constexpr bool RESET = XTRA >= 2;   // p.keep: a check, and now and then a reset, inside every step
     using T = Tiling<E, NW, R>;
     constexpr int RG = T::RG, CGW = T::CGW, CB = T::CB, TT = T::TT;
     constexpr int NB = YB + 2, NC = NB * CB;          // blocks of E columns: y (YB of them) | q | k
@@ -150,11 +153,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     };
     const float *shWy = p.sWy + (int64_t)h * E * Y, *shWq = p.sWq + (int64_t)h * E * E,
                 *shWk = p.sWk + (int64_t)h * E * E, *shwb = p.swb + (int64_t)h * E * 4;
-    if (RESET && (p.mode & kModeFresh)) {
+    if (MODES && (p.mode & kModeFresh)) {
         load_state(shWy, shWq, shWk, shwb, std::false_type{});
     } else {
         load_state(p.Wy + sEY, p.Wq + sEE, p.Wk + sEE, p.wb + sE4, std::false_type{});
-        if (RESET && (p.mode & kModeShift)) load_state(shWy, shWq, shWk, shwb, std::true_type{});   // incoming state is a shift
+        if (MODES && (p.mode & kModeShift)) load_state(shWy, shWq, shWk, shwb, std::true_type{});   // incoming state is a shift
     }
     // Per-step reset: the state is replaced by the weights all batch rows of this head share.  A
     // copy of this lane's part of them is kept in registers when the call can reset (fetching
@@ -184,9 +187,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         wbe = wbe0;
         if constexpr (XC) wye = wye0;
     };
-    const bool softmax_x = RESET && (p.mode & kModeSoftmaxX);
+    const bool softmax_x = MODES && (p.mode & kModeSoftmaxX);
     constexpr bool bf16_io = BF16;
-    static_assert(RESET || !BF16, "bf16 input / output is compiled with the layer extras");
+    static_assert(MODES || !BF16, "bf16 input / output is compiled with the layer extras");
     // rows of the Y-wide tensors start at any word: no vector stores there
     auto store_y = [&](float *base, unsigned row, const float *v) {   // row = offset of the step's row inside the sequence
         if constexpr (XC) {
@@ -414,7 +417,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     }
 
     // the final state, as the shift from the shared weights if that is how the caller keeps it
-    const bool as_shift = RESET && (p.mode & kModeShift);
+    const bool as_shift = MODES && (p.mode & kModeShift);
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         float *dst = b < YB ? p.Wy + sEY + b * E : b == YB ? p.Wq + sEE : p.Wk + sEE;
@@ -848,12 +851,15 @@ int launch_bwd(const SrwmBwdParams &p, hipStream_t s) {
 
 template <int E, int NW, int R, int YB = 1>
 int launch_fwd(const SrwmFwdParams &p, hipStream_t s) {
+    const dim3 grid(p.N * p.H), block(NW * kWave);
     if (p.mode & kModeBf16)
-        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, true, YB, true>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
-    else if (p.keep || p.mode)
-        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, true, YB, false>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, YB, true>), grid, block, 0, s, p);
+    else if (p.keep)
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, YB, false>), grid, block, 0, s, p);
+    else if (p.mode)
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 1, YB, false>), grid, block, 0, s, p);
     else
-        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, false, YB, false>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 0, YB, false>), grid, block, 0, s, p);
     return (int)hipGetLastError();
 }
 
