@@ -5,6 +5,7 @@
     CarryFastFFlayer                  reinforcement_learning/torchbeast/layer.py:128-189 (the RL tree
                                       calls it FastFFlayer too; it threads the memory as state)
     SMFWPlayer                        reinforcement_learning/torchbeast/layer.py:492-586
+    FastFastFFlayer, PseudoSRlayer    reinforcement_learning/torchbeast/layer.py:193-283, :286-336
 
 Same constructor arguments, parameter names and shapes (so state_dicts of the reference load
 unchanged: W_y, W_q, W_k: (1, H, d, d); w_b: (1, H, d, 4); slow_net / out_linear / layer_norm),
@@ -303,3 +304,69 @@ class CarryFastFFlayer(_DeltaBase):
         fast_weights = state.detach().clone()
         out = fast_weight_delta_steps(q, k, v, beta, keep, fast_weights)
         return self._finish(x, out, bsz, slen), fast_weights
+
+
+class FastFastFFlayer(nn.Module):
+    """Delta-rule layer whose memory (d x (3d+1)) generates, per step, the query | key | value | beta
+    of a second delta-rule memory (d x d): reinforcement_learning/torchbeast/layer.py:193-283.  Both
+    memories are passed in as state and the updated ones returned.  The reference binds
+    `fast_weight_memory`, a name none of its files define (:201-202); its arguments are those of the
+    delta-rule operator, which is what runs here."""
+
+    def __init__(self, num_head, dim_head, in_dim, dropout):
+        super().__init__()
+        self.num_head = num_head
+        self.dim_head = dim_head
+        self.in_dim = in_dim
+        self.fw_layer = fast_weight_delta
+        self.very_fw_layer = fast_weight_delta
+        self.cached_fast_weights = nn.Parameter(torch.zeros(1, num_head, dim_head, 3 * dim_head + 1),
+                                                requires_grad=False)
+        self.slow_net = nn.Linear(in_dim, num_head * (5 * dim_head + 2), bias=False)
+        self.layer_norm = nn.LayerNorm(in_dim)
+        self.out_linear = nn.Linear(num_head * dim_head, in_dim, bias=False)
+        self.drop = nn.Dropout(dropout)
+
+    def forward(self, x, state=None):
+        assert state is not None   # as the reference: the outer memory is carried over across episodes
+        slen, bsz, _ = x.size()
+        d = self.dim_head
+        qkvb = self.slow_net(self.layer_norm(x)).view(slen, bsz, self.num_head, 5 * d + 2)
+        q, k, v, beta = torch.split(qkvb, (d, d, 3 * d + 1, 1), -1)
+        beta = torch.sigmoid(beta)
+        q, k, v, beta = (t.permute(1, 2, 0, 3) for t in (q, k, v, beta))
+        fast_weights, very_fast_weights = state
+        out = self.fw_layer(elu_p1_sum_norm_eps(q), elu_p1_sum_norm_eps(k), v, beta, fast_weights)
+        fq, fk, fv, fbeta = torch.split(out, (d,) * 3 + (1,), -1)
+        out = self.very_fw_layer(elu_p1_sum_norm_eps(fq), elu_p1_sum_norm_eps(fk), fv, torch.sigmoid(fbeta),
+                                 very_fast_weights)
+        out = _heads_out(out, bsz, slen, self.num_head * d)
+        out = x + self.drop(self.out_linear(out))
+        return out, (fast_weights.clone(), very_fast_weights.clone())
+
+
+class PseudoSRlayer(nn.Module):
+    """The ablation of the self-referential layer whose weight matrix is never modified: a per-head
+    linear map (reinforcement_learning/torchbeast/layer.py:286-336).  No fast-weight operator is
+    involved; it is here so that the reference's layer set is complete."""
+
+    def __init__(self, num_head, dim_head, in_dim, dropout):
+        super().__init__()
+        self.num_head = num_head
+        self.dim_head = dim_head
+        self.in_dim = in_dim
+        self.W_y = nn.Parameter(torch.empty(num_head, dim_head, dim_head))
+        self.layer_norm = nn.LayerNorm(in_dim)
+        self.out_linear = nn.Linear(num_head * dim_head, in_dim, bias=False)
+        self.drop = nn.Dropout(dropout)
+        self.reset_rec_parameters()
+
+    def reset_rec_parameters(self):
+        nn.init.normal_(self.W_y, mean=0., std=1.0 / math.sqrt(self.dim_head))
+
+    def forward(self, h, state=None):
+        slen, bsz, _ = h.size()
+        x = h.reshape(slen * bsz, self.num_head, self.dim_head).permute(1, 0, 2)   # (H, len*B, d)
+        out = torch.bmm(x, self.W_y).permute(1, 0, 2).reshape(slen, bsz, self.num_head * self.dim_head)
+        out = h + self.drop(self.out_linear(out))
+        return out, state

@@ -161,6 +161,52 @@ def test_delta_layers():
     assert rel_err(new_state.cpu().numpy(), WL.detach().numpy()) < TOL
 
 
+def test_delta_delta_layer():
+    """FastFastFFlayer: a d x (3d+1) delta-rule memory whose readout drives a second, d x d one."""
+    print("case FastFastFFlayer", flush=True)
+    from layer import FastFastFFlayer, elu_p1_sum_norm_eps
+    torch.manual_seed(5)
+    L, B, H, d = 7, 2, 3, 16
+    gpu, cpu = _pair(FastFastFFlayer(H, d, H * d, 0.0))
+    x = torch.randn(L, B, H * d, dtype=torch.float64)
+    go = torch.randn(L, B, H * d, dtype=torch.float64)
+    W0 = torch.randn(B, H, d, 3 * d + 1, dtype=torch.float64) * 0.1
+    V0 = torch.randn(B, H, d, d, dtype=torch.float64) * 0.1
+    xg = x.to(_dev(), torch.float32).requires_grad_(True)
+    out, (Wn, Vn) = gpu(xg, (W0.to(_dev(), torch.float32), V0.to(_dev(), torch.float32)))
+    (out * go.to(_dev(), torch.float32)).sum().backward()
+
+    xc = x.clone().requires_grad_(True)
+    qkvb = cpu.slow_net(cpu.layer_norm(xc)).view(L, B, H, 5 * d + 2)
+    q, k, v, beta = torch.split(qkvb, (d, d, 3 * d + 1, 1), -1)
+    q, k, v, beta = (t.permute(1, 2, 0, 3) for t in (q, k, v, torch.sigmoid(beta)))
+    mid, WL = delta_recurrence(elu_p1_sum_norm_eps(q), elu_p1_sum_norm_eps(k), v, beta, W0)
+    fq, fk, fv, fb = torch.split(mid, (d,) * 3 + (1,), -1)
+    o2, VL = delta_recurrence(elu_p1_sum_norm_eps(fq), elu_p1_sum_norm_eps(fk), fv, torch.sigmoid(fb), V0)
+    ref = xc + cpu.out_linear(o2.transpose(1, 2).reshape(B, L, H * d).transpose(0, 1))
+    (ref * go).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), ref.detach().numpy()) < TOL
+    assert rel_err(Wn.cpu().numpy(), WL.detach().numpy()) < TOL
+    assert rel_err(Vn.cpu().numpy(), VL.detach().numpy()) < TOL
+    assert rel_err(xg.grad.cpu().numpy(), xc.grad.numpy()) < TOL
+    assert rel_err(gpu.slow_net.weight.grad.cpu().numpy(), cpu.slow_net.weight.grad.numpy()) < TOL
+    assert "cached_fast_weights" in gpu.state_dict()
+
+
+def test_pseudo_sr_layer():
+    print("case PseudoSRlayer", flush=True)
+    from layer import PseudoSRlayer
+    torch.manual_seed(6)
+    L, B, H, d = 5, 3, 4, 8
+    gpu, cpu = _pair(PseudoSRlayer(H, d, H * d, 0.0))
+    x = torch.randn(L, B, H * d, dtype=torch.float64)
+    out, state = gpu(x.to(_dev(), torch.float32), None)
+    ref = x + cpu.out_linear(torch.einsum("lbhe,hem->lbhm", x.view(L, B, H, d), cpu.W_y).reshape(L, B, H * d))
+    assert state is None
+    assert rel_err(out.detach().cpu().numpy(), ref.detach().numpy()) < TOL
+    assert set(gpu.state_dict()) == {"W_y", "layer_norm.weight", "layer_norm.bias", "out_linear.weight"}
+
+
 def test_state_dict_names_match_the_reference_layers():
     from layer import FastFFlayer, SRWMlayer
     sd = SRWMlayer(2, 8, 16, 0.0).state_dict()
