@@ -302,6 +302,35 @@ def test_resets_at_tile_boundaries(E, L):
         assert rel_err(fw_.cpu().numpy(), (rs + w).numpy()) < TOL
 
 
+@pytest.mark.parametrize("shape,Y", [((8, 16, 200, 64), None), ((4, 8, 70, 64), 193), ((8, 8, 100, 32), None)])
+def test_repeated_runs_are_bit_identical(shape, Y):
+    """No atomics and a fixed summation order: the same inputs give the same bits every time.  Also a
+    guard for the hand-over buffers between waves (a missing barrier shows up as run-to-run noise)."""
+    print(f"case repeated runs shape={shape} Y={Y}", flush=True)
+    import srwm_hip
+    N, H, L, E = shape
+    x, W, go = srwm_inputs(N, H, L, E, seed=12, w_std=0.1, per_batch_state=True, y_width=Y)
+    Yw = E if Y is None else Y
+    dev = _dev()
+    xd, god = x.to(dev, torch.float32), go.to(dev, torch.float32)
+    first = None
+    for it in range(6):
+        Wd = [w.to(dev, torch.float32).contiguous() for w in W]
+        nan = lambda *s: torch.full(s, float("nan"), device=dev)
+        f = [nan(N, H, L, E), nan(N, H, L, E), nan(N, H, L, 4), nan(N, H, L, Yw), nan(N, H, L, E), nan(N, H, L, E),
+             nan(N, H, L, 4), nan(N, H, L, Yw)]
+        srwm_hip.self_ref_forward(xd, *Wd, *f)
+        gx = nan(N, H, L, E)
+        gW = [torch.full_like(w, float("nan")) for w in Wd]
+        srwm_hip.self_ref_backward(xd, *f[:-1], god, *Wd, gx, *gW, flags=srwm_hip.GRAD_STATE_ZERO)
+        cur = [*f, *Wd, gx, *gW]
+        if first is None:
+            first = cur
+        else:
+            for i, (a, b) in enumerate(zip(first, cur)):
+                assert torch.equal(a, b), (it, i)
+
+
 # ---------------------------------------------------------------- wide output block (self_ref_v1)
 
 @pytest.mark.parametrize("shape,Y,w_std,xsm,per_batch", [
