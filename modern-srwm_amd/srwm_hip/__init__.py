@@ -112,13 +112,15 @@ def _check(code, what):
 
 
 def _require(t, name, shape=None, dtype=torch.float32):
+    # runs some twenty times per operator call, on a path that is host-bound for single-step calls:
+    # only attribute reads and identity / tuple comparisons on the success path
     if not isinstance(t, torch.Tensor):
         raise TypeError(f"{name} must be a torch.Tensor")
-    if t.device.type != "cuda":
+    if not t.is_cuda:
         raise RuntimeError(f"{name} must live on the GPU (got {t.device}); there is no CPU path")
-    if t.dtype != dtype:
+    if t.dtype is not dtype:
         raise TypeError(f"{name} must be {dtype} (got {t.dtype})")
-    if shape is not None and tuple(t.shape) != tuple(shape):
+    if shape is not None and t.shape != shape:
         raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
 
 
@@ -161,7 +163,14 @@ def _has_bf16_kernel(E, M):
     return E == M and E in (8, 16, 32, 64, 128)
 
 
+# torch's own fast path to the current stream's handle (what its compiled-code launchers use); the
+# public Stream object costs several microseconds to build per call
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream(device):
+    if _raw_stream is not None and device.index is not None:
+        return ctypes.c_void_p(_raw_stream(device.index))
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
@@ -357,7 +366,7 @@ def _shared(slow, H, E, Y):
         if t.dim() == 4 and t.shape[0] == 1:
             t = t[0]
         _require(t, nm, shp)
-        out.append(t.detach().contiguous())
+        out.append(t if t.is_contiguous() else t.detach().contiguous())   # only its address is used
     return out
 
 
