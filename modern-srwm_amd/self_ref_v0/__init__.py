@@ -13,6 +13,8 @@ weights, everything saved for the backward and all arithmetic stay float32.
 The weight tensors are OVERWRITTEN with the state after the last step (the layers read
 them back as the carried state); the backward starts from that mutated tensor.
 """
+import threading
+
 import torch
 
 import srwm_hip
@@ -155,6 +157,9 @@ class SelfRefv0Steps(torch.autograd.Function):
 self_ref_v0_steps = SelfRefv0Steps.apply
 
 
+_scratch = threading.local()   # SelfRefLayerFn: write-only buffers of calls that need no gradient
+
+
 class SelfRefLayerFn(torch.autograd.Function):
     """The SRWM operator as the layers call it, with `state + W.repeat(bsz, 1, 1, 1)`, the softmax
     of the input, the final `- W.repeat(...)` and the batch sum of the weight gradients done inside
@@ -190,12 +195,22 @@ class SelfRefLayerFn(torch.autograd.Function):
         wide = lambda: torch.empty((N, H, L, Y), device=dev, dtype=f32)
         small = lambda: torch.empty((N, H, L, 4), device=dev, dtype=f32)
         out = torch.empty((N, H, L, Y), device=dev, dtype=x.dtype)
-        saved = [big(), big(), small(), wide(), big(), big(), small()]
+        needs_grad = any(ctx.needs_input_grad)
+        if needs_grad:
+            saved = [big(), big(), small(), wide(), big(), big(), small()]
+        else:
+            # inference (an RL actor's single-step calls are bound by host time): the per-step vectors
+            # are written and never read, so one set of buffers per thread and shape is reused
+            key = (dev, N, H, L, E, Y)
+            if getattr(_scratch, "key", None) != key:
+                _scratch.key, _scratch.bufs = key, [big(), big(), small(), wide(), big(), big(), small()]
+            saved = _scratch.bufs
         flags = srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_FRESH_STATE if fresh else 0) | \
             (srwm_hip.FLAG_SOFTMAX_INPUT if softmax_input else 0)
         slow = (sW_y, sW_q, sW_k, sw_b)
         srwm_hip.self_ref_layer_forward(x.detach(), None, slow, *state, *saved, out, flags=flags)
-        ctx.save_for_backward(x, *saved, *slow, *state)
+        if needs_grad:
+            ctx.save_for_backward(x, *saved, *slow, *state)
         ctx.softmax_input = softmax_input
         ctx.fresh = fresh
         return (out, *state)
