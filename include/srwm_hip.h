@@ -17,12 +17,14 @@
  *     rejects (nothing was launched); positive = the hipError_t of a failed
  *     launch.  The library never throws and never calls exit/abort.
  *   - Re-entrant: no mutable global state; safe from several host threads on
- *     different streams/devices.
+ *     different streams/devices.  The one exception is srwm_layer_backward_noalloc_f32,
+ *     whose calls on one device share a static device array.
  *   - `flags`: bitwise OR of SRWM_FLAG_*.
  */
 #ifndef SRWM_HIP_H
 #define SRWM_HIP_H
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -37,6 +39,7 @@ extern "C" {
 #define SRWM_ESTRIDE (-3)  /* stride makes an access misaligned or overflows 32-bit indexing */
 #define SRWM_ENOKERNEL (-4) /* no kernel for this combination (bf16 I/O needs E == M in {8,16,32,64,128}
                                and rows aligned to 8 bytes) */
+#define SRWM_ESCRATCH (-5) /* srwm_layer_backward_noalloc_f32: the per-row gradients exceed the static array */
 
 /* backward: what the grad-state buffers hold on entry / exit */
 #define SRWM_GRAD_STATE_ZERO 0u   /* entry contents ignored (dL/dW_L = 0); exit: dL/dW_0 */
@@ -209,6 +212,42 @@ SRWM_API int srwm_layer_backward_f32(const float *x, const int64_t x_strides[3],
                             int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
 /*
+ * srwm_layer_backward_f32 for callers that cannot allocate device memory and have no use for the
+ * per-row state gradients.  No counterpart in the reference.  It exists for code under HIP graph
+ * capture, serving loops and harnesses that must not call hipMalloc: the layers only want the batch
+ * sums gsW_y .. gsw_b (SRlayer / NoCarryOverSRlayer start every call from the shared weights or from
+ * a detached shift), yet srwm_layer_backward_f32 makes them bring [N,H,E,.] buffers for the per-row
+ * gradients that the batch sum is formed from.  Here those live in a static device array inside the
+ * library (srwm_hip_scratch_bytes() bytes, 32 MiB, held by every GPU the library runs on until the
+ * process ends); the function calls no hipMalloc / hipFree and no allocating routine.
+ *   arguments   as srwm_layer_backward_f32 without gW_y .. gw_b; gsW_y .. gsw_b are required
+ *   flags       SRWM_FLAG_STATE_SHIFT, SRWM_FLAG_SOFTMAX_INPUT, SRWM_FLAG_GENERIC; the state gradient at
+ *               the last step is zero (SRWM_GRAD_STATE_ZERO; the other two modes give SRWM_EINVAL)
+ *   limit       N*H*E*(Y+2E+4) floats (each of the four parts rounded up to 64 floats) must fit the
+ *               array: SRWM_ESCRATCH otherwise, nothing launched.  The headline shape N=32, H=16,
+ *               E=Y=64 takes 24.5 MiB.
+ * Results are bit-identical to srwm_layer_backward_f32 (same kernels, same summation order).
+ * Every call on a device uses the same array: calls that overlap on one GPU (two streams, two
+ * threads) race; calls on one stream are ordered and safe.  Nothing in the array has to start at
+ * zero -- the kernels overwrite what the batch sum reads -- so no call clears it.  The array's address
+ * is looked up on the first call on each device (hipGetSymbolAddress); make that call outside stream
+ * capture.
+ */
+SRWM_API int srwm_layer_backward_noalloc_f32(const float *x, const int64_t x_strides[3],
+                            const float *q, const float *k, const float *beta,
+                            const float *y_diff, const float *q_diff, const float *k_diff,
+                            const float *beta_diff,
+                            const float *grad_out, const int64_t grad_out_strides[3],
+                            const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
+                            const float *W_y, const float *W_q, const float *W_k, const float *w_b,
+                            float *grad_x,
+                            float *gsW_y, float *gsW_q, float *gsW_k, float *gsw_b,
+                            int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+
+/* Size in bytes of the static device array behind srwm_layer_backward_noalloc_f32. */
+SRWM_API size_t srwm_hip_scratch_bytes(void);
+
+/*
  * The layer operator with bf16 input and output, fp32 state.  No counterpart in the reference (its
  * kernels are float-only): same contract as srwm_layer_forward_f32 / srwm_layer_backward_f32 with
  *   x, out, grad_out   bf16 (raw 16-bit patterns; strides in bf16 elements)
@@ -364,7 +403,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any signature change); currently 4. */
+/* ABI version of this header (bumped on any signature change); currently 5. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

@@ -1,8 +1,19 @@
 // extern "C" boundary of libsrwm_hip.so (declared in include/srwm_hip.h): argument
-// checks, kernel selection, launch.  No allocation, no synchronisation, no global state.
+// checks, kernel selection, launch.  No allocation, no synchronisation; the only state kept
+// between calls is the address of the static device array behind srwm_layer_backward_noalloc_f32.
 #include "../../include/srwm_hip.h"
 
+#include <atomic>
+#include <mutex>
+
 #include "common.h"
+
+// Device memory of srwm_layer_backward_noalloc_f32: the per-batch-row state gradients that the
+// backward kernel writes and the batch-sum kernel reads.  Part of the code object, so every GPU
+// the library runs on holds its own copy from module load until the process ends.  Host code must
+// not use this name as an address: it asks hipGetSymbolAddress once per device (scratch_base).
+#define SRWM_SCRATCH_FLOATS (8u << 20)   /* 32 MiB */
+static __device__ __align__(256) float scratch[SRWM_SCRATCH_FLOATS];
 
 namespace {
 
@@ -37,6 +48,34 @@ int max_E_for(size_t (*bytes)(int), size_t limit) {
     return e;
 }
 
+// address of `scratch` on the calling thread's current device, resolved on the first call there
+constexpr int kMaxDevices = 64;
+std::atomic<float *> g_scratch_base[kMaxDevices];
+std::mutex g_scratch_mutex;
+
+int scratch_base(float **base) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return SRWM_EINVAL;
+    float *p = g_scratch_base[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        p = g_scratch_base[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            e = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) return (int)e;
+            if (!p) return (int)hipErrorInvalidSymbol;
+            g_scratch_base[dev].store(p, std::memory_order_release);
+        }
+    }
+    *base = p;
+    return SRWM_OK;
+}
+
+// floats of one per-row gradient tensor in `scratch`, rounded up so that the next one starts 256-byte aligned
+int64_t scratch_span(int N, int H, int E, int width) { return ((int64_t)N * H * E * width + 63) / 64 * 64; }
+
 size_t srwm_fwd_sq(int e) { return srwm_fwd_generic_lds_bytes(e, e); }
 size_t srwm_bwd_sq(int e) { return srwm_bwd_generic_lds_bytes(e, e); }
 size_t delta_fwd_sq(int e) { return delta_fwd_generic_lds_bytes(e, e); }
@@ -46,7 +85,9 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 4; }
+int srwm_hip_abi_version(void) { return 5; }
+
+size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
 const char *srwm_hip_strerror(int code) {
     switch (code) {
@@ -55,6 +96,7 @@ const char *srwm_hip_strerror(int code) {
         case SRWM_ESIZE: return "head size not supported: the state does not fit in the CU's LDS";
         case SRWM_ESTRIDE: return "unsupported stride";
         case SRWM_ENOKERNEL: return "no kernel for this dtype / size / alignment combination";
+        case SRWM_ESCRATCH: return "problem too large for the library's static scratch array (see srwm_hip_scratch_bytes)";
         default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown srwm_hip error";
     }
 }
@@ -308,6 +350,31 @@ int srwm_layer_backward_f32(const float *x, const int64_t xs[3], const float *q,
                             float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, float *gsWy,
                             float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
                             unsigned flags, void *stream) {
+    return layer_backward(false, x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, sWy, sWq, sWk, swb, Wy,
+                          Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags,
+                          stream);
+}
+
+int srwm_layer_backward_noalloc_f32(const float *x, const int64_t xs[3], const float *q, const float *k,
+                                    const float *beta, const float *ydiff, const float *qdiff,
+                                    const float *kdiff, const float *bdiff, const float *grad_out,
+                                    const int64_t gs[3], const float *sWy, const float *sWq, const float *sWk,
+                                    const float *swb, const float *Wy, const float *Wq, const float *Wk,
+                                    const float *wb, float *grad_x, float *gsWy, float *gsWq, float *gsWk,
+                                    float *gswb, int N, int H, int L, int E, int Y, unsigned flags, void *stream) {
+    if (!gsWy || !gsWq || !gsWk || !gswb) return SRWM_EINVAL;
+    // the per-row gradients start from nothing: there is no buffer an incoming state gradient could arrive in
+    if (flags & SRWM_GRAD_STATE_MASK) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y)) return SRWM_EINVAL;
+    const int64_t span[4] = {scratch_span(N, H, E, Y), scratch_span(N, H, E, E), scratch_span(N, H, E, E),
+                             scratch_span(N, H, E, 4)};
+    if (span[0] + span[1] + span[2] + span[3] > (int64_t)SRWM_SCRATCH_FLOATS) return SRWM_ESCRATCH;
+    float *base = nullptr;
+    const int r = scratch_base(&base);
+    if (r != SRWM_OK) return r;
+    float *gWy = base, *gWq = gWy + span[0], *gWk = gWq + span[1], *gwb = gWk + span[2];
+    // SRWM_GRAD_STATE_ZERO: the backward kernel overwrites every per-row gradient it owns and the batch
+    // sum reads exactly those, so nothing in the array has to be cleared between calls
     return layer_backward(false, x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, sWy, sWq, sWk, swb, Wy,
                           Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags,
                           stream);

@@ -34,7 +34,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _lib = None
 
@@ -51,6 +51,7 @@ _SIGNATURES = {
     "srwm_backward_wide_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_layer_forward_f32": [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_layer_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_backward_noalloc_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 13 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_layer_forward_bf16": [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_layer_backward_bf16": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
@@ -93,6 +94,8 @@ def lib():
         L.srwm_hip_strerror.argtypes = [_I]
         L.srwm_hip_limits.argtypes = [ctypes.POINTER(_I)] * 3
         L.srwm_hip_limits.restype = _I
+        L.srwm_hip_scratch_bytes.restype = ctypes.c_size_t
+        L.srwm_hip_scratch_bytes.argtypes = []
         _lib = L
     return _lib
 
@@ -466,6 +469,49 @@ def self_ref_layer_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, gr
             *[_ptr(t) for t in st], _ptr(gx[0]), *[_ptr(g) for g in grad_W], *gsl,
             N, H, L, E, Y, flags, _stream(x.device))
     _check(code, name)
+
+
+def scratch_bytes():
+    """Size of the static device array behind self_ref_layer_backward_noalloc."""
+    return int(lib().srwm_hip_scratch_bytes())
+
+
+def self_ref_layer_backward_noalloc(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out, slow,
+                                    W_y, W_q, W_k, w_b, grad_x, grad_slow, flags=0):
+    """self_ref_layer_backward without the per-row gradient tensors: they live in a static device
+    array inside the library, so the call allocates nothing (every tensor must already be dense where
+    the kernels need it dense; nothing is copied here).  grad_slow: four (H, E, .) tensors, required.
+    Raises when N*H*E*(Y+2E+4) floats exceed scratch_bytes().  Calls that overlap on one GPU share the
+    array and race; calls on one stream are ordered."""
+    _require(x, "x")
+    N, H, L, E = x.shape
+    _require(W_y, "W_y")
+    Y = W_y.shape[-1]
+    for t, nm in ((q, "q"), (k, "k"), (q_diff, "q_diff"), (k_diff, "k_diff"), (grad_x, "grad_x")):
+        _require(t, nm, (N, H, L, E))
+    _require(y_diff, "y_diff", (N, H, L, Y))
+    _require(grad_out, "grad_out", (N, H, L, Y))
+    _require(beta, "beta", (N, H, L, 4))
+    _require(beta_diff, "beta_diff", (N, H, L, 4))
+    for t, shp in zip((W_y, W_q, W_k, w_b), ((N, H, E, Y), (N, H, E, E), (N, H, E, E), (N, H, E, 4))):
+        _require(t, "state", shp)
+    sl = _shared(slow, H, E, Y)
+    for g, shp in zip(grad_slow, ((H, E, Y), (H, E, E), (H, E, E), (H, E, 4))):
+        _require(g, "grad_slow", shp)
+    dense = [q, k, beta, y_diff, q_diff, k_diff, beta_diff, W_y, W_q, W_k, w_b, grad_x, *grad_slow]
+    if not all(t.is_contiguous() for t in dense):
+        raise ValueError("self_ref_layer_backward_noalloc copies nothing: saved vectors, state and gradients "
+                         "must be contiguous")
+    (xs, xstr), (gos, gstr) = _strided(x), _strided(grad_out)
+    if xs is not x or gos is not grad_out:
+        raise ValueError("self_ref_layer_backward_noalloc copies nothing: x and grad_out need a contiguous, "
+                         "16-byte aligned last axis")
+    with torch.cuda.device(x.device):
+        code = lib().srwm_layer_backward_noalloc_f32(
+            _ptr(x), xstr, *[_ptr(t) for t in (q, k, beta, y_diff, q_diff, k_diff, beta_diff)], _ptr(grad_out), gstr,
+            *[_ptr(t) for t in sl], *[_ptr(t) for t in (W_y, W_q, W_k, w_b)], _ptr(grad_x),
+            *[_ptr(g) for g in grad_slow], N, H, L, E, Y, flags, _stream(x.device))
+    _check(code, "srwm_layer_backward_noalloc_f32")
 
 
 # names of the extension functions of the reference's wide-output variant

@@ -49,7 +49,8 @@ def test_ctypes_signatures_match_the_header():
     same count, pointers where the header has pointers or arrays, ints where it has ints."""
     import srwm_hip
     protos = _prototypes()
-    aux = {"srwm_hip_abi_version", "srwm_hip_strerror", "srwm_hip_limits", "srwm_hip_lds_probe"}
+    aux = {"srwm_hip_abi_version", "srwm_hip_strerror", "srwm_hip_limits", "srwm_hip_lds_probe",
+           "srwm_hip_scratch_bytes"}
     assert set(protos) - aux == set(srwm_hip._SIGNATURES), set(protos) - aux ^ set(srwm_hip._SIGNATURES)
     for name, args in srwm_hip._SIGNATURES.items():
         params = protos[name]
@@ -147,3 +148,11 @@ def test_argument_validation_needs_no_gpu():
                                                          *[fake() for _ in range(12)], N, H, Ls, E, E, flags, P(None))
     assert layer_f(P(None), 64) == -1                          # the shift form needs the shared weights
     assert layer_f(P(None), 128) == -1                         # so does a fresh start
+    noalloc = lambda n, flags, gs: L.srwm_layer_backward_noalloc_f32(
+        fake(), ok_strides, *[fake() for _ in range(7)], fake(), ok_strides, *[fake() for _ in range(9)],
+        gs, gs, gs, gs, n, H, Ls, E, E, flags, P(None))
+    assert noalloc(N, 0, P(None)) == -1                        # the batch sums are what it is for
+    assert noalloc(N, 1, fake()) == -1                         # no buffer for an incoming state gradient
+    assert noalloc(1 << 16, 0, fake()) == -5                   # SRWM_ESCRATCH: 2^16 x 8 rows of 16 x 52 floats > 32 MiB
+    assert L.srwm_hip_scratch_bytes() == 32 << 20
+    assert b"scratch" in L.srwm_hip_strerror(-5)
