@@ -157,7 +157,27 @@ class SelfRefv0Steps(torch.autograd.Function):
 self_ref_v0_steps = SelfRefv0Steps.apply
 
 
-_scratch = threading.local()   # SelfRefLayerFn: write-only buffers of calls that need no gradient
+# SelfRefLayerFn, calls that need no gradient: their per-step vectors are written and never read,
+# so a thread reuses one set of buffers per (device, stream, shape).  Keyed by stream because the
+# caching allocator only orders reuse of a block on the stream it was allocated on.
+_scratch = threading.local()
+_SCRATCH_SETS = 4   # buffer sets a thread keeps; the oldest is dropped first
+
+
+def _write_only_buffers(dev, shapes):
+    if torch.cuda.is_current_stream_capturing():
+        # a captured graph must own its buffers: these come from the graph's private pool
+        return [torch.empty(s, device=dev, dtype=torch.float32) for s in shapes]
+    sets = getattr(_scratch, "sets", None)
+    if sets is None:
+        sets = _scratch.sets = {}
+    key = (dev, srwm_hip._stream(dev).value, shapes)
+    bufs = sets.get(key)
+    if bufs is None:
+        while len(sets) >= _SCRATCH_SETS:
+            sets.pop(next(iter(sets)))
+        bufs = sets[key] = [torch.empty(s, device=dev, dtype=torch.float32) for s in shapes]
+    return bufs
 
 
 class SelfRefLayerFn(torch.autograd.Function):
@@ -178,7 +198,11 @@ class SelfRefLayerFn(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, x, sW_y, sW_q, sW_k, sw_b, shift_y, shift_q, shift_k, shift_b, softmax_input):
+    def forward(ctx, x, sW_y, sW_q, sW_k, sw_b, shift_y, shift_q, shift_k, shift_b, softmax_input,
+                track=True):
+        # track: whether a backward can follow.  Decided by the caller (self_ref_layer): in here grad
+        # mode is always off, and ctx.needs_input_grad is True for a trainable parameter even under
+        # torch.no_grad().
         N, H, L, E = x.shape
         Y = sW_y.shape[-1]
         dev = x.device
@@ -191,20 +215,14 @@ class SelfRefLayerFn(torch.autograd.Function):
             state = [torch.empty((N, H, E, w), device=dev, dtype=f32) for w in widths]
         else:
             state = [s.detach().clone(memory_format=torch.contiguous_format) for s in shifts]
-        big = lambda: torch.empty((N, H, L, E), device=dev, dtype=f32)
-        wide = lambda: torch.empty((N, H, L, Y), device=dev, dtype=f32)
-        small = lambda: torch.empty((N, H, L, 4), device=dev, dtype=f32)
         out = torch.empty((N, H, L, Y), device=dev, dtype=x.dtype)
-        needs_grad = any(ctx.needs_input_grad)
+        needs_grad = bool(track)
+        shapes = tuple((N, H, L, w) for w in (E, E, 4, Y, E, E, 4))   # q, k, beta, y_diff, q_diff, k_diff, beta_diff
         if needs_grad:
-            saved = [big(), big(), small(), wide(), big(), big(), small()]
+            saved = [torch.empty(s_, device=dev, dtype=f32) for s_ in shapes]
         else:
-            # inference (an RL actor's single-step calls are bound by host time): the per-step vectors
-            # are written and never read, so one set of buffers per thread and shape is reused
-            key = (dev, N, H, L, E, Y)
-            if getattr(_scratch, "key", None) != key:
-                _scratch.key, _scratch.bufs = key, [big(), big(), small(), wide(), big(), big(), small()]
-            saved = _scratch.bufs
+            # inference (an RL actor's single-step calls are bound by host time)
+            saved = _write_only_buffers(dev, shapes)
         flags = srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_FRESH_STATE if fresh else 0) | \
             (srwm_hip.FLAG_SOFTMAX_INPUT if softmax_input else 0)
         slow = (sW_y, sW_q, sW_k, sw_b)
@@ -244,7 +262,15 @@ class SelfRefLayerFn(torch.autograd.Function):
             gs = [(g - m if minus is not None else g).reshape(s.shape) for g, m, s in
                   zip(grad_slow, minus or [None] * 4, slow)]
         gshift = [None] * 4 if ctx.fresh else grad_W
-        return (grad_x.to(x.dtype), *gs, *gshift, None)
+        return (grad_x.to(x.dtype), *gs, *gshift, None, None)
 
 
-self_ref_layer = SelfRefLayerFn.apply
+def self_ref_layer(x, sW_y, sW_q, sW_k, sw_b, shift_y, shift_q, shift_k, shift_b, softmax_input):
+    """SelfRefLayerFn.apply; works out here, where grad mode is still the caller's, whether a
+    backward can follow (no_grad, or nothing that requires grad: the call then saves nothing and
+    reuses its write-only buffers)."""
+    track = torch.is_grad_enabled() and any(
+        t is not None and t.requires_grad
+        for t in (x, sW_y, sW_q, sW_k, sw_b, shift_y, shift_q, shift_k, shift_b))
+    return SelfRefLayerFn.apply(x, sW_y, sW_q, sW_k, sw_b, shift_y, shift_q, shift_k, shift_b, softmax_input,
+                                track)

@@ -145,7 +145,10 @@ def test_hip_stepwise_operators_match_their_fixtures():
     assert rel_err(x.grad.cpu().numpy(), g["grad_x"]) < TOL
     assert rel_err(slow[0].grad.cpu().numpy(), g["grad_slow0"]) < TOL
     for i, (f_, w) in enumerate(zip(fast, slow)):
-        assert rel_err((f_ - w.detach().repeat(N, 1, 1, 1)).cpu().numpy(), g[f"final_shift{i}"]) < 5 * TOL
+        # the operator returns the weights; the shift is their fp32 difference from the shared weights,
+        # so its error is that of the weights and is measured on their scale
+        shift = (f_ - w.detach().repeat(N, 1, 1, 1)).cpu().numpy()
+        assert np.abs(shift - g[f"final_shift{i}"]).max() < TOL * float(f_.abs().max()), i
     g = np.load(STEPS_DELTA)
     leaves = [t(g[n]).requires_grad_(True) for n in ("Q", "K", "V", "beta")]
     W = t(g["W0"]).clone()

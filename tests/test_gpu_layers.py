@@ -97,8 +97,57 @@ def test_srwm_layer_stateful_with_loss_on_state(srwm_layer_path):
     sh2 = [f - w for f, w in zip(f2, slow)]
     (r2.sum() + sum((s * s).sum() for s in sh2)).backward()
     assert rel_err(out2.detach().cpu().numpy(), r2.detach().numpy()) < TOL
-    for n in ("W_y", "W_q", "W_k", "w_b"):
-        assert rel_err(getattr(gpu, n).grad.cpu().numpy(), getattr(cpu, n).grad.numpy()) < 2e-4, n
+    # The shared weights receive sum_n (dL/dW_0[n] - g_shift[n]) from each segment, where g_shift is the
+    # gradient arriving at the returned shift (here 2 * shift, far larger than the result): an fp32
+    # difference of nearly equal numbers.  Its error is measured against the size of the terms that
+    # cancel, sum_n |g_shift[n]|, like every other cancelling sum in these tests.
+    for n, s2 in zip(("W_y", "W_q", "W_k", "w_b"), sh2):
+        got, want = getattr(gpu, n).grad.cpu().double(), getattr(cpu, n).grad
+        scale = max(want.abs().max().item(), (2 * s2.detach()).abs().sum(0).max().item())
+        assert (got - want).abs().max().item() < TOL * scale, n
+
+
+def test_gradient_free_layer_calls_take_the_buffer_reusing_path():
+    """An RL actor calls SRlayer under no_grad with trainable parameters; evaluation code may also
+    freeze the parameters instead.  Both must skip what only a backward needs (fresh per-step buffers,
+    saved tensors) and return bit-identical outputs and shifts to a tracked call, call after call."""
+    print("case SRlayer without gradient", flush=True)
+    import self_ref_v0
+    from layer import SRlayer
+    torch.manual_seed(5)
+    B, H, d = 4, 8, 32
+    gpu = SRlayer(H, d, H * d, 0.0).to(_dev())
+    zero = tuple(torch.zeros(B, H, d, w, device=_dev()) for w in (d, d, d, 4))
+    hs = [torch.randn(1, B, H * d, device=_dev()) for _ in range(3)]
+
+    def run(track):
+        state, outs = zero, []
+        for h in hs:
+            out, state = gpu(h.clone().requires_grad_(track), state)
+            outs.append(out)
+        return outs, state
+
+    ref_outs, ref_state = run(True)
+    assert ref_outs[0].grad_fn is not None
+    self_ref_v0._scratch.sets = {}
+    with torch.no_grad():
+        outs, state = run(False)
+    assert len(self_ref_v0._scratch.sets) == 1                 # one buffer set, reused by the three calls
+    assert all(o.grad_fn is None for o in outs)
+    for a, b in zip(outs + list(state), ref_outs + list(ref_state)):
+        assert torch.equal(a, b.detach())
+    for prm in gpu.parameters():
+        prm.requires_grad_(False)
+    outs, state = run(False)                                   # grad mode on, nothing requires grad
+    assert len(self_ref_v0._scratch.sets) == 1
+    for a, b in zip(outs + list(state), ref_outs + list(ref_state)):
+        assert torch.equal(a, b.detach())
+    for prm in gpu.parameters():
+        prm.requires_grad_(True)
+    outs, _ = run(False)                                       # trainable parameters again: tracked
+    assert outs[0].grad_fn is not None
+    outs[-1].sum().backward()
+    assert gpu.W_q.grad is not None and torch.isfinite(gpu.W_q.grad).all()
 
 
 def test_rl_sr_layers_carry_and_restart(srwm_layer_path):
