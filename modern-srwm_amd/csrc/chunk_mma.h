@@ -207,9 +207,13 @@ struct PrecBf16 {
     }
     // SA / SB: the left / right operand carries a lo part that matters.
     // A single group is issued as the 32-index instruction with its second half zero, so that every
-    // matrix instruction of these kernels is the same opcode: a 16-index MFMA that accumulates
-    // onto the result of a 32-index one (or the reverse) a few instructions later was observed
-    // to read the accumulator before it was written.
+    // matrix instruction of these kernels is the same opcode.  Measured on gfx950 with a stand-alone
+    // kernel: v_mfma_f32_16x16x16_bf16 whose SrcC is the vDst of a v_mfma_f32_16x16x32_bf16 (or the
+    // reverse) reads the accumulator before it is written unless at least 4 wait states (s_nop 3)
+    // separate the two; chains of one opcode are exact back to back.  hipcc of ROCm 7.2 emits no
+    // wait state for that pair (it relies on the same-register forwarding that only holds between
+    // equal opcodes), so whether a mixed chain is right depends on what the scheduler happens to put
+    // in between.  Do not mix the two opcodes on one accumulator.
     template <bool SA, bool SB>
     __device__ static __forceinline__ f32x4 mma(const A &a, const B &b, f32x4 acc) {
         const s16x4 z = {0, 0, 0, 0};

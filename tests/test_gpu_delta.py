@@ -294,6 +294,47 @@ def test_chunkwise_backward_matches_oracle(shape, qk, w0, io, state_grad):
     assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
 
 
+@pytest.mark.parametrize("D,L", [(64, 70), (64, 200), (128, 70), (128, 200), (128, 1024)])
+def test_chunkwise_bf16_runs_are_bit_identical_and_match_the_oracle(D, L):
+    """The matrix-core kernels with bf16 inputs (forward, column sweep, row sweep) at ragged lengths:
+    six runs of forward + backward must agree bit for bit (every word has one writer or meets through
+    a two-addend atomic sum, and no result may depend on instruction timing), and the first run must
+    match the fp64 oracle on the rounded inputs."""
+    print(f"case chunkwise bf16 determinism D={D} L={L}", flush=True)
+    import srwm_hip
+    dev = _dev()
+    N, H = 2, 3
+    q, k, v, beta, W0, go = delta_inputs(N, H, L, D, D, seed=23, qk="l2", w0_std=0.2)
+    qi, ki, vi, bi, goi = (t.to(torch.bfloat16) for t in (q, k, v, beta, go))
+    base = [t.to(torch.float64).numpy() for t in (qi, ki, vi, bi)] + [W0.numpy()]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, goi.to(torch.float64).numpy(), want_grad_W=True)
+    qd, kd, vd, bd, god = (t.to(dev) for t in (qi, ki, vi, bi, goi))
+    nan = lambda *s_, dt=torch.float32: torch.full(s_, float("nan"), device=dev, dtype=dt)
+    runs = []
+    for rep in range(6):
+        W = W0.to(dev, torch.float32).contiguous()
+        vold, vins, out = nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, D, dt=torch.bfloat16)
+        srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out, flags=srwm_hip.FLAG_CHUNKWISE)
+        WL = W.clone()
+        gq, gk, gv, gb, gW = nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, 1), nan(N, H, D, D)
+        srwm_hip.fast_weight_backward(qd, kd, vd, bd, vold, vins, god, W, gq, gk, gv, gb, grad_kv=gW,
+                                      flags=srwm_hip.FLAG_CHUNKWISE)
+        if rep % 2:   # other work between the runs shifts the timing of the next one
+            torch.mm(torch.randn(512, 512, device=dev), torch.randn(512, 512, device=dev))
+        torch.cuda.synchronize()
+        runs.append(dict(out=out, v_old=vold, v_insert=vins, W=WL, W0=W, grad_Q=gq, grad_K=gk, grad_V=gv,
+                         grad_beta=gb, grad_W=gW))
+    for rep, r in enumerate(runs[1:], 1):
+        for n, t in r.items():
+            assert torch.equal(t, runs[0][n]), (rep, n)
+    r = runs[0]
+    errs = {n: rel_err(r[n].float().cpu().numpy(), of[n]) for n in ("out", "v_old", "v_insert", "W")}
+    errs.update({n: rel_err(r[n].cpu().numpy(), ob[n]) for n in ("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W")})
+    bad = {n: e for n, e in errs.items() if not (e < BF16_TOL)}
+    assert not bad, f"over tolerance {BF16_TOL}: {bad}  (all: {errs})"
+
+
 def test_full_config5_properties():
     """benchmark configuration 5 at full size (N=8, H=16, L=4096, E=M=128, bf16 I/O, fp32 memory):
     the step-by-step and the chunkwise forward agree with each other, the backward reverts the
