@@ -2,12 +2,18 @@
 fp64 oracle, through the same host entry points as the fixed cases of the other GPU test files.
 
 Bar: 1e-5 relative to the largest element of each tensor (fp32 arithmetic on both sides of the
-comparison would meet it; the oracle is fp64).  One family of outputs is measured differently: the
-`*_diff` vectors the SRWM forward emits are W^T (q - k), sums with heavy cancellation when q and k
-are close, so their fp32 error is bounded by 1e-5 times |W|^T |q - k| (the size of the terms that
-cancel), not by 1e-5 times the result.  The test computes that scale from the oracle's own vectors.
-The gradient of w_b is, per step, a product with sum(g_ins * diff): it inherits the conditioning of
-the diffs and is allowed 1e-5 times the same amplification factor (about 2 to 4 in these cases).
+comparison would meet it; the oracle is fp64).  Two families of results cannot meet it in every
+case in fp32, whoever computes them, and are held to what fp32 allows instead:
+
+* the `*_diff` vectors the SRWM forward emits are W^T (q - k), sums with heavy cancellation when q
+  and k are close (small weights): their error must stay within 1e-5 times |W|^T |q - k| (the size
+  of the terms that cancel, computed from the oracle's own vectors), AND wherever it exceeds the
+  plain bar it must stay within 3x the error the fp32 build of the C oracle (plain sequential loops)
+  makes on the same case -- measured, on every case, not assumed;
+* the gradient of w_b is, per step, a product with sum(g_ins * diff) over those saved diffs: against
+  the all-fp64 chain it gets the same fp32-oracle allowance; against the fp64 backward run on the
+  vectors the forward kernel itself emitted (so that only the backward kernel's arithmetic is
+  measured) it has to meet the plain bar like every other gradient.
 """
 import math
 import random
@@ -105,23 +111,46 @@ def test_srwm_random_case(c):
     srwm_hip.self_ref_backward(xd, *f[:-1], god, *Wd, gx, *gW, flags=flags | mode)
 
     W0 = [w.numpy() for w in W]
+    gsn = [s.numpy() for s in gs] if mode else None
     of = oracle.srwm_forward(x.numpy(), *W0)
-    ob = oracle.srwm_backward(x.numpy(), of, go.numpy(), grad_state=[s.numpy() for s in gs] if mode else None)
+    ob = oracle.srwm_backward(x.numpy(), of, go.numpy(), grad_state=gsn)
+    # the same case through the fp32 build of the C oracle: what plain fp32 loops achieve
+    f32 = lambda a: np.asarray(a, dtype=np.float32)
+    of32 = oracle.srwm_forward(f32(x.numpy()), *[f32(w) for w in W0], dtype=np.float32)
+    ob32 = oracle.srwm_backward(f32(x.numpy()), of32, f32(go.numpy()), dtype=np.float32,
+                                grad_state=[f32(a) for a in gsn] if mode else None)
+
+    def within_fp32_reach(got, want, want32):
+        """Meets the bar, or errs at most 3x as much as the fp32 oracle does."""
+        err = np.abs(got - want).max()
+        return err < TOL * np.abs(want).max() or err <= 3.0 * np.abs(want32.astype(np.float64) - want).max()
+
     scales = _cancellation_scales(W0, of, L)
     names = ("q", "k", "beta", "y_diff", "q_diff", "k_diff", "beta_diff", "out")
     for n, t in zip(names, f):
         got = t.cpu().numpy()
         if n.endswith("_diff"):
             assert np.abs(got - of[n]).max() <= TOL * max(scales[n], np.abs(of[n]).max()), n
+            assert within_fp32_reach(got, of[n], of32[n]), n
         else:
             assert rel_err(got, of[n]) < TOL, n
     for n, t in zip(("W_y", "W_q", "W_k", "w_b"), Wd):
         assert rel_err(t.cpu().numpy(), of[n]) < TOL, n
     assert rel_err(gx.cpu().numpy(), ob["grad_x"]) < TOL
-    kappa = max(1.0, max(scales[n] / max(float(np.abs(of[n]).max()), 1e-300) for n in scales))
-    for n, t, s in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), gW, gs):
-        want = ob[n] + (s.numpy() if mode == 2 else 0.0)
-        assert rel_err(t.cpu().numpy(), want) < TOL * (kappa if n == "grad_w_b" else 1.0), n
+    acc = lambda n: (gs[("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b").index(n)].numpy() if mode == 2 else 0.0)
+    for n, t in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), gW):
+        got = t.cpu().numpy()
+        if n == "grad_w_b":
+            assert within_fp32_reach(got, ob[n] + acc(n), ob32[n] + f32(acc(n))), n
+        else:
+            assert rel_err(got, ob[n] + acc(n)) < TOL, n
+    # the backward kernel alone: fp64 backward on the vectors (and final state) the forward kernel emitted
+    own = {n: t.cpu().numpy().astype(np.float64) for n, t in zip(names, f)}
+    own.update({n: t.cpu().numpy().astype(np.float64) for n, t in zip(("W_y", "W_q", "W_k", "w_b"), Wd)})
+    ob_own = oracle.srwm_backward(x.numpy(), own, go.numpy(), grad_state=gsn)
+    assert rel_err(gx.cpu().numpy(), ob_own["grad_x"]) < TOL
+    for n, t in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), gW):
+        assert rel_err(t.cpu().numpy(), ob_own[n] + acc(n)) < TOL, n
 
 
 @pytest.mark.parametrize("c", _cases("delta", 64, 4321), ids=_id)
