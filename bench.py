@@ -11,9 +11,14 @@ stream, so torch.cuda.Event brackets exactly the stream the kernels run on.
 Prints ONE JSON line (see the keys below).  `roofline` prices the dominant kernel (the
 backward) against the LDS-bandwidth yardstick of 6 passes over the 64x196 fp32 state per
 (sequence, step); `roofline_fwd_bwd` does the same for the forward+backward pair
-(9 passes), which is the figure the target (>= 50 %) is stated on; `roofline_hbm` gives the
-achieved HBM rate of the operator's I/O contract.  `cpu_baseline` is the per-timestep
-PyTorch recurrence (oracle/recurrence.py) timed on the host cores on a batch slice.
+(9 passes), which is the figure the target (>= 50 %) is stated on; `roofline_valu` /
+`roofline_valu_fwd_bwd` price the same passes as fp32 FLOPs against the vector peak (the state
+lives in registers, so that is the unit that limits the kernels); `roofline_hbm` gives the
+achieved HBM rate of the operator's I/O contract.  Kernel times are medians of the per-step HIP
+event times.  `other_workloads` (default run only) holds forward / backward times and roofline
+fractions of the other benchmark configurations, the chunkwise ones priced in FLOPs against the
+matrix-core peak.  `cpu_baseline` is the per-timestep PyTorch recurrence (oracle/recurrence.py)
+timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
 {srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk}.
@@ -32,16 +37,16 @@ for p in (ROOT, os.path.join(ROOT, "modern-srwm_amd")):
 LDS_PEAK_GBS = 256 * 128 * 2.4          # 256 CUs x 128 B/clk x 2.4 GHz = 78 643 GB/s
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the dominant (backward) kernel, measured with rocprofv3 --pmc FETCH_SIZE and
-# --pmc WRITE_SIZE (two runs; FETCH_SIZE scaled by the factor that makes a plain copy of known size
-# read its size).  Figures and commands: profiles/srwm_c4_kernels.txt, profiles/delta_kernels.txt,
-# profiles/delta_chunk_kernels.txt (backward kernels of the workload: fetch + write).
-MEASURED_TRAFFIC_BYTES = {
-    "srwm_c4": (490413 + 90624) * 1024,
-    "delta_c2": (102444 + 53504) * 1024,
-    "delta_c2_chunk": (82217 + 85992 + 16640 + 36864) * 1024,
-    "delta_c5": (1316522 + 1323008) * 1024,
-    "delta_c5_chunk": (1047391 + 1575757 + 267264 + 532480) * 1024,
+# HBM bytes per launch of the dominant (backward) kernel(s) as the hardware counted them: rocprofv3
+# --pmc FETCH_SIZE and --pmc WRITE_SIZE (two runs of this script; FETCH_SIZE scaled by the factor that
+# makes a plain copy of known size read its size).  A profiler cannot run inside this script, so the
+# figure is carried here with the summary file that holds the runs' commands and counters.
+MEASURED_TRAFFIC = {
+    "srwm_c4": ((490413 + 90624) * 1024, "profiles/srwm_c4_kernels.txt"),
+    "delta_c2": ((102444 + 53504) * 1024, "profiles/delta_kernels.txt"),
+    "delta_c2_chunk": ((82217 + 85992 + 16640 + 36864) * 1024, "profiles/delta_chunk_kernels.txt"),
+    "delta_c5": ((1316522 + 1323008) * 1024, "profiles/delta_kernels.txt"),
+    "delta_c5_chunk": ((1047391 + 1575757 + 267264 + 532480) * 1024, "profiles/delta_chunk_kernels.txt"),
 }
 
 WORKLOADS = {
@@ -247,7 +252,9 @@ def cpu_baseline(op, N, H, L, E, budget_s=20.0):
     batch slice sized to about `budget_s` seconds; tokens/s = slice_N * L / time."""
     import torch
     from oracle.recurrence import delta_recurrence, srwm_recurrence
-    cores = torch.get_num_threads()
+    # threads the recurrence runs on: the box's CPU share (OMP_NUM_THREADS there), never more than the host has
+    cores = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "0")) or torch.get_num_threads()))
+    torch.set_num_threads(cores)
     g = torch.Generator().manual_seed(0)
 
     def run(n):
@@ -315,15 +322,129 @@ def measure_lds_peak(dev):
     return best
 
 
+def chunk_flops(N, H, L, D, C=64):
+    """Algorithmic FLOPs (2 per multiply-add) of the chunkwise delta rule with chunks of C steps:
+    forward  per chunk  K K^T, Q K^T (2 C^2 D), K S, Q S (2 C D^2), triangular solve (C^2 D),
+             tril(B) U (C^2 D), K^T U (C D^2)                                   = 4 C^2 D + 3 C D^2 MACs
+    backward per chunk  the two C x C factors again (2 C^2 D), their use in dU, the solve, G1, X,
+             G1 K, G1^T Q, (X + X^T) K (7 C^2 D), and seven products with the D x D memory or its
+             gradient (S revert, K dS', Q^T dOut, K^T Y, dOut S^T, U dS'^T, Y S^T)   = 9 C^2 D + 7 C D^2 MACs
+    (what the two backward sweeps compute twice -- the revert and dS -- is counted once)."""
+    chunks = N * H * L / C
+    return 2.0 * (4 * C * C * D + 3 * C * D * D) * chunks, 2.0 * (9 * C * C * D + 7 * C * D * D) * chunks
+
+
+def vector_flops(op, N, H, L, E):
+    """Algorithmic fp32 FLOPs of the step-by-step kernels: 2 per element of the state and pass
+    (forward 3 passes SRWM / 2 delta, backward 6 / 4)."""
+    hs = N * H * L
+    if op.startswith("srwm"):
+        S = E * ((3 * E + 1 if op == "srwm_wide" else E) + 2 * E + 4)
+        return 6.0 * S * hs, 12.0 * S * hs
+    return 4.0 * E * E * hs, 8.0 * E * E * hs
+
+
+MFMA_PEAK_TFLOPS = {"delta_bf16": 2500.0, "delta": 157.3}   # dense bf16 / fp32 matrix peak
+VALU_FP32_PEAK_TFLOPS = 157.3
+
+
+def build_workload(name, dev):
+    import torch
+    import srwm_hip
+    op, N, H, L, E = WORKLOADS[name]
+    if op == "srwm":
+        step, t = srwm_step, srwm_setup(N, H, L, E, dev)
+    elif op == "srwm_layer":
+        step, t = srwm_layer_step, srwm_setup(N, H, L, E, dev)
+        t["slow"] = [w[0].contiguous() for w in t["W0"]]
+        t["gslow"] = [torch.empty_like(w) for w in t["slow"]]
+    elif op == "srwm_wide":
+        step, t = srwm_step, srwm_setup(N, H, L, E, dev, 3 * E + 1)
+    elif op == "srwm_steps":
+        step, t = srwm_steps_step, srwm_steps_setup(N, H, L, E, dev)
+    else:
+        step = delta_step
+        t = delta_setup(N, H, L, E, dev, torch.bfloat16 if op == "delta_bf16" else torch.float32)
+        if name.endswith("_chunk"):
+            t["fwd_flags"] = srwm_hip.FLAG_CHUNKWISE
+            t["bwd_flags"] = srwm_hip.FLAG_CHUNKWISE
+    return step, t
+
+
+def time_workload(step, t, steps, warmup):
+    """`warmup` untimed steps, then exactly `steps` steps between two device synchronisations.
+    Returns (wall seconds of the timed region, per-step forward ms, per-step backward ms) -- the
+    per-step figures from HIP events recorded on the stream the kernels are launched on."""
+    import torch
+    for _ in range(warmup):
+        step(t)
+    torch.cuda.synchronize()
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(t, evs[i])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    return elapsed, [e[0].elapsed_time(e[1]) for e in evs], [e[1].elapsed_time(e[2]) for e in evs]
+
+
+def median(xs):
+    xs = sorted(xs)
+    n = len(xs)
+    return xs[n // 2] if n % 2 else 0.5 * (xs[n // 2 - 1] + xs[n // 2])
+
+
+def roof(bound, amount, ms, peak, unit="GB/s"):
+    """amount: bytes (GB/s) or FLOPs (TFLOP/s) per launch; ms: duration of that launch."""
+    ach = amount / (ms * 1e-3) / (1e9 if unit == "GB/s" else 1e12)
+    return {"bound": bound, "achieved": round(ach, 1), "peak": round(peak, 1), "unit": unit,
+            "frac": round(ach / peak, 4), "traffic": None}
+
+
+def rooflines(name, fwd_ms, bwd_ms):
+    """The roofline records of one workload from its median kernel times."""
+    op, N, H, L, E = WORKLOADS[name]
+    lds_f, lds_b, hbm = algorithmic_bytes(op, N, H, L, E)
+    r = {}
+    if name.endswith("_chunk"):
+        # the chunkwise kernels are dense contractions: priced in FLOPs against the matrix-core peak
+        ff, fb = chunk_flops(N, H, L, E)
+        peak = MFMA_PEAK_TFLOPS[op]
+        r["roofline"] = dict(roof("mfma", fb, bwd_ms, peak, "TFLOP/s"), kernel="backward (column sweep + row sweep)")
+        r["roofline_fwd"] = dict(roof("mfma", ff, fwd_ms, peak, "TFLOP/s"), kernel="forward")
+        r["roofline_fwd_bwd"] = roof("mfma", ff + fb, fwd_ms + bwd_ms, peak, "TFLOP/s")
+    else:
+        r["roofline"] = dict(roof("lds", lds_b, bwd_ms, LDS_PEAK_GBS), kernel="backward")
+        r["roofline_fwd_bwd"] = roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS)
+        # the state lives in VGPRs, so the LDS bytes above are a yardstick, not traffic; the unit that
+        # actually limits these kernels is the fp32 vector ALU
+        vf, vb = vector_flops(op, N, H, L, E)
+        r["roofline_valu"] = dict(roof("valu_fp32", vb, bwd_ms, VALU_FP32_PEAK_TFLOPS, "TFLOP/s"), kernel="backward")
+        r["roofline_valu_fwd_bwd"] = roof("valu_fp32", vf + vb, fwd_ms + bwd_ms, VALU_FP32_PEAK_TFLOPS, "TFLOP/s")
+    r["roofline_hbm"] = roof("hbm", hbm, fwd_ms + bwd_ms, HBM_PEAK_GBS)
+    if name in MEASURED_TRAFFIC:
+        nbytes, source = MEASURED_TRAFFIC[name]
+        r["roofline"].update(traffic=nbytes, traffic_kind="hbm_counter", traffic_source=source)
+    return r
+
+
+# Driver-visible figures for the other benchmark configurations: (workload, timed steps, warm-up)
+OTHER_WORKLOADS = (("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
+                   ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="srwm_c4", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--no-lds-probe", action="store_true")
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the compact records of the other configurations that the default run appends")
     a = ap.parse_args()
     if a.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this operator runs on ONE GPU (sequences shard over GPUs without any "
@@ -338,44 +459,11 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     op, N, H, L, E = WORKLOADS[a.workload]
-    if op == "srwm":
-        step, t = srwm_step, srwm_setup(N, H, L, E, dev)
-    elif op == "srwm_layer":
-        step, t = srwm_layer_step, srwm_setup(N, H, L, E, dev)
-        t["slow"] = [w[0].contiguous() for w in t["W0"]]
-        t["gslow"] = [torch.empty_like(w) for w in t["slow"]]
-    elif op == "srwm_wide":
-        step, t = srwm_step, srwm_setup(N, H, L, E, dev, 3 * E + 1)
-    elif op == "srwm_steps":
-        step, t = srwm_steps_step, srwm_steps_setup(N, H, L, E, dev)
-    else:
-        step = delta_step
-        t = delta_setup(N, H, L, E, dev, torch.bfloat16 if op == "delta_bf16" else torch.float32)
-        if a.workload.endswith("_chunk"):
-            t["fwd_flags"] = srwm_hip.FLAG_CHUNKWISE
-            t["bwd_flags"] = srwm_hip.FLAG_CHUNKWISE
-
-    for _ in range(a.warmup):
-        step(t)
-    torch.cuda.synchronize()
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(a.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(a.steps):
-        step(t, evs[i])
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in evs) / a.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in evs) / a.steps
+    step, t = build_workload(a.workload, dev)
+    elapsed, fwd_all, bwd_all = time_workload(step, t, a.steps, a.warmup)
+    fwd_ms, bwd_ms = median(fwd_all), median(bwd_all)
     ms_per_step = elapsed * 1e3 / a.steps
     tokens_per_s = N * L * a.steps / elapsed
-    lds_f, lds_b, hbm = algorithmic_bytes(op, N, H, L, E)
-
-    def roof(bound, bytes_, ms, peak):
-        ach = bytes_ / (ms * 1e-3) / 1e9
-        return {"bound": bound, "achieved": round(ach, 1), "peak": round(peak, 1), "unit": "GB/s",
-                "frac": round(ach / peak, 4), "traffic": None}
 
     res = {
         "metric": "fwd+bwd tokens/sec SRWM B=32 H=16 T=512 d=64; % LDS/HBM roofline"
@@ -386,21 +474,42 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{a.workload}: {op} fwd+bwd N={N} H={H} L={L} E={E}, fp32 state, "
                                "state re-initialised per step, seeded synthetic inputs"},
-        "kernel_ms": {"forward": round(fwd_ms, 4), "backward": round(bwd_ms, 4)},
-        "roofline": dict(roof("lds", lds_b, bwd_ms, LDS_PEAK_GBS), kernel="backward",
-                         traffic=MEASURED_TRAFFIC_BYTES.get(a.workload)),
-        "roofline_fwd_bwd": roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS),
-        "roofline_hbm": roof("hbm", hbm, fwd_ms + bwd_ms, HBM_PEAK_GBS),
+        "kernel_ms": {"forward": round(fwd_ms, 4), "backward": round(bwd_ms, 4), "stat": f"median of {a.steps} steps (HIP events)",
+                      "forward_mean": round(sum(fwd_all) / a.steps, 4), "backward_mean": round(sum(bwd_all) / a.steps, 4)},
     }
+    res.update(rooflines(a.workload, fwd_ms, bwd_ms))
     if op == "srwm_steps":
         res["per_step_loop_ms"] = round(srwm_per_step_loop_ms(t, N, H, L, E, dev), 3)
         res["config"]["workload"] += ("; gradient cut at the carried state, 5 % resets; per_step_loop_ms = the same "
                                       "unroll as L launches of the L = 1 operator (forward + backward)")
     lds_meas = None if a.no_lds_probe else measure_lds_peak(dev)
-    if lds_meas:
+    if lds_meas and res["roofline_fwd_bwd"]["bound"] == "lds":
         res["lds_peak_measured_GBs"] = round(lds_meas, 1)
         res["roofline_fwd_bwd"]["frac_of_measured_lds_peak"] = round(
             res["roofline_fwd_bwd"]["achieved"] / lds_meas, 4)
+    del step, t
+    if a.workload == "srwm_c4" and not a.no_other_workloads:
+        # the other benchmark configurations, timed the same way in the same process (about 2 s of GPU time)
+        others = {}
+        for name, k, w in OTHER_WORKLOADS:
+            torch.cuda.empty_cache()
+            o_op, oN, oH, oL, oE = WORKLOADS[name]
+            st, tt = build_workload(name, dev)
+            el, f_all, b_all = time_workload(st, tt, k, w)
+            f_ms, b_ms = median(f_all), median(b_all)
+            rl = rooflines(name, f_ms, b_ms)
+            rec = {"shape": f"{o_op} N={oN} H={oH} L={oL} E={oE}", "steps": k, "forward_ms": round(f_ms, 4),
+                   "backward_ms": round(b_ms, 4), "ms_per_step": round(el * 1e3 / k, 4),
+                   "tokens_per_s": round(oN * oL * k / el, 1)}
+            main_roof = rl["roofline_fwd_bwd"]
+            rec["fwd_bwd_frac"] = main_roof["frac"]
+            rec["fwd_bwd_bound"] = main_roof["bound"]
+            rec["fwd_bwd_achieved"] = f"{main_roof['achieved']} {main_roof['unit']}"
+            if "roofline_valu_fwd_bwd" in rl:
+                rec["fwd_bwd_frac_valu_fp32"] = rl["roofline_valu_fwd_bwd"]["frac"]
+            others[name] = rec
+            del st, tt
+        res["other_workloads"] = others
     if not a.no_cpu_baseline:
         res["cpu_baseline"] = cpu_baseline("srwm_wide" if op == "srwm_wide" else "srwm" if op.startswith("srwm") else "delta",
                                            N, H, L, E, a.cpu_budget)
