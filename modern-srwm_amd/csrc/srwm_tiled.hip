@@ -315,14 +315,21 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         group_sum_n<RG, NC>(e);
 
         // ---- activations of step t, redundantly in every wave, lane <-> element el
+        // At E = 64 a vector fills the wave and the kernel is bound by instruction issue: the 64-lane
+        // reductions travel in pairs / fours (wave_allreduce_pair, wave_sum_quad), and the sums that do
+        // not depend on the activations (the early b~ of step t+1) ride along with the softmax sums.
+        constexpr bool FULL = E == kWave;
         float mx[2] = {qraw, kraw};
-        group_max_n<E, 2>(mx);
-        const float eq = exp_2ulp(qraw - mx[0]), ek = exp_2ulp(kraw - mx[1]);
+        if constexpr (FULL) wave_allreduce_pair<OpMax>(mx[0], mx[1]);
+        else group_max_n<E, 2>(mx);
+        const float eq = exp_shifted(qraw, mx[0] * kLog2e), ek = exp_shifted(kraw, mx[1] * kLog2e);
         float sm[2] = {eq, ek};
-        group_sum_n<E, 2>(sm);
+        float early_b = wbe * xb, early_y = XC ? wye * xb : early_b;   // -> b~ (and the last y column) of step t+1, before the write
+        if constexpr (FULL) wave_sum_quad(sm[0], sm[1], early_b, early_y);
+        else group_sum_n<E, 2>(sm);
         const float qn = eq * fast_rcp(sm[0]), kn = ek * fast_rcp(sm[1]);
         // sigmoid saturates to 0 / 1 in fp32 well inside +-80; the clamp keeps exp finite
-        const float sg = fast_rcp(1.f + exp_2ulp(-fminf(fmaxf(braw, -80.f), 80.f)));
+        const float sg = fast_rcp(1.f + __builtin_amdgcn_exp2f(fminf(fmaxf(braw, -80.f), 80.f) * -kLog2e));
         const float bt[4] = {quad_broadcast<0>(sg), quad_broadcast<1>(sg), quad_broadcast<2>(sg),
                              quad_broadcast<3>(sg)};
         const float dv = qn - kn;
@@ -353,12 +360,21 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         float s[NS];
         s[0] = wbe * dv;   // -> b diff
         s[1] = kn * xb;    // -> k . x_{t+1}
-        s[2] = wbe * xb;   // -> early b~ of step t+1
+        s[2] = early_b;
         if constexpr (XC) {
             s[3] = wye * dv;
-            s[4] = wye * xb;
+            s[4] = early_y;
         }
-        group_sum_n<E, NS>(s);
+        if constexpr (FULL) {
+            if constexpr (XC) {
+                float dup = s[3];
+                wave_sum_quad(s[0], s[1], s[3], dup);
+            } else {
+                wave_allreduce_pair<OpSum>(s[0], s[1]);
+            }
+        } else {
+            group_sum_n<E, NS>(s);
+        }
         const float pbd = s[0], kx = s[1];
         if (rg == 0) {
             store_y(ydiff_s, oy, &dif[0]);

@@ -310,6 +310,43 @@ __device__ __forceinline__ float swap_add16(float x, float y) {
     return x + y;
 }
 
+// All-reduce of TWO values over the 64 lanes of a wave for little more than the price of one: one
+// v_permlane32_swap folds the halves so that lanes 0..31 carry partial results of `a` and lanes
+// 32..63 those of `b`; the four in-row steps and one row_bcast:15 step then serve both, and lanes
+// 31 / 63 hold the totals.  9 vector instructions instead of 14.
+template <class Op>
+__device__ __forceinline__ void wave_allreduce_pair(float &a, float &b) {
+    float x = a, y = b;
+    swap_pairs<32>(x, y);
+    float v = Op::f(x, y);
+    v = Op::f(v, dpp_mov<kDppXor1>(v));
+    v = Op::f(v, dpp_mov<kDppXor2>(v));
+    v = Op::f(v, dpp_mov<kDppHalfMirror>(v));
+    v = Op::f(v, dpp_mov<kDppMirror>(v));
+    Op::template rows_accumulate<15>(v);
+    a = readlane(v, 31);
+    b = readlane(v, 63);
+}
+
+// Sums of FOUR values over the 64 lanes: two v_permlane32_swap and one v_permlane16_swap leave each
+// 16-lane row with the partial sums of one value (rows 0..3: a, c, b, d), four in-row steps finish
+// them.  14 vector instructions instead of 28; with three values pass the third one twice.
+__device__ __forceinline__ void wave_sum_quad(float &a, float &b, float &c, float &d) {
+    float x0 = a, y0 = b, x1 = c, y1 = d;
+    swap_pairs<32>(x0, y0, x1, y1);
+    float ab = x0 + y0, cd = x1 + y1;
+    swap_pairs<16>(ab, cd);
+    float v = ab + cd;
+    v += dpp_mov<kDppXor1>(v);
+    v += dpp_mov<kDppXor2>(v);
+    v += dpp_mov<kDppHalfMirror>(v);
+    v += dpp_mov<kDppMirror>(v);
+    a = readlane(v, 0);
+    c = readlane(v, 16);
+    b = readlane(v, 32);
+    d = readlane(v, 48);
+}
+
 // exp(x) to about 2 ulp with one v_exp_f32: x*log2(e) is formed in two pieces (product
 // rounding error via fma, low bits of log2(e)) and the small remainder r is applied as
 // 2^r ~ 1 + r ln 2.  Meant for softmax arguments (x <= 0) and clamped sigmoid arguments.
@@ -320,6 +357,16 @@ __device__ __forceinline__ float exp_2ulp(float x) {
     r = fmaf(x, kL2eLo, r);
     const float e = __builtin_amdgcn_exp2f(t);
     return fmaf(e, r * 0.693147180559945309f, e);
+}
+
+// exp(x - m) for a softmax whose normaliser is formed from the same values: one fma and one
+// v_exp_f32.  `m_l2e` = m * log2(e), rounded once and shared by all elements, so its rounding error
+// is a common factor that the normalisation removes; what remains is the rounding of the fma
+// result t and of the constant, a relative error of about |t| * 5e-8 -- below 2 ulp for elements
+// within e^-3 of the largest, and falling in absolute terms for the smaller ones.
+constexpr float kLog2e = 1.44269502162933349609375f;
+__device__ __forceinline__ float exp_shifted(float x, float m_l2e) {
+    return __builtin_amdgcn_exp2f(fmaf(x, kLog2e, -m_l2e));
 }
 
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
