@@ -202,6 +202,52 @@ def test_full_headline_shape_properties():
             assert rel_err(b[n][rows].cpu().numpy(), ob[n]) < TOL, n
 
 
+def test_full_rl_actor_shape_against_the_oracle():
+    """benchmark configuration 3 at full size (N=32, H=8, L=100, E=32: 256 workgroups, one per CU, the
+    regime its timing is quoted in), inputs built the way the RL layer builds them (256 features ->
+    Linear -> heads -> softmax -> permuted view, reinforcement_learning/torchbeast/layer.py:382-385;
+    weights ~ N(0, 1/sqrt(32)), :368-375).  Small enough for the oracle to check EVERY sequence, plus
+    the size-independent properties of the larger shapes."""
+    print("case full C3", flush=True)
+    N, H, L, E = 32, 8, 100, 32
+    g = torch.Generator().manual_seed(0)
+    feats = torch.randn(L, N, H * E, generator=g, dtype=torch.float64)
+    lin = torch.nn.Linear(H * E, H * E).double()
+    with torch.no_grad():
+        bound = 1.0 / math.sqrt(H * E)                      # nn.Linear's default initialisation, seeded here
+        lin.weight.copy_((torch.rand(H * E, H * E, generator=g, dtype=torch.float64) * 2 - 1) * bound)
+        lin.bias.copy_((torch.rand(H * E, generator=g, dtype=torch.float64) * 2 - 1) * bound)
+        proj = torch.softmax(lin(feats).view(L, N, H, E), dim=-1)   # (L, N, H, E) storage ...
+    x = proj.permute(1, 2, 0, 3)                             # ... read as (N, H, L, E) through its strides
+    std = 1.0 / math.sqrt(E)
+    W = [(torch.randn(1, H, E, w, generator=g, dtype=torch.float64) * std).repeat(N, 1, 1, 1) for w in (E, E, E, 4)]
+    go = torch.randn(L, N, H, E, generator=g, dtype=torch.float64).permute(1, 2, 0, 3)
+    assert not x.is_contiguous() and not go.is_contiguous()
+    f, b = run_hip(x, W, go, 0)
+    assert torch.allclose(f["q"].sum(-1), torch.ones_like(f["q"][..., 0]), atol=1e-5)
+    assert torch.allclose(f["k"].sum(-1), torch.ones_like(f["k"][..., 0]), atol=1e-5)
+    assert (f["beta"] > 0).all() and (f["beta"] < 1).all()
+    xn, gon = x.contiguous().numpy(), go.contiguous().numpy()
+    of = oracle.srwm_forward(xn, *[w.numpy() for w in W])
+    ob = oracle.srwm_backward(xn, of, gon)
+    for n in FWD_NAMES + ("W_y", "W_q", "W_k", "w_b"):
+        assert rel_err(f[n].cpu().numpy(), of[n]) < TOL, n
+    for n in b:
+        assert rel_err(b[n].cpu().numpy(), ob[n]) < TOL, n
+    # the backward is linear in the upstream gradient
+    go2 = torch.randn(go.shape, generator=g, dtype=torch.float64)
+    _, b2 = run_hip(x, W, go2, 0)
+    _, b3 = run_hip(x, W, 2 * go - 3 * go2, 0)
+    for n in b:
+        assert rel_err(b3[n].cpu().numpy(), (2 * b[n] - 3 * b2[n]).cpu().numpy()) < 5e-5, n
+    # and the LDS-resident kernels agree at this size too
+    import srwm_hip
+    fg, bg = run_hip(x, W, go, srwm_hip.FLAG_GENERIC)
+    for n in b:
+        assert rel_err(bg[n].cpu().numpy(), ob[n]) < TOL, n
+    assert rel_err(fg["out"].cpu().numpy(), of["out"]) < TOL
+
+
 def test_errors_are_reported_not_swallowed():
     import srwm_hip
     dev = _dev()
