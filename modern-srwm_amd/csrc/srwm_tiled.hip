@@ -318,14 +318,18 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         // At E = 64 a vector fills the wave and the kernel is bound by instruction issue: the 64-lane
         // reductions travel in pairs / fours (wave_allreduce_pair, wave_sum_quad), and the sums that do
         // not depend on the activations (the early b~ of step t+1) ride along with the softmax sums.
-        constexpr bool FULL = E == kWave;
+        // At E = 32 a wave holds each vector twice (lane l and l + 32): one half reduces q, the other k,
+        // and the narrow columns, which differ between the halves, are summed two at a time.
+        constexpr bool FULL = E == kWave, HALF = 2 * E == kWave;
         float mx[2] = {qraw, kraw};
         if constexpr (FULL) wave_allreduce_pair<OpMax>(mx[0], mx[1]);
+        else if constexpr (HALF) half_allreduce_pair<OpMax>(mx[0], mx[1]);
         else group_max_n<E, 2>(mx);
         const float eq = exp_shifted(qraw, mx[0] * kLog2e), ek = exp_shifted(kraw, mx[1] * kLog2e);
         float sm[2] = {eq, ek};
         float early_b = wbe * xb, early_y = XC ? wye * xb : early_b;   // -> b~ (and the last y column) of step t+1, before the write
         if constexpr (FULL) wave_sum_quad(sm[0], sm[1], early_b, early_y);
+        else if constexpr (HALF) half_allreduce_pair<OpSum>(sm[0], sm[1]);
         else group_sum_n<E, 2>(sm);
         const float qn = eq * fast_rcp(sm[0]), kn = ek * fast_rcp(sm[1]);
         // sigmoid saturates to 0 / 1 in fp32 well inside +-80; the clamp keeps exp finite
@@ -372,6 +376,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             } else {
                 wave_allreduce_pair<OpSum>(s[0], s[1]);
             }
+        } else if constexpr (HALF) {
+            half_sum_pair(s[0], s[2]);
+            s[1] = half_sum_uniform(s[1]);
+            if constexpr (XC) half_sum_pair(s[3], s[4]);
         } else {
             group_sum_n<E, NS>(s);
         }

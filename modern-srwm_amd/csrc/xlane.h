@@ -347,6 +347,49 @@ __device__ __forceinline__ void wave_sum_quad(float &a, float &b, float &c, floa
     d = readlane(v, 48);
 }
 
+// The same economy for vectors of 32 elements, which a wave holds twice (lane l and lane l + 32 carry
+// the same element): the lower half reduces `a`, the upper half `b`, and the totals are read from
+// lanes 31 and 63.  8 vector instructions instead of 20.
+template <class Op>
+__device__ __forceinline__ void half_allreduce_pair(float &a, float &b) {
+    float v = (threadIdx.x & 32) ? b : a;
+    v = Op::f(v, dpp_mov<kDppXor1>(v));
+    v = Op::f(v, dpp_mov<kDppXor2>(v));
+    v = Op::f(v, dpp_mov<kDppHalfMirror>(v));
+    v = Op::f(v, dpp_mov<kDppMirror>(v));
+    Op::template rows_accumulate<15>(v);
+    a = readlane(v, 31);
+    b = readlane(v, 63);
+}
+
+// Sums over each 32-lane half of TWO values that differ between the halves; every lane receives the
+// two sums of its own half.  One v_permlane16_swap folds the rows of a half (even rows then carry
+// `a`, odd rows `b`), four in-row steps finish them, a second swap hands each row the other's total.
+__device__ __forceinline__ void half_sum_pair(float &a, float &b) {
+    float x = a, y = b;
+    swap_pairs<16>(x, y);
+    float v = x + y;
+    v += dpp_mov<kDppXor1>(v);
+    v += dpp_mov<kDppXor2>(v);
+    v += dpp_mov<kDppHalfMirror>(v);
+    v += dpp_mov<kDppMirror>(v);
+    x = v;
+    y = v;
+    swap_pairs<16>(x, y);
+    a = x;
+    b = y;
+}
+
+// Sum over the 32 lanes of a value that both halves hold alike (either half's total serves).
+__device__ __forceinline__ float half_sum_uniform(float v) {
+    v += dpp_mov<kDppXor1>(v);
+    v += dpp_mov<kDppXor2>(v);
+    v += dpp_mov<kDppHalfMirror>(v);
+    v += dpp_mov<kDppMirror>(v);
+    OpSum::rows_accumulate<15>(v);
+    return readlane(v, 31);
+}
+
 // exp(x) to about 2 ulp with one v_exp_f32: x*log2(e) is formed in two pieces (product
 // rounding error via fma, low bits of log2(e)) and the small remainder r is applied as
 // 2^r ~ 1 + r ln 2.  Meant for softmax arguments (x <= 0) and clamped sigmoid arguments.
