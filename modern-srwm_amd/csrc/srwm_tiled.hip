@@ -705,13 +705,22 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 pg[beta_of(c)] = fmaf(gdif[c], dif[c], pg[beta_of(c)]);
                 gdif[c] *= bt[beta_of(c)];
             }
-            const float ginsb = group_sum<E>(gbe * kb);
-            const float gdifb = bt[3] * ginsb;
-            float ginsy = 0.f, gdify = 0.f;
+            // sums over a vector's E lanes: paired across the wave (E = 64) or across its two halves
+            // (E = 32, where lane l and l + 32 hold the same element but different narrow columns)
+            constexpr bool FULL = E == kWave, HALF = 2 * E == kWave;
+            float ginsb = gbe * kb, ginsy = XC ? gye * kb : 0.f;
             if constexpr (XC) {
-                ginsy = group_sum<E>(gye * kb);
-                gdify = bt[0] * ginsy;
+                if constexpr (FULL) wave_allreduce_pair<OpSum>(ginsb, ginsy);
+                else if constexpr (HALF) half_sum_pair(ginsb, ginsy);
+                else {
+                    ginsb = group_sum<E>(ginsb);
+                    ginsy = group_sum<E>(ginsy);
+                }
+            } else {
+                ginsb = HALF ? half_sum_each(ginsb) : group_sum<E>(ginsb);
             }
+            const float gdifb = bt[3] * ginsb;
+            const float gdify = bt[0] * ginsy;
 
             // ---- row sums  a = G ins,  u = W_{t-1} g_diff
             float a[R], u[R];
@@ -756,14 +765,17 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             }
             gk -= gq;
             float dqk[2] = {gq * qb, gk * kb};
-            group_sum_n<E, 2>(dqk);
+            if constexpr (FULL) wave_allreduce_pair<OpSum>(dqk[0], dqk[1]);
+            else if constexpr (HALF) half_allreduce_pair<OpSum>(dqk[0], dqk[1]);
+            else group_sum_n<E, 2>(dqk);
             const float gpq = qb * (gq - dqk[0]), gpk = kb * (gk - dqk[1]);
             float gpreb;
             if constexpr (E == kWave && !XC) {
                 // jb == wave: a wave only needs the beta gradient of its own w_b column, one sum instead of three
                 float gbw;
                 if (jb < 3) {
-                    gbw = group_sum<NCG>(gbp[par][lane % NCG][jb]);
+                    static_assert(NCG == 32, "both halves of the wave read the same 32 partial sums");
+                    gbw = half_sum_uniform(gbp[par][lane % NCG][jb]);
                 } else {
                     float p3[4];
                     lds_read_vec<4>(p3, &gbp3[par][0]);
@@ -775,7 +787,12 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 float part[4];
                 lds_read_vec<4>(part, &gbp[par][lane % NCG][0]);
                 float p012[3] = {part[0], part[1], part[2]};
-                group_sum_n<NCG, 3>(p012);
+                if constexpr (NCG == 32) {   // both halves of the wave hold the same 32 partial sums
+                    half_allreduce_pair<OpSum>(p012[0], p012[1]);
+                    p012[2] = half_sum_uniform(p012[2]);
+                } else {
+                    group_sum_n<NCG, 3>(p012);
+                }
 #pragma unroll
                 for (int j = 0; j < 3; ++j) gb[j] = p012[j];
                 float p3[4];

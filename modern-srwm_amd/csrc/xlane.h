@@ -390,6 +390,15 @@ __device__ __forceinline__ float half_sum_uniform(float v) {
     return readlane(v, 31);
 }
 
+// Sum over each 32-lane half of a value that differs between the halves, in every lane of the half.
+__device__ __forceinline__ float half_sum_each(float v) {
+    v += dpp_mov<kDppXor1>(v);
+    v += dpp_mov<kDppXor2>(v);
+    v += dpp_mov<kDppHalfMirror>(v);
+    v += dpp_mov<kDppMirror>(v);
+    return swap_add16(v, v);
+}
+
 // exp(x) to about 2 ulp with one v_exp_f32: x*log2(e) is formed in two pieces (product
 // rounding error via fma, low bits of log2(e)) and the small remainder r is applied as
 // 2^r ~ 1 + r ln 2.  Meant for softmax arguments (x <= 0) and clamped sigmoid arguments.
