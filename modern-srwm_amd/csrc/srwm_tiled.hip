@@ -752,16 +752,31 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             __syncthreads();
 
             // ---- every wave, lane <-> element el: gradients of q, k, beta before activation
-            float gk = rowm[par][0][0][el], gq = rowm[par][1][0][el];
+            float gk, gq;
+            if constexpr (HALF) {
+                // lane l and lane l + 32 would form the same two sums: each half forms one of them
+                const int sel = lane >> 5;   // 0: W g_diff (-> gq), 1: G ins (-> gk)
+                float part = rowm[par][1 - sel][0][el];
 #pragma unroll
-            for (int wv = 1; wv < NW; ++wv) {
-                gk += rowm[par][0][wv][el];
-                gq += rowm[par][1][wv][el];
-            }
+                for (int wv = 1; wv < NW; ++wv) part += rowm[par][1 - sel][wv][el];
 #pragma unroll
-            for (int j = 0; j < NXS; ++j) {
-                gk += rowb[par][0][j][el];
-                gq += rowb[par][1][j][el];
+                for (int j = 0; j < NXS; ++j) part += rowb[par][1 - sel][j][el];
+                gq = part;
+                gk = part;
+                swap_pairs<32>(gq, gk);   // gq: the lower half's sum in both halves, gk: the upper half's
+            } else {
+                gk = rowm[par][0][0][el];
+                gq = rowm[par][1][0][el];
+#pragma unroll
+                for (int wv = 1; wv < NW; ++wv) {
+                    gk += rowm[par][0][wv][el];
+                    gq += rowm[par][1][wv][el];
+                }
+#pragma unroll
+                for (int j = 0; j < NXS; ++j) {
+                    gk += rowb[par][0][j][el];
+                    gq += rowb[par][1][j][el];
+                }
             }
             gk -= gq;
             float dqk[2] = {gq * qb, gk * kb};
@@ -799,10 +814,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                 lds_read_vec<4>(p3, &gbp3[par][0]);
                 gb[3] = (p3[0] + p3[1]) + (p3[2] + p3[3]);
                 if constexpr (XC) gb[0] += gbp3[par][4];
-                float gpb[4];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) gpb[j] = gb[j] * bt[j] * (1.f - bt[j]);
-                gpreb = jb == 0 ? gpb[0] : jb == 1 ? gpb[1] : jb == 2 ? gpb[2] : gpb[3];
+                const float gbj = jb == 0 ? gb[0] : jb == 1 ? gb[1] : jb == 2 ? gb[2] : gb[3];   // this thread's w_b column
+                gpreb = gbj * btj * (1.f - btj);
             }
             if (lane < E) {
                 exch[wave][0][lane] = gpq;
