@@ -449,7 +449,7 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
         } else if (tlen == TT) {
             Ops a, b;
             fetch(a, TT - 1);
-#pragma unroll 1
+#pragma unroll
             for (int tt = TT - 1; tt >= 0; tt -= 2) {
                 fetch(b, tt - 1);
                 step(a, tt);

@@ -151,23 +151,24 @@ __device__ __forceinline__ void wave_lds_fence() {
 // the upper half / odd rows, the pair sums of the old y: a reduce-scatter step that halves
 // the number of live values.  With x == y it is an all-reduce over the pair.
 // (Inline assembly because the compiler builtin of this toolchain returns the first result
-// twice.  The s_nop pairs cover the VALU-write -> swap and swap -> VALU-read wait states the
-// compiler's hazard recogniser cannot insert inside an asm block; swaps on distinct registers
-// need nothing between them, so they are issued in batches.)
+// twice.  The leading s_nop covers the two wait states a swap needs after a vector write of its
+// operands, which the compiler's hazard recogniser cannot insert inside an asm block -- it is what
+// the compiler itself emits around the builtin; nothing is needed between a swap and a vector
+// read of its results, nor between swaps on distinct registers, so they are issued in batches.)
 template <int W>
 __device__ __forceinline__ void swap_pairs(float &x0, float &y0) {
     if constexpr (W == 32)
-        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x0), "+v"(y0));
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(x0), "+v"(y0));
     else
-        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(x0), "+v"(y0));
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(x0), "+v"(y0));
 }
 template <int W>
 __device__ __forceinline__ void swap_pairs(float &x0, float &y0, float &x1, float &y1) {
     if constexpr (W == 32)
-        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\ts_nop 1"
+        asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3"
                      : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1));
     else
-        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\ts_nop 1"
+        asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3"
                      : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1));
 }
 template <int W>
@@ -175,11 +176,11 @@ __device__ __forceinline__ void swap_pairs(float &x0, float &y0, float &x1, floa
                                            float &y2, float &x3, float &y3) {
     if constexpr (W == 32)
         asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\tv_permlane32_swap_b32 %2, %3\n\t"
-                     "v_permlane32_swap_b32 %4, %5\n\tv_permlane32_swap_b32 %6, %7\n\ts_nop 1"
+                     "v_permlane32_swap_b32 %4, %5\n\tv_permlane32_swap_b32 %6, %7"
                      : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1), "+v"(x2), "+v"(y2), "+v"(x3), "+v"(y3));
     else
         asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\t"
-                     "v_permlane16_swap_b32 %4, %5\n\tv_permlane16_swap_b32 %6, %7\n\ts_nop 1"
+                     "v_permlane16_swap_b32 %4, %5\n\tv_permlane16_swap_b32 %6, %7"
                      : "+v"(x0), "+v"(y0), "+v"(x1), "+v"(y1), "+v"(x2), "+v"(y2), "+v"(x3), "+v"(y3));
 }
 
