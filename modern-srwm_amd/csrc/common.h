@@ -132,6 +132,33 @@ __device__ __forceinline__ float wave_max(float v) {
     return v;
 }
 
+// Workgroup -> (sequence, part) for kernels that run MS workgroups per sequence (MS = 1 or 2; the
+// parts own disjoint columns or rows of the memory but read the same input rows).  The 8 XCDs of the
+// device take consecutive workgroups in turn and each has an L2 of its own, so the two parts of a
+// sequence are placed 8 workgroups apart: same XCD, same L2, and the rows the second one asks for
+// are the ones the first has just fetched.  Groups of 16 workgroups hold 8 sequences; what is left
+// over when the number of sequences is not a multiple of 8 is numbered plainly.
+constexpr int kXcds = 8;
+template <int MS>
+__device__ __forceinline__ void seq_and_part(unsigned wg, unsigned nseq, int64_t &seq, int &part) {
+    static_assert(MS == 1 || MS == 2, "workgroups per sequence");
+    if constexpr (MS == 1) {
+        seq = wg;
+        part = 0;
+    } else {
+        const unsigned full = nseq / kXcds * kXcds;   // sequences in complete groups
+        if (wg < 2 * full) {
+            const unsigned grp = wg / (2 * kXcds), r = wg % (2 * kXcds);
+            seq = grp * kXcds + r % kXcds;
+            part = (int)(r / kXcds);
+        } else {
+            const unsigned r = wg - 2 * full;
+            seq = full + r / 2;
+            part = (int)(r % 2);
+        }
+    }
+}
+
 // ---- launchers (each returns a hipError_t as int, 0 = launched) -----------------
 // LDS-resident kernels that accept any E (M) whose state fits in the CU's LDS.
 size_t srwm_fwd_generic_lds_bytes(int E, int Y);

@@ -93,8 +93,10 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
     const int wave = wv & 3, hf = wv >> 2;           // column tile, row half
     const int e0 = hf * EB * 16;                     // first memory row held by this wave
     const int ln = lane & 15, lq = lane >> 4;        // accumulator layout: column ln, rows 4*lq + r
-    const int64_t seq = blockIdx.x / MS;
-    const int m0 = (int)(blockIdx.x % MS) * kMC;     // first memory column of this workgroup
+    int64_t seq;
+    int part;
+    seq_and_part<MS>(blockIdx.x, (unsigned)(p.N * p.H), seq, part);
+    const int m0 = part * kMC;                       // first memory column of this workgroup
     const int cw = 16 * wave;                        // first column of this wave inside the workgroup
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
     const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;

@@ -102,8 +102,10 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
     const int wave = wv & 3, hf = wv >> 2;          // column tile, row half
     const int e0 = hf * EB * 16;                    // first memory row held by this wave
     const int ln = lane & 15, lq = lane >> 4;
-    const int64_t seq = blockIdx.x / MS;
-    const int m0 = (int)(blockIdx.x % MS) * kWC + 16 * wave;   // first memory column of this wave
+    int64_t seq;
+    int part;
+    seq_and_part<MS>(blockIdx.x, (unsigned)(p.N * p.H), seq, part);
+    const int m0 = part * kWC + 16 * wave;          // first memory column of this wave
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
     const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;
     const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
@@ -378,8 +380,10 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     const int wave = wv & 3, hf = wv >> 2;           // row block, column half
     const int m0 = hf * MB * 16;                     // first memory column held by this wave
     const int ln = lane & 15, lq = lane >> 4;
-    const int64_t seq = blockIdx.x / MS;
-    const int e0 = (int)(blockIdx.x % MS) * kWC;     // first memory row of this workgroup
+    int64_t seq;
+    int part;
+    seq_and_part<MS>(blockIdx.x, (unsigned)(p.N * p.H), seq, part);
+    const int e0 = part * kWC;                       // first memory row of this workgroup
     const int cw = 16 * wave;                        // this wave's rows inside it
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
     const TI *qb = p.Q + n * p.qs.n + h * p.qs.h + e0;

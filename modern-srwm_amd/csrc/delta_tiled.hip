@@ -184,8 +184,10 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int rg = lane % RG, cg = wave * CGW + lane / RG;
     const int r0 = rg * R, c0 = cg * CC;
-    const int64_t seq = blockIdx.x / MS;
-    const int m0 = (int)(blockIdx.x % MS) * MC;   // first memory column of this workgroup
+    int64_t seq;
+    int part;
+    seq_and_part<MS>(blockIdx.x, (unsigned)(p.N * p.H), seq, part);
+    const int m0 = part * MC;   // first memory column of this workgroup
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
     const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;
     const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
@@ -324,8 +326,10 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
     const int rg = lane % RG, cg = wave * CGW + lane / RG;
     const int r0 = rg * R, c0 = cg * CC;
-    const int64_t seq = blockIdx.x / MS;
-    const int m0 = (int)(blockIdx.x % MS) * MC;
+    int64_t seq;
+    int part;
+    seq_and_part<MS>(blockIdx.x, (unsigned)(p.N * p.H), seq, part);
+    const int m0 = part * MC;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
     const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;
     const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
