@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace fw {
 
 constexpr int kWave = 64;
@@ -191,5 +193,26 @@ int launch_delta_bwd_chunk(const DeltaBwdParams &p, hipStream_t s);
 int launch_delta_bwd_chunk_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s);
 
 constexpr size_t kMaxLdsBytes = 160 * 1024;  // gfx950: 160 KB of LDS per CU / workgroup
+
+// Lifts the dynamic-LDS limit of kernel K to the device's maximum, once per device and process.
+// The limit is state of the function, shared by all host threads: it is only ever raised, and to
+// the same value by everyone, so concurrent launches with different LDS sizes cannot undercut each
+// other.  Returns a hipError_t as int.
+template <auto K>
+int allow_max_dynamic_lds() {
+    static std::atomic<unsigned long long> done{0};   // one bit per device ordinal
+    int dev = 0, v = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    const unsigned long long bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return 0;
+    e = hipDeviceGetAttribute(&v, hipDeviceAttributeMaxSharedMemoryPerBlock, dev);
+    if (e != hipSuccess) return (int)e;
+    const int lim = v < (int)kMaxLdsBytes ? v : (int)kMaxLdsBytes;
+    e = hipFuncSetAttribute((const void *)K, hipFuncAttributeMaxDynamicSharedMemorySize, lim);
+    if (e != hipSuccess) return (int)e;
+    done.fetch_or(bit, std::memory_order_release);
+    return 0;
+}
 
 }  // namespace fw

@@ -295,9 +295,7 @@ template <class TI, int D, int MS, int KS>
 int launch_chunk(const ChunkFwdP<TI> &p, hipStream_t s) {
     constexpr size_t lds = FwdLds<TI, D, KS>::kBytes;
     static_assert(lds <= kMaxLdsBytes, "LDS budget");
-    hipError_t err = hipFuncSetAttribute((const void *)delta_fwd_chunk_kernel<TI, D, MS, KS>,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (err != hipSuccess) return (int)err;
+    if (const int err = allow_max_dynamic_lds<delta_fwd_chunk_kernel<TI, D, MS, KS>>()) return err;
     hipLaunchKernelGGL((delta_fwd_chunk_kernel<TI, D, MS, KS>), dim3(p.N * p.H * MS), dim3(kThreads * KS), lds, s, p);
     return (int)hipGetLastError();
 }

@@ -622,12 +622,8 @@ template <class TI, int D, int MS, int C2, int KS, int KSR>
 int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
     constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2>::kBytes;
     static_assert(lds1 <= (int)kMaxLdsBytes && lds2 <= (int)kMaxLdsBytes, "LDS budget");
-    hipError_t err = hipFuncSetAttribute((const void *)delta_bwd_chunk_col_kernel<TI, D, MS, KS>,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, lds1);
-    if (err != hipSuccess) return (int)err;
-    err = hipFuncSetAttribute((const void *)delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR>,
-                              hipFuncAttributeMaxDynamicSharedMemorySize, lds2);
-    if (err != hipSuccess) return (int)err;
+    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_col_kernel<TI, D, MS, KS>>()) return err;
+    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR>>()) return err;
     const int grid = p.N * p.H * MS;
     if (MS > 1)   // two workgroups of the column sweep add their parts of grad_beta
         hipLaunchKernelGGL(zero_words_kernel, dim3(256), dim3(256), 0, s, p.gbeta, (int64_t)p.N * p.H * p.L);

@@ -167,18 +167,14 @@ size_t delta_bwd_generic_lds_bytes(int E, int M) {
 
 int launch_delta_fwd_generic(const DeltaFwdParams &p, hipStream_t s) {
     const size_t lds = delta_fwd_generic_lds_bytes(p.E, p.M);
-    hipError_t err = hipFuncSetAttribute((const void *)delta_fwd_generic_kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (err != hipSuccess) return (int)err;
+    if (const int err = allow_max_dynamic_lds<delta_fwd_generic_kernel>()) return err;
     hipLaunchKernelGGL(delta_fwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
     return (int)hipGetLastError();
 }
 
 int launch_delta_bwd_generic(const DeltaBwdParams &p, hipStream_t s) {
     const size_t lds = delta_bwd_generic_lds_bytes(p.E, p.M);
-    hipError_t err = hipFuncSetAttribute((const void *)delta_bwd_generic_kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (err != hipSuccess) return (int)err;
+    if (const int err = allow_max_dynamic_lds<delta_bwd_generic_kernel>()) return err;
     hipLaunchKernelGGL(delta_bwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
     return (int)hipGetLastError();
 }

@@ -333,18 +333,14 @@ size_t srwm_bwd_generic_lds_bytes(int E, int Y) {
 
 int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s) {
     const size_t lds = srwm_fwd_generic_lds_bytes(p.E, p.Y);
-    hipError_t err = hipFuncSetAttribute((const void *)srwm_fwd_generic_kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (err != hipSuccess) return (int)err;
+    if (const int err = allow_max_dynamic_lds<srwm_fwd_generic_kernel>()) return err;
     hipLaunchKernelGGL(srwm_fwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
     return (int)hipGetLastError();
 }
 
 int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s) {
     const size_t lds = srwm_bwd_generic_lds_bytes(p.E, p.Y);
-    hipError_t err = hipFuncSetAttribute((const void *)srwm_bwd_generic_kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (err != hipSuccess) return (int)err;
+    if (const int err = allow_max_dynamic_lds<srwm_bwd_generic_kernel>()) return err;
     hipLaunchKernelGGL(srwm_bwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
     return (int)hipGetLastError();
 }

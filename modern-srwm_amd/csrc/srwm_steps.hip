@@ -289,9 +289,7 @@ size_t replay_lds_bytes(int E, int M) { return sizeof(float) * ((size_t)E * (M |
 
 int launch_replay(const ReplayParams &p, hipStream_t s) {
     const size_t lds = replay_lds_bytes(p.E, p.M);
-    hipError_t err = hipFuncSetAttribute((const void *)replay_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                         (int)lds);
-    if (err != hipSuccess) return (int)err;
+    if (const int err = allow_max_dynamic_lds<replay_kernel>()) return err;
     hipLaunchKernelGGL(replay_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
     return (int)hipGetLastError();
 }

@@ -72,6 +72,50 @@ def test_two_threads_on_their_own_streams():
         assert rel_err(dout.numpy(), df["out"]) < TOL and rel_err(gk.numpy(), db["grad_K"]) < TOL
 
 
+def test_threads_with_different_state_sizes_do_not_disturb_each_other():
+    """Two host threads drive the LDS-resident kernels with different head sizes (12 and 48: a small
+    and a large dynamic LDS request) at the same time.  The per-kernel LDS limit is process-wide state;
+    it must never be lowered under a thread that needs more.  Every call must succeed and reproduce
+    the result of the same call made alone."""
+    print("case two threads, different LDS sizes", flush=True)
+    import srwm_hip
+    dev = _dev()
+
+    def run(E, seed, stream=None):
+        x, W, go = srwm_inputs(2, 2, 9, E, seed=seed, w_std=0.2, per_batch_state=True)
+        xd, god = x.to(dev, torch.float32), go.to(dev, torch.float32)
+        Wd = [w.to(dev, torch.float32).contiguous() for w in W]
+        new = lambda w: torch.empty(2, 2, 9, w, device=dev)
+        f = [new(E), new(E), new(4), new(E), new(E), new(E), new(4), new(E)]
+        srwm_hip.self_ref_forward(xd, *Wd, *f, flags=srwm_hip.FLAG_GENERIC)
+        gx, gW = new(E), [torch.empty_like(w) for w in Wd]
+        srwm_hip.self_ref_backward(xd, *f[:-1], god, *Wd, gx, *gW, flags=srwm_hip.FLAG_GENERIC)
+        (stream or torch.cuda.current_stream(dev)).synchronize()
+        return [f[-1].cpu(), gx.cpu(), gW[1].cpu()]
+
+    alone = {E: run(E, 7) for E in (12, 48)}
+    errors, mismatches = [], []
+
+    def worker(E):
+        try:
+            stream = torch.cuda.Stream(device=dev)
+            with torch.cuda.stream(stream):
+                for _ in range(25):
+                    got = run(E, 7, stream)
+                    if not all(torch.equal(a, b) for a, b in zip(got, alone[E])):
+                        mismatches.append(E)
+        except Exception as e:
+            errors.append((E, e))
+
+    threads = [threading.Thread(target=worker, args=(E,)) for E in (12, 48)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    assert not mismatches, mismatches
+
+
 def test_work_is_ordered_on_the_callers_stream():
     """Inputs are produced on a side stream right before the call and results consumed right
     after it, with no synchronisation in between: correct only if the kernels are enqueued on
