@@ -255,7 +255,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     auto publish = [&](int t, const float (&acc)[NC], float pb, float py) {
         const unsigned oy = t * Y;           // offsets inside the sequence (the launcher bounds L * Y)
         const int par = t & 1;
-        if (rg == 0) {
+        // the RG lanes of a column group hold identical values: all of them store, to the same words,
+        // which is cheaper than masking seven of them off (no branch around the stores)
+        {
             if (bf16_io) {
 #pragma unroll
                 for (int b = 0; b < YB; ++b)
@@ -384,11 +386,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             group_sum_n<E, NS>(s);
         }
         const float pbd = s[0], kx = s[1];
-        if (rg == 0) {
-            store_y(ydiff_s, oy, &dif[0]);
-            store_vec<CB>(at32(qdiff_s, o + (unsigned)c0), &dif[QB]);
-            store_vec<CB>(at32(kdiff_s, o + (unsigned)c0), &dif[KB]);
-        }
+        store_y(ydiff_s, oy, &dif[0]);   // by all RG lanes of the column group, like the readout
+        store_vec<CB>(at32(qdiff_s, o + (unsigned)c0), &dif[QB]);
+        store_vec<CB>(at32(kdiff_s, o + (unsigned)c0), &dif[KB]);
         if (has_b && el == 0) *at32(bdiff_s, ob + jb) = pbd;
         if constexpr (XC) {
             if (has_y && el == 0) *at32(ydiff_s, oy + YB * E) = s[3];
