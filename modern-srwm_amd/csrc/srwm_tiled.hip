@@ -468,10 +468,12 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 //   row sums     G ins, W_{t-1} g_diff, W_{t-1} g_pre (per lane R partial rows -> reduce-scatter
 //                over the wave's 8 column groups with v_permlane{32,16}_swap + one DPP step,
 //                then summed over the waves through LDS)
-// At E = 64, ONE workgroup barrier per step, after the first pair of row sums: the hand-over
-// buffers exist once per step parity, and the grad_x row sums of a step are added up behind the
-// barrier of the following step (the last ones after the loop), so they need no barrier of their
-// own.  The smaller sizes use a second barrier before those sums instead.
+// ONE workgroup barrier per step, after the first pair of row sums: the hand-over buffers exist once
+// per step parity, and the grad_x row sums of a step are added up behind the barrier of the
+// following step (the last ones after the loop), so they need no barrier of their own.  The step
+// loop is unrolled by two, so the parity is a compile-time constant.  Below E = 64 (one workgroup
+// per CU, one wave per SIMD, nothing to hide a latency behind) the operands of a step are read from
+// the tile one step ahead.
 // The seven per-step vectors and beta are streamed through a single LDS tile of TT steps;
 // the next tile is fetched into registers one tile ahead.
 template <int E, int NW, int R, int YB>
@@ -492,13 +494,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     __shared__ __attribute__((aligned(16))) float tyd[TT][YS];      // y_diff of the tile
     __shared__ __attribute__((aligned(16))) float tgo[TT][YS];      // grad_out of the tile
     __shared__ __attribute__((aligned(16))) float tb[2][TT][4];     // beta | beta_diff
-    // Cross-wave hand-over buffers.  ONEBAR (E = 64, where two workgroups share a CU and the step is
-    // bound by instruction issue): one set per step parity, so that a wave may start writing those of
-    // the next step while a slower wave still reads this step's, and one barrier per step.  The
-    // smaller sizes are bound by the latency of a single step; there the parity addressing costs
-    // more than the second barrier, which they keep.
-    constexpr bool ONEBAR = E == kWave;
-    constexpr int NPAR = ONEBAR ? 2 : 1;
+    // Cross-wave hand-over buffers, one set per step parity: a wave may start writing those of the next
+    // step while a slower wave still reads this step's, so ONE barrier per step suffices.  The step
+    // loop is unrolled by two, which makes the parity (and with it every buffer address) a
+    // compile-time constant.
+    constexpr int NPAR = 2;
     __shared__ __attribute__((aligned(16))) float rowm[NPAR][3][NW][E];   // row sums per wave: G ins | W gdiff | W gpre
     __shared__ __attribute__((aligned(16))) float rowb[NPAR][3][NXS][E];  // same, contribution of the narrow columns
     __shared__ __attribute__((aligned(16))) float gbp[NPAR][NCG][4];      // per column group: sum gins*diff per beta
@@ -637,37 +637,65 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     };
     float xb_prev = 0.f;
 
+    // operands of one step, read from the tile in LDS
+    constexpr bool PREF = E < kWave;   // fetch them one step ahead (one workgroup per CU: nothing else hides the LDS latency)
+    struct Ops {
+        float kr[R], qr[R], xr[R], dif[NC], goy[YB * CB], bt[4], bd, btj, kb, qb, xb, ydl, gprey;
+    };
+    auto load_ops = [&](const int tt, Ops &o) __attribute__((always_inline)) {
+        lds_read_vec<R>(o.kr, &tl[VK][tt][r0]);
+        lds_read_vec<R>(o.qr, &tl[VQ][tt][r0]);
+        lds_read_vec<R>(o.xr, &tl[VX][tt][r0]);
+#pragma unroll
+        for (int b = 0; b < YB; ++b) {
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&o.dif[b * CB]), &tyd[tt][b * E + c0]);
+            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&o.goy[b * CB]), &tgo[tt][b * E + c0]);
+        }
+        lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&o.dif[QB]), &tl[VQD][tt][c0]);
+        lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&o.dif[KB]), &tl[VKD][tt][c0]);
+        lds_read_vec<4>(o.bt, &tb[0][tt][0]);
+        o.bd = tb[1][tt][jb & 3];   // this thread's w_b column: beta_diff, beta
+        o.btj = tb[0][tt][jb & 3];
+        o.kb = tl[VK][tt][el];
+        o.qb = tl[VQ][tt][el];
+        o.xb = tl[VX][tt][el];
+        o.ydl = o.gprey = 0.f;
+        if constexpr (XC) {   // last y column: its diff and upstream gradient
+            o.ydl = tyd[tt][YB * E];
+            o.gprey = tgo[tt][YB * E];
+        }
+    };
+
     const int ntiles = (p.L + TT - 1) / TT;
     SRWM_BWD_LOAD_TILE(ntiles - 1);
     SRWM_BWD_STORE_TILE();
     __syncthreads();
 
+    static_assert(TT % 2 == 0, "the parity of a step inside its tile is the parity of the step");
     for (int tile = ntiles - 1; tile >= 0; --tile) {
         const int tlen = min(TT, p.L - tile * TT);
         if (tile > 0) SRWM_BWD_LOAD_TILE(tile - 1);
 
-        for (int tt = tlen - 1; tt >= 0; --tt) {
-            const int t = tile * TT + tt, par = ONEBAR ? (t & 1) : 0;
+        // One step.  PAR: its parity (a type carrying a constant).  cur: its operands; below E = 64 they
+        // were fetched from the tile during the step before (PREF), and this step fetches those of
+        // step tt - 1 into nxt once it is past its barrier.
+        auto step = [&](auto PAR, const int tt, Ops &cur, Ops &nxt) __attribute__((always_inline)) {
+            constexpr int par = decltype(PAR)::value;
+            const int t = tile * TT + tt;
 
-            // ---- operands of the step
-            float kr[R], dvr[R], xr[R];
-            lds_read_vec<R>(kr, &tl[VK][tt][r0]);
-            lds_read_vec<R>(dvr, &tl[VQ][tt][r0]);
-            lds_read_vec<R>(xr, &tl[VX][tt][r0]);
+            const Ops &o = cur;
+            if constexpr (!PREF) load_ops(tt, cur);
+            const float(&kr)[R] = o.kr, (&xr)[R] = o.xr;
+            float dvr[R];
 #pragma unroll
-            for (int i = 0; i < R; ++i) dvr[i] -= kr[i];
+            for (int i = 0; i < R; ++i) dvr[i] = o.qr[i] - o.kr[i];
             float dif[NC], gpre[NC];
 #pragma unroll
-            for (int b = 0; b < YB; ++b) {
-                lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[b * CB]), &tyd[tt][b * E + c0]);
-                lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&gpre[b * CB]), &tgo[tt][b * E + c0]);
-            }
-            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[QB]), &tl[VQD][tt][c0]);
-            lds_read_vec<CB>(*reinterpret_cast<float(*)[CB]>(&dif[KB]), &tl[VKD][tt][c0]);
-            float bt[4];
-            lds_read_vec<4>(bt, &tb[0][tt][0]);
-            const float bd = tb[1][tt][jb & 3], btj = tb[0][tt][jb & 3];   // this thread's w_b column: beta_diff, beta
-            const float kb = tl[VK][tt][el], qb = tl[VQ][tt][el], xb = tl[VX][tt][el];
+            for (int c = 0; c < NC; ++c) dif[c] = o.dif[c];
+#pragma unroll
+            for (int c = 0; c < QB; ++c) gpre[c] = o.goy[c];
+            const float(&bt)[4] = o.bt;
+            const float bd = o.bd, btj = o.btj, kb = o.kb, qb = o.qb, xb = o.xb;
             const float dvb = qb - kb;
 
             // ---- revert the write: W_{t-1} = W_t - k (x) ins
@@ -683,8 +711,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             wbe = fmaf(-kb, insb, wbe);
             float ydl = 0.f, insy = 0.f, gprey = 0.f;   // last y column: its diff, insert and upstream gradient
             if constexpr (XC) {
-                ydl = tyd[tt][YB * E];
-                gprey = tgo[tt][YB * E];
+                ydl = o.ydl;
+                gprey = o.gprey;
                 insy = bt[0] * ydl;
                 wye = fmaf(-kb, insy, wye);
             }
@@ -750,6 +778,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             }
             if (rg == 0) *reinterpret_cast<float4 *>(&gbp[par][cg][0]) = make_float4(pg[0], pg[1], pg[2], 0.f);
             __syncthreads();
+            if constexpr (PREF) {
+                if (tt > 0) load_ops(tt - 1, nxt);   // uniform; the tile's rows are only rewritten after its last step
+            }
 
             // ---- every wave, lane <-> element el: gradients of q, k, beta before activation
             float gk, gq;
@@ -838,14 +869,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             if constexpr (XC) {
                 if (has_y) rowb[par][2][4][el] = wye * gprey;
             }
-            if constexpr (ONEBAR) {
-                // the grad_x partials are summed one step later, behind the next step's barrier: no barrier of their own
-                if (t + 1 < p.L) finish_gx(t + 1, par ^ 1, xb_prev);
-                xb_prev = xb;
-            } else {
-                __syncthreads();
-                finish_gx(t, 0, xb);
-            }
+            // the grad_x partials are summed one step later, behind the next step's barrier: no barrier of their own
+            if (t + 1 < p.L) finish_gx(t + 1, par ^ 1, xb_prev);
+            xb_prev = xb;
 
             // ---- G_{t-1} = G_t + (q - k) (x) g_diff + x (x) g_pre
 #pragma unroll
@@ -856,19 +882,34 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             gbe = fmaf(dvb, gdifb, fmaf(xb, gpreb, gbe));
             if constexpr (XC) gye = fmaf(dvb, gdify, fmaf(xb, gprey, gye));
 
-            if (tt == 0 && tile > 0) {
-                // every wave is past its last read of this tile (all reads precede the
-                // first barrier of the step)
-                SRWM_BWD_STORE_TILE();
-                __syncthreads();
-            }
+        };
+        // full tiles hold an even number of steps, so they are pairs of an odd and an even step; a ragged
+        // tile of odd length starts with one even step on its own
+        using P0 = std::integral_constant<int, 0>;
+        using P1 = std::integral_constant<int, 1>;
+        Ops A, B;
+        int tt = tlen - 1;
+        if (tt & 1) {
+            if constexpr (PREF) load_ops(tt, A);
+        } else {
+            if constexpr (PREF) load_ops(tt, B);
+            step(P0{}, tt, B, A);
+            --tt;
+        }
+        for (; tt >= 1; tt -= 2) {
+            step(P1{}, tt, A, B);
+            step(P0{}, tt - 1, B, A);
+        }
+        if (tile > 0) {
+            // every wave is past its last read of this tile (all reads precede the barrier of the
+            // step, and the last step fetches nothing ahead)
+            SRWM_BWD_STORE_TILE();
+            __syncthreads();
         }
     }
 
-    if constexpr (ONEBAR) {
-        __syncthreads();
-        finish_gx(0, 0, xb_prev);
-    }
+    __syncthreads();
+    finish_gx(0, 0, xb_prev);
 
     {
         const bool accum = p.grad_state_mode == 2u;
