@@ -204,6 +204,32 @@ def test_bf16_io_matches_oracle_on_rounded_inputs(shape, qk):
     assert W.abs().max().item() < 1e-4 * max(1.0, float(np.abs(of["W"]).max()))   # reverted to W_0 = 0
 
 
+def test_two_workgroups_per_sequence_with_a_ragged_sequence_count():
+    """D = 128 with few sequences runs two workgroups per sequence, placed 8 workgroups apart in full
+    groups of 8 sequences and plainly for the rest: 10 sequences exercise both numberings at once, in
+    the step-by-step and in the chunkwise kernels (fp32 inputs, 1e-5 bar)."""
+    print("case D=128, 10 sequences", flush=True)
+    import srwm_hip
+    dev = _dev()
+    N, H, L, D = 2, 5, 70, 128
+    q, k, v, beta, W0, go = delta_inputs(N, H, L, D, D, seed=29, qk="l2", w0_std=0.2)
+    base = [t.numpy() for t in (q, k, v, beta, W0)]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, go.numpy(), want_grad_W=True)
+    qd, kd, vd, bd, god = (t.to(dev, torch.float32) for t in (q, k, v, beta, go))
+    nan = lambda *s_: torch.full(s_, float("nan"), device=dev)
+    for flags in (0, srwm_hip.FLAG_CHUNKWISE):
+        W = W0.to(dev, torch.float32).contiguous()
+        vold, vins, out = nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, D)
+        srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out, flags=flags)
+        assert rel_err(out.cpu().numpy(), of["out"]) < TOL and rel_err(W.cpu().numpy(), of["W"]) < TOL
+        assert rel_err(vins.cpu().numpy(), of["v_insert"]) < TOL
+        gq, gk, gv, gb, gW = nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, 1), nan(N, H, D, D)
+        srwm_hip.fast_weight_backward(qd, kd, vd, bd, vold, vins, god, W, gq, gk, gv, gb, grad_kv=gW, flags=flags)
+        for n, t in (("grad_Q", gq), ("grad_K", gk), ("grad_V", gv), ("grad_beta", gb), ("grad_W", gW)):
+            assert rel_err(t.cpu().numpy(), ob[n]) < TOL, (flags, n)
+
+
 # ------------------------------------------------------------------ chunkwise MFMA forward
 
 @pytest.mark.parametrize("shape,qk,w0,io", [
