@@ -83,6 +83,19 @@ __device__ __forceinline__ T *at32(T *base, unsigned idx) {
     return reinterpret_cast<T *>(reinterpret_cast<char *>(base) + idx * (unsigned)sizeof(T));
 }
 
+// A step parity is handed around either as a run-time int or as a std::integral_constant, in which
+// case everything derived from it (buffer addresses) folds to constants.
+template <class P>
+__device__ __forceinline__ constexpr int parity_of(P p) {
+    if constexpr (std::is_integral_v<P>) return p;
+    else return P::value;
+}
+template <class P>
+__device__ __forceinline__ constexpr auto parity_flipped(P p) {
+    if constexpr (std::is_integral_v<P>) return 1 - p;
+    else return std::integral_constant<int, 1 - P::value>{};
+}
+
 // Softmax over a row of E floats that E/4 consecutive lanes hold as one float4 each.
 template <int E>
 __device__ __forceinline__ float4 row_softmax4(float4 v) {
@@ -104,6 +117,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     constexpr bool MODES = XTRA >= 1;   // p.mode: work outside the step loop only (entry / exit form of the state, input tiles)
     constexpr bool RESET = XTRA >= 2;   // p.keep: a check, and now and then a reset, inside every step
     using T = Tiling<E, NW, R>;
+    using P0 = std::integral_constant<int, 0>;
+    using P1 = std::integral_constant<int, 1>;
     constexpr int RG = T::RG, CGW = T::CGW, CB = T::CB, TT = T::TT;
     constexpr int NB = YB + 2, NC = NB * CB;          // blocks of E columns: y (YB of them) | q | k
     constexpr bool XC = YB > 1;                       // one more y column, held like a column of w_b
@@ -122,6 +137,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     const int el = lane % E;                 // softmax element == row of this thread's w_b entry
     const int jb = tid / E;                  // column of this thread's w_b entry
     const bool has_b = jb < 4;
+    // who stores what inside a step (lane masks that stay in scalar registers across the loop)
+    const bool st_qk = wave == 0 && lane < E, st_beta = wave == NW - 1 && lane < 4, st_exch = lane < E;
 
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
@@ -252,9 +269,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         }
     };
     // hands the readout of step t to the output and, through LDS, to the activations of that step
-    auto publish = [&](int t, const float (&acc)[NC], float pb, float py) {
+    auto publish = [&](auto PARP, int t, const float (&acc)[NC], float pb, float py) __attribute__((always_inline)) {
         const unsigned oy = t * Y;           // offsets inside the sequence (the launcher bounds L * Y)
-        const int par = t & 1;
+        const int par = parity_of(PARP);   // parity of step t
         // the RG lanes of a column group hold identical values: all of them store, to the same words,
         // which is cheaper than masking seven of them off (no branch around the stores)
         {
@@ -291,12 +308,16 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         float xr[R], acc[NC], pb, py = 0.f;
         lds_read_vec<R>(xr, &xt[0][0][r0]);
         readout(xr, xt[0][0][el], acc, pb, py);
-        publish(0, acc, pb, py);
+        publish(P0{}, 0, acc, pb, py);
     }
     __syncthreads();
 
-    for (int t = 0; t < p.L; ++t) {
-        const int par = t & 1, t1 = t + 1;
+    // (below E = 64 the loop is unrolled by two, which makes the parity of a step -- it selects the
+    // hand-over buffers -- a compile-time constant; at E = 64 the rolled loop is the faster one)
+    auto step = [&](auto PAR, const int t) __attribute__((always_inline)) {
+        const int par = parity_of(PAR);
+        const auto PNEXT = parity_flipped(PAR);
+        const int t1 = t + 1;
         const unsigned o = t * E, oy = t * Y, ob = t * 4;   // unsigned: uniform base + 32-bit lane offset addressing
         const int b1 = (t1 / TT) & 1, r1 = t1 % TT;   // where x of step t+1 sits (stale rows past the end: never published)
         const bool have_next = t1 < p.L;
@@ -339,12 +360,12 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         const float bt[4] = {quad_broadcast<0>(sg), quad_broadcast<1>(sg), quad_broadcast<2>(sg),
                              quad_broadcast<3>(sg)};
         const float dv = qn - kn;
-        if (wave == 0 && lane < E) {
+        if (st_qk) {
             *at32(q_s, o + lane) = qn;
             *at32(k_s, o + lane) = kn;
         }
-        if (wave == NW - 1 && lane < 4) *at32(beta_s, ob + lane) = sg;
-        if (lane < E) {
+        if (st_beta) *at32(beta_s, ob + lane) = sg;
+        if (st_exch) {
             exch[wave][0][lane] = dv;
             exch[wave][1][lane] = kn;
         }
@@ -416,7 +437,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             for (int c = 0; c < NC; ++c) e[c] = fmaf(ins[c], kx, e[c]);
             float py = 0.f;
             if constexpr (XC) py = fmaf(insy, kx, s[4]);
-            if (have_next) publish(t1, e, fmaf(insb, kx, s[2]), py);
+            if (have_next) publish(PNEXT, t1, e, fmaf(insb, kx, s[2]), py);
             write_state();
         }
         if constexpr (RESET) {
@@ -424,7 +445,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
                 reset_state();
                 float acc[NC], pb, py = 0.f;
                 readout(xr, xb, acc, pb, py);
-                publish(t1, acc, pb, py);
+                publish(PNEXT, t1, acc, pb, py);
             }
         }
 
@@ -438,6 +459,16 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             }
         }
         __syncthreads();
+    };
+    if constexpr (E == kWave) {
+        for (int t = 0; t < p.L; ++t) step(t & 1, t);
+    } else {
+        int t = 0;
+        for (; t + 1 < p.L; t += 2) {
+            step(P0{}, t);
+            step(P1{}, t + 1);
+        }
+        if (t < p.L) step(P0{}, t);
     }
 
     // the final state, as the shift from the shared weights if that is how the caller keeps it
