@@ -42,11 +42,13 @@ HBM_PEAK_GBS = 8000.0
 # makes a plain copy of known size read its size).  A profiler cannot run inside this script, so the
 # figure is carried here with the summary file that holds the runs' commands and counters.
 MEASURED_TRAFFIC = {
-    "srwm_c4": ((490413 + 90624) * 1024, "profiles/srwm_c4_kernels.txt"),
-    "delta_c2": ((102444 + 53504) * 1024, "profiles/delta_kernels.txt"),
-    "delta_c2_chunk": ((82217 + 85992 + 16640 + 36864) * 1024, "profiles/delta_chunk_kernels.txt"),
-    "delta_c5": ((1316522 + 1323008) * 1024, "profiles/delta_kernels.txt"),
-    "delta_c5_chunk": ((1047391 + 1575757 + 267264 + 532480) * 1024, "profiles/delta_chunk_kernels.txt"),
+    "srwm_c4": ((490453 + 90624) * 1024, "profiles/srwm_c4_kernels.txt"),
+    "srwm_c3": ((26515 + 6400) * 1024, "profiles/srwm_c3_kernels.txt"),
+    "srwm_wide_c3": ((41761 + 8480) * 1024, "profiles/srwm_c3_kernels.txt"),
+    "delta_c2": ((102515 + 53504) * 1024, "profiles/delta_kernels.txt"),
+    "delta_c2_chunk": ((82185 + 85890 + 16640 + 36864) * 1024, "profiles/delta_chunk_kernels.txt"),
+    "delta_c5": ((1054057 + 1323008) * 1024, "profiles/delta_kernels.txt"),
+    "delta_c5_chunk": ((784928 + 922433 + 267264 + 532480) * 1024, "profiles/delta_chunk_kernels.txt"),
 }
 
 WORKLOADS = {
