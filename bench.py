@@ -132,6 +132,7 @@ def srwm_steps_setup(N, H, L, E, dev):
     t["slow"] = [w[0].contiguous() for w in t["W0"]]
     t["Wy_entry"] = torch.empty_like(t["W0"][0])
     t["gWy"] = torch.empty(H, E, E, device=dev)
+    t["gWy_rows"] = torch.empty(N, H, E, E, device=dev)
     return t
 
 
@@ -147,8 +148,8 @@ def srwm_steps_step(t, ev=None):
     if ev:
         ev[1].record()
     sv = t["saved"]
-    srwm_hip.self_ref_readout_grad(sv[1], sv[2], sv[3], t["keep"], t["slow"][0], t["go"], t["Wy_entry"], t["gx"])
-    t["gWy"].copy_(torch.einsum("nhle,nhlm->hem", t["x"], t["go"]))
+    srwm_hip.self_ref_layer_readout_grad(t["x"], sv[1], sv[2], sv[3], t["keep"], t["slow"][0], t["go"], t["Wy_entry"],
+                                         t["gx"], t["gWy_rows"], t["gWy"])
     if ev:
         ev[2].record()
 

@@ -297,6 +297,28 @@ SRWM_API int srwm_readout_grad_wide_f32(const float *k, const float *beta, const
                                int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
 /*
+ * The whole backward of an RL unroll for a layer, in one call: srwm_readout_grad_wide_f32 plus the
+ * gradient of the shared W_y.  No counterpart function in the reference, whose learner calls the
+ * operator's backward once per time step and lets autograd add up the weight gradients
+ * (reinforcement_learning/torchbeast/layer.py:377-421, torchbeast_procgen/model.py:1176-1196).
+ *   x          strided [N,H,L,E]: the operator's input of the forward call (after its softmax where
+ *              the layer soft-maxes it)
+ *   W_y_entry  dense [N,H,E,Y]: the y block before the forward call; with SRWM_FLAG_STATE_SHIFT as the
+ *              difference from sW_y, the form in which the layers carry their state
+ *   sW_y       dense [H,E,Y], required
+ *   grad_x     dense [N,H,L,E]: W_y,t-1 grad_out_t (gradient with respect to x as given here)
+ *   gW_y       dense [N,H,E,Y]: per batch row, sum over t of x_t (x) grad_out_t
+ *   gsW_y      dense [H,E,Y]: its sum over the batch in a fixed order = the gradient of the shared W_y
+ * flags: SRWM_FLAG_GENERIC, SRWM_FLAG_STATE_SHIFT.
+ */
+SRWM_API int srwm_layer_readout_grad_f32(const float *x, const int64_t x_strides[3],
+                                const float *k, const float *beta, const float *y_diff,
+                                const float *keep, const float *sW_y,
+                                const float *grad_out, const int64_t grad_out_strides[3],
+                                const float *W_y_entry, float *grad_x, float *gW_y, float *gsW_y,
+                                int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+
+/*
  * Delta-rule forward.  Replaces fast_weight_forward(), supervised_learning/
  * fast_weight/fast_weight_cuda.cu:182-240 (kernel :17-178).  Per sequence, W is E x M:
  *     v_old = W^T k_t;  ins = beta_t (v_t - v_old);  W += k_t (x) ins;  out_t = W^T q_t
@@ -403,7 +425,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any signature change); currently 5. */
+/* ABI version of this header (bumped on any signature change); currently 6. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

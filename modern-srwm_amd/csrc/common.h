@@ -69,6 +69,12 @@ struct ReplayParams {
     const float *Wreset;   // dense [H,E,M] or nullptr (reset to zero)
     float *u;              // dense [N,H,L,E]
     int N, H, L, E, M;
+    // optional: per sequence, xg = sum over t of x_t (x) g_t (the gradient a matrix read as
+    // out_t = W^T x_t receives when nothing flows back through the recurrence)
+    const float *x;        // [N,H,L,E], strided, or nullptr
+    Strided3 xs;
+    float *xg;             // dense [N,H,E,M]
+    int w0_is_shift;       // W0 holds W - Wreset (Wreset must be given)
 };
 
 struct DeltaFwdParams {
@@ -174,6 +180,7 @@ int launch_replay_tiled(const ReplayParams &p, hipStream_t s);   // -1: no regis
 int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s);
 // dst[j][h, :] = sum over n of src[j][n, h, :] for the four state tensors (y: E x Y, q, k: E x E, b: E x 4)
 int launch_srwm_batch_sum(const float *const src[4], float *const dst[4], int N, int H, int E, int Y, hipStream_t s);
+int launch_batch_sum(const float *src, float *dst, int N, int64_t len, hipStream_t s);   // dst[i] = sum_n src[n][i]
 int launch_delta_fwd_generic(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_bwd_generic(const DeltaBwdParams &p, hipStream_t s);
 

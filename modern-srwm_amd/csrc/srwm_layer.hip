@@ -14,13 +14,23 @@ struct BatchSumParams {
     int N;
 };
 
-__global__ __launch_bounds__(256) void batch_sum_kernel(BatchSumParams p) {
+constexpr int kSumThreads = 64;   // small workgroups: the sums are short, so spread them over many CUs
+
+__global__ __launch_bounds__(kSumThreads) void batch_sum_kernel(BatchSumParams p) {
     const int j = blockIdx.y;
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x, len = p.len[j];
+    const int64_t i = (int64_t)blockIdx.x * kSumThreads + threadIdx.x, len = p.len[j];
     if (i >= len) return;
     const float *s = p.src[j] + i;
     float a = 0.f;   // fixed order over n: the result does not depend on scheduling
-    for (int n = 0; n < p.N; ++n) a += s[(int64_t)n * len];
+    int n = 0;
+    for (; n + 8 <= p.N; n += 8) {   // eight loads in flight, added in order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = s[(int64_t)(n + u) * len];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) a += v[u];
+    }
+    for (; n < p.N; ++n) a += s[(int64_t)n * len];
     p.dst[j][i] = a;
 }
 
@@ -38,7 +48,17 @@ int launch_srwm_batch_sum(const float *const src[4], float *const dst[4], int N,
         mx = p.len[j] > mx ? p.len[j] : mx;
     }
     p.N = N;
-    hipLaunchKernelGGL(batch_sum_kernel, dim3((unsigned)((mx + 255) / 256), 4), dim3(256), 0, s, p);
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((unsigned)((mx + kSumThreads - 1) / kSumThreads), 4), dim3(kSumThreads), 0, s, p);
+    return (int)hipGetLastError();
+}
+
+int launch_batch_sum(const float *src, float *dst, int N, int64_t len, hipStream_t s) {
+    BatchSumParams p{};
+    p.src[0] = src;
+    p.dst[0] = dst;
+    p.len[0] = len;
+    p.N = N;
+    hipLaunchKernelGGL(batch_sum_kernel, dim3((unsigned)((len + kSumThreads - 1) / kSumThreads), 1), dim3(kSumThreads), 0, s, p);
     return (int)hipGetLastError();
 }
 

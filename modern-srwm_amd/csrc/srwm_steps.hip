@@ -41,7 +41,8 @@ __global__ __launch_bounds__(kThreads) void replay_kernel(ReplayParams p) {
     const float *ab = p.a + n * p.as.n + h * p.as.h;
     const float *gb = p.g + n * p.gs.n + h * p.gs.h;
 
-    for (int i = tid; i < E * M; i += kThreads) W[(i / M) * Mp + i % M] = p.W0[seq * E * M + i];
+    for (int i = tid; i < E * M; i += kThreads)
+        W[(i / M) * Mp + i % M] = p.W0[seq * E * M + i] + (p.w0_is_shift ? p.Wreset[(int64_t)h * E * M + i] : 0.f);
 
     // thread e < E holds a[e], thread m < M holds b[m], g[m] of the next step (E, M <= 256)
     float na = 0.f, nb = 0.f, ng = 0.f, ns = 1.f, nkeep = 1.f;
@@ -85,27 +86,47 @@ __global__ __launch_bounds__(kThreads) void replay_kernel(ReplayParams p) {
     }
 }
 
+// xg[seq] = sum_t x_t (x) g_t for the sizes the register-resident kernel does not cover: a thread
+// owns elements of the E x M result and walks the steps (the vectors come from cache).
+__global__ __launch_bounds__(kThreads) void outer_sum_kernel(ReplayParams p) {
+    const int E = p.E, M = p.M;
+    const int64_t seq = blockIdx.x;
+    const int n = (int)(seq / p.H), h = (int)(seq % p.H);
+    const float *xb = p.x + n * p.xs.n + h * p.xs.h;
+    const float *gb = p.g + n * p.gs.n + h * p.gs.h;
+    for (int i = threadIdx.x; i < E * M; i += kThreads) {
+        const int e = i / M, m = i - e * M;
+        float acc = 0.f;
+        for (int t = 0; t < p.L; ++t) acc = fmaf(xb[t * p.xs.l + e], gb[t * p.gs.l + m], acc);
+        p.xg[seq * E * M + i] = acc;
+    }
+}
+
 // Register-resident replay.  NWV waves per sequence; wave w owns rows [w*ER, (w+1)*ER), ER = E/NWV.
 // Inside a wave, CGL consecutive lanes share a block of R rows and split its columns (CB each).
 // M need not be a multiple of CGL or of 4 (the wide output block of the SRWM has M = 3E+1): the
 // lanes then tile MP = M rounded up to a multiple of CGL columns, the surplus columns are zero
 // throughout, and the rows of g and b -- no longer 16-byte aligned -- are fetched word by word.
+// XG: also accumulate sum_t x_t (x) g_t in a second register tile of the same shape (the lanes
+// already hold g_t's columns; the wave's rows of x_t ride in a tile like a_t's).
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <int E, int M, int NWV, int CGL>
+template <int E, int M, int NWV, int CGL, bool XG>
 __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p) {
     constexpr int MP = (M + CGL - 1) / CGL * CGL;
     constexpr bool WORDS = MP != M || M % 4 != 0;   // rows of g, b fetched word by word
     constexpr int ER = E / NWV, RGL = kWave / CGL, R = ER / RGL, CB = MP / CGL;
     constexpr int TT = M > 64 ? 8 : (256 / ER > 16 ? 256 / ER : 16);   // steps per tile
-    constexpr int NG = WORDS ? 1 : TT * M / 4 / kWave, NA = TT * ER / 4 / kWave;   // float4 per lane per tile
+    constexpr int NG = WORDS ? 1 : TT * M / 4 / kWave;                             // float4 per lane per tile
+    constexpr int NAV = TT * ER / 4, NA = (NAV + kWave - 1) / kWave;               // the same for a_t (NAV in all)
     constexpr int NWL = WORDS ? (TT * M + kWave - 1) / kWave : 1;                  // words per lane per tile
     static_assert(ER * NWV == E && R * RGL == ER && CB * CGL == MP && R >= 1 && CB >= 1, "tiling");
-    static_assert((WORDS || NG * 4 * kWave == TT * M) && NA * 4 * kWave == TT * ER && TT <= kWave, "tile loader");
+    static_assert((WORDS || NG * 4 * kWave == TT * M) && ER % 4 == 0 && TT <= kWave, "tile loader");
     static_assert(CGL <= 16, "row sums must stay inside a DPP row");
     __shared__ __attribute__((aligned(16))) float tg[NWV][TT][MP];   // g_t
     __shared__ __attribute__((aligned(16))) float tb[NWV][TT][MP];   // b_t
     __shared__ __attribute__((aligned(16))) float ta[NWV][TT][ER];   // this wave's rows of a_t
+    __shared__ __attribute__((aligned(16))) float tx[XG ? NWV : 1][XG ? TT : 1][ER];   // and of x_t
     __shared__ float tsk[NWV][2][TT];                                // s_t | keep_t
 
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -116,6 +137,7 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
     const float *ab = p.a + n * p.as.n + h * p.as.h + e0;
     const float *gb = p.g + n * p.gs.n + h * p.gs.h;
     const float *bb = p.b + seq * p.L * M;
+    const float *xb = XG ? p.x + n * p.xs.n + h * p.xs.h + e0 : nullptr;
 
     if constexpr (MP != M) {   // the surplus columns of the tiles stay zero: commits only write m < M
         for (int i = lane; i < TT * (MP - M); i += kWave) {
@@ -134,11 +156,57 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
     };
     load_w(p.W0 + seq * E * M);
     const float *wreset = p.Wreset ? p.Wreset + (int64_t)h * E * M : nullptr;
+    // The reset value stays in registers where they suffice: fetching it inside the step loop puts a
+    // wait for ALL outstanding memory operations -- the stores of u included -- into every step.
+    constexpr bool WR_REGS = R * CB * (XG ? 3 : 2) <= 200;
+    float wr[WR_REGS ? R : 1][WR_REGS ? CB : 1];
+    if constexpr (WR_REGS) {
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int c = 0; c < CB; ++c)
+                wr[i][c] = (wreset && (MP == M || c0 + c < M)) ? wreset[(e0 + r0 + i) * M + c0 + c] : 0.f;
+    }
+    if (p.w0_is_shift) {
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int c = 0; c < CB; ++c) {
+                if constexpr (WR_REGS) w[i][c] += wr[i][c];
+                else if (MP == M || c0 + c < M) w[i][c] += wreset[(e0 + r0 + i) * M + c0 + c];
+            }
+    }
+    float xg[XG ? R : 1][XG ? CB : 1];
+    if constexpr (XG) {
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int c = 0; c < CB; ++c) xg[i][c] = 0.f;
+    }
+
+    constexpr bool PREF = CB <= 16;   // wider lane tiles have no registers to spare for a second set of operands
+    struct StepOps {
+        float gv[CB], bv[CB], av[R], xv[XG ? R : 1], sc, keep;
+    };
+    const auto read_ops = [&](const int tt, StepOps &o) __attribute__((always_inline)) {
+#pragma unroll
+        for (int c = 0; c < CB; ++c) {
+            o.gv[c] = tg[wave][tt][c0 + c];
+            o.bv[c] = tb[wave][tt][c0 + c];
+        }
+#pragma unroll
+        for (int i = 0; i < R; ++i) {
+            o.av[i] = ta[wave][tt][r0 + i];
+            if constexpr (XG) o.xv[i] = tx[wave][tt][r0 + i];
+        }
+        o.sc = tsk[wave][0][tt];
+        o.keep = tsk[wave][1][tt];
+    };
 
     // Next tile, staged in registers; rows past the end are clamped (loaded, never used).  The loop
     // starts one tile early so that fetch and commit each appear once in the code: with two call
     // sites the staging arrays end up in scratch memory instead of registers.
-    v4f ng[NG], nb[NG], na[NA];   // native vectors: arrays of HIP float4 structs are not kept in registers here
+    v4f ng[NG], nb[NG], na[NA], nx[XG ? NA : 1];   // native vectors: arrays of HIP float4 structs are not kept in registers here
     float ngw[NWL], nbw[NWL];
     float ns = 1.f, nk = 1.f;
     const int ntiles = (p.L + TT - 1) / TT;
@@ -165,9 +233,10 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
             }
 #pragma unroll
             for (int i = 0; i < NA; ++i) {
-                const int f = lane + i * kWave, row = f / (ER / 4), col = (f % (ER / 4)) * 4;
+                const int f = min(lane + i * kWave, NAV - 1), row = f / (ER / 4), col = (f % (ER / 4)) * 4;
                 const int64_t t = min(tb0 + row, p.L - 1);
                 na[i] = *reinterpret_cast<const v4f *>(ab + t * p.as.l + col);
+                if constexpr (XG) nx[i] = *reinterpret_cast<const v4f *>(xb + t * p.xs.l + col);
             }
             if (lane < TT) {
                 const int64_t t = min(tb0 + lane, p.L - 1);
@@ -176,25 +245,31 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
             }
         }
         const int tlen = tile < 0 ? 0 : min(TT, p.L - tile * TT);
-        for (int tt = 0; tt < tlen; ++tt) {
-            const int t = tile * TT + tt;
-            if (tsk[wave][1][tt] == 0.f) load_w(wreset);   // uniform over the wave
-            float gv[CB], bv[CB], av[R];
-#pragma unroll
-            for (int c = 0; c < CB; ++c) {
-                gv[c] = tg[wave][tt][c0 + c];
-                bv[c] = tb[wave][tt][c0 + c];
+        // One step with the operands in `cur`; those of the next step are read from the tile into `nxt`
+        // first, so that their LDS latency passes under this step's arithmetic (a wave has nobody to
+        // hide it behind: the waves of a sequence never meet, and there is one workgroup per CU).
+        const auto step = [&](const int tt, const StepOps &cur, StepOps &nxt) __attribute__((always_inline)) {
+            if constexpr (PREF) {
+                if (tt + 1 < tlen) read_ops(tt + 1, nxt);
             }
+            const int t = tile * TT + tt;
+            if (cur.keep == 0.f) {   // uniform over the wave
+                if constexpr (WR_REGS) {
 #pragma unroll
-            for (int i = 0; i < R; ++i) av[i] = ta[wave][tt][r0 + i];
-            const float sc = tsk[wave][0][tt];
+                    for (int i = 0; i < R; ++i)
+#pragma unroll
+                        for (int c = 0; c < CB; ++c) w[i][c] = wr[i][c];
+                } else {
+                    load_w(wreset);
+                }
+            }
             // u = W g: the lane's R partial row sums, completed over the CGL lanes of the row block
             float u[R];
 #pragma unroll
             for (int i = 0; i < R; ++i) {
                 u[i] = 0.f;
 #pragma unroll
-                for (int c = 0; c < CB; ++c) u[i] = fmaf(w[i][c], gv[c], u[i]);
+                for (int c = 0; c < CB; ++c) u[i] = fmaf(w[i][c], cur.gv[c], u[i]);
             }
             group_sum_n<CGL, R>(u);
             if (cgl == 0) {
@@ -202,13 +277,33 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
 #pragma unroll
                 for (int i = 0; i < R; ++i) dst[i] = u[i];
             }
-            // the step's write
+            if constexpr (XG) {
 #pragma unroll
-            for (int c = 0; c < CB; ++c) bv[c] *= sc;
+                for (int i = 0; i < R; ++i)
+#pragma unroll
+                    for (int c = 0; c < CB; ++c) xg[i][c] = fmaf(cur.xv[i], cur.gv[c], xg[i][c]);
+            }
+            // the step's write
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
-                for (int c = 0; c < CB; ++c) w[i][c] = fmaf(av[i], bv[c], w[i][c]);
+                for (int c = 0; c < CB; ++c) w[i][c] = fmaf(cur.av[i], cur.sc * cur.bv[c], w[i][c]);
+        };
+        if constexpr (PREF) {
+            StepOps A, B;   // the two take turns, so that no operand is copied between steps
+            if (tlen > 0) read_ops(0, A);
+            int tt = 0;
+            for (; tt + 2 <= tlen; tt += 2) {
+                step(tt, A, B);
+                step(tt + 1, B, A);
+            }
+            if (tt < tlen) step(tt, A, B);
+        } else {
+            StepOps A;
+            for (int tt = 0; tt < tlen; ++tt) {
+                read_ops(tt, A);
+                step(tt, A, A);
+            }
         }
         if (more) {   // commit tile + 1
             wave_lds_fence();   // this wave's reads of the current tile are done
@@ -232,7 +327,9 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
 #pragma unroll
             for (int i = 0; i < NA; ++i) {
                 const int f = lane + i * kWave, row = f / (ER / 4), col = (f % (ER / 4)) * 4;
+                if (NAV % kWave != 0 && f >= NAV) continue;
                 *reinterpret_cast<v4f *>(&ta[wave][row][col]) = na[i];
+                if constexpr (XG) *reinterpret_cast<v4f *>(&tx[wave][row][col]) = nx[i];
             }
             if (lane < TT) {
                 tsk[wave][0][lane] = ns;
@@ -241,18 +338,28 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
             wave_lds_fence();
         }
     }
+    if constexpr (XG) {
+        float *dst = p.xg + seq * E * M;
+#pragma unroll
+        for (int i = 0; i < R; ++i)
+#pragma unroll
+            for (int c = 0; c < CB; ++c)
+                if (MP == M || c0 + c < M) dst[(e0 + r0 + i) * M + c0 + c] = xg[i][c];
+    }
 }
 
 template <int E, int M, int NWV, int CGL>
 int launch_replay_tiled_as(const ReplayParams &p, hipStream_t s) {
-    hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
+    if (p.xg)
+        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, true>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
+    else
+        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, false>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
 template <int E, int NWV, int CGL>
 int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
-    hipLaunchKernelGGL((replay_tiled_kernel<E, E, NWV, CGL>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
-    return (int)hipGetLastError();
+    return launch_replay_tiled_as<E, E, NWV, CGL>(p, s);
 }
 
 bool rows16(const void *ptr, const Strided3 &st) {
@@ -264,11 +371,11 @@ bool rows16(const void *ptr, const Strided3 &st) {
 // Register-resident replay for square matrices with aligned rows and for E x (3E+1) ones (rows of
 // g and b at any alignment); -1 when there is no instantiation.
 int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
-    if (!rows16(p.a, p.as)) return -1;
+    if (!rows16(p.a, p.as) || (p.xg && !rows16(p.x, p.xs))) return -1;
     if (p.M == 3 * p.E + 1) {
         switch (p.E) {
             case 64: return launch_replay_tiled_as<64, 193, 2, 8>(p, s);
-            case 32: return launch_replay_tiled_as<32, 97, 1, 8>(p, s);
+            case 32: return launch_replay_tiled_as<32, 97, 4, 8>(p, s);
             case 16: return launch_replay_tiled_as<16, 49, 1, 8>(p, s);
             case 8: return launch_replay_tiled_as<8, 25, 1, 8>(p, s);
             default: return -1;
@@ -277,8 +384,8 @@ int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
     if (p.E != p.M || !rows16(p.g, p.gs) || (uintptr_t)p.b % 16 || (uintptr_t)p.u % 16) return -1;
     switch (p.E) {
         case 128: return launch_replay_tiled<128, 4, 16>(p, s);
-        case 64: return launch_replay_tiled<64, 2, 8>(p, s);
-        case 32: return launch_replay_tiled<32, 1, 8>(p, s);
+        case 64: return launch_replay_tiled<64, 4, 8>(p, s);
+        case 32: return launch_replay_tiled<32, 4, 8>(p, s);
         case 16: return launch_replay_tiled<16, 1, 8>(p, s);
         case 8: return launch_replay_tiled<8, 1, 8>(p, s);
         default: return -1;
@@ -291,6 +398,7 @@ int launch_replay(const ReplayParams &p, hipStream_t s) {
     const size_t lds = replay_lds_bytes(p.E, p.M);
     if (const int err = allow_max_dynamic_lds<replay_kernel>()) return err;
     hipLaunchKernelGGL(replay_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
+    if (p.xg) hipLaunchKernelGGL(outer_sum_kernel, dim3(p.N * p.H), dim3(kThreads), 0, s, p);
     return (int)hipGetLastError();
 }
 

@@ -19,7 +19,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from fast_weight import fast_weight_delta, fast_weight_delta_steps
-from self_ref_v0 import self_ref_layer, self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
+from self_ref_v0 import self_ref_layer, self_ref_layer_steps, self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
 from self_ref_v1 import self_ref_v1, self_ref_v1_steps
 
 
@@ -155,8 +155,13 @@ class SRlayer(_SRBase):
         does, reinforcement_learning/torchbeast_procgen/model.py:1176-1196), in one kernel launch
         forward and one backward.  h: (T, B, H*d); notdone: (T, B), 0 where an episode ended."""
         assert state is not None
-        x, slen, bsz = self._split(h, True)
         keep = notdone.to(h.dtype).transpose(0, 1).contiguous()            # (B, T)
+        if FUSED_SRWM_LAYER:
+            slen, bsz, _ = h.size()
+            x = h.reshape(slen, bsz, self.num_head, self.dim_head).permute(1, 2, 0, 3)
+            out, *new_state = self_ref_layer_steps(x, keep, *self._slow(), *state, True)
+            return h + self._project(out, bsz, slen), tuple(new_state)
+        x, slen, bsz = self._split(h, True)
         fast = [s.detach() + w.detach().repeat(bsz, 1, 1, 1) for s, w in zip(state, self._slow())]
         out = self_ref_v0_steps(x, keep, *fast, *self._slow())
         out = h + self._project(out, bsz, slen)
@@ -233,20 +238,24 @@ class SMFWPlayer(nn.Module):
         launch per operator.  h: (T, B, H*d); notdone: (T, B), 0 where an episode ended."""
         assert state is not None
         slen, bsz, _ = h.size()
-        x = F.softmax(h.reshape(slen, bsz, self.num_head, self.dim_head), dim=-1).permute(1, 2, 0, 3)
         keep = notdone.to(h.dtype).transpose(0, 1).contiguous()            # (B, T)
         slow = (self.W_y, self.W_q, self.W_k, self.w_b)
         *shift, fast_weights = state
-        fast = [s.detach() + w.detach().repeat(bsz, 1, 1, 1) for s, w in zip(shift, slow)]
-        qkvb = self_ref_v1_steps(x, keep, *fast, *slow)
+        if FUSED_SRWM_LAYER:
+            x = h.reshape(slen, bsz, self.num_head, self.dim_head).permute(1, 2, 0, 3)
+            qkvb, *new_state = self_ref_layer_steps(x, keep, *slow, *shift, True)
+        else:
+            x = F.softmax(h.reshape(slen, bsz, self.num_head, self.dim_head), dim=-1).permute(1, 2, 0, 3)
+            fast = [s.detach() + w.detach().repeat(bsz, 1, 1, 1) for s, w in zip(shift, slow)]
+            qkvb = self_ref_v1_steps(x, keep, *fast, *slow)
+            new_state = [f - w.detach().repeat(bsz, 1, 1, 1) for f, w in zip(fast, slow)]
         q, k, v, beta = torch.split(qkvb, (self.dim_head,) * 3 + (1,), -1)
         memory = fast_weights.detach().clone()
         out = fast_weight_delta_steps(F.softmax(q, dim=-1), F.softmax(k, dim=-1), v, torch.sigmoid(beta),
                                       keep, memory)
         out = _heads_out(out, bsz, slen, self.num_head * self.dim_head)
         out = h + self.drop(self.out_linear(out))
-        new_state = tuple(f - w.detach().repeat(bsz, 1, 1, 1) for f, w in zip(fast, slow))
-        return out, new_state + (memory,)
+        return out, tuple(new_state) + (memory,)
 
 
 class _DeltaBase(nn.Module):

@@ -13,6 +13,7 @@ weights, everything saved for the backward and all arithmetic stay float32.
 The weight tensors are OVERWRITTEN with the state after the last step (the layers read
 them back as the carried state); the backward starts from that mutated tensor.
 """
+import math
 import threading
 
 import torch
@@ -155,6 +156,72 @@ class SelfRefv0Steps(torch.autograd.Function):
 
 
 self_ref_v0_steps = SelfRefv0Steps.apply
+
+
+def _softmax_rows(x):
+    """softmax over the last axis, computed in the order the rows lie in memory (the layers hand
+    over a permuted view; soft-maxing it as it is indexed would copy it first)."""
+    order = sorted(range(x.dim() - 1), key=lambda i: -x.stride(i)) + [x.dim() - 1]
+    y = torch.softmax(x.permute(order), dim=-1)
+    return y.permute([order.index(i) for i in range(x.dim())])
+
+
+class SelfRefLayerStepsFn(torch.autograd.Function):
+    """`self_ref_v0_steps` as the layers call it, with their elementwise work inside the kernels:
+    the `state.detach() + W.repeat(bsz, 1, 1, 1)` that builds the weights, the softmax of the input,
+    the `- W.repeat(...)` that turns the final weights back into the carried shift, and the sum over
+    the batch and the steps that the shared W_y receives as its gradient
+    (reinforcement_learning/torchbeast/layer.py:377-421 for one step; the learner's loop over the
+    steps of an unroll, torchbeast_procgen/model.py:1176-1196).
+
+        out, dW_y, dW_q, dW_k, dw_b = self_ref_layer_steps(x, keep, sW_y, sW_q, sW_k, sw_b,
+                                                           shift_y, shift_q, shift_k, shift_b, softmax_input)
+
+    x: (N, H, L, E), any strides, before its softmax when `softmax_input`; keep: (N, L) float, 0
+    where the carried shift is zeroed before the step, or None; sW_*: the shared weights
+    (1, H, E, .); shift_*: (N, H, E, .) carried shift (not modified, used as given: no gradient
+    flows into it).  Returns the output and the new shift (no gradient flows out of it).
+    Gradients: x, and the shared weights as in `self_ref_v0_steps`.
+    """
+
+    @staticmethod
+    def forward(ctx, x, keep, sW_y, sW_q, sW_k, sw_b, shift_y, shift_q, shift_k, shift_b, softmax_input):
+        N, H, L, E = x.shape
+        Y = sW_y.shape[-1]
+        dev = x.device
+        f32 = torch.float32
+        state = [s.detach().clone(memory_format=torch.contiguous_format) for s in (shift_y, shift_q, shift_k, shift_b)]
+        out = torch.empty((N, H, L, Y), device=dev, dtype=f32)
+        saved = [torch.empty((N, H, L, w), device=dev, dtype=f32) for w in (E, E, 4, Y, E, E, 4)]
+        flags = srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_SOFTMAX_INPUT if softmax_input else 0)
+        srwm_hip.self_ref_layer_forward(x.detach(), keep, (sW_y, sW_q, sW_k, sw_b), *state, *saved, out, flags=flags)
+        ctx.save_for_backward(x, keep, saved[1], saved[2], saved[3], shift_y, sW_y)
+        ctx.softmax_input = softmax_input
+        ctx.slow_shapes = (sW_q.shape, sW_k.shape, sw_b.shape)
+        ctx.mark_non_differentiable(*state)
+        return (out, *state)
+
+    @staticmethod
+    def backward(ctx, grad_out, *_):
+        x, keep, k, beta, y_diff, shift_y, sW_y = ctx.saved_tensors
+        N, H, L, E = x.shape
+        Y = y_diff.shape[-1]
+        dev = x.device
+        sx = _softmax_rows(x) if ctx.softmax_input else x
+        u = torch.empty((N, H, L, E), device=dev, dtype=torch.float32)
+        rows = torch.empty((N, H, E, Y), device=dev, dtype=torch.float32)
+        g_sWy = torch.empty((H, E, Y), device=dev, dtype=torch.float32)
+        srwm_hip.self_ref_layer_readout_grad(sx, k, beta, y_diff, keep, sW_y, grad_out, shift_y, u, rows, g_sWy,
+                                             flags=srwm_hip.FLAG_STATE_SHIFT)
+        grad_x = torch._softmax_backward_data(u, sx, -1, u.dtype) if ctx.softmax_input else u
+        # the other shared weights: zeros, as the per-step calls return (one fill for the three)
+        sizes = [math.prod(s) for s in ctx.slow_shapes]
+        zeros = torch.zeros(sum(sizes), device=dev, dtype=torch.float32).split(sizes)
+        return (grad_x, None, g_sWy.reshape(sW_y.shape), *(z.view(s) for z, s in zip(zeros, ctx.slow_shapes)),
+                None, None, None, None, None)
+
+
+self_ref_layer_steps = SelfRefLayerStepsFn.apply
 
 
 # SelfRefLayerFn, calls that need no gradient: their per-step vectors are written and never read,

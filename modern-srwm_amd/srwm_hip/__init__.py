@@ -34,7 +34,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _lib = None
 
@@ -56,6 +56,7 @@ _SIGNATURES = {
     "srwm_layer_backward_bf16": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_wide_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_readout_grad_f32": [_F, _S] + [_F] * 5 + [_F, _S] + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
     "delta_forward_steps_f32": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -295,6 +296,48 @@ def self_ref_readout_grad(k, beta, y_diff, keep, slow_W_y, grad_out, W_y_entry, 
             _ptr(slow_W_y) if keep is not None else null, _ptr(gos), gstr, _ptr(sv[3]), _ptr(gr[0]),
             N, H, L, E, Y, flags, _stream(k.device))
     _check(code, "srwm_readout_grad_wide_f32")
+
+
+def self_ref_layer_readout_grad(x, k, beta, y_diff, keep, slow_W_y, grad_out, W_y_entry, grad_x, grad_W_y,
+                                grad_slow_W_y, flags=0):
+    """self_ref_readout_grad plus the gradient of the shared W_y, for a layer's whole unroll:
+    grad_x[n, h, t] = W_y,t-1 grad_out[n, h, t]; grad_W_y[n, h] = sum_t x_t (x) grad_out_t
+    ((N, H, E, Y), written); grad_slow_W_y (H, E, Y) = its sum over the batch.  x: the operator's
+    input (soft-maxed if the layer soft-maxes it), any strides.  flags: FLAG_STATE_SHIFT (W_y_entry
+    is the carried shift from the shared weights), FLAG_GENERIC."""
+    _require(k, "k")
+    N, H, L, E = k.shape
+    _require(y_diff, "y_diff")
+    Y = y_diff.shape[-1]
+    _require(x, "x", (N, H, L, E))
+    _require(beta, "beta", (N, H, L, 4))
+    _require(y_diff, "y_diff", (N, H, L, Y))
+    _require(grad_out, "grad_out", (N, H, L, Y))
+    _require(W_y_entry, "W_y_entry", (N, H, E, Y))
+    _require(grad_x, "grad_x", (N, H, L, E))
+    _require(grad_W_y, "grad_W_y", (N, H, E, Y))
+    _require(grad_slow_W_y, "grad_slow_W_y", (H, E, Y))
+    if not (grad_W_y.is_contiguous() and grad_slow_W_y.is_contiguous()):
+        raise ValueError("grad_W_y and grad_slow_W_y must be contiguous")
+    slow_W_y = slow_W_y.detach().reshape(H, E, Y).contiguous()
+    _require(slow_W_y, "slow W_y", (H, E, Y))
+    null = ctypes.c_void_p(None)
+    if keep is not None:
+        _require(keep, "keep", (N, L))
+        keep = keep.contiguous()
+    if k.numel() == 0:
+        grad_W_y.zero_()
+        grad_slow_W_y.zero_()
+        return
+    xs, xstr = _strided(x)
+    gos, gstr = _strided(grad_out)
+    with torch.cuda.device(k.device), _Dense([k, beta, y_diff, W_y_entry], False) as sv, \
+            _Dense([grad_x], True) as gr:
+        code = lib().srwm_layer_readout_grad_f32(
+            _ptr(xs), xstr, _ptr(sv[0]), _ptr(sv[1]), _ptr(sv[2]), _ptr(keep) if keep is not None else null,
+            _ptr(slow_W_y), _ptr(gos), gstr, _ptr(sv[3]), _ptr(gr[0]), _ptr(grad_W_y), _ptr(grad_slow_W_y),
+            N, H, L, E, Y, flags, _stream(k.device))
+    _check(code, "srwm_layer_readout_grad_f32")
 
 
 def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out,

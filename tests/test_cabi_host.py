@@ -154,5 +154,11 @@ def test_argument_validation_needs_no_gpu():
     assert noalloc(N, 0, P(None)) == -1                        # the batch sums are what it is for
     assert noalloc(N, 1, fake()) == -1                         # no buffer for an incoming state gradient
     assert noalloc(1 << 16, 0, fake()) == -5                   # SRWM_ESCRATCH: 2^16 x 8 rows of 16 x 52 floats > 32 MiB
+    readout = lambda sw, gs, flags: L.srwm_layer_readout_grad_f32(
+        fake(), ok_strides, fake(), fake(), fake(), P(None), sw, fake(), ok_strides, fake(), fake(), fake(), gs,
+        N, H, Ls, E, E, flags, P(None))
+    assert readout(P(None), fake(), 64) == -1                  # the shared W_y is always needed
+    assert readout(fake(), P(None), 0) == -1                   # its gradient is what the call is for
+    assert readout(fake(), fake(), 128) == -1                  # a fresh start has no entry state to replay from
     assert L.srwm_hip_scratch_bytes() == 32 << 20
     assert b"scratch" in L.srwm_hip_strerror(-5)

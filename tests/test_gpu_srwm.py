@@ -310,6 +310,58 @@ def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
         assert float(w.grad.abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("shape,Y,resets,softmax", [
+    ((4, 8, 100, 32), None, True, True),      # benchmark configuration 3 shape (batch slice)
+    ((2, 2, 37, 64), None, True, True),
+    ((2, 1, 21, 48), None, True, False),      # LDS-resident replay + the plain outer-sum kernel
+    ((3, 2, 20, 12), None, True, True),
+    ((2, 3, 15, 16), None, False, False),     # keep = None
+    ((2, 2, 30, 32), 97, True, True),         # wide output block
+    ((2, 2, 19, 8), 25, True, False),
+    ((2, 2, 19, 12), 37, True, True),         # wide, LDS-resident replay
+])
+def test_stepwise_layer_operator_matches_the_per_step_reference(shape, Y, resets, softmax):
+    """self_ref_layer_steps (the layers' form of the unroll: shift in, shift out, softmax of the
+    input and the shared-W_y gradient inside the library) vs the literal per-step loop in fp64, the
+    input handed over as the permuted view of (L, N, H*E) storage the layers pass."""
+    print(f"case stepwise layer operator shape={shape} Y={Y} resets={resets} softmax={softmax}", flush=True)
+    from oracle.recurrence import srwm_steps_reference
+    from self_ref_v0 import self_ref_layer_steps
+    from test_oracle_srwm import _steps_inputs
+    dev = _dev()
+    N, H, L, E = shape
+    x, keep, shift, slow, go = _steps_inputs(N, H, L, E, seed=43, resets=resets)
+    g = torch.Generator().manual_seed(7)
+    raw = torch.randn(N, H, L, E, generator=g, dtype=torch.float64) if softmax else x
+    if Y is not None:
+        slow[0] = torch.randn(1, H, E, Y, generator=g, dtype=torch.float64) * 0.4
+        shift[0] = torch.randn(N, H, E, Y, generator=g, dtype=torch.float64) * 0.2
+        go = torch.randn(N, H, L, Y, generator=g, dtype=torch.float64)
+    xr = raw.clone().requires_grad_(True)
+    sr = [w.clone().requires_grad_(True) for w in slow]
+    ref_out, ref_shift = srwm_steps_reference(torch.softmax(xr, -1) if softmax else xr, keep, shift, sr)
+    (ref_out * go).sum().backward()
+
+    f32 = lambda t: t.to(dev, torch.float32)
+    store = f32(raw).permute(2, 0, 1, 3).contiguous().requires_grad_(True)      # (L, N, H, E)
+    sd = [f32(w).requires_grad_(True) for w in slow]
+    shift_d = [f32(s_) for s_ in shift]
+    before = [s_.clone() for s_ in shift_d]
+    out, *new_shift = self_ref_layer_steps(store.permute(1, 2, 0, 3), None if keep is None else f32(keep), *sd,
+                                           *shift_d, softmax)
+    (out * f32(go)).sum().backward()
+    assert rel_err(out.detach().cpu().numpy(), ref_out.detach().numpy()) < TOL
+    for got, want, w in zip(new_shift, ref_shift, slow):       # measured on the weights' scale, as they are carried
+        assert not got.requires_grad
+        assert np.abs(got.cpu().numpy() - want.numpy()).max() < TOL * float((want + w).abs().max())
+    for a, b in zip(shift_d, before):                          # the incoming shift is left alone
+        assert torch.equal(a, b)
+    assert rel_err(store.grad.permute(1, 2, 0, 3).cpu().numpy(), xr.grad.numpy()) < TOL
+    assert rel_err(sd[0].grad.cpu().numpy(), sr[0].grad.numpy()) < TOL
+    for w in sd[1:]:
+        assert w.grad.shape == w.shape and float(w.grad.abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("E,L", [(64, 15), (64, 16), (64, 17), (64, 32), (64, 33), (32, 31), (32, 32), (32, 33),
                                  (32, 64), (16, 16), (16, 17), (8, 32), (8, 33)])
 def test_sequence_lengths_around_the_input_tile_size(E, L):
