@@ -273,3 +273,72 @@ def test_empty_sequences_and_batches():
     (out.sum() + sum(s.sum() for s in shift)).backward()
     assert all(bool((s == 0).all()) for s in shift)            # no steps: the state stays at the shared weights
     assert all(bool((w.grad == 0).all()) for w in slow)        # d(shift)/d(shared) = dW_L/d(shared) - 1 = 0
+
+
+def test_learner_unroll_with_autograd_replays_from_a_captured_hip_graph():
+    """SRlayer.forward_steps (T = 20 steps, resets) forward AND backward through autograd, captured into
+    one graph: every replay with new inputs in the static buffers must equal the eager result bit for
+    bit -- output, carried state, input gradient and every parameter gradient.  Replayed several
+    times with eager work and synchronisations in between, which is what exposes a memset node that
+    a library call might have recorded."""
+    print("case graph replay of the learner unroll", flush=True)
+    import layer
+    dev = _dev()
+    T, B, H, d = 20, 4, 4, 32
+    torch.manual_seed(3)
+    lay = layer.SRlayer(H, d, H * d, 0.0).to(dev)
+    params = [p for p in lay.parameters() if p.requires_grad]
+    g = torch.Generator().manual_seed(9)
+    h_s = torch.zeros(T, B, H * d, device=dev, requires_grad=True)
+    nd_s = torch.ones(T, B, device=dev)
+    go_s = torch.zeros(T, B, H * d, device=dev)
+    st_s = tuple(torch.zeros(B, H, d, w, device=dev) for w in (d, d, d, 4))
+
+    def run(h, nd, st, go):
+        out, new = lay.forward_steps(h, nd, st)
+        out.backward(go)
+        return out, new
+
+    def clear():
+        h_s.grad = None
+        for p in params:
+            p.grad = None
+
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        for _ in range(3):                        # warm-up outside the capture
+            clear()
+            run(h_s, nd_s, st_s, go_s)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize()
+    clear()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_s, new_s = run(h_s, nd_s, st_s, go_s)
+    params = [p for p in params if p.grad is not None]        # the RL layer leaves its LayerNorm unused
+    assert len(params) == 5
+    for it in range(4):
+        h = torch.randn(T, B, H * d, generator=g).to(dev)
+        nd = (torch.rand(T, B, generator=g) > 0.2).float().to(dev)
+        go = torch.randn(T, B, H * d, generator=g).to(dev)
+        st = tuple((torch.randn(B, H, d, w, generator=g) * 0.1).to(dev) for w in (d, d, d, 4))
+        with torch.no_grad():
+            h_s.copy_(h); nd_s.copy_(nd); go_s.copy_(go)
+            for a, b in zip(st_s, st):
+                a.copy_(b)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [out_s.clone(), *[s.clone() for s in new_s], h_s.grad.clone(), *[p.grad.clone() for p in params]]
+        # eager, on fresh tensors holding the same values
+        saved_grads = [p.grad for p in params]
+        for p in params:
+            p.grad = None
+        he = h.clone().requires_grad_(True)
+        oe, ne = run(he, nd, st, go)
+        torch.cuda.synchronize()
+        want = [oe, *ne, he.grad, *[p.grad for p in params]]
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), (it, i)
+        for p, sg in zip(params, saved_grads):    # hand the graph's static gradient buffers back
+            p.grad = sg
