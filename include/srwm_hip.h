@@ -383,6 +383,24 @@ SRWM_API int delta_readout_replay_f32(const float *K, const int64_t k_strides[3]
                              int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
 /*
+ * The whole backward of delta_forward_steps_f32 in one call: delta_readout_replay_f32 followed by the
+ * four per-step formulas above in one elementwise kernel (same regime: the memory carries no gradient).
+ *   Q, K, V, beta, keep, v_old, v_insert   as handed to / left by delta_forward_steps_f32
+ *   W_entry   dense [N,H,E,M]: the memory before that call
+ *   gQ, gK dense [N,H,L,E];  gV dense [N,H,L,M];  gbeta dense [N,H,L,1]   (overwritten; gQ also serves as
+ *   the buffer for u between the two kernels)
+ */
+SRWM_API int delta_steps_backward_f32(const float *Q, const int64_t q_strides[3],
+                             const float *K, const int64_t k_strides[3],
+                             const float *V, const int64_t v_strides[3],
+                             const float *beta, const int64_t beta_strides[3],
+                             const float *keep, const float *v_old, const float *v_insert,
+                             const float *grad_out, const int64_t grad_out_strides[3],
+                             const float *W_entry,
+                             float *gQ, float *gK, float *gV, float *gbeta,
+                             int N, int H, int L, int E, int M, unsigned flags, void *stream);
+
+/*
  * Delta rule with bf16 inputs/outputs and fp32 memory.  No counterpart in the reference
  * (its kernels are float-only, fast_weight_cuda.cu:12-14); same recurrence as
  * delta_forward_f32 / delta_backward_f32 with
@@ -425,7 +443,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any signature change); currently 6. */
+/* ABI version of this header (bumped on any signature change); currently 7. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

@@ -85,7 +85,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 6; }
+int srwm_hip_abi_version(void) { return 7; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -291,6 +291,28 @@ int delta_readout_replay_f32(const float *K, const int64_t ks[3], const float *v
     }
     if (E > 256 || M > 256 || replay_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_replay(p, (hipStream_t)stream);
+}
+
+int delta_steps_backward_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],
+                             const float *V, const int64_t vs[3], const float *beta, const int64_t bs[3],
+                             const float *keep, const float *v_old, const float *v_insert,
+                             const float *grad_out, const int64_t gs[3], const float *W_entry, float *gQ,
+                             float *gK, float *gV, float *gbeta, int N, int H, int L, int E, int M,
+                             unsigned flags, void *stream) {
+    if (!Q || !K || !V || !beta || !v_old || !v_insert || !grad_out || !W_entry || !gQ || !gK || !gV || !gbeta ||
+        !qs || !ks || !vs || !bs || !gs)
+        return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
+        !stride_ok(bs, N, H, L, 1) || !stride_ok(gs, N, H, L, M))
+        return SRWM_ESTRIDE;
+    const int r = delta_readout_replay_f32(K, ks, v_insert, keep, grad_out, gs, W_entry, gQ, N, H, L, E, M, flags,
+                                           stream);
+    if (r) return r;
+    DeltaStepGradParams p{Q, K, V, beta, grad_out, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
+                          {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, {gs[0], gs[1], gs[2]}, v_old, v_insert,
+                          gQ, gK, gV, gbeta, N, H, L, E, M};
+    return launch_delta_step_grads(p, (hipStream_t)stream);
 }
 
 int srwm_backward_wide_f32(const float *x, const int64_t xs[3], const float *q, const float *k,

@@ -77,6 +77,17 @@ struct ReplayParams {
     int w0_is_shift;       // W0 holds W - Wreset (Wreset must be given)
 };
 
+// Per-step gradients of the delta rule when the memory carries no gradient, from u_t = W_{t-1} g_t
+// (which arrives in grad_q):  kq = k.q, ig = v_insert.g:
+//   grad_q = u + ig k,  grad_k = ig q - beta kq u,  grad_v = beta kq g,  grad_beta = kq g.(v - v_old)
+struct DeltaStepGradParams {
+    const float *Q, *K, *V, *beta, *g;
+    Strided3 qs, ks, vs, bs, gs;
+    const float *vold, *vins;               // dense [N,H,L,M]
+    float *gq, *gk, *gv, *gbeta;            // dense; gq holds u on entry
+    int N, H, L, E, M;
+};
+
 struct DeltaFwdParams {
     const float *Q, *K, *V, *beta;
     Strided3 qs, ks, vs, bs;
@@ -177,6 +188,7 @@ int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s);
 size_t replay_lds_bytes(int E, int M);
 int launch_replay(const ReplayParams &p, hipStream_t s);
 int launch_replay_tiled(const ReplayParams &p, hipStream_t s);   // -1: no register-resident instantiation
+int launch_delta_step_grads(const DeltaStepGradParams &p, hipStream_t s);
 int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s);
 // dst[j][h, :] = sum over n of src[j][n, h, :] for the four state tensors (y: E x Y, q, k: E x E, b: E x 4)
 int launch_srwm_batch_sum(const float *const src[4], float *const dst[4], int N, int H, int E, int Y, hipStream_t s);

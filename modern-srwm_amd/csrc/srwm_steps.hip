@@ -102,6 +102,45 @@ __global__ __launch_bounds__(kThreads) void outer_sum_kernel(ReplayParams p) {
     }
 }
 
+// The elementwise end of the delta rule's step-mode backward: 16 lanes per (sequence, step), which
+// walk the vectors of the step with a stride of 16 and meet in three 16-lane sums.
+__global__ __launch_bounds__(kThreads) void delta_step_grads_kernel(DeltaStepGradParams p) {
+    const int gl = threadIdx.x & 15;
+    const int64_t row = (int64_t)blockIdx.x * (kThreads / 16) + (threadIdx.x >> 4);   // (n*H + h)*L + t
+    const int64_t rows = (int64_t)p.N * p.H * p.L;
+    const bool live = row < rows;
+    const int64_t rc = live ? row : rows - 1;   // surplus groups compute on the last row and store nothing
+    const int t = (int)(rc % p.L);
+    const int64_t sq = rc / p.L;
+    const int n = (int)(sq / p.H), h = (int)(sq % p.H);
+    const float *q = p.Q + n * p.qs.n + h * p.qs.h + t * p.qs.l;
+    const float *k = p.K + n * p.ks.n + h * p.ks.h + t * p.ks.l;
+    const float *v = p.V + n * p.vs.n + h * p.vs.h + t * p.vs.l;
+    const float *g = p.g + n * p.gs.n + h * p.gs.h + t * p.gs.l;
+    const float bt = p.beta[n * p.bs.n + h * p.bs.h + t * p.bs.l];
+    const float *vo = p.vold + rc * p.M, *vi = p.vins + rc * p.M;
+    float kq = 0.f, ig = 0.f, gd = 0.f;
+    for (int e = gl; e < p.E; e += 16) kq = fmaf(k[e], q[e], kq);
+    for (int m = gl; m < p.M; m += 16) {
+        const float gm = g[m];
+        ig = fmaf(vi[m], gm, ig);
+        gd = fmaf(gm, v[m] - vo[m], gd);
+    }
+    kq = group_sum<16>(kq);
+    ig = group_sum<16>(ig);
+    gd = group_sum<16>(gd);
+    if (!live) return;
+    const float bkq = bt * kq;
+    float *gq = p.gq + rc * p.E, *gk = p.gk + rc * p.E, *gv = p.gv + rc * p.M;
+    for (int e = gl; e < p.E; e += 16) {
+        const float u = gq[e];
+        gq[e] = fmaf(ig, k[e], u);
+        gk[e] = fmaf(ig, q[e], -bkq * u);
+    }
+    for (int m = gl; m < p.M; m += 16) gv[m] = bkq * g[m];
+    if (gl == 0) p.gbeta[rc] = kq * gd;
+}
+
 // Register-resident replay.  NWV waves per sequence; wave w owns rows [w*ER, (w+1)*ER), ER = E/NWV.
 // Inside a wave, CGL consecutive lanes share a block of R rows and split its columns (CB each).
 // M need not be a multiple of CGL or of 4 (the wide output block of the SRWM has M = 3E+1): the
@@ -390,6 +429,12 @@ int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
         case 8: return launch_replay_tiled<8, 1, 8>(p, s);
         default: return -1;
     }
+}
+
+int launch_delta_step_grads(const DeltaStepGradParams &p, hipStream_t s) {
+    const int64_t rows = (int64_t)p.N * p.H * p.L, per = kThreads / 16;
+    hipLaunchKernelGGL(delta_step_grads_kernel, dim3((unsigned)((rows + per - 1) / per)), dim3(kThreads), 0, s, p);
+    return (int)hipGetLastError();
 }
 
 size_t replay_lds_bytes(int E, int M) { return sizeof(float) * ((size_t)E * (M | 1) + E + 2 * (size_t)M); }

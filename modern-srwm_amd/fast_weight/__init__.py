@@ -109,14 +109,12 @@ class DeltaFastWeightSteps(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_out):
         Q, K, V, beta, keep, V_old, V_insert, W_entry = ctx.saved_tensors
-        u = torch.empty(Q.shape, device=Q.device, dtype=Q.dtype)
-        srwm_hip.fast_weight_readout_replay(K, V_insert, keep, grad_out, W_entry, u)
-        kq = (K * Q).sum(-1, keepdim=True)
-        ig = (V_insert * grad_out).sum(-1, keepdim=True)
-        grad_Q = u + ig * K
-        grad_K = ig * Q - (beta * kq) * u
-        grad_V = (beta * kq) * grad_out
-        grad_beta = kq * (grad_out * (V - V_old)).sum(-1, keepdim=True)
+        N, H, L, E = Q.shape
+        M = V.shape[-1]
+        new = lambda w: torch.empty((N, H, L, w), device=Q.device, dtype=Q.dtype)
+        grad_Q, grad_K, grad_V, grad_beta = new(E), new(E), new(M), new(1)
+        srwm_hip.fast_weight_steps_backward(Q, K, V, beta, keep, V_old, V_insert, grad_out, W_entry,
+                                            grad_Q, grad_K, grad_V, grad_beta)
         return grad_Q, grad_K, grad_V, grad_beta, None, None
 
 

@@ -34,7 +34,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _lib = None
 
@@ -61,6 +61,7 @@ _SIGNATURES = {
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
     "delta_forward_steps_f32": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_readout_replay_f32": [_F, _S] + [_F, _F] + [_F, _S] + [_F, _F] + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_steps_backward_f32": [_F, _S] * 4 + [_F] * 3 + [_F, _S] + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_forward_f32": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_backward_f32": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_forward_bf16": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -645,6 +646,40 @@ def fast_weight_readout_replay(k, v_insert, keep, grad_out, kv_entry, u, flags=0
                                               _ptr(gos), gstr, _ptr(sv[1]), _ptr(d[0]), N, H, L, E, M, flags,
                                               _stream(k.device))
     _check(code, "delta_readout_replay_f32")
+
+
+def fast_weight_steps_backward(q, k, v, beta, keep, v_old, v_insert, grad_out, kv_entry, grad_q, grad_k, grad_v,
+                               grad_beta, flags=0):
+    """The whole backward of fast_weight_forward_steps (the memory carries no gradient): the replay
+    of fast_weight_readout_replay and the per-step formulas, two launches.  grad_q, grad_k: (N, H, L, E);
+    grad_v: (N, H, L, M); grad_beta: (N, H, L, 1); all overwritten."""
+    _require(q, "q")
+    N, H, L, E = q.shape
+    _require(v, "v")
+    M = v.shape[-1]
+    _require(k, "k", (N, H, L, E))
+    _require(v, "v", (N, H, L, M))
+    _require(beta, "beta", (N, H, L, 1))
+    for t, nm in ((v_old, "v_old"), (v_insert, "v_insert"), (grad_out, "grad_out"), (grad_v, "grad_v")):
+        _require(t, nm, (N, H, L, M))
+    _require(kv_entry, "kv_entry", (N, H, E, M))
+    _require(grad_q, "grad_q", (N, H, L, E))
+    _require(grad_k, "grad_k", (N, H, L, E))
+    _require(grad_beta, "grad_beta", (N, H, L, 1))
+    null = ctypes.c_void_p(None)
+    if keep is not None:
+        _require(keep, "keep", (N, L))
+        keep = keep.contiguous()
+    if q.numel() == 0:
+        return
+    (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr), (gos, gstr) = (_strided(t) for t in (q, k, v, beta, grad_out))
+    with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv_entry], False) as sv, \
+            _Dense([grad_q, grad_k, grad_v, grad_beta], True) as d:
+        code = lib().delta_steps_backward_f32(
+            _ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr, _ptr(keep) if keep is not None else null,
+            _ptr(sv[0]), _ptr(sv[1]), _ptr(gos), gstr, _ptr(sv[2]), *[_ptr(t) for t in d], N, H, L, E, M, flags,
+            _stream(q.device))
+    _check(code, "delta_steps_backward_f32")
 
 
 def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v,

@@ -160,5 +160,10 @@ def test_argument_validation_needs_no_gpu():
     assert readout(P(None), fake(), 64) == -1                  # the shared W_y is always needed
     assert readout(fake(), P(None), 0) == -1                   # its gradient is what the call is for
     assert readout(fake(), fake(), 128) == -1                  # a fresh start has no entry state to replay from
+    dsteps = lambda gq, flags: L.delta_steps_backward_f32(
+        *[a for _ in range(4) for a in (fake(), ok_strides)], P(None), fake(), fake(), fake(), ok_strides, fake(),
+        gq, fake(), fake(), fake(), N, H, Ls, E, E, flags, P(None))
+    assert dsteps(P(None), 0) == -1                            # every gradient buffer is required
+    assert dsteps(fake(), 32) == -1                            # there is no chunkwise form of the step mode
     assert L.srwm_hip_scratch_bytes() == 32 << 20
     assert b"scratch" in L.srwm_hip_strerror(-5)

@@ -422,14 +422,17 @@ def test_chunkwise_flag_is_refused_where_there_is_no_kernel():
 
 # ------------------------------------------------------------------ step-wise (RL learner) call pattern
 
-@pytest.mark.parametrize("shape,resets", [
-    ((4, 8, 100, 32, 32), True),     # RL-sized heads, register-resident forward
-    ((2, 2, 40, 64, 64), True),
-    ((2, 3, 25, 12, 20), True),      # E != M: generic forward
-    ((2, 2, 30, 16, 16), False),     # keep = None
+@pytest.mark.parametrize("shape,resets,strided", [
+    ((4, 8, 100, 32, 32), True, False),     # RL-sized heads, register-resident forward
+    ((2, 2, 40, 64, 64), True, False),
+    ((2, 3, 25, 12, 20), True, False),      # E != M: generic forward
+    ((2, 2, 30, 16, 16), False, False),     # keep = None
+    ((3, 2, 37, 32, 32), True, True),       # permuted views of (L, N, H, d) storage, as the layers pass them
+    ((1, 2, 19, 128, 128), True, True),
+    ((2, 1, 21, 20, 12), True, True),
 ])
-def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
-    print(f"case delta stepwise shape={shape} resets={resets}", flush=True)
+def test_stepwise_operator_matches_the_per_step_reference(shape, resets, strided):
+    print(f"case delta stepwise shape={shape} resets={resets} strided={strided}", flush=True)
     from oracle.recurrence import delta_steps_reference
     from fast_weight import fast_weight_delta_steps
     dev = _dev()
@@ -444,11 +447,19 @@ def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
     ref_out, ref_W = delta_steps_reference(*ref_leaves, keep, W0)
     (ref_out * go).sum().backward()
     f32 = lambda t: t.to(dev, torch.float32)
-    leaves = [f32(t).requires_grad_(True) for t in (q, k, v, beta)]
+    if strided:
+        store = [f32(t).permute(2, 0, 1, 3).contiguous().requires_grad_(True) for t in (q, k, v, beta)]
+        leaves = [t.permute(1, 2, 0, 3) for t in store]
+        god = f32(go).permute(2, 0, 1, 3).contiguous().permute(1, 2, 0, 3)
+        grads = lambda: [t.grad.permute(1, 2, 0, 3) for t in store]
+    else:
+        leaves = [f32(t).requires_grad_(True) for t in (q, k, v, beta)]
+        god = f32(go)
+        grads = lambda: [t.grad for t in leaves]
     W = f32(W0).contiguous()
     out = fast_weight_delta_steps(*leaves, None if keep is None else f32(keep), W)
-    (out * f32(go)).sum().backward()
+    out.backward(god)
     assert rel_err(out.detach().cpu().numpy(), ref_out.detach().numpy()) < TOL
     assert rel_err(W.cpu().numpy(), ref_W.numpy()) < TOL
-    for a, b, nm in zip(leaves, ref_leaves, ("grad_Q", "grad_K", "grad_V", "grad_beta")):
-        assert rel_err(a.grad.cpu().numpy(), b.grad.numpy()) < TOL, nm
+    for a, b, nm in zip(grads(), ref_leaves, ("grad_Q", "grad_K", "grad_V", "grad_beta")):
+        assert rel_err(a.cpu().numpy(), b.grad.numpy()) < TOL, nm
