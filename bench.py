@@ -59,7 +59,8 @@ WORKLOADS = {
     # copies), softmax of the layer input inside the kernels, weight gradients summed over the batch
     "srwm_layer_c4": ("srwm_layer", 32, 16, 512, 64),
     # the RL learner's regime on the same shape: gradient cut at the carried state, 5 % resets;
-    # one launch for the unroll (forward) + readout-gradient replay + the batched x (x) g product
+    # one launch for the unroll (forward); backward = the replay of the y block, which also accumulates
+    # x (x) grad_out per sequence, + the batch sum of those tiles (srwm_layer_readout_grad_f32)
     "srwm_c3_steps": ("srwm_steps", 32, 8, 100, 32),
     # the same shape with the output block 3E+1 = 97 columns wide (the self_ref_v1 operator)
     "srwm_wide_c3": ("srwm_wide", 32, 8, 100, 32),
@@ -239,9 +240,12 @@ def algorithmic_bytes(op, N, H, L, E):
         Y = 3 * E + 1
         S = E * (Y + 2 * E + 4)
         return 3 * S * 4 * hs, 6 * S * 4 * hs, (11 * E + 4 * Y + 16) * 4 * hs + 4 * S * 4 * N * H
-    if op == "srwm_steps":   # forward as above; the replay reads and writes the E x E y block once per step
+    if op == "srwm_steps":
+        # forward as above; the backward replays the E x E y block (read for W g, written by the step's update)
+        # and adds x (x) g to a gradient tile of the same shape: 3 passes.  HBM: the backward also reads x and
+        # writes + re-reads the per-sequence gradient tiles that the batch sum adds up.
         S = E * (3 * E + 4)
-        return 3 * S * 4 * hs, 2 * E * E * 4 * hs, ((7 * E + 8) + (4 * E + 4)) * 4 * hs + (2 * S + E * E) * 4 * N * H
+        return 3 * S * 4 * hs, 3 * E * E * 4 * hs, ((7 * E + 8) + (5 * E + 4)) * 4 * hs + (2 * S + 3 * E * E) * 4 * N * H
     S = E * E
     # per (sequence, step): q,k,v,beta in (fwd and bwd), out + grad_out in the I/O type; v_old,
     # v_insert written and read back, and the 3 E-wide gradients + grad_beta written, in fp32
@@ -343,6 +347,8 @@ def vector_flops(op, N, H, L, E):
     hs = N * H * L
     if op.startswith("srwm"):
         S = E * ((3 * E + 1 if op == "srwm_wide" else E) + 2 * E + 4)
+        if op == "srwm_steps":   # the backward only passes over the E x E y block (3 passes, see algorithmic_bytes)
+            return 6.0 * S * hs, 6.0 * E * E * hs
         return 6.0 * S * hs, 12.0 * S * hs
     return 4.0 * E * E * hs, 8.0 * E * E * hs
 
