@@ -439,7 +439,7 @@ def rooflines(name, fwd_ms, bwd_ms):
 
 
 # Driver-visible figures for the other benchmark configurations: (workload, timed steps, warm-up)
-OTHER_WORKLOADS = (("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
+OTHER_WORKLOADS = (("srwm_layer_c4", 50, 10), ("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
                    ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5))
 
 
