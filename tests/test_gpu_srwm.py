@@ -318,6 +318,8 @@ def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
     ((2, 3, 15, 16), None, False, False),     # keep = None
     ((2, 2, 30, 32), 97, True, True),         # wide output block
     ((2, 2, 19, 8), 25, True, False),
+    ((1, 2, 21, 64), 193, True, True),
+    ((2, 2, 18, 16), 49, True, True),
     ((2, 2, 19, 12), 37, True, True),         # wide, LDS-resident replay
 ])
 def test_stepwise_layer_operator_matches_the_per_step_reference(shape, Y, resets, softmax):
