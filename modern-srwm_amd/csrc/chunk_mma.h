@@ -214,13 +214,23 @@ struct PrecBf16 {
     // wait state for that pair (it relies on the same-register forwarding that only holds between
     // equal opcodes), so whether a mixed chain is right depends on what the scheduler happens to put
     // in between.  Do not mix the two opcodes on one accumulator.
+    // The second half of the 32 contraction slots is not left empty when an operand has a lo part:
+    // the hi and lo planes of one operand ride side by side against the other operand twice, so one
+    // instruction forms two of the partial products (a.hi b.hi + a.hi b.lo, ...).
     template <bool SA, bool SB>
     __device__ static __forceinline__ f32x4 mma(const A &a, const B &b, f32x4 acc) {
-        const s16x4 z = {0, 0, 0, 0};
-        const bf16x8 ah = cat(a.hi, z), bh = cat(b.hi, z);
-        if constexpr (SA) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cat(a.lo, z), bh, acc, 0, 0, 0);
-        if constexpr (SB) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, cat(b.lo, z), acc, 0, 0, 0);
-        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, bh, acc, 0, 0, 0);
+        if constexpr (SA && SB) {   // all four partial products in two instructions, the small ones first
+            const bf16x8 bb = cat(b.hi, b.lo);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cat(a.lo, a.lo), bb, acc, 0, 0, 0);
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(cat(a.hi, a.hi), bb, acc, 0, 0, 0);
+        } else if constexpr (SB) {
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(cat(a.hi, a.hi), cat(b.hi, b.lo), acc, 0, 0, 0);
+        } else if constexpr (SA) {
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(cat(a.hi, a.lo), cat(b.hi, b.hi), acc, 0, 0, 0);
+        } else {
+            const s16x4 z = {0, 0, 0, 0};
+            return __builtin_amdgcn_mfma_f32_16x16x32_bf16(cat(a.hi, z), cat(b.hi, z), acc, 0, 0, 0);
+        }
     }
     // two groups of 16 contraction indices in one v_mfma_f32_16x16x32_bf16 (same 16 cycles as the
     // 16-index instruction): lane l supplies slots 4*(l/16) + j of the first group and of the second

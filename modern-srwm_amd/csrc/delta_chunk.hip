@@ -104,6 +104,10 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
     const TI *vb = p.V + n * p.vs.n + h * p.vs.h + m0;
     const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
     float *Wg = p.W + seq * D * D + m0 + cw;
+    // outputs of this sequence; L * D * 4 bytes fit 32 bits (the launcher checks), so rows are reached with
+    // 32-bit byte offsets from these uniform bases
+    float *vold_seq = p.vold + seq * p.L * D, *vins_seq = p.vins + seq * p.L * D;
+    TI *out_seq = p.out + seq * p.L * D;
 
     // this wave's 16 columns of the memory, accumulator layout per 16-row block
     f32x4 s[EB];
@@ -260,15 +264,30 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
             // out = Q S + tril(B) U
             ot[a] = mma_range<X, true, true>(
                 0, a + 1, [&](int b) { return X::lda(Bs, a * 16 + ln, b * 16 + 4 * lq); }, fu, ot[a]);
-            if (a % KS == hf)   // the two waves of a pair share the stores
+            if (a % KS == hf) {   // the two waves of a pair share the stores
+                // one 32-bit byte offset per lane from the sequence's (uniform) base; the rows of the
+                // block follow at compile-time distances
+                const uint32_t o0 = (uint32_t)(((t0 + a * 16 + 4 * lq) * D + m0 + cw + ln) * 4);
+                const auto at = [](auto *base, uint32_t byte_off) {
+                    typedef decltype(base) P;
+                    return reinterpret_cast<P>(reinterpret_cast<char *>(base) + byte_off);
+                };
+                if (t0 + kC <= p.L) {   // a full chunk: no row is past the end
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int t = t0 + a * 16 + 4 * lq + r;
-                if (t < p.L) {
-                    const int64_t o = (seq * p.L + t) * D + m0 + cw + ln;
-                    p.vold[o] = pt[a][r] + y[r];
-                    p.vins[o] = u[a][r];
-                    st_out(p.out + o, ot[a][r]);
+                    for (int r = 0; r < 4; ++r) {
+                        *at(vold_seq, o0 + r * D * 4) = pt[a][r] + y[r];
+                        *at(vins_seq, o0 + r * D * 4) = u[a][r];
+                        st_out(at(out_seq, (o0 + r * D * 4) / 4 * (uint32_t)sizeof(TI)), ot[a][r]);
+                    }
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        if (t0 + a * 16 + 4 * lq + r < p.L) {
+                            *at(vold_seq, o0 + r * D * 4) = pt[a][r] + y[r];
+                            *at(vins_seq, o0 + r * D * 4) = u[a][r];
+                            st_out(at(out_seq, (o0 + r * D * 4) / 4 * (uint32_t)sizeof(TI)), ot[a][r]);
+                        }
+                    }
                 }
             }
         }
@@ -308,6 +327,7 @@ bool rows_ok(const TI *ptr, const Strided3 &s) {
 template <class TI>
 int dispatch_chunk(const ChunkFwdP<TI> &p, int D, hipStream_t s) {
     if (!rows_ok(p.Q, p.qs) || !rows_ok(p.K, p.ks) || !rows_ok(p.V, p.vs)) return -1;
+    if ((int64_t)(p.L + kC) * D * 4 > (int64_t)UINT32_MAX) return -1;   // 32-bit byte offsets inside a sequence
     switch (D) {
         case 128: return launch_chunk<TI, 128, 2, PrecOf<TI>::type::kBf ? 2 : 1>(p, s);
         case 64: return launch_chunk<TI, 64, 1, 1>(p, s);
