@@ -1,5 +1,5 @@
 // Matrix-core building blocks of the chunkwise delta-rule kernels: LDS operand matrices, operand
-// fragments and the product of one group of 16 contraction indices, in two precisions.
+// fragments and the product of one group of 16 contraction indices, in three precisions.
 //
 // Index conventions (verified on gfx950): with lane = 16*lq + ln,
 //   A fragment  row ln of the left operand, contraction slots 4*lq + j (j = 0..3) of the group
@@ -281,6 +281,132 @@ struct PrecBf16 {
     }
 };
 
+// PrecBf16x3: fp32 operands on the bf16 matrix instruction.  A float is cut into three bf16
+// numbers of 8 significant bits each by truncation (hi = bits 31..16 of x, mid = bits 31..16 of
+// x - hi, lo = x - hi - mid, which has at most 8 significant bits left): x = hi + mid + lo
+// exactly.  A product takes the six partial products whose weight is 2^-16 or more relative to
+// hi*hi (hi*hi, hi*mid, mid*hi, mid*mid, hi*lo, lo*hi); every one of them is exact in fp32 and the
+// three dropped ones are below 2^-24, the rounding of an fp32 multiply.  32 contraction indices
+// cost 6 x 16 cycles instead of the 8 x 32 of v_mfma_f32_16x16x4f32.  One opcode throughout, as
+// in PrecBf16.
+struct PrecBf16x3 {
+    static constexpr bool kBf = false;
+    static constexpr int kPad = 4;
+    typedef float elem;
+    template <int LD, bool SPLIT>
+    struct Mat {
+        uint16_t *hi, *mid, *lo;
+        static constexpr int kLd = LD;
+        __host__ __device__ static constexpr int bytes(int rows) { return rows * LD * 2 * 3; }
+        __device__ explicit Mat(void *base, int rows)
+            : hi(static_cast<uint16_t *>(base)), mid(static_cast<uint16_t *>(base) + rows * LD),
+              lo(static_cast<uint16_t *>(base) + 2 * rows * LD) {}
+    };
+    struct A { s16x4 hi, mid, lo; };
+    struct B { s16x4 hi, mid, lo; };
+
+    // bit patterns of the three parts of x, each in the upper half of a word
+    __device__ static __forceinline__ void cut(float x, uint32_t &h, uint32_t &m, uint32_t &l) {
+        const float r1 = x - bf_hi_part(x), r2 = r1 - bf_hi_part(r1);
+        h = __float_as_uint(x);
+        m = __float_as_uint(r1);
+        l = __float_as_uint(r2);
+    }
+    __device__ static __forceinline__ void cut4(const float x[4], uint2 &h, uint2 &m, uint2 &l) {
+        uint32_t hb[4], mb[4], lb[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) cut(x[j], hb[j], mb[j], lb[j]);
+        h = make_uint2(pack_hi16(hb[0], hb[1]), pack_hi16(hb[2], hb[3]));
+        m = make_uint2(pack_hi16(mb[0], mb[1]), pack_hi16(mb[2], mb[3]));
+        l = make_uint2(pack_hi16(lb[0], lb[1]), pack_hi16(lb[2], lb[3]));
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ A lda(const Mat<LD, SP> &m, int row, int k) {
+        const int o = row * LD + k;
+        return A{PrecBf16::rd4(m.hi + o), PrecBf16::rd4(m.mid + o), PrecBf16::rd4(m.lo + o)};
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ A lda_t(const Mat<LD, SP> &m, int k, int col) {
+        return A{PrecBf16::rd4t<LD>(m.hi, k, col), PrecBf16::rd4t<LD>(m.mid, k, col), PrecBf16::rd4t<LD>(m.lo, k, col)};
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ B ldb(const Mat<LD, SP> &m, int n, int k) {
+        const int o = n * LD + k;
+        return B{PrecBf16::rd4(m.hi + o), PrecBf16::rd4(m.mid + o), PrecBf16::rd4(m.lo + o)};
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ B ldb_t(const Mat<LD, SP> &m, int k, int n) {
+        return B{PrecBf16::rd4t<LD>(m.hi, k, n), PrecBf16::rd4t<LD>(m.mid, k, n), PrecBf16::rd4t<LD>(m.lo, k, n)};
+    }
+    __device__ static __forceinline__ B accb(const f32x4 &x) {
+        const float v[4] = {x[0], x[1], x[2], x[3]};
+        uint2 h, m, l;
+        cut4(v, h, m, l);
+        return B{__builtin_bit_cast(s16x4, h), __builtin_bit_cast(s16x4, m), __builtin_bit_cast(s16x4, l)};
+    }
+    __device__ static __forceinline__ B accb_exact(const f32x4 &x) { return accb(x); }
+    __device__ static __forceinline__ B negb(const B &b) {
+        const auto flip = [](const s16x4 &v) {
+            const uint2 u = __builtin_bit_cast(uint2, v);
+            return __builtin_bit_cast(s16x4, make_uint2(u.x ^ 0x80008000u, u.y ^ 0x80008000u));
+        };
+        return B{flip(b.hi), flip(b.mid), flip(b.lo)};
+    }
+    // one group of 16 contraction indices: two partial products side by side per instruction, the
+    // small ones first.  SA / SB are ignored: fp32 inputs are not bf16 numbers either.
+    template <bool SA, bool SB>
+    __device__ static __forceinline__ f32x4 mma(const A &a, const B &b, f32x4 acc) {
+        const bf16x8 bhm = PrecBf16::cat(b.hi, b.mid);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PrecBf16::cat(a.hi, a.lo), PrecBf16::cat(b.lo, b.hi), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PrecBf16::cat(a.mid, a.mid), bhm, acc, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(PrecBf16::cat(a.hi, a.hi), bhm, acc, 0, 0, 0);
+    }
+    template <bool SA, bool SB>
+    __device__ static __forceinline__ f32x4 mma2(const A &a0, const A &a1, const B &b0, const B &b1, f32x4 acc) {
+        const bf16x8 ah = PrecBf16::cat(a0.hi, a1.hi), am = PrecBf16::cat(a0.mid, a1.mid);
+        const bf16x8 bh = PrecBf16::cat(b0.hi, b1.hi), bm = PrecBf16::cat(b0.mid, b1.mid);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(PrecBf16::cat(a0.lo, a1.lo), bh, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, PrecBf16::cat(b0.lo, b1.lo), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am, bm, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(am, bh, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, bm, acc, 0, 0, 0);
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(ah, bh, acc, 0, 0, 0);
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ void st(const Mat<LD, SP> &m, int row, int col, float v) {
+        uint32_t h, md, l;
+        cut(v, h, md, l);
+        const int o = row * LD + col;
+        m.hi[o] = (uint16_t)(h >> 16);
+        m.mid[o] = (uint16_t)(md >> 16);
+        m.lo[o] = (uint16_t)(l >> 16);
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ void st4(const Mat<LD, SP> &m, int row, int col, const float4 &v) {
+        const float x[4] = {v.x, v.y, v.z, v.w};
+        uint2 h, md, l;
+        cut4(x, h, md, l);
+        const int o = row * LD + col;
+        *reinterpret_cast<uint2 *>(m.hi + o) = h;
+        *reinterpret_cast<uint2 *>(m.mid + o) = md;
+        *reinterpret_cast<uint2 *>(m.lo + o) = l;
+    }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ float ld(const Mat<LD, SP> &m, int row, int col) {
+        const int o = row * LD + col;
+        return __uint_as_float((uint32_t)m.hi[o] << 16) + __uint_as_float((uint32_t)m.mid[o] << 16) +
+               __uint_as_float((uint32_t)m.lo[o] << 16);
+    }
+    typedef float4 Raw4;
+    __device__ static __forceinline__ Raw4 ld_raw(const float *g) { return *reinterpret_cast<const float4 *>(g); }
+    __device__ static __forceinline__ Raw4 keep_raw(const Raw4 &v, bool keep) { return PrecF32::keep_raw(v, keep); }
+    __device__ static __forceinline__ float4 raw_f32(const Raw4 &v) { return v; }
+    template <int LD, bool SP>
+    __device__ static __forceinline__ void st_raw(const Mat<LD, SP> &m, int row, int col, const Raw4 &v) {
+        st4(m, row, col, v);
+    }
+};
+
 // Raw bits of one input element and their fp32 value: loads keep the bits, the conversion is
 // done where the value is used, so that a prefetch does not wait for its own loads.
 __device__ __forceinline__ uint32_t ld_bits(const float *p) { return __float_as_uint(*p); }
@@ -291,9 +417,11 @@ __device__ __forceinline__ float bits_f32(uint32_t b) {
     else return __uint_as_float(b);
 }
 
-// fp32 inputs multiply in fp32; bf16 inputs (16-bit patterns) multiply in bf16
-template <class TI> struct PrecOf { typedef PrecF32 type; };
-template <> struct PrecOf<uint16_t> { typedef PrecBf16 type; };
+// bf16 inputs (16-bit patterns) multiply in bf16; fp32 inputs as three bf16 parts where the LDS
+// holds the three planes of every operand matrix (D = 64), in fp32 otherwise
+template <class TI, int D> struct PrecOf { typedef PrecF32 type; };
+template <> struct PrecOf<float, 64> { typedef PrecBf16x3 type; };
+template <int D> struct PrecOf<uint16_t, D> { typedef PrecBf16 type; };
 
 __device__ __forceinline__ uint32_t f2bf_rne(float f) {
     const uint32_t u = __float_as_uint(f);

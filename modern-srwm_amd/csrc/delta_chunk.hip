@@ -52,7 +52,7 @@ struct ChunkFwdP {
 // its partial K S and Q S through LDS.
 template <class TI, int D, int KS>
 struct FwdLds {
-    typedef typename PrecOf<TI>::type X;
+    typedef typename PrecOf<TI, D>::type X;
     static constexpr int LDK = D + X::kPad, LDA = kC + X::kPad, LDD = 16 + X::kPad, LDV = kMC + 4;
     typedef typename X::template Mat<LDK, false> MatK;   // K, Q: the inputs themselves
     typedef typename X::template Mat<LDA, true> MatA;    // A, B: computed
@@ -329,7 +329,7 @@ int dispatch_chunk(const ChunkFwdP<TI> &p, int D, hipStream_t s) {
     if (!rows_ok(p.Q, p.qs) || !rows_ok(p.K, p.ks) || !rows_ok(p.V, p.vs)) return -1;
     if ((int64_t)(p.L + kC) * D * 4 > (int64_t)UINT32_MAX) return -1;   // 32-bit byte offsets inside a sequence
     switch (D) {
-        case 128: return launch_chunk<TI, 128, 2, PrecOf<TI>::type::kBf ? 2 : 1>(p, s);
+        case 128: return launch_chunk<TI, 128, 2, PrecOf<TI, 128>::type::kBf ? 2 : 1>(p, s);
         case 64: return launch_chunk<TI, 64, 1, 1>(p, s);
         default: return -1;
     }

@@ -62,7 +62,7 @@ struct ChunkBwdP {
 // partial K dS' through LDS.
 template <class TI, int D, int KS>
 struct ColLds {
-    typedef typename PrecOf<TI>::type X;
+    typedef typename PrecOf<TI, D>::type X;
     static constexpr int C = 64;
     static constexpr int LDK = D + X::kPad, LDA = C + X::kPad, LDD = 16 + X::kPad;
     typedef typename X::template Mat<LDK, false> MatK;
@@ -336,7 +336,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 // ------------------------------------------------------------------------------------------
 template <class TI, int D, int C>
 struct RowLds {
-    typedef typename PrecOf<TI>::type X;
+    typedef typename PrecOf<TI, D>::type X;
     static constexpr int LDM = D + X::kPad, LDW = kWC + X::kPad, LDC = C + X::kPad;
     typedef typename X::template Mat<LDM, false> MatG;   // dOut: an input
     typedef typename X::template Mat<LDM, true> MatU;    // U, Y: computed
@@ -644,10 +644,10 @@ int dispatch_chunk_bwd(const ChunkBwdP<TI> &p, int D, hipStream_t s) {
         !ok16(p.vold) || !ok16(p.vins) || !ok16(p.W) || !ok16(p.gV) || !ok16(p.gQ) || !ok16(p.gK) ||
         (p.gW && !ok16(p.gW)))
         return -1;
-    constexpr bool bf = PrecOf<TI>::type::kBf;
+    constexpr bool bf = PrecOf<TI, 128>::type::kBf;
     switch (D) {
         case 128: return launch_chunk_bwd<TI, 128, 2, bf ? 64 : 32, bf ? 2 : 1, 2>(p, s);
-        case 64: return launch_chunk_bwd<TI, 64, 1, 64, 1, 2>(p, s);
+        case 64: return launch_chunk_bwd<TI, 64, 1, sizeof(TI) == 2 ? 64 : 32, 1, 2>(p, s);
         default: return -1;
     }
 }
