@@ -5,8 +5,10 @@
 //     (I + strict_lower(diag(beta) A)) U = diag(beta) (V - P)        U rows = v_insert
 //     v_old = P + strict_lower(A) U,   out = Q S + tril(B) U,   S' = S + K^T U
 // which is the per-step recurrence unrolled over the chunk (same results as the sequential
-// kernel up to fp32 summation order).  Every product is a v_mfma_f32_16x16x4f32 (fp32 in,
-// fp32 accumulate), so the fp32 parity bar of the sequential kernels applies here too.
+// kernel up to fp32 summation order).  With fp32 inputs every product keeps fp32 accuracy -- at
+// D = 64 as six bf16 partial products of three-part operands (PrecBf16x3 in chunk_mma.h), at
+// D = 128 as v_mfma_f32_16x16x4f32 -- so the fp32 parity bar of the sequential kernels applies
+// here too; bf16 inputs multiply as hi/lo bf16 pairs (PrecBf16).
 //
 // One workgroup = 4 waves = 64 columns of the memory of one sequence (D = 128: two workgroups
 // per sequence; columns never interact).  Wave w keeps its 16 columns of S in registers in the

@@ -21,10 +21,12 @@
 //                 it reads grad_V back, forms G1 and X cooperatively and writes grad_Q, grad_K,
 //                 the reverted memory and the gradient of the initial memory.  Every word of
 //                 grad_Q / grad_K has one writer: no atomics.
-// Both sweeps revert S and accumulate dS on their own (one extra product each, cheaper than
-// moving the memory between the two layouts every chunk).  With fp32 inputs every product is
-// v_mfma_f32_16x16x4f32; with bf16 inputs it is v_mfma_f32_16x16x32_bf16 on hi/lo split
-// operands (chunk_mma.h), accumulation in fp32 either way.
+// Both sweeps accumulate dS on their own and the row sweep also reverts S (cheaper than moving
+// the memory between the two layouts every chunk; the column sweep needs no S at all).  With fp32
+// inputs a product is six v_mfma_f32_16x16x32_bf16 on three-part operands at D = 64 (fp32
+// accuracy; the row sweep then runs chunks of 32 steps so that the three planes of its operand
+// matrices fit the LDS) and v_mfma_f32_16x16x4f32 at D = 128; with bf16 inputs it is
+// v_mfma_f32_16x16x32_bf16 on hi/lo split operands (chunk_mma.h); accumulation in fp32 always.
 //
 // Replaces fast_weight_backward_value_beta_kernel and fast_weight_backward_query_key_kernel of
 // the reference (supervised_learning/fast_weight/fast_weight_cuda.cu:397-560, :244-393) for
@@ -113,26 +115,20 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
     const TI *gob = p.go + n * p.gs.n + h * p.gs.h + m0 + ln;
     const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
     const float *vob = p.vold + seq * p.L * D + m0 + ln;
-    const float *vib = p.vins + seq * p.L * D + m0 + ln;
-    const float *Wg = p.W + seq * D * D + m0 + ln;
     const float *gWg = (p.gW && p.grad_state_mode != 0u) ? p.gW + seq * D * D + m0 + ln : nullptr;
 
-    // 16 columns of the memory (exit value of the last chunk) and of its gradient
-    f32x4 s[EB], ds[EB];
+    // 16 columns of the gradient of the memory (this sweep needs no value of the memory itself)
+    f32x4 ds[EB];
 #pragma unroll
     for (int eb = 0; eb < EB; ++eb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const int o = (e0 + eb * 16 + 4 * lq + r) * D;
-            s[eb][r] = Wg[o];
-            ds[eb][r] = gWg ? gWg[o] : 0.f;
-        }
+        for (int r = 0; r < 4; ++r) ds[eb][r] = gWg ? gWg[(e0 + eb * 16 + 4 * lq + r) * D] : 0.f;
 
-    // next chunk's inputs: K, Q rows for LDS; U, dOut, V, v_old directly in accumulator layout
+    // next chunk's inputs: K, Q rows for LDS; dOut, V, v_old directly in accumulator layout
     constexpr int NKQ = C * (D / 4) / NT;
     typename X::Raw4 kreg[NKQ], qreg[NKQ];
     // V and v_old only enter grad_beta: a wave loads them for the row blocks whose results it stores
-    f32x4 pu[CB], po[CB / KS];
+    f32x4 po[CB / KS];
     uint32_t pg[CB][4], pv[CB / KS][4], breg = 0u;   // raw bits, converted in commit()
     auto prefetch = [&](int ch) {
         const int t0 = ch * C;
@@ -148,7 +144,6 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int64_t t = min(t0 + cb * 16 + 4 * lq + r, p.L - 1);
-                pu[cb][r] = vib[t * D];
                 pg[cb][r] = ld_bits(gob + t * p.gs.l);
             }
 #pragma unroll
@@ -161,7 +156,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
             }
         breg = ld_bits(bb + (int64_t)min(t0 + (tid % C), p.L - 1) * p.bs.l);
     };
-    f32x4 u[CB], g[CB], vd[CB / KS];   // this chunk: U, dOut, V - v_old (rows past the end zeroed)
+    f32x4 g[CB], vd[CB / KS];   // this chunk: dOut, V - v_old (rows past the end zeroed)
     auto commit = [&](int ch) {
         const int t0 = ch * C;
         const bool full = t0 + C <= p.L;
@@ -177,7 +172,6 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const float m = (full || t0 + cb * 16 + 4 * lq + r < p.L) ? 1.f : 0.f;
-                u[cb][r] = pu[cb][r] * m;
                 g[cb][r] = bits_f32<TI>(pg[cb][r]) * m;
             }
 #pragma unroll
@@ -242,23 +236,15 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
             for (int r = 0; r < 4; ++r) X::st(Di, wave * 16 + 4 * lq + r, ln, inv[r]);
         }
 
-        // ---- independent of the inversion: revert S, dU = K dS' + tril(Q K^T)^T dOut
+        // ---- independent of the inversion: dU = K dS' + tril(Q K^T)^T dOut
         typename X::B gob_[CB];
         f32x4 du[CB];
         {
-            typename X::B nub[CB], dsb[EB];
+            typename X::B dsb[EB];
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
-                nub[cb] = X::accb(-u[cb]);
-                gob_[cb] = X::accb_exact(g[cb]);
-            }
+            for (int cb = 0; cb < CB; ++cb) gob_[cb] = X::accb_exact(g[cb]);
 #pragma unroll
             for (int eb = 0; eb < EB; ++eb) dsb[eb] = X::accb(ds[eb]);
-#pragma unroll
-            for (int eb = 0; eb < EB; ++eb)
-                s[eb] = mma_range<X, false, true>(
-                    0, CB, [&](int cb) { return X::lda_t(Ks, cb * 16 + 4 * lq, e0 + eb * 16 + ln); },
-                    [&](int cb) { return nub[cb]; }, s[eb]);
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) {
                 du[cb] = mma_range<X, false, true>(

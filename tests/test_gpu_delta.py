@@ -241,6 +241,8 @@ def test_two_workgroups_per_sequence_with_a_ragged_sequence_count():
     ((2, 8, 256, 64, 64), "softmax", 0.0, torch.float32),    # benchmark configuration 2 style
     ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # benchmark configuration 5 style, shorter
     ((2, 2, 200, 64, 64), "softmax", 0.2, torch.bfloat16),   # bf16 at D = 64 (four waves, one workgroup per sequence)
+    ((2, 2, 1000, 64, 64), "softmax", 0.5, torch.float32),   # three-part bf16 operands over 16 chunks, large memory
+    ((1, 2, 777, 64, 64), "l2", 0.5, torch.float32),         # the same with unit-norm keys
 ])
 def test_chunkwise_forward_matches_oracle_and_feeds_the_sequential_backward(shape, qk, w0, io):
     """Chunkwise (C = 64) MFMA forward vs the fp64 oracle, then the step-by-step backward run on
@@ -282,6 +284,8 @@ def test_chunkwise_forward_matches_oracle_and_feeds_the_sequential_backward(shap
     ((2, 2, 300, 64, 64), "softmax", 0.2, torch.bfloat16),
     ((1, 2, 512, 128, 128), "l2", 0.0, torch.bfloat16),      # benchmark configuration 5 style, shorter
     ((1, 2, 150, 128, 128), "l2", 0.3, torch.bfloat16),
+    ((2, 2, 1000, 64, 64), "softmax", 0.5, torch.float32),   # three-part bf16 operands, row sweep in chunks of 32
+    ((1, 2, 777, 64, 64), "l2", 0.5, torch.float32),
 ])
 @pytest.mark.parametrize("state_grad", [False, True])
 def test_chunkwise_backward_matches_oracle(shape, qk, w0, io, state_grad):
@@ -320,18 +324,22 @@ def test_chunkwise_backward_matches_oracle(shape, qk, w0, io, state_grad):
     assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
 
 
-@pytest.mark.parametrize("D,L", [(64, 70), (64, 200), (128, 70), (128, 200), (128, 1024)])
-def test_chunkwise_bf16_runs_are_bit_identical_and_match_the_oracle(D, L):
-    """The matrix-core kernels with bf16 inputs (forward, column sweep, row sweep) at ragged lengths:
-    six runs of forward + backward must agree bit for bit (every word has one writer or meets through
-    a two-addend atomic sum, and no result may depend on instruction timing), and the first run must
-    match the fp64 oracle on the rounded inputs."""
-    print(f"case chunkwise bf16 determinism D={D} L={L}", flush=True)
+@pytest.mark.parametrize("D,L,io", [(64, 70, torch.bfloat16), (64, 200, torch.bfloat16), (128, 70, torch.bfloat16),
+                                    (128, 200, torch.bfloat16), (128, 1024, torch.bfloat16),
+                                    (64, 70, torch.float32), (64, 300, torch.float32), (128, 200, torch.float32)])
+def test_chunkwise_runs_are_bit_identical_and_match_the_oracle(D, L, io):
+    """The matrix-core kernels (forward, column sweep, row sweep) at ragged lengths, with bf16 inputs
+    (hi/lo bf16 operands) and with fp32 inputs (three-part bf16 operands at D = 64, fp32 matrix
+    instructions at D = 128): six runs of forward + backward must agree bit for bit (every word has one
+    writer or meets through a two-addend atomic sum, and no result may depend on instruction timing),
+    and the first run must match the fp64 oracle on the inputs as the kernel sees them."""
+    print(f"case chunkwise determinism D={D} L={L} io={io}", flush=True)
     import srwm_hip
     dev = _dev()
     N, H = 2, 3
+    tol = TOL if io == torch.float32 else BF16_TOL
     q, k, v, beta, W0, go = delta_inputs(N, H, L, D, D, seed=23, qk="l2", w0_std=0.2)
-    qi, ki, vi, bi, goi = (t.to(torch.bfloat16) for t in (q, k, v, beta, go))
+    qi, ki, vi, bi, goi = (t.to(io) for t in (q, k, v, beta, go))
     base = [t.to(torch.float64).numpy() for t in (qi, ki, vi, bi)] + [W0.numpy()]
     of = oracle.delta_forward(*base)
     ob = oracle.delta_backward(*base[:4], of, goi.to(torch.float64).numpy(), want_grad_W=True)
@@ -340,7 +348,7 @@ def test_chunkwise_bf16_runs_are_bit_identical_and_match_the_oracle(D, L):
     runs = []
     for rep in range(6):
         W = W0.to(dev, torch.float32).contiguous()
-        vold, vins, out = nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, D, dt=torch.bfloat16)
+        vold, vins, out = nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, D, dt=io)
         srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out, flags=srwm_hip.FLAG_CHUNKWISE)
         WL = W.clone()
         gq, gk, gv, gb, gW = nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, D), nan(N, H, L, 1), nan(N, H, D, D)
@@ -357,8 +365,8 @@ def test_chunkwise_bf16_runs_are_bit_identical_and_match_the_oracle(D, L):
     r = runs[0]
     errs = {n: rel_err(r[n].float().cpu().numpy(), of[n]) for n in ("out", "v_old", "v_insert", "W")}
     errs.update({n: rel_err(r[n].cpu().numpy(), ob[n]) for n in ("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W")})
-    bad = {n: e for n, e in errs.items() if not (e < BF16_TOL)}
-    assert not bad, f"over tolerance {BF16_TOL}: {bad}  (all: {errs})"
+    bad = {n: e for n, e in errs.items() if not (e < tol)}
+    assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
 
 
 def test_full_config5_properties():
