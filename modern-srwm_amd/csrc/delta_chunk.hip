@@ -226,11 +226,12 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
                     f32x4{0.f, 0.f, 0.f, 0.f});
             }
         }
-        if constexpr (KS == 2) {   // hand the partial products to the wave that holds the other rows
+        if constexpr (KS == 2) {   // hand the partial products to the wave that holds the other rows:
+                                   // K S of every row block, Q S of the row blocks whose outputs the other wave forms
 #pragma unroll
             for (int cb = 0; cb < kCB; ++cb) {
                 Xs[(wv * 2 * kCB + cb) * 64 + lane] = pt[cb];
-                Xs[(wv * 2 * kCB + kCB + cb) * 64 + lane] = ot[cb];
+                if (cb % KS != hf) Xs[(wv * 2 * kCB + kCB + cb) * 64 + lane] = ot[cb];
             }
         }
         __syncthreads();   // the four inverses (and the partial products) are visible
@@ -239,9 +240,9 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
 #pragma unroll
             for (int cb = 0; cb < kCB; ++cb) {
                 // both waves of a pair add in the same order (lower rows first): identical results
-                const f32x4 a = Xs[(ow * 2 * kCB + cb) * 64 + lane], b = Xs[(ow * 2 * kCB + kCB + cb) * 64 + lane];
+                const f32x4 a = Xs[(ow * 2 * kCB + cb) * 64 + lane];
                 pt[cb] = hf == 0 ? pt[cb] + a : a + pt[cb];
-                ot[cb] = hf == 0 ? ot[cb] + b : b + ot[cb];
+                if (cb % KS == hf) ot[cb] += Xs[(ow * 2 * kCB + kCB + cb) * 64 + lane];
             }
         }
 
@@ -262,11 +263,11 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
             u[a] = X::template mma<true, true>(X::lda(Di, a * 16 + ln, 4 * lq), X::accb(rhs),
                                                f32x4{0.f, 0.f, 0.f, 0.f});
             ub[a] = X::accb(u[a]);
-            y = X::template mma<true, true>(X::lda(As, a * 16 + ln, a * 16 + 4 * lq), ub[a], y);   // + strict_lower(A_aa) U_a
-            // out = Q S + tril(B) U
-            ot[a] = mma_range<X, true, true>(
-                0, a + 1, [&](int b) { return X::lda(Bs, a * 16 + ln, b * 16 + 4 * lq); }, fu, ot[a]);
-            if (a % KS == hf) {   // the two waves of a pair share the stores
+            if (a % KS == hf) {   // the two waves of a pair share the outputs: each forms and stores every other row block
+                y = X::template mma<true, true>(X::lda(As, a * 16 + ln, a * 16 + 4 * lq), ub[a], y);   // + strict_lower(A_aa) U_a
+                // out = Q S + tril(B) U
+                ot[a] = mma_range<X, true, true>(
+                    0, a + 1, [&](int b) { return X::lda(Bs, a * 16 + ln, b * 16 + 4 * lq); }, fu, ot[a]);
                 // one 32-bit byte offset per lane from the sequence's (uniform) base; the rows of the
                 // block follow at compile-time distances
                 const uint32_t o0 = (uint32_t)(((t0 + a * 16 + 4 * lq) * D + m0 + cw + ln) * 4);
