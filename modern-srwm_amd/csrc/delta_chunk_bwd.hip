@@ -320,7 +320,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 // ------------------------------------------------------------------------------------------
 // Row sweep
 // ------------------------------------------------------------------------------------------
-template <class TI, int D, int C>
+template <class TI, int D, int C, int KS>
 struct RowLds {
     typedef typename PrecOf<TI, D>::type X;
     static constexpr int LDM = D + X::kPad, LDW = kWC + X::kPad, LDC = C + X::kPad;
@@ -335,7 +335,8 @@ struct RowLds {
     static constexpr int oQ = oK + MatK::bytes(C);
     static constexpr int oG1 = oQ + MatK::bytes(C);
     static constexpr int oZ = oG1 + MatC::bytes(C);
-    static constexpr int kBytes = oZ + MatC::bytes(C);
+    static constexpr int oX2 = oZ + MatC::bytes(C);           // KS == 2: [8 waves][C/16/KS tiles][64 lanes] f32x4
+    static constexpr int kBytes = oX2 + (KS == 2 ? 8 * (C / 16 / KS) * 64 * 16 : 0);
     static_assert(MatG::bytes(C) % 16 == 0 && MatU::bytes(C) % 16 == 0 && MatK::bytes(C) % 16 == 0 &&
                       MatC::bytes(C) % 16 == 0, "alignment");
 };
@@ -343,11 +344,12 @@ struct RowLds {
 // KS = 2: 8 waves; a pair of waves owns the same 16 memory rows and splits their columns (the
 // contraction index of dOut S^T, U dS'^T, Y S^T) in halves.  Each computes its half of those
 // products for the whole chunk, hands the part belonging to the other's half of the chunk over
-// through LDS (the K / Q slices are dead by then: their fragments sit in registers), and finishes
-// grad_Q, grad_K for its own half of the chunk.
+// through LDS (the grad_Q part over the K / Q slices, which are dead by then: their fragments sit
+// in registers; the grad_K part through a buffer of its own, so that one barrier serves both), and
+// finishes grad_Q, grad_K for its own half of the chunk.
 template <class TI, int D, int MS, int C, int KS>
 __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(ChunkBwdP<TI> p) {
-    typedef RowLds<TI, D, C> Lds;
+    typedef RowLds<TI, D, C, KS> Lds;
     typedef typename Lds::X X;
     constexpr int NT = kThreads * KS;
     constexpr int CB = C / 16, MBF = D / 16, MB = MBF / KS, NTRI = CB * (CB + 1) / 2;   // MB: column blocks held by a wave
@@ -361,6 +363,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     const typename Lds::MatC G1(smem + Lds::oG1, C), Z(smem + Lds::oZ, C);
 
     f32x4 *Xs = reinterpret_cast<f32x4 *>(smem + Lds::oK);   // KS == 2: [8 waves][CBH tiles][64 lanes]
+    f32x4 *Xs2 = reinterpret_cast<f32x4 *>(smem + Lds::oX2);
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
     const int wave = wv & 3, hf = wv >> 2;           // row block, column half
@@ -546,22 +549,18 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
                 Xs[(wv * CBH + j) * 64 + lane] = hf ? pq[j] : pq[CBH + j];
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) pk[cb] = dk_state(cb);
-            __syncthreads();
-            f32x4 oq[CBH];
 #pragma unroll
-            for (int j = 0; j < CBH; ++j) oq[j] = Xs[((wv ^ 4) * CBH + j) * 64 + lane];
-            __syncthreads();
-#pragma unroll
-            for (int j = 0; j < CBH; ++j) Xs[(wv * CBH + j) * 64 + lane] = hf ? pk[j] : pk[CBH + j];
+            for (int j = 0; j < CBH; ++j) Xs2[(wv * CBH + j) * 64 + lane] = hf ? pk[j] : pk[CBH + j];
             __syncthreads();
             if (hf == 0) {
 #pragma unroll
                 for (int j = 0; j < CBH; ++j)
-                    finish(j, pq[j] + oq[j], pk[j] + Xs[((wv ^ 4) * CBH + j) * 64 + lane]);
+                    finish(j, pq[j] + Xs[((wv ^ 4) * CBH + j) * 64 + lane], pk[j] + Xs2[((wv ^ 4) * CBH + j) * 64 + lane]);
             } else {
 #pragma unroll
                 for (int j = 0; j < CBH; ++j)
-                    finish(CBH + j, pq[CBH + j] + oq[j], pk[CBH + j] + Xs[((wv ^ 4) * CBH + j) * 64 + lane]);
+                    finish(CBH + j, pq[CBH + j] + Xs[((wv ^ 4) * CBH + j) * 64 + lane],
+                           pk[CBH + j] + Xs2[((wv ^ 4) * CBH + j) * 64 + lane]);
             }
         }
         // ---- dS^T += dOut^T Q - Y^T K
@@ -606,7 +605,7 @@ __global__ void zero_words_kernel(float *a, int64_t n) {
 // KS: waves per memory row / column block in the column sweep, KSR: in the row sweep
 template <class TI, int D, int MS, int C2, int KS, int KSR>
 int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
-    constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2>::kBytes;
+    constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2, KSR>::kBytes;
     static_assert(lds1 <= (int)kMaxLdsBytes && lds2 <= (int)kMaxLdsBytes, "LDS budget");
     if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_col_kernel<TI, D, MS, KS>>()) return err;
     if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR>>()) return err;
