@@ -530,8 +530,42 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     // loop is unrolled by two, which makes the parity (and with it every buffer address) a
     // compile-time constant.
     constexpr int NPAR = 2;
+    // Below E = 64 the partial sums of one row lie side by side (part index fastest), so that the lane that
+    // adds them up fetches them with two wide reads -- they sit on the serial chain of a step there.  At
+    // E = 64 the row index is the fastest one: a wave's reduction then stores pairs of rows with one
+    // instruction, which matters more to that issue-bound kernel than the number of reads.
+    constexpr bool HT = E < kWave;
+    constexpr int NXP = NXS <= 4 ? 4 : 8;                                 // narrow columns, padded to whole float4s
     __shared__ __attribute__((aligned(16))) float rowm[NPAR][3][NW][E];   // row sums per wave: G ins | W gdiff | W gpre
-    __shared__ __attribute__((aligned(16))) float rowb[NPAR][3][NXS][E];  // same, contribution of the narrow columns
+    __shared__ __attribute__((aligned(16))) float rowb[NPAR][3][HT ? NXP : NXS][E];  // same, contribution of the narrow columns
+    float(*const rowmT)[3][E][NW] = reinterpret_cast<float(*)[3][E][NW]>(rowm);     // the views used when HT
+    float(*const rowbT)[3][E][NXP] = reinterpret_cast<float(*)[3][E][NXP]>(rowb);
+    // sum of the NW + NXS parts of row e
+    const auto row_total = [&](const int pp, const int which, const int e) {
+        float s;
+        if constexpr (HT) {
+            float pm[NW], pb[4];
+            lds_read_vec<NW>(pm, &rowmT[pp][which][e][0]);
+            lds_read_vec<4>(pb, &rowbT[pp][which][e][0]);
+            s = pm[0];
+#pragma unroll
+            for (int wv = 1; wv < NW; ++wv) s += pm[wv];
+            s += (pb[0] + pb[1]) + (pb[2] + pb[3]);
+            if constexpr (NXS > 4) s += rowbT[pp][which][e][4];
+        } else {
+            s = rowm[pp][which][0][e];
+#pragma unroll
+            for (int wv = 1; wv < NW; ++wv) s += rowm[pp][which][wv][e];
+#pragma unroll
+            for (int j = 0; j < NXS; ++j) s += rowb[pp][which][j][e];
+        }
+        return s;
+    };
+    // this thread's narrow-column part of row e
+    const auto put_narrow = [&](const int pp, const int which, const int e, const int j, const float v) {
+        if constexpr (HT) rowbT[pp][which][e][j] = v;
+        else rowb[pp][which][j][e] = v;
+    };
     __shared__ __attribute__((aligned(16))) float gbp[NPAR][NCG][4];      // per column group: sum gins*diff per beta
     __shared__ __attribute__((aligned(16))) float gbp3[NPAR][8];          // same for the narrow columns
     __shared__ __attribute__((aligned(16))) float exch[NW][2][E];   // per wave: g_pre of the q | k block
@@ -542,6 +576,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     const int el = lane % E;
     const int jb = tid / E;
     const bool has_b = jb < 4;
+    // a wave's reduce-scattered row sums (rows r0 .. r0 + R - 1) into its slots
+    const auto put_rows = [&](const float(&v)[R], const int pp, const int which) {
+        if constexpr (HT) stride8_reduce_scatter<R, NW>(v, &rowmT[pp][which][r0][wave], lane);
+        else stride8_reduce_store<R>(v, &rowm[pp][which][wave][r0], lane);
+    };
 
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
@@ -657,11 +696,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     // element of the softmaxed x_t)
     auto finish_gx = [&](int t, int pp, float xs) {
         if (tid < E) {
-            float s = rowm[pp][2][0][tid];
-#pragma unroll
-            for (int wv = 1; wv < NW; ++wv) s += rowm[pp][2][wv][tid];
-#pragma unroll
-            for (int j = 0; j < NXS; ++j) s += rowb[pp][2][j][tid];
+            float s = row_total(pp, 2, tid);
             if (softmax_x) s = xs * (s - group_sum<E>(s * xs));   // tid < E covers whole lane groups
             p.gx[(seq * p.L + t) * E + tid] = s;
         }
@@ -793,17 +828,17 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                     u[i] = fmaf(w[i][c], gdif[c], u[i]);
                 }
             }
-            stride8_reduce_store<R>(a, &rowm[par][0][wave][r0], lane);
-            stride8_reduce_store<R>(u, &rowm[par][1][wave][r0], lane);
+            put_rows(a, par, 0);
+            put_rows(u, par, 1);
             if (has_b) {
-                rowb[par][0][jb][el] = gbe * insb;
-                rowb[par][1][jb][el] = wbe * gdifb;
+                put_narrow(par, 0, el, jb, gbe * insb);
+                put_narrow(par, 1, el, jb, wbe * gdifb);
                 if (el == 0) gbp3[par][jb] = ginsb * bd;
             }
             if constexpr (XC) {
                 if (has_y) {
-                    rowb[par][0][4][el] = gye * insy;
-                    rowb[par][1][4][el] = wye * gdify;
+                    put_narrow(par, 0, el, 4, gye * insy);
+                    put_narrow(par, 1, el, 4, wye * gdify);
                     if (el == 0) gbp3[par][4] = ginsy * ydl;
                 }
             }
@@ -818,26 +853,27 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             if constexpr (HALF) {
                 // lane l and lane l + 32 would form the same two sums: each half forms one of them
                 const int sel = lane >> 5;   // 0: W g_diff (-> gq), 1: G ins (-> gk)
-                float part = rowm[par][1 - sel][0][el];
-#pragma unroll
-                for (int wv = 1; wv < NW; ++wv) part += rowm[par][1 - sel][wv][el];
-#pragma unroll
-                for (int j = 0; j < NXS; ++j) part += rowb[par][1 - sel][j][el];
+                const float part = row_total(par, 1 - sel, el);
                 gq = part;
                 gk = part;
                 swap_pairs<32>(gq, gk);   // gq: the lower half's sum in both halves, gk: the upper half's
             } else {
-                gk = rowm[par][0][0][el];
-                gq = rowm[par][1][0][el];
+                if constexpr (HT) {
+                    gk = row_total(par, 0, el);
+                    gq = row_total(par, 1, el);
+                } else {
+                    gk = rowm[par][0][0][el];
+                    gq = rowm[par][1][0][el];
 #pragma unroll
-                for (int wv = 1; wv < NW; ++wv) {
-                    gk += rowm[par][0][wv][el];
-                    gq += rowm[par][1][wv][el];
-                }
+                    for (int wv = 1; wv < NW; ++wv) {
+                        gk += rowm[par][0][wv][el];
+                        gq += rowm[par][1][wv][el];
+                    }
 #pragma unroll
-                for (int j = 0; j < NXS; ++j) {
-                    gk += rowb[par][0][j][el];
-                    gq += rowb[par][1][j][el];
+                    for (int j = 0; j < NXS; ++j) {
+                        gk += rowb[par][0][j][el];
+                        gq += rowb[par][1][j][el];
+                    }
                 }
             }
             gk -= gq;
@@ -895,10 +931,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 #pragma unroll
                 for (int c = 0; c < NC; ++c) sx[i] = fmaf(w[i][c], gpre[c], sx[i]);
             }
-            stride8_reduce_store<R>(sx, &rowm[par][2][wave][r0], lane);
-            if (has_b) rowb[par][2][jb][el] = wbe * gpreb;
+            put_rows(sx, par, 2);
+            if (has_b) put_narrow(par, 2, el, jb, wbe * gpreb);
             if constexpr (XC) {
-                if (has_y) rowb[par][2][4][el] = wye * gprey;
+                if (has_y) put_narrow(par, 2, el, 4, wye * gprey);
             }
             // the grad_x partials are summed one step later, behind the next step's barrier: no barrier of their own
             if (t + 1 < p.L) finish_gx(t + 1, par ^ 1, xb_prev);

@@ -238,6 +238,28 @@ __device__ __forceinline__ void stride8_reduce_store(const float (&v)[R], float 
     }
 }
 
+// The same reduction with the results scattered: result i goes to dst[i * STRIDE] (a matrix kept
+// with the reduced index as its row, so that a reader finds all the partial sums of one row side by
+// side).
+template <int R, int STRIDE>
+__device__ __forceinline__ void stride8_reduce_scatter(const float (&v)[R], float *dst, int lane) {
+    constexpr int NA = R >= 2 ? R / 2 : 1;
+    constexpr int NB = NA >= 2 ? NA / 2 : 1;
+    float a[NA], b[NB];
+    swap_halve<32, R>(v, a);
+    swap_halve<16, NA>(a, b);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) b[i] += dpp_mov<kDppRor8>(b[i]);
+    pin_here(b);
+    const int b5 = (lane >> 5) & 1, b4 = (lane >> 4) & 1, b3 = (lane >> 3) & 1;
+    const int idx = (R >= 2 ? NA * b5 : 0) + (NA >= 2 ? NB * b4 : 0);
+    const bool writer = b3 == 0 && (R >= 2 || b5 == 0) && (NA >= 2 || b4 == 0);
+    if (writer) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) dst[(idx + i) * STRIDE] = b[i];
+    }
+}
+
 // Two such reductions at once (R >= 2): the 2R values travel through the swap steps together,
 // lanes 0..31 end up with results of `a` (stored to dst_a), lanes 32..63 with results of `b`.
 template <int R>
