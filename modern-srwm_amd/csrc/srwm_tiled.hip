@@ -627,6 +627,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     // next tile, staged in registers
     float4 n_x, n_go, n_q, n_k, n_yd, n_qd, n_kd, n_bt, n_bd;
     float n_ydw[NWL], n_gow[NWL];   // wide rows start at any word: fetched word by word
+    const int wr0 = tid / Y, wm0 = tid % Y;   // row and column of this thread's first word of a wide tile
 #define SRWM_BWD_LOAD_TILE(tile_)                                                                  \
     do { /* rows past the end of the sequence are clamped: they are loaded but never used */       \
         const int t_ = min((tile_) * TT + ld_row, p.L - 1);                                        \
@@ -643,12 +644,17 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
         n_qd = *reinterpret_cast<const float4 *>(p.qdiff + o_);                                    \
         n_kd = *reinterpret_cast<const float4 *>(p.kdiff + o_);                                    \
         if constexpr (XC) {                                                                        \
+            /* word f = tid + i NT of the tile is (row, column) = (f / Y, f % Y): stepped from   */ \
+            /* the thread's first word, no division; words past the tile repeat its last row    */ \
+            int r_ = wr0, m_ = wm0;                                                                \
             _Pragma("unroll") for (int i_ = 0; i_ < NWL; ++i_) {                                   \
-                const int f_ = min(tid + i_ * NT, TT * Y - 1), r_ = f_ / Y, m_ = f_ - r_ * Y;      \
-                const int64_t tw_ = min((tile_) * TT + r_, p.L - 1);                               \
+                const int64_t tw_ = min((tile_) * TT + min(r_, TT - 1), p.L - 1);                  \
                 n_ydw[i_] = p.ydiff[(seq * p.L + tw_) * Y + m_];                                   \
                 n_gow[i_] = bf16_io ? __uint_as_float((uint32_t)gobase16[tw_ * p.gs_l + m_])       \
                                     : gobase[tw_ * p.gs_l + m_];                                   \
+                m_ += NT % Y;                                                                      \
+                r_ += NT / Y + (m_ >= Y ? 1 : 0);                                                  \
+                m_ -= m_ >= Y ? Y : 0;                                                             \
             }                                                                                      \
         } else {                                                                                   \
             if (bf16_io) {                                                                         \
@@ -673,12 +679,15 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
         *reinterpret_cast<float4 *>(&tl[VQD][ld_row][ld_col]) = n_qd;                              \
         *reinterpret_cast<float4 *>(&tl[VKD][ld_row][ld_col]) = n_kd;                              \
         if constexpr (XC) {                                                                        \
+            int r_ = wr0, m_ = wm0;                                                                \
             _Pragma("unroll") for (int i_ = 0; i_ < NWL; ++i_) {                                   \
-                const int f_ = tid + i_ * NT, r_ = f_ / Y, m_ = f_ - r_ * Y;                       \
-                if (f_ < TT * Y) {                                                                 \
+                if (r_ < TT) {                                                                     \
                     tyd[r_][m_] = n_ydw[i_];                                                       \
                     tgo[r_][m_] = bf16_io ? bf16_bits_to_f32(__float_as_uint(n_gow[i_])) : n_gow[i_]; \
                 }                                                                                  \
+                m_ += NT % Y;                                                                      \
+                r_ += NT / Y + (m_ >= Y ? 1 : 0);                                                  \
+                m_ -= m_ >= Y ? Y : 0;                                                             \
             }                                                                                      \
         } else {                                                                                   \
             if (bf16_io) n_go = bf16x4_to_f32(make_uint2(__float_as_uint(n_go.x), __float_as_uint(n_go.y))); \
