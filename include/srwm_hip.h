@@ -54,6 +54,12 @@ extern "C" {
                                      ones (forward: chunks of 64 steps; backward: a sweep over memory columns and
                                      one over memory rows); E == M in {64, 128}, else SRWM_ENOKERNEL.  Forward and
                                      backward may be mixed freely: both forms emit / consume the same v_old, v_insert */
+#define SRWM_FLAG_EXACT_PRODUCTS 512u /* delta_*_bf16 with SRWM_FLAG_CHUNKWISE: also the matrix products whose result only
+                                        goes into `out`, grad_Q or grad_K are formed from hi + lo operand pairs (errors of
+                                        those outputs ~1e-5 instead of ~3e-3, the bf16 rounding such outputs get anyway;
+                                        forward + backward ~8 % slower).  The memory, v_old, v_insert, grad_V, grad_beta
+                                        and dL/dW_0 are formed from operand pairs in either mode.  Accepted and without
+                                        effect wherever every product is exact already (fp32 inputs, step-by-step kernels). */
 /* srwm_layer_forward_* / srwm_layer_backward_* only: */
 #define SRWM_FLAG_STATE_SHIFT 64u    /* W_y..w_b hold the state MINUS the head's shared weights, on entry and on
                                         exit (how the RL layers carry it, torchbeast/layer.py:389-418) */

@@ -456,8 +456,8 @@ int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const
                       int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
         return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE)) ||
-        flags == (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE))
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS)) ||
+        (flags & (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE)) == (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE))
         return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
         !stride_ok(bs, N, H, L, 1))
@@ -488,7 +488,7 @@ int delta_backward_f32(const float *Q, const int64_t qs[3], const float *K, cons
         return SRWM_EINVAL;
     const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u ||
-        (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE | SRWM_GRAD_STATE_MASK)) ||
+        (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_GRAD_STATE_MASK)) ||
         (flags & (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE)) == (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE))
         return SRWM_EINVAL;
     if (!gW && mode != SRWM_GRAD_STATE_ZERO) return SRWM_EINVAL;
@@ -517,13 +517,14 @@ int delta_forward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K
                        int E, int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
         return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_CHUNKWISE)) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS)))
+        return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
         !stride_ok(bs, N, H, L, 1))
         return SRWM_ESTRIDE;
     DeltaFwdParamsBf16 p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
                          {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
-                         N, H, L, E, M};
+                         N, H, L, E, M, (flags & SRWM_FLAG_EXACT_PRODUCTS) ? 1u : 0u};
     const int r = (flags & SRWM_FLAG_CHUNKWISE) ? launch_delta_fwd_chunk_bf16(p, (hipStream_t)stream)
                                                 : launch_delta_fwd_tiled_bf16(p, (hipStream_t)stream);
     return r >= 0 ? r : SRWM_ENOKERNEL;
@@ -540,7 +541,7 @@ int delta_backward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *
         return SRWM_EINVAL;
     const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u ||
-        (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_GRAD_STATE_MASK)))
+        (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_GRAD_STATE_MASK)))
         return SRWM_EINVAL;
     if (!gW && mode != SRWM_GRAD_STATE_ZERO) return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
@@ -548,7 +549,8 @@ int delta_backward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *
         return SRWM_ESTRIDE;
     DeltaBwdParamsBf16 p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
                          {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, grad_out,
-                         {gs[0], gs[1], gs[2]}, W, gQ, gK, gV, gbeta, gW, N, H, L, E, M, mode};
+                         {gs[0], gs[1], gs[2]}, W, gQ, gK, gV, gbeta, gW, N, H, L, E, M, mode,
+                         (flags & SRWM_FLAG_EXACT_PRODUCTS) ? 1u : 0u};
     const int r = (flags & SRWM_FLAG_CHUNKWISE) ? launch_delta_bwd_chunk_bf16(p, (hipStream_t)stream)
                                                 : launch_delta_bwd_tiled_bf16(p, (hipStream_t)stream);
     return r >= 0 ? r : SRWM_ENOKERNEL;

@@ -9,9 +9,12 @@
 //
 //   PrecF32   operands fp32: one group = four v_mfma_f32_16x16x4f32 (128 cycles per SIMD).
 //   PrecBf16  operands bf16: two groups = one v_mfma_f32_16x16x32_bf16 (16 cycles).  Values that
-//             are not exactly representable in bf16 travel as hi + lo (hi = the upper 16 bits,
-//             lo = bf16 of the exact remainder, 16 significant bits together) and a product
-//             takes the passes hi*hi, hi*lo, lo*hi as needed; accumulation is fp32 either way.
+//             are not exactly representable in bf16 travel as hi + lo (hi = the value rounded to
+//             bf16, lo = the exact remainder rounded to bf16: 16 to 17 significant bits together)
+//             and a product takes the passes hi*hi, hi*lo, lo*hi as needed.  A product whose result
+//             only goes into an output that is rounded to bf16 anyway takes hi*hi alone (template
+//             flags SA = SB = false): hi is the correctly rounded bf16 value, so that is an ordinary
+//             bf16 matrix product with fp32 accumulation.  Accumulation is fp32 either way.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -64,6 +67,7 @@ struct PrecF32 {
     }
     __device__ static __forceinline__ B accb(const f32x4 &x) { return B{x}; }
     __device__ static __forceinline__ B accb_exact(const f32x4 &x) { return B{x}; }
+    __device__ static __forceinline__ B accb1(const f32x4 &x) { return B{x}; }
     __device__ static __forceinline__ B negb(const B &b) { return B{-b.v}; }
     template <bool SA, bool SB>
     __device__ static __forceinline__ f32x4 mma(const A &a, const B &b, f32x4 acc) {
@@ -109,6 +113,17 @@ __device__ __forceinline__ float bf_hi_part(float x) { return __uint_as_float(__
 // upper halves of two words packed into one: (a >> 16) | (b & 0xFFFF0000)
 __device__ __forceinline__ uint32_t pack_hi16(uint32_t a, uint32_t b) {
     return __builtin_amdgcn_perm(b, a, 0x07060302u);
+}
+// two floats rounded to nearest-even bf16 (v_cvt_pk_bf16_f32), a in the lower half
+__device__ __forceinline__ uint32_t pack_bf16_rne(float a, float b) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{a, b}, bf16x2));
+}
+// hi = the pair rounded to bf16, lo = what rounding left, rounded to bf16
+__device__ __forceinline__ void split_bf16_pair(float a, float b, uint32_t &hi, uint32_t &lo) {
+    hi = pack_bf16_rne(a, b);
+    lo = pack_bf16_rne(a - __uint_as_float(hi << 16), b - __uint_as_float(hi & 0xFFFF0000u));
 }
 
 struct PrecBf16 {
@@ -177,17 +192,21 @@ struct PrecBf16 {
         b.lo = SP ? rd4t<LD>(m.lo, k, n) : b.hi;
         return b;
     }
-    // accumulator tile -> right operand: hi = upper 16 bits, lo = upper 16 bits of the remainder
+    // accumulator tile -> right operand, hi and lo part
     __device__ static __forceinline__ B accb(const f32x4 &x) {
-        uint32_t xb[4], lb[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            xb[j] = __float_as_uint(x[j]);
-            lb[j] = __float_as_uint(x[j] - bf_hi_part(x[j]));
-        }
+        uint32_t h0, h1, l0, l1;
+        split_bf16_pair(x[0], x[1], h0, l0);
+        split_bf16_pair(x[2], x[3], h1, l1);
         B b;
-        b.hi = __builtin_bit_cast(s16x4, make_uint2(pack_hi16(xb[0], xb[1]), pack_hi16(xb[2], xb[3])));
-        b.lo = __builtin_bit_cast(s16x4, make_uint2(pack_hi16(lb[0], lb[1]), pack_hi16(lb[2], lb[3])));
+        b.hi = __builtin_bit_cast(s16x4, make_uint2(h0, h1));
+        b.lo = __builtin_bit_cast(s16x4, make_uint2(l0, l1));
+        return b;
+    }
+    // the same without a lo part, for products that take hi * hi alone
+    __device__ static __forceinline__ B accb1(const f32x4 &x) {
+        B b;
+        b.hi = __builtin_bit_cast(s16x4, make_uint2(pack_bf16_rne(x[0], x[1]), pack_bf16_rne(x[2], x[3])));
+        b.lo = b.hi;
         return b;
     }
     // the same for values that are exactly bf16 numbers (no lo part)
@@ -243,18 +262,25 @@ struct PrecBf16 {
     }
     template <int LD, bool SP>
     __device__ static __forceinline__ void st(const Mat<LD, SP> &m, int row, int col, float v) {
-        m.hi[row * LD + col] = (uint16_t)bf_hi_bits(v);
-        if constexpr (SP) m.lo[row * LD + col] = (uint16_t)bf_hi_bits(v - bf_hi_part(v));
+        if constexpr (SP) {
+            uint32_t h, l;
+            split_bf16_pair(v, 0.f, h, l);
+            m.hi[row * LD + col] = (uint16_t)h;
+            m.lo[row * LD + col] = (uint16_t)l;
+        } else {
+            m.hi[row * LD + col] = (uint16_t)pack_bf16_rne(v, 0.f);
+        }
     }
     template <int LD, bool SP>
     __device__ static __forceinline__ void st4(const Mat<LD, SP> &m, int row, int col, const float4 &v) {
-        const uint32_t a = __float_as_uint(v.x), b = __float_as_uint(v.y), c = __float_as_uint(v.z),
-                       d = __float_as_uint(v.w);
-        *reinterpret_cast<uint2 *>(m.hi + row * LD + col) = make_uint2(pack_hi16(a, b), pack_hi16(c, d));
         if constexpr (SP) {
-            const uint32_t la = __float_as_uint(v.x - bf_hi_part(v.x)), lb = __float_as_uint(v.y - bf_hi_part(v.y)),
-                           lc = __float_as_uint(v.z - bf_hi_part(v.z)), ld_ = __float_as_uint(v.w - bf_hi_part(v.w));
-            *reinterpret_cast<uint2 *>(m.lo + row * LD + col) = make_uint2(pack_hi16(la, lb), pack_hi16(lc, ld_));
+            uint32_t h0, h1, l0, l1;
+            split_bf16_pair(v.x, v.y, h0, l0);
+            split_bf16_pair(v.z, v.w, h1, l1);
+            *reinterpret_cast<uint2 *>(m.hi + row * LD + col) = make_uint2(h0, h1);
+            *reinterpret_cast<uint2 *>(m.lo + row * LD + col) = make_uint2(l0, l1);
+        } else {
+            *reinterpret_cast<uint2 *>(m.hi + row * LD + col) = make_uint2(pack_bf16_rne(v.x, v.y), pack_bf16_rne(v.z, v.w));
         }
     }
     template <int LD, bool SP>
@@ -345,6 +371,7 @@ struct PrecBf16x3 {
         return B{__builtin_bit_cast(s16x4, h), __builtin_bit_cast(s16x4, m), __builtin_bit_cast(s16x4, l)};
     }
     __device__ static __forceinline__ B accb_exact(const f32x4 &x) { return accb(x); }
+    __device__ static __forceinline__ B accb1(const f32x4 &x) { return accb(x); }
     __device__ static __forceinline__ B negb(const B &b) {
         const auto flip = [](const s16x4 &v) {
             const uint2 u = __builtin_bit_cast(uint2, v);

@@ -113,6 +113,7 @@ struct DeltaFwdParamsBf16 {
     float *vold, *vins, *W;
     uint16_t *out;
     int N, H, L, E, M;
+    unsigned exact_products;   // chunkwise kernels: every product from hi + lo operand pairs
 };
 
 struct DeltaBwdParamsBf16 {
@@ -126,6 +127,7 @@ struct DeltaBwdParamsBf16 {
     float *gW;
     int N, H, L, E, M;
     unsigned grad_state_mode;
+    unsigned exact_products;   // chunkwise kernels: every product from hi + lo operand pairs
 };
 
 // ---- bf16 <-> fp32 (16-bit patterns; round to nearest even on the way down)

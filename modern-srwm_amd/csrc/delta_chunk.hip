@@ -46,35 +46,40 @@ struct ChunkFwdP {
     float *vold, *vins, *W;
     TI *out;
     int N, H, L;
+    bool exact;   // bf16 inputs: also the products that only feed `out` from hi + lo operand pairs
 };
 
 // LDS carve-up shared by the kernel and the launcher
 // KS = 2: the rows of the memory are split over two groups of four waves (8 waves per workgroup,
 // two per SIMD); a pair of waves owns the same 16 columns, each half of the rows, and exchanges
 // its partial K S and Q S through LDS.
-template <class TI, int D, int KS>
+// OB: the products that only feed `out` (Q S, tril(B) U) take the hi parts of their operands alone
+// (precisions with operand parts; without effect otherwise), and B has no lo part.
+template <class TI, int D, int KS, bool OB>
 struct FwdLds {
     typedef typename PrecOf<TI, D>::type X;
     static constexpr int LDK = D + X::kPad, LDA = kC + X::kPad, LDD = 16 + X::kPad, LDV = kMC + 4;
     typedef typename X::template Mat<LDK, false> MatK;   // K, Q: the inputs themselves
-    typedef typename X::template Mat<LDA, true> MatA;    // A, B: computed
+    typedef typename X::template Mat<LDA, true> MatA;    // A: computed, feeds the solve
+    typedef typename X::template Mat<LDA, !OB> MatB;     // B: computed, only feeds `out`
     typedef typename X::template Mat<LDD, true> MatD;    // inverses of the diagonal blocks
     static constexpr int oK = 0;
     static constexpr int oQ = oK + MatK::bytes(kC);
     static constexpr int oA = oQ + MatK::bytes(kC);
     static constexpr int oB = oA + MatA::bytes(kC);
-    static constexpr int oD = oB + MatA::bytes(kC);
+    static constexpr int oD = oB + MatB::bytes(kC);
     static constexpr int oV = oD + MatD::bytes(kC);            // fp32 [C][LDV]
     static constexpr int oAd = oV + kC * LDV * 4;              // fp32 [C][LDD]: diagonal blocks of A
     static constexpr int oBt = oAd + kC * LDD * 4;             // fp32 [C]: beta
     static constexpr int oX = oBt + kC * 4;                    // KS == 2: [8 waves][2 * kCB tiles][64 lanes] f32x4
     static constexpr int kBytes = oX + (KS == 2 ? 8 * 2 * kCB * 64 * 16 : 0);
-    static_assert(MatK::bytes(kC) % 16 == 0 && MatA::bytes(kC) % 16 == 0 && MatD::bytes(kC) % 16 == 0, "alignment");
+    static_assert(MatK::bytes(kC) % 16 == 0 && MatA::bytes(kC) % 16 == 0 && MatB::bytes(kC) % 16 == 0 &&
+                      MatD::bytes(kC) % 16 == 0, "alignment");
 };
 
-template <class TI, int D, int MS, int KS>
+template <class TI, int D, int MS, int KS, bool OB>
 __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP<TI> p) {
-    typedef FwdLds<TI, D, KS> Lds;
+    typedef FwdLds<TI, D, KS, OB> Lds;
     typedef typename Lds::X X;
     constexpr int NT = kThreads * KS;
     constexpr int EB = D / 16 / KS;     // 16-row blocks of the memory held by this wave
@@ -83,7 +88,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const typename Lds::MatK Ks(smem + Lds::oK, kC), Qs(smem + Lds::oQ, kC);
     const typename Lds::MatA As(smem + Lds::oA, kC);   // strict lower triangle of K K^T
-    const typename Lds::MatA Bs(smem + Lds::oB, kC);   // lower triangle (with diagonal) of Q K^T
+    const typename Lds::MatB Bs(smem + Lds::oB, kC);   // lower triangle (with diagonal) of Q K^T
     const typename Lds::MatD Di(smem + Lds::oD, kC);   // [4][16] inverses of the diagonal blocks of I + L
     float *Vs = reinterpret_cast<float *>(smem + Lds::oV);
     float *Ad = reinterpret_cast<float *>(smem + Lds::oAd);
@@ -221,7 +226,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
                 pt[cb] = mma_range<X, false, true>(
                     0, EB, [&](int eb) { return X::lda(Ks, cb * 16 + ln, e0 + eb * 16 + 4 * lq); }, fb,
                     f32x4{0.f, 0.f, 0.f, 0.f});
-                ot[cb] = mma_range<X, false, true>(
+                ot[cb] = mma_range<X, false, !OB>(   // only feeds `out`
                     0, EB, [&](int eb) { return X::lda(Qs, cb * 16 + ln, e0 + eb * 16 + 4 * lq); }, fb,
                     f32x4{0.f, 0.f, 0.f, 0.f});
             }
@@ -266,7 +271,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
             if (a % KS == hf) {   // the two waves of a pair share the outputs: each forms and stores every other row block
                 y = X::template mma<true, true>(X::lda(As, a * 16 + ln, a * 16 + 4 * lq), ub[a], y);   // + strict_lower(A_aa) U_a
                 // out = Q S + tril(B) U
-                ot[a] = mma_range<X, true, true>(
+                ot[a] = mma_range<X, !OB, !OB>(
                     0, a + 1, [&](int b) { return X::lda(Bs, a * 16 + ln, b * 16 + 4 * lq); }, fu, ot[a]);
                 // one 32-bit byte offset per lane from the sequence's (uniform) base; the rows of the
                 // block follow at compile-time distances
@@ -313,13 +318,21 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
         for (int r = 0; r < 4; ++r) Wg[(e0 + eb * 16 + 4 * lq + r) * D + ln] = s[eb][r];
 }
 
+template <class TI, int D, int MS, int KS, bool OB>
+int launch_chunk_ob(const ChunkFwdP<TI> &p, hipStream_t s) {
+    constexpr size_t lds = FwdLds<TI, D, KS, OB>::kBytes;
+    static_assert(lds <= kMaxLdsBytes, "LDS budget");
+    if (const int err = allow_max_dynamic_lds<delta_fwd_chunk_kernel<TI, D, MS, KS, OB>>()) return err;
+    hipLaunchKernelGGL((delta_fwd_chunk_kernel<TI, D, MS, KS, OB>), dim3(p.N * p.H * MS), dim3(kThreads * KS), lds, s, p);
+    return (int)hipGetLastError();
+}
+
 template <class TI, int D, int MS, int KS>
 int launch_chunk(const ChunkFwdP<TI> &p, hipStream_t s) {
-    constexpr size_t lds = FwdLds<TI, D, KS>::kBytes;
-    static_assert(lds <= kMaxLdsBytes, "LDS budget");
-    if (const int err = allow_max_dynamic_lds<delta_fwd_chunk_kernel<TI, D, MS, KS>>()) return err;
-    hipLaunchKernelGGL((delta_fwd_chunk_kernel<TI, D, MS, KS>), dim3(p.N * p.H * MS), dim3(kThreads * KS), lds, s, p);
-    return (int)hipGetLastError();
+    if constexpr (PrecOf<TI, D>::type::kBf) {
+        if (!p.exact) return launch_chunk_ob<TI, D, MS, KS, true>(p, s);
+    }
+    return launch_chunk_ob<TI, D, MS, KS, false>(p, s);
 }
 
 template <class TI>
@@ -343,14 +356,14 @@ int dispatch_chunk(const ChunkFwdP<TI> &p, int D, hipStream_t s) {
 int launch_delta_fwd_chunk(const DeltaFwdParams &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const ChunkFwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out,
-                             p.N, p.H, p.L};
+                             p.N, p.H, p.L, true};
     return dispatch_chunk(q, p.E, s);
 }
 
 int launch_delta_fwd_chunk_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const ChunkFwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out,
-                              p.N, p.H, p.L};
+                              p.N, p.H, p.L, p.exact_products != 0u};
     return dispatch_chunk(q, p.E, s);
 }
 

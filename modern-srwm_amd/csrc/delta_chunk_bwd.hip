@@ -54,6 +54,7 @@ struct ChunkBwdP {
     float *gW;
     int N, H, L;
     unsigned grad_state_mode;
+    bool exact;   // bf16 inputs: also the products that only feed grad_Q / grad_K from hi + lo operand pairs
 };
 
 // ------------------------------------------------------------------------------------------
@@ -320,14 +321,17 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 // ------------------------------------------------------------------------------------------
 // Row sweep
 // ------------------------------------------------------------------------------------------
-template <class TI, int D, int C, int KS>
+// OB: the products that only feed grad_Q / grad_K (G1, Z, dOut S^T, U dS'^T, Y S^T and those with G1
+// and Z) take the hi parts of their operands alone (precisions with operand parts; without effect
+// otherwise), and G1, Z have no lo part.
+template <class TI, int D, int C, int KS, bool OB>
 struct RowLds {
     typedef typename PrecOf<TI, D>::type X;
     static constexpr int LDM = D + X::kPad, LDW = kWC + X::kPad, LDC = C + X::kPad;
     typedef typename X::template Mat<LDM, false> MatG;   // dOut: an input
     typedef typename X::template Mat<LDM, true> MatU;    // U, Y: computed
     typedef typename X::template Mat<LDW, false> MatK;   // this workgroup's 64 columns of K, Q
-    typedef typename X::template Mat<LDC, true> MatC;    // G1, X + X^T
+    typedef typename X::template Mat<LDC, !OB> MatC;     // G1, X + X^T: only feed grad_Q / grad_K
     static constexpr int oG = 0;
     static constexpr int oU = oG + MatG::bytes(C);
     static constexpr int oY = oU + MatU::bytes(C);
@@ -347,9 +351,9 @@ struct RowLds {
 // through LDS (the grad_Q part over the K / Q slices, which are dead by then: their fragments sit
 // in registers; the grad_K part through a buffer of its own, so that one barrier serves both), and
 // finishes grad_Q, grad_K for its own half of the chunk.
-template <class TI, int D, int MS, int C, int KS>
+template <class TI, int D, int MS, int C, int KS, bool OB>
 __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(ChunkBwdP<TI> p) {
-    typedef RowLds<TI, D, C, KS> Lds;
+    typedef RowLds<TI, D, C, KS, OB> Lds;
     typedef typename Lds::X X;
     constexpr int NT = kThreads * KS;
     constexpr int CB = C / 16, MBF = D / 16, MB = MBF / KS, NTRI = CB * (CB + 1) / 2;   // MB: column blocks held by a wave
@@ -458,9 +462,9 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
             tri_index(pix, ci, cj);
             const auto fb = [&](int mb) { return X::ldb(Us, cj * 16 + ln, mb * 16 + 4 * lq); };
             const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-            const f32x4 accG = mma_range<X, false, true>(
+            const f32x4 accG = mma_range<X, false, !OB>(
                 0, MBF, [&](int mb) { return X::lda(Gs, ci * 16 + ln, mb * 16 + 4 * lq); }, fb, zero);
-            const f32x4 accX = mma_range<X, true, true>(
+            const f32x4 accX = mma_range<X, !OB, !OB>(
                 0, MBF, [&](int mb) { return X::lda(Ys, ci * 16 + ln, mb * 16 + 4 * lq); }, fb, zero);
             const int col = cj * 16 + ln;
 #pragma unroll
@@ -491,11 +495,11 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
         }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-            dstb[mb] = X::accb(dst[mb]);   // dS' (before this chunk's update)
+            dstb[mb] = OB ? X::accb1(dst[mb]) : X::accb(dst[mb]);   // dS' (before this chunk's update); only feeds grad_K
             st[mb] = mma_range<X, true, false>(
                 0, CB, [&](int cb) { return X::lda_t(Us, cb * 16 + 4 * lq, m0 + mb * 16 + ln); },
                 [&](int cb) { return nkb[cb]; }, st[mb]);
-            nstb[mb] = X::accb(-st[mb]);   // -S (entry value)
+            nstb[mb] = OB ? X::accb1(-st[mb]) : X::accb(-st[mb]);   // -S (entry value); only feeds grad_Q / grad_K
         }
         // ---- G1 and Z become visible
         __syncthreads();
@@ -505,25 +509,25 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
         const auto fnk = [&](int b) { return nkb[b]; };
         // the products over memory columns (this wave's columns), for row block cb of the chunk
         const auto dq_state = [&](int cb) {
-            return mma_range<X, false, true>(
+            return mma_range<X, false, !OB>(
                 0, MB, [&](int mb) { return X::lda(Gs, cb * 16 + ln, m0 + mb * 16 + 4 * lq); }, fns,
                 f32x4{0.f, 0.f, 0.f, 0.f});
         };
         const auto dk_state = [&](int cb) {
-            const f32x4 a = mma_range<X, true, true>(
+            const f32x4 a = mma_range<X, !OB, !OB>(
                 0, MB, [&](int mb) { return X::lda(Us, cb * 16 + ln, m0 + mb * 16 + 4 * lq); },
                 [&](int mb) { return dstb[mb]; }, f32x4{0.f, 0.f, 0.f, 0.f});
-            return mma_range<X, true, true>(
+            return mma_range<X, !OB, !OB>(
                 0, MB, [&](int mb) { return X::lda(Ys, cb * 16 + ln, m0 + mb * 16 + 4 * lq); }, fns, a);
         };
         // the products over the chunk's steps, added onto those, and the stores
         const auto finish = [&](int cb, f32x4 dqn, f32x4 dk) {
-            dqn = mma_range<X, true, false>(
+            dqn = mma_range<X, !OB, false>(
                 0, cb + 1, [&](int b) { return X::lda(G1, cb * 16 + ln, b * 16 + 4 * lq); }, fnk, dqn);
-            dk = mma_range<X, true, false>(
+            dk = mma_range<X, !OB, false>(
                 cb, CB, [&](int b) { return X::lda_t(G1, b * 16 + 4 * lq, cb * 16 + ln); },
                 [&](int b) { return qbf[b]; }, dk);
-            dk = mma_range<X, true, false>(
+            dk = mma_range<X, !OB, false>(
                 0, CB, [&](int b) { return X::lda(Z, cb * 16 + ln, b * 16 + 4 * lq); }, fnk, dk);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
@@ -603,18 +607,26 @@ __global__ void zero_words_kernel(float *a, int64_t n) {
 }
 
 // KS: waves per memory row / column block in the column sweep, KSR: in the row sweep
-template <class TI, int D, int MS, int C2, int KS, int KSR>
-int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
-    constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2, KSR>::kBytes;
+template <class TI, int D, int MS, int C2, int KS, int KSR, bool OB>
+int launch_chunk_bwd_ob(const ChunkBwdP<TI> &p, hipStream_t s) {
+    constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2, KSR, OB>::kBytes;
     static_assert(lds1 <= (int)kMaxLdsBytes && lds2 <= (int)kMaxLdsBytes, "LDS budget");
     if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_col_kernel<TI, D, MS, KS>>()) return err;
-    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR>>()) return err;
+    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR, OB>>()) return err;
     const int grid = p.N * p.H * MS;
     if (MS > 1)   // two workgroups of the column sweep add their parts of grad_beta
         hipLaunchKernelGGL(zero_words_kernel, dim3(256), dim3(256), 0, s, p.gbeta, (int64_t)p.N * p.H * p.L);
     hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS, KS>), dim3(grid), dim3(kThreads * KS), lds1, s, p);
-    hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR>), dim3(grid), dim3(kThreads * KSR), lds2, s, p);
+    hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR, OB>), dim3(grid), dim3(kThreads * KSR), lds2, s, p);
     return (int)hipGetLastError();
+}
+
+template <class TI, int D, int MS, int C2, int KS, int KSR>
+int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
+    if constexpr (PrecOf<TI, D>::type::kBf) {
+        if (!p.exact) return launch_chunk_bwd_ob<TI, D, MS, C2, KS, KSR, true>(p, s);
+    }
+    return launch_chunk_bwd_ob<TI, D, MS, C2, KS, KSR, false>(p, s);
 }
 
 template <class TI>
@@ -642,14 +654,14 @@ int dispatch_chunk_bwd(const ChunkBwdP<TI> &p, int D, hipStream_t s) {
 int launch_delta_bwd_chunk(const DeltaBwdParams &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const ChunkBwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
-                             p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode};
+                             p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode, true};
     return dispatch_chunk_bwd(q, p.E, s);
 }
 
 int launch_delta_bwd_chunk_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const ChunkBwdP<uint16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
-                                p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode};
+                                p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode, p.exact_products != 0u};
     return dispatch_chunk_bwd(q, p.E, s);
 }
 

@@ -20,12 +20,17 @@ import srwm_hip
 # v_insert, so forward and backward can be chosen independently.
 CHUNKWISE_FORWARD = "auto"
 CHUNKWISE_BACKWARD = "auto"
+# bfloat16 inputs on the chunkwise kernels: the matrix products whose result only goes into `out`,
+# grad_Q or grad_K are plain bf16 products with fp32 accumulation (those tensors come back in
+# bfloat16 anyway); True forms them from hi + lo operand pairs as well (~8 % slower).  The memory,
+# v_old, v_insert, grad_V and grad_beta do not depend on this.  No effect with float32 inputs.
+EXACT_PRODUCTS = False
 
 
 def _chunk_flags(choice, E, M, L):
     has_kernel = E == M and E in (64, 128)
     if choice is True or (choice == "auto" and has_kernel and L >= 64):
-        return srwm_hip.FLAG_CHUNKWISE
+        return srwm_hip.FLAG_CHUNKWISE | (srwm_hip.FLAG_EXACT_PRODUCTS if EXACT_PRODUCTS else 0)
     return 0
 
 

@@ -30,6 +30,7 @@ GRAD_STATE_IN = 1
 GRAD_STATE_ACCUM = 2
 FLAG_GENERIC = 16
 FLAG_CHUNKWISE = 32     # delta forward: chunkwise MFMA kernel (E == M in {64, 128})
+FLAG_EXACT_PRODUCTS = 512   # chunkwise kernels with bf16 inputs: every product from hi + lo operand pairs
 FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus the shared weights
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
