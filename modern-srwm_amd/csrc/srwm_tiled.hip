@@ -128,8 +128,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     __shared__ __attribute__((aligned(16))) float xt[2][TT][E];   // input tiles, double buffered
     __shared__ float kt[2][TT];                                   // keep flags of the tile's steps
     // the raw readout of a step, by parity: row e = { q~[e], k~[e], b~[e % 4], - }, everything the lane of
-    // element e needs for the activations in ONE read
+    // element e needs for the activations in ONE read (RAW4); the kernel with per-step resets, which is
+    // tighter on registers, is faster with the three vectors apart: q~ | k~ | b~
+    constexpr bool RAW4 = !RESET;
     __shared__ __attribute__((aligned(16))) float raw[2][E][4];
+    float(*const rawv)[4][E] = reinterpret_cast<float(*)[4][E]>(raw);   // the layout used when !RAW4
     __shared__ __attribute__((aligned(16))) float exch[NW][2][E]; // per wave: q-k | k
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
@@ -285,11 +288,20 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             } else {
                 store_y(out_s, oy, &acc[0]);
             }
+            if constexpr (RAW4) {
 #pragma unroll
-            for (int c = 0; c < CB; ++c)
-                *reinterpret_cast<float2 *>(&raw[par][c0 + c][0]) = make_float2(acc[QB + c], acc[KB + c]);
+                for (int c = 0; c < CB; ++c)
+                    *reinterpret_cast<float2 *>(&raw[par][c0 + c][0]) = make_float2(acc[QB + c], acc[KB + c]);
+            } else {
+                store_vec<CB>(&rawv[par][0][c0], &acc[QB]);
+                store_vec<CB>(&rawv[par][1][c0], &acc[KB]);
+            }
         }
-        if (has_b && (el & 3) == jb) raw[par][el][2] = pb;   // every lane of column jb holds the sum
+        if constexpr (RAW4) {
+            if (has_b && (el & 3) == jb) raw[par][el][2] = pb;   // every lane of column jb holds the sum
+        } else {
+            if (has_b && el == 0) rawv[par][2][jb] = pb;
+        }
         if constexpr (XC) {
             if (has_y && el == 0) {
                 if (bf16_io) *at32(out16_s, oy + YB * E) = f32_to_bf16_bits(py);
@@ -329,8 +341,13 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         lds_read_vec<R>(xr, &xt[b1][r1][r0]);
         const float xb = xt[b1][r1][el];
         const bool reset_next = RESET && have_next && kt[b1][r1] == 0.f;   // uniform over the workgroup
-        const float4 raw_el = *reinterpret_cast<const float4 *>(&raw[par][el][0]);
-        const float qraw = raw_el.x, kraw = raw_el.y, braw = raw_el.z;   // el % 4 == lane % 4
+        float qraw, kraw, braw;
+        if constexpr (RAW4) {
+            const float4 raw_el = *reinterpret_cast<const float4 *>(&raw[par][el][0]);
+            qraw = raw_el.x, kraw = raw_el.y, braw = raw_el.z;   // el % 4 == lane % 4
+        } else {
+            qraw = rawv[par][0][el], kraw = rawv[par][1][el], braw = rawv[par][2][lane & 3];
+        }
         float e[NC];
 #pragma unroll
         for (int c = 0; c < NC; ++c) e[c] = 0.f;
