@@ -203,3 +203,67 @@ def test_product_formula_of_the_triangular_block_inverse():
         assert np.allclose(R, ref, rtol=1e-10, atol=1e-10)
         assert np.allclose(Rt, ref.T, rtol=1e-10, atol=1e-10)
         assert np.abs(np.linalg.matrix_power(M, 16)).max() == 0.0
+
+
+def _bf16_trunc(x):
+    """float32 array -> the float32 values of its upper 16 bits (what a bf16 holds after cutting)."""
+    return (x.view(np.uint32) & np.uint32(0xFFFF0000)).view(np.float32)
+
+
+def _bf16_rne(x):
+    """float32 array -> nearest-even bf16, returned as float32."""
+    u = x.view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32)
+
+
+def test_operand_parts_of_the_matrix_core_products():
+    """The arithmetic the chunkwise kernels rely on when they run fp32-accurate products on the bf16
+    matrix instruction, modelled in numpy (fp32 operations where the kernel uses fp32):
+    * cutting a float three times (hi = upper 16 bits, mid = upper 16 bits of x - hi, lo = the rest)
+      gives three bf16 numbers whose sum is x exactly -- every float32, any exponent;
+    * the six partial products hi*hi, hi*mid, mid*hi, mid*mid, hi*lo, lo*hi reproduce a dot product
+      to fp32 accuracy (the three dropped ones are below 2^-24 of the terms);
+    * the rounded pair hi = rne(x), lo = rne(x - hi) represents x to 2^-16, twice as well as the cut
+      pair, and the three products hi*hi, hi*lo, lo*hi give a dot product to ~1e-5."""
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal(400000) * np.exp2(rng.integers(-60, 60, 400000))).astype(np.float32)
+    x[:4] = [0.0, -0.0, np.float32(1.0) - np.float32(2.0 ** -24), np.float32(-3.0000002)]
+    hi = _bf16_trunc(x)
+    r1 = (x - hi).astype(np.float32)
+    mid = _bf16_trunc(r1)
+    lo = (r1 - mid).astype(np.float32)
+    assert np.array_equal(lo, _bf16_trunc(lo))                      # lo is a bf16 number
+    assert np.array_equal(hi.astype(np.float64) + mid.astype(np.float64) + lo.astype(np.float64), x.astype(np.float64))
+
+    a = rng.standard_normal((64, 128)).astype(np.float32)
+    b = rng.standard_normal((128, 64)).astype(np.float32)
+
+    def parts3(m):
+        h = _bf16_trunc(m)
+        r = (m - h).astype(np.float32)
+        mi = _bf16_trunc(r)
+        return [p.astype(np.float64) for p in (h, mi, (r - mi).astype(np.float32))]
+
+    (ah, am, al), (bh, bm, bl) = parts3(a), parts3(b)
+    six = ah @ bh + ah @ bm + am @ bh + am @ bm + ah @ bl + al @ bh
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    scale = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
+    assert (np.abs(six - exact) / scale).max() < 2.0 ** -22
+    five = six - am @ bm                                              # without mid*mid: 2^-16 of the terms, not enough
+    assert (np.abs(five - exact) / scale).max() > 2.0 ** -19
+
+    xs = x[np.isfinite(x) & (np.abs(x) > 1e-30) & (np.abs(x) < 1e30)]
+    h2 = _bf16_rne(xs)
+    l2 = _bf16_rne((xs - h2).astype(np.float32))
+    cut_pair = _bf16_trunc(xs).astype(np.float64) + _bf16_trunc((xs - _bf16_trunc(xs)).astype(np.float32)).astype(np.float64)
+    err_rne = np.abs(h2.astype(np.float64) + l2.astype(np.float64) - xs) / np.abs(xs)
+    err_cut = np.abs(cut_pair - xs) / np.abs(xs)
+    assert err_rne.max() <= 2.0 ** -16 and err_cut.max() <= 2.0 ** -15 and err_rne.mean() < 0.5 * err_cut.mean()
+    ah2, bh2 = _bf16_rne(a), _bf16_rne(b)
+    al2, bl2 = _bf16_rne((a - ah2).astype(np.float32)), _bf16_rne((b - bh2).astype(np.float32))
+    three = (ah2.astype(np.float64) @ bh2.astype(np.float64) + ah2.astype(np.float64) @ bl2.astype(np.float64)
+             + al2.astype(np.float64) @ bh2.astype(np.float64))
+    assert (np.abs(three - exact) / scale).max() < 3e-5
+    one = ah2.astype(np.float64) @ bh2.astype(np.float64)            # a plain bf16 product: bf16-grade, unbiased
+    assert (np.abs(one - exact) / scale).max() < 2.0 ** -8 and abs(((one - exact) / scale).mean()) < 1e-4
