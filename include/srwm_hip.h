@@ -449,7 +449,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any signature change); currently 7. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 8. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

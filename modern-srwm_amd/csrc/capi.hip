@@ -85,7 +85,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 7; }
+int srwm_hip_abi_version(void) { return 8; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 

@@ -35,7 +35,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lib = None
 
