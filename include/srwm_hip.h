@@ -416,6 +416,8 @@ SRWM_API int delta_steps_backward_f32(const float *Q, const int64_t q_strides[3]
  *                                              and gV is re-read by the chunkwise backward;
  *                                              the caller rounds them if it wants bf16)
  * The memory and all accumulation are fp32; `out` is rounded to nearest even.
+ * flags: SRWM_FLAG_CHUNKWISE (and the SRWM_GRAD_STATE_* modes in the backward); with it, the matrix
+ * products that only feed out / gQ / gK are single bf16 products unless SRWM_FLAG_EXACT_PRODUCTS is set.
  */
 SRWM_API int delta_forward_bf16(const uint16_t *Q, const int64_t q_strides[3],
                        const uint16_t *K, const int64_t k_strides[3],
