@@ -241,17 +241,33 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     float *const qdiff_s = p.qdiff + seq * p.L * E, *const kdiff_s = p.kdiff + seq * p.L * E;
     float *const beta_s = p.beta + seq * p.L * 4, *const bdiff_s = p.bdiff + seq * p.L * 4;
     const int ntiles = (p.L + TT - 1) / TT;
+    // Below E = 64 (one wave per SIMD, nothing to hide an LDS round trip behind) the input rows of a step
+    // are read from the tile one step before they are used (XPREF).  The tile after the current one is
+    // then committed when the current one is entered, not when it is left, so that the row to read
+    // ahead is always there; both tiles of the double buffer are filled before the loop.  (Measured: the
+    // plain operator gains 6 % at E = 32; the wide output block and the variant with per-step resets,
+    // which hold more in registers, lose 1-4 %, so they read the row where they use it.)
+    constexpr bool XPREF = E < kWave && !XC && !RESET;
+    static_assert(TT >= 4, "a tile's buffer is rewritten two steps after its last row has been read");
     {
         const float4 x0 = load_tile(0);
         *reinterpret_cast<float4 *>(&xt[0][ld_row][ld_col]) = softmax_x ? row_softmax4<E>(x0) : x0;
+        if (XPREF && ntiles > 1) {
+            const float4 x1 = load_tile(1);
+            *reinterpret_cast<float4 *>(&xt[1][ld_row][ld_col]) = softmax_x ? row_softmax4<E>(x1) : x1;
+        }
     }
-    if (RESET && tid < TT) kt[0][tid] = load_keep(0);
+    if (RESET && tid < TT) {
+        kt[0][tid] = load_keep(0);
+        if (XPREF && ntiles > 1) kt[1][tid] = load_keep(1);
+    }
     __syncthreads();
     float4 xnext = make_float4(0.f, 0.f, 0.f, 0.f);   // the tile after the committed ones, staged in registers
     float knext = 1.f;
-    if (ntiles > 1) {
-        xnext = load_tile(1);
-        knext = load_keep(1);
+    constexpr int kStaged = XPREF ? 2 : 1;            // tiles committed before the loop
+    if (ntiles > kStaged) {
+        xnext = load_tile(kStaged);
+        knext = load_keep(kStaged);
     }
 
     // [y | q~ | k~ | b~] = W^T x of one step, straight from the state in registers
@@ -328,7 +344,15 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 
     // (below E = 64 the loop is unrolled by two, which makes the parity of a step -- it selects the
     // hand-over buffers -- a compile-time constant; at E = 64 the rolled loop is the faster one)
-    auto step = [&](auto PAR, const int t) __attribute__((always_inline)) {
+    struct XRow {
+        float xr[R], xb;
+    };
+    auto read_row = [&](const int t, XRow &o) __attribute__((always_inline)) {   // x of step t (rows past the end: stale, never used)
+        const int b = (t / TT) & 1, r = t % TT;
+        lds_read_vec<R>(o.xr, &xt[b][r][r0]);
+        o.xb = xt[b][r][el];
+    };
+    auto step = [&](auto PAR, const int t, XRow &cur, XRow &nxt) __attribute__((always_inline)) {
         const int par = parity_of(PAR);
         const auto PNEXT = parity_flipped(PAR);
         const int t1 = t + 1;
@@ -337,9 +361,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         const bool have_next = t1 < p.L;
 
         // ---- early part of the next readout: e = W_{t-1}^T x_{t+1}
-        float xr[R];
-        lds_read_vec<R>(xr, &xt[b1][r1][r0]);
-        const float xb = xt[b1][r1][el];
+        if constexpr (!XPREF) read_row(t1, cur);
+        const float(&xr)[R] = cur.xr;
+        const float xb = cur.xb;
         const bool reset_next = RESET && have_next && kt[b1][r1] == 0.f;   // uniform over the workgroup
         float qraw, kraw, braw;
         if constexpr (RAW4) {
@@ -393,6 +417,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         float dvr[R], kr[R];
         lds_read_vec<R>(dvr, &exch[wave][0][r0]);
         lds_read_vec<R>(kr, &exch[wave][1][r0]);
+
+        if constexpr (XPREF) read_row(t + 2, nxt);   // behind the reads of this step's serial chain
 
         // ---- diff = W_{t-1}^T (q - k); with it, the narrow columns and k . x_{t+1}
         float dif[NC];
@@ -469,8 +495,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             }
         }
 
-        // x of step t+2 opens a new tile: commit the staged tile, fetch the one after it
-        if (r1 == TT - 1 && t1 / TT + 1 < ntiles) {
+        // the staged tile is committed and the one after it fetched when x of step t+2 opens a new tile,
+        // or (XPREF) as soon as x of step t+1 has opened one: the other buffer's rows were last read
+        // two steps ago
+        if ((XPREF ? t1 >= TT && r1 == 0 : r1 == TT - 1) && t1 / TT + 1 < ntiles) {
             *reinterpret_cast<float4 *>(&xt[b1 ^ 1][ld_row][ld_col]) = softmax_x ? row_softmax4<E>(xnext) : xnext;
             if (RESET && tid < TT) kt[b1 ^ 1][tid] = knext;
             if (t1 / TT + 2 < ntiles) {
@@ -481,14 +509,17 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         __syncthreads();
     };
     if constexpr (E == kWave) {
-        for (int t = 0; t < p.L; ++t) step(t & 1, t);
+        XRow a;
+        for (int t = 0; t < p.L; ++t) step(t & 1, t, a, a);
     } else {
+        XRow a, b;
+        read_row(1, a);
         int t = 0;
         for (; t + 1 < p.L; t += 2) {
-            step(P0{}, t);
-            step(P1{}, t + 1);
+            step(P0{}, t, a, b);
+            step(P1{}, t + 1, b, a);
         }
-        if (t < p.L) step(P0{}, t);
+        if (t < p.L) step(P0{}, t, a, b);
     }
 
     // the final state, as the shift from the shared weights if that is how the caller keeps it
