@@ -755,10 +755,13 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     // parity pp), through the softmax of the input where the kernel applies it (xs = this thread's
     // element of the softmaxed x_t)
     auto finish_gx = [&](int t, int pp, float xs) {
-        if (tid < E) {
-            float s = row_total(pp, 2, tid);
-            if (softmax_x) s = xs * (s - group_sum<E>(s * xs));   // tid < E covers whole lane groups
-            p.gx[(seq * p.L + t) * E + tid] = s;
+        // below E = 64 by the first E lanes of the LAST wave: the first waves also carry the narrow columns
+        // there (at E = 64 every wave carries one of them)
+        const int e = E < kWave ? tid - (NW - 1) * kWave : tid;
+        if ((unsigned)e < (unsigned)E) {
+            float s = row_total(pp, 2, e);
+            if (softmax_x) s = xs * (s - group_sum<E>(s * xs));   // the E threads are whole lane groups
+            p.gx[(seq * p.L + t) * E + e] = s;
         }
     };
     float xb_prev = 0.f;
