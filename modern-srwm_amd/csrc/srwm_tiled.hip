@@ -142,7 +142,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     const int jb = tid / E;                  // column of this thread's w_b entry
     const bool has_b = jb < 4;
     // who stores what inside a step (lane masks that stay in scalar registers across the loop)
-    const bool st_qk = wave == 0 && lane < E, st_beta = wave == NW - 1 && lane < 4, st_exch = lane < E;
+    // (below E = 64 the first two of the four waves also carry the narrow columns: the other two store q, k and beta)
+    constexpr int WQK = (E < kWave && NW >= 4 && YB == 1) ? 2 : 0;   // (no gain with the wide output block)
+    const bool st_qk = wave == WQK && lane < E, st_beta = wave == NW - 1 && lane < 4, st_exch = lane < E;
 
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
