@@ -128,8 +128,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     __shared__ __attribute__((aligned(16))) float xt[2][TT][E];   // input tiles, double buffered
     __shared__ float kt[2][TT];                                   // keep flags of the tile's steps
     // the raw readout of a step, by parity: row e = { q~[e], k~[e], b~[e % 4], - }, everything the lane of
-    // element e needs for the activations in ONE read (RAW4); the kernel with per-step resets, which is
-    // tighter on registers, is faster with the three vectors apart: q~ | k~ | b~
+    // element e needs for the activations in ONE read (RAW4); the kernel with per-step resets was
+    // measured 4 % slower that way and keeps the three vectors apart: q~ | k~ | b~
     constexpr bool RAW4 = !RESET;
     __shared__ __attribute__((aligned(16))) float raw[2][E][4];
     float(*const rawv)[4][E] = reinterpret_cast<float(*)[4][E]>(raw);   // the layout used when !RAW4
@@ -247,8 +247,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     // are read from the tile one step before they are used (XPREF).  The tile after the current one is
     // then committed when the current one is entered, not when it is left, so that the row to read
     // ahead is always there; both tiles of the double buffer are filled before the loop.  (Measured: the
-    // plain operator gains 6 % at E = 32; the wide output block and the variant with per-step resets,
-    // which hold more in registers, lose 1-4 %, so they read the row where they use it.)
+    // plain operator gains 6 % at E = 32; the wide output block and the variant with per-step resets
+    // lose 1-4 %, so they read the row where they use it.)
     constexpr bool XPREF = E < kWave && !XC && !RESET;
     static_assert(TT >= 4, "a tile's buffer is rewritten two steps after its last row has been read");
     {
