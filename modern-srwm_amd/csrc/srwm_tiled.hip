@@ -960,6 +960,21 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
                     gbw = (p3[0] + p3[1]) + (p3[2] + p3[3]);
                 }
                 gpreb = gbw * btj * (1.f - btj);
+            } else if constexpr (HALF && NCG == 32) {
+                // each 32-lane half is one w_b column (jb; the waves past the fourth column have none and form
+                // a sum nobody uses): it needs the beta gradient of that column alone -- one sum over the 32
+                // column groups instead of three
+                const int j = jb & 3;
+                float gbw = half_sum_each(gbp[par][lane % NCG][j]);
+                if (j == 3) {
+                    float p3[4];
+                    lds_read_vec<4>(p3, &gbp3[par][0]);
+                    gbw = (p3[0] + p3[1]) + (p3[2] + p3[3]);
+                }
+                if constexpr (XC) {
+                    if (j == 0) gbw += gbp3[par][4];
+                }
+                gpreb = gbw * btj * (1.f - btj);
             } else {
                 float gb[4];
                 float part[4];
