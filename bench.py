@@ -43,12 +43,12 @@ HBM_PEAK_GBS = 8000.0
 # figure is carried here with the summary file that holds the runs' commands and counters.
 MEASURED_TRAFFIC = {
     "srwm_c4": ((490441 + 90624) * 1024, "profiles/srwm_c4_kernels.txt"),
-    "srwm_c3": ((26503 + 6400) * 1024, "profiles/srwm_c3_kernels.txt"),
-    "srwm_wide_c3": ((41761 + 8480) * 1024, "profiles/srwm_c3_kernels.txt"),
+    "srwm_c3": ((26513 + 6400) * 1024, "profiles/srwm_c3_kernels.txt"),
+    "srwm_wide_c3": ((41747 + 8480) * 1024, "profiles/srwm_c3_kernels.txt"),
     "delta_c2": ((102515 + 53504) * 1024, "profiles/delta_kernels.txt"),
     "delta_c2_chunk": ((82338 + 85864 + 16640 + 36864) * 1024, "profiles/delta_chunk_kernels.txt"),
     "delta_c5": ((1054057 + 1323008) * 1024, "profiles/delta_kernels.txt"),
-    "delta_c5_chunk": ((784770 + 922425 + 266240 + 532480) * 1024, "profiles/delta_chunk_kernels.txt"),
+    "delta_c5_chunk": ((784769 + 922398 + 266240 + 532480) * 1024, "profiles/delta_chunk_kernels.txt"),
 }
 
 WORKLOADS = {
