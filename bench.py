@@ -380,6 +380,9 @@ def build_workload(name, dev):
         if name.endswith("_chunk"):
             t["fwd_flags"] = srwm_hip.FLAG_CHUNKWISE
             t["bwd_flags"] = srwm_hip.FLAG_CHUNKWISE
+            if op == "delta_bf16":   # as the operator calls it: bf16 gradients, rounded by the kernels themselves
+                for n in ("gq", "gk", "gv"):
+                    t[n] = torch.empty(t[n].shape, device=dev, dtype=torch.bfloat16)
     return step, t
 
 

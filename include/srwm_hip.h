@@ -60,6 +60,12 @@ extern "C" {
                                         forward + backward ~8 % slower).  The memory, v_old, v_insert, grad_V, grad_beta
                                         and dL/dW_0 are formed from operand pairs in either mode.  Accepted and without
                                         effect wherever every product is exact already (fp32 inputs, step-by-step kernels). */
+#define SRWM_FLAG_BF16_GRADS 1024u /* delta_backward_bf16 with SRWM_FLAG_CHUNKWISE only: gQ, gK and gV point to bf16
+                                     buffers (16-bit patterns, same dense layout) and are written rounded to nearest
+                                     even; the second sweep reads grad_V back in bf16, so less memory moves and no
+                                     caller-side rounding pass is needed.  gbeta stays fp32.  Not with
+                                     SRWM_FLAG_EXACT_PRODUCTS and not with gW (the gradient of the memory would be
+                                     accumulated from the rounded grad_V): SRWM_EINVAL. */
 /* srwm_layer_forward_* / srwm_layer_backward_* only: */
 #define SRWM_FLAG_STATE_SHIFT 64u    /* W_y..w_b hold the state MINUS the head's shared weights, on entry and on
                                         exit (how the RL layers carry it, torchbeast/layer.py:389-418) */
@@ -414,10 +420,13 @@ SRWM_API int delta_steps_backward_f32(const float *Q, const int64_t q_strides[3]
  *   W, gW, v_old, v_insert, gQ, gK, gV, gbeta  fp32 (every gradient comes back in fp32: gQ, gK,
  *                                              gbeta may be accumulated by several workgroups
  *                                              and gV is re-read by the chunkwise backward;
- *                                              the caller rounds them if it wants bf16)
+ *                                              the caller rounds them if it wants bf16 -- or sets
+ *                                              SRWM_FLAG_BF16_GRADS, with which gQ, gK, gV are
+ *                                              bf16 buffers that the library rounds into)
  * The memory and all accumulation are fp32; `out` is rounded to nearest even.
  * flags: SRWM_FLAG_CHUNKWISE (and the SRWM_GRAD_STATE_* modes in the backward); with it, the matrix
- * products that only feed out / gQ / gK are single bf16 products unless SRWM_FLAG_EXACT_PRODUCTS is set.
+ * products that only feed out / gQ / gK are single bf16 products unless SRWM_FLAG_EXACT_PRODUCTS is set,
+ * and the backward takes SRWM_FLAG_BF16_GRADS.
  */
 SRWM_API int delta_forward_bf16(const uint16_t *Q, const int64_t q_strides[3],
                        const uint16_t *K, const int64_t k_strides[3],
@@ -433,7 +442,7 @@ SRWM_API int delta_backward_bf16(const uint16_t *Q, const int64_t q_strides[3],
                         const float *v_old, const float *v_insert,
                         const uint16_t *grad_out, const int64_t grad_out_strides[3],
                         float *W,
-                        float *gQ, float *gK, float *gV, float *gbeta, float *gW,
+                        void *gQ, void *gK, void *gV, float *gbeta, float *gW,
                         int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
 /* Largest E the SRWM entry points accept (forward / backward), and the largest
@@ -451,7 +460,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 8. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 9. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

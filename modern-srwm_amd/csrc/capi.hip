@@ -85,7 +85,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 8; }
+int srwm_hip_abi_version(void) { return 9; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -533,24 +533,30 @@ int delta_forward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K
 int delta_backward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K, const int64_t ks[3],
                         const uint16_t *V, const int64_t vs[3], const uint16_t *beta,
                         const int64_t bs[3], const float *v_old, const float *v_insert,
-                        const uint16_t *grad_out, const int64_t gs[3], float *W, float *gQ,
-                        float *gK, float *gV, float *gbeta, float *gW, int N, int H, int L,
+                        const uint16_t *grad_out, const int64_t gs[3], float *W, void *gQ,
+                        void *gK, void *gV, float *gbeta, float *gW, int N, int H, int L,
                         int E, int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !grad_out || !W || !gQ || !gK || !gV ||
         !gbeta || !qs || !ks || !vs || !bs || !gs)
         return SRWM_EINVAL;
     const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u ||
-        (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_GRAD_STATE_MASK)))
+        (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_BF16_GRADS | SRWM_GRAD_STATE_MASK)))
         return SRWM_EINVAL;
     if (!gW && mode != SRWM_GRAD_STATE_ZERO) return SRWM_EINVAL;
+    // rounded gradients: the chunkwise kernels with single products, and no gradient of the memory
+    // (the sweep that would write it takes grad_V back in bf16)
+    if ((flags & SRWM_FLAG_BF16_GRADS) &&
+        (!(flags & SRWM_FLAG_CHUNKWISE) || (flags & SRWM_FLAG_EXACT_PRODUCTS) || gW))
+        return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
         !stride_ok(bs, N, H, L, 1) || !stride_ok(gs, N, H, L, M))
         return SRWM_ESTRIDE;
     DeltaBwdParamsBf16 p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
                          {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, grad_out,
-                         {gs[0], gs[1], gs[2]}, W, gQ, gK, gV, gbeta, gW, N, H, L, E, M, mode,
-                         (flags & SRWM_FLAG_EXACT_PRODUCTS) ? 1u : 0u};
+                         {gs[0], gs[1], gs[2]}, W, static_cast<float *>(gQ), static_cast<float *>(gK),
+                         static_cast<float *>(gV), gbeta, gW, N, H, L, E, M, mode,
+                         (flags & SRWM_FLAG_EXACT_PRODUCTS) ? 1u : 0u, (flags & SRWM_FLAG_BF16_GRADS) ? 1u : 0u};
     const int r = (flags & SRWM_FLAG_CHUNKWISE) ? launch_delta_bwd_chunk_bf16(p, (hipStream_t)stream)
                                                 : launch_delta_bwd_tiled_bf16(p, (hipStream_t)stream);
     return r >= 0 ? r : SRWM_ENOKERNEL;

@@ -128,6 +128,7 @@ struct DeltaBwdParamsBf16 {
     int N, H, L, E, M;
     unsigned grad_state_mode;
     unsigned exact_products;   // chunkwise kernels: every product from hi + lo operand pairs
+    unsigned bf16_grads;       // chunkwise kernels: gQ, gK, gV are bf16 buffers behind the float pointers
 };
 
 // ---- bf16 <-> fp32 (16-bit patterns; round to nearest even on the way down)

@@ -31,6 +31,8 @@
 // Replaces fast_weight_backward_value_beta_kernel and fast_weight_backward_query_key_kernel of
 // the reference (supervised_learning/fast_weight/fast_weight_cuda.cu:397-560, :244-393) for
 // callers that ask for the chunkwise form.
+#include <type_traits>
+
 #include "chunk_mma.h"
 #include "common.h"
 #include "xlane.h"
@@ -55,7 +57,17 @@ struct ChunkBwdP {
     int N, H, L;
     unsigned grad_state_mode;
     bool exact;   // bf16 inputs: also the products that only feed grad_Q / grad_K from hi + lo operand pairs
+    bool bf16_grads;   // bf16 inputs: gQ, gK, gV are bf16 buffers (and the row sweep reads gV back as bf16)
 };
+
+// Gradient stores: fp32 words, or (GB) bf16 rounded to nearest even into the same pointer taken as 16-bit words.
+template <bool GB>
+__device__ __forceinline__ void st_grad(float *g, int64_t i, float v) {
+    if constexpr (GB)
+        reinterpret_cast<uint16_t *>(g)[i] = (uint16_t)pack_bf16_rne(v, 0.f);
+    else
+        g[i] = v;
+}
 
 // ------------------------------------------------------------------------------------------
 // Column sweep
@@ -84,7 +96,8 @@ struct ColLds {
     static_assert(MatK::bytes(C) % 16 == 0 && MatA::bytes(C) % 16 == 0 && MatD::bytes(C) % 16 == 0, "alignment");
 };
 
-template <class TI, int D, int MS, int KS>
+// GB: grad_V goes out in bf16 (the sweep's own dS takes the unrounded value).
+template <class TI, int D, int MS, int KS, bool GB>
 __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(ChunkBwdP<TI> p) {
     typedef ColLds<TI, D, KS> Lds;
     typedef typename Lds::X X;
@@ -287,7 +300,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int t = t0 + a * 16 + 4 * lq + r;
-                    if (t < p.L) p.gV[(seq * p.L + t) * D + m0 + ln] = y[r];
+                    if (t < p.L) st_grad<GB>(p.gV, (seq * p.L + t) * D + m0 + ln, y[r]);
                     gbp[wave * C + a * 16 + 4 * lq + r] = pb[r];   // 16 lanes, same value, same word
                 }
             }
@@ -324,25 +337,27 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 // OB: the products that only feed grad_Q / grad_K (G1, Z, dOut S^T, U dS'^T, Y S^T and those with G1
 // and Z) take the hi parts of their operands alone (precisions with operand parts; without effect
 // otherwise), and G1, Z have no lo part.
-template <class TI, int D, int C, int KS, bool OB>
+// GB: Y = grad_V comes in as bf16 (no lo part), grad_Q and grad_K go out as bf16.
+template <class TI, int D, int C, int KS, bool OB, bool GB>
 struct RowLds {
     typedef typename PrecOf<TI, D>::type X;
     static constexpr int LDM = D + X::kPad, LDW = kWC + X::kPad, LDC = C + X::kPad;
     typedef typename X::template Mat<LDM, false> MatG;   // dOut: an input
-    typedef typename X::template Mat<LDM, true> MatU;    // U, Y: computed
+    typedef typename X::template Mat<LDM, true> MatU;    // U: computed
+    typedef typename X::template Mat<LDM, !GB> MatY;     // Y: computed, unless it arrives rounded
     typedef typename X::template Mat<LDW, false> MatK;   // this workgroup's 64 columns of K, Q
     typedef typename X::template Mat<LDC, !OB> MatC;     // G1, X + X^T: only feed grad_Q / grad_K
     static constexpr int oG = 0;
     static constexpr int oU = oG + MatG::bytes(C);
     static constexpr int oY = oU + MatU::bytes(C);
-    static constexpr int oK = oY + MatU::bytes(C);
+    static constexpr int oK = oY + MatY::bytes(C);
     static constexpr int oQ = oK + MatK::bytes(C);
     static constexpr int oG1 = oQ + MatK::bytes(C);
     static constexpr int oZ = oG1 + MatC::bytes(C);
     static constexpr int oX2 = oZ + MatC::bytes(C);           // KS == 2: [8 waves][C/16/KS tiles][64 lanes] f32x4
     static constexpr int kBytes = oX2 + (KS == 2 ? 8 * (C / 16 / KS) * 64 * 16 : 0);
-    static_assert(MatG::bytes(C) % 16 == 0 && MatU::bytes(C) % 16 == 0 && MatK::bytes(C) % 16 == 0 &&
-                      MatC::bytes(C) % 16 == 0, "alignment");
+    static_assert(MatG::bytes(C) % 16 == 0 && MatU::bytes(C) % 16 == 0 && MatY::bytes(C) % 16 == 0 &&
+                      MatK::bytes(C) % 16 == 0 && MatC::bytes(C) % 16 == 0, "alignment");
 };
 
 // KS = 2: 8 waves; a pair of waves owns the same 16 memory rows and splits their columns (the
@@ -351,9 +366,10 @@ struct RowLds {
 // through LDS (the grad_Q part over the K / Q slices, which are dead by then: their fragments sit
 // in registers; the grad_K part through a buffer of its own, so that one barrier serves both), and
 // finishes grad_Q, grad_K for its own half of the chunk.
-template <class TI, int D, int MS, int C, int KS, bool OB>
+template <class TI, int D, int MS, int C, int KS, bool OB, bool GB>
 __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(ChunkBwdP<TI> p) {
-    typedef RowLds<TI, D, C, KS, OB> Lds;
+    static_assert(!GB || (OB && sizeof(TI) == 2), "rounded gradients: bf16 inputs, single products");
+    typedef RowLds<TI, D, C, KS, OB, GB> Lds;
     typedef typename Lds::X X;
     constexpr int NT = kThreads * KS;
     constexpr int CB = C / 16, MBF = D / 16, MB = MBF / KS, NTRI = CB * (CB + 1) / 2;   // MB: column blocks held by a wave
@@ -362,7 +378,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     static_assert(KS == 1 || (CB % KS == 0 && 8 * CBH * 64 * 16 <= 2 * Lds::MatK::bytes(C)), "exchange buffer");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const typename Lds::MatG Gs(smem + Lds::oG, C);
-    const typename Lds::MatU Us(smem + Lds::oU, C), Ys(smem + Lds::oY, C);
+    const typename Lds::MatU Us(smem + Lds::oU, C);
+    const typename Lds::MatY Ys(smem + Lds::oY, C);
     const typename Lds::MatK Kw(smem + Lds::oK, C), Qw(smem + Lds::oQ, C);
     const typename Lds::MatC G1(smem + Lds::oG1, C), Z(smem + Lds::oZ, C);
 
@@ -382,7 +399,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     const TI *qb = p.Q + n * p.qs.n + h * p.qs.h + e0;
     const TI *kb = p.K + n * p.ks.n + h * p.ks.h + e0;
     const TI *gob = p.go + n * p.gs.n + h * p.gs.h;
-    const float *yb = p.gV + seq * p.L * D;
+    const float *yb = p.gV + seq * p.L * D;                                       // !GB
+    const TI *yb16 = reinterpret_cast<const TI *>(p.gV) + seq * p.L * D;         // GB
     const float *ub = p.vins + seq * p.L * D;
     float *Wg = p.W + seq * D * D + (e0 + cw + ln) * D + m0;       // row e0 + cw + ln of the memory, from column m0
     float *gWg = p.gW ? p.gW + seq * D * D + (e0 + cw + ln) * D + m0 : nullptr;
@@ -407,7 +425,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     constexpr int NK = C * (kWC / 4) / NT;    // ... of the K and Q slices
     static_assert(NG >= 1 && NK >= 1, "chunk too short for the workgroup");
     typename X::Raw4 greg[NG], kreg[NK], qreg[NK];
-    float4 ureg[NG], yreg[NG];
+    float4 ureg[NG];
+    typename std::conditional<GB, typename X::Raw4, float4>::type yreg[NG];
     auto prefetch = [&](int ch) {
         const int t0 = ch * C;
 #pragma unroll
@@ -416,7 +435,10 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
             const int64_t t = min(t0 + row, p.L - 1);
             greg[i] = X::ld_raw(gob + t * p.gs.l + col);
             ureg[i] = *reinterpret_cast<const float4 *>(ub + t * D + col);
-            yreg[i] = *reinterpret_cast<const float4 *>(yb + t * D + col);
+            if constexpr (GB)
+                yreg[i] = X::ld_raw(yb16 + t * D + col);
+            else
+                yreg[i] = *reinterpret_cast<const float4 *>(yb + t * D + col);
         }
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
@@ -436,7 +458,10 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
             const float m = keep ? 1.f : 0.f;
             X::st_raw(Gs, row, col, X::keep_raw(greg[i], keep));
             X::st4(Us, row, col, make_float4(ureg[i].x * m, ureg[i].y * m, ureg[i].z * m, ureg[i].w * m));
-            X::st4(Ys, row, col, make_float4(yreg[i].x * m, yreg[i].y * m, yreg[i].z * m, yreg[i].w * m));
+            if constexpr (GB)
+                X::st_raw(Ys, row, col, X::keep_raw(yreg[i], keep));
+            else
+                X::st4(Ys, row, col, make_float4(yreg[i].x * m, yreg[i].y * m, yreg[i].z * m, yreg[i].w * m));
         }
 #pragma unroll
         for (int i = 0; i < NK; ++i) {
@@ -534,8 +559,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
                 const int t = t0 + cb * 16 + 4 * lq + r;
                 if (t < p.L) {
                     const int64_t o = (seq * p.L + t) * D + e0 + cw + ln;
-                    p.gQ[o] = -dqn[r];
-                    p.gK[o] = dk[r];
+                    st_grad<GB>(p.gQ, o, -dqn[r]);
+                    st_grad<GB>(p.gK, o, dk[r]);
                 }
             }
         };
@@ -573,7 +598,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
             dst[mb] = mma_range<X, false, false>(
                 0, CB, [&](int cb) { return X::lda_t(Gs, cb * 16 + 4 * lq, m0 + mb * 16 + ln); },
                 [&](int cb) { return qbf[cb]; }, dst[mb]);
-            dst[mb] = mma_range<X, true, false>(
+            dst[mb] = mma_range<X, !GB, false>(
                 0, CB, [&](int cb) { return X::lda_t(Ys, cb * 16 + 4 * lq, m0 + mb * 16 + ln); },
                 [&](int cb) { return nkb[cb]; }, dst[mb]);
         }
@@ -607,26 +632,28 @@ __global__ void zero_words_kernel(float *a, int64_t n) {
 }
 
 // KS: waves per memory row / column block in the column sweep, KSR: in the row sweep
-template <class TI, int D, int MS, int C2, int KS, int KSR, bool OB>
+template <class TI, int D, int MS, int C2, int KS, int KSR, bool OB, bool GB>
 int launch_chunk_bwd_ob(const ChunkBwdP<TI> &p, hipStream_t s) {
-    constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2, KSR, OB>::kBytes;
+    constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2, KSR, OB, GB>::kBytes;
     static_assert(lds1 <= (int)kMaxLdsBytes && lds2 <= (int)kMaxLdsBytes, "LDS budget");
-    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_col_kernel<TI, D, MS, KS>>()) return err;
-    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR, OB>>()) return err;
+    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_col_kernel<TI, D, MS, KS, GB>>()) return err;
+    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR, OB, GB>>()) return err;
     const int grid = p.N * p.H * MS;
     if (MS > 1)   // two workgroups of the column sweep add their parts of grad_beta
         hipLaunchKernelGGL(zero_words_kernel, dim3(256), dim3(256), 0, s, p.gbeta, (int64_t)p.N * p.H * p.L);
-    hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS, KS>), dim3(grid), dim3(kThreads * KS), lds1, s, p);
-    hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR, OB>), dim3(grid), dim3(kThreads * KSR), lds2, s, p);
+    hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS, KS, GB>), dim3(grid), dim3(kThreads * KS), lds1, s, p);
+    hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR, OB, GB>), dim3(grid), dim3(kThreads * KSR), lds2, s, p);
     return (int)hipGetLastError();
 }
 
 template <class TI, int D, int MS, int C2, int KS, int KSR>
 int launch_chunk_bwd(const ChunkBwdP<TI> &p, hipStream_t s) {
     if constexpr (PrecOf<TI, D>::type::kBf) {
-        if (!p.exact) return launch_chunk_bwd_ob<TI, D, MS, C2, KS, KSR, true>(p, s);
+        if (!p.exact && p.bf16_grads) return launch_chunk_bwd_ob<TI, D, MS, C2, KS, KSR, true, true>(p, s);
+        if (!p.exact) return launch_chunk_bwd_ob<TI, D, MS, C2, KS, KSR, true, false>(p, s);
     }
-    return launch_chunk_bwd_ob<TI, D, MS, C2, KS, KSR, false>(p, s);
+    if (p.bf16_grads) return -1;   // rounded gradients exist with single products only
+    return launch_chunk_bwd_ob<TI, D, MS, C2, KS, KSR, false, false>(p, s);
 }
 
 template <class TI>
@@ -654,14 +681,14 @@ int dispatch_chunk_bwd(const ChunkBwdP<TI> &p, int D, hipStream_t s) {
 int launch_delta_bwd_chunk(const DeltaBwdParams &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const ChunkBwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
-                             p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode, true};
+                             p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode, true, false};
     return dispatch_chunk_bwd(q, p.E, s);
 }
 
 int launch_delta_bwd_chunk_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const ChunkBwdP<uint16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
-                                p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode, p.exact_products != 0u};
+                                p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode, p.exact_products != 0u, p.bf16_grads != 0u};
     return dispatch_chunk_bwd(q, p.E, s);
 }
 

@@ -31,11 +31,12 @@ GRAD_STATE_ACCUM = 2
 FLAG_GENERIC = 16
 FLAG_CHUNKWISE = 32     # delta forward: chunkwise MFMA kernel (E == M in {64, 128})
 FLAG_EXACT_PRODUCTS = 512   # chunkwise kernels with bf16 inputs: every product from hi + lo operand pairs
+FLAG_BF16_GRADS = 1024      # chunkwise delta backward with bf16 inputs: grad_q, grad_k, grad_v written as bf16 by the library
 FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus the shared weights
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _lib = None
 
@@ -724,11 +725,18 @@ def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, g
     (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr), (gos, gstr) = (
         _strided(t) for t in (q, k, v, beta, grad_out))
     if io == torch.bfloat16:
-        # the library returns every gradient in fp32; bf16 destinations are rounded here
         bf_outs = (grad_q, grad_k, grad_v, grad_beta)
+        # The chunkwise kernels round grad_q, grad_k, grad_v themselves when all three are bf16, no
+        # gradient of the memory is asked for and single products are allowed; grad_beta is fp32 there.
+        native = (bool(flags & FLAG_CHUNKWISE) and not flags & FLAG_EXACT_PRODUCTS and grad_kv is None and
+                  all(t.dtype == torch.bfloat16 for t in bf_outs[:3]))
+        if native:
+            flags |= FLAG_BF16_GRADS
+        # otherwise the library returns every gradient in fp32 and bf16 destinations are rounded here
         grad_q, grad_k, grad_v, grad_beta = (
-            t if t.dtype == torch.float32 else torch.empty(t.shape, device=t.device, dtype=torch.float32)
-            for t in bf_outs)
+            t if t.dtype == torch.float32 or (native and i < 3)
+            else torch.empty(t.shape, device=t.device, dtype=torch.float32)
+            for i, t in enumerate(bf_outs))
     outs = [kv, grad_q, grad_k, grad_v, grad_beta] + ([grad_kv] if grad_kv is not None else [])
     with torch.cuda.device(q.device), _Dense([v_old, v_insert], False) as sv, _Dense(outs, True) as d:
         gkv = _ptr(d[5]) if grad_kv is not None else ctypes.c_void_p(None)

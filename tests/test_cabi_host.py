@@ -144,6 +144,14 @@ def test_argument_validation_needs_no_gpu():
                                                      fake(), fake(), fake(), ok_strides, fake(), fake(), fake(), fake(),
                                                      fake(), gW, N, H, Ls, E, E, flags, P(None))
     assert delta_b(P(None), 1) == -1                           # an incoming state gradient needs the buffer
+    assert delta_b(P(None), 32 | 1024) == -1                   # rounded gradients exist with bf16 inputs only
+    delta_bb = lambda gW, flags, e: L.delta_backward_bf16(*[a for _ in range(4) for a in (fake(), ok_strides)],
+                                                          fake(), fake(), fake(), ok_strides, fake(), fake(), fake(),
+                                                          fake(), fake(), gW, N, H, Ls, e, e, flags, P(None))
+    assert delta_bb(P(None), 1024, E) == -1                    # ... and in the chunkwise kernels only,
+    assert delta_bb(P(None), 32 | 512 | 1024, E) == -1         # with single products,
+    assert delta_bb(fake(), 32 | 1024, E) == -1                # and without the gradient of the memory
+    assert delta_bb(P(None), 32 | 1024, E) == -4               # accepted; SRWM_ENOKERNEL: E = M = 16 has no chunkwise kernel
     layer_f = lambda sw, flags: L.srwm_layer_forward_f32(fake(), ok_strides, P(None), sw, sw, sw, sw,
                                                          *[fake() for _ in range(12)], N, H, Ls, E, E, flags, P(None))
     assert layer_f(P(None), 64) == -1                          # the shift form needs the shared weights

@@ -324,6 +324,56 @@ def test_chunkwise_backward_matches_oracle(shape, qk, w0, io, state_grad):
     assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
 
 
+@pytest.mark.parametrize("shape,qk", [((2, 2, 300, 64, 64), "softmax"), ((1, 3, 512, 128, 128), "l2"),
+                                      ((3, 1, 150, 128, 128), "l2"), ((1, 2, 64, 64, 64), "softmax")])
+def test_chunkwise_backward_with_rounded_gradients(shape, qk):
+    """FLAG_BF16_GRADS: the chunkwise backward writes grad_Q, grad_K, grad_V as bf16 itself and its
+    second sweep reads grad_V back in bf16.  grad_V and grad_beta are those of the fp32-gradient
+    call (grad_V rounded to nearest even, bit for bit: the first sweep computes the same values),
+    grad_Q and grad_K meet the oracle at the bf16 bar and the fp32-gradient call closely, the memory
+    is reverted exactly as there; and the operator takes this path by itself."""
+    print(f"case chunkwise backward, rounded gradients shape={shape}", flush=True)
+    import srwm_hip
+    from fast_weight import fast_weight_delta
+    dev = _dev()
+    q, k, v, beta, W0, go = delta_inputs(*shape, seed=23, qk=qk, w0_std=0.2)
+    qi, ki, vi, bi, goi = (t.to(torch.bfloat16) for t in (q, k, v, beta, go))
+    base = [t.to(torch.float64).numpy() for t in (qi, ki, vi, bi)] + [W0.numpy()]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, goi.to(torch.float64).numpy())
+    N, H, L, E = q.shape
+    qd, kd, vd, bd, god = (t.to(dev) for t in (qi, ki, vi, bi, goi))
+    Wf = W0.to(dev, torch.float32).contiguous()
+    vold, vins = torch.empty(N, H, L, E, device=dev), torch.empty(N, H, L, E, device=dev)
+    out = torch.empty(N, H, L, E, device=dev, dtype=torch.bfloat16)
+    srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, Wf, out, flags=srwm_hip.FLAG_CHUNKWISE)
+    res = {}
+    for name, dt in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        W = Wf.clone()
+        g = [torch.full((N, H, L, w), float("nan"), device=dev, dtype=dt) for w in (E, E, E)]
+        gb = torch.full((N, H, L, 1), float("nan"), device=dev)
+        srwm_hip.fast_weight_backward(qd, kd, vd, bd, vold, vins, god, W, *g, gb, flags=srwm_hip.FLAG_CHUNKWISE)
+        torch.cuda.synchronize()
+        res[name] = g + [gb, W]
+    f, b = res["fp32"], res["bf16"]
+    assert all(t.dtype == torch.bfloat16 for t in b[:3])
+    assert torch.equal(b[2], f[2].to(torch.bfloat16)), "grad_V is the rounded fp32 one"
+    assert torch.equal(b[3], f[3]) and torch.equal(b[4], f[4]), "grad_beta and the reverted memory do not depend on the mode"
+    for i, n in ((0, "grad_Q"), (1, "grad_K"), (2, "grad_V")):
+        e = rel_err(b[i].float().cpu().numpy(), ob[n])
+        assert e < BF16_TOL, (n, e)
+        d = rel_err(b[i].float().cpu().numpy(), f[i].cpu().numpy())
+        assert d < 6e-3, (n, d)          # one bf16 rounding of the result (2^-8) plus the rounded grad_V behind it
+    # the operator: bf16 leaves get bf16 gradients, equal to the ones above
+    leaves = [t.clone().requires_grad_() for t in (qd, kd, vd, bd)]
+    Wop = W0.to(dev, torch.float32).contiguous()
+    fast_weight_delta(*leaves, Wop).backward(god)
+    torch.cuda.synchronize()
+    for i in range(3):
+        assert leaves[i].grad.dtype == torch.bfloat16 and torch.equal(leaves[i].grad, b[i]), i
+    assert torch.equal(leaves[3].grad, f[3].to(torch.bfloat16))
+
+
 @pytest.mark.parametrize("D,L,io,exact", [(64, 70, torch.bfloat16, False), (64, 200, torch.bfloat16, False),
                                           (128, 70, torch.bfloat16, False), (128, 200, torch.bfloat16, False),
                                           (128, 1024, torch.bfloat16, False),
