@@ -48,7 +48,7 @@ MEASURED_TRAFFIC = {
     "delta_c2": ((102515 + 53504) * 1024, "profiles/delta_kernels.txt"),
     "delta_c2_chunk": ((82338 + 85864 + 16640 + 36864) * 1024, "profiles/delta_chunk_kernels.txt"),
     "delta_c5": ((1054057 + 1323008) * 1024, "profiles/delta_kernels.txt"),
-    "delta_c5_chunk": ((784769 + 922398 + 266240 + 532480) * 1024, "profiles/delta_chunk_kernels.txt"),
+    "delta_c5_chunk": ((784770 + 791806 + 135168 + 270336) * 1024, "profiles/delta_chunk_kernels.txt"),
 }
 
 WORKLOADS = {
@@ -70,7 +70,7 @@ WORKLOADS = {
     # same shapes with the chunkwise matrix-core kernels (forward, and the two backward sweeps)
     "delta_c2_chunk": ("delta", 32, 8, 256, 64),
     "delta_c5f32_chunk": ("delta", 8, 16, 4096, 128),
-    "delta_c5_chunk": ("delta_bf16", 8, 16, 4096, 128),
+    "delta_c5_chunk": ("delta_bf16", 8, 16, 4096, 128),   # gradients in bf16 as well (rounded by the kernels)
 }
 
 
@@ -230,7 +230,7 @@ def delta_step(t, ev=None):
         ev[2].record()
 
 
-def algorithmic_bytes(op, N, H, L, E):
+def algorithmic_bytes(op, N, H, L, E, bf16_grads=False):
     """(lds_fwd, lds_bwd, hbm_total) bytes per launch pair."""
     hs = N * H * L
     if op in ("srwm", "srwm_layer"):
@@ -249,9 +249,11 @@ def algorithmic_bytes(op, N, H, L, E):
     S = E * E
     # per (sequence, step): q,k,v,beta in (fwd and bwd), out + grad_out in the I/O type; v_old,
     # v_insert written and read back, and the 3 E-wide gradients + grad_beta written, in fp32
+    # (bf16_grads: the three E-wide gradients in bf16, as the chunkwise bf16 workload writes them)
     b = 2 if op == "delta_bf16" else 4
     io_elems = 2 * (3 * E + 1) + 2 * E
-    return 2 * S * 4 * hs, 4 * S * 4 * hs, (io_elems * b + (4 * E + 3 * E + 1) * 4) * hs + 3 * S * 4 * N * H
+    grads = 3 * E * (2 if bf16_grads else 4) + 4
+    return 2 * S * 4 * hs, 4 * S * 4 * hs, (io_elems * b + 4 * E * 4 + grads) * hs + 3 * S * 4 * N * H
 
 
 def cpu_baseline(op, N, H, L, E, budget_s=20.0):
@@ -420,7 +422,7 @@ def roof(bound, amount, ms, peak, unit="GB/s"):
 def rooflines(name, fwd_ms, bwd_ms):
     """The roofline records of one workload from its median kernel times."""
     op, N, H, L, E = WORKLOADS[name]
-    lds_f, lds_b, hbm = algorithmic_bytes(op, N, H, L, E)
+    lds_f, lds_b, hbm = algorithmic_bytes(op, N, H, L, E, bf16_grads=name.endswith("_chunk") and op == "delta_bf16")
     r = {}
     if name.endswith("_chunk"):
         # the chunkwise kernels are dense contractions: priced in FLOPs against the matrix-core peak
