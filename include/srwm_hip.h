@@ -63,7 +63,10 @@ extern "C" {
 #define SRWM_FLAG_BF16_GRADS 1024u /* delta_backward_bf16 with SRWM_FLAG_CHUNKWISE only: gQ, gK and gV point to bf16
                                      buffers (16-bit patterns, same dense layout) and are written rounded to nearest
                                      even; the second sweep reads grad_V back in bf16, so less memory moves and no
-                                     caller-side rounding pass is needed.  gbeta stays fp32.  Not with
+                                     caller-side rounding pass is needed.  gbeta stays fp32 and is read off that
+                                     sweep's product Y U^T (its diagonal is beta^2 times the sum that grad_beta is;
+                                     single bf16 products, ~1e-3), so V and v_old are not read at all -- except
+                                     for rows with |beta| < 2^-24, which the first sweep forms directly.  Not with
                                      SRWM_FLAG_EXACT_PRODUCTS and not with gW (the gradient of the memory would be
                                      accumulated from the rounded grad_V): SRWM_EINVAL. */
 /* srwm_layer_forward_* / srwm_layer_backward_* only: */

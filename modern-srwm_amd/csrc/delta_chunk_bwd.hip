@@ -60,6 +60,11 @@ struct ChunkBwdP {
     bool bf16_grads;   // bf16 inputs: gQ, gK, gV are bf16 buffers (and the row sweep reads gV back as bf16)
 };
 
+// With rounded gradients (GB) grad_beta is read off the second sweep's own product: Y U^T has
+// beta_t^2 sum_m dR_tm (V - v_old)_tm on its diagonal, so the first sweep needs neither V nor v_old.
+// Rows whose |beta| is below this bound cannot be divided back and take the direct form there.
+constexpr float kTinyBeta = 5.9604645e-8f;   // 2^-24
+
 // Gradient stores: fp32 words, or (GB) bf16 rounded to nearest even into the same pointer taken as 16-bit words.
 template <bool GB>
 __device__ __forceinline__ void st_grad(float *g, int64_t i, float v) {
@@ -96,7 +101,8 @@ struct ColLds {
     static_assert(MatK::bytes(C) % 16 == 0 && MatA::bytes(C) % 16 == 0 && MatD::bytes(C) % 16 == 0, "alignment");
 };
 
-// GB: grad_V goes out in bf16 (the sweep's own dS takes the unrounded value).
+// GB: grad_V goes out in bf16 (the sweep's own dS takes the unrounded value), and grad_beta is left to
+// the row sweep except for rows with |beta| < kTinyBeta, whose V and v_old are fetched when they occur.
 template <class TI, int D, int MS, int KS, bool GB>
 __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(ChunkBwdP<TI> p) {
     typedef ColLds<TI, D, KS> Lds;
@@ -160,14 +166,16 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
                 const int64_t t = min(t0 + cb * 16 + 4 * lq + r, p.L - 1);
                 pg[cb][r] = ld_bits(gob + t * p.gs.l);
             }
+        if constexpr (!GB) {
 #pragma unroll
-        for (int j = 0; j < CB / KS; ++j)
+            for (int j = 0; j < CB / KS; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int64_t t = min(t0 + (j * KS + hf) * 16 + 4 * lq + r, p.L - 1);
-                po[j][r] = vob[t * D];
-                pv[j][r] = ld_bits(vb + t * p.vs.l);
-            }
+                for (int r = 0; r < 4; ++r) {
+                    const int64_t t = min(t0 + (j * KS + hf) * 16 + 4 * lq + r, p.L - 1);
+                    po[j][r] = vob[t * D];
+                    pv[j][r] = ld_bits(vb + t * p.vs.l);
+                }
+        }
         breg = ld_bits(bb + (int64_t)min(t0 + (tid % C), p.L - 1) * p.bs.l);
     };
     f32x4 g[CB], vd[CB / KS];   // this chunk: dOut, V - v_old (rows past the end zeroed)
@@ -188,13 +196,15 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
                 const float m = (full || t0 + cb * 16 + 4 * lq + r < p.L) ? 1.f : 0.f;
                 g[cb][r] = bits_f32<TI>(pg[cb][r]) * m;
             }
+        if constexpr (!GB) {
 #pragma unroll
-        for (int j = 0; j < CB / KS; ++j)
+            for (int j = 0; j < CB / KS; ++j)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float m = (full || t0 + (j * KS + hf) * 16 + 4 * lq + r < p.L) ? 1.f : 0.f;
-                vd[j][r] = (bits_f32<TI>(pv[j][r]) - po[j][r]) * m;
-            }
+                for (int r = 0; r < 4; ++r) {
+                    const float m = (full || t0 + (j * KS + hf) * 16 + 4 * lq + r < p.L) ? 1.f : 0.f;
+                    vd[j][r] = (bits_f32<TI>(pv[j][r]) - po[j][r]) * m;
+                }
+        }
         if (tid < C) bts[tid] = (t0 + tid < p.L) ? bits_f32<TI>(breg) : 0.f;
     };
 
@@ -205,6 +215,24 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
     for (int ch = nchunks - 1; ch >= 0; --ch) {
         const int t0 = ch * C;
         if (ch > 0) prefetch(ch - 1);
+        // grad_beta is formed here (!GB), or only for the rows of this chunk with a tiny beta (the same
+        // answer in every wave: C lanes look at the C betas)
+        static_assert(C == kWave, "one beta per lane");
+        bool gb_here = !GB;
+        if constexpr (GB) {
+            gb_here = __builtin_amdgcn_ballot_w64(fabsf(bts[lane]) < kTinyBeta && t0 + lane < p.L) != 0ull;
+            if (gb_here) {
+#pragma unroll
+                for (int j = 0; j < CB / KS; ++j)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const int row = (j * KS + hf) * 16 + 4 * lq + r;
+                        const int64_t t = min(t0 + row, p.L - 1);
+                        const bool mine = t0 + row < p.L && fabsf(bts[row]) < kTinyBeta;
+                        vd[j][r] = mine ? bits_f32<TI>(ld_bits(vb + t * p.vs.l)) - vob[t * D] : 0.f;
+                    }
+            }
+        }
 
         // ---- (K K^T)^T strict upper and tril(Q K^T)^T: 10 pairs of tiles (a pair shares its right
         //      operand), stored transposed
@@ -293,15 +321,19 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
             for (int r = 0; r < 4; ++r) y[r] = bts[a * 16 + 4 * lq + r] * dr[r];
             nyb[a] = X::accb(-y);
             if (a % KS == hf) {   // wave-uniform: the two waves of a pair share the stores
-                float pb[4];
-#pragma unroll
-                for (int r = 0; r < 4; ++r) pb[r] = dr[r] * vd[a / KS][r];
-                group_sum_n<16, 4>(pb);   // over the wave's 16 columns
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int t = t0 + a * 16 + 4 * lq + r;
                     if (t < p.L) st_grad<GB>(p.gV, (seq * p.L + t) * D + m0 + ln, y[r]);
-                    gbp[wave * C + a * 16 + 4 * lq + r] = pb[r];   // 16 lanes, same value, same word
+                }
+                if (gb_here) {
+                    float pb[4];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) pb[r] = dr[r] * vd[a / KS][r];
+                    group_sum_n<16, 4>(pb);   // over the wave's 16 columns
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        gbp[wave * C + a * 16 + 4 * lq + r] = pb[r];   // 16 lanes, same value, same word
                 }
             }
         }
@@ -316,7 +348,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
                 [&](int cb) { return nyb[cb]; }, ds[eb]);
         }
         __syncthreads();   // every wave is done with the chunk's LDS; grad_beta parts are visible
-        if (tid < C && t0 + tid < p.L) {
+        if (gb_here && tid < C && t0 + tid < p.L && (!GB || fabsf(bts[tid]) < kTinyBeta)) {
             const float sum = gbp[tid] + gbp[C + tid] + gbp[2 * C + tid] + gbp[3 * C + tid];
             if constexpr (MS == 1) {
                 p.gbeta[seq * p.L + t0 + tid] = sum;
@@ -337,7 +369,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 // OB: the products that only feed grad_Q / grad_K (G1, Z, dOut S^T, U dS'^T, Y S^T and those with G1
 // and Z) take the hi parts of their operands alone (precisions with operand parts; without effect
 // otherwise), and G1, Z have no lo part.
-// GB: Y = grad_V comes in as bf16 (no lo part), grad_Q and grad_K go out as bf16.
+// GB: Y = grad_V comes in as bf16 (no lo part), grad_Q and grad_K go out as bf16, and grad_beta is the
+// diagonal of Y U^T over beta^2 (rows with |beta| >= kTinyBeta; the column sweep has written the others).
 template <class TI, int D, int C, int KS, bool OB, bool GB>
 struct RowLds {
     typedef typename PrecOf<TI, D>::type X;
@@ -355,7 +388,8 @@ struct RowLds {
     static constexpr int oG1 = oQ + MatK::bytes(C);
     static constexpr int oZ = oG1 + MatC::bytes(C);
     static constexpr int oX2 = oZ + MatC::bytes(C);           // KS == 2: [8 waves][C/16/KS tiles][64 lanes] f32x4
-    static constexpr int kBytes = oX2 + (KS == 2 ? 8 * (C / 16 / KS) * 64 * 16 : 0);
+    static constexpr int oBt = oX2 + (KS == 2 ? 8 * (C / 16 / KS) * 64 * 16 : 0);   // GB: fp32 [C]: beta
+    static constexpr int kBytes = oBt + (GB ? C * 4 : 0);
     static_assert(MatG::bytes(C) % 16 == 0 && MatU::bytes(C) % 16 == 0 && MatY::bytes(C) % 16 == 0 &&
                       MatK::bytes(C) % 16 == 0 && MatC::bytes(C) % 16 == 0, "alignment");
 };
@@ -385,6 +419,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
 
     f32x4 *Xs = reinterpret_cast<f32x4 *>(smem + Lds::oK);   // KS == 2: [8 waves][CBH tiles][64 lanes]
     f32x4 *Xs2 = reinterpret_cast<f32x4 *>(smem + Lds::oX2);
+    float *bts = reinterpret_cast<float *>(smem + Lds::oBt);   // GB only
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
     const int wave = wv & 3, hf = wv >> 2;           // row block, column half
@@ -402,6 +437,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     const float *yb = p.gV + seq * p.L * D;                                       // !GB
     const TI *yb16 = reinterpret_cast<const TI *>(p.gV) + seq * p.L * D;         // GB
     const float *ub = p.vins + seq * p.L * D;
+    const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
     float *Wg = p.W + seq * D * D + (e0 + cw + ln) * D + m0;       // row e0 + cw + ln of the memory, from column m0
     float *gWg = p.gW ? p.gW + seq * D * D + (e0 + cw + ln) * D + m0 : nullptr;
     const bool g_in = gWg && p.grad_state_mode != 0u;
@@ -427,6 +463,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     typename X::Raw4 greg[NG], kreg[NK], qreg[NK];
     float4 ureg[NG];
     typename std::conditional<GB, typename X::Raw4, float4>::type yreg[NG];
+    uint32_t breg = 0u;
     auto prefetch = [&](int ch) {
         const int t0 = ch * C;
 #pragma unroll
@@ -447,10 +484,14 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
             kreg[i] = X::ld_raw(kb + t * p.ks.l + col);
             qreg[i] = X::ld_raw(qb + t * p.qs.l + col);
         }
+        if constexpr (GB) breg = ld_bits(bb + (int64_t)min(t0 + (tid % C), p.L - 1) * p.bs.l);
     };
     auto commit = [&](int ch) {
         const int t0 = ch * C;
         const bool full = t0 + C <= p.L;
+        if constexpr (GB) {
+            if (tid < C) bts[tid] = bits_f32<TI>(breg);
+        }
 #pragma unroll
         for (int i = 0; i < NG; ++i) {
             const int f = tid + i * NT, row = f / (D / 4), col = (f % (D / 4)) * 4;
@@ -507,6 +548,11 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
                     const int row = ci * 16 + 4 * lq + r;
                     if (col <= row) X::st(Z, row, col, col < row ? accX[r] : 0.f);
                     if (col < row) X::st(Z, col, row, accX[r]);
+                    if constexpr (GB) {   // the diagonal of Y U^T: beta^2 times the sum that grad_beta is
+                        const float bt = bts[row];
+                        if (col == row && part == 0 && t0 + row < p.L && fabsf(bt) >= kTinyBeta)
+                            p.gbeta[seq * p.L + t0 + row] = accX[r] / (bt * bt);
+                    }
                 }
             }
         }

@@ -324,19 +324,28 @@ def test_chunkwise_backward_matches_oracle(shape, qk, w0, io, state_grad):
     assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
 
 
-@pytest.mark.parametrize("shape,qk", [((2, 2, 300, 64, 64), "softmax"), ((1, 3, 512, 128, 128), "l2"),
-                                      ((3, 1, 150, 128, 128), "l2"), ((1, 2, 64, 64, 64), "softmax")])
-def test_chunkwise_backward_with_rounded_gradients(shape, qk):
+@pytest.mark.parametrize("shape,qk,small_betas", [
+    ((2, 2, 300, 64, 64), "softmax", False), ((1, 3, 512, 128, 128), "l2", False),
+    ((3, 1, 150, 128, 128), "l2", False), ((1, 2, 64, 64, 64), "softmax", False),
+    ((2, 2, 300, 64, 64), "softmax", True), ((1, 3, 200, 128, 128), "l2", True)])
+def test_chunkwise_backward_with_rounded_gradients(shape, qk, small_betas):
     """FLAG_BF16_GRADS: the chunkwise backward writes grad_Q, grad_K, grad_V as bf16 itself and its
-    second sweep reads grad_V back in bf16.  grad_V and grad_beta are those of the fp32-gradient
-    call (grad_V rounded to nearest even, bit for bit: the first sweep computes the same values),
-    grad_Q and grad_K meet the oracle at the bf16 bar and the fp32-gradient call closely, the memory
-    is reverted exactly as there; and the operator takes this path by itself."""
-    print(f"case chunkwise backward, rounded gradients shape={shape}", flush=True)
+    second sweep reads grad_V back in bf16.  grad_V is that of the fp32-gradient call rounded to
+    nearest even, bit for bit (the first sweep computes the same values), grad_Q, grad_K and
+    grad_beta (read off the diagonal of the second sweep's Y U^T, divided by beta^2) meet the oracle
+    at the bf16 bar and the fp32-gradient call closely, the memory is reverted exactly as there; and
+    the operator takes this path by itself.  small_betas: some betas are zero or too small to divide
+    by -- those rows of grad_beta come from the first sweep, formed directly."""
+    print(f"case chunkwise backward, rounded gradients shape={shape} small_betas={small_betas}", flush=True)
     import srwm_hip
     from fast_weight import fast_weight_delta
     dev = _dev()
     q, k, v, beta, W0, go = delta_inputs(*shape, seed=23, qk=qk, w0_std=0.2)
+    if small_betas:
+        beta = beta.clone()
+        beta[:, :, ::7] = 0.0
+        beta[:, :, 3::11] = 1e-9
+        beta[:, 0, 128:192] = 0.0      # a whole chunk of one sequence
     qi, ki, vi, bi, goi = (t.to(torch.bfloat16) for t in (q, k, v, beta, go))
     base = [t.to(torch.float64).numpy() for t in (qi, ki, vi, bi)] + [W0.numpy()]
     of = oracle.delta_forward(*base)
@@ -358,8 +367,11 @@ def test_chunkwise_backward_with_rounded_gradients(shape, qk):
     f, b = res["fp32"], res["bf16"]
     assert all(t.dtype == torch.bfloat16 for t in b[:3])
     assert torch.equal(b[2], f[2].to(torch.bfloat16)), "grad_V is the rounded fp32 one"
-    assert torch.equal(b[3], f[3]) and torch.equal(b[4], f[4]), "grad_beta and the reverted memory do not depend on the mode"
-    for i, n in ((0, "grad_Q"), (1, "grad_K"), (2, "grad_V")):
+    assert torch.equal(b[4], f[4]), "the reverted memory does not depend on the mode"
+    if small_betas:   # the rows that the first sweep forms directly are those of the fp32-gradient call
+        tiny = (bi.float().abs() < 2.0 ** -24).to(dev)
+        assert tiny.any() and torch.equal(b[3][tiny], f[3][tiny])
+    for i, n in ((0, "grad_Q"), (1, "grad_K"), (2, "grad_V"), (3, "grad_beta")):
         e = rel_err(b[i].float().cpu().numpy(), ob[n])
         assert e < BF16_TOL, (n, e)
         d = rel_err(b[i].float().cpu().numpy(), f[i].cpu().numpy())
@@ -371,7 +383,7 @@ def test_chunkwise_backward_with_rounded_gradients(shape, qk):
     torch.cuda.synchronize()
     for i in range(3):
         assert leaves[i].grad.dtype == torch.bfloat16 and torch.equal(leaves[i].grad, b[i]), i
-    assert torch.equal(leaves[3].grad, f[3].to(torch.bfloat16))
+    assert torch.equal(leaves[3].grad, b[3].to(torch.bfloat16))
 
 
 @pytest.mark.parametrize("D,L,io,exact", [(64, 70, torch.bfloat16, False), (64, 200, torch.bfloat16, False),
