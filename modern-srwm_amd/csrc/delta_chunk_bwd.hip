@@ -388,8 +388,8 @@ struct RowLds {
     static constexpr int oG1 = oQ + MatK::bytes(C);
     static constexpr int oZ = oG1 + MatC::bytes(C);
     static constexpr int oX2 = oZ + MatC::bytes(C);           // KS == 2: [8 waves][C/16/KS tiles][64 lanes] f32x4
-    static constexpr int oBt = oX2 + (KS == 2 ? 8 * (C / 16 / KS) * 64 * 16 : 0);   // GB: fp32 [C]: beta
-    static constexpr int kBytes = oBt + (GB ? C * 4 : 0);
+    static constexpr int oBt = oX2 + (KS == 2 ? 8 * (C / 16 / KS) * 64 * 16 : 0);   // GB: fp32 [C]: beta, [C]: diagonal of Y U^T
+    static constexpr int kBytes = oBt + (GB ? 2 * C * 4 : 0);
     static_assert(MatG::bytes(C) % 16 == 0 && MatU::bytes(C) % 16 == 0 && MatY::bytes(C) % 16 == 0 &&
                       MatK::bytes(C) % 16 == 0 && MatC::bytes(C) % 16 == 0, "alignment");
 };
@@ -420,6 +420,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     f32x4 *Xs = reinterpret_cast<f32x4 *>(smem + Lds::oK);   // KS == 2: [8 waves][CBH tiles][64 lanes]
     f32x4 *Xs2 = reinterpret_cast<f32x4 *>(smem + Lds::oX2);
     float *bts = reinterpret_cast<float *>(smem + Lds::oBt);   // GB only
+    float *yud = bts + C;                                       // GB only
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
     const int wave = wv & 3, hf = wv >> 2;           // row block, column half
@@ -484,13 +485,15 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
             kreg[i] = X::ld_raw(kb + t * p.ks.l + col);
             qreg[i] = X::ld_raw(qb + t * p.qs.l + col);
         }
-        if constexpr (GB) breg = ld_bits(bb + (int64_t)min(t0 + (tid % C), p.L - 1) * p.bs.l);
+        if constexpr (GB) {   // the last wave's lanes carry the chunk's betas
+            if (tid >= NT - C) breg = ld_bits(bb + (int64_t)min(t0 + tid - (NT - C), p.L - 1) * p.bs.l);
+        }
     };
     auto commit = [&](int ch) {
         const int t0 = ch * C;
         const bool full = t0 + C <= p.L;
         if constexpr (GB) {
-            if (tid < C) bts[tid] = bits_f32<TI>(breg);
+            if (tid >= NT - C) bts[tid - (NT - C)] = bits_f32<TI>(breg);
         }
 #pragma unroll
         for (int i = 0; i < NG; ++i) {
@@ -549,9 +552,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
                     if (col <= row) X::st(Z, row, col, col < row ? accX[r] : 0.f);
                     if (col < row) X::st(Z, col, row, accX[r]);
                     if constexpr (GB) {   // the diagonal of Y U^T: beta^2 times the sum that grad_beta is
-                        const float bt = bts[row];
-                        if (col == row && part == 0 && t0 + row < p.L && fabsf(bt) >= kTinyBeta)
-                            p.gbeta[seq * p.L + t0 + row] = accX[r] / (bt * bt);
+                        if (col == row) yud[row] = accX[r];
                     }
                 }
             }
@@ -574,6 +575,13 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
         }
         // ---- G1 and Z become visible
         __syncthreads();
+        if constexpr (GB) {   // grad_beta of the chunk, by the lanes of the last wave
+            const int row = tid - (NT - C);
+            if (part == 0 && row >= 0 && t0 + row < p.L) {
+                const float bt = bts[row];
+                if (fabsf(bt) >= kTinyBeta) p.gbeta[seq * p.L + t0 + row] = yud[row] / (bt * bt);
+            }
+        }
 
         // ---- grad_Q = dOut S^T + G1 K,  grad_K = G1^T Q + U dS'^T - Y S^T - Z K
         const auto fns = [&](int mb) { return nstb[mb]; };
