@@ -60,10 +60,18 @@ struct ChunkBwdP {
     bool bf16_grads;   // bf16 inputs: gQ, gK, gV are bf16 buffers (and the row sweep reads gV back as bf16)
 };
 
-// With rounded gradients (GB) grad_beta is read off the second sweep's own product: Y U^T has
-// beta_t^2 sum_m dR_tm (V - v_old)_tm on its diagonal, so the first sweep needs neither V nor v_old.
-// Rows whose |beta| is below this bound cannot be divided back and take the direct form there.
+// grad_beta can be read off the second sweep's own product: Y U^T has beta_t^2 sum_m dR_tm (V - v_old)_tm
+// on its diagonal, so the first sweep then needs neither V nor v_old (gathers in accumulator layout,
+// which it waits for).  Rows whose |beta| is below this bound cannot be divided back and take the
+// direct form in the first sweep.
 constexpr float kTinyBeta = 5.9604645e-8f;   // 2^-24
+// Done wherever that product is as accurate as the caller's grad_beta: fp32 inputs (every product at
+// fp32 accuracy) and bf16 inputs with rounded gradients (GB; single bf16 products, ~1e-3).  With bf16
+// inputs and fp32 gradients Y U^T is a single bf16 product while grad_beta is promised to ~1e-5.
+template <class X, bool GB>
+struct RowFormsGradBeta {
+    static constexpr bool value = GB || !X::kBf;
+};
 
 // Gradient stores: fp32 words, or (GB) bf16 rounded to nearest even into the same pointer taken as 16-bit words.
 template <bool GB>
@@ -84,8 +92,9 @@ template <class TI, int D, int KS>
 struct ColLds {
     typedef typename PrecOf<TI, D>::type X;
     static constexpr int C = 64;
-    static constexpr int LDK = D + X::kPad, LDA = C + X::kPad, LDD = 16 + X::kPad;
+    static constexpr int LDK = D + X::kPad, LDA = C + X::kPad, LDD = 16 + X::kPad, LDG = kWC + X::kPad;
     typedef typename X::template Mat<LDK, false> MatK;
+    typedef typename X::template Mat<LDG, false> MatG;   // the workgroup's columns of dOut
     typedef typename X::template Mat<LDA, true> MatA;
     typedef typename X::template Mat<LDD, true> MatD;
     static constexpr int oK = 0;
@@ -97,16 +106,20 @@ struct ColLds {
     static constexpr int oBt = oAd + C * LDD * 4;              // fp32 [C]: beta
     static constexpr int oGb = oBt + C * 4;                    // fp32 [4][C]: per-wave parts of grad_beta
     static constexpr int oX = oGb + 4 * C * 4;                 // KS == 2: [8 waves][C/16 tiles][64 lanes] f32x4
-    static constexpr int kBytes = oX + (KS == 2 ? 8 * (C / 16) * 64 * 16 : 0);
-    static_assert(MatK::bytes(C) % 16 == 0 && MatA::bytes(C) % 16 == 0 && MatD::bytes(C) % 16 == 0, "alignment");
+    static constexpr int oG = oX + (KS == 2 ? 8 * (C / 16) * 64 * 16 : 0);
+    static constexpr int kBytes = oG + MatG::bytes(C);
+    static_assert(MatK::bytes(C) % 16 == 0 && MatA::bytes(C) % 16 == 0 && MatD::bytes(C) % 16 == 0 &&
+                      MatG::bytes(C) % 16 == 0, "alignment");
 };
 
-// GB: grad_V goes out in bf16 (the sweep's own dS takes the unrounded value), and grad_beta is left to
-// the row sweep except for rows with |beta| < kTinyBeta, whose V and v_old are fetched when they occur.
+// GB: grad_V goes out in bf16 (the sweep's own dS takes the unrounded value).  Where the row sweep forms
+// grad_beta (RowFormsGradBeta) only rows with |beta| < kTinyBeta are left here: their V and v_old are
+// fetched when they occur.
 template <class TI, int D, int MS, int KS, bool GB>
 __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(ChunkBwdP<TI> p) {
     typedef ColLds<TI, D, KS> Lds;
     typedef typename Lds::X X;
+    constexpr bool DG = RowFormsGradBeta<X, GB>::value;
     constexpr int NT = kThreads * KS;
     constexpr int C = Lds::C, CB = C / 16, EB = D / 16 / KS, LDD = Lds::LDD;   // EB: row blocks held by this wave
     static_assert(MS * kWC == D, "column split");
@@ -119,6 +132,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
     float *bts = reinterpret_cast<float *>(smem + Lds::oBt);
     float *gbp = reinterpret_cast<float *>(smem + Lds::oGb);
     f32x4 *Xs = reinterpret_cast<f32x4 *>(smem + Lds::oX);
+    const typename Lds::MatG Gs(smem + Lds::oG, C);    // dOut, this workgroup's columns
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
     const int wave = wv & 3, hf = wv >> 2;          // column tile, row half
@@ -132,7 +146,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
     const TI *qb = p.Q + n * p.qs.n + h * p.qs.h;
     const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
     const TI *vb = p.V + n * p.vs.n + h * p.vs.h + m0 + ln;
-    const TI *gob = p.go + n * p.gs.n + h * p.gs.h + m0 + ln;
+    const TI *gob = p.go + n * p.gs.n + h * p.gs.h + part * kWC;
     const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
     const float *vob = p.vold + seq * p.L * D + m0 + ln;
     const float *gWg = (p.gW && p.grad_state_mode != 0u) ? p.gW + seq * D * D + m0 + ln : nullptr;
@@ -144,12 +158,14 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 #pragma unroll
         for (int r = 0; r < 4; ++r) ds[eb][r] = gWg ? gWg[(e0 + eb * 16 + 4 * lq + r) * D] : 0.f;
 
-    // next chunk's inputs: K, Q rows for LDS; dOut, V, v_old directly in accumulator layout
-    constexpr int NKQ = C * (D / 4) / NT;
-    typename X::Raw4 kreg[NKQ], qreg[NKQ];
+    // next chunk's inputs: K, Q and dOut rows for LDS (whole rows: the matrix operands are read from there,
+    // dOut transposed); V, v_old directly in accumulator layout
+    constexpr int NKQ = C * (D / 4) / NT, NGO = C * (kWC / 4) / NT;
+    static_assert(NGO >= 1, "too many threads for the dOut loader");
+    typename X::Raw4 kreg[NKQ], qreg[NKQ], greg[NGO];
     // V and v_old only enter grad_beta: a wave loads them for the row blocks whose results it stores
     f32x4 po[CB / KS];
-    uint32_t pg[CB][4], pv[CB / KS][4], breg = 0u;   // raw bits, converted in commit()
+    uint32_t pv[CB / KS][4], breg = 0u;   // raw bits, converted in commit()
     auto prefetch = [&](int ch) {
         const int t0 = ch * C;
 #pragma unroll
@@ -160,13 +176,11 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
             qreg[i] = X::ld_raw(qb + (int64_t)t * p.qs.l + col);
         }
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const int64_t t = min(t0 + cb * 16 + 4 * lq + r, p.L - 1);
-                pg[cb][r] = ld_bits(gob + t * p.gs.l);
-            }
-        if constexpr (!GB) {
+        for (int i = 0; i < NGO; ++i) {
+            const int f = tid + i * NT, row = f / (kWC / 4), col = (f % (kWC / 4)) * 4;
+            greg[i] = X::ld_raw(gob + (int64_t)min(t0 + row, p.L - 1) * p.gs.l + col);
+        }
+        if constexpr (!DG) {
 #pragma unroll
             for (int j = 0; j < CB / KS; ++j)
 #pragma unroll
@@ -178,7 +192,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
         }
         breg = ld_bits(bb + (int64_t)min(t0 + (tid % C), p.L - 1) * p.bs.l);
     };
-    f32x4 g[CB], vd[CB / KS];   // this chunk: dOut, V - v_old (rows past the end zeroed)
+    f32x4 vd[CB / KS];   // this chunk: V - v_old (rows past the end zeroed)
     auto commit = [&](int ch) {
         const int t0 = ch * C;
         const bool full = t0 + C <= p.L;
@@ -190,13 +204,11 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
             X::st_raw(Qs, row, col, X::keep_raw(qreg[i], keep));
         }
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float m = (full || t0 + cb * 16 + 4 * lq + r < p.L) ? 1.f : 0.f;
-                g[cb][r] = bits_f32<TI>(pg[cb][r]) * m;
-            }
-        if constexpr (!GB) {
+        for (int i = 0; i < NGO; ++i) {
+            const int f = tid + i * NT, row = f / (kWC / 4), col = (f % (kWC / 4)) * 4;
+            X::st_raw(Gs, row, col, X::keep_raw(greg[i], full || t0 + row < p.L));
+        }
+        if constexpr (!DG) {
 #pragma unroll
             for (int j = 0; j < CB / KS; ++j)
 #pragma unroll
@@ -215,11 +227,11 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
     for (int ch = nchunks - 1; ch >= 0; --ch) {
         const int t0 = ch * C;
         if (ch > 0) prefetch(ch - 1);
-        // grad_beta is formed here (!GB), or only for the rows of this chunk with a tiny beta (the same
+        // grad_beta is formed here (!DG), or only for the rows of this chunk with a tiny beta (the same
         // answer in every wave: C lanes look at the C betas)
         static_assert(C == kWave, "one beta per lane");
-        bool gb_here = !GB;
-        if constexpr (GB) {
+        bool gb_here = !DG;
+        if constexpr (DG) {
             gb_here = __builtin_amdgcn_ballot_w64(fabsf(bts[lane]) < kTinyBeta && t0 + lane < p.L) != 0ull;
             if (gb_here) {
 #pragma unroll
@@ -284,7 +296,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
         {
             typename X::B dsb[EB];
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) gob_[cb] = X::accb_exact(g[cb]);
+            for (int cb = 0; cb < CB; ++cb) gob_[cb] = X::ldb_t(Gs, cb * 16 + 4 * lq, 16 * wave + ln);
 #pragma unroll
             for (int eb = 0; eb < EB; ++eb) dsb[eb] = X::accb(ds[eb]);
 #pragma unroll
@@ -348,7 +360,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
                 [&](int cb) { return nyb[cb]; }, ds[eb]);
         }
         __syncthreads();   // every wave is done with the chunk's LDS; grad_beta parts are visible
-        if (gb_here && tid < C && t0 + tid < p.L && (!GB || fabsf(bts[tid]) < kTinyBeta)) {
+        if (gb_here && tid < C && t0 + tid < p.L && (!DG || fabsf(bts[tid]) < kTinyBeta)) {
             const float sum = gbp[tid] + gbp[C + tid] + gbp[2 * C + tid] + gbp[3 * C + tid];
             if constexpr (MS == 1) {
                 p.gbeta[seq * p.L + t0 + tid] = sum;
@@ -369,8 +381,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 // OB: the products that only feed grad_Q / grad_K (G1, Z, dOut S^T, U dS'^T, Y S^T and those with G1
 // and Z) take the hi parts of their operands alone (precisions with operand parts; without effect
 // otherwise), and G1, Z have no lo part.
-// GB: Y = grad_V comes in as bf16 (no lo part), grad_Q and grad_K go out as bf16, and grad_beta is the
-// diagonal of Y U^T over beta^2 (rows with |beta| >= kTinyBeta; the column sweep has written the others).
+// GB: Y = grad_V comes in as bf16 (no lo part), grad_Q and grad_K go out as bf16.  RowFormsGradBeta: grad_beta
+// is the diagonal of Y U^T over beta^2 (rows with |beta| >= kTinyBeta; the column sweep has written the others).
 template <class TI, int D, int C, int KS, bool OB, bool GB>
 struct RowLds {
     typedef typename PrecOf<TI, D>::type X;
@@ -388,8 +400,8 @@ struct RowLds {
     static constexpr int oG1 = oQ + MatK::bytes(C);
     static constexpr int oZ = oG1 + MatC::bytes(C);
     static constexpr int oX2 = oZ + MatC::bytes(C);           // KS == 2: [8 waves][C/16/KS tiles][64 lanes] f32x4
-    static constexpr int oBt = oX2 + (KS == 2 ? 8 * (C / 16 / KS) * 64 * 16 : 0);   // GB: fp32 [C]: beta, [C]: diagonal of Y U^T
-    static constexpr int kBytes = oBt + (GB ? 2 * C * 4 : 0);
+    static constexpr int oBt = oX2 + (KS == 2 ? 8 * (C / 16 / KS) * 64 * 16 : 0);   // grad_beta formed here: fp32 [C]: beta, [C]: diagonal of Y U^T
+    static constexpr int kBytes = oBt + (RowFormsGradBeta<X, GB>::value ? 2 * C * 4 : 0);
     static_assert(MatG::bytes(C) % 16 == 0 && MatU::bytes(C) % 16 == 0 && MatY::bytes(C) % 16 == 0 &&
                       MatK::bytes(C) % 16 == 0 && MatC::bytes(C) % 16 == 0, "alignment");
 };
@@ -405,6 +417,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     static_assert(!GB || (OB && sizeof(TI) == 2), "rounded gradients: bf16 inputs, single products");
     typedef RowLds<TI, D, C, KS, OB, GB> Lds;
     typedef typename Lds::X X;
+    constexpr bool DG = RowFormsGradBeta<X, GB>::value;
     constexpr int NT = kThreads * KS;
     constexpr int CB = C / 16, MBF = D / 16, MB = MBF / KS, NTRI = CB * (CB + 1) / 2;   // MB: column blocks held by a wave
     constexpr int CBH = CB / KS;                                                         // chunk row blocks a wave finishes
@@ -419,8 +432,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
 
     f32x4 *Xs = reinterpret_cast<f32x4 *>(smem + Lds::oK);   // KS == 2: [8 waves][CBH tiles][64 lanes]
     f32x4 *Xs2 = reinterpret_cast<f32x4 *>(smem + Lds::oX2);
-    float *bts = reinterpret_cast<float *>(smem + Lds::oBt);   // GB only
-    float *yud = bts + C;                                       // GB only
+    float *bts = reinterpret_cast<float *>(smem + Lds::oBt);   // DG only
+    float *yud = bts + C;                                       // DG only
 
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
     const int wave = wv & 3, hf = wv >> 2;           // row block, column half
@@ -485,14 +498,14 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
             kreg[i] = X::ld_raw(kb + t * p.ks.l + col);
             qreg[i] = X::ld_raw(qb + t * p.qs.l + col);
         }
-        if constexpr (GB) {   // the last wave's lanes carry the chunk's betas
+        if constexpr (DG) {   // the last wave's lanes carry the chunk's betas
             if (tid >= NT - C) breg = ld_bits(bb + (int64_t)min(t0 + tid - (NT - C), p.L - 1) * p.bs.l);
         }
     };
     auto commit = [&](int ch) {
         const int t0 = ch * C;
         const bool full = t0 + C <= p.L;
-        if constexpr (GB) {
+        if constexpr (DG) {
             if (tid >= NT - C) bts[tid - (NT - C)] = bits_f32<TI>(breg);
         }
 #pragma unroll
@@ -551,7 +564,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
                     const int row = ci * 16 + 4 * lq + r;
                     if (col <= row) X::st(Z, row, col, col < row ? accX[r] : 0.f);
                     if (col < row) X::st(Z, col, row, accX[r]);
-                    if constexpr (GB) {   // the diagonal of Y U^T: beta^2 times the sum that grad_beta is
+                    if constexpr (DG) {   // the diagonal of Y U^T: beta^2 times the sum that grad_beta is
                         if (col == row) yud[row] = accX[r];
                     }
                 }
@@ -575,7 +588,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
         }
         // ---- G1 and Z become visible
         __syncthreads();
-        if constexpr (GB) {   // grad_beta of the chunk, by the lanes of the last wave
+        if constexpr (DG) {   // grad_beta of the chunk, by the lanes of the last wave
             const int row = tid - (NT - C);
             if (part == 0 && row >= 0 && t0 + row < p.L) {
                 const float bt = bts[row];

@@ -324,6 +324,42 @@ def test_chunkwise_backward_matches_oracle(shape, qk, w0, io, state_grad):
     assert not bad, f"over tolerance {tol}: {bad}  (all: {errs})"
 
 
+@pytest.mark.parametrize("shape,qk", [((2, 2, 300, 64, 64), "softmax"), ((1, 3, 200, 128, 128), "l2")])
+def test_chunkwise_backward_with_betas_too_small_to_divide_by(shape, qk):
+    """With fp32 inputs the chunkwise backward reads grad_beta off the diagonal of its second sweep's
+    Y U^T, divided by beta^2; rows whose beta is zero or below 2^-24 are formed directly by the first
+    sweep instead.  Both kinds of row meet the fp64 oracle at the fp32 bar."""
+    print(f"case chunkwise backward, zero and tiny betas shape={shape}", flush=True)
+    import srwm_hip
+    dev = _dev()
+    q, k, v, beta, W0, go = delta_inputs(*shape, seed=29, qk=qk, w0_std=0.2)
+    beta = beta.clone()
+    beta[:, :, ::7] = 0.0
+    beta[:, :, 3::11] = 1e-9
+    beta[:, :, 5::13] = 1e-6          # small, but divided by
+    beta[:, 0, 128:192] = 0.0         # a whole chunk of one sequence
+    q, k, v, beta, go = (t.to(torch.float32) for t in (q, k, v, beta, go))
+    base = [t.to(torch.float64).numpy() for t in (q, k, v, beta)] + [W0.numpy()]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, go.to(torch.float64).numpy())
+    N, H, L, E = q.shape
+    qd, kd, vd, bd, god = (t.to(dev) for t in (q, k, v, beta, go))
+    W = W0.to(dev, torch.float32).contiguous()
+    vold, vins, out = (torch.empty(N, H, L, E, device=dev) for _ in range(3))
+    srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out, flags=srwm_hip.FLAG_CHUNKWISE)
+    g = [torch.full((N, H, L, w), float("nan"), device=dev) for w in (E, E, E, 1)]
+    srwm_hip.fast_weight_backward(qd, kd, vd, bd, vold, vins, god, W, *g, flags=srwm_hip.FLAG_CHUNKWISE)
+    torch.cuda.synchronize()
+    for t, n in zip(g, ("grad_Q", "grad_K", "grad_V", "grad_beta")):
+        e = rel_err(t.cpu().numpy(), ob[n])
+        assert e < TOL, (n, e)
+    gb, ref = g[3].cpu().numpy(), ob["grad_beta"]
+    scale = np.abs(ref).max()
+    for name, rows in (("zero", beta.numpy() == 0.0), ("tiny", beta.numpy() == np.float32(1e-9)),
+                       ("small", beta.numpy() == np.float32(1e-6))):
+        assert rows.any() and np.abs(gb[rows] - ref[rows]).max() < TOL * scale, name
+
+
 @pytest.mark.parametrize("shape,qk,small_betas", [
     ((2, 2, 300, 64, 64), "softmax", False), ((1, 3, 512, 128, 128), "l2", False),
     ((3, 1, 150, 128, 128), "l2", False), ((1, 2, 64, 64, 64), "softmax", False),
