@@ -46,9 +46,9 @@ MEASURED_TRAFFIC = {
     "srwm_c3": ((26513 + 6400) * 1024, "profiles/srwm_c3_kernels.txt"),
     "srwm_wide_c3": ((41747 + 8480) * 1024, "profiles/srwm_c3_kernels.txt"),
     "delta_c2": ((102515 + 53504) * 1024, "profiles/delta_kernels.txt"),
-    "delta_c2_chunk": ((82338 + 85864 + 16640 + 36864) * 1024, "profiles/delta_chunk_kernels.txt"),
+    "delta_c2_chunk": ((49621 + 86137 + 16384 + 37120) * 1024, "profiles/delta_chunk_kernels.txt"),
     "delta_c5": ((1054057 + 1323008) * 1024, "profiles/delta_kernels.txt"),
-    "delta_c5_chunk": ((784770 + 791806 + 135168 + 270336) * 1024, "profiles/delta_chunk_kernels.txt"),
+    "delta_c5_chunk": ((392985 + 792838 + 131072 + 272384) * 1024, "profiles/delta_chunk_kernels.txt"),
 }
 
 WORKLOADS = {
