@@ -65,12 +65,13 @@ struct ChunkBwdP {
 // which it waits for).  Rows whose |beta| is below this bound cannot be divided back and take the
 // direct form in the first sweep.
 constexpr float kTinyBeta = 5.9604645e-8f;   // 2^-24
-// Done wherever that product is as accurate as the caller's grad_beta: fp32 inputs (every product at
-// fp32 accuracy) and bf16 inputs with rounded gradients (GB; single bf16 products, ~1e-3).  With bf16
-// inputs and fp32 gradients Y U^T is a single bf16 product while grad_beta is promised to ~1e-5.
-template <class X, bool GB>
+// Done wherever that product is as accurate as the caller's grad_beta: fp32 inputs and bf16 inputs with
+// operand pairs everywhere (!OB) -- every product at ~1e-5 or better -- and bf16 inputs with rounded
+// gradients (GB; single bf16 products, ~1e-3).  With bf16 inputs, single products and fp32 gradients
+// Y U^T is a single bf16 product while grad_beta is promised to ~1e-5: the direct form stays.
+template <class X, bool OB, bool GB>
 struct RowFormsGradBeta {
-    static constexpr bool value = GB || !X::kBf;
+    static constexpr bool value = GB || !X::kBf || !OB;
 };
 
 // Gradient stores: fp32 words, or (GB) bf16 rounded to nearest even into the same pointer taken as 16-bit words.
@@ -112,14 +113,13 @@ struct ColLds {
                       MatG::bytes(C) % 16 == 0, "alignment");
 };
 
-// GB: grad_V goes out in bf16 (the sweep's own dS takes the unrounded value).  Where the row sweep forms
-// grad_beta (RowFormsGradBeta) only rows with |beta| < kTinyBeta are left here: their V and v_old are
-// fetched when they occur.
-template <class TI, int D, int MS, int KS, bool GB>
+// GB: grad_V goes out in bf16 (the sweep's own dS takes the unrounded value).  DG: the row sweep forms
+// grad_beta (RowFormsGradBeta) and only rows with |beta| < kTinyBeta are left here: their V and v_old
+// are fetched when they occur.
+template <class TI, int D, int MS, int KS, bool GB, bool DG>
 __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(ChunkBwdP<TI> p) {
     typedef ColLds<TI, D, KS> Lds;
     typedef typename Lds::X X;
-    constexpr bool DG = RowFormsGradBeta<X, GB>::value;
     constexpr int NT = kThreads * KS;
     constexpr int C = Lds::C, CB = C / 16, EB = D / 16 / KS, LDD = Lds::LDD;   // EB: row blocks held by this wave
     static_assert(MS * kWC == D, "column split");
@@ -401,7 +401,7 @@ struct RowLds {
     static constexpr int oZ = oG1 + MatC::bytes(C);
     static constexpr int oX2 = oZ + MatC::bytes(C);           // KS == 2: [8 waves][C/16/KS tiles][64 lanes] f32x4
     static constexpr int oBt = oX2 + (KS == 2 ? 8 * (C / 16 / KS) * 64 * 16 : 0);   // grad_beta formed here: fp32 [C]: beta, [C]: diagonal of Y U^T
-    static constexpr int kBytes = oBt + (RowFormsGradBeta<X, GB>::value ? 2 * C * 4 : 0);
+    static constexpr int kBytes = oBt + (RowFormsGradBeta<X, OB, GB>::value ? 2 * C * 4 : 0);
     static_assert(MatG::bytes(C) % 16 == 0 && MatU::bytes(C) % 16 == 0 && MatY::bytes(C) % 16 == 0 &&
                       MatK::bytes(C) % 16 == 0 && MatC::bytes(C) % 16 == 0, "alignment");
 };
@@ -417,7 +417,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_row_kernel(Chunk
     static_assert(!GB || (OB && sizeof(TI) == 2), "rounded gradients: bf16 inputs, single products");
     typedef RowLds<TI, D, C, KS, OB, GB> Lds;
     typedef typename Lds::X X;
-    constexpr bool DG = RowFormsGradBeta<X, GB>::value;
+    constexpr bool DG = RowFormsGradBeta<X, OB, GB>::value;
     constexpr int NT = kThreads * KS;
     constexpr int CB = C / 16, MBF = D / 16, MB = MBF / KS, NTRI = CB * (CB + 1) / 2;   // MB: column blocks held by a wave
     constexpr int CBH = CB / KS;                                                         // chunk row blocks a wave finishes
@@ -702,13 +702,14 @@ __global__ void zero_words_kernel(float *a, int64_t n) {
 template <class TI, int D, int MS, int C2, int KS, int KSR, bool OB, bool GB>
 int launch_chunk_bwd_ob(const ChunkBwdP<TI> &p, hipStream_t s) {
     constexpr int lds1 = ColLds<TI, D, KS>::kBytes, lds2 = RowLds<TI, D, C2, KSR, OB, GB>::kBytes;
+    constexpr bool DG = RowFormsGradBeta<typename PrecOf<TI, D>::type, OB, GB>::value;
     static_assert(lds1 <= (int)kMaxLdsBytes && lds2 <= (int)kMaxLdsBytes, "LDS budget");
-    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_col_kernel<TI, D, MS, KS, GB>>()) return err;
+    if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_col_kernel<TI, D, MS, KS, GB, DG>>()) return err;
     if (const int err = allow_max_dynamic_lds<delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR, OB, GB>>()) return err;
     const int grid = p.N * p.H * MS;
     if (MS > 1)   // two workgroups of the column sweep add their parts of grad_beta
         hipLaunchKernelGGL(zero_words_kernel, dim3(256), dim3(256), 0, s, p.gbeta, (int64_t)p.N * p.H * p.L);
-    hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS, KS, GB>), dim3(grid), dim3(kThreads * KS), lds1, s, p);
+    hipLaunchKernelGGL((delta_bwd_chunk_col_kernel<TI, D, MS, KS, GB, DG>), dim3(grid), dim3(kThreads * KS), lds1, s, p);
     hipLaunchKernelGGL((delta_bwd_chunk_row_kernel<TI, D, MS, C2, KSR, OB, GB>), dim3(grid), dim3(kThreads * KSR), lds2, s, p);
     return (int)hipGetLastError();
 }
