@@ -21,7 +21,7 @@ matrix-core peak.  `cpu_baseline` is the per-timestep PyTorch recurrence (oracle
 timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk}.
+{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (the last through the autograd operator)}.
 """
 import argparse
 import json
@@ -71,6 +71,9 @@ WORKLOADS = {
     "delta_c2_chunk": ("delta", 32, 8, 256, 64),
     "delta_c5f32_chunk": ("delta", 8, 16, 4096, 128),
     "delta_c5_chunk": ("delta_bf16", 8, 16, 4096, 128),   # gradients in bf16 as well (rounded by the kernels)
+    # the same through the autograd operator fast_weight_delta (allocations, saved tensors and the autograd
+    # engine inside the timed steps): what a model that calls the operator gets
+    "delta_c5_op_chunk": ("delta_bf16", 8, 16, 4096, 128),
 }
 
 
@@ -230,6 +233,21 @@ def delta_step(t, ev=None):
         ev[2].record()
 
 
+def delta_op_step(t, ev=None):
+    from fast_weight import fast_weight_delta
+    t["W"].zero_()
+    if ev:
+        ev[0].record()
+    out = fast_weight_delta(t["q"], t["k"], t["v"], t["beta"], t["W"])
+    if ev:
+        ev[1].record()
+    out.backward(t["go"])
+    if ev:
+        ev[2].record()
+    for n in ("q", "k", "v", "beta"):
+        t[n].grad = None
+
+
 def algorithmic_bytes(op, N, H, L, E, bf16_grads=False):
     """(lds_fwd, lds_bwd, hbm_total) bytes per launch pair."""
     hs = N * H * L
@@ -379,7 +397,11 @@ def build_workload(name, dev):
     else:
         step = delta_step
         t = delta_setup(N, H, L, E, dev, torch.bfloat16 if op == "delta_bf16" else torch.float32)
-        if name.endswith("_chunk"):
+        if "_op_" in name:   # the operator picks the chunkwise kernels and bf16 gradients by itself
+            step = delta_op_step
+            for n in ("q", "k", "v", "beta"):
+                t[n].requires_grad_()
+        elif name.endswith("_chunk"):
             t["fwd_flags"] = srwm_hip.FLAG_CHUNKWISE
             t["bwd_flags"] = srwm_hip.FLAG_CHUNKWISE
             if op == "delta_bf16":   # as the operator calls it: bf16 gradients, rounded by the kernels themselves
@@ -451,7 +473,7 @@ def rooflines(name, fwd_ms, bwd_ms):
 
 # Driver-visible figures for the other benchmark configurations: (workload, timed steps, warm-up)
 OTHER_WORKLOADS = (("srwm_layer_c4", 50, 10), ("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
-                   ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5))
+                   ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5), ("delta_c5_op_chunk", 40, 5))
 
 
 def main():
