@@ -21,7 +21,7 @@ matrix-core peak.  `cpu_baseline` is the per-timestep PyTorch recurrence (oracle
 timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (the last through the autograd operator)}.
+{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (through the autograd operator), delta_prologue_c2 (the layers' prologue kernels, HBM-bound)}.
 """
 import argparse
 import json
@@ -74,6 +74,9 @@ WORKLOADS = {
     # the same through the autograd operator fast_weight_delta (allocations, saved tensors and the autograd
     # engine inside the timed steps): what a model that calls the operator gets
     "delta_c5_op_chunk": ("delta_bf16", 8, 16, 4096, 128),
+    # the prologue of the delta-rule layers at the shape of configuration 2 (projection rows [q~ | k~ | v | b~] ->
+    # normalised q, k, v, beta) and its backward: two memory-bound launches, priced against HBM
+    "delta_prologue_c2": ("delta_prologue", 32, 8, 256, 64),
 }
 
 
@@ -248,9 +251,37 @@ def delta_op_step(t, ev=None):
         t[n].grad = None
 
 
+def delta_prologue_setup(N, H, L, E, dev):
+    import torch
+    g = torch.Generator().manual_seed(0)
+    W = 3 * E + 1
+    t = dict(rows=torch.randn(L, N, H, W, generator=g).to(dev))
+    for n, w in (("gq", E), ("gk", E), ("gv", E), ("gb", 1)):
+        t[n] = torch.randn(N, H, L, w, generator=g).to(dev)
+    return t
+
+
+def delta_prologue_step(t, ev=None):
+    import srwm_hip
+    E = t["gq"].shape[-1]
+    if ev:
+        ev[0].record()
+    q, k, v, beta, sums = srwm_hip.delta_layer_prologue(t["rows"], E, E)
+    if ev:
+        ev[1].record()
+    srwm_hip.delta_layer_prologue_grad(t["gq"], t["gk"], t["gv"], t["gb"], q, k, beta, sums)
+    if ev:
+        ev[2].record()
+
+
 def algorithmic_bytes(op, N, H, L, E, bf16_grads=False):
     """(lds_fwd, lds_bwd, hbm_total) bytes per launch pair."""
     hs = N * H * L
+    if op == "delta_prologue":
+        # forward: the row in, q, k, v, beta and the two normalisers out; backward: the four gradients, q, k,
+        # beta and the normalisers in, the row's gradient out.  No state: nothing to pass over in LDS.
+        W = 3 * E + 1
+        return 0, 0, ((W + W + 2) + (W + 2 * E + 3 + W)) * 4 * hs
     if op in ("srwm", "srwm_layer"):
         S = E * (3 * E + 4)
         return 3 * S * 4 * hs, 6 * S * 4 * hs, (15 * E + 16) * 4 * hs + 4 * S * 4 * N * H
@@ -394,6 +425,8 @@ def build_workload(name, dev):
         step, t = srwm_step, srwm_setup(N, H, L, E, dev, 3 * E + 1)
     elif op == "srwm_steps":
         step, t = srwm_steps_step, srwm_steps_setup(N, H, L, E, dev)
+    elif op == "delta_prologue":
+        step, t = delta_prologue_step, delta_prologue_setup(N, H, L, E, dev)
     else:
         step = delta_step
         t = delta_setup(N, H, L, E, dev, torch.bfloat16 if op == "delta_bf16" else torch.float32)
@@ -446,6 +479,13 @@ def rooflines(name, fwd_ms, bwd_ms):
     op, N, H, L, E = WORKLOADS[name]
     lds_f, lds_b, hbm = algorithmic_bytes(op, N, H, L, E, bf16_grads=name.endswith("_chunk") and op == "delta_bf16")
     r = {}
+    if op == "delta_prologue":
+        W = 3 * E + 1
+        hs = N * H * L
+        r["roofline"] = dict(roof("hbm", (W + 2 * E + 3 + W) * 4 * hs, bwd_ms, HBM_PEAK_GBS), kernel="backward")
+        r["roofline_fwd"] = dict(roof("hbm", (W + W + 2) * 4 * hs, fwd_ms, HBM_PEAK_GBS), kernel="forward")
+        r["roofline_fwd_bwd"] = roof("hbm", hbm, fwd_ms + bwd_ms, HBM_PEAK_GBS)
+        return r
     if name.endswith("_chunk"):
         # the chunkwise kernels are dense contractions: priced in FLOPs against the matrix-core peak
         ff, fb = chunk_flops(N, H, L, E)
@@ -473,7 +513,7 @@ def rooflines(name, fwd_ms, bwd_ms):
 
 # Driver-visible figures for the other benchmark configurations: (workload, timed steps, warm-up)
 OTHER_WORKLOADS = (("srwm_layer_c4", 50, 10), ("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
-                   ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5), ("delta_c5_op_chunk", 40, 5))
+                   ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5), ("delta_c5_op_chunk", 40, 5), ("delta_prologue_c2", 100, 20))
 
 
 def main():

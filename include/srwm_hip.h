@@ -69,6 +69,8 @@ extern "C" {
                                      for rows with |beta| < 2^-24, which the first sweep forms directly.  Not with
                                      SRWM_FLAG_EXACT_PRODUCTS and not with gW (the gradient of the memory would be
                                      accumulated from the rounded grad_V): SRWM_EINVAL. */
+#define SRWM_FLAG_NORM_EPS 2048u   /* delta_layer_prologue_f32 only: 1e-5 is added to the normalisers of q and k (the RL
+                                     tree's layers, reinforcement_learning/torchbeast/layer.py:30-33) */
 /* srwm_layer_forward_* / srwm_layer_backward_* only: */
 #define SRWM_FLAG_STATE_SHIFT 64u    /* W_y..w_b hold the state MINUS the head's shared weights, on entry and on
                                         exit (how the RL layers carry it, torchbeast/layer.py:389-418) */
@@ -448,6 +450,31 @@ SRWM_API int delta_backward_bf16(const uint16_t *Q, const int64_t q_strides[3],
                         void *gQ, void *gK, void *gV, float *gbeta, float *gW,
                         int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
+/*
+ * Prologue of the delta-rule layers in one pass, and its backward in one pass.  The layers project their
+ * input to one row [q~ | k~ | v | b~] of 2E + M + 1 floats per (step, batch row, head) and reach the
+ * operator's arguments through a chain of tensor operations (supervised_learning/layer.py:72-90;
+ * reinforcement_learning/torchbeast/layer.py:149-165, :219-236):
+ *     q = a(q~) / sum_e a(q~),  k likewise,  a(x) = elu(x) + 1,  beta = sigmoid(b~)
+ * (with SRWM_FLAG_NORM_EPS: 1e-5 added to the sums).  No counterpart among the reference's kernels: there
+ * these are about twenty elementwise / reduction launches forward and backward.
+ *   rows       dense [L, N, H, 2E+M+1]: the projection as the layer's linear map leaves it
+ *   q, k       dense [L, N, H, E];  v dense [L, N, H, M];  beta dense [L, N, H]  (the operator reads them
+ *              as [N, H, L, .] through strides (H*w, w, N*H*w))
+ *   sums       dense [L, N, H, 2]: the two normalisers, for the backward
+ *   gq, gk, gv, gbeta   strided [N, H, L, .]: the operator's gradients
+ *   grad_rows  dense [L, N, H, 2E+M+1]: the gradient of `rows`
+ */
+SRWM_API int delta_layer_prologue_f32(const float *rows, float *q, float *k, float *v, float *beta, float *sums,
+                             int N, int H, int L, int E, int M, unsigned flags, void *stream);
+SRWM_API int delta_layer_prologue_grad_f32(const float *gq, const int64_t gq_strides[3],
+                                  const float *gk, const int64_t gk_strides[3],
+                                  const float *gv, const int64_t gv_strides[3],
+                                  const float *gbeta, const int64_t gbeta_strides[3],
+                                  const float *q, const float *k, const float *beta, const float *sums,
+                                  float *grad_rows,
+                                  int N, int H, int L, int E, int M, unsigned flags, void *stream);
+
 /* Largest E the SRWM entry points accept (forward / backward), and the largest
  * E == M the delta entry points accept, on the current device. */
 SRWM_API int srwm_hip_limits(int *srwm_fwd_max_E, int *srwm_bwd_max_E, int *delta_max_EM);
@@ -463,7 +490,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 9. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 10. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

@@ -85,7 +85,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 9; }
+int srwm_hip_abi_version(void) { return 10; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -313,6 +313,31 @@ int delta_steps_backward_f32(const float *Q, const int64_t qs[3], const float *K
                           {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, {gs[0], gs[1], gs[2]}, v_old, v_insert,
                           gQ, gK, gV, gbeta, N, H, L, E, M};
     return launch_delta_step_grads(p, (hipStream_t)stream);
+}
+
+int delta_layer_prologue_f32(const float *rows, float *q, float *k, float *v, float *beta, float *sums, int N, int H,
+                             int L, int E, int M, unsigned flags, void *stream) {
+    if (!rows || !q || !k || !v || !beta || !sums) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_NORM_EPS)) return SRWM_EINVAL;
+    const int r = launch_delta_prologue(rows, q, k, v, beta, sums, N, H, L, E, M,
+                                        (flags & SRWM_FLAG_NORM_EPS) ? 1e-5f : 0.f, (hipStream_t)stream);
+    return r >= 0 ? r : SRWM_ESIZE;
+}
+
+int delta_layer_prologue_grad_f32(const float *gq, const int64_t gqs[3], const float *gk, const int64_t gks[3],
+                                  const float *gv, const int64_t gvs[3], const float *gbeta, const int64_t gbs[3],
+                                  const float *q, const float *k, const float *beta, const float *sums,
+                                  float *grad_rows, int N, int H, int L, int E, int M, unsigned flags, void *stream) {
+    if (!gq || !gk || !gv || !gbeta || !q || !k || !beta || !sums || !grad_rows || !gqs || !gks || !gvs || !gbs)
+        return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || flags) return SRWM_EINVAL;
+    if (!stride_ok(gqs, N, H, L, E) || !stride_ok(gks, N, H, L, E) || !stride_ok(gvs, N, H, L, M) ||
+        !stride_ok(gbs, N, H, L, 1))
+        return SRWM_ESTRIDE;
+    const int r = launch_delta_prologue_grad(gq, {gqs[0], gqs[1], gqs[2]}, gk, {gks[0], gks[1], gks[2]}, gv,
+                                             {gvs[0], gvs[1], gvs[2]}, gbeta, {gbs[0], gbs[1], gbs[2]}, q, k, beta,
+                                             sums, grad_rows, N, H, L, E, M, (hipStream_t)stream);
+    return r >= 0 ? r : SRWM_ESIZE;
 }
 
 int srwm_backward_wide_f32(const float *x, const int64_t xs[3], const float *q, const float *k,

@@ -196,6 +196,14 @@ int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s);
 // dst[j][h, :] = sum over n of src[j][n, h, :] for the four state tensors (y: E x Y, q, k: E x E, b: E x 4)
 int launch_srwm_batch_sum(const float *const src[4], float *const dst[4], int N, int H, int E, int Y, hipStream_t s);
 int launch_batch_sum(const float *src, float *dst, int N, int64_t len, hipStream_t s);   // dst[i] = sum_n src[n][i]
+// Prologue of the delta-rule layers (rows [q~ | k~ | v | b~] -> normalised q, k; v; beta) and its backward; -1 if
+// the grid would not fit.
+int launch_delta_prologue(const float *x, float *q, float *k, float *v, float *beta, float *sums, int N, int H,
+                          int L, int E, int M, float eps, hipStream_t s);
+int launch_delta_prologue_grad(const float *gq, const Strided3 &gqs, const float *gk, const Strided3 &gks,
+                               const float *gv, const Strided3 &gvs, const float *gb, const Strided3 &gbs,
+                               const float *q, const float *k, const float *beta, const float *sums, float *gx,
+                               int N, int H, int L, int E, int M, hipStream_t s);
 int launch_delta_fwd_generic(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_bwd_generic(const DeltaBwdParams &p, hipStream_t s);
 

@@ -87,6 +87,39 @@ class DeltaFastWeight(torch.autograd.Function):
 fast_weight_delta = DeltaFastWeight.apply
 
 
+class DeltaLayerInputs(torch.autograd.Function):
+    """The prologue of the delta-rule layers in one launch (and one for its backward) instead of the
+    chain of tensor operations of supervised_learning/layer.py:72-90 and
+    reinforcement_learning/torchbeast/layer.py:149-165:
+
+        q, k, v, beta = delta_layer_inputs(qkvb, E, M, eps)
+
+    qkvb: (len, B, H, 2E+M+1) float32 -- the projection [q~ | k~ | v | b~]; returns the operator's
+    arguments q, k: (B, H, len, E) = sum_norm(elu(.) + 1) (the sum plus 1e-5 when `eps`), v: (B, H, len, M),
+    beta: (B, H, len, 1) = sigmoid, as permuted views of dense (len, B, H, .) tensors."""
+
+    @staticmethod
+    def forward(ctx, qkvb, E, M, eps):
+        q, k, v, beta, sums = srwm_hip.delta_layer_prologue(qkvb.contiguous(), E, M, eps)
+        ctx.save_for_backward(q, k, beta, sums)
+        ctx.v_width = M
+        return q.permute(1, 2, 0, 3), k.permute(1, 2, 0, 3), v.permute(1, 2, 0, 3), beta.unsqueeze(-1).permute(1, 2, 0, 3)
+
+    @staticmethod
+    def backward(ctx, grad_q, grad_k, grad_v, grad_beta):
+        q, k, beta, sums = ctx.saved_tensors
+        L, N, H, E = q.shape
+        zeros = lambda w: torch.zeros((N, H, L, w), device=q.device, dtype=torch.float32)
+        grad_q = zeros(E) if grad_q is None else grad_q
+        grad_k = zeros(E) if grad_k is None else grad_k
+        grad_beta = zeros(1) if grad_beta is None else grad_beta
+        grad_v = zeros(ctx.v_width) if grad_v is None else grad_v
+        return srwm_hip.delta_layer_prologue_grad(grad_q, grad_k, grad_v, grad_beta, q, k, beta, sums), None, None, None
+
+
+delta_layer_inputs = DeltaLayerInputs.apply
+
+
 class DeltaFastWeightSteps(torch.autograd.Function):
     """All time steps of an RL unroll in one launch, with the semantics of calling
     `fast_weight_delta` once per step on `memory * notdone` (reinforcement_learning/

@@ -18,7 +18,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from fast_weight import fast_weight_delta, fast_weight_delta_steps
+from fast_weight import delta_layer_inputs, fast_weight_delta, fast_weight_delta_steps
 from self_ref_v0 import self_ref_layer, self_ref_layer_steps, self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
 from self_ref_v1 import self_ref_v1, self_ref_v1_steps
 
@@ -27,6 +27,10 @@ from self_ref_v1 import self_ref_v1, self_ref_v1_steps
 # carried shift and batch-summed weight gradients inside the kernels).  False: they spell the
 # reference's tensor operations out around the plain operator; both give the same results.
 FUSED_SRWM_LAYER = True
+# True: the delta-rule layers turn their projection into the operator's arguments (elu + 1, sum
+# normalisation, sigmoid, the permuted views) with one kernel, and its gradient with another.  False:
+# the reference's chain of tensor operations; both give the same results.
+FUSED_DELTA_LAYER = True
 
 
 def elu_p1(x):
@@ -258,6 +262,18 @@ class SMFWPlayer(nn.Module):
         return out, tuple(new_state) + (memory,)
 
 
+def _delta_inputs(qkvb, E, M, eps):
+    """(len, B, H, 2E+M+1) projection -> q, k, v, beta as (B, H, len, .): supervised_learning/layer.py:74-90,
+    reinforcement_learning/torchbeast/layer.py:152-165."""
+    if FUSED_DELTA_LAYER and qkvb.is_cuda and qkvb.dtype == torch.float32:
+        return delta_layer_inputs(qkvb, E, M, eps)
+    q, k, v, beta = torch.split(qkvb, (E, E, M, 1), -1)
+    beta = torch.sigmoid(beta)
+    q, k, v, beta = (t.permute(1, 2, 0, 3) for t in (q, k, v, beta))
+    normalise = elu_p1_sum_norm_eps if eps else (lambda t: sum_norm(elu_p1(t)))
+    return normalise(q), normalise(k), v, beta
+
+
 class _DeltaBase(nn.Module):
     def __init__(self, num_head, dim_head, in_dim, dropout):
         super().__init__()
@@ -270,13 +286,11 @@ class _DeltaBase(nn.Module):
         self.out_linear = nn.Linear(num_head * dim_head, in_dim, bias=False)
         self.drop = nn.Dropout(dropout)
 
-    def _qkvb(self, x, normalise):
+    def _qkvb(self, x, eps):
+        """eps: the normaliser of q and k is their sum plus 1e-5 (the RL tree's layers) or the sum alone."""
         slen, bsz, _ = x.size()
         qkvb = self.slow_net(self.layer_norm(x)).view(slen, bsz, self.num_head, 3 * self.dim_head + 1)
-        q, k, v, beta = torch.split(qkvb, (self.dim_head,) * 3 + (1,), -1)
-        beta = torch.sigmoid(beta)
-        q, k, v, beta = (t.permute(1, 2, 0, 3) for t in (q, k, v, beta))
-        return normalise(q), normalise(k), v, beta, slen, bsz
+        return _delta_inputs(qkvb, self.dim_head, self.dim_head, eps) + (slen, bsz)
 
     def _finish(self, x, out, bsz, slen):
         out = _heads_out(out, bsz, slen, self.num_head * self.dim_head)
@@ -287,7 +301,7 @@ class FastFFlayer(_DeltaBase):
     """Supervised delta-rule layer: the memory starts from zero at every call."""
 
     def forward(self, x):
-        q, k, v, beta, slen, bsz = self._qkvb(x, lambda t: sum_norm(elu_p1(t)))
+        q, k, v, beta, slen, bsz = self._qkvb(x, False)
         fast_weights = torch.zeros(bsz, self.num_head, self.dim_head, self.dim_head, device=k.device)
         out = self.fw_layer(q, k, v, beta, fast_weights)
         return self._finish(x, out, bsz, slen)
@@ -298,7 +312,7 @@ class CarryFastFFlayer(_DeltaBase):
 
     def forward(self, x, state=None):
         assert state is not None
-        q, k, v, beta, slen, bsz = self._qkvb(x, elu_p1_sum_norm_eps)
+        q, k, v, beta, slen, bsz = self._qkvb(x, True)
         fast_weights = state
         out = self.fw_layer(q, k, v, beta, fast_weights)
         return self._finish(x, out, bsz, slen), fast_weights.clone()
@@ -308,7 +322,7 @@ class CarryFastFFlayer(_DeltaBase):
         x[t:t+1] with the memory multiplied by notdone[t] first (the learner's loop,
         reinforcement_learning/torchbeast_procgen/model.py:1176-1196).  x: (T, B, D); notdone: (T, B)."""
         assert state is not None
-        q, k, v, beta, slen, bsz = self._qkvb(x, elu_p1_sum_norm_eps)
+        q, k, v, beta, slen, bsz = self._qkvb(x, True)
         keep = notdone.to(x.dtype).transpose(0, 1).contiguous()
         fast_weights = state.detach().clone()
         out = fast_weight_delta_steps(q, k, v, beta, keep, fast_weights)
@@ -341,11 +355,9 @@ class FastFastFFlayer(nn.Module):
         slen, bsz, _ = x.size()
         d = self.dim_head
         qkvb = self.slow_net(self.layer_norm(x)).view(slen, bsz, self.num_head, 5 * d + 2)
-        q, k, v, beta = torch.split(qkvb, (d, d, 3 * d + 1, 1), -1)
-        beta = torch.sigmoid(beta)
-        q, k, v, beta = (t.permute(1, 2, 0, 3) for t in (q, k, v, beta))
+        q, k, v, beta = _delta_inputs(qkvb, d, 3 * d + 1, True)
         fast_weights, very_fast_weights = state
-        out = self.fw_layer(elu_p1_sum_norm_eps(q), elu_p1_sum_norm_eps(k), v, beta, fast_weights)
+        out = self.fw_layer(q, k, v, beta, fast_weights)
         fq, fk, fv, fbeta = torch.split(out, (d,) * 3 + (1,), -1)
         out = self.very_fw_layer(elu_p1_sum_norm_eps(fq), elu_p1_sum_norm_eps(fk), fv, torch.sigmoid(fbeta),
                                  very_fast_weights)

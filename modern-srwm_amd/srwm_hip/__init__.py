@@ -32,11 +32,12 @@ FLAG_GENERIC = 16
 FLAG_CHUNKWISE = 32     # delta forward: chunkwise MFMA kernel (E == M in {64, 128})
 FLAG_EXACT_PRODUCTS = 512   # chunkwise kernels with bf16 inputs: every product from hi + lo operand pairs
 FLAG_BF16_GRADS = 1024      # chunkwise delta backward with bf16 inputs: grad_q, grad_k, grad_v written as bf16 by the library
+FLAG_NORM_EPS = 2048        # delta_layer_prologue: 1e-5 added to the normalisers of q and k
 FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus the shared weights
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 _lib = None
 
@@ -68,6 +69,8 @@ _SIGNATURES = {
     "delta_backward_f32": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_forward_bf16": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_backward_bf16": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_layer_prologue_f32": [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_layer_prologue_grad_f32": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
 }
 
 
@@ -682,6 +685,51 @@ def fast_weight_steps_backward(q, k, v, beta, keep, v_old, v_insert, grad_out, k
             _ptr(sv[0]), _ptr(sv[1]), _ptr(gos), gstr, _ptr(sv[2]), *[_ptr(t) for t in d], N, H, L, E, M, flags,
             _stream(q.device))
     _check(code, "delta_steps_backward_f32")
+
+
+def delta_layer_prologue(rows, E, M, eps=False):
+    """rows: (L, N, H, 2E+M+1) float32, contiguous -- the delta-rule layers' projection [q~ | k~ | v | b~].
+    Returns q, k: (L, N, H, E) normalised (elu + 1 over its sum, plus 1e-5 when `eps`), v: (L, N, H, M),
+    beta: (L, N, H) = sigmoid, sums: (L, N, H, 2), all freshly allocated and contiguous, from one launch."""
+    _require(rows, "rows")
+    L, N, H, W = rows.shape
+    if W != 2 * E + M + 1 or not rows.is_contiguous():
+        raise ValueError(f"rows must be contiguous with last axis 2E+M+1 = {2 * E + M + 1} (got {tuple(rows.shape)})")
+    new = lambda *sh: torch.empty(sh, device=rows.device, dtype=torch.float32)
+    q, k, v, beta, sums = new(L, N, H, E), new(L, N, H, E), new(L, N, H, M), new(L, N, H), new(L, N, H, 2)
+    if rows.numel():
+        with torch.cuda.device(rows.device):
+            code = lib().delta_layer_prologue_f32(_ptr(rows), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(sums),
+                                                  N, H, L, E, M, FLAG_NORM_EPS if eps else 0, _stream(rows.device))
+        _check(code, "delta_layer_prologue_f32")
+    return q, k, v, beta, sums
+
+
+def delta_layer_prologue_grad(grad_q, grad_k, grad_v, grad_beta, q, k, beta, sums):
+    """Backward of delta_layer_prologue.  grad_q, grad_k: (N, H, L, E), grad_v: (N, H, L, M), grad_beta:
+    (N, H, L, 1), any strides with a contiguous last axis (the operator's gradients as they are);
+    q, k, beta, sums as delta_layer_prologue returned them.  Returns the gradient of `rows`, (L, N, H, 2E+M+1)."""
+    L, N, H, E = q.shape
+    M = grad_v.shape[-1]
+    _require(q, "q")
+    _require(k, "k", (L, N, H, E))
+    _require(beta, "beta", (L, N, H))
+    _require(sums, "sums", (L, N, H, 2))
+    gs = []
+    for t, nm, w in ((grad_q, "grad_q", E), (grad_k, "grad_k", E), (grad_v, "grad_v", M), (grad_beta, "grad_beta", 1)):
+        _require(t, nm, (N, H, L, w))
+        if w > 1 and t.stride(-1) != 1:
+            t = t.contiguous()
+        gs.append((t, (ctypes.c_int64 * 3)(*t.stride()[:3])))
+    q, k, beta, sums = (t.contiguous() for t in (q, k, beta, sums))
+    grad_rows = torch.empty((L, N, H, 2 * E + M + 1), device=q.device, dtype=torch.float32)
+    if grad_rows.numel():
+        with torch.cuda.device(q.device):
+            code = lib().delta_layer_prologue_grad_f32(
+                *[a for t, st in gs for a in (_ptr(t), st)], _ptr(q), _ptr(k), _ptr(beta), _ptr(sums), _ptr(grad_rows),
+                N, H, L, E, M, 0, _stream(q.device))
+        _check(code, "delta_layer_prologue_grad_f32")
+    return grad_rows
 
 
 def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v,

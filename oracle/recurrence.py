@@ -109,3 +109,20 @@ def delta_steps_reference(Q, K, V, beta, keep, W0):
         W = W.detach()
         outs.append(out)
     return torch.cat(outs, dim=2), W
+
+
+def delta_layer_inputs_reference(qkvb, E, M, eps):
+    """The prologue of the reference's delta-rule layers as they spell it in tensor operations
+    (supervised_learning/layer.py:74-90; with ``eps`` the RL tree's normalisation,
+    reinforcement_learning/torchbeast/layer.py:30-33, :152-165): from the projection
+    ``qkvb`` (len, B, H, 2E+M+1) = [q~ | k~ | v | b~] to the operator's arguments
+    q, k (B, H, len, E), v (B, H, len, M), beta (B, H, len, 1)."""
+    q, k, v, beta = torch.split(qkvb, (E, E, M, 1), -1)
+    beta = torch.sigmoid(beta)
+    q, k, v, beta = (t.permute(1, 2, 0, 3) for t in (q, k, v, beta))
+
+    def normalise(t):
+        y = F.elu(t, 1., False) + 1.
+        return y / (y.sum(-1, keepdim=True) + (1e-5 if eps else 0.0))
+
+    return normalise(q), normalise(k), v, beta

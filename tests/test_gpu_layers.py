@@ -174,7 +174,52 @@ def test_rl_sr_layers_carry_and_restart(srwm_layer_path):
     assert st is None and rel_err(out.detach().cpu().numpy(), ref.detach().numpy()) < TOL
 
 
-def test_delta_layers():
+@pytest.fixture(params=[True, False], ids=["fused", "spelled-out"])
+def delta_layer_path(request):
+    """Runs a test once with the one-launch prologue of the delta-rule layers and once with the
+    reference's tensor operations."""
+    import layer
+    old = layer.FUSED_DELTA_LAYER
+    layer.FUSED_DELTA_LAYER = request.param
+    yield request.param
+    layer.FUSED_DELTA_LAYER = old
+
+
+@pytest.mark.parametrize("L,B,H,E,M,eps", [(9, 3, 4, 16, 16, False), (5, 2, 3, 64, 64, True), (3, 2, 2, 128, 128, False),
+                                            (4, 1, 5, 20, 61, True), (1, 1, 1, 8, 8, False), (130, 2, 8, 32, 32, True)])
+def test_delta_layer_prologue_matches_the_tensor_operations(L, B, H, E, M, eps):
+    """delta_layer_inputs (one launch forward, one backward) against the fp64 statement of the layers'
+    tensor operations: q, k, v, beta and the gradient of the projection, at 1e-5 of each tensor's
+    maximum.  The gradients arrive as the operator leaves them: (B, H, len, .) contiguous."""
+    print(f"case delta layer prologue L={L} B={B} H={H} E={E} M={M} eps={eps}", flush=True)
+    from fast_weight import delta_layer_inputs
+    from oracle.recurrence import delta_layer_inputs_reference
+    g = torch.Generator().manual_seed(L + E)
+    x = (2.0 * torch.randn(L, B, H, 2 * E + M + 1, generator=g)).to(torch.float32)
+    gs = [torch.randn(B, H, L, w, generator=g) for w in (E, E, M, 1)]
+    xc = x.to(torch.float64).requires_grad_(True)
+    ref = delta_layer_inputs_reference(xc, E, M, eps)
+    sum((r * gi.to(torch.float64)).sum() for r, gi in zip(ref, gs)).backward()
+    xg = x.to(_dev()).requires_grad_(True)
+    out = delta_layer_inputs(xg, E, M, eps)
+    sum((o * gi.to(_dev())).sum() for o, gi in zip(out, gs)).backward()
+    torch.cuda.synchronize()
+    for name, o, r in zip(("q", "k", "v", "beta"), out, ref):
+        assert o.shape == r.shape, name
+        assert rel_err(o.detach().cpu().numpy(), r.detach().numpy()) < 1e-5, name
+    assert rel_err(xg.grad.cpu().numpy(), xc.grad.numpy()) < 1e-5
+    # a gradient that arrives through a permuted view, and one that does not arrive at all
+    xg2 = x.to(_dev()).requires_grad_(True)
+    q2, k2, v2, b2 = delta_layer_inputs(xg2, E, M, eps)
+    gq_view = gs[0].to(_dev()).permute(2, 0, 1, 3).contiguous().permute(1, 2, 0, 3)
+    ((q2 * gq_view).sum() + (b2 * gs[3].to(_dev())).sum()).backward()
+    xc2 = x.to(torch.float64).requires_grad_(True)
+    r2 = delta_layer_inputs_reference(xc2, E, M, eps)
+    ((r2[0] * gs[0].to(torch.float64)).sum() + (r2[3] * gs[3].to(torch.float64)).sum()).backward()
+    assert rel_err(xg2.grad.cpu().numpy(), xc2.grad.numpy()) < 1e-5
+
+
+def test_delta_layers(delta_layer_path):
     print("case FastFFlayer / CarryFastFFlayer", flush=True)
     from layer import CarryFastFFlayer, FastFFlayer, elu_p1, elu_p1_sum_norm_eps, sum_norm
     torch.manual_seed(3)
@@ -210,7 +255,7 @@ def test_delta_layers():
     assert rel_err(new_state.cpu().numpy(), WL.detach().numpy()) < TOL
 
 
-def test_delta_delta_layer():
+def test_delta_delta_layer(delta_layer_path):
     """FastFastFFlayer: a d x (3d+1) delta-rule memory whose readout drives a second, d x d one."""
     print("case FastFastFFlayer", flush=True)
     from layer import FastFastFFlayer, elu_p1_sum_norm_eps

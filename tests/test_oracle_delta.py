@@ -267,3 +267,28 @@ def test_operand_parts_of_the_matrix_core_products():
     assert (np.abs(three - exact) / scale).max() < 3e-5
     one = ah2.astype(np.float64) @ bh2.astype(np.float64)            # a plain bf16 product: bf16-grade, unbiased
     assert (np.abs(one - exact) / scale).max() < 2.0 ** -8 and abs(((one - exact) / scale).mean()) < 1e-4
+
+
+def test_layer_prologue_reference_closed_forms():
+    """The tensor-operation statement of the delta layers' prologue against what the mathematics fixes:
+    elu(x) + 1 is exp(x) for x <= 0, so rows of non-positive q~ give q = softmax(q~); for x > 0 it is
+    x + 1, so positive rows give (x + 1) / (sum x + E); beta is the logistic function; v passes
+    through; with eps the rows sum to s / (s + 1e-5); and the whole is a permutation of the axes."""
+    from oracle.recurrence import delta_layer_inputs_reference
+    g = torch.Generator().manual_seed(0)
+    L, B, H, E, M = 5, 2, 3, 7, 4
+    x = torch.randn(L, B, H, 2 * E + M + 1, generator=g, dtype=torch.float64)
+    x[..., :E] = -x[..., :E].abs()            # q~ <= 0
+    x[..., E:2 * E] = x[..., E:2 * E].abs()   # k~ > 0
+    q, k, v, beta = delta_layer_inputs_reference(x, E, M, False)
+    assert q.shape == (B, H, L, E) and k.shape == (B, H, L, E) and v.shape == (B, H, L, M) and beta.shape == (B, H, L, 1)
+    xp = x.permute(1, 2, 0, 3)
+    assert torch.allclose(q, torch.softmax(xp[..., :E], -1), atol=1e-14)
+    kk = xp[..., E:2 * E]
+    assert torch.allclose(k, (kk + 1) / (kk.sum(-1, keepdim=True) + E), atol=1e-14)
+    assert torch.equal(v, xp[..., 2 * E:2 * E + M])
+    assert torch.allclose(beta, 1 / (1 + torch.exp(-xp[..., -1:])), atol=1e-14)
+    qe, ke, _, _ = delta_layer_inputs_reference(x, E, M, True)
+    s = (kk + 1).sum(-1, keepdim=True)
+    assert torch.allclose(ke.sum(-1, keepdim=True), s / (s + 1e-5), atol=1e-14)
+    assert torch.allclose(qe, q * 1.0 / (1.0 + 1e-5), atol=1e-14)   # softmax rows have s = 1
