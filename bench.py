@@ -21,7 +21,7 @@ matrix-core peak.  `cpu_baseline` is the per-timestep PyTorch recurrence (oracle
 timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (through the autograd operator), delta_prologue_c2 (the layers' prologue kernels, HBM-bound)}.
+{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (through the autograd operator), delta_prologue_c2 (the layers' prologue kernels, HBM-bound), delta_layer_c2 (a whole delta-rule layer)}.
 """
 import argparse
 import json
@@ -77,6 +77,9 @@ WORKLOADS = {
     # the prologue of the delta-rule layers at the shape of configuration 2 (projection rows [q~ | k~ | v | b~] ->
     # normalised q, k, v, beta) and its backward: two memory-bound launches, priced against HBM
     "delta_prologue_c2": ("delta_prologue", 32, 8, 256, 64),
+    # a whole delta-rule layer at that shape (layer.FastFFlayer, model width 256: layer norm, projection, prologue,
+    # recurrence, output map, residual) through autograd: the recurrence kernels are a quarter of it
+    "delta_layer_c2": ("delta_layer", 32, 8, 256, 64),
 }
 
 
@@ -274,9 +277,46 @@ def delta_prologue_step(t, ev=None):
         ev[2].record()
 
 
+def delta_layer_setup(N, H, L, E, dev, width=256):
+    import torch
+    import layer
+    torch.manual_seed(0)
+    g = torch.Generator().manual_seed(0)
+    return dict(mod=layer.FastFFlayer(H, E, width, 0.0).to(dev),
+                x=torch.randn(L, N, width, generator=g).to(dev).requires_grad_(),
+                go=torch.randn(L, N, width, generator=g).to(dev))
+
+
+def delta_layer_step(t, ev=None):
+    if ev:
+        ev[0].record()
+    out = t["mod"](t["x"])
+    if ev:
+        ev[1].record()
+    out.backward(t["go"])
+    if ev:
+        ev[2].record()
+    t["x"].grad = None
+    for w in t["mod"].parameters():
+        w.grad = None
+
+
+def delta_layer_tensor_ops_ms(t, steps=30):
+    """The same layer with its prologue spelled out in tensor operations (as the reference's layer.py does)."""
+    import layer
+    old, layer.FUSED_DELTA_LAYER = layer.FUSED_DELTA_LAYER, False
+    try:
+        _, f, b = time_workload(delta_layer_step, t, steps, 5)
+    finally:
+        layer.FUSED_DELTA_LAYER = old
+    return median(f) + median(b)
+
+
 def algorithmic_bytes(op, N, H, L, E, bf16_grads=False):
     """(lds_fwd, lds_bwd, hbm_total) bytes per launch pair."""
     hs = N * H * L
+    if op == "delta_layer":   # the recurrence inside the layer
+        op = "delta"
     if op == "delta_prologue":
         # forward: the row in, q, k, v, beta and the two normalisers out; backward: the four gradients, q, k,
         # beta and the normalisers in, the row's gradient out.  No state: nothing to pass over in LDS.
@@ -427,6 +467,8 @@ def build_workload(name, dev):
         step, t = srwm_steps_step, srwm_steps_setup(N, H, L, E, dev)
     elif op == "delta_prologue":
         step, t = delta_prologue_step, delta_prologue_setup(N, H, L, E, dev)
+    elif op == "delta_layer":
+        step, t = delta_layer_step, delta_layer_setup(N, H, L, E, dev)
     else:
         step = delta_step
         t = delta_setup(N, H, L, E, dev, torch.bfloat16 if op == "delta_bf16" else torch.float32)
@@ -513,7 +555,7 @@ def rooflines(name, fwd_ms, bwd_ms):
 
 # Driver-visible figures for the other benchmark configurations: (workload, timed steps, warm-up)
 OTHER_WORKLOADS = (("srwm_layer_c4", 50, 10), ("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
-                   ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5), ("delta_c5_op_chunk", 40, 5), ("delta_prologue_c2", 100, 20))
+                   ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5), ("delta_c5_op_chunk", 40, 5), ("delta_prologue_c2", 100, 20), ("delta_layer_c2", 50, 10))
 
 
 def main():
@@ -560,6 +602,10 @@ def main():
                       "forward_mean": round(sum(fwd_all) / a.steps, 4), "backward_mean": round(sum(bwd_all) / a.steps, 4)},
     }
     res.update(rooflines(a.workload, fwd_ms, bwd_ms))
+    if op == "delta_layer":
+        res["tensor_ops_prologue_ms"] = round(delta_layer_tensor_ops_ms(t), 4)
+        res["config"]["workload"] += ("; a whole FastFFlayer of width 256 through autograd; tensor_ops_prologue_ms = forward + "
+                                      "backward with the layer's prologue as tensor operations instead of the one-launch kernels")
     if op == "srwm_steps":
         res["per_step_loop_ms"] = round(srwm_per_step_loop_ms(t, N, H, L, E, dev), 3)
         res["config"]["workload"] += ("; gradient cut at the carried state, 5 % resets; per_step_loop_ms = the same "
@@ -592,6 +638,9 @@ def main():
             if "roofline_lds_yardstick" in rl:
                 rec["fwd_bwd_frac_lds_yardstick"] = rl["roofline_lds_yardstick"]["frac"]
                 rec["fwd_bwd_frac_hbm"] = rl["roofline_hbm"]["frac"]
+            if o_op == "delta_layer":
+                rec["fwd_bwd_bound"] = "lds yardstick of the recurrence alone; the layer also runs two linear maps and a layer norm"
+                rec["tensor_ops_prologue_ms"] = round(delta_layer_tensor_ops_ms(tt), 4)
             others[name] = rec
             del st, tt
         res["other_workloads"] = others
