@@ -312,7 +312,7 @@ def delta_layer_tensor_ops_ms(t, steps=30):
     return median(f) + median(b)
 
 
-def algorithmic_bytes(op, N, H, L, E, bf16_grads=False):
+def algorithmic_bytes(op, N, H, L, E, bf16_grads=False, no_v_old=False):
     """(lds_fwd, lds_bwd, hbm_total) bytes per launch pair."""
     hs = N * H * L
     if op == "delta_layer":   # the recurrence inside the layer
@@ -338,11 +338,13 @@ def algorithmic_bytes(op, N, H, L, E, bf16_grads=False):
     S = E * E
     # per (sequence, step): q,k,v,beta in (fwd and bwd), out + grad_out in the I/O type; v_old,
     # v_insert written and read back, and the 3 E-wide gradients + grad_beta written, in fp32
-    # (bf16_grads: the three E-wide gradients in bf16, as the chunkwise bf16 workload writes them)
+    # (bf16_grads: the three E-wide gradients in bf16, as the chunkwise bf16 workload writes them;
+    # no_v_old: the chunkwise pair neither writes nor reads v_old, and its backward does not read v)
     b = 2 if op == "delta_bf16" else 4
-    io_elems = 2 * (3 * E + 1) + 2 * E
+    io_elems = 2 * (3 * E + 1) + 2 * E - (E if no_v_old else 0)
     grads = 3 * E * (2 if bf16_grads else 4) + 4
-    return 2 * S * 4 * hs, 4 * S * 4 * hs, (io_elems * b + 4 * E * 4 + grads) * hs + 3 * S * 4 * N * H
+    saved = (2 if no_v_old else 4) * E * 4
+    return 2 * S * 4 * hs, 4 * S * 4 * hs, (io_elems * b + saved + grads) * hs + 3 * S * 4 * N * H
 
 
 def cpu_baseline(op, N, H, L, E, budget_s=20.0):
@@ -477,7 +479,8 @@ def build_workload(name, dev):
             for n in ("q", "k", "v", "beta"):
                 t[n].requires_grad_()
         elif name.endswith("_chunk"):
-            t["fwd_flags"] = srwm_hip.FLAG_CHUNKWISE
+            # as the operator calls the pair: v_old only where the chunkwise backward reads it
+            t["fwd_flags"] = srwm_hip.FLAG_CHUNKWISE | srwm_hip.FLAG_SPARSE_V_OLD
             t["bwd_flags"] = srwm_hip.FLAG_CHUNKWISE
             if op == "delta_bf16":   # as the operator calls it: bf16 gradients, rounded by the kernels themselves
                 for n in ("gq", "gk", "gv"):
@@ -519,7 +522,8 @@ def roof(bound, amount, ms, peak, unit="GB/s"):
 def rooflines(name, fwd_ms, bwd_ms):
     """The roofline records of one workload from its median kernel times."""
     op, N, H, L, E = WORKLOADS[name]
-    lds_f, lds_b, hbm = algorithmic_bytes(op, N, H, L, E, bf16_grads=name.endswith("_chunk") and op == "delta_bf16")
+    lds_f, lds_b, hbm = algorithmic_bytes(op, N, H, L, E, bf16_grads=name.endswith("_chunk") and op == "delta_bf16",
+                                          no_v_old=name.endswith("_chunk"))
     r = {}
     if op == "delta_prologue":
         W = 3 * E + 1

@@ -69,6 +69,13 @@ extern "C" {
                                      for rows with |beta| < 2^-24, which the first sweep forms directly.  Not with
                                      SRWM_FLAG_EXACT_PRODUCTS and not with gW (the gradient of the memory would be
                                      accumulated from the rounded grad_V): SRWM_EINVAL. */
+#define SRWM_FLAG_SPARSE_V_OLD 4096u /* delta_forward_* with SRWM_FLAG_CHUNKWISE only: v_old is written only for the steps
+                                       with |beta| < 2^-24.  For callers whose backward is the chunkwise one in a mode that
+                                       reads grad_beta off its second sweep (fp32 inputs; bf16 inputs with
+                                       SRWM_FLAG_BF16_GRADS or SRWM_FLAG_EXACT_PRODUCTS): those steps are all it reads of
+                                       v_old, so a quarter of the forward's writes never happens.  The step-by-step
+                                       backward, and the chunkwise one with bf16 inputs, single products and fp32
+                                       gradients, need every row: do not set it for them. */
 #define SRWM_FLAG_NORM_EPS 2048u   /* delta_layer_prologue_f32 only: 1e-5 is added to the normalisers of q and k (the RL
                                      tree's layers, reinforcement_learning/torchbeast/layer.py:30-33) */
 /* srwm_layer_forward_* / srwm_layer_backward_* only: */
@@ -490,7 +497,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 10. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 11. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

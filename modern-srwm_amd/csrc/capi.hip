@@ -85,7 +85,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 10; }
+int srwm_hip_abi_version(void) { return 11; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -481,15 +481,17 @@ int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const
                       int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
         return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS)) ||
-        (flags & (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE)) == (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE))
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) ||
+        (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_SPARSE_V_OLD)) ||
+        (flags & (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE)) == (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE) ||
+        ((flags & SRWM_FLAG_SPARSE_V_OLD) && !(flags & SRWM_FLAG_CHUNKWISE)))
         return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
         !stride_ok(bs, N, H, L, 1))
         return SRWM_ESTRIDE;
     DeltaFwdParams p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
                      {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
-                     N, H, L, E, M};
+                     N, H, L, E, M, nullptr, (flags & SRWM_FLAG_SPARSE_V_OLD) ? 1u : 0u};
     hipStream_t s = (hipStream_t)stream;
     if (flags & SRWM_FLAG_CHUNKWISE) {
         const int r = launch_delta_fwd_chunk(p, s);
@@ -542,14 +544,16 @@ int delta_forward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K
                        int E, int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
         return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS)))
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) ||
+        (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_SPARSE_V_OLD)) ||
+        ((flags & SRWM_FLAG_SPARSE_V_OLD) && !(flags & SRWM_FLAG_CHUNKWISE)))
         return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
         !stride_ok(bs, N, H, L, 1))
         return SRWM_ESTRIDE;
     DeltaFwdParamsBf16 p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
                          {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
-                         N, H, L, E, M, (flags & SRWM_FLAG_EXACT_PRODUCTS) ? 1u : 0u};
+                         N, H, L, E, M, (flags & SRWM_FLAG_EXACT_PRODUCTS) ? 1u : 0u, (flags & SRWM_FLAG_SPARSE_V_OLD) ? 1u : 0u};
     const int r = (flags & SRWM_FLAG_CHUNKWISE) ? launch_delta_fwd_chunk_bf16(p, (hipStream_t)stream)
                                                 : launch_delta_fwd_tiled_bf16(p, (hipStream_t)stream);
     return r >= 0 ? r : SRWM_ENOKERNEL;

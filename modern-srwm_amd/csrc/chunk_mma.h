@@ -434,6 +434,10 @@ struct PrecBf16x3 {
     }
 };
 
+// The chunkwise backward divides by beta^2 where it reads grad_beta off its second sweep; rows whose
+// |beta| is below this bound take the direct form, the only use of v_old there.
+constexpr float kTinyBeta = 5.9604645e-8f;   // 2^-24
+
 // Raw bits of one input element and their fp32 value: loads keep the bits, the conversion is
 // done where the value is used, so that a prefetch does not wait for its own loads.
 __device__ __forceinline__ uint32_t ld_bits(const float *p) { return __float_as_uint(*p); }

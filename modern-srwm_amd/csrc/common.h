@@ -94,6 +94,7 @@ struct DeltaFwdParams {
     float *vold, *vins, *W, *out;
     int N, H, L, E, M;
     const float *keep;   // optional dense [N,L]: the memory is zeroed before step t where keep[n][t] == 0
+    unsigned sparse_vold;   // chunkwise kernel: v_old is written only for steps with |beta| < 2^-24
 };
 
 struct DeltaBwdParams {
@@ -114,6 +115,7 @@ struct DeltaFwdParamsBf16 {
     uint16_t *out;
     int N, H, L, E, M;
     unsigned exact_products;   // chunkwise kernels: every product from hi + lo operand pairs
+    unsigned sparse_vold;      // chunkwise kernel: v_old is written only for steps with |beta| < 2^-24
 };
 
 struct DeltaBwdParamsBf16 {

@@ -47,6 +47,7 @@ struct ChunkFwdP {
     TI *out;
     int N, H, L;
     bool exact;   // bf16 inputs: also the products that only feed `out` from hi + lo operand pairs
+    bool sparse_vold;   // v_old goes out only for steps with |beta| < kTinyBeta (all the chunkwise backward reads of it)
 };
 
 // LDS carve-up shared by the kernel and the launcher
@@ -269,7 +270,10 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
                                                f32x4{0.f, 0.f, 0.f, 0.f});
             ub[a] = X::accb(u[a]);
             if (a % KS == hf) {   // the two waves of a pair share the outputs: each forms and stores every other row block
-                y = X::template mma<true, true>(X::lda(As, a * 16 + ln, a * 16 + 4 * lq), ub[a], y);   // + strict_lower(A_aa) U_a
+                // v_old of this block is wanted: always, or only if one of its steps has a tiny beta (wave-uniform)
+                const bool vo = !p.sparse_vold ||
+                                __builtin_amdgcn_ballot_w64(fabsf(bts[a * 16 + ln]) < kTinyBeta && t0 + a * 16 + ln < p.L) != 0ull;
+                if (vo) y = X::template mma<true, true>(X::lda(As, a * 16 + ln, a * 16 + 4 * lq), ub[a], y);   // + strict_lower(A_aa) U_a
                 // out = Q S + tril(B) U
                 ot[a] = mma_range<X, !OB, !OB>(
                     0, a + 1, [&](int b) { return X::lda(Bs, a * 16 + ln, b * 16 + 4 * lq); }, fu, ot[a]);
@@ -283,7 +287,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
                 if (t0 + kC <= p.L) {   // a full chunk: no row is past the end
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
-                        *at(vold_seq, o0 + r * D * 4) = pt[a][r] + y[r];
+                        if (vo && (!p.sparse_vold || fabsf(bts[a * 16 + 4 * lq + r]) < kTinyBeta))
+                            *at(vold_seq, o0 + r * D * 4) = pt[a][r] + y[r];
                         *at(vins_seq, o0 + r * D * 4) = u[a][r];
                         st_out(at(out_seq, (o0 + r * D * 4) / 4 * (uint32_t)sizeof(TI)), ot[a][r]);
                     }
@@ -291,7 +296,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         if (t0 + a * 16 + 4 * lq + r < p.L) {
-                            *at(vold_seq, o0 + r * D * 4) = pt[a][r] + y[r];
+                            if (vo && (!p.sparse_vold || fabsf(bts[a * 16 + 4 * lq + r]) < kTinyBeta))
+                                *at(vold_seq, o0 + r * D * 4) = pt[a][r] + y[r];
                             *at(vins_seq, o0 + r * D * 4) = u[a][r];
                             st_out(at(out_seq, (o0 + r * D * 4) / 4 * (uint32_t)sizeof(TI)), ot[a][r]);
                         }
@@ -356,14 +362,14 @@ int dispatch_chunk(const ChunkFwdP<TI> &p, int D, hipStream_t s) {
 int launch_delta_fwd_chunk(const DeltaFwdParams &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const ChunkFwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out,
-                             p.N, p.H, p.L, true};
+                             p.N, p.H, p.L, true, p.sparse_vold != 0u};
     return dispatch_chunk(q, p.E, s);
 }
 
 int launch_delta_fwd_chunk_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const ChunkFwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out,
-                              p.N, p.H, p.L, p.exact_products != 0u};
+                              p.N, p.H, p.L, p.exact_products != 0u, p.sparse_vold != 0u};
     return dispatch_chunk(q, p.E, s);
 }
 

@@ -63,8 +63,7 @@ struct ChunkBwdP {
 // grad_beta can be read off the second sweep's own product: Y U^T has beta_t^2 sum_m dR_tm (V - v_old)_tm
 // on its diagonal, so the first sweep then needs neither V nor v_old (gathers in accumulator layout,
 // which it waits for).  Rows whose |beta| is below this bound cannot be divided back and take the
-// direct form in the first sweep.
-constexpr float kTinyBeta = 5.9604645e-8f;   // 2^-24
+// direct form in the first sweep (kTinyBeta, chunk_mma.h).
 // Done wherever that product is as accurate as the caller's grad_beta: fp32 inputs and bf16 inputs with
 // operand pairs everywhere (!OB) -- every product at ~1e-5 or better -- and bf16 inputs with rounded
 // gradients (GB; single bf16 products, ~1e-3).  With bf16 inputs, single products and fp32 gradients

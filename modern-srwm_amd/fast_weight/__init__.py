@@ -35,7 +35,12 @@ def _chunk_flags(choice, E, M, L):
 
 
 def _forward_flags(E, M, L):
-    return _chunk_flags(CHUNKWISE_FORWARD, E, M, L)
+    flags = _chunk_flags(CHUNKWISE_FORWARD, E, M, L)
+    # when the backward is the chunkwise one too, all it reads of v_old are the steps whose beta is too
+    # small to divide by (it reads grad_beta off its own products): the forward writes only those
+    if flags and _chunk_flags(CHUNKWISE_BACKWARD, E, M, L):
+        flags |= srwm_hip.FLAG_SPARSE_V_OLD
+    return flags
 
 
 def causal_dot_product_cuda(q, k, v, beta, v_old, v_insert, kv, out):

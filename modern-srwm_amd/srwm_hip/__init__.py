@@ -32,12 +32,13 @@ FLAG_GENERIC = 16
 FLAG_CHUNKWISE = 32     # delta forward: chunkwise MFMA kernel (E == M in {64, 128})
 FLAG_EXACT_PRODUCTS = 512   # chunkwise kernels with bf16 inputs: every product from hi + lo operand pairs
 FLAG_BF16_GRADS = 1024      # chunkwise delta backward with bf16 inputs: grad_q, grad_k, grad_v written as bf16 by the library
+FLAG_SPARSE_V_OLD = 4096    # chunkwise delta forward: v_old only for steps with |beta| < 2^-24 (all a chunkwise backward reads of it)
 FLAG_NORM_EPS = 2048        # delta_layer_prologue: 1e-5 added to the normalisers of q and k
 FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus the shared weights
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _lib = None
 

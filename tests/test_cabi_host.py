@@ -140,6 +140,8 @@ def test_argument_validation_needs_no_gpu():
     assert delta_f(16 | 32, E) == -1                           # generic and chunkwise exclude each other
     assert delta_f(0, 0) == -1                                 # value width 0
     assert delta_f(32, E) == -4                                # SRWM_ENOKERNEL: no chunkwise kernel for E = M = 16
+    assert delta_f(4096, E) == -1                              # v_old for the tiny betas only: a mode of the chunkwise kernels
+    assert delta_f(32 | 4096, E) == -4                         # accepted with them
     delta_b = lambda gW, flags: L.delta_backward_f32(*[a for _ in range(4) for a in (fake(), ok_strides)],
                                                      fake(), fake(), fake(), ok_strides, fake(), fake(), fake(), fake(),
                                                      fake(), gW, N, H, Ls, E, E, flags, P(None))

@@ -360,6 +360,45 @@ def test_chunkwise_backward_with_betas_too_small_to_divide_by(shape, qk):
         assert rows.any() and np.abs(gb[rows] - ref[rows]).max() < TOL * scale, name
 
 
+@pytest.mark.parametrize("shape,io", [((2, 2, 300, 64, 64), torch.float32), ((1, 3, 200, 128, 128), torch.bfloat16),
+                                      ((1, 2, 150, 128, 128), torch.float32)])
+def test_chunkwise_forward_can_leave_out_the_v_old_that_nobody_reads(shape, io):
+    """FLAG_SPARSE_V_OLD: the chunkwise forward writes v_old only where |beta| < 2^-24 -- all that the
+    chunkwise backward reads of it -- and everything else as without the flag; a backward fed with
+    that v_old returns bit for bit what it returns from the complete one.  The operator sets the flag
+    when both of its halves are chunkwise."""
+    print(f"case chunkwise forward, sparse v_old shape={shape} io={io}", flush=True)
+    import srwm_hip
+    dev = _dev()
+    q, k, v, beta, W0, go = delta_inputs(*shape, seed=31, qk="l2", w0_std=0.2)
+    beta = beta.clone()
+    beta[:, :, ::7] = 0.0
+    beta[:, :, 3::11] = 1e-9
+    N, H, L, E = q.shape
+    qd, kd, vd, bd, god = (t.to(io).to(dev) for t in (q, k, v, beta, go))
+    tiny = (bd.float().abs() < 2.0 ** -24).expand(N, H, L, E)
+    res = {}
+    for name, fl in (("full", 0), ("sparse", srwm_hip.FLAG_SPARSE_V_OLD)):
+        W = W0.to(dev, torch.float32).contiguous()
+        vold = torch.full((N, H, L, E), float("nan"), device=dev)
+        vins = torch.empty(N, H, L, E, device=dev)
+        out = torch.empty(N, H, L, E, device=dev, dtype=io)
+        srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out, flags=srwm_hip.FLAG_CHUNKWISE | fl)
+        gdt = io
+        g = [torch.empty((N, H, L, E), device=dev, dtype=gdt) for _ in range(3)] + [torch.empty((N, H, L, 1), device=dev)]
+        Wb = W.clone()
+        srwm_hip.fast_weight_backward(qd, kd, vd, bd, vold, vins, god, Wb, *g, flags=srwm_hip.FLAG_CHUNKWISE)
+        torch.cuda.synchronize()
+        res[name] = (vold, vins, out, W, g, Wb)
+    f, s = res["full"], res["sparse"]
+    assert torch.equal(f[1], s[1]) and torch.equal(f[2], s[2]) and torch.equal(f[3], s[3])
+    assert tiny.any() and torch.equal(s[0][tiny], f[0][tiny]) and bool(torch.isnan(s[0][~tiny]).all())
+    assert not torch.isnan(f[0]).any()
+    for a, b in zip(f[4], s[4]):
+        assert torch.equal(a, b)
+    assert torch.equal(f[5], s[5])
+
+
 @pytest.mark.parametrize("shape,qk,small_betas", [
     ((2, 2, 300, 64, 64), "softmax", False), ((1, 3, 512, 128, 128), "l2", False),
     ((3, 1, 150, 128, 128), "l2", False), ((1, 2, 64, 64, 64), "softmax", False),
