@@ -48,7 +48,7 @@ MEASURED_TRAFFIC = {
     "delta_c2": ((102515 + 53504) * 1024, "profiles/delta_kernels.txt"),
     "delta_c2_chunk": ((49621 + 86137 + 16384 + 37120) * 1024, "profiles/delta_chunk_kernels.txt"),
     "delta_c5": ((1054057 + 1323008) * 1024, "profiles/delta_kernels.txt"),
-    "delta_c5_chunk": ((392985 + 792838 + 131072 + 272384) * 1024, "profiles/delta_chunk_kernels.txt"),
+    "delta_c5_chunk": ((392971 + 792824 + 131072 + 272384) * 1024, "profiles/delta_chunk_kernels.txt"),
 }
 
 WORKLOADS = {
