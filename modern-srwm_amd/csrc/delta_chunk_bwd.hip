@@ -16,11 +16,15 @@
 // two sweeps with the memory tiled the other way round:
 //   column sweep  a wave owns 16 columns of S and dS (rows in the registers); it solves the
 //                 upper triangular system by 16-row block back substitution (diagonal blocks
-//                 inverted on the matrix cores, one per wave) and writes grad_V and grad_beta;
+//                 inverted on the matrix cores, one per wave) and writes grad_V;
 //   row sweep     a wave owns 16 rows of S and dS, held transposed (columns in the registers);
 //                 it reads grad_V back, forms G1 and X cooperatively and writes grad_Q, grad_K,
 //                 the reverted memory and the gradient of the initial memory.  Every word of
 //                 grad_Q / grad_K has one writer: no atomics.
+// grad_beta = rowsum(dR * (V - v_old)) is the diagonal of Y U^T over beta^2 (Y = beta dR, U = beta
+// (V - v_old)), a product the row sweep forms anyway: it is read off there, except where that
+// product is less accurate than the caller's grad_beta or beta is too small to divide by -- then the
+// column sweep forms it directly from V and v_old (RowFormsGradBeta, kTinyBeta).
 // Both sweeps accumulate dS on their own and the row sweep also reverts S (cheaper than moving
 // the memory between the two layouts every chunk; the column sweep needs no S at all).  With fp32
 // inputs a product is six v_mfma_f32_16x16x32_bf16 on three-part operands at D = 64 (fp32
