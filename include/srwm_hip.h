@@ -482,6 +482,18 @@ SRWM_API int delta_layer_prologue_grad_f32(const float *gq, const int64_t gq_str
                                   float *grad_rows,
                                   int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
+/* The same with every tensor in bf16 (16-bit patterns, rounded to nearest even on the way out) except the normalisers;
+ * arithmetic in fp32.  For layers that run in bf16 in front of delta_forward_bf16 / delta_backward_bf16. */
+SRWM_API int delta_layer_prologue_bf16(const uint16_t *rows, uint16_t *q, uint16_t *k, uint16_t *v, uint16_t *beta,
+                              float *sums, int N, int H, int L, int E, int M, unsigned flags, void *stream);
+SRWM_API int delta_layer_prologue_grad_bf16(const uint16_t *gq, const int64_t gq_strides[3],
+                                   const uint16_t *gk, const int64_t gk_strides[3],
+                                   const uint16_t *gv, const int64_t gv_strides[3],
+                                   const uint16_t *gbeta, const int64_t gbeta_strides[3],
+                                   const uint16_t *q, const uint16_t *k, const uint16_t *beta, const float *sums,
+                                   uint16_t *grad_rows,
+                                   int N, int H, int L, int E, int M, unsigned flags, void *stream);
+
 /* Largest E the SRWM entry points accept (forward / backward), and the largest
  * E == M the delta entry points accept, on the current device. */
 SRWM_API int srwm_hip_limits(int *srwm_fwd_max_E, int *srwm_bwd_max_E, int *delta_max_EM);
@@ -497,7 +509,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 11. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 12. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

@@ -85,7 +85,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 11; }
+int srwm_hip_abi_version(void) { return 12; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -337,6 +337,32 @@ int delta_layer_prologue_grad_f32(const float *gq, const int64_t gqs[3], const f
     const int r = launch_delta_prologue_grad(gq, {gqs[0], gqs[1], gqs[2]}, gk, {gks[0], gks[1], gks[2]}, gv,
                                              {gvs[0], gvs[1], gvs[2]}, gbeta, {gbs[0], gbs[1], gbs[2]}, q, k, beta,
                                              sums, grad_rows, N, H, L, E, M, (hipStream_t)stream);
+    return r >= 0 ? r : SRWM_ESIZE;
+}
+
+int delta_layer_prologue_bf16(const uint16_t *rows, uint16_t *q, uint16_t *k, uint16_t *v, uint16_t *beta, float *sums,
+                              int N, int H, int L, int E, int M, unsigned flags, void *stream) {
+    if (!rows || !q || !k || !v || !beta || !sums) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_NORM_EPS)) return SRWM_EINVAL;
+    const int r = launch_delta_prologue_bf16(rows, q, k, v, beta, sums, N, H, L, E, M,
+                                             (flags & SRWM_FLAG_NORM_EPS) ? 1e-5f : 0.f, (hipStream_t)stream);
+    return r >= 0 ? r : SRWM_ESIZE;
+}
+
+int delta_layer_prologue_grad_bf16(const uint16_t *gq, const int64_t gqs[3], const uint16_t *gk, const int64_t gks[3],
+                                   const uint16_t *gv, const int64_t gvs[3], const uint16_t *gbeta,
+                                   const int64_t gbs[3], const uint16_t *q, const uint16_t *k, const uint16_t *beta,
+                                   const float *sums, uint16_t *grad_rows, int N, int H, int L, int E, int M,
+                                   unsigned flags, void *stream) {
+    if (!gq || !gk || !gv || !gbeta || !q || !k || !beta || !sums || !grad_rows || !gqs || !gks || !gvs || !gbs)
+        return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || flags) return SRWM_EINVAL;
+    if (!stride_ok(gqs, N, H, L, E) || !stride_ok(gks, N, H, L, E) || !stride_ok(gvs, N, H, L, M) ||
+        !stride_ok(gbs, N, H, L, 1))
+        return SRWM_ESTRIDE;
+    const int r = launch_delta_prologue_grad_bf16(gq, {gqs[0], gqs[1], gqs[2]}, gk, {gks[0], gks[1], gks[2]}, gv,
+                                                  {gvs[0], gvs[1], gvs[2]}, gbeta, {gbs[0], gbs[1], gbs[2]}, q, k,
+                                                  beta, sums, grad_rows, N, H, L, E, M, (hipStream_t)stream);
     return r >= 0 ? r : SRWM_ESIZE;
 }
 

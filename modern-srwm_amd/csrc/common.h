@@ -206,6 +206,13 @@ int launch_delta_prologue_grad(const float *gq, const Strided3 &gqs, const float
                                const float *gv, const Strided3 &gvs, const float *gb, const Strided3 &gbs,
                                const float *q, const float *k, const float *beta, const float *sums, float *gx,
                                int N, int H, int L, int E, int M, hipStream_t s);
+// the same with every tensor but the normalisers in bf16
+int launch_delta_prologue_bf16(const uint16_t *x, uint16_t *q, uint16_t *k, uint16_t *v, uint16_t *beta, float *sums,
+                               int N, int H, int L, int E, int M, float eps, hipStream_t s);
+int launch_delta_prologue_grad_bf16(const uint16_t *gq, const Strided3 &gqs, const uint16_t *gk, const Strided3 &gks,
+                                    const uint16_t *gv, const Strided3 &gvs, const uint16_t *gb, const Strided3 &gbs,
+                                    const uint16_t *q, const uint16_t *k, const uint16_t *beta, const float *sums,
+                                    uint16_t *gx, int N, int H, int L, int E, int M, hipStream_t s);
 int launch_delta_fwd_generic(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_bwd_generic(const DeltaBwdParams &p, hipStream_t s);
 

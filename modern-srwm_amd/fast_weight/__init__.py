@@ -99,7 +99,7 @@ class DeltaLayerInputs(torch.autograd.Function):
 
         q, k, v, beta = delta_layer_inputs(qkvb, E, M, eps)
 
-    qkvb: (len, B, H, 2E+M+1) float32 -- the projection [q~ | k~ | v | b~]; returns the operator's
+    qkvb: (len, B, H, 2E+M+1) float32 or bfloat16 -- the projection [q~ | k~ | v | b~]; returns the operator's
     arguments q, k: (B, H, len, E) = sum_norm(elu(.) + 1) (the sum plus 1e-5 when `eps`), v: (B, H, len, M),
     beta: (B, H, len, 1) = sigmoid, as permuted views of dense (len, B, H, .) tensors."""
 
@@ -114,7 +114,7 @@ class DeltaLayerInputs(torch.autograd.Function):
     def backward(ctx, grad_q, grad_k, grad_v, grad_beta):
         q, k, beta, sums = ctx.saved_tensors
         L, N, H, E = q.shape
-        zeros = lambda w: torch.zeros((N, H, L, w), device=q.device, dtype=torch.float32)
+        zeros = lambda w: torch.zeros((N, H, L, w), device=q.device, dtype=q.dtype)
         grad_q = zeros(E) if grad_q is None else grad_q
         grad_k = zeros(E) if grad_k is None else grad_k
         grad_beta = zeros(1) if grad_beta is None else grad_beta

@@ -265,7 +265,7 @@ class SMFWPlayer(nn.Module):
 def _delta_inputs(qkvb, E, M, eps):
     """(len, B, H, 2E+M+1) projection -> q, k, v, beta as (B, H, len, .): supervised_learning/layer.py:74-90,
     reinforcement_learning/torchbeast/layer.py:152-165."""
-    if FUSED_DELTA_LAYER and qkvb.is_cuda and qkvb.dtype == torch.float32:
+    if FUSED_DELTA_LAYER and qkvb.is_cuda and qkvb.dtype in (torch.float32, torch.bfloat16):
         return delta_layer_inputs(qkvb, E, M, eps)
     q, k, v, beta = torch.split(qkvb, (E, E, M, 1), -1)
     beta = torch.sigmoid(beta)

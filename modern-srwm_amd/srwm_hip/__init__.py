@@ -38,7 +38,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 _lib = None
 
@@ -72,6 +72,8 @@ _SIGNATURES = {
     "delta_backward_bf16": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_layer_prologue_f32": [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_layer_prologue_grad_f32": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_layer_prologue_bf16": [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_layer_prologue_grad_bf16": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
 }
 
 
@@ -689,20 +691,24 @@ def fast_weight_steps_backward(q, k, v, beta, keep, v_old, v_insert, grad_out, k
 
 
 def delta_layer_prologue(rows, E, M, eps=False):
-    """rows: (L, N, H, 2E+M+1) float32, contiguous -- the delta-rule layers' projection [q~ | k~ | v | b~].
+    """rows: (L, N, H, 2E+M+1) float32 or bfloat16, contiguous -- the delta-rule layers' projection [q~ | k~ | v | b~].
     Returns q, k: (L, N, H, E) normalised (elu + 1 over its sum, plus 1e-5 when `eps`), v: (L, N, H, M),
-    beta: (L, N, H) = sigmoid, sums: (L, N, H, 2), all freshly allocated and contiguous, from one launch."""
-    _require(rows, "rows")
+    beta: (L, N, H) = sigmoid, in the type of `rows`, and sums: (L, N, H, 2) float32; all freshly allocated and
+    contiguous, from one launch."""
+    io = rows.dtype if isinstance(rows, torch.Tensor) and rows.dtype == torch.bfloat16 else torch.float32
+    _require(rows, "rows", None, io)
     L, N, H, W = rows.shape
     if W != 2 * E + M + 1 or not rows.is_contiguous():
         raise ValueError(f"rows must be contiguous with last axis 2E+M+1 = {2 * E + M + 1} (got {tuple(rows.shape)})")
-    new = lambda *sh: torch.empty(sh, device=rows.device, dtype=torch.float32)
-    q, k, v, beta, sums = new(L, N, H, E), new(L, N, H, E), new(L, N, H, M), new(L, N, H), new(L, N, H, 2)
+    new = lambda *sh: torch.empty(sh, device=rows.device, dtype=io)
+    q, k, v, beta = new(L, N, H, E), new(L, N, H, E), new(L, N, H, M), new(L, N, H)
+    sums = torch.empty((L, N, H, 2), device=rows.device, dtype=torch.float32)
     if rows.numel():
+        fn = lib().delta_layer_prologue_bf16 if io == torch.bfloat16 else lib().delta_layer_prologue_f32
         with torch.cuda.device(rows.device):
-            code = lib().delta_layer_prologue_f32(_ptr(rows), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(sums),
-                                                  N, H, L, E, M, FLAG_NORM_EPS if eps else 0, _stream(rows.device))
-        _check(code, "delta_layer_prologue_f32")
+            code = fn(_ptr(rows), _ptr(q), _ptr(k), _ptr(v), _ptr(beta), _ptr(sums),
+                      N, H, L, E, M, FLAG_NORM_EPS if eps else 0, _stream(rows.device))
+        _check(code, fn.__name__)
     return q, k, v, beta, sums
 
 
@@ -712,24 +718,25 @@ def delta_layer_prologue_grad(grad_q, grad_k, grad_v, grad_beta, q, k, beta, sum
     q, k, beta, sums as delta_layer_prologue returned them.  Returns the gradient of `rows`, (L, N, H, 2E+M+1)."""
     L, N, H, E = q.shape
     M = grad_v.shape[-1]
-    _require(q, "q")
-    _require(k, "k", (L, N, H, E))
-    _require(beta, "beta", (L, N, H))
+    io = q.dtype if isinstance(q, torch.Tensor) and q.dtype == torch.bfloat16 else torch.float32
+    _require(q, "q", None, io)
+    _require(k, "k", (L, N, H, E), io)
+    _require(beta, "beta", (L, N, H), io)
     _require(sums, "sums", (L, N, H, 2))
     gs = []
     for t, nm, w in ((grad_q, "grad_q", E), (grad_k, "grad_k", E), (grad_v, "grad_v", M), (grad_beta, "grad_beta", 1)):
-        _require(t, nm, (N, H, L, w))
+        _require(t, nm, (N, H, L, w), io)
         if w > 1 and t.stride(-1) != 1:
             t = t.contiguous()
         gs.append((t, (ctypes.c_int64 * 3)(*t.stride()[:3])))
     q, k, beta, sums = (t.contiguous() for t in (q, k, beta, sums))
-    grad_rows = torch.empty((L, N, H, 2 * E + M + 1), device=q.device, dtype=torch.float32)
+    grad_rows = torch.empty((L, N, H, 2 * E + M + 1), device=q.device, dtype=io)
     if grad_rows.numel():
+        fn = lib().delta_layer_prologue_grad_bf16 if io == torch.bfloat16 else lib().delta_layer_prologue_grad_f32
         with torch.cuda.device(q.device):
-            code = lib().delta_layer_prologue_grad_f32(
-                *[a for t, st in gs for a in (_ptr(t), st)], _ptr(q), _ptr(k), _ptr(beta), _ptr(sums), _ptr(grad_rows),
-                N, H, L, E, M, 0, _stream(q.device))
-        _check(code, "delta_layer_prologue_grad_f32")
+            code = fn(*[a for t, st in gs for a in (_ptr(t), st)], _ptr(q), _ptr(k), _ptr(beta), _ptr(sums),
+                      _ptr(grad_rows), N, H, L, E, M, 0, _stream(q.device))
+        _check(code, fn.__name__)
     return grad_rows
 
 

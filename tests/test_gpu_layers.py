@@ -219,6 +219,58 @@ def test_delta_layer_prologue_matches_the_tensor_operations(L, B, H, E, M, eps):
     assert rel_err(xg2.grad.cpu().numpy(), xc2.grad.numpy()) < 1e-5
 
 
+@pytest.mark.parametrize("L,B,H,E,M,eps", [(9, 3, 4, 16, 16, False), (6, 2, 3, 64, 64, True), (3, 2, 2, 128, 128, False),
+                                            (130, 2, 4, 32, 32, True)])
+def test_delta_layer_prologue_in_bf16(L, B, H, E, M, eps):
+    """The bf16 twins of the prologue kernels (every tensor but the normalisers in bf16, arithmetic in
+    fp32) against the fp64 statement on the same bf16-rounded projection: outputs within the rounding
+    of a bf16 result, the gradient of the projection within the bf16 bar."""
+    print(f"case delta layer prologue bf16 L={L} B={B} H={H} E={E} M={M} eps={eps}", flush=True)
+    from fast_weight import delta_layer_inputs
+    from oracle.recurrence import delta_layer_inputs_reference
+    g = torch.Generator().manual_seed(L + E)
+    x = (2.0 * torch.randn(L, B, H, 2 * E + M + 1, generator=g)).to(torch.bfloat16)
+    gs = [torch.randn(B, H, L, w, generator=g).to(torch.bfloat16) for w in (E, E, M, 1)]
+    xc = x.to(torch.float64).requires_grad_(True)
+    ref = delta_layer_inputs_reference(xc, E, M, eps)
+    sum((r * gi.to(torch.float64)).sum() for r, gi in zip(ref, gs)).backward()
+    xg = x.to(_dev()).requires_grad_(True)
+    out = delta_layer_inputs(xg, E, M, eps)
+    sum((o.float() * gi.to(_dev()).float()).sum() for o, gi in zip(out, gs)).backward()
+    torch.cuda.synchronize()
+    for name, o, r in zip(("q", "k", "v", "beta"), out, ref):
+        assert o.dtype == torch.bfloat16 and o.shape == r.shape, name
+        assert rel_err(o.detach().float().cpu().numpy(), r.detach().numpy()) < 4e-3, name   # 2^-9 of the value, rounded once
+    assert xg.grad.dtype == torch.bfloat16
+    assert rel_err(xg.grad.float().cpu().numpy(), xc.grad.numpy()) < 2e-2
+
+
+def test_delta_layer_in_bf16_takes_the_one_launch_prologue():
+    """A FastFFlayer held in bf16 runs the bf16 prologue and the bf16 delta-rule operator; with the
+    prologue spelled out in (bf16) tensor operations it gives the same result within bf16 rounding."""
+    print("case FastFFlayer bf16", flush=True)
+    import layer
+    from layer import FastFFlayer
+    torch.manual_seed(11)
+    L, B, H, d = 70, 2, 2, 64
+    mod = FastFFlayer(H, d, H * d, 0.0).to(_dev()).to(torch.bfloat16)
+    x = torch.randn(L, B, H * d, device=_dev()).to(torch.bfloat16)
+    go = torch.randn(L, B, H * d, device=_dev()).to(torch.bfloat16)
+    res = {}
+    for fused in (True, False):
+        layer.FUSED_DELTA_LAYER = fused
+        try:
+            xi = x.clone().requires_grad_(True)
+            out = mod(xi)
+            out.backward(go)
+            res[fused] = (out.detach().float(), xi.grad.float(), mod.slow_net.weight.grad.float().clone())
+            mod.zero_grad()
+        finally:
+            layer.FUSED_DELTA_LAYER = True
+    for a, b, name in zip(res[True], res[False], ("out", "grad_x", "grad_slow_net")):
+        assert a.dtype == torch.float32 and rel_err(a.cpu().numpy(), b.cpu().numpy()) < 3e-2, name
+
+
 def test_delta_layers(delta_layer_path):
     print("case FastFFlayer / CarryFastFFlayer", flush=True)
     from layer import CarryFastFFlayer, FastFFlayer, elu_p1, elu_p1_sum_norm_eps, sum_norm
