@@ -43,15 +43,25 @@ def _forward_flags(E, M, L):
     return flags
 
 
-def causal_dot_product_cuda(q, k, v, beta, v_old, v_insert, kv, out):
-    srwm_hip.fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out,
-                                 flags=_forward_flags(q.shape[-1], v.shape[-1], q.shape[2]))
+def causal_dot_product_cuda(q, k, v, beta, v_old, v_insert, kv, out, flags=None):
+    """The reference's extension function (same eight arguments).  flags: the kernel choice, by default
+    what the module switches say now; returns the flags used."""
+    if flags is None:
+        flags = _forward_flags(q.shape[-1], v.shape[-1], q.shape[2])
+    srwm_hip.fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=flags)
+    return flags
 
 
-def causal_dot_backward_cuda(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v, grad_beta):
+def causal_dot_backward_cuda(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v, grad_beta,
+                             forward_flags=0):
+    """The reference's extension function (same twelve arguments).  forward_flags: what the forward ran
+    with -- a forward that wrote v_old only where a chunkwise backward reads it gets a chunkwise backward
+    whatever the switch says by now."""
+    flags = _chunk_flags(CHUNKWISE_BACKWARD, q.shape[-1], v.shape[-1], q.shape[2])
+    if forward_flags & srwm_hip.FLAG_SPARSE_V_OLD and not flags:
+        flags = _chunk_flags(True, q.shape[-1], v.shape[-1], q.shape[2])
     srwm_hip.fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v,
-                                  grad_beta,
-                                  flags=_chunk_flags(CHUNKWISE_BACKWARD, q.shape[-1], v.shape[-1], q.shape[2]))
+                                  grad_beta, flags=flags)
 
 
 class DeltaFastWeight(torch.autograd.Function):
@@ -69,7 +79,7 @@ class DeltaFastWeight(torch.autograd.Function):
         out = torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
         V_old = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
         V_insert = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
-        DeltaFastWeight.dot[device.type](Q.data, K.data, V.data, beta.data, V_old, V_insert, W, out)
+        ctx.forward_flags = DeltaFastWeight.dot[device.type](Q.data, K.data, V.data, beta.data, V_old, V_insert, W, out)
         ctx.save_for_backward(Q, K, V, beta, V_old, V_insert, W)
         return out
 
@@ -84,7 +94,7 @@ class DeltaFastWeight(torch.autograd.Function):
             grad_out = grad_out.to(Q.dtype)
         DeltaFastWeight.dot_backward[Q.device.type](
             Q.data, K.data, V.data, beta.data, V_old.data, V_insert.data, grad_out, W.data,
-            grad_Q, grad_K, grad_V, grad_beta)
+            grad_Q, grad_K, grad_V, grad_beta, forward_flags=ctx.forward_flags or 0)
         return grad_Q, grad_K, grad_V, grad_beta, None
 
 

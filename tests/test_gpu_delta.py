@@ -397,6 +397,20 @@ def test_chunkwise_forward_can_leave_out_the_v_old_that_nobody_reads(shape, io):
     for a, b in zip(f[4], s[4]):
         assert torch.equal(a, b)
     assert torch.equal(f[5], s[5])
+    # the operator: a forward that left rows of v_old out gets the chunkwise backward even if the switch
+    # has been turned since
+    import fast_weight
+    leaves = [t.clone().requires_grad_() for t in (qd, kd, vd, bd)]
+    out = fast_weight.fast_weight_delta(*leaves, W0.to(dev, torch.float32).contiguous())
+    old = fast_weight.CHUNKWISE_BACKWARD
+    fast_weight.CHUNKWISE_BACKWARD = False
+    try:
+        out.backward(god)
+    finally:
+        fast_weight.CHUNKWISE_BACKWARD = old
+    torch.cuda.synchronize()
+    for i in range(3):
+        assert torch.equal(leaves[i].grad, f[4][i]), i
 
 
 @pytest.mark.parametrize("shape,qk,small_betas", [
