@@ -175,5 +175,14 @@ def test_argument_validation_needs_no_gpu():
         gq, fake(), fake(), fake(), N, H, Ls, E, E, flags, P(None))
     assert dsteps(P(None), 0) == -1                            # every gradient buffer is required
     assert dsteps(fake(), 32) == -1                            # there is no chunkwise form of the step mode
+    prologue = lambda rows, flags, e: L.delta_layer_prologue_f32(rows, *[fake() for _ in range(5)], N, H, Ls, e, e, flags, P(None))
+    assert prologue(P(None), 0, E) == -1                       # every buffer is required
+    assert prologue(fake(), 32, E) == -1                       # the only flag it knows is the 1e-5 of the RL tree's normalisation
+    assert prologue(fake(), 2048, 0) == -1                     # empty rows
+    pgrad = lambda st, flags: L.delta_layer_prologue_grad_bf16(*[a for _ in range(4) for a in (fake(), st)],
+                                                               *[fake() for _ in range(5)], N, H, Ls, E, E, flags, P(None))
+    assert pgrad(None, 0) == -1                                # gradients come with their strides
+    assert pgrad(ok_strides, 2048) == -1                       # the backward takes no flag
+    assert pgrad(huge, 0) == -3                                # SRWM_ESTRIDE
     assert L.srwm_hip_scratch_bytes() == 32 << 20
     assert b"scratch" in L.srwm_hip_strerror(-5)
