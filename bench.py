@@ -21,7 +21,7 @@ matrix-core peak.  `cpu_baseline` is the per-timestep PyTorch recurrence (oracle
 timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (through the autograd operator), delta_prologue_c2 (the layers' prologue kernels, HBM-bound), delta_layer_c2 (a whole delta-rule layer)}.
+{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (through the autograd operator), delta_prologue_c2, delta_prologue_c5 (the layers' prologue kernels, fp32 and bf16, HBM-bound), delta_layer_c2 (a whole delta-rule layer)}.
 """
 import argparse
 import json
@@ -77,6 +77,8 @@ WORKLOADS = {
     # the prologue of the delta-rule layers at the shape of configuration 2 (projection rows [q~ | k~ | v | b~] ->
     # normalised q, k, v, beta) and its backward: two memory-bound launches, priced against HBM
     "delta_prologue_c2": ("delta_prologue", 32, 8, 256, 64),
+    # the same in bf16 at the shape of configuration 5
+    "delta_prologue_c5": ("delta_prologue_bf16", 8, 16, 4096, 128),
     # a whole delta-rule layer at that shape (layer.FastFFlayer, model width 256: layer norm, projection, prologue,
     # recurrence, output map, residual) through autograd: the recurrence kernels are a quarter of it
     "delta_layer_c2": ("delta_layer", 32, 8, 256, 64),
@@ -254,13 +256,14 @@ def delta_op_step(t, ev=None):
         t[n].grad = None
 
 
-def delta_prologue_setup(N, H, L, E, dev):
+def delta_prologue_setup(N, H, L, E, dev, bf16=False):
     import torch
     g = torch.Generator().manual_seed(0)
     W = 3 * E + 1
-    t = dict(rows=torch.randn(L, N, H, W, generator=g).to(dev))
+    dt = torch.bfloat16 if bf16 else torch.float32
+    t = dict(rows=torch.randn(L, N, H, W, generator=g).to(dev, dt))
     for n, w in (("gq", E), ("gk", E), ("gv", E), ("gb", 1)):
-        t[n] = torch.randn(N, H, L, w, generator=g).to(dev)
+        t[n] = torch.randn(N, H, L, w, generator=g).to(dev, dt)
     return t
 
 
@@ -312,16 +315,21 @@ def delta_layer_tensor_ops_ms(t, steps=30):
     return median(f) + median(b)
 
 
+def prologue_bytes(op, N, H, L, E):
+    """(forward, backward) HBM bytes of the layers' prologue kernels.  Forward: the row in, q, k, v, beta and the two
+    normalisers (fp32 in either type) out; backward: the four gradients, q, k, beta and the normalisers in, the
+    row's gradient out.  No state: nothing to pass over in LDS."""
+    W, es, hs = 3 * E + 1, 2 if op.endswith("bf16") else 4, N * H * L
+    return ((W + W) * es + 8) * hs, ((W + 2 * E + 1 + W) * es + 8) * hs
+
+
 def algorithmic_bytes(op, N, H, L, E, bf16_grads=False, no_v_old=False):
     """(lds_fwd, lds_bwd, hbm_total) bytes per launch pair."""
     hs = N * H * L
     if op == "delta_layer":   # the recurrence inside the layer
         op = "delta"
-    if op == "delta_prologue":
-        # forward: the row in, q, k, v, beta and the two normalisers out; backward: the four gradients, q, k,
-        # beta and the normalisers in, the row's gradient out.  No state: nothing to pass over in LDS.
-        W = 3 * E + 1
-        return 0, 0, ((W + W + 2) + (W + 2 * E + 3 + W)) * 4 * hs
+    if op in ("delta_prologue", "delta_prologue_bf16"):
+        return 0, 0, sum(prologue_bytes(op, N, H, L, E))
     if op in ("srwm", "srwm_layer"):
         S = E * (3 * E + 4)
         return 3 * S * 4 * hs, 6 * S * 4 * hs, (15 * E + 16) * 4 * hs + 4 * S * 4 * N * H
@@ -467,8 +475,8 @@ def build_workload(name, dev):
         step, t = srwm_step, srwm_setup(N, H, L, E, dev, 3 * E + 1)
     elif op == "srwm_steps":
         step, t = srwm_steps_step, srwm_steps_setup(N, H, L, E, dev)
-    elif op == "delta_prologue":
-        step, t = delta_prologue_step, delta_prologue_setup(N, H, L, E, dev)
+    elif op in ("delta_prologue", "delta_prologue_bf16"):
+        step, t = delta_prologue_step, delta_prologue_setup(N, H, L, E, dev, bf16=op.endswith("bf16"))
     elif op == "delta_layer":
         step, t = delta_layer_step, delta_layer_setup(N, H, L, E, dev)
     else:
@@ -525,11 +533,10 @@ def rooflines(name, fwd_ms, bwd_ms):
     lds_f, lds_b, hbm = algorithmic_bytes(op, N, H, L, E, bf16_grads=name.endswith("_chunk") and op == "delta_bf16",
                                           no_v_old=name.endswith("_chunk"))
     r = {}
-    if op == "delta_prologue":
-        W = 3 * E + 1
-        hs = N * H * L
-        r["roofline"] = dict(roof("hbm", (W + 2 * E + 3 + W) * 4 * hs, bwd_ms, HBM_PEAK_GBS), kernel="backward")
-        r["roofline_fwd"] = dict(roof("hbm", (W + W + 2) * 4 * hs, fwd_ms, HBM_PEAK_GBS), kernel="forward")
+    if op in ("delta_prologue", "delta_prologue_bf16"):
+        bf, bb = prologue_bytes(op, N, H, L, E)
+        r["roofline"] = dict(roof("hbm", bb, bwd_ms, HBM_PEAK_GBS), kernel="backward")
+        r["roofline_fwd"] = dict(roof("hbm", bf, fwd_ms, HBM_PEAK_GBS), kernel="forward")
         r["roofline_fwd_bwd"] = roof("hbm", hbm, fwd_ms + bwd_ms, HBM_PEAK_GBS)
         return r
     if name.endswith("_chunk"):
@@ -559,7 +566,8 @@ def rooflines(name, fwd_ms, bwd_ms):
 
 # Driver-visible figures for the other benchmark configurations: (workload, timed steps, warm-up)
 OTHER_WORKLOADS = (("srwm_layer_c4", 50, 10), ("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
-                   ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5), ("delta_c5_op_chunk", 40, 5), ("delta_prologue_c2", 100, 20), ("delta_layer_c2", 50, 10))
+                   ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5), ("delta_c5_op_chunk", 40, 5), ("delta_prologue_c2", 100, 20), ("delta_prologue_c5", 40, 5),
+                   ("delta_layer_c2", 50, 10))
 
 
 def main():
@@ -598,7 +606,7 @@ def main():
                   if a.workload == "srwm_c4" else f"fwd+bwd tokens/sec {a.workload}",
         "value": round(tokens_per_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps,
         "warmup": a.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32" if op != "delta_bf16" else "f32 (bf16 I/O)",
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32 (bf16 I/O)" if op.endswith("bf16") else "f32",
         "data": "synthetic",
         "config": {"workload": f"{a.workload}: {op} fwd+bwd N={N} H={H} L={L} E={E}, fp32 state, "
                                "state re-initialised per step, seeded synthetic inputs"},

@@ -11,12 +11,13 @@
 // writes q, k, v, beta (dense rows in the row order of the input, which the operator reads through
 // strides), and one kernel turns the operator's four gradients into the gradient of the rows.
 //
-// A wave owns a row; its lanes own the elements e, e + 64, ...  Arithmetic in fp32; the tensors are fp32 or,
-// for the bf16 twins, bf16 throughout (the two normalisers stay fp32).  Rows of up to 128
-// elements per part (the sizes the layers use) take a form in which a wave works on four rows at once and
-// issues all their loads before it uses any: one row per wave leaves too few bytes in flight to cover the
-// memory latency (at E = M = 64 and 65 536 rows: 24.5 + 35.2 us and 4 TB/s with one row per wave,
-// 19.6 + 27.7 us and 5 TB/s with four; eight gain nothing more).
+// Arithmetic in fp32; the tensors are fp32 or, for the bf16 twins, bf16 throughout (the two normalisers stay
+// fp32).  Three forms.  The general one: a wave owns a row, its lanes the elements e, e + 64, ...  Rows of up to
+// 128 elements per part (the sizes the layers use): a wave works on four rows at once and issues all their loads
+// before it uses any -- one row per wave leaves too few bytes in flight to cover the memory latency (fp32, E = M =
+// 64, 65 536 rows: 24.5 + 35.2 us and 4 TB/s with one row per wave, 19.6 + 27.7 us and 5 TB/s with four; eight
+// gain nothing more).  bf16 with even E, M <= 128: rows staged through LDS and 2 or 4 adjacent elements per lane,
+// see there.
 #include "common.h"
 #include "xlane.h"
 
@@ -235,60 +236,212 @@ __global__ __launch_bounds__(kWave *kRowsPerGroup) void delta_prologue_grad_smal
     }
 }
 
-// ---- forward with the rows staged through LDS (bf16) ---------------------------------------------------
+// ---- bf16: rows staged through LDS, 2 or 4 elements per lane ---------------------------------------------
 // The rows are 2E + M + 1 elements long, an odd number: every other row starts off a 4-byte boundary, so lanes
-// that address rows can move one bf16 element each, and an instruction that moves 64 x 2 bytes keeps the
-// address path as busy as one that moves 64 x 16.  Sixteen consecutive rows are one aligned, contiguous piece
-// of memory: a workgroup brings that piece into LDS with 16-byte loads and addresses rows only there; q, k, v
-// rows are aligned and go out as element pairs.  E and M even and at most 128.  (At E = M = 128 in bf16, 524 288
-// rows: 233 -> 157 us.  With fp32 rows the four-rows-per-wave form is as fast or faster, and so it is for the
-// backward, whose gradients lie in the operator's order and are scattered rows either way; a form that also
-// transposes q, k, v and the gradients into the operator's order through LDS tiles was slower in both.)
+// that address rows in global memory can move one bf16 element each, and these kernels are bound by the number of
+// memory instructions, not by the bytes (with one element per lane and instruction the bf16 backward took as long
+// as the fp32 one, for half the bytes).  Sixteen consecutive rows are one aligned, contiguous piece of memory: a
+// workgroup moves that piece between global memory and LDS with 16-byte accesses and addresses rows only in LDS.
+// The rows of q, k, v and of the gradients are aligned: a lane owns a pair of adjacent elements of each and moves
+// it with one 4-byte access, or four with one 8-byte access where E and M are multiples of 4 and the rows start
+// on 8-byte boundaries; LPR = 16, 32 or 64 lanes share a row, so a wave works on 4, 2 or 1 rows at a time with
+// few idle lanes.  E and M even and at most 128.  (524 288 rows, forward + backward: E = M = 128 157 + 371 us with
+// one element per lane (the forward already staged), 152 + 250 us with pairs, 148 + 217 us with fours, which is
+// 5.5 and 5.0 TB/s; E = M = 64 126 + 214 -> 79 + 112 us.  fp32 rows move 4 bytes per lane as they are and reach 5.6 and
+// 5.0 TB/s at that size in the four-rows-per-wave form.)
 constexpr int kStageRows = 16;            // per workgroup: 4 waves x 4 rows
 constexpr int kStageThreads = 4 * kWave;
 
-__device__ __forceinline__ void st_pair(float *p, float a, float b) { *reinterpret_cast<float2 *>(p) = make_float2(a, b); }
-__device__ __forceinline__ void st_pair(uint16_t *p, float a, float b) {
-    *reinterpret_cast<uint32_t *>(p) = (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+// VE = 2 or 4 adjacent bf16 elements as one 4- or 8-byte word
+template <int VE> struct Pack;
+template <> struct Pack<2> { typedef uint32_t type; };
+template <> struct Pack<4> { typedef uint2 type; };
+__device__ __forceinline__ uint32_t word_of(uint32_t w, int) { return w; }
+__device__ __forceinline__ uint32_t word_of(uint2 w, int j) { return j ? w.y : w.x; }
+template <int VE>
+__device__ __forceinline__ typename Pack<VE>::type ld_pack(const uint16_t *p, bool in) {
+    typedef typename Pack<VE>::type P;
+    return in ? *reinterpret_cast<const P *>(p) : P{};
+}
+template <int VE, class P>
+__device__ __forceinline__ void unpack(P w, float (&f)[VE]) {
+#pragma unroll
+    for (int j = 0; j < VE; j += 2) {
+        f[j] = __uint_as_float(word_of(w, j / 2) << 16);
+        f[j + 1] = __uint_as_float(word_of(w, j / 2) & 0xFFFF0000u);
+    }
+}
+__device__ __forceinline__ uint32_t pack_pair(float a, float b) {
+    return (uint32_t)f32_to_bf16_bits(a) | ((uint32_t)f32_to_bf16_bits(b) << 16);
+}
+__device__ __forceinline__ void st_pack(uint16_t *p, const float (&f)[2]) {
+    *reinterpret_cast<uint32_t *>(p) = pack_pair(f[0], f[1]);
+}
+__device__ __forceinline__ void st_pack(uint16_t *p, const float (&f)[4]) {
+    *reinterpret_cast<uint2 *>(p) = make_uint2(pack_pair(f[0], f[1]), pack_pair(f[2], f[3]));
+}
+__device__ __forceinline__ void st_raw(uint16_t *p, const uint16_t (&f)[2]) {
+    *reinterpret_cast<uint32_t *>(p) = (uint32_t)f[0] | ((uint32_t)f[1] << 16);
+}
+__device__ __forceinline__ void st_raw(uint16_t *p, const uint16_t (&f)[4]) {
+    *reinterpret_cast<uint2 *>(p) = make_uint2((uint32_t)f[0] | ((uint32_t)f[1] << 16), (uint32_t)f[2] | ((uint32_t)f[3] << 16));
 }
 
-template <class T>
-__global__ __launch_bounds__(kStageThreads) void delta_prologue_staged_kernel(PrologueP<T> p) {
+// the piece of 16 rows (or fewer, at the end) between global memory and LDS: 16-byte vectors, the last few
+// elements singly; the piece starts on a 16-byte boundary
+template <bool IN>
+__device__ __forceinline__ void move_rows(uint16_t *lds, uint16_t *glob, int count, int tid) {
+    const int nv = count / 8;
+    for (int i = tid; i < nv; i += kStageThreads) {
+        if constexpr (IN)
+            reinterpret_cast<uint4 *>(lds)[i] = reinterpret_cast<const uint4 *>(glob)[i];
+        else
+            reinterpret_cast<uint4 *>(glob)[i] = reinterpret_cast<const uint4 *>(lds)[i];
+    }
+    for (int i = nv * 8 + tid; i < count; i += kStageThreads) {
+        if constexpr (IN)
+            lds[i] = glob[i];
+        else
+            glob[i] = lds[i];
+    }
+}
+
+template <int LPR, int VE>
+__global__ __launch_bounds__(kStageThreads) void delta_prologue_staged_kernel(PrologueP<uint16_t> p) {
+    constexpr int RPP = kWave / LPR;   // rows a wave works on at once
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    T *sx = reinterpret_cast<T *>(smem);
+    uint16_t *sx = reinterpret_cast<uint16_t *>(smem);
     const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    const int sub = lane / LPR, sl = lane % LPR;
     const int64_t row0 = (int64_t)blockIdx.x * kStageRows;
     const int nrows = (int)(p.rows - row0 < kStageRows ? p.rows - row0 : kStageRows);
     const int E = p.E, M = p.M, W = 2 * E + M + 1;
-    {   // the group's rows: 16-byte vectors, the last few elements singly (both ends 16-byte aligned)
-        constexpr int VE = 16 / (int)sizeof(T);
-        const T *src = p.x + row0 * W;
-        const int count = nrows * W, nv = count / VE;
-        for (int i = tid; i < nv; i += kStageThreads) reinterpret_cast<uint4 *>(sx)[i] = reinterpret_cast<const uint4 *>(src)[i];
-        for (int i = nv * VE + tid; i < count; i += kStageThreads) sx[i] = src[i];
-    }
+    move_rows<true>(sx, const_cast<uint16_t *>(p.x) + row0 * W, nrows * W, tid);
     __syncthreads();
-    const int e0 = 2 * lane;   // this lane's pair in each part
+    const int e0 = VE * sl;   // this lane's elements in each part
     const bool ie = e0 < E, im = e0 < M;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int lr = 4 * wv + r;
-        if (lr >= nrows) break;   // the same in every lane of a wave
+    for (int r = 0; r < 4; r += RPP) {
+        if (4 * wv + r >= nrows) break;   // the same in every lane of a wave
+        const int lr = 4 * wv + r + sub;
+        const bool live = lr < nrows;
         const int64_t row = row0 + lr;
-        const T *x = sx + lr * W;
-        const float q0 = ie ? elu_p1(ldf(x + e0)) : 0.f, q1 = ie ? elu_p1(ldf(x + e0 + 1)) : 0.f;
-        const float k0 = ie ? elu_p1(ldf(x + E + e0)) : 0.f, k1 = ie ? elu_p1(ldf(x + E + e0 + 1)) : 0.f;
-        const float sq = wave_sum(q0 + q1) + p.eps, sk = wave_sum(k0 + k1) + p.eps;
-        if (ie) {
-            st_pair(p.q + row * E + e0, q0 / sq, q1 / sq);
-            st_pair(p.k + row * E + e0, k0 / sk, k1 / sk);
+        const uint16_t *x = sx + (live ? lr : 0) * W;
+        float q[VE], k[VE], tq = 0.f, tk = 0.f;
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+            q[j] = ie ? elu_p1(ldf(x + e0 + j)) : 0.f;
+            k[j] = ie ? elu_p1(ldf(x + E + e0 + j)) : 0.f;
+            tq += q[j];
+            tk += k[j];
         }
-        if (im) st_pair(p.v + row * M + e0, ldf(x + 2 * E + e0), ldf(x + 2 * E + e0 + 1));   // bf16 -> fp32 -> bf16 is exact
-        if (lane == 0) {
+        const float sq = group_sum<LPR>(tq) + p.eps, sk = group_sum<LPR>(tk) + p.eps;
+        if (live && ie) {
+#pragma unroll
+            for (int j = 0; j < VE; ++j) {
+                q[j] /= sq;
+                k[j] /= sk;
+            }
+            st_pack(p.q + row * E + e0, q);
+            st_pack(p.k + row * E + e0, k);
+        }
+        if (live && im) {
+            uint16_t v[VE];
+#pragma unroll
+            for (int j = 0; j < VE; ++j) v[j] = x[2 * E + e0 + j];
+            st_raw(p.v + row * M + e0, v);
+        }
+        if (live && sl == 0) {
             stf(p.beta + row, 1.f / (1.f + __expf(-ldf(x + 2 * E + M))));
-            p.sums[2 * row] = sq;
-            p.sums[2 * row + 1] = sk;
+            *reinterpret_cast<float2 *>(p.sums + 2 * row) = make_float2(sq, sk);
         }
+    }
+}
+
+// Backward: the gradients and the saved q, k of the wave's four rows are all requested before the first is used;
+// the rows of the result are put together in LDS and leave as one piece.
+template <int LPR, int VE>
+__global__ __launch_bounds__(kStageThreads) void delta_prologue_grad_staged_kernel(PrologueGradP<uint16_t> p) {
+    constexpr int RPP = kWave / LPR, NP = 4 / RPP;   // rows at once, passes
+    typedef typename Pack<VE>::type P;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    uint16_t *sx = reinterpret_cast<uint16_t *>(smem);
+    const int tid = threadIdx.x, lane = tid & (kWave - 1), wv = tid / kWave;
+    const int sub = lane / LPR, sl = lane % LPR;
+    const int64_t rows = (int64_t)p.L * p.N * p.H;
+    const int64_t row0 = (int64_t)blockIdx.x * kStageRows;
+    const int nrows = (int)(rows - row0 < kStageRows ? rows - row0 : kStageRows);
+    const int E = p.E, M = p.M, W = 2 * E + M + 1;
+    const int e0 = VE * sl;
+    const bool ie = e0 < E, im = e0 < M;
+    P gq[NP], gk[NP], gv[NP], q[NP], k[NP];
+    uint16_t gb[NP], bt[NP];
+    float2 sm[NP];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int64_t row = min(row0 + 4 * wv + i * RPP + sub, rows - 1);   // rows past the end repeat the last one
+        const int h = (int)(row % p.H), n = (int)((row / p.H) % p.N), l = (int)(row / ((int64_t)p.H * p.N));
+        gq[i] = ld_pack<VE>(p.gq + n * p.gqs.n + h * p.gqs.h + l * p.gqs.l + e0, ie);
+        gk[i] = ld_pack<VE>(p.gk + n * p.gks.n + h * p.gks.h + l * p.gks.l + e0, ie);
+        gv[i] = ld_pack<VE>(p.gv + n * p.gvs.n + h * p.gvs.h + l * p.gvs.l + e0, im);
+        q[i] = ld_pack<VE>(p.q + row * E + e0, ie);
+        k[i] = ld_pack<VE>(p.k + row * E + e0, ie);
+        gb[i] = p.gb[n * p.gbs.n + h * p.gbs.h + l * p.gbs.l];
+        bt[i] = p.beta[row];
+        sm[i] = *reinterpret_cast<const float2 *>(p.sums + 2 * row);
+    }
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+        const int lr = 4 * wv + i * RPP + sub;
+        const bool live = lr < nrows;
+        uint16_t *gx = sx + lr * W;
+        float qf[VE], kf[VE], gqf[VE], gkf[VE], tq = 0.f, tk = 0.f;
+        unpack<VE>(q[i], qf);
+        unpack<VE>(k[i], kf);
+        unpack<VE>(gq[i], gqf);
+        unpack<VE>(gk[i], gkf);
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {   // lanes past E hold zeros
+            tq += gqf[j] * qf[j];
+            tk += gkf[j] * kf[j];
+        }
+        const float dq = group_sum<LPR>(tq), dk = group_sum<LPR>(tk);
+        const float sq = sm[i].x, sk = sm[i].y;
+        if (live && ie) {
+#pragma unroll
+            for (int j = 0; j < VE; ++j) {
+                const float a = qf[j] * sq, b = kf[j] * sk;
+                gx[e0 + j] = f32_to_bf16_bits((gqf[j] - dq) / sq * (a > 1.f ? 1.f : a));
+                gx[E + e0 + j] = f32_to_bf16_bits((gkf[j] - dk) / sk * (b > 1.f ? 1.f : b));
+            }
+        }
+        if (live && im) {
+#pragma unroll
+            for (int j = 0; j < VE; ++j) gx[2 * E + e0 + j] = (uint16_t)(word_of(gv[i], j / 2) >> (16 * (j & 1)));
+        }
+        const float btf = ldf(&bt[i]);
+        if (live && sl == 0) gx[2 * E + M] = f32_to_bf16_bits(ldf(&gb[i]) * btf * (1.f - btf));
+    }
+    __syncthreads();
+    move_rows<false>(sx, p.gx + row0 * W, nrows * W, tid);
+}
+
+// The staged kernels' form for the sizes: VE elements per lane (4 where everything is a multiple of 4 and rows start on
+// 8-byte boundaries), LPR lanes per row.  `f` launches the kernel it is handed <LPR, VE> of.
+template <class F>
+void pick_staged_form(int widest, bool quads, F f) {
+    const int lanes = widest / (quads ? 4 : 2);
+    if (quads) {
+        if (lanes <= 16)
+            f(std::integral_constant<int, 16>(), std::integral_constant<int, 4>());
+        else
+            f(std::integral_constant<int, 32>(), std::integral_constant<int, 4>());
+    } else if (lanes <= 16) {
+        f(std::integral_constant<int, 16>(), std::integral_constant<int, 2>());
+    } else if (lanes <= 32) {
+        f(std::integral_constant<int, 32>(), std::integral_constant<int, 2>());
+    } else {
+        f(std::integral_constant<int, 64>(), std::integral_constant<int, 2>());
     }
 }
 
@@ -299,13 +452,20 @@ int launch_prologue(const T *x, T *q, T *k, T *v, T *beta, float *sums, int N, i
                     hipStream_t s) {
     const int64_t rows = (int64_t)L * N * H;
     const PrologueP<T> p{x, q, k, v, beta, sums, rows, E, M, eps};
-    if (sizeof(T) == 2 && E % 2 == 0 && M % 2 == 0 && E <= 2 * kWave && M <= 2 * kWave && aligned_to(x, 16) &&
-        aligned_to(q, 4) && aligned_to(k, 4) && aligned_to(v, 4)) {
-        const int64_t groups = (rows + kStageRows - 1) / kStageRows;
-        if (groups > 0x7FFFFFFF) return -1;
-        hipLaunchKernelGGL(delta_prologue_staged_kernel<T>, dim3((unsigned)groups), dim3(kStageThreads),
-                           kStageRows * (2 * E + M + 1) * sizeof(T), s, p);
-        return (int)hipGetLastError();
+    if constexpr (sizeof(T) == 2) {
+        if (E % 2 == 0 && M % 2 == 0 && E <= 2 * kWave && M <= 2 * kWave && aligned_to(x, 16) && aligned_to(q, 4) &&
+            aligned_to(k, 4) && aligned_to(v, 4) && aligned_to(sums, 8)) {
+            const int64_t groups = (rows + kStageRows - 1) / kStageRows;
+            if (groups > 0x7FFFFFFF) return -1;
+            const dim3 grid((unsigned)groups), block(kStageThreads);
+            const size_t lds = kStageRows * (2 * E + M + 1) * sizeof(T);
+            const bool quads = E % 4 == 0 && M % 4 == 0 && aligned_to(q, 8) && aligned_to(k, 8) && aligned_to(v, 8);
+            pick_staged_form(max(E, M), quads, [&](auto lpr, auto ve) {
+                hipLaunchKernelGGL((delta_prologue_staged_kernel<decltype(lpr)::value, decltype(ve)::value>), grid, block,
+                                   lds, s, p);
+            });
+            return (int)hipGetLastError();
+        }
     }
     const int epl = (max(E, M) + kWave - 1) / kWave;   // elements of a part per lane
     const bool small = epl <= 2;
@@ -328,6 +488,25 @@ int launch_prologue_grad(const T *gq, const Strided3 &gqs, const T *gk, const St
                          const float *sums, T *gx, int N, int H, int L, int E, int M, hipStream_t s) {
     const int64_t rows = (int64_t)L * N * H;
     const PrologueGradP<T> p{gq, gk, gv, gb, gqs, gks, gvs, gbs, q, k, beta, sums, gx, N, H, L, E, M};
+    if constexpr (sizeof(T) == 2) {
+        const auto rows_on = [](const void *base, const Strided3 &st, int el) {   // rows start on multiples of `el` elements
+            return aligned_to(base, 2 * el) && st.n % el == 0 && st.h % el == 0 && st.l % el == 0;
+        };
+        if (E % 2 == 0 && M % 2 == 0 && E <= 2 * kWave && M <= 2 * kWave && aligned_to(gx, 16) && aligned_to(q, 4) &&
+            aligned_to(k, 4) && aligned_to(sums, 8) && rows_on(gq, gqs, 2) && rows_on(gk, gks, 2) && rows_on(gv, gvs, 2)) {
+            const int64_t groups = (rows + kStageRows - 1) / kStageRows;
+            if (groups > 0x7FFFFFFF) return -1;
+            const dim3 grid((unsigned)groups), block(kStageThreads);
+            const size_t lds = kStageRows * (2 * E + M + 1) * sizeof(T);
+            const bool quads = E % 4 == 0 && M % 4 == 0 && aligned_to(q, 8) && aligned_to(k, 8) && rows_on(gq, gqs, 4) &&
+                               rows_on(gk, gks, 4) && rows_on(gv, gvs, 4);
+            pick_staged_form(max(E, M), quads, [&](auto lpr, auto ve) {
+                hipLaunchKernelGGL((delta_prologue_grad_staged_kernel<decltype(lpr)::value, decltype(ve)::value>), grid,
+                                   block, lds, s, p);
+            });
+            return (int)hipGetLastError();
+        }
+    }
     const int epl = (max(E, M) + kWave - 1) / kWave;
     const bool small = epl <= 2;
     const int per_group = kRowsPerGroup * (small ? kRowsPerWave : 1);

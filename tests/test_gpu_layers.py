@@ -220,7 +220,9 @@ def test_delta_layer_prologue_matches_the_tensor_operations(L, B, H, E, M, eps):
 
 
 @pytest.mark.parametrize("L,B,H,E,M,eps", [(9, 3, 4, 16, 16, False), (6, 2, 3, 64, 64, True), (3, 2, 2, 128, 128, False),
-                                            (130, 2, 4, 32, 32, True)])
+                                            (130, 2, 4, 32, 32, True), (7, 3, 1, 6, 6, True), (5, 1, 3, 40, 8, False),
+                                            (11, 1, 3, 66, 66, True), (3, 5, 1, 126, 128, False), (4, 1, 5, 64, 128, True),
+                                            (2, 3, 3, 8, 4, False), (1, 1, 1, 128, 128, True), (3, 2, 2, 33, 64, False)])
 def test_delta_layer_prologue_in_bf16(L, B, H, E, M, eps):
     """The bf16 twins of the prologue kernels (every tensor but the normalisers in bf16, arithmetic in
     fp32) against the fp64 statement on the same bf16-rounded projection: outputs within the rounding
@@ -243,6 +245,43 @@ def test_delta_layer_prologue_in_bf16(L, B, H, E, M, eps):
         assert rel_err(o.detach().float().cpu().numpy(), r.detach().numpy()) < 4e-3, name   # 2^-9 of the value, rounded once
     assert xg.grad.dtype == torch.bfloat16
     assert rel_err(xg.grad.float().cpu().numpy(), xc.grad.numpy()) < 2e-2
+
+
+@pytest.mark.parametrize("E,M", [(128, 128), (64, 64), (32, 16)])
+def test_delta_layer_prologue_gradient_takes_gradients_wherever_they_lie(E, M):
+    """The bf16 backward moves 4 or 2 adjacent elements per lane where the gradients' rows start on 8- or 4-byte
+    boundaries and single elements otherwise: the operator's own layout, rows cut out of wider buffers at an even and
+    at an odd element, and a batch-major copy all give the gradient of the fp64 statement."""
+    print(f"case delta layer prologue bf16 gradient layouts E={E} M={M}", flush=True)
+    import srwm_hip
+    from oracle.recurrence import delta_layer_inputs_reference
+    L, B, H = 21, 2, 3   # 126 rows: the last group of 16 is cut short
+    g = torch.Generator().manual_seed(E + M)
+    x = (2.0 * torch.randn(L, B, H, 2 * E + M + 1, generator=g)).to(torch.bfloat16)
+    gs = [torch.randn(B, H, L, w, generator=g).to(torch.bfloat16) for w in (E, E, M, 1)]
+    q, k, v, beta, sums = srwm_hip.delta_layer_prologue(x.to(_dev()), E, M, True)
+    # the gradient of the rows through the fp64 statement, from the kernel's own (rounded) q, k, beta as the kernel does
+    xc = x.to(torch.float64).requires_grad_(True)
+    ref = delta_layer_inputs_reference(xc, E, M, True)
+    sum((r * gi.to(torch.float64)).sum() for r, gi in zip(ref, gs)).backward()
+    want = xc.grad.numpy()
+
+    def cut_out(t, at):   # the same values as rows of a buffer `at` elements wider, starting at element `at`
+        wide = torch.zeros(*t.shape[:-1], t.shape[-1] + at + (at & 1), dtype=t.dtype, device=_dev())
+        wide[..., at:at + t.shape[-1]] = t.to(_dev())
+        return wide[..., at:at + t.shape[-1]]
+
+    layouts = {
+        "operator": [t.to(_dev()) for t in gs],
+        "cut at 2": [cut_out(t, 2) for t in gs[:3]] + [gs[3].to(_dev())],
+        "cut at 1": [cut_out(t, 1) for t in gs[:3]] + [gs[3].to(_dev())],
+        "step-major": [t.to(_dev()).permute(2, 0, 1, 3).contiguous().permute(1, 2, 0, 3) for t in gs],
+    }
+    for name, gd in layouts.items():
+        got = srwm_hip.delta_layer_prologue_grad(gd[0], gd[1], gd[2], gd[3], q, k, beta, sums)
+        torch.cuda.synchronize()
+        assert got.dtype == torch.bfloat16 and got.shape == x.shape, name
+        assert rel_err(got.float().cpu().numpy(), want) < 2e-2, name
 
 
 def test_delta_layer_in_bf16_takes_the_one_launch_prologue():
