@@ -347,14 +347,19 @@ SRWM_API int srwm_layer_readout_grad_f32(const float *x, const int64_t x_strides
  * fast_weight/fast_weight_cuda.cu:182-240 (kernel :17-178).  Per sequence, W is E x M:
  *     v_old = W^T k_t;  ins = beta_t (v_t - v_old);  W += k_t (x) ins;  out_t = W^T q_t
  *   Q,K      strided [N,H,L,E];  V strided [N,H,L,M];  beta strided [N,H,L,1]
- *   v_old, v_insert, out   dense [N,H,L,M] (overwritten)
+ *   v_old, v_insert   dense [N,H,L,M] (overwritten)
+ *   out      [N,H,L,M] (overwritten), dense when out_strides is NULL, else with those strides (in elements,
+ *            of N, H, L; rows contiguous) -- rows that share memory are refused (SRWM_ESTRIDE).  The
+ *            reference's layers go on with out.transpose(1, 2).reshape(N, L, H*M).transpose(0, 1)
+ *            (supervised_learning/layer.py:96-101): with the strides of a [L,N,H,M] buffer,
+ *            (H*M, M, N*H*M), that chain is a view and the two copies it otherwise makes are not needed.
  *   W        dense [N,H,E,M], in: W_0, out: W_L (in place, as the reference, :171-177)
  */
 SRWM_API int delta_forward_f32(const float *Q, const int64_t q_strides[3],
                       const float *K, const int64_t k_strides[3],
                       const float *V, const int64_t v_strides[3],
                       const float *beta, const int64_t beta_strides[3],
-                      float *v_old, float *v_insert, float *W, float *out,
+                      float *v_old, float *v_insert, float *W, float *out, const int64_t out_strides[3],
                       int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
 /*
@@ -444,7 +449,7 @@ SRWM_API int delta_forward_bf16(const uint16_t *Q, const int64_t q_strides[3],
                        const uint16_t *K, const int64_t k_strides[3],
                        const uint16_t *V, const int64_t v_strides[3],
                        const uint16_t *beta, const int64_t beta_strides[3],
-                       float *v_old, float *v_insert, float *W, uint16_t *out,
+                       float *v_old, float *v_insert, float *W, uint16_t *out, const int64_t out_strides[3],
                        int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
 SRWM_API int delta_backward_bf16(const uint16_t *Q, const int64_t q_strides[3],
@@ -509,7 +514,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 12. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 13. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

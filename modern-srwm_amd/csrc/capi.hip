@@ -29,6 +29,27 @@ bool stride_ok(const int64_t s[3], int N, int H, int L, int width) {
     return ext > 0 && ext < ((int64_t)1 << 40);
 }
 
+// Strides of an OUTPUT of shape [N][H][L][width] with a contiguous last axis: besides the above, no two rows may
+// share memory -- in the order of their strides, each axis steps over everything the smaller ones span.
+bool out_stride_ok(const int64_t s[3], int N, int H, int L, int width) {
+    if (!stride_ok(s, N, H, L, width)) return false;
+    int64_t st[3] = {s[0], s[1], s[2]}, ex[3] = {N, H, L};
+    for (int i = 0; i < 3; ++i)
+        for (int j = i + 1; j < 3; ++j)
+            if (st[j] < st[i]) {
+                const int64_t a = st[i], b = ex[i];
+                st[i] = st[j], ex[i] = ex[j];
+                st[j] = a, ex[j] = b;
+            }
+    int64_t span = width;   // elements covered by the axes handled so far
+    for (int i = 0; i < 3; ++i) {
+        if (ex[i] == 1) continue;   // the stride of an axis of one is never used
+        if (st[i] < span) return false;
+        span = st[i] * ex[i];
+    }
+    return true;
+}
+
 bool dims_ok(int N, int H, int L, int E) {
     if (N <= 0 || H <= 0 || L <= 0 || E <= 0) return false;
     return (int64_t)N * H < ((int64_t)1 << 31) && (int64_t)N * H * L * (int64_t)E < ((int64_t)1 << 40);
@@ -85,7 +106,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 12; }
+int srwm_hip_abi_version(void) { return 13; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -267,7 +288,7 @@ int delta_forward_steps_f32(const float *Q, const int64_t qs[3], const float *K,
         return SRWM_ESTRIDE;
     DeltaFwdParams p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
                      {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
-                     N, H, L, E, M, keep};
+                     {(int64_t)H * L * M, (int64_t)L * M, (int64_t)M}, N, H, L, E, M, keep};
     hipStream_t s = (hipStream_t)stream;
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_delta_fwd_tiled(p, s);
@@ -503,20 +524,22 @@ int srwm_backward_bf16(const uint16_t *x, const int64_t xs[3], const float *q, c
 
 int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],
                       const float *V, const int64_t vs[3], const float *beta, const int64_t bs[3],
-                      float *v_old, float *v_insert, float *W, float *out, int N, int H, int L, int E,
-                      int M, unsigned flags, void *stream) {
+                      float *v_old, float *v_insert, float *W, float *out, const int64_t os[3], int N, int H,
+                      int L, int E, int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
         return SRWM_EINVAL;
+    const int64_t dense_out[3] = {(int64_t)H * L * M, (int64_t)L * M, (int64_t)M};
+    if (!os) os = dense_out;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) ||
         (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_SPARSE_V_OLD)) ||
         (flags & (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE)) == (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE) ||
         ((flags & SRWM_FLAG_SPARSE_V_OLD) && !(flags & SRWM_FLAG_CHUNKWISE)))
         return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
-        !stride_ok(bs, N, H, L, 1))
+        !stride_ok(bs, N, H, L, 1) || !out_stride_ok(os, N, H, L, M))
         return SRWM_ESTRIDE;
     DeltaFwdParams p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
-                     {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
+                     {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out, {os[0], os[1], os[2]},
                      N, H, L, E, M, nullptr, (flags & SRWM_FLAG_SPARSE_V_OLD) ? 1u : 0u};
     hipStream_t s = (hipStream_t)stream;
     if (flags & SRWM_FLAG_CHUNKWISE) {
@@ -566,19 +589,21 @@ int delta_backward_f32(const float *Q, const int64_t qs[3], const float *K, cons
 
 int delta_forward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K, const int64_t ks[3],
                        const uint16_t *V, const int64_t vs[3], const uint16_t *beta, const int64_t bs[3],
-                       float *v_old, float *v_insert, float *W, uint16_t *out, int N, int H, int L,
-                       int E, int M, unsigned flags, void *stream) {
+                       float *v_old, float *v_insert, float *W, uint16_t *out, const int64_t os[3], int N,
+                       int H, int L, int E, int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
         return SRWM_EINVAL;
+    const int64_t dense_out[3] = {(int64_t)H * L * M, (int64_t)L * M, (int64_t)M};
+    if (!os) os = dense_out;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) ||
         (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_SPARSE_V_OLD)) ||
         ((flags & SRWM_FLAG_SPARSE_V_OLD) && !(flags & SRWM_FLAG_CHUNKWISE)))
         return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
-        !stride_ok(bs, N, H, L, 1))
+        !stride_ok(bs, N, H, L, 1) || !out_stride_ok(os, N, H, L, M))
         return SRWM_ESTRIDE;
     DeltaFwdParamsBf16 p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
-                         {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
+                         {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out, {os[0], os[1], os[2]},
                          N, H, L, E, M, (flags & SRWM_FLAG_EXACT_PRODUCTS) ? 1u : 0u, (flags & SRWM_FLAG_SPARSE_V_OLD) ? 1u : 0u};
     const int r = (flags & SRWM_FLAG_CHUNKWISE) ? launch_delta_fwd_chunk_bf16(p, (hipStream_t)stream)
                                                 : launch_delta_fwd_tiled_bf16(p, (hipStream_t)stream);

@@ -92,6 +92,7 @@ struct DeltaFwdParams {
     const float *Q, *K, *V, *beta;
     Strided3 qs, ks, vs, bs;
     float *vold, *vins, *W, *out;
+    Strided3 os;         // of out; v_old and v_insert are dense
     int N, H, L, E, M;
     const float *keep;   // optional dense [N,L]: the memory is zeroed before step t where keep[n][t] == 0
     unsigned sparse_vold;   // chunkwise kernel: v_old is written only for steps with |beta| < 2^-24
@@ -113,6 +114,7 @@ struct DeltaFwdParamsBf16 {
     Strided3 qs, ks, vs, bs;
     float *vold, *vins, *W;
     uint16_t *out;
+    Strided3 os;
     int N, H, L, E, M;
     unsigned exact_products;   // chunkwise kernels: every product from hi + lo operand pairs
     unsigned sparse_vold;      // chunkwise kernel: v_old is written only for steps with |beta| < 2^-24

@@ -45,6 +45,7 @@ struct ChunkFwdP {
     Strided3 qs, ks, vs, bs;
     float *vold, *vins, *W;
     TI *out;
+    Strided3 os;   // of out
     int N, H, L;
     bool exact;   // bf16 inputs: also the products that only feed `out` from hi + lo operand pairs
     bool sparse_vold;   // v_old goes out only for steps with |beta| < kTinyBeta (all the chunkwise backward reads of it)
@@ -112,10 +113,10 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
     const TI *vb = p.V + n * p.vs.n + h * p.vs.h + m0;
     const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
     float *Wg = p.W + seq * D * D + m0 + cw;
-    // outputs of this sequence; L * D * 4 bytes fit 32 bits (the launcher checks), so rows are reached with
-    // 32-bit byte offsets from these uniform bases
+    // saved vectors of this sequence; L * D * 4 bytes fit 32 bits (the launcher checks), so rows are reached with
+    // 32-bit byte offsets from these uniform bases.  `out` has strides of its own.
     float *vold_seq = p.vold + seq * p.L * D, *vins_seq = p.vins + seq * p.L * D;
-    TI *out_seq = p.out + seq * p.L * D;
+    TI *out_seq = p.out + n * p.os.n + h * p.os.h + m0 + cw + ln;
 
     // this wave's 16 columns of the memory, accumulator layout per 16-row block
     f32x4 s[EB];
@@ -284,13 +285,14 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
                     typedef decltype(base) P;
                     return reinterpret_cast<P>(reinterpret_cast<char *>(base) + byte_off);
                 };
+                TI *orow = out_seq + (int64_t)(t0 + a * 16 + 4 * lq) * p.os.l;
                 if (t0 + kC <= p.L) {   // a full chunk: no row is past the end
 #pragma unroll
                     for (int r = 0; r < 4; ++r) {
                         if (vo && (!p.sparse_vold || fabsf(bts[a * 16 + 4 * lq + r]) < kTinyBeta))
                             *at(vold_seq, o0 + r * D * 4) = pt[a][r] + y[r];
                         *at(vins_seq, o0 + r * D * 4) = u[a][r];
-                        st_out(at(out_seq, (o0 + r * D * 4) / 4 * (uint32_t)sizeof(TI)), ot[a][r]);
+                        st_out(orow + r * p.os.l, ot[a][r]);
                     }
                 } else {
 #pragma unroll
@@ -299,7 +301,7 @@ __global__ __launch_bounds__(kThreads *KS) void delta_fwd_chunk_kernel(ChunkFwdP
                             if (vo && (!p.sparse_vold || fabsf(bts[a * 16 + 4 * lq + r]) < kTinyBeta))
                                 *at(vold_seq, o0 + r * D * 4) = pt[a][r] + y[r];
                             *at(vins_seq, o0 + r * D * 4) = u[a][r];
-                            st_out(at(out_seq, (o0 + r * D * 4) / 4 * (uint32_t)sizeof(TI)), ot[a][r]);
+                            st_out(orow + r * p.os.l, ot[a][r]);
                         }
                     }
                 }
@@ -361,14 +363,14 @@ int dispatch_chunk(const ChunkFwdP<TI> &p, int D, hipStream_t s) {
 
 int launch_delta_fwd_chunk(const DeltaFwdParams &p, hipStream_t s) {
     if (p.E != p.M) return -1;
-    const ChunkFwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out,
+    const ChunkFwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.os,
                              p.N, p.H, p.L, true, p.sparse_vold != 0u};
     return dispatch_chunk(q, p.E, s);
 }
 
 int launch_delta_fwd_chunk_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s) {
     if (p.E != p.M) return -1;
-    const ChunkFwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out,
+    const ChunkFwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.os,
                               p.N, p.H, p.L, p.exact_products != 0u, p.sparse_vold != 0u};
     return dispatch_chunk(q, p.E, s);
 }

@@ -35,6 +35,7 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_generic_kernel(DeltaFwdPar
         const float *vt = p.V + n * p.vs.n + h * p.vs.h + t * p.vs.l;
         const float b = p.beta[n * p.bs.n + h * p.bs.h + t * p.bs.l];
         const int64_t om = (seq * p.L + t) * M;
+        float *ot = p.out + n * p.os.n + h * p.os.h + t * p.os.l;
         __syncthreads();  // previous step's readers of ks/qs are done (and W is loaded)
         if (p.keep && p.keep[(int64_t)n * p.L + t] == 0.f) {   // uniform: the memory restarts from zero
             for (int i = tid; i < E * Mp; i += kThreads) W[i] = 0.f;
@@ -56,7 +57,7 @@ __global__ __launch_bounds__(kThreads) void delta_fwd_generic_kernel(DeltaFwdPar
             }
             p.vold[om + m] = vo;
             p.vins[om + m] = ins;
-            p.out[om + m] = o;
+            ot[m] = o;
         }
     }
     __syncthreads();

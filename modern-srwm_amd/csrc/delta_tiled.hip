@@ -148,6 +148,7 @@ struct FwdP {
     Strided3 qs, ks, vs, bs;
     float *vold, *vins, *W;
     TI *out;
+    Strided3 os;
     int N, H, L;
     const float *keep;   // optional [N,L]: zero the memory before step t where keep[n][t] == 0
 };
@@ -302,7 +303,8 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
         const int64_t om = (seq * p.L + tile * TT) * D + m0;
         flush_rows<NT, MC>(&ot[buf][OVO][0][0], p.vold + om, D, tlen, tid);
         flush_rows<NT, MC>(&ot[buf][OVI][0][0], p.vins + om, D, tlen, tid);
-        flush_rows<NT, MC>(&ot[buf][OOUT][0][0], p.out + om, D, tlen, tid);
+        flush_rows<NT, MC>(&ot[buf][OOUT][0][0], p.out + n * p.os.n + h * p.os.h + (int64_t)(tile * TT) * p.os.l + m0,
+                           p.os.l, tlen, tid);
     }
 
 #pragma unroll
@@ -557,7 +559,7 @@ constexpr int kSplitBelowSequences = 192;
 template <class TI>
 int dispatch_fwd(const FwdP<TI> &p, int D, hipStream_t s) {
     if (!row_ok(p.Q, p.qs) || !row_ok(p.K, p.ks) || !row_ok(p.V, p.vs) || !ok16(p.vold) || !ok16(p.vins) ||
-        !ok16(p.out) || !ok16(p.W))
+        !row_ok(p.out, p.os) || !ok16(p.W))
         return -1;
     const bool split = p.N * p.H <= kSplitBelowSequences;
     switch (D) {
@@ -591,7 +593,7 @@ int dispatch_bwd(const BwdP<TI> &p, int D, hipStream_t s) {
 
 int launch_delta_fwd_tiled(const DeltaFwdParams &p, hipStream_t s) {
     if (p.E != p.M) return -1;
-    const FwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.N, p.H, p.L,
+    const FwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.os, p.N, p.H, p.L,
                         p.keep};
     return dispatch_fwd(q, p.E, s);
 }
@@ -605,7 +607,7 @@ int launch_delta_bwd_tiled(const DeltaBwdParams &p, hipStream_t s) {
 
 int launch_delta_fwd_tiled_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s) {
     if (p.E != p.M) return -1;
-    const FwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.N, p.H, p.L,
+    const FwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.os, p.N, p.H, p.L,
                          nullptr};
     return dispatch_fwd(q, p.E, s);
 }

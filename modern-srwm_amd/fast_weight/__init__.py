@@ -76,7 +76,9 @@ class DeltaFastWeight(torch.autograd.Function):
         device = Q.device
         N, H, L, E = Q.shape
         _, _, _, M = V.shape
-        out = torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
+        # in the memory layout of V (as elementwise tensor operations do): the layers hand in step-major views,
+        # and with a step-major `out` their transpose / reshape / transpose on the way to the output map is a view
+        out = torch.empty_like(V)
         V_old = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
         V_insert = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
         ctx.forward_flags = DeltaFastWeight.dot[device.type](Q.data, K.data, V.data, beta.data, V_old, V_insert, W, out)

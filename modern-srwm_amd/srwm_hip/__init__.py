@@ -38,7 +38,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _lib = None
 
@@ -66,9 +66,9 @@ _SIGNATURES = {
     "delta_forward_steps_f32": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_readout_replay_f32": [_F, _S] + [_F, _F] + [_F, _S] + [_F, _F] + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_steps_backward_f32": [_F, _S] * 4 + [_F] * 3 + [_F, _S] + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
-    "delta_forward_f32": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_forward_f32": [_F, _S] * 4 + [_F] * 4 + [_S] + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_backward_f32": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
-    "delta_forward_bf16": [_F, _S] * 4 + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_forward_bf16": [_F, _S] * 4 + [_F] * 4 + [_S] + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_backward_bf16": [_F, _S] * 4 + [_F, _F] + [_F, _S] + [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_layer_prologue_f32": [_F] * 6 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_layer_prologue_grad_f32": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -574,7 +574,8 @@ self_ref_backward_v1 = self_ref_backward
 
 def fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=0):
     """Delta-rule forward.  kv ([N,H,E,M], fp32) is overwritten with the final memory.
-    q, k, v, beta and out are all float32 or all bfloat16; v_old, v_insert and kv are float32."""
+    q, k, v, beta and out are all float32 or all bfloat16; v_old, v_insert and kv are float32.
+    out may have any strides with a contiguous last axis (a permuted buffer is written in place)."""
     io = q.dtype if isinstance(q, torch.Tensor) and q.dtype == torch.bfloat16 else torch.float32
     _require(q, "q", None, io)
     N, H, L, E = q.shape
@@ -597,9 +598,12 @@ def fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=0):
         return
     fn = lib().delta_forward_bf16 if io == torch.bfloat16 else lib().delta_forward_f32
     (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr) = (_strided(t) for t in (q, k, v, beta))
-    with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv, out], True) as d:
+    by_strides = out.stride(-1) == 1 or M == 1
+    with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv], True) as d, _Dense([] if by_strides else [out], True) as o:
+        ot = out if by_strides else o[0]
         code = fn(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
-                  *[_ptr(t) for t in d], N, H, L, E, M, flags, _stream(q.device))
+                  *[_ptr(t) for t in d], _ptr(ot), (ctypes.c_int64 * 3)(*ot.stride()[:3]), N, H, L, E, M, flags,
+                  _stream(q.device))
     _check(code, fn.__name__)
 
 

@@ -135,13 +135,18 @@ def test_argument_validation_needs_no_gpu():
     srwm_b = lambda flags: L.srwm_backward_f32(fake(), ok_strides, *[fake() for _ in range(7)], fake(), ok_strides,
                                                *[fake() for _ in range(9)], N, H, Ls, E, flags, P(None))
     assert srwm_b(3) == -1                                     # grad-state mode 3 does not exist
-    delta_f = lambda flags, m: L.delta_forward_f32(*[a for _ in range(4) for a in (fake(), ok_strides)],
-                                                   *[fake() for _ in range(4)], N, H, Ls, E, m, flags, P(None))
+    delta_f = lambda flags, m, os=None: L.delta_forward_f32(*[a for _ in range(4) for a in (fake(), ok_strides)],
+                                                            *[fake() for _ in range(4)], os, N, H, Ls, E, m, flags, P(None))
     assert delta_f(16 | 32, E) == -1                           # generic and chunkwise exclude each other
     assert delta_f(0, 0) == -1                                 # value width 0
     assert delta_f(32, E) == -4                                # SRWM_ENOKERNEL: no chunkwise kernel for E = M = 16
     assert delta_f(4096, E) == -1                              # v_old for the tiny betas only: a mode of the chunkwise kernels
     assert delta_f(32 | 4096, E) == -4                         # accepted with them
+    i3 = lambda *v: (ctypes.c_int64 * 3)(*v)
+    assert delta_f(32, E, i3(H * E, E, N * H * E)) == -4       # out as a [L,N,H,M] buffer: accepted
+    assert delta_f(32, E, i3(H * E, E // 2, N * H * E)) == -3  # SRWM_ESTRIDE: rows of out overlap
+    assert delta_f(32, E, i3(0, E, N * H * E)) == -3           # batch rows on top of each other
+    assert delta_f(32, E, i3(H * E, E, -N * H * E)) == -3      # an output is not written backwards
     delta_b = lambda gW, flags: L.delta_backward_f32(*[a for _ in range(4) for a in (fake(), ok_strides)],
                                                      fake(), fake(), fake(), ok_strides, fake(), fake(), fake(), fake(),
                                                      fake(), gW, N, H, Ls, E, E, flags, P(None))

@@ -641,3 +641,73 @@ def test_stepwise_operator_matches_the_per_step_reference(shape, resets, strided
     assert rel_err(W.cpu().numpy(), ref_W.numpy()) < TOL
     for a, b, nm in zip(grads(), ref_leaves, ("grad_Q", "grad_K", "grad_V", "grad_beta")):
         assert rel_err(a.cpu().numpy(), b.grad.numpy()) < TOL, nm
+
+
+@pytest.mark.parametrize("shape,flags,bf16", [
+    ((2, 3, 20, 16, 16), 0, False),       # register-tiled kernel
+    ((2, 3, 20, 16, 16), 16, False),      # generic kernel
+    ((2, 2, 9, 24, 40), 0, False),        # E != M: generic kernel
+    ((2, 2, 130, 64, 64), 32, False),     # chunkwise, fp32, ragged last chunk
+    ((1, 3, 70, 128, 128), 32, True),     # chunkwise, bf16, two workgroups per sequence
+    ((2, 2, 33, 32, 32), 0, True),        # register-tiled kernel, bf16
+])
+def test_forward_writes_out_through_strides(shape, flags, bf16):
+    """`out` may be a permuted or padded buffer: the same kernels write it in place, bit for bit what they write
+    into a dense one, and touch nothing between its rows.  A last axis that is not contiguous is staged through a
+    dense copy by the Python layer."""
+    print(f"case strided out shape={shape} flags={flags} bf16={bf16}", flush=True)
+    import srwm_hip
+    N, H, L, E, M = shape
+    dt = torch.bfloat16 if bf16 else torch.float32
+    q, k, v, beta, W0, _ = delta_inputs(*shape, seed=3, qk="softmax", w0_std=0.1)
+    qd, kd, vd, bd = (t.to(_dev(), torch.float32).to(dt) for t in (q, k, v, beta))
+
+    def run(out):
+        W = W0.to(_dev(), torch.float32).contiguous()
+        vold, vins = (torch.empty(N, H, L, M, device=_dev()) for _ in range(2))
+        srwm_hip.fast_weight_forward(qd, kd, vd, bd, vold, vins, W, out, flags=flags)
+        torch.cuda.synchronize()
+        return vins, W
+
+    dense = torch.full((N, H, L, M), float("nan"), device=_dev(), dtype=dt)
+    ref_vins, ref_W = run(dense)
+    assert torch.isfinite(dense.float()).all()
+    mark = 7.0
+    step_major = torch.full((L, N, H, M), mark, device=_dev(), dtype=dt)
+    padded = torch.full((N, H, L, M + 4), mark, device=_dev(), dtype=dt)
+    every_other = torch.full((N, H, L, 2 * M), mark, device=_dev(), dtype=dt)
+    for name, buf, view in (("step-major", step_major, step_major.permute(1, 2, 0, 3)), ("padded rows", padded, padded[..., :M]),
+                            ("every other element", every_other, every_other[..., ::2])):
+        vins, W = run(view)
+        assert torch.equal(view, dense), name
+        assert torch.equal(vins, ref_vins) and torch.equal(W, ref_W), name
+    assert (padded[..., M:] == mark).all() and (every_other[..., 1::2] == mark).all()
+
+
+def test_operator_output_takes_the_layout_of_v():
+    """The autograd operator allocates `out` like V: from step-major views (what the layers hand in) the layers'
+    transpose / reshape / transpose chain on the result is a view of a contiguous [L, N, H*M] tensor, and the
+    values and gradients are those of the batch-major call."""
+    print("case operator output layout", flush=True)
+    from fast_weight import fast_weight_delta
+    N, H, L, D = 2, 3, 70, 64
+    q, k, v, beta, W0, go = delta_inputs(N, H, L, D, D, seed=5, qk="softmax", w0_std=0.0)
+    res = {}
+    for layout in ("batch-major", "step-major"):
+        args = []
+        for t in (q, k, v, beta):
+            t = t.to(_dev(), torch.float32)
+            if layout == "step-major":
+                t = t.permute(2, 0, 1, 3).contiguous().permute(1, 2, 0, 3)
+            args.append(t.requires_grad_(True))
+        W = W0.to(_dev(), torch.float32).contiguous()
+        out = fast_weight_delta(*args, W)
+        chain = out.transpose(1, 2).reshape(N, L, H * D).transpose(0, 1)
+        if layout == "step-major":
+            assert chain.is_contiguous() and chain.data_ptr() == out.data_ptr()
+        else:
+            assert out.is_contiguous()
+        (chain * go.to(_dev()).transpose(1, 2).reshape(N, L, H * D).transpose(0, 1)).sum().backward()
+        res[layout] = [out.detach()] + [a.grad for a in args]
+    for a, b in zip(res["batch-major"], res["step-major"]):
+        assert torch.equal(a, b)
