@@ -141,13 +141,18 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
-def _strided(t):
-    """A tensor the kernels can read through (n, h, l) strides: last axis contiguous, rows
-    16-byte aligned.  Anything else is copied."""
+def _rows_ok(t):
+    """Can the kernels address this tensor through (n, h, l) strides: last axis contiguous, rows
+    aligned to four elements."""
     ok = t.stride(-1) == 1 or t.shape[-1] == 1
     if ok and t.shape[-1] % 4 == 0:
         ok = t.data_ptr() % (4 * t.element_size()) == 0 and all(s % 4 == 0 for s in t.stride()[:3])
-    if not ok:
+    return ok
+
+
+def _strided(t):
+    """A tensor the kernels can read through (n, h, l) strides.  Anything else is copied."""
+    if not _rows_ok(t):
         t = t.contiguous()
     return t, (ctypes.c_int64 * 3)(*t.stride()[:3])
 
@@ -598,7 +603,7 @@ def fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=0):
         return
     fn = lib().delta_forward_bf16 if io == torch.bfloat16 else lib().delta_forward_f32
     (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr) = (_strided(t) for t in (q, k, v, beta))
-    by_strides = out.stride(-1) == 1 or M == 1
+    by_strides = _rows_ok(out)
     with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv], True) as d, _Dense([] if by_strides else [out], True) as o:
         ot = out if by_strides else o[0]
         code = fn(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,

@@ -675,13 +675,14 @@ def test_forward_writes_out_through_strides(shape, flags, bf16):
     mark = 7.0
     step_major = torch.full((L, N, H, M), mark, device=_dev(), dtype=dt)
     padded = torch.full((N, H, L, M + 4), mark, device=_dev(), dtype=dt)
+    odd = torch.full((N, H, L, M + 1), mark, device=_dev(), dtype=dt)   # rows off the alignment the kernels store with
     every_other = torch.full((N, H, L, 2 * M), mark, device=_dev(), dtype=dt)
-    for name, buf, view in (("step-major", step_major, step_major.permute(1, 2, 0, 3)), ("padded rows", padded, padded[..., :M]),
-                            ("every other element", every_other, every_other[..., ::2])):
+    for name, view in (("step-major", step_major.permute(1, 2, 0, 3)), ("padded rows", padded[..., :M]),
+                       ("rows at odd offsets", odd[..., 1:]), ("every other element", every_other[..., ::2])):
         vins, W = run(view)
         assert torch.equal(view, dense), name
         assert torch.equal(vins, ref_vins) and torch.equal(W, ref_W), name
-    assert (padded[..., M:] == mark).all() and (every_other[..., 1::2] == mark).all()
+    assert (padded[..., M:] == mark).all() and (odd[..., 0] == mark).all() and (every_other[..., 1::2] == mark).all()
 
 
 def test_operator_output_takes_the_layout_of_v():
