@@ -388,8 +388,8 @@ SRWM_API int delta_backward_f32(const float *Q, const int64_t q_strides[3],
  * (reinforcement_learning/torchbeast_procgen/model.py:1176-1196, torchbeast/layer.py:128-189),
  * where the memory receives no gradient (fast_weight/__init__.py:95-100 returns None for it).
  *
- * delta_forward_steps_f32: as delta_forward_f32, the memory zeroed before step t of batch row n
- * where keep[n][t] == 0 (keep: dense [N,L] or NULL).
+ * delta_forward_steps_f32: as delta_forward_f32 (out_strides included), the memory zeroed before step t
+ * of batch row n where keep[n][t] == 0 (keep: dense [N,L] or NULL).
  *
  * delta_readout_replay_f32: u[n][h][t] = W_{t-1} grad_out[n][h][t] (dense [N,H,L,E]) with W
  * replayed from W_entry (the memory handed to delta_forward_steps_f32, before that call) through
@@ -402,7 +402,7 @@ SRWM_API int delta_forward_steps_f32(const float *Q, const int64_t q_strides[3],
                             const float *V, const int64_t v_strides[3],
                             const float *beta, const int64_t beta_strides[3],
                             const float *keep,
-                            float *v_old, float *v_insert, float *W, float *out,
+                            float *v_old, float *v_insert, float *W, float *out, const int64_t out_strides[3],
                             int N, int H, int L, int E, int M, unsigned flags, void *stream);
 
 SRWM_API int delta_readout_replay_f32(const float *K, const int64_t k_strides[3],

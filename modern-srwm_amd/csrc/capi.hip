@@ -278,17 +278,19 @@ int srwm_readout_grad_f32(const float *k, const float *beta, const float *ydiff,
 
 int delta_forward_steps_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],
                             const float *V, const int64_t vs[3], const float *beta, const int64_t bs[3],
-                            const float *keep, float *v_old, float *v_insert, float *W, float *out, int N,
-                            int H, int L, int E, int M, unsigned flags, void *stream) {
+                            const float *keep, float *v_old, float *v_insert, float *W, float *out,
+                            const int64_t os[3], int N, int H, int L, int E, int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
         return SRWM_EINVAL;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    const int64_t dense_out[3] = {(int64_t)H * L * M, (int64_t)L * M, (int64_t)M};
+    if (!os) os = dense_out;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
-        !stride_ok(bs, N, H, L, 1))
+        !stride_ok(bs, N, H, L, 1) || !out_stride_ok(os, N, H, L, M))
         return SRWM_ESTRIDE;
     DeltaFwdParams p{Q, K, V, beta, {qs[0], qs[1], qs[2]}, {ks[0], ks[1], ks[2]},
                      {vs[0], vs[1], vs[2]}, {bs[0], bs[1], bs[2]}, v_old, v_insert, W, out,
-                     {(int64_t)H * L * M, (int64_t)L * M, (int64_t)M}, N, H, L, E, M, keep};
+                     {os[0], os[1], os[2]}, N, H, L, E, M, keep};
     hipStream_t s = (hipStream_t)stream;
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_delta_fwd_tiled(p, s);

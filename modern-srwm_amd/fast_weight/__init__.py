@@ -155,7 +155,7 @@ class DeltaFastWeightSteps(torch.autograd.Function):
         N, H, L, E = Q.shape
         M = V.shape[-1]
         new = lambda: torch.empty((N, H, L, M), device=Q.device, dtype=Q.dtype)
-        out, V_old, V_insert = new(), new(), new()
+        out, V_old, V_insert = torch.empty_like(V), new(), new()   # out in the memory layout of V, as fast_weight_delta
         W_entry = W.detach().clone()
         srwm_hip.fast_weight_forward_steps(Q.data, K.data, V.data, beta.data, keep, V_old, V_insert, W.data, out)
         ctx.save_for_backward(Q, K, V, beta, keep, V_old, V_insert, W_entry)

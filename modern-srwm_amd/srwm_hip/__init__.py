@@ -63,7 +63,7 @@ _SIGNATURES = {
     "srwm_layer_readout_grad_f32": [_F, _S] + [_F] * 5 + [_F, _S] + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
-    "delta_forward_steps_f32": [_F, _S] * 4 + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "delta_forward_steps_f32": [_F, _S] * 4 + [_F] * 5 + [_S] + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_readout_replay_f32": [_F, _S] + [_F, _F] + [_F, _S] + [_F, _F] + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_steps_backward_f32": [_F, _S] * 4 + [_F] * 3 + [_F, _S] + [_F] * 5 + [_I] * 5 + [_U, ctypes.c_void_p],
     "delta_forward_f32": [_F, _S] * 4 + [_F] * 4 + [_S] + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -632,10 +632,13 @@ def fast_weight_forward_steps(q, k, v, beta, keep, v_old, v_insert, kv, out, fla
     if q.numel() == 0 or v.numel() == 0:
         return
     (qs, qstr), (ks, kstr), (vs, vstr), (bs, bstr) = (_strided(t) for t in (q, k, v, beta))
-    with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv, out], True) as d:
+    by_strides = _rows_ok(out)
+    with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv], True) as d, _Dense([] if by_strides else [out], True) as o:
+        ot = out if by_strides else o[0]
         code = lib().delta_forward_steps_f32(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
                                              _ptr(keep) if keep is not None else null,
-                                             *[_ptr(t) for t in d], N, H, L, E, M, flags, _stream(q.device))
+                                             *[_ptr(t) for t in d], _ptr(ot), (ctypes.c_int64 * 3)(*ot.stride()[:3]),
+                                             N, H, L, E, M, flags, _stream(q.device))
     _check(code, "delta_forward_steps_f32")
 
 

@@ -685,14 +685,16 @@ def test_forward_writes_out_through_strides(shape, flags, bf16):
     assert (padded[..., M:] == mark).all() and (odd[..., 0] == mark).all() and (every_other[..., 1::2] == mark).all()
 
 
-def test_operator_output_takes_the_layout_of_v():
-    """The autograd operator allocates `out` like V: from step-major views (what the layers hand in) the layers'
+@pytest.mark.parametrize("steps", [False, True], ids=["fast_weight_delta", "fast_weight_delta_steps"])
+def test_operator_output_takes_the_layout_of_v(steps):
+    """The autograd operators allocate `out` like V: from step-major views (what the layers hand in) the layers'
     transpose / reshape / transpose chain on the result is a view of a contiguous [L, N, H*M] tensor, and the
     values and gradients are those of the batch-major call."""
-    print("case operator output layout", flush=True)
-    from fast_weight import fast_weight_delta
+    print(f"case operator output layout steps={steps}", flush=True)
+    from fast_weight import fast_weight_delta, fast_weight_delta_steps
     N, H, L, D = 2, 3, 70, 64
     q, k, v, beta, W0, go = delta_inputs(N, H, L, D, D, seed=5, qk="softmax", w0_std=0.0)
+    keep = (torch.rand(N, L, generator=torch.Generator().manual_seed(1)) > 0.1).float().to(_dev())
     res = {}
     for layout in ("batch-major", "step-major"):
         args = []
@@ -702,7 +704,7 @@ def test_operator_output_takes_the_layout_of_v():
                 t = t.permute(2, 0, 1, 3).contiguous().permute(1, 2, 0, 3)
             args.append(t.requires_grad_(True))
         W = W0.to(_dev(), torch.float32).contiguous()
-        out = fast_weight_delta(*args, W)
+        out = fast_weight_delta_steps(*args, keep, W) if steps else fast_weight_delta(*args, W)
         chain = out.transpose(1, 2).reshape(N, L, H * D).transpose(0, 1)
         if layout == "step-major":
             assert chain.is_contiguous() and chain.data_ptr() == out.data_ptr()
