@@ -25,6 +25,11 @@ CHUNKWISE_BACKWARD = "auto"
 # bfloat16 anyway); True forms them from hi + lo operand pairs as well (~8 % slower).  The memory,
 # v_old, v_insert, grad_V and grad_beta do not depend on this.  No effect with float32 inputs.
 EXACT_PRODUCTS = False
+# Memory layout of `out`: True allocates it like V (what elementwise tensor operations do with their operand), so that
+# the step-major views the layers hand in give a step-major `out` and their transpose / reshape / transpose on the way
+# to the output map (supervised_learning/layer.py:98-100) is a view; False always allocates a contiguous (N, H, L, M)
+# tensor as the reference does (for callers that go on with .view()).  The values are the same.
+OUT_LIKE_V = True
 
 
 def _chunk_flags(choice, E, M, L):
@@ -76,9 +81,7 @@ class DeltaFastWeight(torch.autograd.Function):
         device = Q.device
         N, H, L, E = Q.shape
         _, _, _, M = V.shape
-        # in the memory layout of V (as elementwise tensor operations do): the layers hand in step-major views,
-        # and with a step-major `out` their transpose / reshape / transpose on the way to the output map is a view
-        out = torch.empty_like(V)
+        out = torch.empty_like(V) if OUT_LIKE_V else torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
         V_old = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
         V_insert = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
         ctx.forward_flags = DeltaFastWeight.dot[device.type](Q.data, K.data, V.data, beta.data, V_old, V_insert, W, out)
@@ -155,7 +158,7 @@ class DeltaFastWeightSteps(torch.autograd.Function):
         N, H, L, E = Q.shape
         M = V.shape[-1]
         new = lambda: torch.empty((N, H, L, M), device=Q.device, dtype=Q.dtype)
-        out, V_old, V_insert = torch.empty_like(V), new(), new()   # out in the memory layout of V, as fast_weight_delta
+        out, V_old, V_insert = torch.empty_like(V) if OUT_LIKE_V else new(), new(), new()   # as fast_weight_delta
         W_entry = W.detach().clone()
         srwm_hip.fast_weight_forward_steps(Q.data, K.data, V.data, beta.data, keep, V_old, V_insert, W.data, out)
         ctx.save_for_backward(Q, K, V, beta, keep, V_old, V_insert, W_entry)

@@ -714,3 +714,11 @@ def test_operator_output_takes_the_layout_of_v(steps):
         res[layout] = [out.detach()] + [a.grad for a in args]
     for a, b in zip(res["batch-major"], res["step-major"]):
         assert torch.equal(a, b)
+    import fast_weight
+    fast_weight.OUT_LIKE_V = False        # the reference's allocation: dense whatever V looks like
+    try:
+        W = W0.to(_dev(), torch.float32).contiguous()
+        out = fast_weight_delta_steps(*args, keep, W) if steps else fast_weight_delta(*args, W)
+        assert out.is_contiguous() and torch.equal(out, res["batch-major"][0])
+    finally:
+        fast_weight.OUT_LIKE_V = True
