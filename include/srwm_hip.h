@@ -216,13 +216,20 @@ SRWM_API int srwm_forward_steps_f32(const float *x, const int64_t x_strides[3], 
  *                                 shared weights receive through the initial state (second launch, fixed
  *                                 summation order)
  *   grad_x      with SRWM_FLAG_SOFTMAX_INPUT the gradient of the un-soft-maxed input
+ *   out_strides, grad_x_strides   element strides (N, H, L; rows contiguous) of out [N,H,L,Y] and grad_x
+ *                                 [N,H,L,E], or NULL = dense.  The layers hand x in as a view of their
+ *                                 [L, N, H*E] input and reshape out back to that form
+ *                                 (supervised_learning/layer.py:161-165, :184-186): with the strides of a
+ *                                 [L,N,H,.] buffer, (H*w, w, N*H*w), neither direction needs a copy.  Rows that
+ *                                 share memory are refused (SRWM_ESTRIDE).
  */
 SRWM_API int srwm_layer_forward_f32(const float *x, const int64_t x_strides[3], const float *keep,
                            const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
                            float *W_y, float *W_q, float *W_k, float *w_b,
                            float *q, float *k, float *beta,
                            float *y_diff, float *q_diff, float *k_diff, float *beta_diff,
-                           float *out, int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+                           float *out, const int64_t out_strides[3],
+                           int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
 SRWM_API int srwm_layer_backward_f32(const float *x, const int64_t x_strides[3],
                             const float *q, const float *k, const float *beta,
@@ -231,7 +238,8 @@ SRWM_API int srwm_layer_backward_f32(const float *x, const int64_t x_strides[3],
                             const float *grad_out, const int64_t grad_out_strides[3],
                             const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
                             const float *W_y, const float *W_q, const float *W_k, const float *w_b,
-                            float *grad_x, float *gW_y, float *gW_q, float *gW_k, float *gw_b,
+                            float *grad_x, const int64_t grad_x_strides[3],
+                            float *gW_y, float *gW_q, float *gW_k, float *gw_b,
                             float *gsW_y, float *gsW_q, float *gsW_k, float *gsw_b,
                             int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
@@ -264,7 +272,7 @@ SRWM_API int srwm_layer_backward_noalloc_f32(const float *x, const int64_t x_str
                             const float *grad_out, const int64_t grad_out_strides[3],
                             const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
                             const float *W_y, const float *W_q, const float *W_k, const float *w_b,
-                            float *grad_x,
+                            float *grad_x, const int64_t grad_x_strides[3],
                             float *gsW_y, float *gsW_q, float *gsW_k, float *gsw_b,
                             int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
@@ -284,7 +292,8 @@ SRWM_API int srwm_layer_forward_bf16(const uint16_t *x, const int64_t x_strides[
                             float *W_y, float *W_q, float *W_k, float *w_b,
                             float *q, float *k, float *beta,
                             float *y_diff, float *q_diff, float *k_diff, float *beta_diff,
-                            uint16_t *out, int N, int H, int L, int E, int Y, unsigned flags, void *stream);
+                            uint16_t *out, const int64_t out_strides[3],
+                            int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
 SRWM_API int srwm_layer_backward_bf16(const uint16_t *x, const int64_t x_strides[3],
                              const float *q, const float *k, const float *beta,
@@ -293,7 +302,8 @@ SRWM_API int srwm_layer_backward_bf16(const uint16_t *x, const int64_t x_strides
                              const uint16_t *grad_out, const int64_t grad_out_strides[3],
                              const float *sW_y, const float *sW_q, const float *sW_k, const float *sw_b,
                              const float *W_y, const float *W_q, const float *W_k, const float *w_b,
-                             float *grad_x, float *gW_y, float *gW_q, float *gW_k, float *gw_b,
+                             float *grad_x, const int64_t grad_x_strides[3],
+                             float *gW_y, float *gW_q, float *gW_k, float *gw_b,
                              float *gsW_y, float *gsW_q, float *gsW_k, float *gsw_b,
                              int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
@@ -514,7 +524,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 13. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 14. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

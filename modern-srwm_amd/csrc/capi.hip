@@ -106,7 +106,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 13; }
+int srwm_hip_abi_version(void) { return 14; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -167,8 +167,8 @@ int srwm_forward_f32(const float *x, const int64_t xs[3], float *Wy, float *Wq, 
 static int layer_forward(bool io16, const float *x, const int64_t xs[3], const float *keep, const float *sWy,
                          const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
                          float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
-                         float *qdiff, float *kdiff, float *bdiff, float *out, int N, int H, int L,
-                         int E, int Y, unsigned flags, void *stream) {
+                         float *qdiff, float *kdiff, float *bdiff, float *out, const int64_t os[3], int N, int H,
+                         int L, int E, int Y, unsigned flags, void *stream) {
     if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
         !out || !xs)
         return SRWM_EINVAL;
@@ -176,11 +176,12 @@ static int layer_forward(bool io16, const float *x, const int64_t xs[3], const f
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || (flags & ~known)) return SRWM_EINVAL;
     const bool needs_shared = keep || (flags & (SRWM_FLAG_STATE_SHIFT | SRWM_FLAG_FRESH_STATE));
     if (needs_shared && (!sWy || !sWq || !sWk || !swb)) return SRWM_EINVAL;
-    if (!stride_ok(xs, N, H, L, E)) return SRWM_ESTRIDE;
+    if (!stride_ok(xs, N, H, L, E) || (os && !out_stride_ok(os, N, H, L, Y))) return SRWM_ESTRIDE;
     SrwmFwdParams p{x, xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff,
                     out, N, H, L, E, keep, sWy, sWq, sWk, swb, Y};
     p.mode = ((flags & SRWM_FLAG_STATE_SHIFT) ? kModeShift : 0u) | ((flags & SRWM_FLAG_FRESH_STATE) ? kModeFresh : 0u) |
              ((flags & SRWM_FLAG_SOFTMAX_INPUT) ? kModeSoftmaxX : 0u) | (io16 ? kModeBf16 : 0u);
+    if (os) p.os_n = os[0], p.os_h = os[1], p.os_l = os[2];
     hipStream_t s = (hipStream_t)stream;
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_fwd_tiled(p, s);
@@ -193,19 +194,19 @@ static int layer_forward(bool io16, const float *x, const int64_t xs[3], const f
 int srwm_layer_forward_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
                            const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
                            float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
-                           float *qdiff, float *kdiff, float *bdiff, float *out, int N, int H, int L,
-                           int E, int Y, unsigned flags, void *stream) {
+                           float *qdiff, float *kdiff, float *bdiff, float *out, const int64_t os[3], int N,
+                           int H, int L, int E, int Y, unsigned flags, void *stream) {
     return layer_forward(false, x, xs, keep, sWy, sWq, sWk, swb, Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff,
-                         bdiff, out, N, H, L, E, Y, flags, stream);
+                         bdiff, out, os, N, H, L, E, Y, flags, stream);
 }
 
 int srwm_layer_forward_bf16(const uint16_t *x, const int64_t xs[3], const float *keep, const float *sWy,
                             const float *sWq, const float *sWk, const float *swb, float *Wy, float *Wq,
                             float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
-                            float *qdiff, float *kdiff, float *bdiff, uint16_t *out, int N, int H, int L,
-                            int E, int Y, unsigned flags, void *stream) {
+                            float *qdiff, float *kdiff, float *bdiff, uint16_t *out, const int64_t os[3], int N,
+                            int H, int L, int E, int Y, unsigned flags, void *stream) {
     return layer_forward(true, reinterpret_cast<const float *>(x), xs, keep, sWy, sWq, sWk, swb, Wy, Wq, Wk, wb, q,
-                         k, beta, ydiff, qdiff, kdiff, bdiff, reinterpret_cast<float *>(out), N, H, L, E, Y, flags,
+                         k, beta, ydiff, qdiff, kdiff, bdiff, reinterpret_cast<float *>(out), os, N, H, L, E, Y, flags,
                          stream);
 }
 
@@ -215,7 +216,7 @@ int srwm_forward_bf16(const uint16_t *x, const int64_t xs[3], float *Wy, float *
                       void *stream) {
     if (flags & ~(SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
     return srwm_layer_forward_bf16(x, xs, nullptr, nullptr, nullptr, nullptr, nullptr, Wy, Wq, Wk, wb, q, k, beta,
-                                   ydiff, qdiff, kdiff, bdiff, out, N, H, L, E, E, flags, stream);
+                                   ydiff, qdiff, kdiff, bdiff, out, nullptr, N, H, L, E, E, flags, stream);
 }
 
 int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *keep, const float *sWy,
@@ -225,7 +226,7 @@ int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *kee
                            int E, unsigned flags, void *stream) {
     if (flags & ~(SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
     return srwm_layer_forward_f32(x, xs, keep, sWy, sWq, sWk, swb, Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff,
-                                  kdiff, bdiff, out, N, H, L, E, E, flags, stream);
+                                  kdiff, bdiff, out, nullptr, N, H, L, E, E, flags, stream);
 }
 
 int srwm_readout_grad_wide_f32(const float *k, const float *beta, const float *ydiff, const float *keep,
@@ -430,8 +431,8 @@ static int layer_backward(bool io16, const float *x, const int64_t xs[3], const 
                           const float *bdiff, const float *grad_out, const int64_t gs[3],
                           const float *sWy, const float *sWq, const float *sWk, const float *swb,
                           const float *Wy, const float *Wq, const float *Wk, const float *wb,
-                          float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, float *gsWy,
-                          float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
+                          float *grad_x, const int64_t gxs[3], float *gWy, float *gWq, float *gWk, float *gwb,
+                          float *gsWy, float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
                           unsigned flags, void *stream) {
     if (!x || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff || !grad_out || !Wy || !Wq ||
         !Wk || !wb || !grad_x || !gWy || !gWq || !gWk || !gwb || !xs || !gs)
@@ -442,12 +443,14 @@ static int layer_backward(bool io16, const float *x, const int64_t xs[3], const 
     if ((flags & SRWM_FLAG_STATE_SHIFT) && (!sWy || !sWq || !sWk || !swb)) return SRWM_EINVAL;
     const bool sums = gsWy || gsWq || gsWk || gswb;
     if (sums && (!gsWy || !gsWq || !gsWk || !gswb)) return SRWM_EINVAL;
-    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, Y)) return SRWM_ESTRIDE;
+    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, Y) || (gxs && !out_stride_ok(gxs, N, H, L, E)))
+        return SRWM_ESTRIDE;
     SrwmBwdParams p{x, xs[0], xs[1], xs[2], q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out,
                     gs[0], gs[1], gs[2], Wy, Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, N, H, L, E, mode, Y,
                     sWy, sWq, sWk, swb};
     p.mode = ((flags & SRWM_FLAG_STATE_SHIFT) ? kModeShift : 0u) | ((flags & SRWM_FLAG_SOFTMAX_INPUT) ? kModeSoftmaxX : 0u) |
              (io16 ? kModeBf16 : 0u);
+    if (gxs) p.gxs_n = gxs[0], p.gxs_h = gxs[1], p.gxs_l = gxs[2];
     hipStream_t s = (hipStream_t)stream;
     int r = -1;
     if (!(flags & SRWM_FLAG_GENERIC)) r = launch_srwm_bwd_tiled(p, s);
@@ -466,11 +469,11 @@ int srwm_layer_backward_f32(const float *x, const int64_t xs[3], const float *q,
                             const float *bdiff, const float *grad_out, const int64_t gs[3],
                             const float *sWy, const float *sWq, const float *sWk, const float *swb,
                             const float *Wy, const float *Wq, const float *Wk, const float *wb,
-                            float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, float *gsWy,
-                            float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
+                            float *grad_x, const int64_t gxs[3], float *gWy, float *gWq, float *gWk, float *gwb,
+                            float *gsWy, float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
                             unsigned flags, void *stream) {
     return layer_backward(false, x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, sWy, sWq, sWk, swb, Wy,
-                          Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags,
+                          Wq, Wk, wb, grad_x, gxs, gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags,
                           stream);
 }
 
@@ -479,8 +482,9 @@ int srwm_layer_backward_noalloc_f32(const float *x, const int64_t xs[3], const f
                                     const float *kdiff, const float *bdiff, const float *grad_out,
                                     const int64_t gs[3], const float *sWy, const float *sWq, const float *sWk,
                                     const float *swb, const float *Wy, const float *Wq, const float *Wk,
-                                    const float *wb, float *grad_x, float *gsWy, float *gsWq, float *gsWk,
-                                    float *gswb, int N, int H, int L, int E, int Y, unsigned flags, void *stream) {
+                                    const float *wb, float *grad_x, const int64_t gxs[3], float *gsWy, float *gsWq,
+                                    float *gsWk, float *gswb, int N, int H, int L, int E, int Y, unsigned flags,
+                                    void *stream) {
     if (!gsWy || !gsWq || !gsWk || !gswb) return SRWM_EINVAL;
     // the per-row gradients start from nothing: there is no buffer an incoming state gradient could arrive in
     if (flags & SRWM_GRAD_STATE_MASK) return SRWM_EINVAL;
@@ -495,7 +499,7 @@ int srwm_layer_backward_noalloc_f32(const float *x, const int64_t xs[3], const f
     // SRWM_GRAD_STATE_ZERO: the backward kernel overwrites every per-row gradient it owns and the batch
     // sum reads exactly those, so nothing in the array has to be cleared between calls
     return layer_backward(false, x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, sWy, sWq, sWk, swb, Wy,
-                          Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags,
+                          Wq, Wk, wb, grad_x, gxs, gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags,
                           stream);
 }
 
@@ -504,12 +508,12 @@ int srwm_layer_backward_bf16(const uint16_t *x, const int64_t xs[3], const float
                              const float *bdiff, const uint16_t *grad_out, const int64_t gs[3],
                              const float *sWy, const float *sWq, const float *sWk, const float *swb,
                              const float *Wy, const float *Wq, const float *Wk, const float *wb,
-                             float *grad_x, float *gWy, float *gWq, float *gWk, float *gwb, float *gsWy,
-                             float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
+                             float *grad_x, const int64_t gxs[3], float *gWy, float *gWq, float *gWk, float *gwb,
+                             float *gsWy, float *gsWq, float *gsWk, float *gswb, int N, int H, int L, int E, int Y,
                              unsigned flags, void *stream) {
     return layer_backward(true, reinterpret_cast<const float *>(x), xs, q, k, beta, ydiff, qdiff, kdiff, bdiff,
                           reinterpret_cast<const float *>(grad_out), gs, sWy, sWq, sWk, swb, Wy, Wq, Wk, wb, grad_x,
-                          gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags, stream);
+                          gxs, gWy, gWq, gWk, gwb, gsWy, gsWq, gsWk, gswb, N, H, L, E, Y, flags, stream);
 }
 
 int srwm_backward_bf16(const uint16_t *x, const int64_t xs[3], const float *q, const float *k,
@@ -520,8 +524,8 @@ int srwm_backward_bf16(const uint16_t *x, const int64_t xs[3], const float *q, c
                        void *stream) {
     if (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)) return SRWM_EINVAL;
     return srwm_layer_backward_bf16(x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, nullptr, nullptr,
-                                    nullptr, nullptr, Wy, Wq, Wk, wb, grad_x, gWy, gWq, gWk, gwb, nullptr, nullptr,
-                                    nullptr, nullptr, N, H, L, E, E, flags, stream);
+                                    nullptr, nullptr, Wy, Wq, Wk, wb, grad_x, nullptr, gWy, gWq, gWk, gwb, nullptr,
+                                    nullptr, nullptr, nullptr, N, H, L, E, E, flags, stream);
 }
 
 int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const int64_t ks[3],

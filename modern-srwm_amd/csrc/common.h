@@ -30,6 +30,7 @@ struct SrwmFwdParams {
     const float *sWy, *sWq, *sWk, *swb;   // [H,E,Y], [H,E,E] x 2, [H,E,4]
     int Y;   // columns of W_y, out and ydiff (E for the plain operator)
     unsigned mode;   // kMode* bits
+    int64_t os_n = 0, os_h = 0, os_l = 0;   // element strides of out; all zero: dense [N,H,L,Y] (see with_out_strides)
 };
 
 struct SrwmBwdParams {
@@ -45,7 +46,18 @@ struct SrwmBwdParams {
     int Y;   // columns of W_y, grad_out, ydiff and gWy (E for the plain operator)
     const float *sWy, *sWq, *sWk, *swb;   // shared weights, read when mode has kModeShift
     unsigned mode;   // kMode* bits
+    int64_t gxs_n = 0, gxs_h = 0, gxs_l = 0;   // element strides of gx; all zero: dense [N,H,L,E]
 };
+
+// the parameter blocks with the strides of a dense output filled in where the caller left them zero
+inline SrwmFwdParams with_out_strides(SrwmFwdParams p) {
+    if (!p.os_n && !p.os_h && !p.os_l) p.os_n = (int64_t)p.H * p.L * p.Y, p.os_h = (int64_t)p.L * p.Y, p.os_l = p.Y;
+    return p;
+}
+inline SrwmBwdParams with_out_strides(SrwmBwdParams p) {
+    if (!p.gxs_n && !p.gxs_h && !p.gxs_l) p.gxs_n = (int64_t)p.H * p.L * p.E, p.gxs_h = (int64_t)p.L * p.E, p.gxs_l = p.E;
+    return p;
+}
 
 struct Strided3 {
     int64_t n, h, l;

@@ -90,6 +90,7 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
         const float *xt = p.x + n * p.xs_n + h * p.xs_h + t * p.xs_l;
         const uint16_t *xt16 = reinterpret_cast<const uint16_t *>(p.x) + n * p.xs_n + h * p.xs_h + t * p.xs_l;
         const int64_t o = (seq * p.L + t) * E, oy = (seq * p.L + t) * Y, ob = (seq * p.L + t) * 4;
+        const int64_t oo = (seq / p.H) * p.os_n + (seq % p.H) * p.os_h + t * p.os_l;   // of out
         if (p.keep && p.keep[(int64_t)n * p.L + t] == 0.f) {   // uniform: per-step reset to the shared weights
             load_state(W, Cp, shWy, shWq, shWk, shwb, E, Y, tid);
         }
@@ -105,8 +106,8 @@ __global__ __launch_bounds__(kThreads) void srwm_fwd_generic_kernel(SrwmFwdParam
             for (int e = 0; e < E; ++e) a = fmaf(W[e * Cp + m], xs[e], a);
             pre[m] = a;
             if (m < Y) {
-                if (bf16_io) reinterpret_cast<uint16_t *>(p.out)[oy + m] = f32_to_bf16_bits(a);
-                else p.out[oy + m] = a;
+                if (bf16_io) reinterpret_cast<uint16_t *>(p.out)[oo + m] = f32_to_bf16_bits(a);
+                else p.out[oo + m] = a;
             }
         }
         __syncthreads();
@@ -204,6 +205,7 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
         const uint16_t *xt16 = reinterpret_cast<const uint16_t *>(p.x) + n * p.xs_n + h * p.xs_h + t * p.xs_l;
         const uint16_t *got16 = reinterpret_cast<const uint16_t *>(p.go) + n * p.gs_n + h * p.gs_h + t * p.gs_l;
         const int64_t o = (seq * p.L + t) * E, oy = (seq * p.L + t) * Y, ob = (seq * p.L + t) * 4;
+        const int64_t ogx = (seq / p.H) * p.gxs_n + (seq % p.H) * p.gxs_h + t * p.gxs_l;   // of grad_x
         for (int e = tid; e < E; e += kThreads) {
             xs[e] = bf16_io ? bf16_bits_to_f32(xt16[e]) : xt[e];
             qs[e] = p.q[o + e];
@@ -280,7 +282,7 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
             a = wave_sum(a);
             if (lane == 0) {
                 if (smx) gq[e] = a;
-                else p.gx[o + e] = a;
+                else p.gx[ogx + e] = a;
             }
         }
         if (smx) {
@@ -289,7 +291,7 @@ __global__ __launch_bounds__(kThreads) void srwm_bwd_generic_kernel(SrwmBwdParam
                 float d = 0.f;
                 for (int i = lane; i < E; i += kWave) d = fmaf(gq[i], xs[i], d);
                 d = wave_sum(d);
-                for (int i = lane; i < E; i += kWave) p.gx[o + i] = xs[i] * (gq[i] - d);
+                for (int i = lane; i < E; i += kWave) p.gx[ogx + i] = xs[i] * (gq[i] - d);
             }
         }
         // column pass: G += (q - k) (x) g_diff + x (x) g_pre
@@ -334,14 +336,14 @@ size_t srwm_bwd_generic_lds_bytes(int E, int Y) {
 int launch_srwm_fwd_generic(const SrwmFwdParams &p, hipStream_t s) {
     const size_t lds = srwm_fwd_generic_lds_bytes(p.E, p.Y);
     if (const int err = allow_max_dynamic_lds<srwm_fwd_generic_kernel>()) return err;
-    hipLaunchKernelGGL(srwm_fwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
+    hipLaunchKernelGGL(srwm_fwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, with_out_strides(p));
     return (int)hipGetLastError();
 }
 
 int launch_srwm_bwd_generic(const SrwmBwdParams &p, hipStream_t s) {
     const size_t lds = srwm_bwd_generic_lds_bytes(p.E, p.Y);
     if (const int err = allow_max_dynamic_lds<srwm_bwd_generic_kernel>()) return err;
-    hipLaunchKernelGGL(srwm_bwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
+    hipLaunchKernelGGL(srwm_bwd_generic_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, with_out_strides(p));
     return (int)hipGetLastError();
 }
 

@@ -236,9 +236,12 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     auto load_keep = [&](int tile) -> float {
         return (RESET && p.keep && tid < TT) ? p.keep[(int64_t)n * p.L + min(tile * TT + tid, p.L - 1)] : 1.f;
     };
-    // outputs of this sequence: uniform bases, 32-bit offsets per step
-    float *const out_s = p.out + seq * p.L * Y, *const ydiff_s = p.ydiff + seq * p.L * Y;
-    uint16_t *const out16_s = reinterpret_cast<uint16_t *>(p.out) + seq * p.L * Y;
+    // outputs of this sequence: uniform bases, 32-bit offsets per step.  `out` has strides of its own in the
+    // forms with the layer extras (the plain operator's is dense).
+    const int64_t out_0 = MODES ? n * p.os_n + h * p.os_h : seq * p.L * Y;
+    const unsigned out_l = MODES ? (unsigned)p.os_l : (unsigned)Y;
+    float *const out_s = p.out + out_0, *const ydiff_s = p.ydiff + seq * p.L * Y;
+    uint16_t *const out16_s = reinterpret_cast<uint16_t *>(p.out) + out_0;
     float *const q_s = p.q + seq * p.L * E, *const k_s = p.k + seq * p.L * E;
     float *const qdiff_s = p.qdiff + seq * p.L * E, *const kdiff_s = p.kdiff + seq * p.L * E;
     float *const beta_s = p.beta + seq * p.L * 4, *const bdiff_s = p.bdiff + seq * p.L * 4;
@@ -292,7 +295,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     };
     // hands the readout of step t to the output and, through LDS, to the activations of that step
     auto publish = [&](auto PARP, int t, const float (&acc)[NC], float pb, float py) __attribute__((always_inline)) {
-        const unsigned oy = t * Y;           // offsets inside the sequence (the launcher bounds L * Y)
+        const unsigned oy = t * out_l;       // offset inside the sequence (the launcher bounds it)
         const int par = parity_of(PARP);   // parity of step t
         // the RG lanes of a column group hold identical values: all of them store, to the same words,
         // which is cheaper than masking seven of them off (no branch around the stores)
@@ -756,6 +759,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     // grad_x of step t: the row sums W_{t-1} g_pre of all waves and of the narrow columns (buffers of
     // parity pp), through the softmax of the input where the kernel applies it (xs = this thread's
     // element of the softmaxed x_t)
+    float *const gx_s = p.gx + n * p.gxs_n + h * p.gxs_h;
     auto finish_gx = [&](int t, int pp, float xs) {
         // below E = 64 by the first E lanes of the LAST wave: the first waves also carry the narrow columns
         // there (at E = 64 every wave carries one of them)
@@ -763,7 +767,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
         if ((unsigned)e < (unsigned)E) {
             float s = row_total(pp, 2, e);
             if (softmax_x) s = xs * (s - group_sum<E>(s * xs));   // the E threads are whole lane groups
-            p.gx[(seq * p.L + t) * E + e] = s;
+            gx_s[(int64_t)t * p.gxs_l + e] = s;
         }
     };
     float xb_prev = 0.f;
@@ -1087,18 +1091,20 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 
 template <int E, int NW, int R, int YB = 1>
 int launch_bwd(const SrwmBwdParams &p, hipStream_t s) {
-    hipLaunchKernelGGL((srwm_bwd_tiled_kernel<E, NW, R, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, p);
+    hipLaunchKernelGGL((srwm_bwd_tiled_kernel<E, NW, R, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, with_out_strides(p));
     return (int)hipGetLastError();
 }
 
 template <int E, int NW, int R, int YB = 1>
-int launch_fwd(const SrwmFwdParams &p, hipStream_t s) {
-    const dim3 grid(p.N * p.H), block(NW * kWave);
+int launch_fwd(const SrwmFwdParams &p0, hipStream_t s) {
+    const dim3 grid(p0.N * p0.H), block(NW * kWave);
+    const bool strided_out = p0.os_n || p0.os_h || p0.os_l;   // the plain operator's kernel writes a dense out
+    const SrwmFwdParams p = with_out_strides(p0);
     if (p.mode & kModeBf16)
         hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, YB, true>), grid, block, 0, s, p);
     else if (p.keep)
         hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, YB, false>), grid, block, 0, s, p);
-    else if (p.mode)
+    else if (p.mode || strided_out)
         hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 1, YB, false>), grid, block, 0, s, p);
     else
         hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 0, YB, false>), grid, block, 0, s, p);
@@ -1113,6 +1119,8 @@ bool aligned16(const void *ptr, int64_t a, int64_t b, int64_t c) {
 
 int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
     if ((int64_t)p.L * (p.Y > p.E ? p.Y : p.E) >= ((int64_t)1 << 29)) return -1;   // 32-bit offsets inside a sequence
+    if ((int64_t)p.L * p.os_l >= ((int64_t)1 << 29) || p.os_l < 0) return -1;
+    if (!(p.mode & kModeBf16) && (p.os_n % 4 || p.os_h % 4 || p.os_l % 4)) return -1;   // vector stores to fp32 rows of out
     if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l)) return -1;
     const void *dense[] = {p.q, p.k, p.beta, p.ydiff, p.qdiff, p.kdiff, p.bdiff, p.out};
     for (const void *d : dense)

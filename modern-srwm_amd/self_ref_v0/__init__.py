@@ -247,6 +247,16 @@ def _write_only_buffers(dev, shapes):
     return bufs
 
 
+def _rows_like(x, width, dtype):
+    """An (N, H, L, width) tensor whose rows lie in memory in the order of x's: the layers hand x in as a view of
+    their (L, N, H*E) input, and with `out` and `grad_x` in that order too the reshapes on either side of the
+    operator (supervised_learning/layer.py:161-165, :184-186) are views instead of copies."""
+    N, H, L, _ = x.shape
+    if L > 1 and x.stride(-1) == 1 and x.stride(2) > x.stride(0) > x.stride(1) > 0:   # step-major
+        return torch.empty((L, N, H, width), device=x.device, dtype=dtype).permute(1, 2, 0, 3)
+    return torch.empty((N, H, L, width), device=x.device, dtype=dtype)
+
+
 class SelfRefLayerFn(torch.autograd.Function):
     """The SRWM operator as the layers call it, with `state + W.repeat(bsz, 1, 1, 1)`, the softmax
     of the input, the final `- W.repeat(...)` and the batch sum of the weight gradients done inside
@@ -273,6 +283,9 @@ class SelfRefLayerFn(torch.autograd.Function):
         N, H, L, E = x.shape
         Y = sW_y.shape[-1]
         dev = x.device
+        # outputs the loss does not depend on (the new shift, for the layers that detach it) reach backward as None
+        # instead of as freshly filled zero tensors
+        ctx.set_materialize_grads(False)
         shifts = (shift_y, shift_q, shift_k, shift_b)
         fresh = shift_y is None
         assert all((s is None) == fresh for s in shifts), "give all four shifts or none"
@@ -282,7 +295,7 @@ class SelfRefLayerFn(torch.autograd.Function):
             state = [torch.empty((N, H, E, w), device=dev, dtype=f32) for w in widths]
         else:
             state = [s.detach().clone(memory_format=torch.contiguous_format) for s in shifts]
-        out = torch.empty((N, H, L, Y), device=dev, dtype=x.dtype)
+        out = _rows_like(x, Y, x.dtype)
         needs_grad = bool(track)
         shapes = tuple((N, H, L, w) for w in (E, E, 4, Y, E, E, 4))   # q, k, beta, y_diff, q_diff, k_diff, beta_diff
         if needs_grad:
@@ -308,6 +321,8 @@ class SelfRefLayerFn(torch.autograd.Function):
         Y = slow[0].shape[-1]
         g_state = (g_y, g_q, g_k, g_b)
         has_gs = any(g is not None for g in g_state)
+        if grad_out is None:   # the loss depends on the returned shift only
+            grad_out = torch.zeros((N, H, L, Y), device=x.device, dtype=x.dtype)
         if has_gs:   # the loss also depends on the returned shift: private contiguous copies, zeros where unused
             grad_W = [torch.zeros_like(s) if g is None else g.clone(memory_format=torch.contiguous_format)
                       for g, s in zip(g_state, state)]
@@ -320,7 +335,7 @@ class SelfRefLayerFn(torch.autograd.Function):
             if need_slow else None
         # d(shift_out)/d(shared) = dW_L/d(shared) - 1: the incoming state gradient is taken off again
         minus = [g.sum(0) for g in grad_W] if (has_gs and need_slow) else None
-        grad_x = torch.empty(x.shape, device=x.device, dtype=torch.float32)
+        grad_x = _rows_like(x, E, torch.float32)
         flags = mode | srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_SOFTMAX_INPUT if ctx.softmax_input else 0)
         srwm_hip.self_ref_layer_backward(x, *saved, grad_out.to(x.dtype), slow, *state, grad_x, grad_W, grad_slow,
                                          flags=flags)

@@ -38,7 +38,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 _lib = None
 
@@ -53,11 +53,11 @@ _SIGNATURES = {
     "srwm_backward_bf16": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_forward_wide_f32": [_F, _S] + [_F] * 12 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_backward_wide_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 5 + [_U, ctypes.c_void_p],
-    "srwm_layer_forward_f32": [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
-    "srwm_layer_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
-    "srwm_layer_backward_noalloc_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 13 + [_I] * 5 + [_U, ctypes.c_void_p],
-    "srwm_layer_forward_bf16": [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
-    "srwm_layer_backward_bf16": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 17 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_forward_f32": [_F, _S] + [_F] * 17 + [_S] + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_S] + [_F] * 8 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_backward_noalloc_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_S] + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_forward_bf16": [_F, _S] + [_F] * 17 + [_S] + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_backward_bf16": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_S] + [_F] * 8 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_wide_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_layer_readout_grad_f32": [_F, _S] + [_F] * 5 + [_F, _S] + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -227,7 +227,7 @@ def self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, 
         elif io == torch.bfloat16:   # wide output block: the layer entry point without any of its extras
             name = "srwm_layer_forward_bf16"
             code = lib().srwm_layer_forward_bf16(_ptr(xs), xstr, null, null, null, null, null,
-                                                 *[_ptr(t) for t in d], N, H, L, E, Y, flags, _stream(x.device))
+                                                 *[_ptr(t) for t in d], None, N, H, L, E, Y, flags, _stream(x.device))
         elif Y == E:
             name = "srwm_forward_f32"
             code = lib().srwm_forward_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
@@ -402,7 +402,7 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
             name = "srwm_layer_backward_bf16"
             code = lib().srwm_layer_backward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
                                                   null, null, null, null, *[_ptr(t) for t in st],
-                                                  *[_ptr(t) for t in gr], null, null, null, null,
+                                                  _ptr(gr[0]), None, *[_ptr(t) for t in gr[1:]], null, null, null, null,
                                                   N, H, L, E, Y, flags, _stream(x.device))
         elif Y == E:
             name = "srwm_backward_f32"
@@ -466,12 +466,16 @@ def self_ref_layer_forward(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff
                     w.copy_(sw.unsqueeze(0).expand_as(w))
         return
     xs, xstr = _strided(x)
+    by_strides = _rows_ok(out)   # a permuted buffer is written in place
     with torch.cuda.device(x.device), \
-            _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out], True) as d:
+            _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff], True) as d, \
+            _Dense([] if by_strides else [out], True) as o:
+        ot = out if by_strides else o[0]
         name = "srwm_layer_forward_bf16" if io == torch.bfloat16 else "srwm_layer_forward_f32"
         code = getattr(lib(), name)(
             _ptr(xs), xstr, _ptr(keep) if keep is not None else null, *[_ptr(t) for t in sl],
-            *[_ptr(t) for t in d], N, H, L, E, Y, flags, _stream(x.device))
+            *[_ptr(t) for t in d], _ptr(ot), (ctypes.c_int64 * 3)(*ot.stride()[:3]), N, H, L, E, Y, flags,
+            _stream(x.device))
     _check(code, name)
 
 
@@ -519,11 +523,13 @@ def self_ref_layer_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, gr
     gos, gstr = _strided(grad_out)
     with torch.cuda.device(x.device), \
             _Dense([q, k, beta, y_diff, q_diff, k_diff, beta_diff], False) as sv, \
-            _Dense([W_y, W_q, W_k, w_b], False) as st, _Dense([grad_x], True) as gx:
+            _Dense([W_y, W_q, W_k, w_b], False) as st, \
+            _Dense([] if grad_x.stride(-1) == 1 else [grad_x], True) as gx:
+        gxt = gx[0] if gx else grad_x   # any row strides: the kernels store grad_x element by element
         name = "srwm_layer_backward_bf16" if io == torch.bfloat16 else "srwm_layer_backward_f32"
         code = getattr(lib(), name)(
             _ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr, *[_ptr(t) for t in sl],
-            *[_ptr(t) for t in st], _ptr(gx[0]), *[_ptr(g) for g in grad_W], *gsl,
+            *[_ptr(t) for t in st], _ptr(gxt), (ctypes.c_int64 * 3)(*gxt.stride()[:3]), *[_ptr(g) for g in grad_W], *gsl,
             N, H, L, E, Y, flags, _stream(x.device))
     _check(code, name)
 
@@ -566,7 +572,7 @@ def self_ref_layer_backward_noalloc(x, q, k, beta, y_diff, q_diff, k_diff, beta_
     with torch.cuda.device(x.device):
         code = lib().srwm_layer_backward_noalloc_f32(
             _ptr(x), xstr, *[_ptr(t) for t in (q, k, beta, y_diff, q_diff, k_diff, beta_diff)], _ptr(grad_out), gstr,
-            *[_ptr(t) for t in sl], *[_ptr(t) for t in (W_y, W_q, W_k, w_b)], _ptr(grad_x),
+            *[_ptr(t) for t in sl], *[_ptr(t) for t in (W_y, W_q, W_k, w_b)], _ptr(grad_x), None,
             *[_ptr(g) for g in grad_slow], N, H, L, E, Y, flags, _stream(x.device))
     _check(code, "srwm_layer_backward_noalloc_f32")
 

@@ -159,12 +159,19 @@ def test_argument_validation_needs_no_gpu():
     assert delta_bb(P(None), 32 | 512 | 1024, E) == -1         # with single products,
     assert delta_bb(fake(), 32 | 1024, E) == -1                # and without the gradient of the memory
     assert delta_bb(P(None), 32 | 1024, E) == -4               # accepted; SRWM_ENOKERNEL: E = M = 16 has no chunkwise kernel
-    layer_f = lambda sw, flags: L.srwm_layer_forward_f32(fake(), ok_strides, P(None), sw, sw, sw, sw,
-                                                         *[fake() for _ in range(12)], N, H, Ls, E, E, flags, P(None))
+    layer_f = lambda sw, flags, os=None: L.srwm_layer_forward_f32(fake(), ok_strides, P(None), sw, sw, sw, sw,
+                                                                  *[fake() for _ in range(12)], os, N, H, Ls, E, E, flags,
+                                                                  P(None))
     assert layer_f(P(None), 64) == -1                          # the shift form needs the shared weights
     assert layer_f(P(None), 128) == -1                         # so does a fresh start
+    assert layer_f(fake(), 128, (ctypes.c_int64 * 3)(H * E, E // 2, N * H * E)) == -3   # SRWM_ESTRIDE: rows of out overlap
+    layer_b = lambda gxs: L.srwm_layer_backward_f32(
+        fake(), ok_strides, *[fake() for _ in range(7)], fake(), ok_strides, *[fake() for _ in range(9)], gxs,
+        *[fake() for _ in range(8)], N, H, Ls, E, E, 3, P(None))
+    assert layer_b(None) == -1                                 # grad-state mode 3 does not exist (dense grad_x accepted)
+    assert layer_b((ctypes.c_int64 * 3)(0, E, N * H * E)) == -1   # the flags are checked before the strides
     noalloc = lambda n, flags, gs: L.srwm_layer_backward_noalloc_f32(
-        fake(), ok_strides, *[fake() for _ in range(7)], fake(), ok_strides, *[fake() for _ in range(9)],
+        fake(), ok_strides, *[fake() for _ in range(7)], fake(), ok_strides, *[fake() for _ in range(9)], None,
         gs, gs, gs, gs, n, H, Ls, E, E, flags, P(None))
     assert noalloc(N, 0, P(None)) == -1                        # the batch sums are what it is for
     assert noalloc(N, 1, fake()) == -1                         # no buffer for an incoming state gradient

@@ -560,3 +560,38 @@ def test_rl_self_modifying_layer_whole_unroll_equals_the_per_step_loop():
             ref = loop_grads[n]
             got = p.grad if p.grad is not None else torch.zeros_like(ref)
             assert (got - ref).abs().max().item() < 2e-5 * max(1e-6, ref.abs().max().item()), n
+
+
+@pytest.mark.parametrize("E,wide,bf16", [(16, False, False), (64, False, False), (32, True, False), (32, False, True),
+                                         (24, False, False)])   # E = 24: the LDS-resident kernels
+def test_layer_operator_keeps_the_row_order_of_its_input(E, wide, bf16):
+    """self_ref_layer allocates `out` and the gradient of x with their rows in the memory order of x's: handed the
+    layers' view of a (L, N, H*E) input, the reshape of `out` back to (L, N, H*Y) is a view of a contiguous tensor
+    and so is the gradient that reaches the input; the values are those of a batch-major call, bit for bit."""
+    print(f"case layer operator row order E={E} wide={wide} bf16={bf16}", flush=True)
+    from self_ref_v0 import self_ref_layer
+    torch.manual_seed(E)
+    N, H, L = 3, 2, 9
+    Y = 3 * E + 1 if wide else E
+    dt = torch.bfloat16 if bf16 else torch.float32
+    slow = [(0.1 * torch.randn(1, H, E, w, device=_dev())).requires_grad_(True) for w in (Y, E, E, 4)]
+    h0 = torch.randn(L, N, H * E, device=_dev()).to(dt)
+    go = torch.randn(N, H, L, Y, device=_dev()).to(dt)
+    res = {}
+    for layout in ("step-major", "batch-major"):
+        h = h0.clone().requires_grad_(True)
+        x = h.reshape(L, N, H, E).permute(1, 2, 0, 3)
+        if layout == "batch-major":
+            x = x.contiguous()
+        out, *shift = self_ref_layer(x, *slow, None, None, None, None, True)
+        if layout == "step-major":
+            chain = out.transpose(1, 2).reshape(N, L, H * Y).transpose(0, 1)
+            assert chain.is_contiguous() and chain.data_ptr() == out.data_ptr()
+        else:
+            assert out.is_contiguous()
+        (out.float() * go.float()).sum().backward()
+        res[layout] = [out.detach(), h.grad.clone()] + [w.grad.clone() for w in slow] + [s.detach() for s in shift]
+        for w in slow:
+            w.grad = None
+    for a, b in zip(res["step-major"], res["batch-major"]):
+        assert torch.equal(a, b)
