@@ -191,7 +191,7 @@ class SelfRefLayerStepsFn(torch.autograd.Function):
         dev = x.device
         f32 = torch.float32
         state = [s.detach().clone(memory_format=torch.contiguous_format) for s in (shift_y, shift_q, shift_k, shift_b)]
-        out = torch.empty((N, H, L, Y), device=dev, dtype=f32)
+        out = _rows_like(x, Y, f32)
         saved = [torch.empty((N, H, L, w), device=dev, dtype=f32) for w in (E, E, 4, Y, E, E, 4)]
         flags = srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_SOFTMAX_INPUT if softmax_input else 0)
         srwm_hip.self_ref_layer_forward(x.detach(), keep, (sW_y, sW_q, sW_k, sw_b), *state, *saved, out, flags=flags)
