@@ -46,6 +46,11 @@ def elu_p1_sum_norm_eps(x):
     return y / (y.sum(-1, keepdim=True) + 1e-5)
 
 
+def _keep_rows(notdone, dtype):
+    """(T, B) notdone -> (B, T) keep flags in `dtype`: conversion and transposition in one copy."""
+    return torch.empty((notdone.shape[1], notdone.shape[0]), device=notdone.device, dtype=dtype).copy_(notdone.t())
+
+
 def _heads_out(out, bsz, slen, width):
     """(B, H, len, d) -> (len, B, H*d)"""
     return out.transpose(1, 2).reshape(bsz, slen, width).transpose(0, 1)
@@ -159,7 +164,7 @@ class SRlayer(_SRBase):
         does, reinforcement_learning/torchbeast_procgen/model.py:1176-1196), in one kernel launch
         forward and one backward.  h: (T, B, H*d); notdone: (T, B), 0 where an episode ended."""
         assert state is not None
-        keep = notdone.to(h.dtype).transpose(0, 1).contiguous()            # (B, T)
+        keep = _keep_rows(notdone, h.dtype)                                # (B, T)
         if FUSED_SRWM_LAYER:
             slen, bsz, _ = h.size()
             x = h.reshape(slen, bsz, self.num_head, self.dim_head).permute(1, 2, 0, 3)
@@ -242,7 +247,7 @@ class SMFWPlayer(nn.Module):
         launch per operator.  h: (T, B, H*d); notdone: (T, B), 0 where an episode ended."""
         assert state is not None
         slen, bsz, _ = h.size()
-        keep = notdone.to(h.dtype).transpose(0, 1).contiguous()            # (B, T)
+        keep = _keep_rows(notdone, h.dtype)                                # (B, T)
         slow = (self.W_y, self.W_q, self.W_k, self.w_b)
         *shift, fast_weights = state
         if FUSED_SRWM_LAYER:
@@ -323,7 +328,7 @@ class CarryFastFFlayer(_DeltaBase):
         reinforcement_learning/torchbeast_procgen/model.py:1176-1196).  x: (T, B, D); notdone: (T, B)."""
         assert state is not None
         q, k, v, beta, slen, bsz = self._qkvb(x, True)
-        keep = notdone.to(x.dtype).transpose(0, 1).contiguous()
+        keep = _keep_rows(notdone, x.dtype)
         fast_weights = state.detach().clone()
         out = fast_weight_delta_steps(q, k, v, beta, keep, fast_weights)
         return self._finish(x, out, bsz, slen), fast_weights

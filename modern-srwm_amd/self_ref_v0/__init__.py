@@ -190,7 +190,10 @@ class SelfRefLayerStepsFn(torch.autograd.Function):
         Y = sW_y.shape[-1]
         dev = x.device
         f32 = torch.float32
-        state = [s.detach().clone(memory_format=torch.contiguous_format) for s in (shift_y, shift_q, shift_k, shift_b)]
+        ctx.set_materialize_grads(False)   # no zero tensors for the gradients of the returned shift, which nobody reads
+        shifts = [s.detach() for s in (shift_y, shift_q, shift_k, shift_b)]
+        state = [torch.empty(s.shape, device=dev, dtype=f32) for s in shifts]
+        torch._foreach_copy_(state, shifts)   # one launch for the four
         out = _rows_like(x, Y, f32)
         saved = [torch.empty((N, H, L, w), device=dev, dtype=f32) for w in (E, E, 4, Y, E, E, 4)]
         flags = srwm_hip.FLAG_STATE_SHIFT | (srwm_hip.FLAG_SOFTMAX_INPUT if softmax_input else 0)
@@ -207,6 +210,8 @@ class SelfRefLayerStepsFn(torch.autograd.Function):
         N, H, L, E = x.shape
         Y = y_diff.shape[-1]
         dev = x.device
+        if grad_out is None:   # the loss does not depend on the output
+            return (None,) * 11
         sx = _softmax_rows(x) if ctx.softmax_input else x
         u = torch.empty((N, H, L, E), device=dev, dtype=torch.float32)
         rows = torch.empty((N, H, E, Y), device=dev, dtype=torch.float32)
