@@ -112,8 +112,11 @@ __device__ __forceinline__ float4 row_softmax4(float4 v) {
 // (p.keep), which adds a check to every step and a register copy of the shared weights.
 // BF16: x and out are bf16 behind the float pointers (a compile-time switch: the output store
 // sits inside the step).
-template <int E, int NW, int R, int XTRA, int YB, bool BF16>
+// SO: `out` is addressed through its strides (p.os_*) instead of as a dense tensor: a compile-time switch, because
+// a second set of row offsets inside the step costs the forms whose steps are shortest about 4 %.
+template <int E, int NW, int R, int XTRA, int YB, bool BF16, bool SO = (XTRA >= 1)>
 __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams p) {
+    static_assert(XTRA >= 1 || !SO, "the plain operator's out is dense");
     constexpr bool MODES = XTRA >= 1;   // p.mode: work outside the step loop only (entry / exit form of the state, input tiles)
     constexpr bool RESET = XTRA >= 2;   // p.keep: a check, and now and then a reset, inside every step
     using T = Tiling<E, NW, R>;
@@ -236,10 +239,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     auto load_keep = [&](int tile) -> float {
         return (RESET && p.keep && tid < TT) ? p.keep[(int64_t)n * p.L + min(tile * TT + tid, p.L - 1)] : 1.f;
     };
-    // outputs of this sequence: uniform bases, 32-bit offsets per step.  `out` has strides of its own in the
-    // forms with the layer extras (the plain operator's is dense).
-    const int64_t out_0 = MODES ? n * p.os_n + h * p.os_h : seq * p.L * Y;
-    const unsigned out_l = MODES ? (unsigned)p.os_l : (unsigned)Y;
+    // outputs of this sequence: uniform bases, 32-bit offsets per step.  `out` has strides of its own where SO.
+    const int64_t out_0 = SO ? n * p.os_n + h * p.os_h : seq * p.L * Y;
+    const unsigned out_l = SO ? (unsigned)p.os_l : (unsigned)Y;
     float *const out_s = p.out + out_0, *const ydiff_s = p.ydiff + seq * p.L * Y;
     uint16_t *const out16_s = reinterpret_cast<uint16_t *>(p.out) + out_0;
     float *const q_s = p.q + seq * p.L * E, *const k_s = p.k + seq * p.L * E;
@@ -294,8 +296,9 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         }
     };
     // hands the readout of step t to the output and, through LDS, to the activations of that step
-    auto publish = [&](auto PARP, int t, const float (&acc)[NC], float pb, float py) __attribute__((always_inline)) {
-        const unsigned oy = t * out_l;       // offset inside the sequence (the launcher bounds it)
+    // (oy: offset of the step's row of `out` inside the sequence, t * out_l, which the launcher bounds; formed by the
+    // caller ahead of time, the stores here are on the step's critical path)
+    auto publish = [&](auto PARP, const unsigned oy, const float (&acc)[NC], float pb, float py) __attribute__((always_inline)) {
         const int par = parity_of(PARP);   // parity of step t
         // the RG lanes of a column group hold identical values: all of them store, to the same words,
         // which is cheaper than masking seven of them off (no branch around the stores)
@@ -343,7 +346,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         float xr[R], acc[NC], pb, py = 0.f;
         lds_read_vec<R>(xr, &xt[0][0][r0]);
         readout(xr, xt[0][0][el], acc, pb, py);
-        publish(P0{}, 0, acc, pb, py);
+        publish(P0{}, 0u, acc, pb, py);
     }
     __syncthreads();
 
@@ -362,6 +365,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         const auto PNEXT = parity_flipped(PAR);
         const int t1 = t + 1;
         const unsigned o = t * E, oy = t * Y, ob = t * 4;   // unsigned: uniform base + 32-bit lane offset addressing
+        const unsigned oo1 = SO ? (unsigned)t1 * out_l : oy + Y;   // row of step t + 1 in `out`
         const int b1 = (t1 / TT) & 1, r1 = t1 % TT;   // where x of step t+1 sits (stale rows past the end: never published)
         const bool have_next = t1 < p.L;
 
@@ -488,7 +492,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
             for (int c = 0; c < NC; ++c) e[c] = fmaf(ins[c], kx, e[c]);
             float py = 0.f;
             if constexpr (XC) py = fmaf(insy, kx, s[4]);
-            if (have_next) publish(PNEXT, t1, e, fmaf(insb, kx, s[2]), py);
+            if (have_next) publish(PNEXT, oo1, e, fmaf(insb, kx, s[2]), py);
             write_state();
         }
         if constexpr (RESET) {
@@ -496,7 +500,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
                 reset_state();
                 float acc[NC], pb, py = 0.f;
                 readout(xr, xb, acc, pb, py);
-                publish(PNEXT, t1, acc, pb, py);
+                publish(PNEXT, oo1, acc, pb, py);
             }
         }
 
@@ -1098,12 +1102,15 @@ int launch_bwd(const SrwmBwdParams &p, hipStream_t s) {
 template <int E, int NW, int R, int YB = 1>
 int launch_fwd(const SrwmFwdParams &p0, hipStream_t s) {
     const dim3 grid(p0.N * p0.H), block(NW * kWave);
-    const bool strided_out = p0.os_n || p0.os_h || p0.os_l;   // the plain operator's kernel writes a dense out
     const SrwmFwdParams p = with_out_strides(p0);
+    // the plain operator's kernel and the dense form of the one with resets write a dense out
+    const bool strided_out = p.os_n != (int64_t)p.H * p.L * p.Y || p.os_h != (int64_t)p.L * p.Y || p.os_l != p.Y;
     if (p.mode & kModeBf16)
         hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, YB, true>), grid, block, 0, s, p);
+    else if (p.keep && strided_out)
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, YB, false, true>), grid, block, 0, s, p);
     else if (p.keep)
-        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, YB, false>), grid, block, 0, s, p);
+        hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, YB, false, false>), grid, block, 0, s, p);
     else if (p.mode || strided_out)
         hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 1, YB, false>), grid, block, 0, s, p);
     else
