@@ -1127,7 +1127,8 @@ bool aligned16(const void *ptr, int64_t a, int64_t b, int64_t c) {
 int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
     if ((int64_t)p.L * (p.Y > p.E ? p.Y : p.E) >= ((int64_t)1 << 29)) return -1;   // 32-bit offsets inside a sequence
     if ((int64_t)p.L * p.os_l >= ((int64_t)1 << 29) || p.os_l < 0) return -1;
-    if (!(p.mode & kModeBf16) && (p.os_n % 4 || p.os_h % 4 || p.os_l % 4)) return -1;   // vector stores to fp32 rows of out
+    // vector stores to fp32 rows of out (the wide output block and bf16 go out element by element)
+    if (p.Y == p.E && !(p.mode & kModeBf16) && (p.os_n % 4 || p.os_h % 4 || p.os_l % 4)) return -1;
     if (!aligned16(p.x, p.xs_n, p.xs_h, p.xs_l)) return -1;
     const void *dense[] = {p.q, p.k, p.beta, p.ydiff, p.qdiff, p.kdiff, p.bdiff, p.out};
     for (const void *d : dense)
