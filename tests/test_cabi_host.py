@@ -198,3 +198,25 @@ def test_argument_validation_needs_no_gpu():
     assert pgrad(huge, 0) == -3                                # SRWM_ESTRIDE
     assert L.srwm_hip_scratch_bytes() == 32 << 20
     assert b"scratch" in L.srwm_hip_strerror(-5)
+
+
+def test_layout_helpers_of_the_host_layer():
+    """The helpers that decide memory layouts, on CPU tensors: output rows follow the row order of a step-major
+    input view (so that the layers' reshape back is a view) and stay dense otherwise; the keep flags of the step
+    mode are the transposed, converted notdone mask."""
+    import layer
+    import self_ref_v0
+    L, N, H, E, Y = 5, 3, 2, 4, 13
+    h = torch.randn(L, N, H * E)
+    x = h.reshape(L, N, H, E).permute(1, 2, 0, 3)                      # what the layers hand to the operator
+    out = self_ref_v0._rows_like(x, Y, torch.float32)
+    assert out.shape == (N, H, L, Y) and out.stride() == (H * Y, Y, N * H * Y, 1)
+    chain = out.transpose(1, 2).reshape(N, L, H * Y).transpose(0, 1)  # supervised_learning/layer.py:184-186
+    assert chain.is_contiguous() and chain.data_ptr() == out.data_ptr()
+    assert self_ref_v0._rows_like(x.contiguous(), Y, torch.float32).is_contiguous()
+    assert self_ref_v0._rows_like(x[:, :, :1], Y, torch.float32).is_contiguous()          # one step: nothing to reorder
+    assert self_ref_v0._rows_like(x[..., ::2], Y, torch.bfloat16).is_contiguous()         # rows not contiguous: dense
+    notdone = torch.rand(L, N) > 0.3
+    keep = layer._keep_rows(notdone, torch.float32)
+    assert keep.shape == (N, L) and keep.is_contiguous() and keep.dtype == torch.float32
+    assert torch.equal(keep, notdone.t().float())
