@@ -21,7 +21,7 @@ matrix-core peak.  `cpu_baseline` is the per-timestep PyTorch recurrence (oracle
 timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (through the autograd operator), delta_prologue_c2, delta_prologue_c5 (the layers' prologue kernels, fp32 and bf16, HBM-bound), delta_layer_c2 (a whole delta-rule layer)}.
+{srwm_c3, srwm_generic_c4 (the LDS-resident kernel family at the headline shape), srwm_e48, delta_e96 (head sizes without a register-resident instantiation of their own), srwm_d16, srwm_rl_d16 (the head size the reference trains with), srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (through the autograd operator), delta_prologue_c2, delta_prologue_c5 (the layers' prologue kernels, fp32 and bf16, HBM-bound), delta_layer_c2 (a whole delta-rule layer)}.
 """
 import argparse
 import json
@@ -64,6 +64,15 @@ WORKLOADS = {
     "srwm_c3_steps": ("srwm_steps", 32, 8, 100, 32),
     # the same shape with the output block 3E+1 = 97 columns wide (the self_ref_v1 operator)
     "srwm_wide_c3": ("srwm_wide", 32, 8, 100, 32),
+    # the headline shape forced onto the LDS-resident kernels (the family that serves any head size the CU's LDS
+    # holds), and two natural sizes that have no register-resident instantiation of their own
+    "srwm_generic_c4": ("srwm", 32, 16, 512, 64),
+    "srwm_e48": ("srwm", 32, 16, 512, 48),
+    "delta_e96": ("delta", 32, 8, 256, 96),
+    # the head size the reference's authors train with (d_head = 16): the few-shot learner's shape
+    # (supervised_learning/README.md:24-40) and the RL learner's unroll (reinforcement_learning/README.md:23-52)
+    "srwm_d16": ("srwm", 64, 16, 150, 16),
+    "srwm_rl_d16": ("srwm", 32, 8, 50, 16),
     "delta_c2": ("delta", 32, 8, 256, 64),
     "delta_c5f32": ("delta", 8, 16, 4096, 128),
     "delta_c5": ("delta_bf16", 8, 16, 4096, 128),     # bf16 q/k/v/beta/out/grads, fp32 memory
@@ -111,11 +120,11 @@ def srwm_step(t, ev=None):
         w.copy_(w0)                     # what `.repeat(bsz,1,1,1)` does in the layer
     if ev:
         ev[0].record()
-    srwm_hip.self_ref_forward(t["x"], *t["W"], *t["saved"], t["out"])
+    srwm_hip.self_ref_forward(t["x"], *t["W"], *t["saved"], t["out"], flags=t.get("flags", 0))
     if ev:
         ev[1].record()
     srwm_hip.self_ref_backward(t["x"], *t["saved"], t["go"], *t["W"], t["gx"], *t["gW"],
-                               flags=srwm_hip.GRAD_STATE_ZERO)
+                               flags=srwm_hip.GRAD_STATE_ZERO | t.get("flags", 0))
     if ev:
         ev[2].record()
 
@@ -467,6 +476,8 @@ def build_workload(name, dev):
     op, N, H, L, E = WORKLOADS[name]
     if op == "srwm":
         step, t = srwm_step, srwm_setup(N, H, L, E, dev)
+        if "_generic_" in name:
+            t["flags"] = srwm_hip.FLAG_GENERIC
     elif op == "srwm_layer":
         step, t = srwm_layer_step, srwm_setup(N, H, L, E, dev)
         t["slow"] = [w[0].contiguous() for w in t["W0"]]
@@ -550,8 +561,11 @@ def rooflines(name, fwd_ms, bwd_ms):
         # LDS-resident memory): a chunkwise kernel does not make those passes, so it may exceed it
         r["roofline_lds_yardstick"] = roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS)
     else:
-        r["roofline"] = dict(roof("lds", lds_b, bwd_ms, LDS_PEAK_GBS), kernel="backward")
-        r["roofline_fwd_bwd"] = roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS)
+        note = ("yardstick, not utilisation: the bytes are the minimal passes over a state held in LDS, but these kernels "
+                "hold the state in VGPRs and never move them, so the fraction can pass 1; the physical bound is "
+                "roofline_valu (fp32 vector ALU)")
+        r["roofline"] = dict(roof("lds", lds_b, bwd_ms, LDS_PEAK_GBS), kernel="backward", note=note)
+        r["roofline_fwd_bwd"] = dict(roof("lds", lds_f + lds_b, fwd_ms + bwd_ms, LDS_PEAK_GBS), note=note)
         # the state lives in VGPRs, so the LDS bytes above are a yardstick, not traffic; the unit that
         # actually limits these kernels is the fp32 vector ALU
         vf, vb = vector_flops(op, N, H, L, E)
@@ -565,7 +579,8 @@ def rooflines(name, fwd_ms, bwd_ms):
 
 
 # Driver-visible figures for the other benchmark configurations: (workload, timed steps, warm-up)
-OTHER_WORKLOADS = (("srwm_layer_c4", 50, 10), ("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
+OTHER_WORKLOADS = (("srwm_layer_c4", 50, 10), ("srwm_generic_c4", 5, 2), ("srwm_e48", 20, 5), ("srwm_d16", 100, 20),
+                   ("srwm_rl_d16", 100, 20), ("delta_e96", 50, 10), ("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
                    ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5), ("delta_c5_op_chunk", 40, 5), ("delta_prologue_c2", 100, 20), ("delta_prologue_c5", 40, 5),
                    ("delta_layer_c2", 50, 10))
 

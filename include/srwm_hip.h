@@ -50,6 +50,10 @@ extern "C" {
                                      it, :1213-1229); equal to ZERO when the buffers arrive zeroed. */
 #define SRWM_GRAD_STATE_MASK 3u
 #define SRWM_FLAG_GENERIC 16u     /* force the any-size LDS-resident kernel (testing / comparison) */
+#define SRWM_FLAG_NO_FALLBACK 8192u /* every entry point with two kernel families: return SRWM_ENOKERNEL where the
+                                      register-resident kernels do not take the call (head size without an
+                                      instantiation, misaligned base or strides) instead of running the several times
+                                      slower LDS-resident ones.  Not together with SRWM_FLAG_GENERIC (SRWM_EINVAL). */
 #define SRWM_FLAG_CHUNKWISE 32u   /* delta rule only: chunkwise matrix-core kernels instead of the step-by-step
                                      ones (forward: chunks of 64 steps; backward: a sweep over memory columns and
                                      one over memory rows); E == M in {64, 128}, else SRWM_ENOKERNEL.  Forward and
@@ -75,7 +79,9 @@ extern "C" {
                                        SRWM_FLAG_BF16_GRADS or SRWM_FLAG_EXACT_PRODUCTS): those steps are all it reads of
                                        v_old, so a quarter of the forward's writes never happens.  The step-by-step
                                        backward, and the chunkwise one with bf16 inputs, single products and fp32
-                                       gradients, need every row: do not set it for them. */
+                                       gradients, need every row.  delta_backward_* take the flag as the statement
+                                       "the forward ran with it": they return SRWM_EINVAL in exactly those modes
+                                       instead of reading rows nobody wrote. */
 #define SRWM_FLAG_NORM_EPS 2048u   /* delta_layer_prologue_f32 only: 1e-5 is added to the normalisers of q and k (the RL
                                      tree's layers, reinforcement_learning/torchbeast/layer.py:30-33) */
 /* srwm_layer_forward_* / srwm_layer_backward_* only: */
@@ -524,7 +530,7 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 14. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 15. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

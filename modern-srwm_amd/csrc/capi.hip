@@ -97,6 +97,11 @@ int scratch_base(float **base) {
 // floats of one per-row gradient tensor in `scratch`, rounded up so that the next one starts 256-byte aligned
 int64_t scratch_span(int N, int H, int E, int width) { return ((int64_t)N * H * E * width + 63) / 64 * 64; }
 
+// kernel-family bits every entry point with two families takes; asking for the LDS-resident family and
+// forbidding it at once is refused
+constexpr unsigned kFamily = SRWM_FLAG_GENERIC | SRWM_FLAG_NO_FALLBACK;
+bool family_ok(unsigned flags) { return (flags & kFamily) != kFamily; }
+
 size_t srwm_fwd_sq(int e) { return srwm_fwd_generic_lds_bytes(e, e); }
 size_t srwm_bwd_sq(int e) { return srwm_bwd_generic_lds_bytes(e, e); }
 size_t delta_fwd_sq(int e) { return delta_fwd_generic_lds_bytes(e, e); }
@@ -106,7 +111,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 14; }
+int srwm_hip_abi_version(void) { return 15; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -140,7 +145,7 @@ int srwm_forward_wide_f32(const float *x, const int64_t xs[3], float *Wy, float 
     if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
         !out || !xs)
         return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || (flags & ~(SRWM_FLAG_GENERIC))) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || !family_ok(flags) || !family_ok(flags) || (flags & ~kFamily)) return SRWM_EINVAL;
     if (!stride_ok(xs, N, H, L, E)) return SRWM_ESTRIDE;
     SrwmFwdParams p{x, xs[0], xs[1], xs[2], Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff, kdiff, bdiff,
                     out, N, H, L, E};
@@ -149,6 +154,7 @@ int srwm_forward_wide_f32(const float *x, const int64_t xs[3], float *Wy, float 
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_fwd_tiled(p, s);
         if (r >= 0) return r;
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
     }
     if (srwm_fwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_srwm_fwd_generic(p, s);
@@ -172,8 +178,8 @@ static int layer_forward(bool io16, const float *x, const int64_t xs[3], const f
     if (!x || !Wy || !Wq || !Wk || !wb || !q || !k || !beta || !ydiff || !qdiff || !kdiff || !bdiff ||
         !out || !xs)
         return SRWM_EINVAL;
-    const unsigned known = SRWM_FLAG_GENERIC | SRWM_FLAG_STATE_SHIFT | SRWM_FLAG_FRESH_STATE | SRWM_FLAG_SOFTMAX_INPUT;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || (flags & ~known)) return SRWM_EINVAL;
+    const unsigned known = kFamily | SRWM_FLAG_STATE_SHIFT | SRWM_FLAG_FRESH_STATE | SRWM_FLAG_SOFTMAX_INPUT;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || !family_ok(flags) || (flags & ~known)) return SRWM_EINVAL;
     const bool needs_shared = keep || (flags & (SRWM_FLAG_STATE_SHIFT | SRWM_FLAG_FRESH_STATE));
     if (needs_shared && (!sWy || !sWq || !sWk || !swb)) return SRWM_EINVAL;
     if (!stride_ok(xs, N, H, L, E) || (os && !out_stride_ok(os, N, H, L, Y))) return SRWM_ESTRIDE;
@@ -186,6 +192,7 @@ static int layer_forward(bool io16, const float *x, const int64_t xs[3], const f
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_fwd_tiled(p, s);
         if (r >= 0) return r;
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
     }
     if (srwm_fwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_srwm_fwd_generic(p, s);
@@ -214,7 +221,7 @@ int srwm_forward_bf16(const uint16_t *x, const int64_t xs[3], float *Wy, float *
                       float *q, float *k, float *beta, float *ydiff, float *qdiff, float *kdiff,
                       float *bdiff, uint16_t *out, int N, int H, int L, int E, unsigned flags,
                       void *stream) {
-    if (flags & ~(SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    if (!family_ok(flags) || !family_ok(flags) || (flags & ~kFamily)) return SRWM_EINVAL;
     return srwm_layer_forward_bf16(x, xs, nullptr, nullptr, nullptr, nullptr, nullptr, Wy, Wq, Wk, wb, q, k, beta,
                                    ydiff, qdiff, kdiff, bdiff, out, nullptr, N, H, L, E, E, flags, stream);
 }
@@ -224,7 +231,7 @@ int srwm_forward_steps_f32(const float *x, const int64_t xs[3], const float *kee
                            float *Wk, float *wb, float *q, float *k, float *beta, float *ydiff,
                            float *qdiff, float *kdiff, float *bdiff, float *out, int N, int H, int L,
                            int E, unsigned flags, void *stream) {
-    if (flags & ~(SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    if (!family_ok(flags) || !family_ok(flags) || (flags & ~kFamily)) return SRWM_EINVAL;
     return srwm_layer_forward_f32(x, xs, keep, sWy, sWq, sWk, swb, Wy, Wq, Wk, wb, q, k, beta, ydiff, qdiff,
                                   kdiff, bdiff, out, nullptr, N, H, L, E, E, flags, stream);
 }
@@ -234,13 +241,14 @@ int srwm_readout_grad_wide_f32(const float *k, const float *beta, const float *y
                                const float *Wy_entry, float *grad_x, int N, int H, int L, int E, int Y,
                                unsigned flags, void *stream) {
     if (!k || !beta || !ydiff || !grad_out || !gs || !Wy_entry || !grad_x || (keep && !sWy)) return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || !family_ok(flags) || (flags & ~kFamily)) return SRWM_EINVAL;
     if (!stride_ok(gs, N, H, L, Y)) return SRWM_ESTRIDE;
     ReplayParams p{k, {(int64_t)H * L * E, (int64_t)L * E, E}, ydiff, beta, 4, keep, grad_out,
                    {gs[0], gs[1], gs[2]}, Wy_entry, keep ? sWy : nullptr, grad_x, N, H, L, E, Y};
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_replay_tiled(p, (hipStream_t)stream);
         if (r >= 0) return r;
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
     }
     if (E > 256 || Y > 256 || replay_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_replay(p, (hipStream_t)stream);
@@ -253,7 +261,7 @@ int srwm_layer_readout_grad_f32(const float *x, const int64_t xs[3], const float
                                 unsigned flags, void *stream) {
     if (!x || !xs || !k || !beta || !ydiff || !sWy || !grad_out || !gs || !Wy_entry || !grad_x || !gWy || !gsWy)
         return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_STATE_SHIFT)))
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || !family_ok(flags) || (flags & ~(kFamily | SRWM_FLAG_STATE_SHIFT)))
         return SRWM_EINVAL;
     if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, Y)) return SRWM_ESTRIDE;
     ReplayParams p{k, {(int64_t)H * L * E, (int64_t)L * E, E}, ydiff, beta, 4, keep, grad_out,
@@ -262,6 +270,7 @@ int srwm_layer_readout_grad_f32(const float *x, const int64_t xs[3], const float
     hipStream_t s = (hipStream_t)stream;
     int r = (flags & SRWM_FLAG_GENERIC) ? -1 : launch_replay_tiled(p, s);
     if (r < 0) {
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
         if (E > 256 || Y > 256 || replay_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
         r = launch_replay(p, s);
     }
@@ -283,7 +292,7 @@ int delta_forward_steps_f32(const float *Q, const int64_t qs[3], const float *K,
                             const int64_t os[3], int N, int H, int L, int E, int M, unsigned flags, void *stream) {
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !W || !out || !qs || !ks || !vs || !bs)
         return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || !family_ok(flags) || (flags & ~kFamily)) return SRWM_EINVAL;
     const int64_t dense_out[3] = {(int64_t)H * L * M, (int64_t)L * M, (int64_t)M};
     if (!os) os = dense_out;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
@@ -296,6 +305,7 @@ int delta_forward_steps_f32(const float *Q, const int64_t qs[3], const float *K,
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_delta_fwd_tiled(p, s);
         if (r >= 0) return r;
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
     }
     if (delta_fwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_delta_fwd_generic(p, s);
@@ -305,13 +315,14 @@ int delta_readout_replay_f32(const float *K, const int64_t ks[3], const float *v
                              const float *grad_out, const int64_t gs[3], const float *W_entry, float *u,
                              int N, int H, int L, int E, int M, unsigned flags, void *stream) {
     if (!K || !ks || !v_insert || !grad_out || !gs || !W_entry || !u) return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || !family_ok(flags) || (flags & ~kFamily)) return SRWM_EINVAL;
     if (!stride_ok(ks, N, H, L, E) || !stride_ok(gs, N, H, L, M)) return SRWM_ESTRIDE;
     ReplayParams p{K, {ks[0], ks[1], ks[2]}, v_insert, nullptr, 0, keep, grad_out, {gs[0], gs[1], gs[2]},
                    W_entry, nullptr, u, N, H, L, E, M};
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_replay_tiled(p, (hipStream_t)stream);
         if (r >= 0) return r;
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
     }
     if (E > 256 || M > 256 || replay_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_replay(p, (hipStream_t)stream);
@@ -326,7 +337,7 @@ int delta_steps_backward_f32(const float *Q, const int64_t qs[3], const float *K
     if (!Q || !K || !V || !beta || !v_old || !v_insert || !grad_out || !W_entry || !gQ || !gK || !gV || !gbeta ||
         !qs || !ks || !vs || !bs || !gs)
         return SRWM_EINVAL;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || (flags & ~SRWM_FLAG_GENERIC)) return SRWM_EINVAL;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || !family_ok(flags) || (flags & ~kFamily)) return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
         !stride_ok(bs, N, H, L, 1) || !stride_ok(gs, N, H, L, M))
         return SRWM_ESTRIDE;
@@ -401,7 +412,7 @@ int srwm_backward_wide_f32(const float *x, const int64_t xs[3], const float *q, 
         return SRWM_EINVAL;
     const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || mode == 3u ||
-        (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)))
+        !family_ok(flags) || (flags & ~(kFamily | SRWM_GRAD_STATE_MASK)))
         return SRWM_EINVAL;
     if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, Y)) return SRWM_ESTRIDE;
     SrwmBwdParams p{x, xs[0], xs[1], xs[2], q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out,
@@ -410,6 +421,7 @@ int srwm_backward_wide_f32(const float *x, const int64_t xs[3], const float *q, 
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_bwd_tiled(p, s);
         if (r >= 0) return r;
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
     }
     if (srwm_bwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_srwm_bwd_generic(p, s);
@@ -438,8 +450,8 @@ static int layer_backward(bool io16, const float *x, const int64_t xs[3], const 
         !Wk || !wb || !grad_x || !gWy || !gWq || !gWk || !gwb || !xs || !gs)
         return SRWM_EINVAL;
     const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
-    const unsigned known = SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK | SRWM_FLAG_STATE_SHIFT | SRWM_FLAG_SOFTMAX_INPUT;
-    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || mode == 3u || (flags & ~known)) return SRWM_EINVAL;
+    const unsigned known = kFamily | SRWM_GRAD_STATE_MASK | SRWM_FLAG_STATE_SHIFT | SRWM_FLAG_SOFTMAX_INPUT;
+    if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || mode == 3u || !family_ok(flags) || (flags & ~known)) return SRWM_EINVAL;
     if ((flags & SRWM_FLAG_STATE_SHIFT) && (!sWy || !sWq || !sWk || !swb)) return SRWM_EINVAL;
     const bool sums = gsWy || gsWq || gsWk || gswb;
     if (sums && (!gsWy || !gsWq || !gsWk || !gswb)) return SRWM_EINVAL;
@@ -455,6 +467,7 @@ static int layer_backward(bool io16, const float *x, const int64_t xs[3], const 
     int r = -1;
     if (!(flags & SRWM_FLAG_GENERIC)) r = launch_srwm_bwd_tiled(p, s);
     if (r < 0) {
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
         if (srwm_bwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
         r = launch_srwm_bwd_generic(p, s);
     }
@@ -522,7 +535,7 @@ int srwm_backward_bf16(const uint16_t *x, const int64_t xs[3], const float *q, c
                        const float *Wq, const float *Wk, const float *wb, float *grad_x, float *gWy,
                        float *gWq, float *gWk, float *gwb, int N, int H, int L, int E, unsigned flags,
                        void *stream) {
-    if (flags & ~(SRWM_FLAG_GENERIC | SRWM_GRAD_STATE_MASK)) return SRWM_EINVAL;
+    if (!family_ok(flags) || (flags & ~(kFamily | SRWM_GRAD_STATE_MASK))) return SRWM_EINVAL;
     return srwm_layer_backward_bf16(x, xs, q, k, beta, ydiff, qdiff, kdiff, bdiff, grad_out, gs, nullptr, nullptr,
                                     nullptr, nullptr, Wy, Wq, Wk, wb, grad_x, nullptr, gWy, gWq, gWk, gwb, nullptr,
                                     nullptr, nullptr, nullptr, N, H, L, E, E, flags, stream);
@@ -537,7 +550,7 @@ int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const
     const int64_t dense_out[3] = {(int64_t)H * L * M, (int64_t)L * M, (int64_t)M};
     if (!os) os = dense_out;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) ||
-        (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_SPARSE_V_OLD)) ||
+        !family_ok(flags) || (flags & ~(kFamily | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_SPARSE_V_OLD)) ||
         (flags & (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE)) == (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE) ||
         ((flags & SRWM_FLAG_SPARSE_V_OLD) && !(flags & SRWM_FLAG_CHUNKWISE)))
         return SRWM_EINVAL;
@@ -555,6 +568,7 @@ int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_delta_fwd_tiled(p, s);
         if (r >= 0) return r;
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
     }
     if (delta_fwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_delta_fwd_generic(p, s);
@@ -570,9 +584,13 @@ int delta_backward_f32(const float *Q, const int64_t qs[3], const float *K, cons
         return SRWM_EINVAL;
     const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u ||
-        (flags & ~(SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_GRAD_STATE_MASK)) ||
+        !family_ok(flags) ||
+        (flags & ~(kFamily | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_SPARSE_V_OLD |
+                   SRWM_GRAD_STATE_MASK)) ||
         (flags & (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE)) == (SRWM_FLAG_GENERIC | SRWM_FLAG_CHUNKWISE))
         return SRWM_EINVAL;
+    // a v_old that holds only the steps with a tiny beta serves the chunkwise backward alone
+    if ((flags & SRWM_FLAG_SPARSE_V_OLD) && !(flags & SRWM_FLAG_CHUNKWISE)) return SRWM_EINVAL;
     if (!gW && mode != SRWM_GRAD_STATE_ZERO) return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
         !stride_ok(bs, N, H, L, 1) || !stride_ok(gs, N, H, L, M))
@@ -588,6 +606,7 @@ int delta_backward_f32(const float *Q, const int64_t qs[3], const float *K, cons
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_delta_bwd_tiled(p, s);
         if (r >= 0) return r;
+        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
     }
     if (delta_bwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_delta_bwd_generic(p, s);
@@ -602,7 +621,7 @@ int delta_forward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *K
     const int64_t dense_out[3] = {(int64_t)H * L * M, (int64_t)L * M, (int64_t)M};
     if (!os) os = dense_out;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) ||
-        (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_SPARSE_V_OLD)) ||
+        (flags & ~(SRWM_FLAG_NO_FALLBACK | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_SPARSE_V_OLD)) ||
         ((flags & SRWM_FLAG_SPARSE_V_OLD) && !(flags & SRWM_FLAG_CHUNKWISE)))
         return SRWM_EINVAL;
     if (!stride_ok(qs, N, H, L, E) || !stride_ok(ks, N, H, L, E) || !stride_ok(vs, N, H, L, M) ||
@@ -627,7 +646,14 @@ int delta_backward_bf16(const uint16_t *Q, const int64_t qs[3], const uint16_t *
         return SRWM_EINVAL;
     const unsigned mode = flags & SRWM_GRAD_STATE_MASK;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, M) || mode == 3u ||
-        (flags & ~(SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_BF16_GRADS | SRWM_GRAD_STATE_MASK)))
+        (flags & ~(SRWM_FLAG_NO_FALLBACK | SRWM_FLAG_CHUNKWISE | SRWM_FLAG_EXACT_PRODUCTS | SRWM_FLAG_BF16_GRADS |
+                   SRWM_FLAG_SPARSE_V_OLD | SRWM_GRAD_STATE_MASK)))
+        return SRWM_EINVAL;
+    // a v_old that holds only the steps with a tiny beta: the chunkwise backward in the modes whose second
+    // sweep forms grad_beta (rounded gradients, or operand pairs everywhere); with single products and
+    // fp32 gradients the first sweep reads every row of v_old
+    if ((flags & SRWM_FLAG_SPARSE_V_OLD) &&
+        (!(flags & SRWM_FLAG_CHUNKWISE) || !(flags & (SRWM_FLAG_BF16_GRADS | SRWM_FLAG_EXACT_PRODUCTS))))
         return SRWM_EINVAL;
     if (!gW && mode != SRWM_GRAD_STATE_ZERO) return SRWM_EINVAL;
     // rounded gradients: the chunkwise kernels with single products, and no gradient of the memory

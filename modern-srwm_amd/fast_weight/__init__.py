@@ -25,11 +25,13 @@ CHUNKWISE_BACKWARD = "auto"
 # bfloat16 anyway); True forms them from hi + lo operand pairs as well (~8 % slower).  The memory,
 # v_old, v_insert, grad_V and grad_beta do not depend on this.  No effect with float32 inputs.
 EXACT_PRODUCTS = False
-# Memory layout of `out`: True allocates it like V (what elementwise tensor operations do with their operand), so that
-# the step-major views the layers hand in give a step-major `out` and their transpose / reshape / transpose on the way
-# to the output map (supervised_learning/layer.py:98-100) is a view; False always allocates a contiguous (N, H, L, M)
-# tensor as the reference does (for callers that go on with .view()).  The values are the same.
-OUT_LIKE_V = True
+# Memory layout of `out`.  False (the default, what the reference does): a contiguous (N, H, L, M) tensor whatever
+# the inputs look like, so callers may go on with .view().  True: allocated like V (what elementwise tensor
+# operations do with their operand), so that the step-major views the layers hand in give a step-major `out` and their
+# transpose / reshape / transpose on the way to the output map (supervised_learning/layer.py:98-100) is a view
+# instead of two copies.  The values are the same.  The layer modules of this package ask for the second form call
+# by call (fast_weight_delta_rows, fast_weight_delta_steps_rows); this switch changes the plain operators.
+OUT_LIKE_V = False
 
 
 def _chunk_flags(choice, E, M, L):
@@ -50,9 +52,9 @@ def _forward_flags(E, M, L):
 
 def causal_dot_product_cuda(q, k, v, beta, v_old, v_insert, kv, out, flags=None):
     """The reference's extension function (same eight arguments).  flags: the kernel choice, by default
-    what the module switches say now; returns the flags used."""
+    what the module switches say now with a complete v_old (any backward can follow); returns the flags used."""
     if flags is None:
-        flags = _forward_flags(q.shape[-1], v.shape[-1], q.shape[2])
+        flags = _chunk_flags(CHUNKWISE_FORWARD, q.shape[-1], v.shape[-1], q.shape[2])
     srwm_hip.fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=flags)
     return flags
 
@@ -61,10 +63,10 @@ def causal_dot_backward_cuda(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_
                              forward_flags=0):
     """The reference's extension function (same twelve arguments).  forward_flags: what the forward ran
     with -- a forward that wrote v_old only where a chunkwise backward reads it gets a chunkwise backward
-    whatever the switch says by now."""
+    whatever the switch says by now, and the library refuses the modes that would read the rows left out."""
     flags = _chunk_flags(CHUNKWISE_BACKWARD, q.shape[-1], v.shape[-1], q.shape[2])
-    if forward_flags & srwm_hip.FLAG_SPARSE_V_OLD and not flags:
-        flags = _chunk_flags(True, q.shape[-1], v.shape[-1], q.shape[2])
+    if forward_flags & srwm_hip.FLAG_SPARSE_V_OLD:
+        flags = (flags or _chunk_flags(True, q.shape[-1], v.shape[-1], q.shape[2])) | srwm_hip.FLAG_SPARSE_V_OLD
     srwm_hip.fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, grad_k, grad_v,
                                   grad_beta, flags=flags)
 
@@ -75,16 +77,20 @@ class DeltaFastWeight(torch.autograd.Function):
     dot_backward = {"cuda": causal_dot_backward_cuda}
 
     @staticmethod
-    def forward(ctx, Q, K, V, beta, W):
+    def forward(ctx, Q, K, V, beta, W, out_like_v=None):
         for t in (Q, K, V, beta, W):
             assert t.device.type != "cpu"
         device = Q.device
         N, H, L, E = Q.shape
         _, _, _, M = V.shape
-        out = torch.empty_like(V) if OUT_LIKE_V else torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
+        ctx.n_inputs = 5 if out_like_v is None else 6
+        like_v = OUT_LIKE_V if out_like_v is None else out_like_v
+        out = torch.empty_like(V) if like_v else torch.empty((N, H, L, M), device=device, dtype=Q.dtype)
         V_old = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
         V_insert = torch.empty((N, H, L, M), device=device, dtype=W.dtype)
-        ctx.forward_flags = DeltaFastWeight.dot[device.type](Q.data, K.data, V.data, beta.data, V_old, V_insert, W, out)
+        # the operator knows which backward follows, so only it lets the forward leave rows of v_old out
+        ctx.forward_flags = DeltaFastWeight.dot[device.type](Q.data, K.data, V.data, beta.data, V_old, V_insert, W, out,
+                                                             flags=_forward_flags(E, M, L))
         ctx.save_for_backward(Q, K, V, beta, V_old, V_insert, W)
         return out
 
@@ -100,11 +106,16 @@ class DeltaFastWeight(torch.autograd.Function):
         DeltaFastWeight.dot_backward[Q.device.type](
             Q.data, K.data, V.data, beta.data, V_old.data, V_insert.data, grad_out, W.data,
             grad_Q, grad_K, grad_V, grad_beta, forward_flags=ctx.forward_flags or 0)
-        return grad_Q, grad_K, grad_V, grad_beta, None
+        return (grad_Q, grad_K, grad_V, grad_beta, None, None)[:ctx.n_inputs]
 
 
 # Alias the autograd functions to python style snake case naming
 fast_weight_delta = DeltaFastWeight.apply
+
+
+def fast_weight_delta_rows(Q, K, V, beta, W):
+    """fast_weight_delta with `out` allocated in the memory order of V's rows (see OUT_LIKE_V)."""
+    return DeltaFastWeight.apply(Q, K, V, beta, W, True)
 
 
 class DeltaLayerInputs(torch.autograd.Function):
@@ -152,13 +163,15 @@ class DeltaFastWeightSteps(torch.autograd.Function):
     OVERWRITTEN with the memory after the last step (the carried state)."""
 
     @staticmethod
-    def forward(ctx, Q, K, V, beta, keep, W):
+    def forward(ctx, Q, K, V, beta, keep, W, out_like_v=None):
         for t in (Q, K, V, beta, W):
             assert t.device.type != "cpu"
         N, H, L, E = Q.shape
         M = V.shape[-1]
         new = lambda: torch.empty((N, H, L, M), device=Q.device, dtype=Q.dtype)
-        out, V_old, V_insert = torch.empty_like(V) if OUT_LIKE_V else new(), new(), new()   # as fast_weight_delta
+        ctx.n_inputs = 6 if out_like_v is None else 7
+        like_v = OUT_LIKE_V if out_like_v is None else out_like_v
+        out, V_old, V_insert = torch.empty_like(V) if like_v else new(), new(), new()   # as fast_weight_delta
         W_entry = W.detach().clone()
         srwm_hip.fast_weight_forward_steps(Q.data, K.data, V.data, beta.data, keep, V_old, V_insert, W.data, out)
         ctx.save_for_backward(Q, K, V, beta, keep, V_old, V_insert, W_entry)
@@ -173,7 +186,12 @@ class DeltaFastWeightSteps(torch.autograd.Function):
         grad_Q, grad_K, grad_V, grad_beta = new(E), new(E), new(M), new(1)
         srwm_hip.fast_weight_steps_backward(Q, K, V, beta, keep, V_old, V_insert, grad_out, W_entry,
                                             grad_Q, grad_K, grad_V, grad_beta)
-        return grad_Q, grad_K, grad_V, grad_beta, None, None
+        return (grad_Q, grad_K, grad_V, grad_beta, None, None, None)[:ctx.n_inputs]
 
 
 fast_weight_delta_steps = DeltaFastWeightSteps.apply
+
+
+def fast_weight_delta_steps_rows(Q, K, V, beta, keep, W):
+    """fast_weight_delta_steps with `out` allocated in the memory order of V's rows (see OUT_LIKE_V)."""
+    return DeltaFastWeightSteps.apply(Q, K, V, beta, keep, W, True)

@@ -18,7 +18,11 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from fast_weight import delta_layer_inputs, fast_weight_delta, fast_weight_delta_steps
+# the delta-rule operators with `out` in the memory order of the step-major views these layers hand in, so that the
+# reshape chain behind them (_heads_out) is a view; the plain operators return the reference's dense (N, H, L, M)
+from fast_weight import delta_layer_inputs
+from fast_weight import fast_weight_delta_rows as fast_weight_delta
+from fast_weight import fast_weight_delta_steps_rows as fast_weight_delta_steps
 from self_ref_v0 import self_ref_layer, self_ref_layer_steps, self_ref_v0, self_ref_v0_steps, stateful_self_ref_v0
 from self_ref_v1 import self_ref_v1, self_ref_v1_steps
 

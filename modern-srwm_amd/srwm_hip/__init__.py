@@ -29,6 +29,7 @@ GRAD_STATE_ZERO = 0
 GRAD_STATE_IN = 1
 GRAD_STATE_ACCUM = 2
 FLAG_GENERIC = 16
+FLAG_NO_FALLBACK = 8192    # raise where the register-resident kernels do not take the call instead of running the LDS-resident ones
 FLAG_CHUNKWISE = 32     # delta forward: chunkwise MFMA kernel (E == M in {64, 128})
 FLAG_EXACT_PRODUCTS = 512   # chunkwise kernels with bf16 inputs: every product from hi + lo operand pairs
 FLAG_BF16_GRADS = 1024      # chunkwise delta backward with bf16 inputs: grad_q, grad_k, grad_v written as bf16 by the library
@@ -38,7 +39,11 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 14
+ABI_VERSION = 15
+
+# True: a call that the register-resident kernels do not take (head size without an instantiation, misaligned
+# base or strides) raises instead of running on the several times slower LDS-resident kernels
+NO_FALLBACK = False
 
 _lib = None
 
@@ -137,6 +142,10 @@ def _require(t, name, shape=None, dtype=torch.float32):
         raise ValueError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
 
 
+def _fam(flags):
+    return flags | FLAG_NO_FALLBACK if NO_FALLBACK and not flags & FLAG_GENERIC else flags
+
+
 def _ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
@@ -222,20 +231,20 @@ def self_ref_forward(x, W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, 
             _Dense([W_y, W_q, W_k, w_b, q, k, beta, y_diff, q_diff, k_diff, beta_diff, out], True) as d:
         if io == torch.bfloat16 and Y == E:
             name = "srwm_forward_bf16"
-            code = lib().srwm_forward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
+            code = lib().srwm_forward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, _fam(flags),
                                            _stream(x.device))
         elif io == torch.bfloat16:   # wide output block: the layer entry point without any of its extras
             name = "srwm_layer_forward_bf16"
             code = lib().srwm_layer_forward_bf16(_ptr(xs), xstr, null, null, null, null, null,
-                                                 *[_ptr(t) for t in d], None, N, H, L, E, Y, flags, _stream(x.device))
+                                                 *[_ptr(t) for t in d], None, N, H, L, E, Y, _fam(flags), _stream(x.device))
         elif Y == E:
             name = "srwm_forward_f32"
-            code = lib().srwm_forward_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, flags,
+            code = lib().srwm_forward_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, _fam(flags),
                                           _stream(x.device))
         else:
             name = "srwm_forward_wide_f32"
             code = lib().srwm_forward_wide_f32(_ptr(xs), xstr, *[_ptr(t) for t in d], N, H, L, E, Y,
-                                               flags, _stream(x.device))
+                                               _fam(flags), _stream(x.device))
     _check(code, name)
 
 
@@ -277,7 +286,7 @@ def self_ref_forward_steps(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff
         code = lib().srwm_forward_steps_f32(
             _ptr(xs), xstr, _ptr(keep) if keep is not None else null,
             *[(_ptr(t) if keep is not None else t) for t in sl],
-            *[_ptr(t) for t in d], N, H, L, E, flags, _stream(x.device))
+            *[_ptr(t) for t in d], N, H, L, E, _fam(flags), _stream(x.device))
     _check(code, "srwm_forward_steps_f32")
 
 
@@ -308,7 +317,7 @@ def self_ref_readout_grad(k, beta, y_diff, keep, slow_W_y, grad_out, W_y_entry, 
         code = lib().srwm_readout_grad_wide_f32(
             _ptr(sv[0]), _ptr(sv[1]), _ptr(sv[2]), _ptr(keep) if keep is not None else null,
             _ptr(slow_W_y) if keep is not None else null, _ptr(gos), gstr, _ptr(sv[3]), _ptr(gr[0]),
-            N, H, L, E, Y, flags, _stream(k.device))
+            N, H, L, E, Y, _fam(flags), _stream(k.device))
     _check(code, "srwm_readout_grad_wide_f32")
 
 
@@ -350,7 +359,7 @@ def self_ref_layer_readout_grad(x, k, beta, y_diff, keep, slow_W_y, grad_out, W_
         code = lib().srwm_layer_readout_grad_f32(
             _ptr(xs), xstr, _ptr(sv[0]), _ptr(sv[1]), _ptr(sv[2]), _ptr(keep) if keep is not None else null,
             _ptr(slow_W_y), _ptr(gos), gstr, _ptr(sv[3]), _ptr(gr[0]), _ptr(grad_W_y), _ptr(grad_slow_W_y),
-            N, H, L, E, Y, flags, _stream(k.device))
+            N, H, L, E, Y, _fam(flags), _stream(k.device))
     _check(code, "srwm_layer_readout_grad_f32")
 
 
@@ -396,24 +405,24 @@ def self_ref_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, grad_out
             name = "srwm_backward_bf16"
             code = lib().srwm_backward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
                                             *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
-                                            N, H, L, E, flags, _stream(x.device))
+                                            N, H, L, E, _fam(flags), _stream(x.device))
         elif io == torch.bfloat16:
             null = ctypes.c_void_p(None)
             name = "srwm_layer_backward_bf16"
             code = lib().srwm_layer_backward_bf16(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
                                                   null, null, null, null, *[_ptr(t) for t in st],
                                                   _ptr(gr[0]), None, *[_ptr(t) for t in gr[1:]], null, null, null, null,
-                                                  N, H, L, E, Y, flags, _stream(x.device))
+                                                  N, H, L, E, Y, _fam(flags), _stream(x.device))
         elif Y == E:
             name = "srwm_backward_f32"
             code = lib().srwm_backward_f32(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
                                            *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
-                                           N, H, L, E, flags, _stream(x.device))
+                                           N, H, L, E, _fam(flags), _stream(x.device))
         else:
             name = "srwm_backward_wide_f32"
             code = lib().srwm_backward_wide_f32(_ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr,
                                                 *[_ptr(t) for t in st], *[_ptr(t) for t in gr],
-                                                N, H, L, E, Y, flags, _stream(x.device))
+                                                N, H, L, E, Y, _fam(flags), _stream(x.device))
     _check(code, name)
 
 
@@ -474,7 +483,7 @@ def self_ref_layer_forward(x, keep, slow, W_y, W_q, W_k, w_b, q, k, beta, y_diff
         name = "srwm_layer_forward_bf16" if io == torch.bfloat16 else "srwm_layer_forward_f32"
         code = getattr(lib(), name)(
             _ptr(xs), xstr, _ptr(keep) if keep is not None else null, *[_ptr(t) for t in sl],
-            *[_ptr(t) for t in d], _ptr(ot), (ctypes.c_int64 * 3)(*ot.stride()[:3]), N, H, L, E, Y, flags,
+            *[_ptr(t) for t in d], _ptr(ot), (ctypes.c_int64 * 3)(*ot.stride()[:3]), N, H, L, E, Y, _fam(flags),
             _stream(x.device))
     _check(code, name)
 
@@ -530,7 +539,7 @@ def self_ref_layer_backward(x, q, k, beta, y_diff, q_diff, k_diff, beta_diff, gr
         code = getattr(lib(), name)(
             _ptr(xs), xstr, *[_ptr(t) for t in sv], _ptr(gos), gstr, *[_ptr(t) for t in sl],
             *[_ptr(t) for t in st], _ptr(gxt), (ctypes.c_int64 * 3)(*gxt.stride()[:3]), *[_ptr(g) for g in grad_W], *gsl,
-            N, H, L, E, Y, flags, _stream(x.device))
+            N, H, L, E, Y, _fam(flags), _stream(x.device))
     _check(code, name)
 
 
@@ -558,6 +567,8 @@ def self_ref_layer_backward_noalloc(x, q, k, beta, y_diff, q_diff, k_diff, beta_
     _require(beta_diff, "beta_diff", (N, H, L, 4))
     for t, shp in zip((W_y, W_q, W_k, w_b), ((N, H, E, Y), (N, H, E, E), (N, H, E, E), (N, H, E, 4))):
         _require(t, "state", shp)
+    if not all(isinstance(t, torch.Tensor) and t.is_contiguous() for t in slow):
+        raise ValueError("self_ref_layer_backward_noalloc copies nothing: the shared weights must be contiguous")
     sl = _shared(slow, H, E, Y)
     for g, shp in zip(grad_slow, ((H, E, Y), (H, E, E), (H, E, E), (H, E, 4))):
         _require(g, "grad_slow", shp)
@@ -573,7 +584,7 @@ def self_ref_layer_backward_noalloc(x, q, k, beta, y_diff, q_diff, k_diff, beta_
         code = lib().srwm_layer_backward_noalloc_f32(
             _ptr(x), xstr, *[_ptr(t) for t in (q, k, beta, y_diff, q_diff, k_diff, beta_diff)], _ptr(grad_out), gstr,
             *[_ptr(t) for t in sl], *[_ptr(t) for t in (W_y, W_q, W_k, w_b)], _ptr(grad_x), None,
-            *[_ptr(g) for g in grad_slow], N, H, L, E, Y, flags, _stream(x.device))
+            *[_ptr(g) for g in grad_slow], N, H, L, E, Y, _fam(flags), _stream(x.device))
     _check(code, "srwm_layer_backward_noalloc_f32")
 
 
@@ -613,7 +624,7 @@ def fast_weight_forward(q, k, v, beta, v_old, v_insert, kv, out, flags=0):
     with torch.cuda.device(q.device), _Dense([v_old, v_insert, kv], True) as d, _Dense([] if by_strides else [out], True) as o:
         ot = out if by_strides else o[0]
         code = fn(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
-                  *[_ptr(t) for t in d], _ptr(ot), (ctypes.c_int64 * 3)(*ot.stride()[:3]), N, H, L, E, M, flags,
+                  *[_ptr(t) for t in d], _ptr(ot), (ctypes.c_int64 * 3)(*ot.stride()[:3]), N, H, L, E, M, _fam(flags),
                   _stream(q.device))
     _check(code, fn.__name__)
 
@@ -644,7 +655,7 @@ def fast_weight_forward_steps(q, k, v, beta, keep, v_old, v_insert, kv, out, fla
         code = lib().delta_forward_steps_f32(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
                                              _ptr(keep) if keep is not None else null,
                                              *[_ptr(t) for t in d], _ptr(ot), (ctypes.c_int64 * 3)(*ot.stride()[:3]),
-                                             N, H, L, E, M, flags, _stream(q.device))
+                                             N, H, L, E, M, _fam(flags), _stream(q.device))
     _check(code, "delta_forward_steps_f32")
 
 
@@ -669,7 +680,7 @@ def fast_weight_readout_replay(k, v_insert, keep, grad_out, kv_entry, u, flags=0
     (ks, kstr), (gos, gstr) = _strided(k), _strided(grad_out)
     with torch.cuda.device(k.device), _Dense([v_insert, kv_entry], False) as sv, _Dense([u], True) as d:
         code = lib().delta_readout_replay_f32(_ptr(ks), kstr, _ptr(sv[0]), _ptr(keep) if keep is not None else null,
-                                              _ptr(gos), gstr, _ptr(sv[1]), _ptr(d[0]), N, H, L, E, M, flags,
+                                              _ptr(gos), gstr, _ptr(sv[1]), _ptr(d[0]), N, H, L, E, M, _fam(flags),
                                               _stream(k.device))
     _check(code, "delta_readout_replay_f32")
 
@@ -703,7 +714,7 @@ def fast_weight_steps_backward(q, k, v, beta, keep, v_old, v_insert, grad_out, k
             _Dense([grad_q, grad_k, grad_v, grad_beta], True) as d:
         code = lib().delta_steps_backward_f32(
             _ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr, _ptr(keep) if keep is not None else null,
-            _ptr(sv[0]), _ptr(sv[1]), _ptr(gos), gstr, _ptr(sv[2]), *[_ptr(t) for t in d], N, H, L, E, M, flags,
+            _ptr(sv[0]), _ptr(sv[1]), _ptr(gos), gstr, _ptr(sv[2]), *[_ptr(t) for t in d], N, H, L, E, M, _fam(flags),
             _stream(q.device))
     _check(code, "delta_steps_backward_f32")
 
@@ -816,7 +827,7 @@ def fast_weight_backward(q, k, v, beta, v_old, v_insert, grad_out, kv, grad_q, g
         gkv = _ptr(d[5]) if grad_kv is not None else ctypes.c_void_p(None)
         code = fn(_ptr(qs), qstr, _ptr(ks), kstr, _ptr(vs), vstr, _ptr(bs), bstr,
                   _ptr(sv[0]), _ptr(sv[1]), _ptr(gos), gstr,
-                  *[_ptr(t) for t in d[:5]], gkv, N, H, L, E, M, flags, _stream(q.device))
+                  *[_ptr(t) for t in d[:5]], gkv, N, H, L, E, M, _fam(flags), _stream(q.device))
     _check(code, fn.__name__)
     if io == torch.bfloat16:
         for dst, src in zip(bf_outs, (grad_q, grad_k, grad_v, grad_beta)):

@@ -130,6 +130,9 @@ def test_argument_validation_needs_no_gpu():
     assert srwm_f(fake(), ok_strides, N, -3, 0) == -1          # negative head size
     assert srwm_f(fake(), ok_strides, N, E, 32) == -1          # the chunkwise flag means nothing to the SRWM
     assert srwm_f(fake(), ok_strides, N, E, 1 << 20) == -1     # unknown flag bit
+    assert srwm_f(fake(), ok_strides, N, E, 16 | 8192) == -1   # the LDS-resident kernels asked for and forbidden at once
+    assert srwm_f(fake(), ok_strides, N, 24, 8192) == -4       # SRWM_ENOKERNEL: no register-resident kernel for E = 24, and no fallback wanted
+    assert srwm_f(P(0x1004), ok_strides, N, E, 8192) == -4     # nor for a base that is not 16-byte aligned
     assert srwm_f(fake(), huge, N, E, 0) == -3                 # SRWM_ESTRIDE: extent overflows the 2^40 bound
     assert srwm_f(fake(), ok_strides, N, 4096, 0) == -2        # SRWM_ESIZE: 4096 x 12292 floats fit no CU
     srwm_b = lambda flags: L.srwm_backward_f32(fake(), ok_strides, *[fake() for _ in range(7)], fake(), ok_strides,
@@ -159,6 +162,14 @@ def test_argument_validation_needs_no_gpu():
     assert delta_bb(P(None), 32 | 512 | 1024, E) == -1         # with single products,
     assert delta_bb(fake(), 32 | 1024, E) == -1                # and without the gradient of the memory
     assert delta_bb(P(None), 32 | 1024, E) == -4               # accepted; SRWM_ENOKERNEL: E = M = 16 has no chunkwise kernel
+    # "the forward left rows of v_old out" (4096): refused by every backward that reads all rows of it
+    assert delta_b(P(None), 4096) == -1                        # the step-by-step sweep
+    assert delta_b(P(None), 16 | 4096) == -1                   # the LDS-resident one
+    assert delta_b(P(None), 32 | 4096) == -4                   # chunkwise, fp32: accepted (no kernel at E = M = 16)
+    assert delta_bb(P(None), 4096, E) == -1                    # bf16 step-by-step
+    assert delta_bb(P(None), 32 | 4096, E) == -1               # chunkwise with single products and fp32 gradients
+    assert delta_bb(P(None), 32 | 512 | 4096, E) == -4         # operand pairs everywhere: accepted
+    assert delta_bb(P(None), 32 | 1024 | 4096, E) == -4        # rounded gradients: accepted
     layer_f = lambda sw, flags, os=None: L.srwm_layer_forward_f32(fake(), ok_strides, P(None), sw, sw, sw, sw,
                                                                   *[fake() for _ in range(12)], os, N, H, Ls, E, E, flags,
                                                                   P(None))

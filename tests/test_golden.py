@@ -149,6 +149,13 @@ def test_hip_stepwise_operators_match_their_fixtures():
         # so its error is that of the weights and is measured on their scale
         shift = (f_ - w.detach().repeat(N, 1, 1, 1)).cpu().numpy()
         assert np.abs(shift - g[f"final_shift{i}"]).max() < TOL * float(f_.abs().max()), i
+    # the layers' path carries the shift itself in and out of the kernel: held to the fixture on the shift's own scale
+    from self_ref_v0 import self_ref_layer_steps
+    res = self_ref_layer_steps(t(g["x"]), t(g["keep"]), *[w.detach() for w in slow], *[t(g[f"shift{i}"]) for i in range(4)],
+                               False)
+    assert rel_err(res[0].cpu().numpy(), g["out"]) < TOL
+    for i in range(4):
+        assert rel_err(res[1 + i].cpu().numpy(), g[f"final_shift{i}"]) < 5 * TOL, i
     g = np.load(STEPS_DELTA)
     leaves = [t(g[n]).requires_grad_(True) for n in ("Q", "K", "V", "beta")]
     W = t(g["W0"]).clone()

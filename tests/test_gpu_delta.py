@@ -411,6 +411,39 @@ def test_chunkwise_forward_can_leave_out_the_v_old_that_nobody_reads(shape, io):
     torch.cuda.synchronize()
     for i in range(3):
         assert torch.equal(leaves[i].grad, f[4][i]), i
+    # the extension-level functions: a forward called with the reference's eight arguments writes every row of
+    # v_old (any backward may follow), and a backward told that rows were left out refuses the modes that
+    # would read them instead of returning a wrong grad_beta
+    vold = torch.full((N, H, L, E), float("nan"), device=dev)
+    W = W0.to(dev, torch.float32).contiguous()
+    used = fast_weight.causal_dot_product_cuda(qd, kd, vd, bd, vold, torch.empty_like(vold), W,
+                                               torch.empty(N, H, L, E, device=dev, dtype=io))
+    torch.cuda.synchronize()
+    assert used & srwm_hip.FLAG_CHUNKWISE and not used & srwm_hip.FLAG_SPARSE_V_OLD and not torch.isnan(vold).any()
+    g32 = [torch.empty((N, H, L, E), device=dev) for _ in range(3)] + [torch.empty((N, H, L, 1), device=dev)]
+    sparse = srwm_hip.FLAG_SPARSE_V_OLD
+    with pytest.raises(RuntimeError, match="invalid argument"):      # step-by-step backward
+        srwm_hip.fast_weight_backward(qd, kd, vd, bd, s[0], s[1], god, s[3].clone(), *g32, flags=sparse)
+    if io == torch.bfloat16:
+        with pytest.raises(RuntimeError, match="invalid argument"):  # chunkwise, single products, fp32 gradients
+            srwm_hip.fast_weight_backward(qd, kd, vd, bd, s[0], s[1], god, s[3].clone(), *g32,
+                                          flags=srwm_hip.FLAG_CHUNKWISE | sparse)
+        # the same call on the complete v_old, poisoned where the sparse one is empty, would have read the poison
+        srwm_hip.fast_weight_backward(qd, kd, vd, bd, f[0], f[1], god, f[3].clone(), *g32, flags=srwm_hip.FLAG_CHUNKWISE)
+        torch.cuda.synchronize()
+        assert not torch.isnan(g32[3]).any()
+        gexact = [torch.empty_like(t) for t in g32]
+        srwm_hip.fast_weight_backward(qd, kd, vd, bd, s[0], s[1], god, s[3].clone(), *gexact,
+                                      flags=srwm_hip.FLAG_CHUNKWISE | srwm_hip.FLAG_EXACT_PRODUCTS | sparse)
+        torch.cuda.synchronize()
+        assert not any(torch.isnan(t).any() for t in gexact)
+        assert float((gexact[3] - g32[3]).abs().max()) < 2e-3 * float(g32[3].abs().max())
+    else:
+        srwm_hip.fast_weight_backward(qd, kd, vd, bd, s[0], s[1], god, s[3].clone(), *g32,
+                                      flags=srwm_hip.FLAG_CHUNKWISE | sparse)
+        torch.cuda.synchronize()
+        for a, b in zip(g32, f[4]):
+            assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("shape,qk,small_betas", [
@@ -577,7 +610,26 @@ def test_full_config5_properties():
                                   flags=srwm_hip.FLAG_CHUNKWISE | srwm_hip.FLAG_EXACT_PRODUCTS)
     for a, b, n in ((xq, sq, "grad_Q"), (xk, sk, "grad_K"), (xv, sv, "grad_V"), (xb, sb, "grad_beta")):
         assert (a - b).abs().max().item() < 2e-3 * b.abs().max().item(), ("exact products", n)
-    for (n_, h_) in ((0, 0), (7, 15)):
+    # the pair as the operator (and the benchmark) runs it at this size: the forward leaves out the rows of v_old
+    # that nobody reads, the backward writes grad_Q, grad_K, grad_V as bf16 itself and reads grad_beta off its
+    # second sweep -- all 128 sequences, two workgroups each
+    W4 = torch.zeros(N, H, E, E, device=dev)
+    b_vold, b_vins, b_out = new(E, f32), new(E, f32), new(E, torch.bfloat16)
+    srwm_hip.fast_weight_forward(qd, kd, vd, bd, b_vold, b_vins, W4, b_out,
+                                 flags=srwm_hip.FLAG_CHUNKWISE | srwm_hip.FLAG_SPARSE_V_OLD)
+    assert torch.equal(W4, WL) and torch.equal(b_vins, r["v_insert"]) and torch.equal(b_out, r["out"])
+    assert bool(torch.isnan(b_vold).all())   # no beta of this input is below 2^-24: not one row is written
+    bf = torch.bfloat16
+    bq, bk, bv, bb = new(E, bf), new(E, bf), new(E, bf), new(1, f32)
+    srwm_hip.fast_weight_backward(qd, kd, vd, bd, b_vold, b_vins, god, W4, bq, bk, bv, bb,
+                                  flags=srwm_hip.FLAG_CHUNKWISE | srwm_hip.FLAG_SPARSE_V_OLD)
+    torch.cuda.synchronize()
+    assert torch.equal(W4, r["W"])                       # reverted exactly as with fp32 gradients
+    assert torch.equal(bv, gv.to(bf))                    # grad_V: the fp32 result rounded, bit for bit
+    for a, b, n in ((bq, sq, "grad_Q"), (bk, sk, "grad_K"), (bb, sb, "grad_beta")):
+        assert torch.isfinite(a).all(), n
+        assert (a.float() - b).abs().max().item() < BF16_TOL * b.abs().max().item(), ("as benchmarked", n)
+    for (n_, h_) in ((0, 0), (3, 9), (7, 15)):
         sl = (slice(n_, n_ + 1), slice(h_, h_ + 1))
         base = [t[sl].float().cpu().to(torch.float64).numpy() for t in (qd, kd, vd, bd)] + [W0[sl].double().numpy()]
         of = oracle.delta_forward(*base)
@@ -586,6 +638,8 @@ def test_full_config5_properties():
         assert rel_err(r["out"][sl].float().cpu().numpy(), of["out"]) < BF16_TOL
         for t, n in ((gq, "grad_Q"), (gk, "grad_K"), (gv, "grad_V"), (gb, "grad_beta")):
             assert rel_err(t[sl].float().cpu().numpy(), ob[n]) < BF16_TOL, n
+        for t, n in ((bq, "grad_Q"), (bk, "grad_K"), (bv, "grad_V"), (bb, "grad_beta")):
+            assert rel_err(t[sl].float().cpu().numpy(), ob[n]) < BF16_TOL, ("as benchmarked", n)
 
 
 def test_chunkwise_flag_is_refused_where_there_is_no_kernel():
@@ -691,7 +745,8 @@ def test_operator_output_takes_the_layout_of_v(steps):
     transpose / reshape / transpose chain on the result is a view of a contiguous [L, N, H*M] tensor, and the
     values and gradients are those of the batch-major call."""
     print(f"case operator output layout steps={steps}", flush=True)
-    from fast_weight import fast_weight_delta, fast_weight_delta_steps
+    from fast_weight import fast_weight_delta_rows, fast_weight_delta_steps_rows
+    import fast_weight
     N, H, L, D = 2, 3, 70, 64
     q, k, v, beta, W0, go = delta_inputs(N, H, L, D, D, seed=5, qk="softmax", w0_std=0.0)
     keep = (torch.rand(N, L, generator=torch.Generator().manual_seed(1)) > 0.1).float().to(_dev())
@@ -704,7 +759,7 @@ def test_operator_output_takes_the_layout_of_v(steps):
                 t = t.permute(2, 0, 1, 3).contiguous().permute(1, 2, 0, 3)
             args.append(t.requires_grad_(True))
         W = W0.to(_dev(), torch.float32).contiguous()
-        out = fast_weight_delta_steps(*args, keep, W) if steps else fast_weight_delta(*args, W)
+        out = fast_weight_delta_steps_rows(*args, keep, W) if steps else fast_weight_delta_rows(*args, W)
         chain = out.transpose(1, 2).reshape(N, L, H * D).transpose(0, 1)
         if layout == "step-major":
             assert chain.is_contiguous() and chain.data_ptr() == out.data_ptr()
@@ -714,11 +769,16 @@ def test_operator_output_takes_the_layout_of_v(steps):
         res[layout] = [out.detach()] + [a.grad for a in args]
     for a, b in zip(res["batch-major"], res["step-major"]):
         assert torch.equal(a, b)
-    import fast_weight
-    fast_weight.OUT_LIKE_V = False        # the reference's allocation: dense whatever V looks like
+    # the drop-in operators allocate as the reference does: dense whatever V looks like, so .view() works on the result
+    assert fast_weight.OUT_LIKE_V is False
+    W = W0.to(_dev(), torch.float32).contiguous()
+    out = fast_weight.fast_weight_delta_steps(*args, keep, W) if steps else fast_weight.fast_weight_delta(*args, W)
+    assert out.is_contiguous() and torch.equal(out.view(N, H, L, D), res["batch-major"][0])
+    out.sum().backward()
+    fast_weight.OUT_LIKE_V = True         # the module switch turns the plain operators into the step-major form
     try:
         W = W0.to(_dev(), torch.float32).contiguous()
-        out = fast_weight_delta_steps(*args, keep, W) if steps else fast_weight_delta(*args, W)
-        assert out.is_contiguous() and torch.equal(out, res["batch-major"][0])
+        out = fast_weight.fast_weight_delta_steps(*args, keep, W) if steps else fast_weight.fast_weight_delta(*args, W)
+        assert not out.is_contiguous() and torch.equal(out, res["batch-major"][0])
     finally:
-        fast_weight.OUT_LIKE_V = True
+        fast_weight.OUT_LIKE_V = False

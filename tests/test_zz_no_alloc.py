@@ -12,8 +12,10 @@ import srwm_hip
 pytestmark = pytest.mark.gpu
 
 
-def _case(N, H, L, E, Y, seed, shift, generic=False):
-    """Layer forward on the GPU, then the backward through both entry points."""
+def _case(N, H, L, E, Y, seed, shift, generic=False, poison=False, check_memory=False):
+    """Layer forward on the GPU, then the backward through both entry points.  poison: the upstream gradient of the
+    no-alloc call is NaN, so every per-row gradient it leaves in the static array is NaN (nothing is compared).
+    check_memory: the no-alloc call must leave the device's free memory and torch's allocator as they were."""
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(seed)
     std = 1.0 / math.sqrt(E)
@@ -39,8 +41,18 @@ def _case(N, H, L, E, Y, seed, shift, generic=False):
     # the entry point under test: poisoned outputs, so that a skipped write shows
     gx = torch.full((N, H, L, E), float("nan"), **f32)
     gs = [torch.full((H, E, w), float("nan"), **f32) for w in (Y, E, E, 4)]
+    if poison:
+        go = torch.full_like(go, float("nan"))
+    torch.cuda.synchronize()
+    before = (torch.cuda.mem_get_info(dev)[0], torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev))
     srwm_hip.self_ref_layer_backward_noalloc(x, *saved, go, slow, *state, gx, gs, flags=base)
     torch.cuda.synchronize()
+    after = (torch.cuda.mem_get_info(dev)[0], torch.cuda.memory_allocated(dev), torch.cuda.memory_reserved(dev))
+    if check_memory:
+        assert after == before, (before, after)
+    if poison:
+        assert bool(torch.isnan(gs[0]).all())
+        return
     assert torch.isfinite(gx_ref).all() and all(torch.isfinite(t).all() for t in gs_ref)
     assert torch.equal(gx, gx_ref)
     for a, b, per_row in zip(gs, gs_ref, gW):
@@ -52,11 +64,28 @@ def _case(N, H, L, E, Y, seed, shift, generic=False):
 def test_noalloc_backward_equals_the_allocating_one_on_calls_in_a_row():
     print("case no-alloc layer backward: large, then smaller, then wide, then LDS-resident kernels", flush=True)
     _case(8, 8, 40, 32, 32, seed=1, shift=False)
-    _case(3, 4, 17, 32, 32, seed=2, shift=True)        # smaller input right after: the array still holds call 1
+    _case(8, 8, 40, 32, 32, seed=1, shift=False, check_memory=True)   # kernels loaded by now: nothing may be allocated
+    _case(8, 8, 40, 32, 32, seed=7, shift=False, poison=True)         # leaves NaN in every word the next calls reuse
+    _case(3, 4, 17, 32, 32, seed=2, shift=True, check_memory=True)    # smaller input right after: the array still holds the NaNs
     _case(2, 16, 33, 64, 64, seed=3, shift=False)      # headline head size
     _case(3, 4, 12, 32, 97, seed=4, shift=True)        # wide output block
     _case(2, 3, 9, 12, 12, seed=5, shift=False, generic=True)
     _case(1, 1, 5, 8, 8, seed=6, shift=False)          # smallest
+
+
+def test_noalloc_wrapper_copies_nothing():
+    """The Python wrapper refuses tensors it would have to copy (a copy allocates), the shared weights included."""
+    print("case no-alloc layer backward: non-contiguous shared weights", flush=True)
+    dev = torch.device("cuda:0")
+    N, H, L, E = 2, 2, 3, 8
+    z = lambda *s: torch.zeros(*s, device=dev)
+    saved = [z(N, H, L, w) for w in (E, E, 4, E, E, E, 4)]
+    state = [z(N, H, E, w) for w in (E, E, E, 4)]
+    slow = [z(H, E, w) for w in (E, E, E, 4)]
+    slow[1] = z(H, E, 2 * E)[:, :, ::2]
+    gs = [z(H, E, w) for w in (E, E, E, 4)]
+    with pytest.raises(ValueError, match="copies nothing"):
+        srwm_hip.self_ref_layer_backward_noalloc(z(N, H, L, E), *saved, z(N, H, L, E), slow, *state, z(N, H, L, E), gs)
 
 
 def test_noalloc_backward_refuses_what_does_not_fit():
