@@ -595,3 +595,61 @@ def test_layer_operator_keeps_the_row_order_of_its_input(E, wide, bf16):
             w.grad = None
     for a, b in zip(res["step-major"], res["batch-major"]):
         assert torch.equal(a, b)
+
+
+@pytest.fixture
+def no_fallback():
+    """Any call that the register-resident kernels do not take raises instead of running on the LDS-resident ones."""
+    import srwm_hip
+    srwm_hip.NO_FALLBACK = True
+    yield
+    srwm_hip.NO_FALLBACK = False
+
+
+@pytest.mark.parametrize("d", [8, 16, 32, 64])
+def test_layers_at_the_compiled_head_sizes_never_fall_back(d, no_fallback):
+    """Every operator call the layer modules make at head sizes with a register-resident instantiation -- forward,
+    backward and the step mode, narrow and wide output block, fused and spelled out -- is taken by those kernels:
+    the layouts the layers produce (step-major views, step-major outputs, rows of 3d + 1 words) must not drop a call
+    onto the several times slower LDS-resident family unnoticed."""
+    print(f"case layers without fallback d={d}", flush=True)
+    import layer
+    import srwm_hip
+    dev = _dev()
+    torch.manual_seed(d)
+    T, B, H = 6, 3, 2
+    h = torch.randn(T, B, H * d, device=dev)
+    notdone = (torch.rand(T, B, device=dev) > 0.3).float()
+    for fused in (True, False):
+        layer.FUSED_SRWM_LAYER, old = fused, layer.FUSED_SRWM_LAYER
+        try:
+            lay = layer.SRWMlayer(H, d, H * d, 0.0, use_input_softmax=True).to(dev)
+            lay(h.clone().requires_grad_(True)).sum().backward()
+            rl = layer.SRlayer(H, d, H * d, 0.0).to(dev)
+            st = tuple(torch.zeros(B, H, d, w, device=dev) for w in (d, d, d, 4))
+            out, st = rl(h.clone().requires_grad_(True), st)
+            out.sum().backward()
+            out, st = rl.forward_steps(h.clone().requires_grad_(True), notdone, st)
+            out.sum().backward()
+            sm = layer.SMFWPlayer(H, d, H * d, 0.0).to(dev)
+            st = tuple(torch.zeros(B, H, d, w, device=dev) for w in (3 * d + 1, d, d, 4, d))
+            out, st = sm(h.clone().requires_grad_(True), st)
+            out.sum().backward()
+            out, st = sm.forward_steps(h.clone().requires_grad_(True), notdone, st)
+            out.sum().backward()
+        finally:
+            layer.FUSED_SRWM_LAYER = old
+    ff = layer.FastFFlayer(H, d, H * d, 0.0).to(dev)
+    ff(h.clone().requires_grad_(True)).sum().backward()
+    cf = layer.CarryFastFFlayer(H, d, H * d, 0.0).to(dev)
+    out, mem = cf(h.clone().requires_grad_(True), torch.zeros(B, H, d, d, device=dev))
+    out.sum().backward()
+    out, mem = cf.forward_steps(h.clone().requires_grad_(True), notdone, mem)
+    out.sum().backward()
+    torch.cuda.synchronize()
+    # and the switch does what it says: a head size without an instantiation raises
+    z = lambda *s: torch.zeros(*s, device=dev)
+    with pytest.raises(RuntimeError, match="no kernel"):
+        srwm_hip.self_ref_forward(z(1, 1, 2, 1000), z(1, 1, 1000, 1000), z(1, 1, 1000, 1000), z(1, 1, 1000, 1000),
+                                  z(1, 1, 1000, 4), z(1, 1, 2, 1000), z(1, 1, 2, 1000), z(1, 1, 2, 4), z(1, 1, 2, 1000),
+                                  z(1, 1, 2, 1000), z(1, 1, 2, 1000), z(1, 1, 2, 4), z(1, 1, 2, 1000))
