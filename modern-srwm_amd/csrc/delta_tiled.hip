@@ -1,4 +1,5 @@
-// Register-resident delta-rule kernels for square memories (E == M = D in {8,16,32,64,128}).
+// Register-resident delta-rule kernels for square memories (E == M = D in {8,16,32,64,128}), which also serve any
+// fp32 E x M memory with E, M multiples of 4 up to 128 as the next such square, zero-padded (template flag PAD).
 //
 // One workgroup of NW wave64s owns one (batch, head) sequence for all L steps; the D x D
 // memory W (and its gradient G in the backward) lives in registers, cut into tiles of
@@ -105,38 +106,42 @@ __device__ __forceinline__ void wr(bf16_t *dst, const float (&src)[N]) {
 
 // One tile vector (TT steps x W elements) moved global -> registers (as fp32) -> LDS as float4s.
 // Rows past the end of the sequence are clamped to the last one: loaded, never used.
-template <int NT, int TT, int W>
+// PAD: rows in global memory hold `width` <= W elements (a multiple of 4); the threads past the end of a row
+// fetch its last four elements instead (no branch around the loads) and commit zeros.
+template <int NT, int TT, int W, bool PAD = false>
 struct TileVec {
     static constexpr int NV4 = TT * W / 4;           // float4s per tile vector
     static constexpr int LD = (NV4 + NT - 1) / NT;   // float4 loads per thread
     float4 r[LD];
     template <class TI>
-    __device__ __forceinline__ void load(const TI *base, int64_t step_stride, int t0, int L, int tid) {
+    __device__ __forceinline__ void load(const TI *base, int64_t step_stride, int t0, int L, int tid, int width = W) {
 #pragma unroll
         for (int j = 0; j < LD; ++j) {
             const int f = min(tid + j * NT, NV4 - 1);
             const int row = min(t0 + f / (W / 4), L - 1), col = (f % (W / 4)) * 4;
-            r[j] = ld4(base + (int64_t)row * step_stride + col);
+            r[j] = ld4(base + (int64_t)row * step_stride + (PAD ? min(col, width - 4) : col));
         }
     }
-    __device__ __forceinline__ void store(float *lds, int tid) const {
+    __device__ __forceinline__ void store(float *lds, int tid, int width = W) const {
 #pragma unroll
         for (int j = 0; j < LD; ++j) {
             const int f = tid + j * NT;
-            if (f < NV4) reinterpret_cast<float4 *>(lds)[f] = r[j];
+            const bool real = !PAD || (f % (W / 4)) * 4 < width;
+            if (f < NV4) reinterpret_cast<float4 *>(lds)[f] = real ? r[j] : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
 };
 
 // Stores one staged tile vector (rows x W floats in LDS) to rows of `row_stride` elements in
 // global memory, 4 elements per thread and store: consecutive lanes -> consecutive addresses.
-template <int NT, int W, class TO>
+// PAD: only the first `width` elements of a row exist in global memory.
+template <int NT, int W, bool PAD = false, class TO>
 __device__ __forceinline__ void flush_rows(const float *lds, TO *gbase, int64_t row_stride, int rows,
-                                           int tid) {
+                                           int tid, int width = W) {
     for (int f = tid; f < rows * (W / 4); f += NT) {
         const float4 v = reinterpret_cast<const float4 *>(lds)[f];
         const float a[4] = {v.x, v.y, v.z, v.w};
-        wr<4>(gbase + (int64_t)(f / (W / 4)) * row_stride + (f % (W / 4)) * 4, a);
+        if (!PAD || (f % (W / 4)) * 4 < width) wr<4>(gbase + (int64_t)(f / (W / 4)) * row_stride + (f % (W / 4)) * 4, a);
     }
 }
 
@@ -151,6 +156,7 @@ struct FwdP {
     Strided3 os;
     int N, H, L;
     const float *keep;   // optional [N,L]: zero the memory before step t where keep[n][t] == 0
+    int E, M;            // rows and columns of the memory as the caller holds it (both D unless PAD)
 };
 template <class TI>
 struct BwdP {
@@ -165,12 +171,19 @@ struct BwdP {
     float *gW;
     int N, H, L;
     unsigned grad_state_mode;
+    int E, M;            // rows and columns of the memory as the caller holds it (both D unless PAD)
 };
 
-template <class TI, int D, int MS, int NW, int R, int TT, bool RESET>
+// PAD: the caller's memory is p.E x p.M, both multiples of 4 and at most D, not both equal to it.  The kernel runs as
+// for D x D on a memory whose rows from p.E on and columns from p.M on are zero and stay zero (zero elements of k
+// never write; a zero column with a zero v reads out and inserts zero): rows of q, k are p.E long and rows of v and
+// of every output p.M long in global memory, zero-filled in LDS, and nothing is stored for the padding.
+template <class TI, int D, int MS, int NW, int R, int TT, bool RESET, bool PAD = false>
 __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) {
+    static_assert(!PAD || MS == 1, "padded sizes: one workgroup per sequence");
     using T = DTiling<D, MS, NW, R, TT>;
     constexpr int RG = T::RG, CGW = T::CGW, CC = T::CC, MC = T::MC, NT = T::NT;
+    const int Ea = PAD ? p.E : D, Ma = PAD ? p.M : D;
     enum { OVO, OVI, OOUT, NOUT };
     __shared__ __attribute__((aligned(16))) float tq[2][TT][D];
     __shared__ __attribute__((aligned(16))) float tk[2][TT][D];
@@ -194,27 +207,35 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
     const TI *kb = p.K + n * p.ks.n + h * p.ks.h;
     const TI *vb = p.V + n * p.vs.n + h * p.vs.h + m0;
     const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
-    float *Wg = p.W + seq * D * D + m0;
+    float *Wg = p.W + seq * Ea * Ma + m0;
+    const bool col_real = !PAD || c0 < Ma;   // this lane's columns exist (CC divides 4, which divides p.M: all or none)
 
     float w[R][CC];
 #pragma unroll
-    for (int i = 0; i < R; ++i) rd<CC>(w[i], Wg + (r0 + i) * D + c0);
+    for (int i = 0; i < R; ++i) {
+        if (!PAD || (r0 + i < Ea && col_real)) {
+            rd<CC>(w[i], Wg + (r0 + i) * Ma + c0);
+        } else {
+#pragma unroll
+            for (int c = 0; c < CC; ++c) w[i][c] = 0.f;
+        }
+    }
 
-    TileVec<NT, TT, D> nq, nk;
-    TileVec<NT, TT, MC> nv;
+    TileVec<NT, TT, D, PAD> nq, nk;
+    TileVec<NT, TT, MC, PAD> nv;
     float nb = 0.f, nkeep = 1.f;
     auto load_tile = [&](int tile) {
         const int t0 = tile * TT;
-        nq.load(qb, p.qs.l, t0, p.L, tid);
-        nk.load(kb, p.ks.l, t0, p.L, tid);
-        nv.load(vb, p.vs.l, t0, p.L, tid);
+        nq.load(qb, p.qs.l, t0, p.L, tid, Ea);
+        nk.load(kb, p.ks.l, t0, p.L, tid, Ea);
+        nv.load(vb, p.vs.l, t0, p.L, tid, Ma);
         nb = ld1(bb + (int64_t)min(t0 + (tid % TT), p.L - 1) * p.bs.l);
         if constexpr (RESET) nkeep = p.keep[(int64_t)n * p.L + min(t0 + (tid % TT), p.L - 1)];
     };
     auto store_tile = [&](int buf) {
-        nq.store(&tq[buf][0][0], tid);
-        nk.store(&tk[buf][0][0], tid);
-        nv.store(&tv[buf][0][0], tid);
+        nq.store(&tq[buf][0][0], tid, Ea);
+        nk.store(&tk[buf][0][0], tid, Ea);
+        nv.store(&tv[buf][0][0], tid, Ma);
         if (tid < TT) tbeta[buf][tid] = nb;
         if (RESET && tid < TT) tkeep[buf][tid] = nkeep;
     };
@@ -300,21 +321,24 @@ __global__ __launch_bounds__(NW *kWave) void delta_fwd_tiled_kernel(FwdP<TI> p) 
         }
         if (tile + 1 < ntiles) store_tile(buf ^ 1);
         __syncthreads();
-        const int64_t om = (seq * p.L + tile * TT) * D + m0;
-        flush_rows<NT, MC>(&ot[buf][OVO][0][0], p.vold + om, D, tlen, tid);
-        flush_rows<NT, MC>(&ot[buf][OVI][0][0], p.vins + om, D, tlen, tid);
-        flush_rows<NT, MC>(&ot[buf][OOUT][0][0], p.out + n * p.os.n + h * p.os.h + (int64_t)(tile * TT) * p.os.l + m0,
-                           p.os.l, tlen, tid);
+        const int64_t om = (seq * p.L + tile * TT) * Ma + m0;
+        flush_rows<NT, MC, PAD>(&ot[buf][OVO][0][0], p.vold + om, Ma, tlen, tid, Ma);
+        flush_rows<NT, MC, PAD>(&ot[buf][OVI][0][0], p.vins + om, Ma, tlen, tid, Ma);
+        flush_rows<NT, MC, PAD>(&ot[buf][OOUT][0][0], p.out + n * p.os.n + h * p.os.h + (int64_t)(tile * TT) * p.os.l + m0,
+                                p.os.l, tlen, tid, Ma);
     }
 
 #pragma unroll
-    for (int i = 0; i < R; ++i) wr<CC>(Wg + (r0 + i) * D + c0, w[i]);
+    for (int i = 0; i < R; ++i)
+        if (!PAD || (r0 + i < Ea && col_real)) wr<CC>(Wg + (r0 + i) * Ma + c0, w[i]);
 }
 
-template <class TI, int D, int MS, int NW, int R, int TT>
+template <class TI, int D, int MS, int NW, int R, int TT, bool PAD = false>
 __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) {
+    static_assert(!PAD || MS == 1, "padded sizes: one workgroup per sequence");
     using T = DTiling<D, MS, NW, R, TT>;
     constexpr int RG = T::RG, CGW = T::CGW, NCG = T::NCG, CC = T::CC, MC = T::MC, NT = T::NT;
+    const int Ea = PAD ? p.E : D, Ma = PAD ? p.M : D;   // the memory as the caller holds it, zero-padded to D x D here
     enum { CV, CVO, CVI, CGO, NCV };                                  // column-side vectors of a step
     __shared__ __attribute__((aligned(16))) float tq[2][TT][D];
     __shared__ __attribute__((aligned(16))) float tk[2][TT][D];
@@ -338,42 +362,49 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
     const TI *vb = p.V + n * p.vs.n + h * p.vs.h + m0;
     const TI *gob = p.go + n * p.gs.n + h * p.gs.h + m0;
     const TI *bb = p.beta + n * p.bs.n + h * p.bs.h;
-    const float *vob = p.vold + seq * p.L * D + m0;
-    const float *vib = p.vins + seq * p.L * D + m0;
-    float *Wg = p.W + seq * D * D + m0;
-    float *gWg = p.gW ? p.gW + seq * D * D + m0 : nullptr;
+    const float *vob = p.vold + seq * p.L * Ma + m0;
+    const float *vib = p.vins + seq * p.L * Ma + m0;
+    float *Wg = p.W + seq * Ea * Ma + m0;
+    float *gWg = p.gW ? p.gW + seq * Ea * Ma + m0 : nullptr;
     const bool g_in = gWg && p.grad_state_mode != 0u;
+    const bool col_real = !PAD || c0 < Ma;   // this lane's columns exist (all of them or none)
 
     float w[R][CC], g[R][CC];
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-        rd<CC>(w[i], Wg + (r0 + i) * D + c0);
-        if (g_in) {
-            rd<CC>(g[i], gWg + (r0 + i) * D + c0);
+        const bool real = !PAD || (r0 + i < Ea && col_real);
+        if (real) {
+            rd<CC>(w[i], Wg + (r0 + i) * Ma + c0);
+        } else {
+#pragma unroll
+            for (int c = 0; c < CC; ++c) w[i][c] = 0.f;
+        }
+        if (g_in && real) {
+            rd<CC>(g[i], gWg + (r0 + i) * Ma + c0);
         } else {
 #pragma unroll
             for (int c = 0; c < CC; ++c) g[i][c] = 0.f;
         }
     }
 
-    TileVec<NT, TT, D> nq, nk;
-    TileVec<NT, TT, MC> nc[NCV];
+    TileVec<NT, TT, D, PAD> nq, nk;
+    TileVec<NT, TT, MC, PAD> nc[NCV];
     float nb = 0.f;
     auto load_tile = [&](int tile) {
         const int t0 = tile * TT;
-        nq.load(qb, p.qs.l, t0, p.L, tid);
-        nk.load(kb, p.ks.l, t0, p.L, tid);
-        nc[CV].load(vb, p.vs.l, t0, p.L, tid);
-        nc[CVO].load(vob, D, t0, p.L, tid);
-        nc[CVI].load(vib, D, t0, p.L, tid);
-        nc[CGO].load(gob, p.gs.l, t0, p.L, tid);
+        nq.load(qb, p.qs.l, t0, p.L, tid, Ea);
+        nk.load(kb, p.ks.l, t0, p.L, tid, Ea);
+        nc[CV].load(vb, p.vs.l, t0, p.L, tid, Ma);
+        nc[CVO].load(vob, Ma, t0, p.L, tid, Ma);
+        nc[CVI].load(vib, Ma, t0, p.L, tid, Ma);
+        nc[CGO].load(gob, p.gs.l, t0, p.L, tid, Ma);
         nb = ld1(bb + (int64_t)min(t0 + (tid % TT), p.L - 1) * p.bs.l);
     };
     auto store_tile = [&](int buf) {
-        nq.store(&tq[buf][0][0], tid);
-        nk.store(&tk[buf][0][0], tid);
+        nq.store(&tq[buf][0][0], tid, Ea);
+        nk.store(&tk[buf][0][0], tid, Ea);
 #pragma unroll
-        for (int v = 0; v < NCV; ++v) nc[v].store(&tc[buf][v][0][0], tid);
+        for (int v = 0; v < NCV; ++v) nc[v].store(&tc[buf][v][0][0], tid, Ma);
         if (tid < TT) tbeta[buf][tid] = nb;
     };
 
@@ -480,10 +511,12 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
                 sq += rowq[tt][wv][e];
                 sk += rowk[tt][wv][e];
             }
-            const int64_t oe = (seq * p.L + tile * TT + tt) * D + e;
+            const int64_t oe = (seq * p.L + tile * TT + tt) * Ea + e;
             if constexpr (MS == 1) {
-                p.gQ[oe] = sq;
-                p.gK[oe] = sk;
+                if (!PAD || e < Ea) {
+                    p.gQ[oe] = sq;
+                    p.gK[oe] = sk;
+                }
             } else {
                 atomicAdd(p.gQ + oe, sq);
                 atomicAdd(p.gK + oe, sk);
@@ -499,7 +532,7 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
                 atomicAdd(p.gbeta + seq * p.L + tile * TT + tid, s);
             }
         }
-        flush_rows<NT, MC>(&gvt[0][0], p.gV + (seq * p.L + tile * TT) * D + m0, D, tlen, tid);
+        flush_rows<NT, MC, PAD>(&gvt[0][0], p.gV + (seq * p.L + tile * TT) * Ma + m0, Ma, tlen, tid, Ma);
         if (tile > 0) store_tile(buf ^ 1);
         __syncthreads();
     }
@@ -507,9 +540,10 @@ __global__ __launch_bounds__(NW *kWave) void delta_bwd_tiled_kernel(BwdP<TI> p) 
     const bool accum = gWg && p.grad_state_mode == 2u;
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-        wr<CC>(Wg + (r0 + i) * D + c0, w[i]);
+        if (PAD && !(r0 + i < Ea && col_real)) continue;
+        wr<CC>(Wg + (r0 + i) * Ma + c0, w[i]);
         if (gWg) {
-            float *d = gWg + (r0 + i) * D + c0;
+            float *d = gWg + (r0 + i) * Ma + c0;
 #pragma unroll
             for (int c = 0; c < CC; ++c) d[c] = accum ? d[c] + g[i][c] : g[i][c];
         }
@@ -524,24 +558,24 @@ __global__ void zero_fill_kernel(float *a, int64_t na, float *b, int64_t nb, flo
     for (int64_t j = i; j < nc; j += stride) c[j] = 0.f;
 }
 
-template <class TI, int D, int MS, int NW, int R, int TT>
+template <class TI, int D, int MS, int NW, int R, int TT, bool PAD = false>
 int launch_f(const FwdP<TI> &p, hipStream_t s) {
     if (p.keep)
-        hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, MS, NW, R, TT, true>), dim3(p.N * p.H * MS),
+        hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, MS, NW, R, TT, true, PAD>), dim3(p.N * p.H * MS),
                            dim3(NW * kWave), 0, s, p);
     else
-        hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, MS, NW, R, TT, false>), dim3(p.N * p.H * MS),
+        hipLaunchKernelGGL((delta_fwd_tiled_kernel<TI, D, MS, NW, R, TT, false, PAD>), dim3(p.N * p.H * MS),
                            dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
-template <class TI, int D, int MS, int NW, int R, int TT>
+template <class TI, int D, int MS, int NW, int R, int TT, bool PAD = false>
 int launch_b(const BwdP<TI> &p, hipStream_t s) {
     if (MS > 1) {
         const int64_t ne = (int64_t)p.N * p.H * p.L * D, nb = (int64_t)p.N * p.H * p.L;
         hipLaunchKernelGGL(zero_fill_kernel, dim3(1024), dim3(256), 0, s, p.gQ, ne, p.gK, ne, p.gbeta, nb);
     }
-    hipLaunchKernelGGL((delta_bwd_tiled_kernel<TI, D, MS, NW, R, TT>), dim3(p.N * p.H * MS),
+    hipLaunchKernelGGL((delta_bwd_tiled_kernel<TI, D, MS, NW, R, TT, PAD>), dim3(p.N * p.H * MS),
                        dim3(NW * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
@@ -556,11 +590,36 @@ bool ok16(const void *ptr) { return (uintptr_t)ptr % 16 == 0; }
 // Two workgroups per sequence pay off when one per sequence would leave compute units idle.
 constexpr int kSplitBelowSequences = 192;
 
+// The compiled size that serves an E x M memory: E = M = D itself, or (fp32, both multiples of 4, whose rows keep
+// their 16-byte alignment) the smallest D that holds both, run in its padded form.  0: none.
 template <class TI>
-int dispatch_fwd(const FwdP<TI> &p, int D, hipStream_t s) {
+int tiled_size_for(int E, int M, bool &pad) {
+    const int big = E > M ? E : M;
+    if (E <= 0 || M <= 0 || big > 128 || E % 4 || M % 4) return 0;
+    const int D = big <= 8 ? 8 : big <= 16 ? 16 : big <= 32 ? 32 : big <= 64 ? 64 : 128;
+    pad = E != D || M != D;
+    return (pad && sizeof(TI) != 4) ? 0 : D;
+}
+
+template <class TI>
+int dispatch_fwd(const FwdP<TI> &p, hipStream_t s) {
     if (!row_ok(p.Q, p.qs) || !row_ok(p.K, p.ks) || !row_ok(p.V, p.vs) || !ok16(p.vold) || !ok16(p.vins) ||
         !row_ok(p.out, p.os) || !ok16(p.W))
         return -1;
+    bool pad = false;
+    const int D = tiled_size_for<TI>(p.E, p.M, pad);
+    if constexpr (sizeof(TI) == 4) {
+        if (pad) {
+            switch (D) {
+                case 128: return launch_f<TI, 128, 1, 8, 16, 8, true>(p, s);
+                case 64: return launch_f<TI, 64, 1, 4, 8, 16, true>(p, s);
+                case 32: return launch_f<TI, 32, 1, 2, 4, 16, true>(p, s);
+                case 16: return launch_f<TI, 16, 1, 1, 2, 16, true>(p, s);
+                case 8: return launch_f<TI, 8, 1, 1, 1, 32, true>(p, s);
+                default: return -1;
+            }
+        }
+    }
     const bool split = p.N * p.H <= kSplitBelowSequences;
     switch (D) {
         case 128: return split ? launch_f<TI, 128, 2, 8, 8, 8>(p, s) : launch_f<TI, 128, 1, 8, 16, 8>(p, s);
@@ -573,11 +632,25 @@ int dispatch_fwd(const FwdP<TI> &p, int D, hipStream_t s) {
 }
 
 template <class TI>
-int dispatch_bwd(const BwdP<TI> &p, int D, hipStream_t s) {
+int dispatch_bwd(const BwdP<TI> &p, hipStream_t s) {
     if (!row_ok(p.Q, p.qs) || !row_ok(p.K, p.ks) || !row_ok(p.V, p.vs) || !row_ok(p.go, p.gs) ||
         !ok16(p.vold) || !ok16(p.vins) || !ok16(p.W) || !ok16(p.gV) || !ok16(p.gQ) || !ok16(p.gK) ||
         (p.gW && !ok16(p.gW)))
         return -1;
+    bool pad = false;
+    const int D = tiled_size_for<TI>(p.E, p.M, pad);
+    if constexpr (sizeof(TI) == 4) {
+        if (pad) {
+            switch (D) {
+                case 128: return launch_b<TI, 128, 1, 8, 16, 8, true>(p, s);
+                case 64: return launch_b<TI, 64, 1, 8, 4, 16, true>(p, s);
+                case 32: return launch_b<TI, 32, 1, 2, 4, 16, true>(p, s);
+                case 16: return launch_b<TI, 16, 1, 1, 2, 16, true>(p, s);
+                case 8: return launch_b<TI, 8, 1, 1, 1, 32, true>(p, s);
+                default: return -1;
+            }
+        }
+    }
     const bool split = p.N * p.H <= kSplitBelowSequences;
     switch (D) {
         case 128: return split ? launch_b<TI, 128, 2, 8, 8, 8>(p, s) : launch_b<TI, 128, 1, 8, 16, 8>(p, s);
@@ -592,31 +665,29 @@ int dispatch_bwd(const BwdP<TI> &p, int D, hipStream_t s) {
 }  // namespace
 
 int launch_delta_fwd_tiled(const DeltaFwdParams &p, hipStream_t s) {
-    if (p.E != p.M) return -1;
     const FwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.os, p.N, p.H, p.L,
-                        p.keep};
-    return dispatch_fwd(q, p.E, s);
+                        p.keep, p.E, p.M};
+    return dispatch_fwd(q, s);
 }
 
 int launch_delta_bwd_tiled(const DeltaBwdParams &p, hipStream_t s) {
-    if (p.E != p.M) return -1;
     const BwdP<float> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
-                        p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode};
-    return dispatch_bwd(q, p.E, s);
+                        p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode, p.E, p.M};
+    return dispatch_bwd(q, s);
 }
 
 int launch_delta_fwd_tiled_bf16(const DeltaFwdParamsBf16 &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const FwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.W, p.out, p.os, p.N, p.H, p.L,
-                         nullptr};
-    return dispatch_fwd(q, p.E, s);
+                         nullptr, p.E, p.M};
+    return dispatch_fwd(q, s);
 }
 
 int launch_delta_bwd_tiled_bf16(const DeltaBwdParamsBf16 &p, hipStream_t s) {
     if (p.E != p.M) return -1;
     const BwdP<bf16_t> q{p.Q, p.K, p.V, p.beta, p.qs, p.ks, p.vs, p.bs, p.vold, p.vins, p.go, p.gs, p.W,
-                         p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode};
-    return dispatch_bwd(q, p.E, s);
+                         p.gQ, p.gK, p.gV, p.gbeta, p.gW, p.N, p.H, p.L, p.grad_state_mode, p.E, p.M};
+    return dispatch_bwd(q, s);
 }
 
 }  // namespace fw

@@ -150,10 +150,15 @@ __global__ __launch_bounds__(kThreads) void delta_step_grads_kernel(DeltaStepGra
 // already hold g_t's columns; the wave's rows of x_t ride in a tile like a_t's).
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-template <int E, int M, int NWV, int CGL, bool XG>
+// PAD (square instantiations): the caller's matrix is p.E x p.M, multiples of 4 and at most E x M.  The kernel runs on
+// the matrix padded with zero rows and columns, which stay zero; rows of a, x are p.E and rows of g, b p.M long in
+// global memory, zero-filled in the tiles, and nothing is stored for the padding.
+template <int E, int M, int NWV, int CGL, bool XG, bool PAD = false>
 __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p) {
     constexpr int MP = (M + CGL - 1) / CGL * CGL;
     constexpr bool WORDS = MP != M || M % 4 != 0;   // rows of g, b fetched word by word
+    static_assert(!PAD || !WORDS, "padded sizes: rows fetched as 16-byte words");
+    const int Ea = PAD ? p.E : E, Ma = PAD ? p.M : M;
     constexpr int ER = E / NWV, RGL = kWave / CGL, R = ER / RGL, CB = MP / CGL;
     constexpr int TT = M > 64 ? 8 : (256 / ER > 16 ? 256 / ER : 16);   // steps per tile
     constexpr int NG = WORDS ? 1 : TT * M / 4 / kWave;                             // float4 per lane per tile
@@ -175,7 +180,7 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
     const float *ab = p.a + n * p.as.n + h * p.as.h + e0;
     const float *gb = p.g + n * p.gs.n + h * p.gs.h;
-    const float *bb = p.b + seq * p.L * M;
+    const float *bb = p.b + seq * p.L * Ma;
     const float *xb = XG ? p.x + n * p.xs.n + h * p.xs.h + e0 : nullptr;
 
     if constexpr (MP != M) {   // the surplus columns of the tiles stay zero: commits only write m < M
@@ -191,10 +196,11 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
         for (int i = 0; i < R; ++i)
 #pragma unroll
             for (int c = 0; c < CB; ++c)
-                w[i][c] = (src && (MP == M || c0 + c < M)) ? src[(e0 + r0 + i) * M + c0 + c] : 0.f;
+                w[i][c] = (src && (MP == M || c0 + c < M) && (!PAD || (e0 + r0 + i < Ea && c0 + c < Ma)))
+                              ? src[(e0 + r0 + i) * Ma + c0 + c] : 0.f;
     };
-    load_w(p.W0 + seq * E * M);
-    const float *wreset = p.Wreset ? p.Wreset + (int64_t)h * E * M : nullptr;
+    load_w(p.W0 + seq * Ea * Ma);
+    const float *wreset = p.Wreset ? p.Wreset + (int64_t)h * Ea * Ma : nullptr;
     // The reset value stays in registers where they suffice: fetching it inside the step loop puts a
     // wait for ALL outstanding memory operations -- the stores of u included -- into every step.
     constexpr bool WR_REGS = R * CB * (XG ? 3 : 2) <= 200;
@@ -204,7 +210,8 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
         for (int i = 0; i < R; ++i)
 #pragma unroll
             for (int c = 0; c < CB; ++c)
-                wr[i][c] = (wreset && (MP == M || c0 + c < M)) ? wreset[(e0 + r0 + i) * M + c0 + c] : 0.f;
+                wr[i][c] = (wreset && (MP == M || c0 + c < M) && (!PAD || (e0 + r0 + i < Ea && c0 + c < Ma)))
+                               ? wreset[(e0 + r0 + i) * Ma + c0 + c] : 0.f;
     }
     if (p.w0_is_shift) {
 #pragma unroll
@@ -212,7 +219,8 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
 #pragma unroll
             for (int c = 0; c < CB; ++c) {
                 if constexpr (WR_REGS) w[i][c] += wr[i][c];
-                else if (MP == M || c0 + c < M) w[i][c] += wreset[(e0 + r0 + i) * M + c0 + c];
+                else if ((MP == M || c0 + c < M) && (!PAD || (e0 + r0 + i < Ea && c0 + c < Ma)))
+                    w[i][c] += wreset[(e0 + r0 + i) * Ma + c0 + c];
             }
     }
     float xg[XG ? R : 1][XG ? CB : 1];
@@ -265,17 +273,19 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
 #pragma unroll
                 for (int i = 0; i < NG; ++i) {
                     const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
+                    const int colg = PAD ? min(col, Ma - 4) : col;   // past the end of a row: its last words, zeroed at the commit
                     const int64_t t = min(tb0 + row, p.L - 1);
-                    ng[i] = *reinterpret_cast<const v4f *>(gb + t * p.gs.l + col);
-                    nb[i] = *reinterpret_cast<const v4f *>(bb + t * M + col);
+                    ng[i] = *reinterpret_cast<const v4f *>(gb + t * p.gs.l + colg);
+                    nb[i] = *reinterpret_cast<const v4f *>(bb + t * Ma + colg);
                 }
             }
 #pragma unroll
             for (int i = 0; i < NA; ++i) {
                 const int f = min(lane + i * kWave, NAV - 1), row = f / (ER / 4), col = (f % (ER / 4)) * 4;
+                const int colg = PAD ? min(e0 + col, Ea - 4) - e0 : col;
                 const int64_t t = min(tb0 + row, p.L - 1);
-                na[i] = *reinterpret_cast<const v4f *>(ab + t * p.as.l + col);
-                if constexpr (XG) nx[i] = *reinterpret_cast<const v4f *>(xb + t * p.xs.l + col);
+                na[i] = *reinterpret_cast<const v4f *>(ab + t * p.as.l + colg);
+                if constexpr (XG) nx[i] = *reinterpret_cast<const v4f *>(xb + t * p.xs.l + colg);
             }
             if (lane < TT) {
                 const int64_t t = min(tb0 + lane, p.L - 1);
@@ -312,9 +322,10 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
             }
             group_sum_n<CGL, R>(u);
             if (cgl == 0) {
-                float *dst = p.u + (seq * p.L + t) * E + e0 + r0;
+                float *dst = p.u + (seq * p.L + t) * Ea + e0 + r0;
 #pragma unroll
-                for (int i = 0; i < R; ++i) dst[i] = u[i];
+                for (int i = 0; i < R; ++i)
+                    if (!PAD || e0 + r0 + i < Ea) dst[i] = u[i];
             }
             if constexpr (XG) {
 #pragma unroll
@@ -359,16 +370,20 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
 #pragma unroll
                 for (int i = 0; i < NG; ++i) {
                     const int f = lane + i * kWave, row = f / (M / 4), col = (f % (M / 4)) * 4;
-                    *reinterpret_cast<v4f *>(&tg[wave][row][col]) = ng[i];
-                    *reinterpret_cast<v4f *>(&tb[wave][row][col]) = nb[i];
+                    const v4f zero = {0.f, 0.f, 0.f, 0.f};
+                    const bool real = !PAD || col < Ma;
+                    *reinterpret_cast<v4f *>(&tg[wave][row][col]) = real ? ng[i] : zero;
+                    *reinterpret_cast<v4f *>(&tb[wave][row][col]) = real ? nb[i] : zero;
                 }
             }
 #pragma unroll
             for (int i = 0; i < NA; ++i) {
                 const int f = lane + i * kWave, row = f / (ER / 4), col = (f % (ER / 4)) * 4;
                 if (NAV % kWave != 0 && f >= NAV) continue;
-                *reinterpret_cast<v4f *>(&ta[wave][row][col]) = na[i];
-                if constexpr (XG) *reinterpret_cast<v4f *>(&tx[wave][row][col]) = nx[i];
+                const v4f zero = {0.f, 0.f, 0.f, 0.f};
+                const bool real = !PAD || e0 + col < Ea;
+                *reinterpret_cast<v4f *>(&ta[wave][row][col]) = real ? na[i] : zero;
+                if constexpr (XG) *reinterpret_cast<v4f *>(&tx[wave][row][col]) = real ? nx[i] : zero;
             }
             if (lane < TT) {
                 tsk[wave][0][lane] = ns;
@@ -378,27 +393,30 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
         }
     }
     if constexpr (XG) {
-        float *dst = p.xg + seq * E * M;
+        float *dst = p.xg + seq * Ea * Ma;
 #pragma unroll
         for (int i = 0; i < R; ++i)
 #pragma unroll
             for (int c = 0; c < CB; ++c)
-                if (MP == M || c0 + c < M) dst[(e0 + r0 + i) * M + c0 + c] = xg[i][c];
+                if ((MP == M || c0 + c < M) && (!PAD || (e0 + r0 + i < Ea && c0 + c < Ma)))
+                    dst[(e0 + r0 + i) * Ma + c0 + c] = xg[i][c];
     }
 }
 
-template <int E, int M, int NWV, int CGL>
+template <int E, int M, int NWV, int CGL, bool PAD = false>
 int launch_replay_tiled_as(const ReplayParams &p, hipStream_t s) {
     if (p.xg)
-        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, true>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
+        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, true, PAD>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
     else
-        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, false>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
+        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, false, PAD>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
     return (int)hipGetLastError();
 }
 
-template <int E, int NWV, int CGL>
+// square instantiation D x D for a p.E x p.M matrix that fits it: as it is, or zero-padded
+template <int D, int NWV, int CGL>
 int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
-    return launch_replay_tiled_as<E, E, NWV, CGL>(p, s);
+    if (p.E != D || p.M != D) return launch_replay_tiled_as<D, D, NWV, CGL, true>(p, s);
+    return launch_replay_tiled_as<D, D, NWV, CGL>(p, s);
 }
 
 bool rows16(const void *ptr, const Strided3 &st) {
@@ -420,8 +438,11 @@ int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
             default: return -1;
         }
     }
-    if (p.E != p.M || !rows16(p.g, p.gs) || (uintptr_t)p.b % 16 || (uintptr_t)p.u % 16) return -1;
-    switch (p.E) {
+    if (!rows16(p.g, p.gs) || (uintptr_t)p.b % 16 || (uintptr_t)p.u % 16) return -1;
+    // sizes between the compiled ones (multiples of 4, whose rows keep their alignment) run on the next square, zero-padded
+    const int big = p.E > p.M ? p.E : p.M;
+    if (p.E % 4 || p.M % 4 || big > 128) return -1;
+    switch (big <= 8 ? 8 : big <= 16 ? 16 : big <= 32 ? 32 : big <= 64 ? 64 : 128) {
         case 128: return launch_replay_tiled<128, 4, 16>(p, s);
         case 64: return launch_replay_tiled<64, 4, 8>(p, s);
         case 32: return launch_replay_tiled<32, 4, 8>(p, s);

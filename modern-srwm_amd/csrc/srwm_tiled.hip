@@ -114,9 +114,14 @@ __device__ __forceinline__ float4 row_softmax4(float4 v) {
 // sits inside the step).
 // SO: `out` is addressed through its strides (p.os_*) instead of as a dense tensor: a compile-time switch, because
 // a second set of row offsets inside the step costs the forms whose steps are shortest about 4 %.
-template <int E, int NW, int R, int XTRA, int YB, bool BF16, bool SO = (XTRA >= 1)>
+// PAD: the head size of the call, p.E, is a multiple of 4 below E.  The kernel runs as for E on a state whose rows and
+// columns from p.E on are zero and stay zero (a zero row of k never writes, a zero column of the state reads out zero):
+// rows of x and of the saved vectors are p.E long in memory and zero-filled in LDS, the padded elements enter the two
+// softmaxes as -1e30 (their q and k are exactly 0), and nothing is stored for them.
+template <int E, int NW, int R, int XTRA, int YB, bool BF16, bool SO = (XTRA >= 1), bool PAD = false>
 __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams p) {
     static_assert(XTRA >= 1 || !SO, "the plain operator's out is dense");
+    static_assert(!PAD || (SO && YB == 1), "padded head sizes: narrow output block, out through its strides");
     constexpr bool MODES = XTRA >= 1;   // p.mode: work outside the step loop only (entry / exit form of the state, input tiles)
     constexpr bool RESET = XTRA >= 2;   // p.keep: a check, and now and then a reset, inside every step
     using T = Tiling<E, NW, R>;
@@ -127,6 +132,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     constexpr bool XC = YB > 1;                       // one more y column, held like a column of w_b
     constexpr int Y = XC ? YB * E + 1 : E;            // row length of W_y, out, y_diff
     constexpr int QB = YB * CB, KB = (YB + 1) * CB;   // first lane column of the q / k block
+    const int Ea = PAD ? p.E : E, Ya = PAD ? p.E : Y; // row lengths in global memory (constants unless PAD)
+    constexpr float kPadLogit = -1e30f;               // what a padded element is to a softmax
 
     __shared__ __attribute__((aligned(16))) float xt[2][TT][E];   // input tiles, double buffered
     __shared__ float kt[2][TT];                                   // keep flags of the tile's steps
@@ -144,14 +151,16 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     const int el = lane % E;                 // softmax element == row of this thread's w_b entry
     const int jb = tid / E;                  // column of this thread's w_b entry
     const bool has_b = jb < 4;
+    const bool el_real = !PAD || el < Ea;    // not a padded element
+    const bool col_real = !PAD || c0 < Ea;   // this lane's columns exist (CB divides 4, which divides p.E: all of them or none)
     // who stores what inside a step (lane masks that stay in scalar registers across the loop)
     // (below E = 64 the first two of the four waves also carry the narrow columns: the other two store q, k and beta)
     constexpr int WQK = (E < kWave && NW >= 4 && YB == 1) ? 2 : 0;   // (no gain with the wide output block)
-    const bool st_qk = wave == WQK && lane < E, st_beta = wave == NW - 1 && lane < 4, st_exch = lane < E;
+    const bool st_qk = wave == WQK && lane < Ea, st_beta = wave == NW - 1 && lane < 4, st_exch = lane < E;
 
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
-    const int64_t sEE = seq * E * E, sEY = seq * E * Y, sE4 = seq * E * 4;
+    const int64_t sEE = seq * Ea * Ea, sEY = seq * Ea * Ya, sE4 = seq * Ea * 4;
     const float *xbase = p.x + n * p.xs_n + h * p.xs_h;
     const bool has_y = XC && jb == 0;        // thread holds row el of the last y column
 
@@ -163,22 +172,22 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const float *src = b < YB ? Wy + b * E : b == YB ? Wq : Wk;
-            const int ld = b < YB ? Y : E;
+            const int ld = b < YB ? Ya : Ea;
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < CB; ++c) {
-                    const float v = src[(r0 + i) * ld + c0 + c];
+                    const float v = (!PAD || (r0 + i < Ea && col_real)) ? src[(r0 + i) * ld + c0 + c] : 0.f;
                     w[i][b * CB + c] = ADD ? w[i][b * CB + c] + v : v;
                 }
         }
-        if (has_b) wbe = ADD ? wbe + wb[el * 4 + jb] : wb[el * 4 + jb];
+        if (has_b && el_real) wbe = ADD ? wbe + wb[el * 4 + jb] : wb[el * 4 + jb];
         if constexpr (XC) {
             if (has_y) wye = ADD ? wye + Wy[el * Y + YB * E] : Wy[el * Y + YB * E];
         }
     };
-    const float *shWy = p.sWy + (int64_t)h * E * Y, *shWq = p.sWq + (int64_t)h * E * E,
-                *shWk = p.sWk + (int64_t)h * E * E, *shwb = p.swb + (int64_t)h * E * 4;
+    const float *shWy = p.sWy + (int64_t)h * Ea * Ya, *shWq = p.sWq + (int64_t)h * Ea * Ea,
+                *shWk = p.sWk + (int64_t)h * Ea * Ea, *shwb = p.swb + (int64_t)h * Ea * 4;
     if (MODES && (p.mode & kModeFresh)) {
         load_state(shWy, shWq, shWk, shwb, std::false_type{});
     } else {
@@ -194,13 +203,14 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             const float *src = b < YB ? shWy + b * E : b == YB ? shWq : shWk;
-            const int ld = b < YB ? Y : E;
+            const int ld = b < YB ? Ya : Ea;
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
-                for (int c = 0; c < CB; ++c) w0[i][b * CB + c] = src[(r0 + i) * ld + c0 + c];
+                for (int c = 0; c < CB; ++c)
+                    w0[i][b * CB + c] = (!PAD || (r0 + i < Ea && col_real)) ? src[(r0 + i) * ld + c0 + c] : 0.f;
         }
-        if (has_b) wbe0 = shwb[el * 4 + jb];
+        if (has_b && el_real) wbe0 = shwb[el * 4 + jb];
         if constexpr (XC) {
             if (has_y) wye0 = shWy[el * Y + YB * E];
         }
@@ -224,7 +234,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 #pragma unroll
                 for (int c = 0; c < CB; ++c) *at32(base, row + (unsigned)(b * E + c0 + c)) = v[b * CB + c];
         } else {
-            store_vec<CB>(at32(base, row + (unsigned)c0), v);
+            if (col_real) store_vec<CB>(at32(base, row + (unsigned)c0), v);
         }
     };
 
@@ -233,6 +243,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     const uint16_t *xbase16 = reinterpret_cast<const uint16_t *>(p.x) + n * p.xs_n + h * p.xs_h;
     auto load_tile = [&](int tile) -> float4 {
         const int t = min(tile * TT + ld_row, p.L - 1);  // rows past the end: loaded, never used
+        if (PAD && ld_col >= Ea) {   // past the end of the row: nothing to the readouts, nothing to a softmax of the input
+            const float v = softmax_x ? kPadLogit : 0.f;
+            return make_float4(v, v, v, v);
+        }
         if (bf16_io) return bf16x4_to_f32(*reinterpret_cast<const uint2 *>(xbase16 + t * p.xs_l + ld_col));
         return *reinterpret_cast<const float4 *>(xbase + t * p.xs_l + ld_col);
     };
@@ -242,10 +256,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     // outputs of this sequence: uniform bases, 32-bit offsets per step.  `out` has strides of its own where SO.
     const int64_t out_0 = SO ? n * p.os_n + h * p.os_h : seq * p.L * Y;
     const unsigned out_l = SO ? (unsigned)p.os_l : (unsigned)Y;
-    float *const out_s = p.out + out_0, *const ydiff_s = p.ydiff + seq * p.L * Y;
+    float *const out_s = p.out + out_0, *const ydiff_s = p.ydiff + seq * p.L * Ya;
     uint16_t *const out16_s = reinterpret_cast<uint16_t *>(p.out) + out_0;
-    float *const q_s = p.q + seq * p.L * E, *const k_s = p.k + seq * p.L * E;
-    float *const qdiff_s = p.qdiff + seq * p.L * E, *const kdiff_s = p.kdiff + seq * p.L * E;
+    float *const q_s = p.q + seq * p.L * Ea, *const k_s = p.k + seq * p.L * Ea;
+    float *const qdiff_s = p.qdiff + seq * p.L * Ea, *const kdiff_s = p.kdiff + seq * p.L * Ea;
     float *const beta_s = p.beta + seq * p.L * 4, *const bdiff_s = p.bdiff + seq * p.L * 4;
     const int ntiles = (p.L + TT - 1) / TT;
     // Below E = 64 (one wave per SIMD, nothing to hide an LDS round trip behind) the input rows of a step
@@ -308,7 +322,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
                 for (int b = 0; b < YB; ++b)
 #pragma unroll
                     for (int c = 0; c < CB; ++c)
-                        *at32(out16_s, oy + (unsigned)(b * E + c0 + c)) = f32_to_bf16_bits(acc[b * CB + c]);
+                        if (col_real) *at32(out16_s, oy + (unsigned)(b * E + c0 + c)) = f32_to_bf16_bits(acc[b * CB + c]);
             } else {
                 store_y(out_s, oy, &acc[0]);
             }
@@ -364,7 +378,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         const int par = parity_of(PAR);
         const auto PNEXT = parity_flipped(PAR);
         const int t1 = t + 1;
-        const unsigned o = t * E, oy = t * Y, ob = t * 4;   // unsigned: uniform base + 32-bit lane offset addressing
+        const unsigned o = t * Ea, oy = t * Ya, ob = t * 4;   // unsigned: uniform base + 32-bit lane offset addressing
         const unsigned oo1 = SO ? (unsigned)t1 * out_l : oy + Y;   // row of step t + 1 in `out`
         const int b1 = (t1 / TT) & 1, r1 = t1 % TT;   // where x of step t+1 sits (stale rows past the end: never published)
         const bool have_next = t1 < p.L;
@@ -381,6 +395,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         } else {
             qraw = rawv[par][0][el], kraw = rawv[par][1][el], braw = rawv[par][2][lane & 3];
         }
+        if (PAD && !el_real) qraw = kraw = kPadLogit;
         float e[NC];
 #pragma unroll
         for (int c = 0; c < NC; ++c) e[c] = 0.f;
@@ -463,8 +478,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
         }
         const float pbd = s[0], kx = s[1];
         store_y(ydiff_s, oy, &dif[0]);   // by all RG lanes of the column group, like the readout
-        store_vec<CB>(at32(qdiff_s, o + (unsigned)c0), &dif[QB]);
-        store_vec<CB>(at32(kdiff_s, o + (unsigned)c0), &dif[KB]);
+        if (col_real) {
+            store_vec<CB>(at32(qdiff_s, o + (unsigned)c0), &dif[QB]);
+            store_vec<CB>(at32(kdiff_s, o + (unsigned)c0), &dif[KB]);
+        }
         if (has_b && el == 0) *at32(bdiff_s, ob + jb) = pbd;
         if constexpr (XC) {
             if (has_y && el == 0) *at32(ydiff_s, oy + YB * E) = s[3];
@@ -537,16 +554,16 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
     for (int b = 0; b < NB; ++b) {
         float *dst = b < YB ? p.Wy + sEY + b * E : b == YB ? p.Wq + sEE : p.Wk + sEE;
         const float *base = b < YB ? shWy + b * E : b == YB ? shWq : shWk;
-        const int ld = b < YB ? Y : E;
+        const int ld = b < YB ? Ya : Ea;
 #pragma unroll
         for (int i = 0; i < R; ++i)
 #pragma unroll
             for (int c = 0; c < CB; ++c) {
                 const int o = (r0 + i) * ld + c0 + c;
-                dst[o] = as_shift ? w[i][b * CB + c] - base[o] : w[i][b * CB + c];
+                if (!PAD || (r0 + i < Ea && col_real)) dst[o] = as_shift ? w[i][b * CB + c] - base[o] : w[i][b * CB + c];
             }
     }
-    if (has_b) p.wb[sE4 + el * 4 + jb] = as_shift ? wbe - shwb[el * 4 + jb] : wbe;
+    if (has_b && el_real) p.wb[sE4 + el * 4 + jb] = as_shift ? wbe - shwb[el * 4 + jb] : wbe;
     if constexpr (XC) {
         if (has_y) p.Wy[sEY + el * Y + YB * E] = as_shift ? wye - shWy[el * Y + YB * E] : wye;
     }
@@ -567,8 +584,13 @@ __global__ __launch_bounds__(NW *kWave) void srwm_fwd_tiled_kernel(SrwmFwdParams
 // the tile one step ahead.
 // The seven per-step vectors and beta are streamed through a single LDS tile of TT steps;
 // the next tile is fetched into registers one tile ahead.
-template <int E, int NW, int R, int YB>
-__global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams p) {
+// PAD: p.E is a multiple of 4 below E; as in the forward, the state and its gradient are zero from row / column p.E on
+// and stay so (the padded elements of x, q, k and of every saved vector are zero in LDS), and nothing is stored for them.
+// (the padded form at E = 64 is held to two waves per SIMD: its few extra address registers would otherwise push it
+// over half of the register file, and one wave per SIMD costs half the speed)
+template <int E, int NW, int R, int YB, bool PAD = false>
+__global__ __launch_bounds__(NW *kWave, (PAD && E == 64) ? 2 : 1) void srwm_bwd_tiled_kernel(SrwmBwdParams p) {
+    static_assert(!PAD || YB == 1, "padded head sizes: narrow output block");
     using T = Tiling<E, NW, R>;
     constexpr int RG = T::RG, CGW = T::CGW, NCG = T::NCG, CB = T::CB, TT = T::TT, NT = T::NT;
     static_assert(RG == 8, "row-sum reduction assumes column groups 8 lanes apart");
@@ -579,6 +601,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     constexpr int QB = YB * CB, KB = (YB + 1) * CB;   // first lane column of the q / k block
     constexpr int NXS = XC ? 5 : 4;                   // narrow columns: w_b and the last y column
     constexpr int NWL = XC ? (TT * Y + NT - 1) / NT : 1;   // words per thread of a wide tile
+    const int Ea = PAD ? p.E : E, Ya = PAD ? p.E : Y;      // row lengths in global memory (constants unless PAD)
     enum { VX, VQ, VK, VQD, VKD, NVEC };
 
     __shared__ __attribute__((aligned(16))) float tl[NVEC][TT][E];  // per-step vectors of the tile
@@ -636,6 +659,8 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     const int el = lane % E;
     const int jb = tid / E;
     const bool has_b = jb < 4;
+    const bool el_real = !PAD || el < Ea;    // not a padded element
+    const bool col_real = !PAD || c0 < Ea;   // this lane's columns exist (all of them or none)
     // a wave's reduce-scattered row sums (rows r0 .. r0 + R - 1) into its slots
     const auto put_rows = [&](const float(&v)[R], const int pp, const int which) {
         if constexpr (HT) stride8_reduce_scatter<R, NW>(v, &rowmT[pp][which][r0][wave], lane);
@@ -644,34 +669,35 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 
     const int64_t seq = blockIdx.x;
     const int n = (int)(seq / p.H), h = (int)(seq % p.H);
-    const int64_t sEE = seq * E * E, sEY = seq * E * Y, sE4 = seq * E * 4;
+    const int64_t sEE = seq * Ea * Ea, sEY = seq * Ea * Ya, sE4 = seq * Ea * 4;
     const float *xbase = p.x + n * p.xs_n + h * p.xs_h;
     const float *gobase = p.go + n * p.gs_n + h * p.gs_h;
     const bool has_y = XC && jb == 0;        // thread holds row el of the last y column
 
     // the final state; given as its shift from the head's shared weights when the caller keeps it so
     const bool as_shift = p.mode & kModeShift;
-    const float *shWy = p.sWy + (int64_t)h * E * Y, *shWq = p.sWq + (int64_t)h * E * E,
-                *shWk = p.sWk + (int64_t)h * E * E, *shwb = p.swb + (int64_t)h * E * 4;
+    const float *shWy = p.sWy + (int64_t)h * Ea * Ya, *shWq = p.sWq + (int64_t)h * Ea * Ea,
+                *shWk = p.sWk + (int64_t)h * Ea * Ea, *shwb = p.swb + (int64_t)h * Ea * 4;
     float w[R][NC], g[R][NC];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         const float *src = b < YB ? p.Wy + sEY + b * E : b == YB ? p.Wq + sEE : p.Wk + sEE;
         const float *base = b < YB ? shWy + b * E : b == YB ? shWq : shWk;
         const float *gsrc = b < YB ? p.gWy + sEY + b * E : b == YB ? p.gWq + sEE : p.gWk + sEE;
-        const int ld = b < YB ? Y : E;
+        const int ld = b < YB ? Ya : Ea;
 #pragma unroll
         for (int i = 0; i < R; ++i)
 #pragma unroll
             for (int c = 0; c < CB; ++c) {
                 const int o = (r0 + i) * ld + c0 + c;
-                w[i][b * CB + c] = as_shift ? src[o] + base[o] : src[o];
-                g[i][b * CB + c] = p.grad_state_mode ? gsrc[o] : 0.f;
+                const bool real = !PAD || (r0 + i < Ea && col_real);
+                w[i][b * CB + c] = !real ? 0.f : as_shift ? src[o] + base[o] : src[o];
+                g[i][b * CB + c] = (real && p.grad_state_mode) ? gsrc[o] : 0.f;
             }
     }
-    float wbe = has_b ? p.wb[sE4 + el * 4 + jb] : 0.f;
-    if (has_b && as_shift) wbe += shwb[el * 4 + jb];
-    float gbe = (has_b && p.grad_state_mode) ? p.gwb[sE4 + el * 4 + jb] : 0.f;
+    float wbe = (has_b && el_real) ? p.wb[sE4 + el * 4 + jb] : 0.f;
+    if (has_b && el_real && as_shift) wbe += shwb[el * 4 + jb];
+    float gbe = (has_b && el_real && p.grad_state_mode) ? p.gwb[sE4 + el * 4 + jb] : 0.f;
     float wye = 0.f, gye = 0.f;
     if constexpr (XC) {
         wye = has_y ? p.Wy[sEY + el * Y + YB * E] : 0.f;
@@ -684,6 +710,10 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
     const uint16_t *gobase16 = reinterpret_cast<const uint16_t *>(p.go) + n * p.gs_n + h * p.gs_h;
 
     const int ld_row = tid / (E / 4), ld_col = (tid % (E / 4)) * 4;
+    // PAD: the threads whose four elements lie past the end of a row fetch the row's last four instead (no branch
+    // around the loads) and commit zeros to the tile
+    const bool ld_real = !PAD || ld_col < Ea;
+    const int ld_colg = PAD ? min(ld_col, Ea - 4) : ld_col;   // column of the fetch in global memory
     // next tile, staged in registers
     float4 n_x, n_go, n_q, n_k, n_yd, n_qd, n_kd, n_bt, n_bd;
     float n_ydw[NWL], n_gow[NWL];   // wide rows start at any word: fetched word by word
@@ -691,13 +721,13 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 #define SRWM_BWD_LOAD_TILE(tile_)                                                                  \
     do { /* rows past the end of the sequence are clamped: they are loaded but never used */       \
         const int t_ = min((tile_) * TT + ld_row, p.L - 1);                                        \
-        const int64_t o_ = (seq * p.L + t_) * E + ld_col;                                          \
+        const int64_t o_ = (seq * p.L + t_) * Ea + ld_colg;                                        \
         if (bf16_io) { /* raw bits: widened when the tile is committed, so the fetch is not waited for */ \
-            const uint2 u_ = *reinterpret_cast<const uint2 *>(xbase16 + t_ * p.xs_l + ld_col);     \
+            const uint2 u_ = *reinterpret_cast<const uint2 *>(xbase16 + t_ * p.xs_l + ld_colg);    \
             n_x.x = __uint_as_float(u_.x);                                                         \
             n_x.y = __uint_as_float(u_.y);                                                         \
         } else {                                                                                   \
-            n_x = *reinterpret_cast<const float4 *>(xbase + t_ * p.xs_l + ld_col);                 \
+            n_x = *reinterpret_cast<const float4 *>(xbase + t_ * p.xs_l + ld_colg);                \
         }                                                                                          \
         n_q = *reinterpret_cast<const float4 *>(p.q + o_);                                         \
         n_k = *reinterpret_cast<const float4 *>(p.k + o_);                                         \
@@ -718,11 +748,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
             }                                                                                      \
         } else {                                                                                   \
             if (bf16_io) {                                                                         \
-                const uint2 u_ = *reinterpret_cast<const uint2 *>(gobase16 + t_ * p.gs_l + ld_col); \
+                const uint2 u_ = *reinterpret_cast<const uint2 *>(gobase16 + t_ * p.gs_l + ld_colg); \
                 n_go.x = __uint_as_float(u_.x);                                                    \
                 n_go.y = __uint_as_float(u_.y);                                                    \
             } else {                                                                               \
-                n_go = *reinterpret_cast<const float4 *>(gobase + t_ * p.gs_l + ld_col);           \
+                n_go = *reinterpret_cast<const float4 *>(gobase + t_ * p.gs_l + ld_colg);          \
             }                                                                                      \
             n_yd = *reinterpret_cast<const float4 *>(p.ydiff + o_);                                \
         }                                                                                          \
@@ -733,6 +763,11 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 #define SRWM_BWD_STORE_TILE()                                                                      \
     do {                                                                                           \
         if (bf16_io) n_x = bf16x4_to_f32(make_uint2(__float_as_uint(n_x.x), __float_as_uint(n_x.y))); \
+        if (PAD && !ld_real) { /* past the end of the rows: zeros; nothing to a softmax of the input */ \
+            const float px_ = softmax_x ? -1e30f : 0.f;                                            \
+            n_x = make_float4(px_, px_, px_, px_);                                                 \
+            n_q = n_k = n_qd = n_kd = n_go = n_yd = make_float4(0.f, 0.f, 0.f, 0.f);               \
+        }                                                                                          \
         *reinterpret_cast<float4 *>(&tl[VX][ld_row][ld_col]) = softmax_x ? row_softmax4<E>(n_x) : n_x; \
         *reinterpret_cast<float4 *>(&tl[VQ][ld_row][ld_col]) = n_q;                                \
         *reinterpret_cast<float4 *>(&tl[VK][ld_row][ld_col]) = n_k;                                \
@@ -771,7 +806,7 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
         if ((unsigned)e < (unsigned)E) {
             float s = row_total(pp, 2, e);
             if (softmax_x) s = xs * (s - group_sum<E>(s * xs));   // the E threads are whole lane groups
-            gx_s[(int64_t)t * p.gxs_l + e] = s;
+            if (!PAD || e < Ea) gx_s[(int64_t)t * p.gxs_l + e] = s;
         }
     };
     float xb_prev = 0.f;
@@ -1071,16 +1106,16 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 #pragma unroll
         for (int b = 0; b < NB; ++b) {
             float *dst = b < YB ? p.gWy + sEY + b * E : b == YB ? p.gWq + sEE : p.gWk + sEE;
-            const int ld = b < YB ? Y : E;
+            const int ld = b < YB ? Ya : Ea;
 #pragma unroll
             for (int i = 0; i < R; ++i)
 #pragma unroll
                 for (int c = 0; c < CB; ++c) {
                     float *d = &dst[(r0 + i) * ld + c0 + c];
-                    *d = accum ? *d + g[i][b * CB + c] : g[i][b * CB + c];
+                    if (!PAD || (r0 + i < Ea && col_real)) *d = accum ? *d + g[i][b * CB + c] : g[i][b * CB + c];
                 }
         }
-        if (has_b) {
+        if (has_b && el_real) {
             float *d = &p.gwb[sE4 + el * 4 + jb];
             *d = accum ? *d + gbe : gbe;
         }
@@ -1095,7 +1130,14 @@ __global__ __launch_bounds__(NW *kWave) void srwm_bwd_tiled_kernel(SrwmBwdParams
 
 template <int E, int NW, int R, int YB = 1>
 int launch_bwd(const SrwmBwdParams &p, hipStream_t s) {
-    hipLaunchKernelGGL((srwm_bwd_tiled_kernel<E, NW, R, YB>), dim3(p.N * p.H), dim3(NW * kWave), 0, s, with_out_strides(p));
+    const dim3 grid(p.N * p.H), block(NW * kWave);
+    if constexpr (YB == 1) {
+        if (p.E != E) {   // a head size below E: the padded form
+            hipLaunchKernelGGL((srwm_bwd_tiled_kernel<E, NW, R, 1, true>), grid, block, 0, s, with_out_strides(p));
+            return (int)hipGetLastError();
+        }
+    }
+    hipLaunchKernelGGL((srwm_bwd_tiled_kernel<E, NW, R, YB>), grid, block, 0, s, with_out_strides(p));
     return (int)hipGetLastError();
 }
 
@@ -1103,6 +1145,17 @@ template <int E, int NW, int R, int YB = 1>
 int launch_fwd(const SrwmFwdParams &p0, hipStream_t s) {
     const dim3 grid(p0.N * p0.H), block(NW * kWave);
     const SrwmFwdParams p = with_out_strides(p0);
+    if constexpr (YB == 1) {
+        if (p.E != E) {   // a head size below E: the padded forms, all of which write out through its strides
+            if (p.mode & kModeBf16)
+                hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, 1, true, true, true>), grid, block, 0, s, p);
+            else if (p.keep)
+                hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 2, 1, false, true, true>), grid, block, 0, s, p);
+            else
+                hipLaunchKernelGGL((srwm_fwd_tiled_kernel<E, NW, R, 1, 1, false, true, true>), grid, block, 0, s, p);
+            return (int)hipGetLastError();
+        }
+    }
     // the plain operator's kernel and the dense form of the one with resets write a dense out
     const bool strided_out = p.os_n != (int64_t)p.H * p.L * p.Y || p.os_h != (int64_t)p.L * p.Y || p.os_l != p.Y;
     if (p.mode & kModeBf16)
@@ -1120,6 +1173,13 @@ int launch_fwd(const SrwmFwdParams &p0, hipStream_t s) {
 
 bool aligned16(const void *ptr, int64_t a, int64_t b, int64_t c) {
     return ((uintptr_t)ptr % 16 == 0) && a % 4 == 0 && b % 4 == 0 && c % 4 == 0;
+}
+
+// The compiled head size that serves a head size E with the narrow output block: E itself, or (for multiples of 4,
+// whose rows keep their 16-byte alignment) the next one above it, run in its padded form.  0: none.
+int tiled_size_for(int E) {
+    if (E <= 0 || E > 64 || E % 4) return 0;
+    return E <= 8 ? 8 : E <= 16 ? 16 : E <= 32 ? 32 : 64;
 }
 
 }  // namespace
@@ -1143,7 +1203,7 @@ int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
         }
     }
     if (p.Y != p.E) return -1;
-    switch (p.E) {
+    switch (tiled_size_for(p.E)) {
         case 64: return launch_fwd<64, 4, 16>(p, s);
         case 32: return launch_fwd<32, 4, 4>(p, s);
         case 16: return launch_fwd<16, 1, 2>(p, s);
@@ -1167,7 +1227,7 @@ int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s) {
         }
     }
     if (p.Y != p.E || (uintptr_t)p.ydiff % 16 || !aligned16(p.go, p.gs_n, p.gs_h, p.gs_l)) return -1;
-    switch (p.E) {
+    switch (tiled_size_for(p.E)) {
         case 64: return launch_bwd<64, 4, 8>(p, s);
         case 32: return launch_bwd<32, 4, 4>(p, s);
         case 16: return launch_bwd<16, 1, 2>(p, s);

@@ -131,7 +131,7 @@ def test_argument_validation_needs_no_gpu():
     assert srwm_f(fake(), ok_strides, N, E, 32) == -1          # the chunkwise flag means nothing to the SRWM
     assert srwm_f(fake(), ok_strides, N, E, 1 << 20) == -1     # unknown flag bit
     assert srwm_f(fake(), ok_strides, N, E, 16 | 8192) == -1   # the LDS-resident kernels asked for and forbidden at once
-    assert srwm_f(fake(), ok_strides, N, 24, 8192) == -4       # SRWM_ENOKERNEL: no register-resident kernel for E = 24, and no fallback wanted
+    assert srwm_f(fake(), ok_strides, N, 6, 8192) == -4        # SRWM_ENOKERNEL: no register-resident kernel serves E = 6, and no fallback wanted
     assert srwm_f(P(0x1004), ok_strides, N, E, 8192) == -4     # nor for a base that is not 16-byte aligned
     assert srwm_f(fake(), huge, N, E, 0) == -3                 # SRWM_ESTRIDE: extent overflows the 2^40 bound
     assert srwm_f(fake(), ok_strides, N, 4096, 0) == -2        # SRWM_ESIZE: 4096 x 12292 floats fit no CU

@@ -52,7 +52,9 @@ def run_hip(q, k, v, beta, W0, go, flags=0, grad_state=None, want_grad_W=False):
     ((2, 3, 50, 16, 16), "softmax", 0.3),
     ((2, 2, 40, 32, 32), "l2", 0.0),
     ((1, 4, 300, 128, 128), "l2", 0.0),     # benchmark configuration 5's state size, fp32 I/O, short
-    ((2, 3, 17, 8, 12), "l2", 0.5),          # E != M -> generic kernel
+    ((2, 3, 17, 8, 12), "l2", 0.5),          # E != M: the 16 x 16 kernel on a padded memory
+    ((2, 2, 40, 96, 96), "l2", 0.1),         # between the compiled sizes: the 128 x 128 kernel
+    ((1, 2, 23, 6, 10), "softmax", 0.4),     # not multiples of 4: LDS-resident kernels
     ((2, 2, 1, 16, 16), "softmax", 0.2),     # L = 1
 ])
 def test_matches_fp64_oracle(shape, qk, w0, flags):
@@ -70,6 +72,36 @@ def test_matches_fp64_oracle(shape, qk, w0, flags):
                        max(1e-30, np.abs(of["W"]).max()))
     bad = {n: e for n, e in errs.items() if not (e < TOL)}
     assert not bad, f"over tolerance {TOL}: {bad}  (all: {errs})"
+
+
+@pytest.fixture
+def no_fallback():
+    """Any call that the register-resident kernels do not take raises instead of running on the LDS-resident ones."""
+    import srwm_hip
+    srwm_hip.NO_FALLBACK = True
+    yield
+    srwm_hip.NO_FALLBACK = False
+
+
+@pytest.mark.parametrize("E,M", [(12, 12), (24, 24), (40, 40), (48, 48), (96, 96), (112, 112), (4, 4), (8, 12), (32, 64),
+                                 (64, 32), (100, 36), (20, 128), (16, 4)])
+def test_sizes_between_the_compiled_ones_run_on_the_register_resident_kernels(E, M, no_fallback):
+    """Any memory of E x M with both multiples of 4 up to 128 is served by the next compiled square on a zero-padded
+    memory (not by the several times slower LDS-resident kernels): operator with the gradient of the memory in all
+    modes, strided views as the layers pass them, and the step mode with resets."""
+    print(f"case padded delta E={E} M={M}", flush=True)
+    import srwm_hip
+    test_matches_fp64_oracle((2, 3, 37, E, M), "softmax" if E % 8 else "l2", 0.3, 0)
+    q, k, v, beta, W0, go = delta_inputs(2, 2, 21, E, M, seed=4, w0_std=0.4)
+    gs = torch.randn(W0.shape, generator=torch.Generator().manual_seed(5), dtype=torch.float64)
+    base = [t.numpy() for t in (q, k, v, beta, W0)]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, go.numpy(), grad_state=gs.numpy())
+    _, b = run_hip(q, k, v, beta, W0, go, 0, grad_state=gs)
+    for n in ("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W"):
+        assert rel_err(b[n].cpu().numpy(), ob[n]) < TOL, n
+    test_stepwise_operator_matches_the_per_step_reference((2, 2, 25, E, M), True, False)
+    test_stepwise_operator_matches_the_per_step_reference((2, 2, 25, E, M), True, True)
 
 
 @pytest.mark.parametrize("flags", KERNELS)

@@ -79,12 +79,58 @@ KERNELS = [pytest.param(0, id="default"), pytest.param(16, id="generic")]
     ((1, 3, 7, 5), 0.8, False, True),                  # odd head size -> generic kernel
     ((2, 2, 1, 16), 0.3, True, True),                  # L = 1 (how the RL actors call it)
     ((1, 2, 33, 64), 0.1, True, True),                 # E = 64 with a stronger state
-    ((1, 1, 40, 12), 0.4, False, True),                # E not a power of two
+    ((1, 1, 40, 12), 0.4, False, True),                # E not a power of two: the E = 16 kernel on a padded state
+    ((2, 3, 37, 24), 0.2, True, True),                 # ... the E = 32 kernel
+    ((1, 2, 70, 48), 0.1, False, True),                # ... the E = 64 kernel
+    ((2, 2, 45, 40), 0.02, False, False),
+    ((1, 2, 9, 4), 0.7, True, True),
+    ((1, 1, 13, 20), 0.3, False, True),
+    ((1, 2, 21, 60), 0.1, True, True),
+    ((1, 1, 19, 36), 0.15, False, True),
+    ((1, 2, 11, 6), 0.5, True, True),                  # not a multiple of 4: LDS-resident kernels
 ])
 def test_matches_fp64_oracle(shape, w_std, xsm, per_batch, flags):
     print(f"case shape={shape} w_std={w_std} flags={flags}", flush=True)
     x, W, go = srwm_inputs(*shape, seed=0, w_std=w_std, x_softmax=xsm, per_batch_state=per_batch)
     check_against_oracle(x, W, go, flags)
+
+
+@pytest.fixture
+def no_fallback():
+    """Any call that the register-resident kernels do not take raises instead of running on the LDS-resident ones."""
+    import srwm_hip
+    srwm_hip.NO_FALLBACK = True
+    yield
+    srwm_hip.NO_FALLBACK = False
+
+
+@pytest.mark.parametrize("E", [4, 12, 20, 24, 28, 36, 40, 44, 48, 52, 56, 60])
+def test_head_sizes_between_the_compiled_ones_run_on_the_register_resident_kernels(E, no_fallback):
+    """Every multiple of 4 up to 64 is served by the next compiled size on a zero-padded state (not by the several
+    times slower LDS-resident kernels): plain operator with all grad-state modes and strided views, the layer
+    operator (shared weights, shift, softmax of the input, strided out), and bf16 input / output."""
+    print(f"case padded head size E={E}", flush=True)
+    x, W, go = srwm_inputs(2, 3, 37, E, seed=E, w_std=0.5 / math.sqrt(E), x_softmax=bool(E % 8), per_batch_state=True)
+    check_against_oracle(x, W, go, 0)
+    import srwm_hip
+    g = torch.Generator().manual_seed(7)
+    gs = [torch.randn(w.shape, generator=g, dtype=torch.float64) for w in W]
+    of = oracle.srwm_forward(x.numpy(), *[w.numpy() for w in W])
+    ob = oracle.srwm_backward(x.numpy(), of, go.numpy(), grad_state=[s.numpy() for s in gs])
+    _, b_in = run_hip(x, W, go, 0, grad_state=gs, mode=srwm_hip.GRAD_STATE_IN)
+    _, b_acc = run_hip(x, W, go, 0, grad_state=gs, mode=srwm_hip.GRAD_STATE_ACCUM)
+    assert rel_err(b_in["grad_x"].cpu().numpy(), ob["grad_x"]) < TOL
+    for n, s_ in zip(("grad_W_y", "grad_W_q", "grad_W_k", "grad_w_b"), gs):
+        assert rel_err(b_in[n].cpu().numpy(), ob[n]) < TOL, n
+        assert rel_err(b_acc[n].cpu().numpy(), ob[n] + s_.numpy()) < TOL, n
+    test_fused_layer_operator_matches_fp64_autograd((2, 3, 14, E), E, False, False)
+    test_fused_layer_operator_matches_fp64_autograd((2, 3, 14, E), E, False, True)
+    test_bf16_fused_layer_operator((2, 3, 9, E), E)
+    test_bf16_io_matches_the_oracle_on_the_rounded_inputs((2, 2, 9, E), 0.5 / math.sqrt(E), True, None, 0)
+    # the step mode: forward with resets, replay of the y block, the layers' form of both
+    test_stepwise_operator_matches_the_per_step_reference((3, 2, 20, E), True)
+    test_stepwise_layer_operator_matches_the_per_step_reference((2, 2, 21, E), None, True, True)
+    test_stepwise_layer_operator_matches_the_per_step_reference((2, 1, 9, E), None, False, False)
 
 
 @pytest.mark.parametrize("flags", KERNELS)
