@@ -439,6 +439,40 @@ def measure_lds_peak(dev):
     return best
 
 
+LATENCY_PROBES = ("v_fma_f32", "v_add_f32 dpp row_shr", "v_exp_f32 + v_mul_f32", "v_rcp_f32",
+                  "ds_write_b32 -> wave fence -> ds_read_b32", "ds_read_b128, address from the previous read",
+                  "ds_write_b32 -> s_barrier -> ds_read_b32 (4 waves)", "s_barrier (4 waves)",
+                  "v_permlane32_swap + v_add_f32 + v_mul_f32", "v_readlane_b32 -> v_fma_f32 (scalar operand) + v_mul_f32")
+
+
+def measure_latencies(dev, iters=200):
+    """Shader-clock ticks per dependent operation, one wave per SIMD (the library's latency probe): what the serial
+    chain of a recurrence step is made of.  Returns {name: ticks per operation, slowest of the four waves}."""
+    import ctypes
+    import torch
+    import srwm_hip
+    L = srwm_hip.lib()
+    L.srwm_hip_latency_probe.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                         ctypes.POINTER(ctypes.c_int)]
+    L.srwm_hip_latency_probe.restype = ctypes.c_int
+    cyc = torch.zeros(4, dtype=torch.int64, device=dev)
+    sink = torch.zeros(256, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+    out = {}
+    for which, name in enumerate(LATENCY_PROBES):
+        ops = ctypes.c_int()
+        best = None
+        for rep in range(3):
+            if L.srwm_hip_latency_probe(ctypes.c_void_p(cyc.data_ptr()), ctypes.c_void_p(sink.data_ptr()), which, iters, stream,
+                                        ctypes.byref(ops)):
+                return None
+            torch.cuda.synchronize()
+            t = float(cyc.max()) / ops.value
+            best = t if best is None else min(best, t)
+        out[name] = round(best, 1)
+    return out
+
+
 def chunk_flops(N, H, L, D, C=64):
     """Algorithmic FLOPs (2 per multiply-add) of the chunkwise delta rule with chunks of C steps:
     forward  per chunk  K K^T, Q K^T (2 C^2 D), K S, Q S (2 C D^2), triangular solve (C^2 D),
@@ -594,6 +628,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--no-lds-probe", action="store_true")
+    ap.add_argument("--latency-probe", action="store_true",
+                    help="instead of a workload: print the dependent-issue latencies the library's probe kernel measures")
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the compact records of the other configurations that the default run appends")
     a = ap.parse_args()
@@ -609,6 +645,10 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(2)
     dev = torch.device("cuda:0")
+    if a.latency_probe:
+        print(json.dumps({"latency_probe_ticks_per_dependent_op": measure_latencies(dev),
+                          "note": "shader-clock ticks (clock64), one workgroup of four waves, one wave per SIMD"}))
+        return
     op, N, H, L, E = WORKLOADS[a.workload]
     step, t = build_workload(a.workload, dev)
     elapsed, fwd_all, bwd_all = time_workload(step, t, a.steps, a.warmup)

@@ -527,6 +527,17 @@ SRWM_API int srwm_hip_limits(int *srwm_fwd_max_E, int *srwm_bwd_max_E, int *delt
 SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes_per_lane, void *stream,
                                 double *bytes_read);
 
+/* Measurement aid, not part of the operator path: enqueues ONE workgroup of four waves (one per SIMD, where nothing
+ * hides a latency) in which every wave runs iters x 64 operations of kind `which`, each depending on the one before:
+ *   0 v_fma_f32   1 v_add_f32 with a DPP row shift   2 v_exp_f32 + v_mul_f32   3 v_rcp_f32
+ *   4 ds_write_b32 -> wave fence -> ds_read_b32   5 ds_read_b128 addressed by the previous read
+ *   6 ds_write_b32 -> s_barrier -> ds_read_b32 of another wave's word   7 s_barrier alone
+ *   8 v_permlane32_swap_b32 + v_add_f32 + v_mul_f32   9 v_readlane_b32 -> v_fma_f32 with the scalar + v_mul_f32
+ * and writes the shader-clock ticks each wave took to cycles[0..3] (device); sink: 256 floats (device) that receive
+ * the chains' results.  *ops_per_wave (host) = iters x 64. */
+SRWM_API int srwm_hip_latency_probe(long long *cycles, float *sink, int which, int iters, void *stream,
+                                    int *ops_per_wave);
+
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
