@@ -346,7 +346,9 @@ SRWM_API int srwm_readout_grad_wide_f32(const float *k, const float *beta, const
  *   W_y_entry  dense [N,H,E,Y]: the y block before the forward call; with SRWM_FLAG_STATE_SHIFT as the
  *              difference from sW_y, the form in which the layers carry their state
  *   sW_y       dense [H,E,Y], required
- *   grad_x     dense [N,H,L,E]: W_y,t-1 grad_out_t (gradient with respect to x as given here)
+ *   grad_x     [N,H,L,E] at grad_x_strides (NULL = dense; last axis contiguous, rows must not overlap):
+ *              W_y,t-1 grad_out_t, the gradient with respect to x as given here.  With the strides of x a
+ *              layer gets it in the memory order of its input, so what follows it needs no copy
  *   gW_y       dense [N,H,E,Y]: per batch row, sum over t of x_t (x) grad_out_t
  *   gsW_y      dense [H,E,Y]: its sum over the batch in a fixed order = the gradient of the shared W_y
  * flags: SRWM_FLAG_GENERIC, SRWM_FLAG_STATE_SHIFT.
@@ -355,7 +357,8 @@ SRWM_API int srwm_layer_readout_grad_f32(const float *x, const int64_t x_strides
                                 const float *k, const float *beta, const float *y_diff,
                                 const float *keep, const float *sW_y,
                                 const float *grad_out, const int64_t grad_out_strides[3],
-                                const float *W_y_entry, float *grad_x, float *gW_y, float *gsW_y,
+                                const float *W_y_entry, float *grad_x, const int64_t grad_x_strides[3],
+                                float *gW_y, float *gsW_y,
                                 int N, int H, int L, int E, int Y, unsigned flags, void *stream);
 
 /*
@@ -541,7 +544,7 @@ SRWM_API int srwm_hip_latency_probe(long long *cycles, float *sink, int which, i
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 15. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 16. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

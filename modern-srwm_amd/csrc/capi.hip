@@ -111,7 +111,7 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 15; }
+int srwm_hip_abi_version(void) { return 16; }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -257,16 +257,18 @@ int srwm_readout_grad_wide_f32(const float *k, const float *beta, const float *y
 int srwm_layer_readout_grad_f32(const float *x, const int64_t xs[3], const float *k, const float *beta,
                                 const float *ydiff, const float *keep, const float *sWy,
                                 const float *grad_out, const int64_t gs[3], const float *Wy_entry,
-                                float *grad_x, float *gWy, float *gsWy, int N, int H, int L, int E, int Y,
-                                unsigned flags, void *stream) {
+                                float *grad_x, const int64_t gxs[3], float *gWy, float *gsWy, int N, int H, int L, int E,
+                                int Y, unsigned flags, void *stream) {
     if (!x || !xs || !k || !beta || !ydiff || !sWy || !grad_out || !gs || !Wy_entry || !grad_x || !gWy || !gsWy)
         return SRWM_EINVAL;
     if (!dims_ok(N, H, L, E) || !dims_ok(N, H, L, Y) || !family_ok(flags) || (flags & ~(kFamily | SRWM_FLAG_STATE_SHIFT)))
         return SRWM_EINVAL;
-    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, Y)) return SRWM_ESTRIDE;
+    if (!stride_ok(xs, N, H, L, E) || !stride_ok(gs, N, H, L, Y) || (gxs && !out_stride_ok(gxs, N, H, L, E)))
+        return SRWM_ESTRIDE;
     ReplayParams p{k, {(int64_t)H * L * E, (int64_t)L * E, E}, ydiff, beta, 4, keep, grad_out,
                    {gs[0], gs[1], gs[2]}, Wy_entry, sWy, grad_x, N, H, L, E, Y,
                    x, {xs[0], xs[1], xs[2]}, gWy, (flags & SRWM_FLAG_STATE_SHIFT) ? 1 : 0};
+    if (gxs) p.us = Strided3{gxs[0], gxs[1], gxs[2]};
     hipStream_t s = (hipStream_t)stream;
     int r = (flags & SRWM_FLAG_GENERIC) ? -1 : launch_replay_tiled(p, s);
     if (r < 0) {

@@ -79,7 +79,7 @@ struct ReplayParams {
     Strided3 gs;
     const float *W0;       // dense [N,H,E,M]: W before step 0
     const float *Wreset;   // dense [H,E,M] or nullptr (reset to zero)
-    float *u;              // dense [N,H,L,E]
+    float *u;              // [N,H,L,E], rows at the strides `us` below
     int N, H, L, E, M;
     // optional: per sequence, xg = sum over t of x_t (x) g_t (the gradient a matrix read as
     // out_t = W^T x_t receives when nothing flows back through the recurrence)
@@ -87,7 +87,13 @@ struct ReplayParams {
     Strided3 xs;
     float *xg;             // dense [N,H,E,M]
     int w0_is_shift;       // W0 holds W - Wreset (Wreset must be given)
+    Strided3 us;           // element strides of u (last axis contiguous); all zero: dense [N,H,L,E] (see with_u_strides)
 };
+
+inline ReplayParams with_u_strides(ReplayParams p) {
+    if (!p.us.n && !p.us.h && !p.us.l) p.us = Strided3{(int64_t)p.H * p.L * p.E, (int64_t)p.L * p.E, (int64_t)p.E};
+    return p;
+}
 
 // Per-step gradients of the delta rule when the memory carries no gradient, from u_t = W_{t-1} g_t
 // (which arrives in grad_q):  kq = k.q, ig = v_insert.g:

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(kThreads) void replay_kernel(ReplayParams p) {
             float acc = 0.f;
             for (int m = gl; m < M; m += 16) acc = fmaf(W[e * Mp + m], gv[m], acc);
             acc = group_sum<16>(acc);
-            if (gl == 0) p.u[(seq * p.L + t) * E + e] = acc;
+            if (gl == 0) p.u[n * p.us.n + h * p.us.h + t * p.us.l + e] = acc;
         }
         __syncthreads();
         // the step's write
@@ -181,6 +181,7 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
     const float *ab = p.a + n * p.as.n + h * p.as.h + e0;
     const float *gb = p.g + n * p.gs.n + h * p.gs.h;
     const float *bb = p.b + seq * p.L * Ma;
+    float *ub = p.u + n * p.us.n + h * p.us.h;
     const float *xb = XG ? p.x + n * p.xs.n + h * p.xs.h + e0 : nullptr;
 
     if constexpr (MP != M) {   // the surplus columns of the tiles stay zero: commits only write m < M
@@ -322,7 +323,7 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
             }
             group_sum_n<CGL, R>(u);
             if (cgl == 0) {
-                float *dst = p.u + (seq * p.L + t) * Ea + e0 + r0;
+                float *dst = ub + t * p.us.l + e0 + r0;
 #pragma unroll
                 for (int i = 0; i < R; ++i)
                     if (!PAD || e0 + r0 + i < Ea) dst[i] = u[i];
@@ -406,9 +407,9 @@ __global__ __launch_bounds__(NWV *kWave) void replay_tiled_kernel(ReplayParams p
 template <int E, int M, int NWV, int CGL, bool PAD = false>
 int launch_replay_tiled_as(const ReplayParams &p, hipStream_t s) {
     if (p.xg)
-        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, true, PAD>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
+        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, true, PAD>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, with_u_strides(p));
     else
-        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, false, PAD>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, p);
+        hipLaunchKernelGGL((replay_tiled_kernel<E, M, NWV, CGL, false, PAD>), dim3(p.N * p.H), dim3(NWV * kWave), 0, s, with_u_strides(p));
     return (int)hipGetLastError();
 }
 
@@ -463,7 +464,7 @@ size_t replay_lds_bytes(int E, int M) { return sizeof(float) * ((size_t)E * (M |
 int launch_replay(const ReplayParams &p, hipStream_t s) {
     const size_t lds = replay_lds_bytes(p.E, p.M);
     if (const int err = allow_max_dynamic_lds<replay_kernel>()) return err;
-    hipLaunchKernelGGL(replay_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, p);
+    hipLaunchKernelGGL(replay_kernel, dim3(p.N * p.H), dim3(kThreads), lds, s, with_u_strides(p));
     if (p.xg) hipLaunchKernelGGL(outer_sum_kernel, dim3(p.N * p.H), dim3(kThreads), 0, s, p);
     return (int)hipGetLastError();
 }

@@ -158,12 +158,26 @@ class SelfRefv0Steps(torch.autograd.Function):
 self_ref_v0_steps = SelfRefv0Steps.apply
 
 
+def _memory_order(x):
+    return sorted(range(x.dim() - 1), key=lambda i: -x.stride(i)) + [x.dim() - 1]
+
+
 def _softmax_rows(x):
     """softmax over the last axis, computed in the order the rows lie in memory (the layers hand
     over a permuted view; soft-maxing it as it is indexed would copy it first)."""
-    order = sorted(range(x.dim() - 1), key=lambda i: -x.stride(i)) + [x.dim() - 1]
+    order = _memory_order(x)
     y = torch.softmax(x.permute(order), dim=-1)
     return y.permute([order.index(i) for i in range(x.dim())])
+
+
+def _softmax_rows_backward(g, y):
+    """Gradient of the softmax over the last axis, g and its output y given with their rows in the same memory order
+    (both are then passed as the contiguous tensors they are views of: no copy, and the result keeps that order)."""
+    order = _memory_order(y)
+    if g.stride() != y.stride():
+        return torch._softmax_backward_data(g, y, -1, g.dtype)
+    r = torch._softmax_backward_data(g.permute(order), y.permute(order), -1, g.dtype)
+    return r.permute([order.index(i) for i in range(y.dim())])
 
 
 class SelfRefLayerStepsFn(torch.autograd.Function):
@@ -213,12 +227,12 @@ class SelfRefLayerStepsFn(torch.autograd.Function):
         if grad_out is None:   # the loss does not depend on the output
             return (None,) * 11
         sx = _softmax_rows(x) if ctx.softmax_input else x
-        u = torch.empty((N, H, L, E), device=dev, dtype=torch.float32)
+        u = _rows_like(sx, E, torch.float32)   # in the memory order of x: what follows it, and the reshape behind it, copy nothing
         rows = torch.empty((N, H, E, Y), device=dev, dtype=torch.float32)
         g_sWy = torch.empty((H, E, Y), device=dev, dtype=torch.float32)
         srwm_hip.self_ref_layer_readout_grad(sx, k, beta, y_diff, keep, sW_y, grad_out, shift_y, u, rows, g_sWy,
                                              flags=srwm_hip.FLAG_STATE_SHIFT)
-        grad_x = torch._softmax_backward_data(u, sx, -1, u.dtype) if ctx.softmax_input else u
+        grad_x = _softmax_rows_backward(u, sx) if ctx.softmax_input else u
         # the other shared weights: zeros, as the per-step calls return (one fill for the three)
         sizes = [math.prod(s) for s in ctx.slow_shapes]
         zeros = torch.zeros(sum(sizes), device=dev, dtype=torch.float32).split(sizes)

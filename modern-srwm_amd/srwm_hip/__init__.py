@@ -39,7 +39,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 # True: a call that the register-resident kernels do not take (head size without an instantiation, misaligned
 # base or strides) raises instead of running on the several times slower LDS-resident kernels
@@ -65,7 +65,7 @@ _SIGNATURES = {
     "srwm_layer_backward_bf16": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_S] + [_F] * 8 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_forward_steps_f32": [_F, _S] + [_F] * 17 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_wide_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 5 + [_U, ctypes.c_void_p],
-    "srwm_layer_readout_grad_f32": [_F, _S] + [_F] * 5 + [_F, _S] + [_F] * 4 + [_I] * 5 + [_U, ctypes.c_void_p],
+    "srwm_layer_readout_grad_f32": [_F, _S] + [_F] * 5 + [_F, _S] + [_F, _F, _S] + [_F] * 2 + [_I] * 5 + [_U, ctypes.c_void_p],
     "srwm_readout_grad_f32": [_F] * 5 + [_F, _S] + [_F] * 2 + [_I] * 4 + [_U, ctypes.c_void_p],
     "srwm_backward_f32": [_F, _S] + [_F] * 7 + [_F, _S] + [_F] * 9 + [_I] * 4 + [_U, ctypes.c_void_p],
     "delta_forward_steps_f32": [_F, _S] * 4 + [_F] * 5 + [_S] + [_I] * 5 + [_U, ctypes.c_void_p],
@@ -355,11 +355,12 @@ def self_ref_layer_readout_grad(x, k, beta, y_diff, keep, slow_W_y, grad_out, W_
     xs, xstr = _strided(x)
     gos, gstr = _strided(grad_out)
     with torch.cuda.device(k.device), _Dense([k, beta, y_diff, W_y_entry], False) as sv, \
-            _Dense([grad_x], True) as gr:
+            _Dense([] if grad_x.stride(-1) == 1 else [grad_x], True) as gr:
+        gxt = gr[0] if gr else grad_x   # rows at any strides: a permuted buffer is written in place
         code = lib().srwm_layer_readout_grad_f32(
             _ptr(xs), xstr, _ptr(sv[0]), _ptr(sv[1]), _ptr(sv[2]), _ptr(keep) if keep is not None else null,
-            _ptr(slow_W_y), _ptr(gos), gstr, _ptr(sv[3]), _ptr(gr[0]), _ptr(grad_W_y), _ptr(grad_slow_W_y),
-            N, H, L, E, Y, _fam(flags), _stream(k.device))
+            _ptr(slow_W_y), _ptr(gos), gstr, _ptr(sv[3]), _ptr(gxt), (ctypes.c_int64 * 3)(*gxt.stride()[:3]),
+            _ptr(grad_W_y), _ptr(grad_slow_W_y), N, H, L, E, Y, _fam(flags), _stream(k.device))
     _check(code, "srwm_layer_readout_grad_f32")
 
 

@@ -187,12 +187,13 @@ def test_argument_validation_needs_no_gpu():
     assert noalloc(N, 0, P(None)) == -1                        # the batch sums are what it is for
     assert noalloc(N, 1, fake()) == -1                         # no buffer for an incoming state gradient
     assert noalloc(1 << 16, 0, fake()) == -5                   # SRWM_ESCRATCH: 2^16 x 8 rows of 16 x 52 floats > 32 MiB
-    readout = lambda sw, gs, flags: L.srwm_layer_readout_grad_f32(
-        fake(), ok_strides, fake(), fake(), fake(), P(None), sw, fake(), ok_strides, fake(), fake(), fake(), gs,
+    readout = lambda sw, gs, flags, gxs=None: L.srwm_layer_readout_grad_f32(
+        fake(), ok_strides, fake(), fake(), fake(), P(None), sw, fake(), ok_strides, fake(), fake(), gxs, fake(), gs,
         N, H, Ls, E, E, flags, P(None))
     assert readout(P(None), fake(), 64) == -1                  # the shared W_y is always needed
     assert readout(fake(), P(None), 0) == -1                   # its gradient is what the call is for
     assert readout(fake(), fake(), 128) == -1                  # a fresh start has no entry state to replay from
+    assert readout(fake(), fake(), 0, (ctypes.c_int64 * 3)(H * E, E // 2, N * H * E)) == -3   # SRWM_ESTRIDE: rows of grad_x overlap
     dsteps = lambda gq, flags: L.delta_steps_backward_f32(
         *[a for _ in range(4) for a in (fake(), ok_strides)], P(None), fake(), fake(), fake(), ok_strides, fake(),
         gq, fake(), fake(), fake(), N, H, Ls, E, E, flags, P(None))
