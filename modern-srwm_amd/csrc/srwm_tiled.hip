@@ -602,7 +602,7 @@ __global__ __launch_bounds__(NW *kWave, (PAD && E == 64) ? 2 : 1) void srwm_bwd_
     constexpr int NXS = XC ? 5 : 4;                   // narrow columns: w_b and the last y column
     constexpr int NWL = XC ? (TT * Y + NT - 1) / NT : 1;   // words per thread of a wide tile
     const int Ea = PAD ? p.E : E, Ya = PAD ? p.E : Y;      // row lengths in global memory (constants unless PAD)
-    enum { VX, VQ, VK, VQD, VKD, NVEC };
+    enum { VX, VQ, VK, VQD, VKD, NVEC };   // (the tile holds q - k in place of q: that difference is what the tile lanes use)
 
     __shared__ __attribute__((aligned(16))) float tl[NVEC][TT][E];  // per-step vectors of the tile
     __shared__ __attribute__((aligned(16))) float tyd[TT][YS];      // y_diff of the tile
@@ -769,7 +769,8 @@ __global__ __launch_bounds__(NW *kWave, (PAD && E == 64) ? 2 : 1) void srwm_bwd_
             n_q = n_k = n_qd = n_kd = n_go = n_yd = make_float4(0.f, 0.f, 0.f, 0.f);               \
         }                                                                                          \
         *reinterpret_cast<float4 *>(&tl[VX][ld_row][ld_col]) = softmax_x ? row_softmax4<E>(n_x) : n_x; \
-        *reinterpret_cast<float4 *>(&tl[VQ][ld_row][ld_col]) = n_q;                                \
+        *reinterpret_cast<float4 *>(&tl[VQ][ld_row][ld_col]) =                                     \
+            make_float4(n_q.x - n_k.x, n_q.y - n_k.y, n_q.z - n_k.z, n_q.w - n_k.w);               \
         *reinterpret_cast<float4 *>(&tl[VK][ld_row][ld_col]) = n_k;                                \
         *reinterpret_cast<float4 *>(&tl[VQD][ld_row][ld_col]) = n_qd;                              \
         *reinterpret_cast<float4 *>(&tl[VKD][ld_row][ld_col]) = n_kd;                              \
@@ -814,11 +815,11 @@ __global__ __launch_bounds__(NW *kWave, (PAD && E == 64) ? 2 : 1) void srwm_bwd_
     // operands of one step, read from the tile in LDS
     constexpr bool PREF = E < kWave;   // fetch them one step ahead (one workgroup per CU: nothing else hides the LDS latency)
     struct Ops {
-        float kr[R], qr[R], xr[R], dif[NC], goy[YB * CB], bt[4], bd, btj, kb, qb, xb, ydl, gprey;
+        float kr[R], dvr[R], xr[R], dif[NC], goy[YB * CB], bt[4], bd, btj, kb, dvb, xb, ydl, gprey;   // dv = q - k
     };
     auto load_ops = [&](const int tt, Ops &o) __attribute__((always_inline)) {
         lds_read_vec<R>(o.kr, &tl[VK][tt][r0]);
-        lds_read_vec<R>(o.qr, &tl[VQ][tt][r0]);
+        lds_read_vec<R>(o.dvr, &tl[VQ][tt][r0]);
         lds_read_vec<R>(o.xr, &tl[VX][tt][r0]);
 #pragma unroll
         for (int b = 0; b < YB; ++b) {
@@ -831,7 +832,7 @@ __global__ __launch_bounds__(NW *kWave, (PAD && E == 64) ? 2 : 1) void srwm_bwd_
         o.bd = tb[1][tt][jb & 3];   // this thread's w_b column: beta_diff, beta
         o.btj = tb[0][tt][jb & 3];
         o.kb = tl[VK][tt][el];
-        o.qb = tl[VQ][tt][el];
+        o.dvb = tl[VQ][tt][el];
         o.xb = tl[VX][tt][el];
         o.ydl = o.gprey = 0.f;
         if constexpr (XC) {   // last y column: its diff and upstream gradient
@@ -859,18 +860,15 @@ __global__ __launch_bounds__(NW *kWave, (PAD && E == 64) ? 2 : 1) void srwm_bwd_
 
             const Ops &o = cur;
             if constexpr (!PREF) load_ops(tt, cur);
-            const float(&kr)[R] = o.kr, (&xr)[R] = o.xr;
-            float dvr[R];
-#pragma unroll
-            for (int i = 0; i < R; ++i) dvr[i] = o.qr[i] - o.kr[i];
+            const float(&kr)[R] = o.kr, (&xr)[R] = o.xr, (&dvr)[R] = o.dvr;
             float dif[NC], gpre[NC];
 #pragma unroll
             for (int c = 0; c < NC; ++c) dif[c] = o.dif[c];
 #pragma unroll
             for (int c = 0; c < QB; ++c) gpre[c] = o.goy[c];
             const float(&bt)[4] = o.bt;
-            const float bd = o.bd, btj = o.btj, kb = o.kb, qb = o.qb, xb = o.xb;
-            const float dvb = qb - kb;
+            const float bd = o.bd, btj = o.btj, kb = o.kb, dvb = o.dvb, xb = o.xb;
+            const float qb = dvb + kb;
 
             // ---- revert the write: W_{t-1} = W_t - k (x) ins
             constexpr auto beta_of = [](int c) { return c / CB < YB ? 0 : c / CB - YB + 1; };
