@@ -239,6 +239,7 @@ int launch_delta_bwd_generic(const DeltaBwdParams &p, hipStream_t s);
 // Register-resident kernels for the head sizes that are compiled in; return -1
 // when E (E, M) has no specialisation so the caller can fall back to the generic kernel.
 int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s);
+int launch_srwm_fwd_col16(const SrwmFwdParams &p, hipStream_t s);   // E = 16 fp32, a column of the state per lane; -1: not a call for it
 int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s);
 int launch_delta_fwd_tiled(const DeltaFwdParams &p, hipStream_t s);
 int launch_delta_bwd_tiled(const DeltaBwdParams &p, hipStream_t s);

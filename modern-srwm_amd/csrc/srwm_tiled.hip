@@ -1183,6 +1183,10 @@ int tiled_size_for(int E) {
 }  // namespace
 
 int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
+    if (p.E == 16 && p.Y == 16) {   // the authors' head size has a forward of its own (srwm_col16.hip)
+        const int r = launch_srwm_fwd_col16(p, s);
+        if (r >= 0) return r;
+    }
     if ((int64_t)p.L * (p.Y > p.E ? p.Y : p.E) >= ((int64_t)1 << 29)) return -1;   // 32-bit offsets inside a sequence
     if ((int64_t)p.L * p.os_l >= ((int64_t)1 << 29) || p.os_l < 0) return -1;
     // vector stores to fp32 rows of out (the wide output block and bf16 go out element by element)

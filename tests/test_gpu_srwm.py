@@ -323,8 +323,9 @@ def test_errors_are_reported_not_swallowed():
 @pytest.mark.parametrize("shape,resets", [
     ((4, 8, 100, 32), True),      # benchmark configuration 3 shape (batch slice): register-resident kernel
     ((2, 2, 37, 64), True),
-    ((3, 2, 20, 12), True),       # generic kernel
+    ((3, 2, 20, 12), True),       # the E = 16 kernel on a padded state
     ((2, 3, 15, 16), False),      # keep = None
+    ((3, 2, 37, 16), True),       # E = 16: the forward with a column of the state per lane, resets across tile boundaries
 ])
 def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
     """self_ref_v0_steps (one launch for the unroll, resets inside the kernel, gradient cut at the
@@ -362,6 +363,7 @@ def test_stepwise_operator_matches_the_per_step_reference(shape, resets):
     ((2, 1, 21, 48), None, True, False),      # LDS-resident replay + the plain outer-sum kernel
     ((3, 2, 20, 12), None, True, True),
     ((2, 3, 15, 16), None, False, False),     # keep = None
+    ((2, 3, 35, 16), None, True, True),       # E = 16 with resets, shift in and out, softmax of the input
     ((2, 2, 30, 32), 97, True, True),         # wide output block
     ((2, 2, 19, 8), 25, True, False),
     ((1, 2, 21, 64), 193, True, True),
@@ -411,7 +413,8 @@ def test_stepwise_layer_operator_matches_the_per_step_reference(shape, Y, resets
 
 
 @pytest.mark.parametrize("E,L", [(64, 15), (64, 16), (64, 17), (64, 32), (64, 33), (32, 31), (32, 32), (32, 33),
-                                 (32, 64), (16, 16), (16, 17), (8, 32), (8, 33)])
+                                 (32, 64), (16, 16), (16, 17), (8, 32), (8, 33), (16, 2), (16, 15), (16, 31), (16, 32), (16, 33),
+                                 (16, 49)])
 def test_sequence_lengths_around_the_input_tile_size(E, L):
     """The kernels stream the per-step vectors through LDS tiles of 16 or 32 steps and the forward
     prepares the readout of step t+1 during step t: lengths one below, at and one above a whole
@@ -421,7 +424,7 @@ def test_sequence_lengths_around_the_input_tile_size(E, L):
     check_against_oracle(x, W, go, 0)
 
 
-@pytest.mark.parametrize("E,L", [(64, 40), (32, 70)])
+@pytest.mark.parametrize("E,L", [(64, 40), (32, 70), (16, 50)])
 def test_resets_at_tile_boundaries(E, L):
     """Resets right before the first step, before the last step and on either side of every tile
     boundary, in different batch rows and in the same one."""
@@ -432,7 +435,7 @@ def test_resets_at_tile_boundaries(E, L):
     dev = _dev()
     N, H = 4, 2
     x, keep, shift, slow, go = _steps_inputs(N, H, L, E, seed=5, resets=True)
-    tile = 16 if E == 64 else 32
+    tile = 16 if E in (16, 64) else 32
     keep[:] = 1.0
     keep[0, 0] = keep[0, L - 1] = 0.0
     for b in range(tile, L, tile):
@@ -573,6 +576,7 @@ def test_wide_rejects_a_state_that_does_not_fit():
 
 @pytest.mark.parametrize("shape,Y,generic", [
     ((3, 4, 20, 32), 32, False),
+    ((3, 4, 37, 16), 16, False),       # the head size with a forward kernel of its own
     ((2, 16, 70, 64), 64, False),      # headline head size
     ((3, 4, 20, 32), 97, False),       # wide output block
     ((2, 3, 9, 12), 12, True),         # LDS-resident kernels (no register tiling for E = 12)
