@@ -1232,7 +1232,10 @@ int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s) {
     switch (tiled_size_for(p.E)) {
         case 64: return launch_bwd<64, 4, 8>(p, s);
         case 32: return launch_bwd<32, 4, 4>(p, s);
-        case 16: return launch_bwd<16, 1, 2>(p, s);
+        case 16:
+            // two waves per sequence shorten the step while every wave still has a SIMD of its own (256 CUs x 4);
+            // beyond that one wave per sequence does less work in total
+            return 2 * p.N * p.H <= 1024 ? launch_bwd<16, 2, 2>(p, s) : launch_bwd<16, 1, 2>(p, s);
         case 8: return launch_bwd<8, 1, 1>(p, s);
         default: return -1;
     }

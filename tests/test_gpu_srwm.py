@@ -95,6 +95,16 @@ def test_matches_fp64_oracle(shape, w_std, xsm, per_batch, flags):
     check_against_oracle(x, W, go, flags)
 
 
+@pytest.mark.parametrize("E", [16, 12])
+def test_many_short_sequences_at_the_small_head_size(E, no_fallback):
+    """At E = 16 the backward uses two waves per sequence while every wave has a SIMD to itself and one wave per sequence
+    beyond that (more than 512 sequences): both forms, also on the padded state of E = 12."""
+    for NH in ((4, 8), (65, 8)):
+        print(f"case many sequences E={E} NH={NH}", flush=True)
+        x, W, go = srwm_inputs(*NH, 12, E, seed=3, w_std=0.3, x_softmax=True, per_batch_state=NH[0] < 8)
+        check_against_oracle(x, W, go, 0)
+
+
 @pytest.fixture
 def no_fallback():
     """Any call that the register-resident kernels do not take raises instead of running on the LDS-resident ones."""
