@@ -541,10 +541,16 @@ SRWM_API int srwm_hip_lds_probe(float *out, int workgroups, int iters, int bytes
 SRWM_API int srwm_hip_latency_probe(long long *cycles, float *sink, int which, int iters, void *stream,
                                     int *ops_per_wave);
 
+/* Number of calls since the library was loaded that the register-resident kernels did not take (head size, alignment)
+ * and the LDS-resident kernels, several times slower, served instead; calls made with SRWM_FLAG_GENERIC are not
+ * counted.  For a caller that wants to notice the slow path without refusing it (SRWM_FLAG_NO_FALLBACK refuses it).
+ * No counterpart in the reference, which has one kernel family. */
+SRWM_API uint64_t srwm_hip_fallback_calls(void);
+
 /* Human-readable text for a return code of the functions above. */
 SRWM_API const char *srwm_hip_strerror(int code);
 
-/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 16. */
+/* ABI version of this header (bumped on any change of a signature or of the flag set); currently 17. */
 SRWM_API int srwm_hip_abi_version(void);
 
 #ifdef __cplusplus

@@ -102,6 +102,17 @@ int64_t scratch_span(int N, int H, int E, int width) { return ((int64_t)N * H * 
 constexpr unsigned kFamily = SRWM_FLAG_GENERIC | SRWM_FLAG_NO_FALLBACK;
 bool family_ok(unsigned flags) { return (flags & kFamily) != kFamily; }
 
+// Calls that the register-resident kernels declined and the LDS-resident ones then served, since the library was
+// loaded (calls that asked for the LDS-resident family are not counted).  A counter only: nothing reads it on the
+// way of a call.
+std::atomic<unsigned long long> g_fallback_calls{0};
+// After a declined launch: true if the caller refuses the LDS-resident kernels; else the call counts as fallen back.
+bool refuses_fallback(unsigned flags) {
+    if (flags & SRWM_FLAG_NO_FALLBACK) return true;
+    g_fallback_calls.fetch_add(1, std::memory_order_relaxed);
+    return false;
+}
+
 size_t srwm_fwd_sq(int e) { return srwm_fwd_generic_lds_bytes(e, e); }
 size_t srwm_bwd_sq(int e) { return srwm_bwd_generic_lds_bytes(e, e); }
 size_t delta_fwd_sq(int e) { return delta_fwd_generic_lds_bytes(e, e); }
@@ -111,7 +122,9 @@ size_t delta_bwd_sq(int e) { return delta_bwd_generic_lds_bytes(e, e); }
 
 extern "C" {
 
-int srwm_hip_abi_version(void) { return 16; }
+int srwm_hip_abi_version(void) { return 17; }
+
+uint64_t srwm_hip_fallback_calls(void) { return g_fallback_calls.load(std::memory_order_relaxed); }
 
 size_t srwm_hip_scratch_bytes(void) { return (size_t)SRWM_SCRATCH_FLOATS * sizeof(float); }
 
@@ -154,7 +167,7 @@ int srwm_forward_wide_f32(const float *x, const int64_t xs[3], float *Wy, float 
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_fwd_tiled(p, s);
         if (r >= 0) return r;
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
     }
     if (srwm_fwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_srwm_fwd_generic(p, s);
@@ -192,7 +205,7 @@ static int layer_forward(bool io16, const float *x, const int64_t xs[3], const f
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_fwd_tiled(p, s);
         if (r >= 0) return r;
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
     }
     if (srwm_fwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_srwm_fwd_generic(p, s);
@@ -248,7 +261,7 @@ int srwm_readout_grad_wide_f32(const float *k, const float *beta, const float *y
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_replay_tiled(p, (hipStream_t)stream);
         if (r >= 0) return r;
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
     }
     if (E > 256 || Y > 256 || replay_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_replay(p, (hipStream_t)stream);
@@ -272,7 +285,7 @@ int srwm_layer_readout_grad_f32(const float *x, const int64_t xs[3], const float
     hipStream_t s = (hipStream_t)stream;
     int r = (flags & SRWM_FLAG_GENERIC) ? -1 : launch_replay_tiled(p, s);
     if (r < 0) {
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
         if (E > 256 || Y > 256 || replay_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
         r = launch_replay(p, s);
     }
@@ -307,7 +320,7 @@ int delta_forward_steps_f32(const float *Q, const int64_t qs[3], const float *K,
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_delta_fwd_tiled(p, s);
         if (r >= 0) return r;
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
     }
     if (delta_fwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_delta_fwd_generic(p, s);
@@ -324,7 +337,7 @@ int delta_readout_replay_f32(const float *K, const int64_t ks[3], const float *v
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_replay_tiled(p, (hipStream_t)stream);
         if (r >= 0) return r;
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
     }
     if (E > 256 || M > 256 || replay_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_replay(p, (hipStream_t)stream);
@@ -423,7 +436,7 @@ int srwm_backward_wide_f32(const float *x, const int64_t xs[3], const float *q, 
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_srwm_bwd_tiled(p, s);
         if (r >= 0) return r;
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
     }
     if (srwm_bwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
     return launch_srwm_bwd_generic(p, s);
@@ -469,7 +482,7 @@ static int layer_backward(bool io16, const float *x, const int64_t xs[3], const 
     int r = -1;
     if (!(flags & SRWM_FLAG_GENERIC)) r = launch_srwm_bwd_tiled(p, s);
     if (r < 0) {
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
         if (srwm_bwd_generic_lds_bytes(E, Y) > lds_limit()) return SRWM_ESIZE;
         r = launch_srwm_bwd_generic(p, s);
     }
@@ -570,7 +583,7 @@ int delta_forward_f32(const float *Q, const int64_t qs[3], const float *K, const
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_delta_fwd_tiled(p, s);
         if (r >= 0) return r;
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
     }
     if (delta_fwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_delta_fwd_generic(p, s);
@@ -608,7 +621,7 @@ int delta_backward_f32(const float *Q, const int64_t qs[3], const float *K, cons
     if (!(flags & SRWM_FLAG_GENERIC)) {
         const int r = launch_delta_bwd_tiled(p, s);
         if (r >= 0) return r;
-        if (flags & SRWM_FLAG_NO_FALLBACK) return SRWM_ENOKERNEL;
+        if (refuses_fallback(flags)) return SRWM_ENOKERNEL;
     }
     if (delta_bwd_generic_lds_bytes(E, M) > lds_limit()) return SRWM_ESIZE;
     return launch_delta_bwd_generic(p, s);

@@ -39,7 +39,7 @@ FLAG_STATE_SHIFT = 64      # layer entry points: the state tensors hold W minus 
 FLAG_FRESH_STATE = 128     # layer forward: start from the shared weights
 FLAG_SOFTMAX_INPUT = 256   # layer entry points: x is given before its softmax
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 # True: a call that the register-resident kernels do not take (head size without an instantiation, misaligned
 # base or strides) raises instead of running on the several times slower LDS-resident kernels
@@ -111,8 +111,16 @@ def lib():
         L.srwm_hip_limits.restype = _I
         L.srwm_hip_scratch_bytes.restype = ctypes.c_size_t
         L.srwm_hip_scratch_bytes.argtypes = []
+        L.srwm_hip_fallback_calls.restype = ctypes.c_uint64
+        L.srwm_hip_fallback_calls.argtypes = []
         _lib = L
     return _lib
+
+
+def fallback_calls():
+    """Calls since the library was loaded that the register-resident kernels did not take (head size, alignment) and the
+    several times slower LDS-resident kernels served; calls that asked for those with FLAG_GENERIC are not counted."""
+    return int(lib().srwm_hip_fallback_calls())
 
 
 def limits(device=None):

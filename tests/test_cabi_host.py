@@ -50,7 +50,7 @@ def test_ctypes_signatures_match_the_header():
     import srwm_hip
     protos = _prototypes()
     aux = {"srwm_hip_abi_version", "srwm_hip_strerror", "srwm_hip_limits", "srwm_hip_lds_probe",
-           "srwm_hip_latency_probe", "srwm_hip_scratch_bytes"}
+           "srwm_hip_latency_probe", "srwm_hip_scratch_bytes", "srwm_hip_fallback_calls"}
     assert set(protos) - aux == set(srwm_hip._SIGNATURES), set(protos) - aux ^ set(srwm_hip._SIGNATURES)
     for name, args in srwm_hip._SIGNATURES.items():
         params = protos[name]

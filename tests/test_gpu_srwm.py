@@ -105,6 +105,18 @@ def test_many_short_sequences_at_the_small_head_size(E, no_fallback):
         check_against_oracle(x, W, go, 0)
 
 
+def test_calls_served_by_the_slower_kernel_family_are_counted():
+    """A head size that is no multiple of 4 runs on the LDS-resident kernels and shows in the library's counter (one
+    count for the forward, one for the backward); a compiled size, a padded one and an explicit request for the
+    LDS-resident family do not."""
+    import srwm_hip
+    for E, flags, expect in ((16, 0, 0), (12, 0, 0), (6, 0, 2), (16, srwm_hip.FLAG_GENERIC, 0)):
+        x, W, go = srwm_inputs(1, 2, 5, E, seed=1, w_std=0.3)
+        before = srwm_hip.fallback_calls()
+        run_hip(x, W, go, flags)
+        assert srwm_hip.fallback_calls() - before == expect, (E, flags)
+
+
 @pytest.fixture
 def no_fallback():
     """Any call that the register-resident kernels do not take raises instead of running on the LDS-resident ones."""
