@@ -21,7 +21,7 @@ matrix-core peak.  `cpu_baseline` is the per-timestep PyTorch recurrence (oracle
 timed on the host cores on a batch slice.
 
 Other workloads (parity-test configurations, not the headline): --workload
-{srwm_c3, srwm_generic_c4 (the LDS-resident kernel family at the headline shape), srwm_e48, delta_e96 (head sizes without a register-resident instantiation of their own), srwm_d16, srwm_rl_d16 (the head size the reference trains with), srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (through the autograd operator), delta_prologue_c2, delta_prologue_c5 (the layers' prologue kernels, fp32 and bf16, HBM-bound), delta_layer_c2 (a whole delta-rule layer)}.
+{srwm_c3, srwm_generic_c4 (the LDS-resident kernel family at the headline shape), srwm_e48, delta_e96 (head sizes without a register-resident instantiation of their own), srwm_d16, srwm_rl_d16 (the head size the reference trains with), srwm_c3_b128 (configuration 3 at a batch of 128), srwm_layer_c4, srwm_c3_steps, srwm_wide_c3, delta_c2, delta_c5f32, delta_c5, delta_c2_chunk, delta_c5f32_chunk, delta_c5_chunk, delta_c5_op_chunk (through the autograd operator), delta_prologue_c2, delta_prologue_c5 (the layers' prologue kernels, fp32 and bf16, HBM-bound), delta_layer_c2 (a whole delta-rule layer)}.
 """
 import argparse
 import json
@@ -73,6 +73,9 @@ WORKLOADS = {
     # (supervised_learning/README.md:24-40) and the RL learner's unroll (reinforcement_learning/README.md:23-52)
     "srwm_d16": ("srwm", 64, 16, 150, 16),
     "srwm_rl_d16": ("srwm", 32, 8, 50, 16),
+    # benchmark configuration 3 at four times its batch: more sequences than the device has room for at four waves
+    # each, where the E = 32 kernels run with two waves per sequence
+    "srwm_c3_b128": ("srwm", 128, 8, 100, 32),
     "delta_c2": ("delta", 32, 8, 256, 64),
     "delta_c5f32": ("delta", 8, 16, 4096, 128),
     "delta_c5": ("delta_bf16", 8, 16, 4096, 128),     # bf16 q/k/v/beta/out/grads, fp32 memory
@@ -614,7 +617,7 @@ def rooflines(name, fwd_ms, bwd_ms):
 
 # Driver-visible figures for the other benchmark configurations: (workload, timed steps, warm-up)
 OTHER_WORKLOADS = (("srwm_layer_c4", 50, 10), ("srwm_generic_c4", 5, 2), ("srwm_e48", 20, 5), ("srwm_d16", 100, 20),
-                   ("srwm_rl_d16", 100, 20), ("delta_e96", 50, 10), ("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
+                   ("srwm_rl_d16", 100, 20), ("srwm_c3_b128", 50, 10), ("delta_e96", 50, 10), ("srwm_c3", 100, 20), ("srwm_c3_steps", 100, 20), ("srwm_wide_c3", 100, 20), ("delta_c2", 100, 20),
                    ("delta_c2_chunk", 100, 20), ("delta_c5", 20, 3), ("delta_c5_chunk", 40, 5), ("delta_c5_op_chunk", 40, 5), ("delta_prologue_c2", 100, 20), ("delta_prologue_c5", 40, 5),
                    ("delta_layer_c2", 50, 10))
 

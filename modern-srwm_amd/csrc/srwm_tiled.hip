@@ -1173,6 +1173,14 @@ bool aligned16(const void *ptr, int64_t a, int64_t b, int64_t c) {
     return ((uintptr_t)ptr % 16 == 0) && a % 4 == 0 && b % 4 == 0 && c % 4 == 0;
 }
 
+// E = 32 has two tilings.  Four waves per sequence make the shortest step while there are SIMDs to spare: up to 512
+// sequences (256 CUs x 4 SIMDs, two waves on each).  Beyond that the calls are bound by the number of instructions
+// issued, and two waves per sequence issue fewer of them: every wave of a workgroup runs both softmaxes and the
+// reductions of its own tile, so halving the waves saves a quarter of the forward's and of the backward's
+// instructions (1 024 sequences of 100 steps: forward 0.118 -> 0.081 ms, backward 0.213 -> 0.145 ms; at 512 the four
+// waves win, 0.075 + 0.114 against 0.077 + 0.133 ms).
+bool many_sequences(int N, int H) { return (int64_t)N * H > 512; }
+
 // The compiled head size that serves a head size E with the narrow output block: E itself, or (for multiples of 4,
 // whose rows keep their 16-byte alignment) the next one above it, run in its padded form.  0: none.
 int tiled_size_for(int E) {
@@ -1198,7 +1206,7 @@ int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
     if (p.Y == 3 * p.E + 1) {   // wide output block: three tiled blocks of E columns and one more column
         switch (p.E) {
             case 64: return launch_fwd<64, 4, 16, 3>(p, s);
-            case 32: return launch_fwd<32, 4, 4, 3>(p, s);
+            case 32: return many_sequences(p.N, p.H) ? launch_fwd<32, 2, 8, 3>(p, s) : launch_fwd<32, 4, 4, 3>(p, s);
             case 16: return launch_fwd<16, 1, 2, 3>(p, s);
             case 8: return launch_fwd<8, 1, 1, 3>(p, s);
             default: return -1;
@@ -1207,7 +1215,7 @@ int launch_srwm_fwd_tiled(const SrwmFwdParams &p, hipStream_t s) {
     if (p.Y != p.E) return -1;
     switch (tiled_size_for(p.E)) {
         case 64: return launch_fwd<64, 4, 16>(p, s);
-        case 32: return launch_fwd<32, 4, 4>(p, s);
+        case 32: return many_sequences(p.N, p.H) ? launch_fwd<32, 2, 8>(p, s) : launch_fwd<32, 4, 4>(p, s);
         case 16: return launch_fwd<16, 1, 2>(p, s);
         case 8: return launch_fwd<8, 1, 1>(p, s);
         default: return -1;
@@ -1222,7 +1230,7 @@ int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s) {
     if (p.Y == 3 * p.E + 1) {   // grad_out and y_diff rows are read word by word: any alignment
         switch (p.E) {
             case 64: return launch_bwd<64, 4, 8, 3>(p, s);
-            case 32: return launch_bwd<32, 4, 4, 3>(p, s);
+            case 32: return many_sequences(p.N, p.H) ? launch_bwd<32, 2, 4, 3>(p, s) : launch_bwd<32, 4, 4, 3>(p, s);
             case 16: return launch_bwd<16, 1, 2, 3>(p, s);
             case 8: return launch_bwd<8, 1, 1, 3>(p, s);
             default: return -1;
@@ -1231,7 +1239,7 @@ int launch_srwm_bwd_tiled(const SrwmBwdParams &p, hipStream_t s) {
     if (p.Y != p.E || (uintptr_t)p.ydiff % 16 || !aligned16(p.go, p.gs_n, p.gs_h, p.gs_l)) return -1;
     switch (tiled_size_for(p.E)) {
         case 64: return launch_bwd<64, 4, 8>(p, s);
-        case 32: return launch_bwd<32, 4, 4>(p, s);
+        case 32: return many_sequences(p.N, p.H) ? launch_bwd<32, 2, 4>(p, s) : launch_bwd<32, 4, 4>(p, s);
         case 16:
             // two waves per sequence shorten the step while every wave still has a SIMD of its own (256 CUs x 4);
             // beyond that one wave per sequence does less work in total

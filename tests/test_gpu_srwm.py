@@ -95,14 +95,26 @@ def test_matches_fp64_oracle(shape, w_std, xsm, per_batch, flags):
     check_against_oracle(x, W, go, flags)
 
 
-@pytest.mark.parametrize("E", [16, 12])
-def test_many_short_sequences_at_the_small_head_size(E, no_fallback):
-    """At E = 16 the backward uses two waves per sequence while every wave has a SIMD to itself and one wave per sequence
-    beyond that (more than 512 sequences): both forms, also on the padded state of E = 12."""
+@pytest.mark.parametrize("E", [16, 12, 32, 24])
+def test_both_tilings_of_the_small_head_sizes(E, no_fallback):
+    """At E = 16 (backward) and E = 32 (both directions) a sequence gets more waves while every wave has a SIMD to
+    itself and fewer beyond 512 sequences: both tilings, also on the padded states of E = 12 and E = 24."""
     for NH in ((4, 8), (65, 8)):
         print(f"case many sequences E={E} NH={NH}", flush=True)
         x, W, go = srwm_inputs(*NH, 12, E, seed=3, w_std=0.3, x_softmax=True, per_batch_state=NH[0] < 8)
         check_against_oracle(x, W, go, 0)
+
+
+def test_layer_forms_of_the_many_sequence_tiling(no_fallback):
+    """The two-wave tiling of E = 32 in the forms the layers call: shared weights with and without the state shift,
+    bf16 input / output, the wide output block, resets in the step mode."""
+    print("case many sequences, layer forms", flush=True)
+    test_fused_layer_operator_matches_fp64_autograd((65, 8, 6, 32), 32, False, False)
+    test_fused_layer_operator_matches_fp64_autograd((65, 8, 5, 24), 24, False, True)
+    test_fused_layer_operator_matches_fp64_autograd((65, 8, 5, 32), 97, False, True)
+    test_bf16_fused_layer_operator((65, 8, 5, 32), 32)
+    test_wide_matches_fp64_oracle((65, 8, 7, 32), 97, 0.2, True, False)
+    test_stepwise_layer_operator_matches_the_per_step_reference((65, 8, 6, 32), None, True, True)
 
 
 def test_calls_served_by_the_slower_kernel_family_are_counted():
