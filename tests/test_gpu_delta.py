@@ -104,6 +104,22 @@ def test_sizes_between_the_compiled_ones_run_on_the_register_resident_kernels(E,
     test_stepwise_operator_matches_the_per_step_reference((2, 2, 25, E, M), True, True)
 
 
+@pytest.mark.parametrize("E,M", [(64, 64), (48, 40)])
+def test_backward_tiling_for_many_sequences(E, M, no_fallback):
+    """Beyond 512 sequences the step-by-step backward at D = 64 runs with two waves per sequence instead of eight: same
+    results to the bar, with and without an incoming gradient of the memory, also on a padded memory."""
+    print(f"case many sequences delta E={E} M={M}", flush=True)
+    test_matches_fp64_oracle((65, 8, 9, E, M), "softmax", 0.3, 0)
+    q, k, v, beta, W0, go = delta_inputs(130, 4, 7, E, M, seed=6, w0_std=0.4)
+    gs = torch.randn(W0.shape, generator=torch.Generator().manual_seed(5), dtype=torch.float64)
+    base = [t.numpy() for t in (q, k, v, beta, W0)]
+    of = oracle.delta_forward(*base)
+    ob = oracle.delta_backward(*base[:4], of, go.numpy(), grad_state=gs.numpy())
+    _, b = run_hip(q, k, v, beta, W0, go, 0, grad_state=gs)
+    for n in ("grad_Q", "grad_K", "grad_V", "grad_beta", "grad_W"):
+        assert rel_err(b[n].cpu().numpy(), ob[n]) < TOL, n
+
+
 @pytest.mark.parametrize("flags", KERNELS)
 def test_incoming_state_gradient(flags):
     print(f"case incoming grad flags={flags}", flush=True)
