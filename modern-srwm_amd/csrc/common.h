@@ -275,4 +275,14 @@ int allow_max_dynamic_lds() {
     return 0;
 }
 
+// The SRWM kernels at E = 32 have two tilings.  Four waves per sequence make the shortest step while there are SIMDs
+// to spare: up to 512 sequences (256 CUs x 4 SIMDs, two waves on each).  Beyond that the calls are bound by the number of instructions
+// issued, and two waves per sequence issue fewer of them: every wave of a workgroup runs both softmaxes and the
+// reductions of its own tile, so halving the waves saves a quarter of the forward's and of the backward's
+// instructions (1 024 sequences of 100 steps: forward 0.118 -> 0.081 ms, backward 0.213 -> 0.145 ms; at 512 the four
+// waves win, 0.075 + 0.114 against 0.077 + 0.133 ms).
+// The replay kernel of the step mode follows the same rule (its waves each fetch the whole g_t and b_t tiles: 1 024
+// sequences of 100 steps 0.056 -> 0.042 ms with two waves, 256 sequences 0.030 -> 0.033 ms).
+inline bool many_sequences(int N, int H) { return (int64_t)N * H > 512; }
+
 }  // namespace fw

@@ -446,7 +446,7 @@ int launch_replay_tiled(const ReplayParams &p, hipStream_t s) {
     switch (big <= 8 ? 8 : big <= 16 ? 16 : big <= 32 ? 32 : big <= 64 ? 64 : 128) {
         case 128: return launch_replay_tiled<128, 4, 16>(p, s);
         case 64: return launch_replay_tiled<64, 4, 8>(p, s);
-        case 32: return launch_replay_tiled<32, 4, 8>(p, s);
+        case 32: return many_sequences(p.N, p.H) ? launch_replay_tiled<32, 2, 8>(p, s) : launch_replay_tiled<32, 4, 8>(p, s);
         case 16: return launch_replay_tiled<16, 1, 8>(p, s);
         case 8: return launch_replay_tiled<8, 1, 8>(p, s);
         default: return -1;

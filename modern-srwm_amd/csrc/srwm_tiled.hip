@@ -1173,14 +1173,6 @@ bool aligned16(const void *ptr, int64_t a, int64_t b, int64_t c) {
     return ((uintptr_t)ptr % 16 == 0) && a % 4 == 0 && b % 4 == 0 && c % 4 == 0;
 }
 
-// E = 32 has two tilings.  Four waves per sequence make the shortest step while there are SIMDs to spare: up to 512
-// sequences (256 CUs x 4 SIMDs, two waves on each).  Beyond that the calls are bound by the number of instructions
-// issued, and two waves per sequence issue fewer of them: every wave of a workgroup runs both softmaxes and the
-// reductions of its own tile, so halving the waves saves a quarter of the forward's and of the backward's
-// instructions (1 024 sequences of 100 steps: forward 0.118 -> 0.081 ms, backward 0.213 -> 0.145 ms; at 512 the four
-// waves win, 0.075 + 0.114 against 0.077 + 0.133 ms).
-bool many_sequences(int N, int H) { return (int64_t)N * H > 512; }
-
 // The compiled head size that serves a head size E with the narrow output block: E itself, or (for multiples of 4,
 // whose rows keep their 16-byte alignment) the next one above it, run in its padded form.  0: none.
 int tiled_size_for(int E) {

@@ -768,6 +768,7 @@ def test_bf16_fused_layer_operator(shape, Y):
 
 @pytest.mark.parametrize("E,NH,L,M", [(8, (2, 3), 70, 8), (16, (2, 2), 33, 16), (32, (4, 8), 100, 32),
                                       (64, (2, 4), 50, 64), (128, (1, 2), 41, 128),
+                                      (32, (65, 8), 21, 32),   # more than 512 sequences: the two-wave tiling of E = 32
                                       # the wide output block, M = 3E+1 (rows of g and b at any alignment)
                                       (8, (2, 3), 70, 25), (16, (2, 2), 33, 49), (32, (4, 8), 100, 97),
                                       (64, (2, 2), 19, 193)])
