@@ -628,6 +628,9 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="srwm_c4", choices=sorted(WORKLOADS))
+    ap.add_argument("--shape", default=None, metavar="OP:N:H:L:E",
+                    help="instead of a named workload: a shape of your own, e.g. srwm:128:8:100:32 or delta_bf16:16:16:2048:128 "
+                         "(OP as in the WORKLOADS table; add ':chunk' for the chunkwise delta kernels)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-budget", type=float, default=20.0)
     ap.add_argument("--no-lds-probe", action="store_true")
@@ -652,6 +655,14 @@ def main():
         print(json.dumps({"latency_probe_ticks_per_dependent_op": measure_latencies(dev),
                           "note": "shader-clock ticks (clock64), one workgroup of four waves, one wave per SIMD"}))
         return
+    if a.shape:
+        parts = a.shape.split(":")
+        ops = sorted({w[0] for w in WORKLOADS.values()})
+        if len(parts) not in (5, 6) or parts[0] not in ops or (len(parts) == 6 and parts[5] != "chunk"):
+            ap.error(f"--shape wants OP:N:H:L:E[:chunk] with OP one of {ops}")
+        a.workload = "custom_chunk" if len(parts) == 6 else "custom"
+        WORKLOADS[a.workload] = (parts[0],) + tuple(int(v) for v in parts[1:5])
+        a.no_cpu_baseline = a.no_other_workloads = True
     op, N, H, L, E = WORKLOADS[a.workload]
     step, t = build_workload(a.workload, dev)
     elapsed, fwd_all, bwd_all = time_workload(step, t, a.steps, a.warmup)
