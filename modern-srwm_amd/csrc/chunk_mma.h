@@ -129,6 +129,15 @@ __device__ __forceinline__ void split_bf16_pair(float a, float b, uint32_t &hi, 
 struct PrecBf16 {
     static constexpr bool kBf = true;
     static constexpr int kPad = 4;        // rows of (LD * 2) bytes: LD = 4 (mod 64) keeps 8-byte reads conflict free
+    // Wider padding for matrices of 128-element rows that are mostly read TRANSPOSED (rd4t: the 16 lanes of a group
+    // address 4 rows x 32 bytes, the next group the 4 rows below).  With kPad a row starts 2 banks after the one above
+    // it, so the four 8-bank pieces of a group overlap; with 20 / 28 more elements a row starts 10 / 14 banks on: the
+    // pieces of a group are disjoint, with 28 those of two groups as well, and plain 8-byte reads of 16 rows stay
+    // conflict free (start banks all even and distinct).  Measured at config 5 (bf16, D = 128), HIP events: row sweep
+    // + column sweep 0.784 -> 0.731 ms (rows of 156 in the row sweep, 148 in the column sweep), forward 0.374 ->
+    // 0.362 ms (rows of 148); pads of 8 .. 68 were tried, the curve is flat from 20 to 52.  At D = 64 (fp32 cut in
+    // three, one wave per SIMD) the kernels are bound by their instruction stream and no padding changed anything.
+    static constexpr int kPadWide = 20, kPadWidest = 28;
     typedef uint16_t elem;
     // Two planes (hi, lo) of LD bf16 per row; matrices whose values are exact in bf16 (SPLIT
     // false) have no lo plane.

@@ -57,10 +57,18 @@ struct ChunkFwdP {
 // its partial K S and Q S through LDS.
 // OB: the products that only feed `out` (Q S, tril(B) U) take the hi parts of their operands alone
 // (precisions with operand parts; without effect otherwise), and B has no lo part.
+// Padding of the 128-element rows of K and Q (PrecBf16::kPadWide): where the LDS budget has room for it
+template <class X, int D, bool ROOM>
+constexpr int row_pad() {
+    if constexpr (X::kBf && D == 128 && ROOM) return X::kPadWide;
+    else return X::kPad;
+}
+
 template <class TI, int D, int KS, bool OB>
 struct FwdLds {
     typedef typename PrecOf<TI, D>::type X;
-    static constexpr int LDK = D + X::kPad, LDA = kC + X::kPad, LDD = 16 + X::kPad, LDV = kMC + 4;
+    static constexpr int LDA = kC + X::kPad, LDD = 16 + X::kPad, LDV = kMC + 4;
+    static constexpr int LDK = D + row_pad<X, D, OB>();   // K is read transposed for S += K^T U
     typedef typename X::template Mat<LDK, false> MatK;   // K, Q: the inputs themselves
     typedef typename X::template Mat<LDA, true> MatA;    // A: computed, feeds the solve
     typedef typename X::template Mat<LDA, !OB> MatB;     // B: computed, only feeds `out`

@@ -92,11 +92,19 @@ __device__ __forceinline__ void st_grad(float *g, int64_t i, float v) {
 // KS = 2: the rows of S and dS are split over two groups of four waves (8 waves per workgroup, two
 // per SIMD); a pair of waves owns the same 16 columns, each half of the rows, and exchanges its
 // partial K dS' through LDS.
+// Padding of 128-element rows of matrices that are read transposed, where the LDS budget has room for it
+template <class X, int D, bool ROOM>
+constexpr int wide_pad(bool widest) {
+    if constexpr (X::kBf && D == 128 && ROOM) return widest ? X::kPadWidest : X::kPadWide;
+    else return X::kPad;
+}
+
 template <class TI, int D, int KS>
 struct ColLds {
     typedef typename PrecOf<TI, D>::type X;
     static constexpr int C = 64;
-    static constexpr int LDK = D + X::kPad, LDA = C + X::kPad, LDD = 16 + X::kPad, LDG = kWC + X::kPad;
+    static constexpr int LDA = C + X::kPad, LDD = 16 + X::kPad, LDG = kWC + X::kPad;
+    static constexpr int LDK = D + wide_pad<X, D, true>(false);   // transposed reads: PrecBf16::kPadWide
     typedef typename X::template Mat<LDK, false> MatK;
     typedef typename X::template Mat<LDG, false> MatG;   // the workgroup's columns of dOut
     typedef typename X::template Mat<LDA, true> MatA;
@@ -389,7 +397,8 @@ __global__ __launch_bounds__(kThreads *KS) void delta_bwd_chunk_col_kernel(Chunk
 template <class TI, int D, int C, int KS, bool OB, bool GB>
 struct RowLds {
     typedef typename PrecOf<TI, D>::type X;
-    static constexpr int LDM = D + X::kPad, LDW = kWC + X::kPad, LDC = C + X::kPad;
+    static constexpr int LDW = kWC + X::kPad, LDC = C + X::kPad;
+    static constexpr int LDM = D + wide_pad<X, D, OB>(true);   // dOut, U, Y: read transposed (PrecBf16::kPadWidest)
     typedef typename X::template Mat<LDM, false> MatG;   // dOut: an input
     typedef typename X::template Mat<LDM, true> MatU;    // U: computed
     typedef typename X::template Mat<LDM, !GB> MatY;     // Y: computed, unless it arrives rounded
